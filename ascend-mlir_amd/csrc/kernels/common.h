@@ -1,0 +1,99 @@
+// Shared device helpers for the gfx950 fused kernels: 128-bit vector types,
+// f16/bf16 <-> f32 conversion with one round-to-nearest-even, DPP wavefront
+// reduction, and the host-side launch bookkeeping.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace afir {
+
+constexpr int kWave = 64;        // CDNA wavefront width
+constexpr int kNumCU = 256;      // MI355X compute units (8 XCDs x 32)
+constexpr int kNumXCD = 8;
+
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+struct LaunchStatus {
+  uint32_t code;
+  const char *message;  // static string
+};
+
+// ---- storage conversions (device) -----------------------------------------
+
+__device__ __forceinline__ float f16_lo(uint32_t packed) {
+  return (float)__builtin_bit_cast(f16x2, packed).x;
+}
+__device__ __forceinline__ float f16_hi(uint32_t packed) {
+  return (float)__builtin_bit_cast(f16x2, packed).y;
+}
+// two floats -> packed f16 pair, each rounded to nearest even
+__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
+  f16x2 v;
+  v.x = (_Float16)lo;
+  v.y = (_Float16)hi;
+  return __builtin_bit_cast(uint32_t, v);
+}
+
+__device__ __forceinline__ float bf16_lo(uint32_t packed) {
+  return __uint_as_float(packed << 16);
+}
+__device__ __forceinline__ float bf16_hi(uint32_t packed) {
+  return __uint_as_float(packed & 0xffff0000u);
+}
+__device__ __forceinline__ uint32_t f32_to_bf16_rne(float f) {
+  uint32_t u = __float_as_uint(f);
+  uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+  // NaN: keep it a NaN after truncation
+  return (f != f) ? ((u >> 16) | 0x40u) : r;
+}
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return (f32_to_bf16_rne(lo) & 0xffffu) | (f32_to_bf16_rne(hi) << 16);
+}
+
+// ---- wavefront reduction on DPP -------------------------------------------
+
+template <int kCtrl>
+__device__ __forceinline__ float dpp_add(float v) {
+  int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(v), kCtrl, 0xf, 0xf, true);
+  return v + __int_as_float(moved);
+}
+
+// Sum over the 64 lanes; every lane returns the total.  Within a row of 16
+// lanes: quad butterflies, then half-row and row mirrors; the four row totals
+// are then read with readlane and added in a fixed order.
+__device__ __forceinline__ float wave_sum(float v) {
+  v = dpp_add<0xB1>(v);   // quad_perm [1,0,3,2]
+  v = dpp_add<0x4E>(v);   // quad_perm [2,3,0,1]
+  v = dpp_add<0x141>(v);  // row_half_mirror
+  v = dpp_add<0x140>(v);  // row_mirror
+  int iv = __float_as_int(v);
+  float r0 = __int_as_float(__builtin_amdgcn_readlane(iv, 0));
+  float r1 = __int_as_float(__builtin_amdgcn_readlane(iv, 16));
+  float r2 = __int_as_float(__builtin_amdgcn_readlane(iv, 32));
+  float r3 = __int_as_float(__builtin_amdgcn_readlane(iv, 48));
+  return (r0 + r1) + (r2 + r3);
+}
+
+// ---- streaming memory access ------------------------------------------------
+
+template <typename T>
+__device__ __forceinline__ T load_nt(const T *p) {
+  return __builtin_nontemporal_load(p);
+}
+template <typename T>
+__device__ __forceinline__ void store_nt(T *p, T v) {
+  __builtin_nontemporal_store(v, p);
+}
+
+__host__ inline bool aligned16(const void *p) {
+  return (reinterpret_cast<uintptr_t>(p) & 15u) == 0;
+}
+
+}  // namespace afir

@@ -1,0 +1,161 @@
+// Row gather fused with scale and shift, f16:
+//   out[r,:] = f16(table[idx[r],:] * scale + shift)
+// (the fused gather region of --fuse-gather-elementwise,
+// lib/Conversion/FuseGatherElementwise/FuseGatherElementwisePass.cpp:61-303, in
+// the embedding flavour lib/Conversion/MarkStructuredOps/MarkStructuredOpsPass.cpp:141-145;
+// golden style examples/gather-elementwise-fusion/gen_data.py:62-67: f32
+// arithmetic, one round-to-nearest-even to f16).
+//
+// HBM-bound: each gathered row is read once and written once.  A lane owns one
+// 16-byte column chunk for the whole launch, so its eight scale and shift
+// values live in registers as f32.  A wave covers 1 KiB of a row per load;
+// kRowsInFlight rows are fetched before the first is used, and the row index
+// of each is wave-uniform.  The product of two f16 values is exact in f32, so
+// the fused multiply-add rounds exactly like the unfused golden.
+#include "kernels.h"
+
+namespace afir {
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kRowsInFlight = 4;
+
+__device__ __forceinline__ u32x4 scale_shift(u32x4 t, const float *s, const float *h) {
+  u32x4 r;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    float lo = f16_lo(t[d]) * s[2 * d] + h[2 * d];
+    float hi = f16_hi(t[d]) * s[2 * d + 1] + h[2 * d + 1];
+    r[d] = pack_f16(lo, hi);
+  }
+  return r;
+}
+
+// dim % 8 == 0, 16-byte aligned buffers.  The workgroup is laid out as
+// (lanes_per_row x rows_per_pass): lanes_per_row = min(256, dim/8 rounded up
+// to a multiple of 64) so that a wave never straddles two rows.
+__global__ __launch_bounds__(kThreads) void gather_scale_shift_f16_vec(
+    const uint16_t *__restrict__ table, const int32_t *__restrict__ idx,
+    const uint16_t *__restrict__ scale, const uint16_t *__restrict__ shift,
+    uint16_t *__restrict__ out, int32_t *__restrict__ error_flag, uint32_t rows, int chunks,
+    int64_t nidx, int lanes_per_row, int64_t rows_per_block) {
+  const int rows_per_pass = kThreads / lanes_per_row;
+  const int slot = threadIdx.x / lanes_per_row;  // wave-uniform
+  const int lane_col = threadIdx.x % lanes_per_row;
+  const int64_t dim = (int64_t)chunks * 8;
+  const u32x4 nan_row = {0x7e007e00u, 0x7e007e00u, 0x7e007e00u, 0x7e007e00u};
+
+  for (int64_t blk = blockIdx.x; blk * rows_per_block < nidx; blk += gridDim.x) {
+    const int64_t r_begin = blk * rows_per_block;
+    const int64_t r_end = (r_begin + rows_per_block < nidx) ? r_begin + rows_per_block : nidx;
+    for (int col = lane_col; col < chunks; col += lanes_per_row) {
+      u32x4 sraw = *reinterpret_cast<const u32x4 *>(scale + (int64_t)col * 8);
+      u32x4 hraw = *reinterpret_cast<const u32x4 *>(shift + (int64_t)col * 8);
+      float s[8], h[8];
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        s[2 * d] = f16_lo(sraw[d]);
+        s[2 * d + 1] = f16_hi(sraw[d]);
+        h[2 * d] = f16_lo(hraw[d]);
+        h[2 * d + 1] = f16_hi(hraw[d]);
+      }
+      for (int64_t r = r_begin + slot; r < r_end; r += (int64_t)rows_per_pass * kRowsInFlight) {
+        u32x4 v[kRowsInFlight];
+        bool live[kRowsInFlight], good[kRowsInFlight];
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+          const int64_t rr = r + (int64_t)u * rows_per_pass;
+          live[u] = rr < r_end;
+          good[u] = false;
+          if (live[u]) {
+            const uint32_t src = (uint32_t)idx[rr];
+            good[u] = src < rows;
+            if (good[u])
+              v[u] = load_nt(reinterpret_cast<const u32x4 *>(table + (int64_t)src * dim) + col);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+          const int64_t rr = r + (int64_t)u * rows_per_pass;
+          if (live[u]) {
+            u32x4 res = good[u] ? scale_shift(v[u], s, h) : nan_row;
+            store_nt(reinterpret_cast<u32x4 *>(out + rr * dim) + col, res);
+            if (!good[u] && error_flag && col == 0) atomicOr(error_flag, 1);
+          }
+        }
+      }
+    }
+  }
+}
+
+// Any dim / alignment: one wave per row, 2-byte accesses.
+__global__ __launch_bounds__(kThreads) void gather_scale_shift_f16_any(
+    const uint16_t *__restrict__ table, const int32_t *__restrict__ idx,
+    const uint16_t *__restrict__ scale, const uint16_t *__restrict__ shift,
+    uint16_t *__restrict__ out, int32_t *__restrict__ error_flag, uint32_t rows, int64_t dim,
+    int64_t nidx) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t wave = (int64_t)blockIdx.x * (kThreads / kWave) + (threadIdx.x >> 6);
+  const int64_t nwaves = (int64_t)gridDim.x * (kThreads / kWave);
+  for (int64_t r = wave; r < nidx; r += nwaves) {
+    const uint32_t src = (uint32_t)idx[r];
+    const bool good = src < rows;
+    if (!good && error_flag && lane == 0) atomicOr(error_flag, 1);
+    for (int64_t j = lane; j < dim; j += kWave) {
+      uint16_t res = 0x7e00u;
+      if (good) {
+        float t = (float)__builtin_bit_cast(_Float16, table[(int64_t)src * dim + j]);
+        float s = (float)__builtin_bit_cast(_Float16, scale[j]);
+        float h = (float)__builtin_bit_cast(_Float16, shift[j]);
+        res = __builtin_bit_cast(uint16_t, (_Float16)(t * s + h));
+      }
+      out[r * dim + j] = res;
+    }
+  }
+}
+
+}  // namespace
+
+LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx,
+                                       const uint16_t *scale, const uint16_t *shift,
+                                       uint16_t *out, int32_t *error_flag, int64_t rows,
+                                       int64_t dim, int64_t nidx, uint32_t block_dim,
+                                       hipStream_t stream) {
+  if (rows < 0 || dim < 0 || nidx < 0) return invalid("gather_scale_shift: negative extent");
+  if (nidx == 0 || dim == 0) return ok_status();
+  if (!idx || !out || !scale || !shift) return invalid("gather_scale_shift: null tensor pointer");
+  if (rows > 0 && !table) return invalid("gather_scale_shift: null table pointer");
+  if (rows > 0x7fffffffLL) return invalid("gather_scale_shift: table rows exceed int32 index range");
+  if (dim > 0x7fffffffLL || nidx > INT64_MAX / dim / 4 || (rows && rows > INT64_MAX / dim / 4))
+    return invalid("gather_scale_shift: extent overflow");
+
+  const bool vec = (dim % 8 == 0) && aligned16(table) && aligned16(scale) && aligned16(shift) &&
+                   aligned16(out);
+  if (vec) {
+    const int chunks = (int)(dim / 8);
+    int lanes_per_row = ((chunks + kWave - 1) / kWave) * kWave;
+    if (lanes_per_row > kThreads) lanes_per_row = kThreads;
+    if (lanes_per_row == 192) lanes_per_row = 256;  // must divide the workgroup
+    const int rows_per_pass = kThreads / lanes_per_row;
+    // rows handled by one workgroup before it moves on: enough to amortise the
+    // scale/shift registers, small enough to spread over all CUs
+    int64_t rows_per_block = (int64_t)rows_per_pass * kRowsInFlight * 2;
+    int64_t blocks = (nidx + rows_per_block - 1) / rows_per_block;
+    if (block_dim) blocks = block_dim;
+    if (blocks > 0x7fffffff) blocks = 0x7fffffff;
+    hipLaunchKernelGGL(gather_scale_shift_f16_vec, dim3((unsigned)blocks), dim3(kThreads), 0,
+                       stream, table, idx, scale, shift, out, error_flag, (uint32_t)rows, chunks,
+                       nidx, lanes_per_row, rows_per_block);
+  } else {
+    int64_t blocks = (nidx + 3) / 4;
+    if (block_dim) blocks = block_dim;
+    if (blocks > 0x7fffffff) blocks = 0x7fffffff;
+    hipLaunchKernelGGL(gather_scale_shift_f16_any, dim3((unsigned)blocks), dim3(kThreads), 0,
+                       stream, table, idx, scale, shift, out, error_flag, (uint32_t)rows, dim,
+                       nidx);
+  }
+  return after_launch();
+}
+
+}  // namespace afir

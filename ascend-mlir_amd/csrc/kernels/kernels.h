@@ -1,0 +1,49 @@
+// Host-side entry points of the gfx950 fused kernels (C++ level).  The C ABI
+// in include/afir_hip_kernels.h is a thin layer over these.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "common.h"
+
+namespace afir {
+
+// out = (a + b) * b, f32, n = rows * cols elements.
+LaunchStatus launch_fused_add_mul(const float *a, const float *b, float *out,
+                                  int64_t rows, int64_t cols, uint32_t block_dim,
+                                  hipStream_t stream);
+
+// y[i] = sum_j (x[i,j] + bias[j]), f32.
+LaunchStatus launch_broadcast_add_reducesum(const float *x, const float *bias, float *y,
+                                            int64_t m, int64_t n, uint32_t block_dim,
+                                            hipStream_t stream);
+
+// out[b,j,i] = f16(relu(x[b,i,j]) + c[j]).
+LaunchStatus launch_relu_broadcast_add_transpose(const uint16_t *x, const uint16_t *c,
+                                                 uint16_t *out, int64_t nb, int64_t m,
+                                                 int64_t n, uint32_t block_dim,
+                                                 hipStream_t stream);
+
+// out[r,:] = f16(table[idx[r],:] * scale + shift).
+LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx,
+                                       const uint16_t *scale, const uint16_t *shift,
+                                       uint16_t *out, int32_t *error_flag, int64_t rows,
+                                       int64_t dim, int64_t nidx, uint32_t block_dim,
+                                       hipStream_t stream);
+
+// out = bf16(max(v, v*alpha)), v = A@B + bias, f32 accumulate.
+LaunchStatus launch_matmul_add_leakyrelu(const uint16_t *a, const uint16_t *b,
+                                         const uint16_t *bias, uint16_t *out, int64_t m,
+                                         int64_t k, int64_t n, float alpha,
+                                         uint32_t block_dim, hipStream_t stream);
+
+inline LaunchStatus ok_status() { return LaunchStatus{0u, ""}; }
+inline LaunchStatus invalid(const char *msg) { return LaunchStatus{1u, msg}; }
+inline LaunchStatus after_launch() {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return LaunchStatus{2u, hipGetErrorString(e)};
+  return ok_status();
+}
+
+}  // namespace afir

@@ -1,0 +1,282 @@
+// Matmul + bias + leaky relu, bf16 in / f32 accumulate / bf16 out:
+//   out = bf16(max(v, v*alpha)),  v = A[M,K] @ B[K,N] + bias[N]
+// (mix kernel of lib/Target/CannKernel/CannTranslation.cpp:1573-1628,1848-1869;
+// IR examples/matmul-add-leakyrelu/step0_input.mlir:22-52; golden
+// examples/matmul-add-leakyrelu/gen_data.py:33-36 restated for bf16).
+//
+// MFMA-bound.  One workgroup owns a BM x BN tile of the output and walks K in
+// steps of 64.  Per step the A tile [BM][64] is copied to LDS as it lies in
+// memory; the B tile [64][BN] is transposed on the way (each lane fetches a
+// 4(k) x 8(n) block with four 128-bit loads, permutes bytes in registers and
+// writes eight 64-bit LDS words), so that both MFMA operands are eight
+// K-contiguous bf16 values = one 128-bit LDS read per lane.  LDS rows are 128
+// data bytes + 16 pad bytes, which spreads the 32 rows of an operand read
+// over all banks.  Two LDS stages: the next K step is fetched into registers
+// before the MFMAs of the current step are issued and written to the other
+// stage afterwards, one barrier per step.
+//
+// The MFMA is v_mfma_f32_32x32x16_bf16 with the operands swapped (B^T tile
+// as the row operand, A tile as the column operand), so a lane ends up holding
+// four consecutive n for one m: the epilogue adds bias, applies max(v, v*alpha)
+// in f32, rounds once to bf16 and stores 64 bits per lane.
+//
+// Workgroup ids are remapped so that the 32 workgroups resident on one XCD
+// (ids congruent mod 8) form a compact patch of output tiles and share their A
+// and B panels through that XCD's L2.
+#include "kernels.h"
+
+namespace afir {
+
+namespace {
+
+constexpr int kBK = 64;
+constexpr int kPitch = kBK * 2 + 16;  // bytes per LDS row
+
+__device__ __forceinline__ uint32_t perm_lo(uint32_t hi_row, uint32_t lo_row) {
+  return __builtin_amdgcn_perm(hi_row, lo_row, 0x05040100u);
+}
+__device__ __forceinline__ uint32_t perm_hi(uint32_t hi_row, uint32_t lo_row) {
+  return __builtin_amdgcn_perm(hi_row, lo_row, 0x07060302u);
+}
+
+__device__ __forceinline__ void map_tile(int p, int tiles_m, int tiles_n, int &tm, int &tn) {
+  const int ntiles = tiles_m * tiles_n;
+  int q = p;
+  if ((ntiles % kNumXCD) == 0) q = (p % kNumXCD) * (ntiles / kNumXCD) + p / kNumXCD;
+  constexpr int kGroupM = 4;
+  const int per_group = kGroupM * tiles_n;
+  const int group = q / per_group, within = q % per_group;
+  const int first_m = group * kGroupM;
+  const int gsize = (tiles_m - first_m < kGroupM) ? tiles_m - first_m : kGroupM;
+  tm = first_m + within % gsize;
+  tn = within / gsize;
+}
+
+template <int WAVES_M, int WAVES_N, int TM, int TN>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void matmul_bias_leakyrelu_bf16_mfma(
+    const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
+    const uint16_t *__restrict__ bias, uint16_t *__restrict__ out, int M, int K, int N,
+    float alpha, int tiles_m, int tiles_n) {
+  constexpr int NT = WAVES_M * WAVES_N * 64;
+  constexpr int BM = WAVES_M * TM * 32, BN = WAVES_N * TN * 32;
+  constexpr int A_STAGE = BM * kPitch, B_STAGE = BN * kPitch, STAGE = A_STAGE + B_STAGE;
+  constexpr int A_ITERS = BM * 8 / NT;              // 16-byte chunks of A per lane per step
+  constexpr int B_ITERS = 16 * (BN / 8) / NT;       // 4x8 blocks of B per lane per step
+  static_assert(A_ITERS >= 1 && B_ITERS >= 1, "tile too small for the workgroup");
+  static_assert((BM * 8) % NT == 0 && (16 * (BN / 8)) % NT == 0, "uneven loader split");
+  extern __shared__ __align__(16) unsigned char smem[];
+
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int wm = wave / WAVES_N, wn = wave % WAVES_N;
+  const int KT = K / kBK;
+
+  for (int p = blockIdx.x; p < tiles_m * tiles_n; p += gridDim.x) {
+    int tile_m, tile_n;
+    map_tile(p, tiles_m, tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    u32x4 ra[A_ITERS];
+    u32x4 rb[B_ITERS][4];
+
+    auto fetch = [&](int kt) {
+      const int k0 = kt * kBK;
+#pragma unroll
+      for (int i = 0; i < A_ITERS; ++i) {
+        const int id = t + NT * i, row = id >> 3, c = id & 7;
+        ra[i] = *reinterpret_cast<const u32x4 *>(A + (int64_t)(m0 + row) * K + k0 + c * 8);
+      }
+#pragma unroll
+      for (int i = 0; i < B_ITERS; ++i) {
+        const int bi = t + NT * i;
+        const int half = bi & 1, kq = (bi >> 1) & 3, ncl = (bi >> 3) & 7, rest = bi >> 6;
+        const int kg = (((rest & 1) * 4 + kq) << 1) + half;
+        const int nc = (rest >> 1) * 8 + ncl;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          rb[i][r] = *reinterpret_cast<const u32x4 *>(B + (int64_t)(k0 + kg * 4 + r) * N + n0 +
+                                                      nc * 8);
+      }
+    };
+
+    auto stash = [&](int stage) {
+      unsigned char *As = smem + stage * STAGE;
+      unsigned char *Bs = As + A_STAGE;
+#pragma unroll
+      for (int i = 0; i < A_ITERS; ++i) {
+        const int id = t + NT * i, row = id >> 3, c = id & 7;
+        *reinterpret_cast<u32x4 *>(As + row * kPitch + c * 16) = ra[i];
+      }
+#pragma unroll
+      for (int i = 0; i < B_ITERS; ++i) {
+        const int bi = t + NT * i;
+        const int half = bi & 1, kq = (bi >> 1) & 3, ncl = (bi >> 3) & 7, rest = bi >> 6;
+        const int kg = (((rest & 1) * 4 + kq) << 1) + half;
+        const int nc = (rest >> 1) * 8 + ncl;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int d = j >> 1;
+          u32x2 w;
+          if (j & 1) {
+            w.x = perm_hi(rb[i][1][d], rb[i][0][d]);
+            w.y = perm_hi(rb[i][3][d], rb[i][2][d]);
+          } else {
+            w.x = perm_lo(rb[i][1][d], rb[i][0][d]);
+            w.y = perm_lo(rb[i][3][d], rb[i][2][d]);
+          }
+          *reinterpret_cast<u32x2 *>(Bs + (nc * 8 + j) * kPitch + kg * 8) = w;
+        }
+      }
+    };
+
+    auto compute = [&](int stage) {
+      const unsigned char *As = smem + stage * STAGE;
+      const unsigned char *Bs = As + A_STAGE;
+      const int lrow = lane & 31, lk = lane >> 5;
+#pragma unroll
+      for (int ks = 0; ks < kBK / 16; ++ks) {
+        bf16x8 fa[TM], fb[TN];
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          fa[i] = *reinterpret_cast<const bf16x8 *>(As + ((wm * TM + i) * 32 + lrow) * kPitch +
+                                                    (ks * 2 + lk) * 16);
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          fb[j] = *reinterpret_cast<const bf16x8 *>(Bs + ((wn * TN + j) * 32 + lrow) * kPitch +
+                                                    (ks * 2 + lk) * 16);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+      }
+    };
+
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    for (int kt = 0; kt < KT; ++kt) {
+      const int cur = kt & 1;
+      if (kt + 1 < KT) fetch(kt + 1);
+      compute(cur);
+      if (kt + 1 < KT) stash(cur ^ 1);
+      __syncthreads();
+    }
+
+    // epilogue: lane holds m = lane%32, n = 8q + 4*(lane/32) + e
+    const int lm = lane & 31, lq = lane >> 5;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + (wn * TN + j) * 32 + 8 * q + 4 * lq;
+        const u32x2 braw = *reinterpret_cast<const u32x2 *>(bias + n);
+        const float b0 = bf16_lo(braw.x), b1 = bf16_hi(braw.x);
+        const float b2 = bf16_lo(braw.y), b3 = bf16_hi(braw.y);
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+          const int m = m0 + (wm * TM + i) * 32 + lm;
+          float v0 = acc[i][j][4 * q + 0] + b0;
+          float v1 = acc[i][j][4 * q + 1] + b1;
+          float v2 = acc[i][j][4 * q + 2] + b2;
+          float v3 = acc[i][j][4 * q + 3] + b3;
+          v0 = fmaxf(v0, v0 * alpha);
+          v1 = fmaxf(v1, v1 * alpha);
+          v2 = fmaxf(v2, v2 * alpha);
+          v3 = fmaxf(v3, v3 * alpha);
+          u32x2 w;
+          w.x = pack_bf16(v0, v1);
+          w.y = pack_bf16(v2, v3);
+          *reinterpret_cast<u32x2 *>(out + (int64_t)m * N + n) = w;
+        }
+      }
+    }
+  }
+}
+
+// Any shape: 16x16 output tile per workgroup, f32 FMAs, bounds-checked.
+__global__ __launch_bounds__(256) void matmul_bias_leakyrelu_bf16_any(
+    const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
+    const uint16_t *__restrict__ bias, uint16_t *__restrict__ out, int M, int K, int N,
+    float alpha, int tiles_m, int tiles_n) {
+  __shared__ float As[16][17], Bs[16][17];
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  for (int p = blockIdx.x; p < tiles_m * tiles_n; p += gridDim.x) {
+    const int m = (p / tiles_n) * 16 + ty, n = (p % tiles_n) * 16 + tx;
+    float acc = 0.f;
+    for (int k0 = 0; k0 < K; k0 += 16) {
+      const int ka = k0 + tx, kb = k0 + ty;
+      As[ty][tx] = (m < M && ka < K) ? __uint_as_float((uint32_t)A[(int64_t)m * K + ka] << 16) : 0.f;
+      Bs[ty][tx] = (kb < K && n < N) ? __uint_as_float((uint32_t)B[(int64_t)kb * N + n] << 16) : 0.f;
+      __syncthreads();
+#pragma unroll
+      for (int kk = 0; kk < 16; ++kk) acc += As[ty][kk] * Bs[kk][tx];
+      __syncthreads();
+    }
+    if (m < M && n < N) {
+      float v = acc + __uint_as_float((uint32_t)bias[n] << 16);
+      v = fmaxf(v, v * alpha);
+      out[(int64_t)m * N + n] = (uint16_t)f32_to_bf16_rne(v);
+    }
+  }
+}
+
+template <int WAVES_M, int WAVES_N, int TM, int TN>
+LaunchStatus launch_mfma(const uint16_t *a, const uint16_t *b, const uint16_t *bias,
+                         uint16_t *out, int m, int k, int n, float alpha, uint32_t block_dim,
+                         hipStream_t stream) {
+  constexpr int NT = WAVES_M * WAVES_N * 64;
+  constexpr int BM = WAVES_M * TM * 32, BN = WAVES_N * TN * 32;
+  constexpr size_t kLds = 2 * (size_t)(BM + BN) * kPitch;
+  auto kernel = matmul_bias_leakyrelu_bf16_mfma<WAVES_M, WAVES_N, TM, TN>;
+  static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                                               (int)kLds);
+  if (attr != hipSuccess) return LaunchStatus{2u, hipGetErrorString(attr)};
+  const int tiles_m = m / BM, tiles_n = n / BN;
+  int64_t blocks = (int64_t)tiles_m * tiles_n;
+  if (block_dim) blocks = block_dim;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(NT), kLds, stream, a, b, bias, out, m, k,
+                     n, alpha, tiles_m, tiles_n);
+  return after_launch();
+}
+
+}  // namespace
+
+LaunchStatus launch_matmul_add_leakyrelu(const uint16_t *a, const uint16_t *b,
+                                         const uint16_t *bias, uint16_t *out, int64_t m,
+                                         int64_t k, int64_t n, float alpha, uint32_t block_dim,
+                                         hipStream_t stream) {
+  if (m < 0 || k < 0 || n < 0) return invalid("matmul_add_leakyrelu: negative extent");
+  if (m == 0 || n == 0) return ok_status();
+  if (!out || !bias) return invalid("matmul_add_leakyrelu: null tensor pointer");
+  if (k > 0 && (!a || !b)) return invalid("matmul_add_leakyrelu: null input matrix");
+  if (m > 0x7fffffff || n > 0x7fffffff || k > 0x7fffffff)
+    return invalid("matmul_add_leakyrelu: extent exceeds 2^31-1");
+  if ((m * n) / n != m || m * n > INT64_MAX / 4 || (k && (m * k > INT64_MAX / 4 || k * n > INT64_MAX / 4)))
+    return invalid("matmul_add_leakyrelu: extent overflow");
+
+  const bool al = aligned16(a) && aligned16(b) && aligned16(out) &&
+                  ((reinterpret_cast<uintptr_t>(bias) & 7u) == 0);
+  if (al && k >= kBK && k % kBK == 0 && m % 256 == 0 && n % 256 == 0)
+    return launch_mfma<2, 4, 4, 2>(a, b, bias, out, (int)m, (int)k, (int)n, alpha, block_dim, stream);
+  if (al && k >= kBK && k % kBK == 0 && m % 128 == 0 && n % 128 == 0)
+    return launch_mfma<2, 2, 2, 2>(a, b, bias, out, (int)m, (int)k, (int)n, alpha, block_dim, stream);
+
+  const int tiles_m = (int)((m + 15) / 16), tiles_n = (int)((n + 15) / 16);
+  int64_t blocks = (int64_t)tiles_m * tiles_n;
+  if (block_dim) blocks = block_dim;
+  if (blocks > 0x7fffffff) blocks = 0x7fffffff;
+  hipLaunchKernelGGL(matmul_bias_leakyrelu_bf16_any, dim3((unsigned)blocks), dim3(256), 0, stream,
+                     a, b, bias, out, (int)m, (int)k, (int)n, alpha, tiles_m, tiles_n);
+  return after_launch();
+}
+
+}  // namespace afir

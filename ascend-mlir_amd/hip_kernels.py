@@ -1,0 +1,234 @@
+"""ctypes binding of the fused-kernel C ABI (include/afir_hip_kernels.h).
+
+Tensors are torch CUDA(ROCm) tensors used purely as device buffers; every
+function launches on torch's current stream unless `stream` (a raw
+hipStream_t value) is given, and returns the output tensor.  Nothing here
+computes on the host.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import struct
+
+from . import KERNELS_LIB
+
+
+class AfirHipError(RuntimeError):
+    pass
+
+
+class _KernelInfo(ctypes.Structure):
+    _fields_ = [("name", ctypes.c_char_p), ("symbol", ctypes.c_char_p),
+                ("num_inputs", ctypes.c_int), ("num_outputs", ctypes.c_int),
+                ("num_tiling_fields", ctypes.c_int),
+                ("tiling_fields", ctypes.POINTER(ctypes.c_char_p)),
+                ("signature", ctypes.c_char_p)]
+
+
+EXPORTED_SYMBOLS = [
+    "afir_hip_last_error",
+    "afir_hip_launch_fused_add_mul",
+    "afir_hip_launch_broadcast_add_reducesum",
+    "afir_hip_launch_relu_broadcast_add_transpose",
+    "afir_hip_launch_gather_scale_shift",
+    "afir_hip_launch_matmul_add_leakyrelu",
+    "afir_hip_kernel_count",
+    "afir_hip_kernel_info",
+    "afir_hip_find_kernel",
+    "afir_hip_launch",
+]
+
+_lib = None
+
+
+def load():
+    """dlopen the kernel library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(KERNELS_LIB):
+        raise AfirHipError(
+            f"{KERNELS_LIB} is missing: build it with "
+            "`python ascend-mlir_amd/build.py` (there is no CPU fallback)")
+    L = ctypes.CDLL(KERNELS_LIB)
+    vp, u32 = ctypes.c_void_p, ctypes.c_uint32
+    L.afir_hip_last_error.restype = ctypes.c_char_p
+    for name, nptr in [("afir_hip_launch_fused_add_mul", 5),
+                       ("afir_hip_launch_broadcast_add_reducesum", 5),
+                       ("afir_hip_launch_relu_broadcast_add_transpose", 5),
+                       ("afir_hip_launch_gather_scale_shift", 7),
+                       ("afir_hip_launch_matmul_add_leakyrelu", 6)]:
+        fn = getattr(L, name)
+        fn.restype = u32
+        fn.argtypes = [u32, vp] + [vp] * nptr
+    L.afir_hip_kernel_count.restype = ctypes.c_int
+    L.afir_hip_kernel_info.restype = ctypes.POINTER(_KernelInfo)
+    L.afir_hip_kernel_info.argtypes = [ctypes.c_int]
+    L.afir_hip_find_kernel.restype = ctypes.POINTER(_KernelInfo)
+    L.afir_hip_find_kernel.argtypes = [ctypes.c_char_p]
+    L.afir_hip_launch.restype = u32
+    L.afir_hip_launch.argtypes = [ctypes.c_char_p, u32, vp, ctypes.c_int,
+                                  ctypes.POINTER(vp), vp, vp, ctypes.c_size_t]
+    _lib = L
+    return L
+
+
+def kernel_table():
+    L = load()
+    out = []
+    for i in range(L.afir_hip_kernel_count()):
+        k = L.afir_hip_kernel_info(i).contents
+        out.append({
+            "name": k.name.decode(), "symbol": k.symbol.decode(),
+            "num_inputs": k.num_inputs, "num_outputs": k.num_outputs,
+            "tiling_fields": [k.tiling_fields[j].decode()
+                              for j in range(k.num_tiling_fields)],
+            "signature": k.signature.decode()})
+    return out
+
+
+def pack_tiling(*fields) -> bytes:
+    return struct.pack("<%dq" % len(fields), *[int(f) for f in fields])
+
+
+def f32_bits(x: float) -> int:
+    return struct.unpack("<I", struct.pack("<f", x))[0]
+
+
+def _check(rc):
+    if rc != 0:
+        raise AfirHipError(f"rc={rc}: {load().afir_hip_last_error().decode()}")
+
+
+def _stream(stream):
+    if stream is not None:
+        return ctypes.c_void_p(stream)
+    import torch
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _dev(t, dtype, what):
+    import torch
+    if not isinstance(t, torch.Tensor) or not t.is_cuda:
+        raise AfirHipError(f"{what}: expected a device tensor")
+    if t.dtype != dtype:
+        raise AfirHipError(f"{what}: expected {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise AfirHipError(f"{what}: expected a contiguous tensor")
+    return t
+
+
+def launch_raw(symbol: str, block_dim: int, stream, ptrs, tiling: bytes):
+    """Call a launcher symbol with raw device addresses (ints)."""
+    L = load()
+    fn = getattr(L, symbol)
+    buf = ctypes.create_string_buffer(tiling, len(tiling))
+    args = [ctypes.c_void_p(p) for p in ptrs]
+    return fn(ctypes.c_uint32(block_dim), _stream(stream), *args,
+              ctypes.cast(buf, ctypes.c_void_p))
+
+
+def fused_add_mul(a, b, out=None, block_dim=0, stream=None):
+    import torch
+    _dev(a, torch.float32, "a"); _dev(b, torch.float32, "b")
+    if a.shape != b.shape:
+        raise AfirHipError("fused_add_mul: a and b must have the same shape")
+    if out is None:
+        out = torch.empty_like(a)
+    _dev(out, torch.float32, "out")
+    rows = a.shape[0] if a.dim() > 0 else 1
+    cols = a.numel() // rows if rows else 0
+    _check(launch_raw("afir_hip_launch_fused_add_mul", block_dim, stream,
+                      [a.data_ptr(), b.data_ptr(), out.data_ptr(), 0],
+                      pack_tiling(rows, cols)))
+    return out
+
+
+def broadcast_add_reducesum(x, bias, out=None, block_dim=0, stream=None):
+    import torch
+    _dev(x, torch.float32, "x"); _dev(bias, torch.float32, "bias")
+    m, n = x.shape
+    if bias.shape != (n,):
+        raise AfirHipError("broadcast_add_reducesum: bias must have shape [N]")
+    if out is None:
+        out = torch.empty((m,), dtype=torch.float32, device=x.device)
+    _dev(out, torch.float32, "out")
+    _check(launch_raw("afir_hip_launch_broadcast_add_reducesum", block_dim, stream,
+                      [x.data_ptr(), bias.data_ptr(), out.data_ptr(), 0],
+                      pack_tiling(m, n)))
+    return out
+
+
+def relu_broadcast_add_transpose(x, c, out=None, block_dim=0, stream=None):
+    import torch
+    _dev(x, torch.float16, "x"); _dev(c, torch.float16, "c")
+    b, m, n = x.shape
+    if c.shape != (n,):
+        raise AfirHipError("relu_broadcast_add_transpose: c must have shape [N]")
+    if out is None:
+        out = torch.empty((b, n, m), dtype=torch.float16, device=x.device)
+    _dev(out, torch.float16, "out")
+    _check(launch_raw("afir_hip_launch_relu_broadcast_add_transpose", block_dim, stream,
+                      [x.data_ptr(), c.data_ptr(), out.data_ptr(), 0],
+                      pack_tiling(b, m, n)))
+    return out
+
+
+def gather_scale_shift(table, indices, scale, shift, out=None, workspace=None,
+                       block_dim=0, stream=None):
+    import torch
+    _dev(table, torch.float16, "table"); _dev(indices, torch.int32, "indices")
+    _dev(scale, torch.float16, "scale"); _dev(shift, torch.float16, "shift")
+    v, d = table.shape
+    (r,) = indices.shape
+    if scale.shape != (d,) or shift.shape != (d,):
+        raise AfirHipError("gather_scale_shift: scale/shift must have shape [D]")
+    if out is None:
+        out = torch.empty((r, d), dtype=torch.float16, device=table.device)
+    _dev(out, torch.float16, "out")
+    ws = workspace.data_ptr() if workspace is not None else 0
+    _check(launch_raw("afir_hip_launch_gather_scale_shift", block_dim, stream,
+                      [table.data_ptr(), indices.data_ptr(), scale.data_ptr(),
+                       shift.data_ptr(), out.data_ptr(), ws],
+                      pack_tiling(v, d, r)))
+    return out
+
+
+def matmul_add_leakyrelu(a, b, bias, alpha=0.01, out=None, block_dim=0, stream=None):
+    import torch
+    _dev(a, torch.bfloat16, "a"); _dev(b, torch.bfloat16, "b")
+    _dev(bias, torch.bfloat16, "bias")
+    m, k = a.shape
+    k2, n = b.shape
+    if k != k2 or bias.shape != (n,):
+        raise AfirHipError("matmul_add_leakyrelu: shape mismatch")
+    if out is None:
+        out = torch.empty((m, n), dtype=torch.bfloat16, device=a.device)
+    _dev(out, torch.bfloat16, "out")
+    _check(launch_raw("afir_hip_launch_matmul_add_leakyrelu", block_dim, stream,
+                      [a.data_ptr(), b.data_ptr(), bias.data_ptr(), out.data_ptr(), 0],
+                      pack_tiling(m, k, n, f32_bits(alpha))))
+    return out
+
+
+def prepare(symbol: str, ptrs, tiling: bytes, block_dim: int = 0, stream=None):
+    """Pre-marshal one launch; returns a zero-argument callable that issues it
+    (used by tight loops such as the benchmark to keep host overhead down).
+    The stream is captured now."""
+    L = load()
+    fn = getattr(L, symbol)
+    buf = ctypes.create_string_buffer(tiling, len(tiling))
+    args = [ctypes.c_uint32(block_dim), _stream(stream)]
+    args += [ctypes.c_void_p(p) for p in ptrs]
+    args.append(ctypes.cast(buf, ctypes.c_void_p))
+
+    def call(_fn=fn, _args=tuple(args), _keep=buf):
+        rc = _fn(*_args)
+        if rc:
+            _check(rc)
+    return call

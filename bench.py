@@ -1,0 +1,376 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused-kernel hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1|c3|c4|c5]
+                    [--all/--no-all] [--no-cpu-baseline]
+
+A step is one launch of the workload's fused kernel over one batch of seeded
+synthetic input already resident in HBM.  Buffer sets are rotated between
+steps so that the working set (several hundred MB) cannot be served from the
+256 MB last-level cache.  Prints ONE JSON line.
+
+  value            algorithmic GB/s (TFLOP/s for c5) over the K timed steps,
+                   wall clock between two device synchronisations
+  roofline         algorithmic bytes (flops) per launch / average launch
+                   duration from HIP events recorded on the launch stream
+                   around the same K steps, against the published peak
+  cpu_baseline     the C restatement of the reference golden ("port"), timed
+                   on this host's cores on a bounded sample
+  workloads        with --all (default): the same figures for all five
+                   configurations, each parity-checked against the oracle
+"""
+from __future__ import annotations
+
+import argparse
+import importlib.util
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = "fused-kernel HBM GB/s (% of peak); matmul+epilogue TFLOP/s; 1 GPU"
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (two runs), scaled by the same counters' reading for a plain copy kernel of
+# known size; None until measured.  Source: profiles/*_pmc.txt.
+MEASURED_TRAFFIC = {"c1": None, "c2": None, "c3": None, "c4": None, "c5": None}
+
+
+def load_package():
+    name = "ascend_mlir_amd"
+    if name in sys.modules:
+        return sys.modules[name]
+    pkg_dir = os.path.join(ROOT, "ascend-mlir_amd")
+    spec = importlib.util.spec_from_file_location(
+        name, os.path.join(pkg_dir, "__init__.py"), submodule_search_locations=[pkg_dir])
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules[name] = mod
+    spec.loader.exec_module(mod)
+    return mod
+
+
+class Workload:
+    """One configuration: seeded inputs, launch closures over `nsets` buffer
+    sets, algorithmic work, parity check and CPU baseline."""
+
+    key = ""
+    title = ""
+    dtype = ""
+    bound = "hbm"
+
+    def work(self):           # bytes (hbm) or flops (mfma) per launch
+        raise NotImplementedError
+
+
+def _dev(torch, a):
+    return torch.from_numpy(a).cuda()
+
+
+def _dev_bf16(torch, bits):
+    import numpy as np
+    return torch.from_numpy(bits.view(np.int16)).cuda().view(torch.bfloat16)
+
+
+def make_workload(key, torch, H, O, C):
+    import numpy as np
+
+    w = Workload()
+    w.key = key
+    if key == "c1":
+        a, b = O.gen_c1()
+        w.title = "c1 fused add->mul out=(a+b)*b f32 [4096,4096]"
+        w.dtype, w.symbol = "f32", "afir_hip_launch_fused_add_mul"
+        w.work = lambda: O.algorithmic_bytes("c1", m=4096, n=4096)
+        w.nsets = 3
+        sets = []
+        da, db = _dev(torch, a), _dev(torch, b)
+        for i in range(w.nsets):
+            ia, ib = (da, db) if i == 0 else (da.clone(), db.clone())
+            out = torch.empty_like(ia)
+            sets.append((ia, ib, out))
+        w.sets = sets
+        w.launches = [H.prepare(w.symbol, [s[0].data_ptr(), s[1].data_ptr(), s[2].data_ptr(), 0],
+                                H.pack_tiling(4096, 4096)) for s in sets]
+
+        def parity():
+            want = O.golden_c1(a, b)
+            got = sets[0][2].cpu().numpy()
+            return {"bar": "bit-exact", "passed": got.tobytes() == want.tobytes(),
+                    "mismatches": int((got != want).sum())}
+        w.parity = parity
+
+        def cpu(budget_s):
+            t0 = time.perf_counter(); reps = 0
+            while True:
+                C.add_mul_f32(a, b); reps += 1
+                if time.perf_counter() - t0 > budget_s or reps >= 50:
+                    break
+            dt = (time.perf_counter() - t0) / reps
+            return w.work() / dt / 1e9, f"full workload, mean of {reps} runs"
+        w.cpu = cpu
+    elif key == "c2":
+        x, bias = O.gen_c2()
+        w.title = "c2 broadcast-add-reduce y=rowsum(x+bias) f32 [8192,4096]+[4096]->[8192]"
+        w.dtype, w.symbol = "f32", "afir_hip_launch_broadcast_add_reducesum"
+        w.work = lambda: O.algorithmic_bytes("c2", m=8192, n=4096)
+        w.nsets = 4
+        dx, dbias = _dev(torch, x), _dev(torch, bias)
+        sets = []
+        for i in range(w.nsets):
+            ix = dx if i == 0 else dx.clone()
+            sets.append((ix, dbias, torch.empty((8192,), dtype=torch.float32, device="cuda")))
+        w.sets = sets
+        w.launches = [H.prepare(w.symbol, [s[0].data_ptr(), s[1].data_ptr(), s[2].data_ptr(), 0],
+                                H.pack_tiling(8192, 4096)) for s in sets]
+
+        def parity():
+            want = O.golden_c2(x, bias).astype(np.float64)
+            got = sets[0][2].cpu().numpy().astype(np.float64)
+            scale = np.abs(x.astype(np.float64) + bias).sum(axis=1)
+            err = np.abs(got - want)
+            ok = err <= 1e-5 * np.abs(want) + 1e-7 * scale
+            rel = err / np.maximum(np.abs(want), 1e-30)
+            return {"bar": "<=1e-5 rel (+1e-7*sum|terms| floor)", "passed": bool(ok.all()),
+                    "mismatches": int((~ok).sum()), "max_abs": float(err.max()),
+                    "median_rel": float(np.median(rel))}
+        w.parity = parity
+
+        def cpu(budget_s):
+            t0 = time.perf_counter(); reps = 0
+            while True:
+                C.bcast_add_rowsum_f32(x, bias); reps += 1
+                if time.perf_counter() - t0 > budget_s or reps >= 100:
+                    break
+            dt = (time.perf_counter() - t0) / reps
+            return w.work() / dt / 1e9, f"full workload, mean of {reps} runs"
+        w.cpu = cpu
+    elif key == "c3":
+        x, c = O.gen_c3()
+        w.title = "c3 relu-broadcast-transpose out=transpose(relu(x)+c) f16 [64,1024,512]->[64,512,1024]"
+        w.dtype, w.symbol = "f16", "afir_hip_launch_relu_broadcast_add_transpose"
+        w.work = lambda: O.algorithmic_bytes("c3", b=64, m=1024, n=512)
+        w.nsets = 4
+        dx, dc = _dev(torch, x), _dev(torch, c)
+        sets = []
+        for i in range(w.nsets):
+            ix = dx if i == 0 else dx.clone()
+            sets.append((ix, dc, torch.empty((64, 512, 1024), dtype=torch.float16, device="cuda")))
+        w.sets = sets
+        w.launches = [H.prepare(w.symbol, [s[0].data_ptr(), s[1].data_ptr(), s[2].data_ptr(), 0],
+                                H.pack_tiling(64, 1024, 512)) for s in sets]
+
+        def parity():
+            want = O.golden_c3(x, c)
+            got = sets[0][2].cpu().numpy()
+            return {"bar": "bit-exact (<=1e-2 rel required)",
+                    "passed": got.tobytes() == want.tobytes(),
+                    "mismatches": int((got.view(np.uint16) != want.view(np.uint16)).sum())}
+        w.parity = parity
+
+        def cpu(budget_s):
+            t0 = time.perf_counter(); reps = 0
+            while True:
+                C.relu_bcast_add_transpose_f16(x, c); reps += 1
+                if time.perf_counter() - t0 > budget_s or reps >= 20:
+                    break
+            dt = (time.perf_counter() - t0) / reps
+            return w.work() / dt / 1e9, f"full workload, mean of {reps} runs"
+        w.cpu = cpu
+    elif key == "c4":
+        table, idx, scale, shift = O.gen_c4()
+        w.title = ("c4 gather-elementwise out=table[idx]*scale+shift f16 table [131072,1024], "
+                   "int32 idx [32768]")
+        w.dtype, w.symbol = "f16", "afir_hip_launch_gather_scale_shift"
+        w.work = lambda: O.algorithmic_bytes("c4", nidx=32768, dim=1024)
+        w.nsets = 3
+        dt_, dsc, dsh = _dev(torch, table), _dev(torch, scale), _dev(torch, shift)
+        rng = np.random.default_rng(7)
+        sets = []
+        for i in range(w.nsets):
+            # the table (256 MiB) is shared; each set gathers a different
+            # seeded index vector, so consecutive launches touch different rows
+            ii = idx if i == 0 else rng.integers(0, 131072, 32768, dtype=np.int64).astype(np.int32)
+            sets.append((dt_, _dev(torch, ii), dsc, dsh,
+                         torch.empty((32768, 1024), dtype=torch.float16, device="cuda")))
+        w.sets = sets
+        w.launches = [H.prepare(w.symbol, [s[0].data_ptr(), s[1].data_ptr(), s[2].data_ptr(),
+                                           s[3].data_ptr(), s[4].data_ptr(), 0],
+                                H.pack_tiling(131072, 1024, 32768)) for s in sets]
+
+        def parity():
+            want = O.golden_c4(table, idx, scale, shift)
+            got = sets[0][4].cpu().numpy()
+            return {"bar": "bit-exact", "passed": got.tobytes() == want.tobytes(),
+                    "mismatches": int((got.view(np.uint16) != want.view(np.uint16)).sum())}
+        w.parity = parity
+
+        def cpu(budget_s):
+            t0 = time.perf_counter(); reps = 0
+            while True:
+                C.gather_scale_shift_f16(table, idx, scale, shift); reps += 1
+                if time.perf_counter() - t0 > budget_s or reps >= 20:
+                    break
+            dt = (time.perf_counter() - t0) / reps
+            return w.work() / dt / 1e9, f"full workload, mean of {reps} runs"
+        w.cpu = cpu
+    elif key == "c5":
+        a, b, bias = O.gen_c5()
+        w.title = ("c5 matmul-add-leakyrelu out=leakyrelu(A@B+bias,0.01) bf16 8192x8192x8192, "
+                   "fp32 accumulate")
+        w.dtype, w.symbol, w.bound = "bf16", "afir_hip_launch_matmul_add_leakyrelu", "mfma"
+        w.work = lambda: O.algorithmic_flops_c5(8192, 8192, 8192)
+        w.nsets = 2
+        da, db, dbias = _dev_bf16(torch, a), _dev_bf16(torch, b), _dev_bf16(torch, bias)
+        sets = []
+        for i in range(w.nsets):
+            ia, ib = (da, db) if i == 0 else (da.clone(), db.clone())
+            sets.append((ia, ib, dbias,
+                         torch.empty((8192, 8192), dtype=torch.bfloat16, device="cuda")))
+        w.sets = sets
+        w.launches = [H.prepare(w.symbol, [s[0].data_ptr(), s[1].data_ptr(), s[2].data_ptr(),
+                                           s[3].data_ptr(), 0],
+                                H.pack_tiling(8192, 8192, 8192, H.f32_bits(0.01))) for s in sets]
+
+        def parity():
+            rows = np.arange(0, 8192, 61)[:128]          # strided row sample, full K and N
+            want = O.golden_c5_rows(a, b, bias, rows, 0.01)
+            got = sets[0][3][torch.from_numpy(rows).cuda()].view(torch.int16).cpu().numpy() \
+                .view(np.uint16)
+            r = O.compare_outputs([(got, "bf16")], [(want, "bf16")], 1e-5, 1e-2)
+            return {"bar": "<=1e-2 rel (atol 1e-5), 128 sampled rows x 8192 cols",
+                    "passed": bool(r["passed"]), "mismatches": int(r["mismatches"]),
+                    "max_abs": float(r["max_abs_diff"]),
+                    "bit_identical_frac": float((got == want).mean())}
+        w.parity = parity
+
+        def cpu(budget_s):
+            rows = 64
+            t0 = time.perf_counter()
+            C.matmul_bias_leakyrelu_bf16(a[:rows], b, bias, 0.01)
+            dt = time.perf_counter() - t0
+            return (2.0 * rows * 8192 * 8192) / dt / 1e12, \
+                f"{rows} of 8192 output rows (full K and N), one run"
+        w.cpu = cpu
+    else:
+        raise SystemExit(f"unknown workload {key}")
+    return w
+
+
+def run_workload(w, torch, steps, warmup):
+    n = len(w.launches)
+    for i in range(warmup):
+        w.launches[i % n]()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for i in range(steps):
+        w.launches[i % n]()
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ev_ms = e0.elapsed_time(e1)
+    return wall, ev_ms
+
+
+def summarize(w, wall, ev_ms, steps):
+    work = w.work()
+    avg_launch_s = ev_ms / 1e3 / steps
+    if w.bound == "hbm":
+        value, unit = work * steps / wall / 1e9, "GB/s"
+        achieved, peak = work / avg_launch_s / 1e9, HBM_PEAK_GBS
+    else:
+        value, unit = work * steps / wall / 1e12, "TFLOP/s"
+        achieved, peak = work / avg_launch_s / 1e12, MFMA_BF16_PEAK_TFLOPS
+    roof = {"bound": w.bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
+            "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(w.key),
+            "avg_launch_us": round(avg_launch_s * 1e6, 3),
+            "work_per_launch": work}
+    return value, unit, roof
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=None)
+    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--all", dest="all", action="store_true", default=True)
+    ap.add_argument("--no-all", dest="all", action="store_false")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this build runs the fused-kernel path on ONE GPU; "
+                         "--gpus must be 1 (no collectives or sharding are part of it)")
+
+    import torch
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py: no GPU visible; the HIP path has no CPU fallback")
+    load_package()
+    from ascend_mlir_amd import hip_kernels as H
+    H.load()
+    from oracle import afir_oracle as O
+    from oracle import c_oracle as C
+
+    def steps_for(key):
+        if args.steps is not None:
+            return args.steps
+        return 50 if key == "c5" else 300
+
+    def warm_for(key):
+        if args.warmup is not None:
+            return args.warmup
+        return 5 if key == "c5" else 30
+
+    order = [args.workload] + ([k for k in ["c1", "c2", "c3", "c4", "c5"] if k != args.workload]
+                               if args.all else [])
+    results = []
+    for key in order:
+        w = make_workload(key, torch, H, O, C)
+        steps, warmup = steps_for(key), warm_for(key)
+        wall, ev_ms = run_workload(w, torch, steps, warmup)
+        value, unit, roof = summarize(w, wall, ev_ms, steps)
+        par = w.parity()
+        entry = {"workload": w.title, "value": round(value, 2), "unit": unit, "steps": steps,
+                 "warmup": warmup, "ms_per_step": round(wall * 1e3 / steps, 5), "dtype": w.dtype,
+                 "buffer_sets": w.nsets, "roofline": roof, "parity": par}
+        if not args.no_cpu_baseline:
+            budget = args.cpu_seconds if key == args.workload else min(3.0, args.cpu_seconds)
+            v, sample = w.cpu(budget)
+            entry["cpu_baseline"] = {"value": round(v, 4), "unit": unit, "cores": C.threads(),
+                                     "kind": "port", "sample": sample,
+                                     "host_cpus": os.cpu_count()}
+        results.append(entry)
+        del w
+        torch.cuda.empty_cache()
+
+    main_e = results[0]
+    line = {
+        "metric": METRIC, "value": main_e["value"], "unit": main_e["unit"], "n_gpus": 1,
+        "steps": main_e["steps"], "warmup": main_e["warmup"],
+        "ms_per_step": main_e["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": main_e["dtype"], "data": "synthetic",
+        "config": {"workload": main_e["workload"], "seed": 42,
+                   "buffer_sets": main_e["buffer_sets"]},
+        "roofline": {k: main_e["roofline"][k] for k in
+                     ("bound", "achieved", "peak", "unit", "frac", "traffic")},
+        "parity": main_e["parity"],
+    }
+    if "cpu_baseline" in main_e:
+        line["cpu_baseline"] = {k: main_e["cpu_baseline"][k] for k in
+                                ("value", "unit", "cores", "kind", "sample")}
+    line["device"] = torch.cuda.get_device_name(0)
+    if args.all:
+        line["workloads"] = results
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,152 @@
+/*
+ * afir_hip_kernels.h — C ABI of the gfx950 fused-kernel library
+ * (libafir_hip_kernels.so).
+ *
+ * This is the seam the reference runtime already has for "a shared library
+ * that exports one launcher symbol per kernel": its runner dlopen()s the
+ * artifact, dlsym()s the symbol and calls
+ *
+ *     uint32_t fn(uint32_t blockDim, void *stream, void *a0 ... void *a15)
+ *
+ * with [inputs..., outputs..., workspace, tiling], non-zero meaning failure,
+ * and synchronises the stream afterwards
+ * (reference: lib/Runtime/Execution/NativeExecutionRunner.cpp:616-636,753-785;
+ * generated launcher prototype lib/Runtime/Mix/MixStubTemplate.cpp:57-77).
+ * Every launcher below has exactly that shape, so a runner that binds the
+ * reference's dynamic-library artifacts binds these without a new call path.
+ *
+ * Conventions
+ *   - all tensor pointers are DEVICE pointers, row-major, densely packed;
+ *   - `stream` is a hipStream_t (NULL = the default stream); launches are
+ *     asynchronous, the caller synchronises;
+ *   - `tiling` points to HOST memory holding the packed TilingData of the
+ *     kernel: little-endian int64 fields in the order documented per kernel
+ *     (the byte string the reference's TilingSchema::pack produces,
+ *     lib/Runtime/Support/TilingSchema.cpp:61-100).  HIP passes kernel
+ *     arguments by value, so the launcher reads the shapes on the host — the
+ *     reference's vec-kernel convention of passing tiling as trailing words of
+ *     the argument buffer (NativeExecutionRunner.cpp:438-454) rather than its
+ *     mix-kernel convention of a device copy;
+ *   - field names follow the reference's generated TilingData:
+ *     dim_arg<A>_<D> = extent of dimension D of argument A, arguments counted
+ *     over (inputs..., outputs...)
+ *     (lib/Conversion/AscendCPrepareForEmit/AscendCPrepareForEmitPass.cpp:107-254);
+ *   - `block_dim` = number of workgroups to launch; 0 lets the launcher size
+ *     the grid for the 256 CUs of an MI355X (every kernel is grid-strided, so
+ *     any positive value is correct);
+ *   - `workspace` may be NULL unless stated; kernels that report data errors
+ *     (gather index out of range) set the first 4 bytes to non-zero when it is
+ *     given;
+ *   - return 0 on success, AFIR_HIP_E_* otherwise; afir_hip_last_error()
+ *     returns the calling thread's last message.
+ *
+ * Numerics: every kernel computes in float32 and rounds once (nearest even)
+ * to the storage type, like the reference's numpy goldens
+ * (examples/xx/gen_data.py: "compute in f32, cast to storage dtype").
+ */
+#ifndef AFIR_HIP_KERNELS_H
+#define AFIR_HIP_KERNELS_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define AFIR_HIP_OK 0u
+#define AFIR_HIP_E_INVALID 1u  /* bad pointer / shape / tiling bytes          */
+#define AFIR_HIP_E_LAUNCH 2u   /* HIP reported an error at launch             */
+#define AFIR_HIP_E_UNKNOWN 3u  /* no kernel of that name                      */
+
+/* Message for the calling thread's most recent non-zero return ("" if none). */
+const char *afir_hip_last_error(void);
+
+/* ---- fused elementwise chain: out = (a + b) * b ---------------------------
+ * Replaces the lowering of afir.add -> afir.mul
+ * (lib/Conversion/AFIRToASCIR/Math/Elementwise.cpp:25-57; chain from
+ * README.md:191-197).  f32, a/b/out of identical shape.
+ * TilingData { int64 dim_arg0_0 (rows); int64 dim_arg0_1 (cols); }            */
+uint32_t afir_hip_launch_fused_add_mul(uint32_t block_dim, void *stream,
+                                       void *a, void *b, void *out,
+                                       void *workspace, void *tiling);
+
+/* ---- broadcast add + row sum: y[i] = sum_j (x[i,j] + bias[j]) -------------
+ * Replaces the reduction-generic lowering
+ * (lib/Conversion/LinalgToAscendC/ComputeConversion.cpp:246-750, emitted
+ * ReduceSum at lib/Target/CannKernel/CannTranslation.cpp:2384-2484).
+ * f32 x[M,N], bias[N], y[M]; float32 accumulation.
+ * TilingData { int64 dim_arg0_0 (M); int64 dim_arg0_1 (N); }                  */
+uint32_t afir_hip_launch_broadcast_add_reducesum(uint32_t block_dim, void *stream,
+                                                 void *x, void *bias, void *y,
+                                                 void *workspace, void *tiling);
+
+/* ---- relu + broadcast add + transpose ------------------------------------
+ * out[b,j,i] = f16(relu(x[b,i,j]) + c[j]); x f16 [B,M,N], c f16 [N],
+ * out f16 [B,N,M].  Replaces the parallel generic with a PureTranspose input
+ * map and a PureBroadcast input (ComputeConversion.cpp:265-333,1290-1640;
+ * transpose emission :775-826).
+ * TilingData { int64 dim_arg0_0 (B); int64 dim_arg0_1 (M); int64 dim_arg0_2 (N); } */
+uint32_t afir_hip_launch_relu_broadcast_add_transpose(uint32_t block_dim, void *stream,
+                                                      void *x, void *c, void *out,
+                                                      void *workspace, void *tiling);
+
+/* ---- row gather + scale + shift -------------------------------------------
+ * out[r,:] = f16(table[indices[r],:] * scale + shift); table f16 [V,D],
+ * indices int32 [R] in [0,V), scale/shift f16 [D], out f16 [R,D].
+ * Replaces the fused gather region (--fuse-gather-elementwise,
+ * lib/Conversion/FuseGatherElementwise/FuseGatherElementwisePass.cpp:61-303;
+ * row loop ComputeConversion.cpp:828-1272) in its embedding (row) flavour
+ * (lib/Conversion/MarkStructuredOps/MarkStructuredOpsPass.cpp:141-145).
+ * An index outside [0,V) yields a row of NaN and, when workspace is given,
+ * a non-zero int32 at workspace[0]; it never reads outside the table.
+ * TilingData { int64 dim_arg0_0 (V); int64 dim_arg0_1 (D); int64 dim_arg1_0 (R); } */
+uint32_t afir_hip_launch_gather_scale_shift(uint32_t block_dim, void *stream,
+                                            void *table, void *indices,
+                                            void *scale, void *shift, void *out,
+                                            void *workspace, void *tiling);
+
+/* ---- matmul + bias + leaky relu --------------------------------------------
+ * out = bf16(leakyrelu(A @ B + bias, alpha)); A bf16 [M,K], B bf16 [K,N]
+ * (not transposed), bias bf16 [N], out bf16 [M,N]; float32 accumulation on
+ * the matrix cores, epilogue fused before the store.  leakyrelu(x) is
+ * max(x, x*alpha) as the reference IR spells it
+ * (examples/matmul-add-leakyrelu/step0_input.mlir:40-52).  Replaces the mix
+ * kernel (lib/Target/CannKernel/CannTranslation.cpp:1573-1628,1848-1869;
+ * epilogue vocabulary BiasAddLeakyRelu,
+ * lib/Conversion/MarkStructuredOps/AnnotateMixMatmulSemanticsPass.cpp:79-342).
+ * TilingData { int64 dim_arg0_0 (M); int64 dim_arg0_1 (K); int64 dim_arg1_1 (N);
+ *              int64 alpha_f32_bits (IEEE-754 bits of alpha in the low 32 bits) } */
+uint32_t afir_hip_launch_matmul_add_leakyrelu(uint32_t block_dim, void *stream,
+                                              void *a, void *b, void *bias, void *out,
+                                              void *workspace, void *tiling);
+
+/* ---- registry + name-based dispatch -----------------------------------------
+ * What a runner needs to bind a kernel by the name an artifact manifest
+ * carries (kernel_name=..., lib/Runtime/Artifact/VecCubeArtifactBackend.cpp:62-106)
+ * and to build its tiling schema. */
+typedef struct AfirHipKernelInfo {
+  const char *name;           /* e.g. "broadcast_add_reducesum"                */
+  const char *symbol;         /* launcher symbol exported by this library       */
+  int num_inputs;
+  int num_outputs;
+  int num_tiling_fields;
+  const char *const *tiling_fields; /* names, in TilingData order, all int64   */
+  const char *signature;      /* human-readable: dtypes and shapes             */
+} AfirHipKernelInfo;
+
+int afir_hip_kernel_count(void);
+const AfirHipKernelInfo *afir_hip_kernel_info(int index);
+const AfirHipKernelInfo *afir_hip_find_kernel(const char *name);
+
+/* Launch by name.  args = [inputs..., outputs...] device pointers
+ * (num_args must equal num_inputs + num_outputs of the kernel); tiling_len is
+ * checked against 8 * num_tiling_fields. */
+uint32_t afir_hip_launch(const char *kernel_name, uint32_t block_dim, void *stream,
+                         int num_args, void *const *args, void *workspace,
+                         const void *tiling, size_t tiling_len);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* AFIR_HIP_KERNELS_H */

@@ -1,0 +1,322 @@
+"""Parity of the HIP fused kernels (called through the C ABI) with the CPU
+oracle on the same seeded inputs.  Needs an MI355X: run with -m gpu.
+
+Bars: bit-exact for the f32 add/mul chain, the f16 transpose chain and the
+gather; <= 1e-5 relative (with an absolute floor of 1e-7 * sum|terms|, the
+scale of one rounding of the row's terms) for the f32 row sum; <= 1e-2 relative (atol 1e-5)
+for the bf16 matmul epilogue.
+"""
+import numpy as np
+import pytest
+
+from oracle import afir_oracle as O
+from oracle import c_oracle as C
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def H(pkg):
+    from ascend_mlir_amd import hip_kernels
+    hip_kernels.load()          # raises if the library is not built
+    assert torch.cuda.is_available(), "no GPU visible"
+    return hip_kernels
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def dev_bf16(bits):
+    return torch.from_numpy(np.ascontiguousarray(bits).view(np.int16)).cuda().view(torch.bfloat16)
+
+
+def host_bf16(t):
+    return t.view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+# ---------------------------------------------------------------- C1 --------
+
+@pytest.mark.parametrize("shape", [(4, 4), (1, 1), (257, 129), (1024, 1024), (3, 100003)])
+def test_c1_small_bit_exact(H, shape):
+    a, b = O.gen_c1(shape)
+    out = H.fused_add_mul(dev(a), dev(b)).cpu().numpy()
+    assert out.tobytes() == O.golden_c1(a, b).tobytes()
+    assert out.tobytes() == C.add_mul_f32(a, b).tobytes()
+
+
+def test_c1_full_size_bit_exact(H):
+    a, b = O.gen_c1()
+    out = H.fused_add_mul(dev(a), dev(b)).cpu().numpy()
+    assert out.tobytes() == O.golden_c1(a, b).tobytes()
+
+
+def test_c1_empty_unaligned_and_blockdim(H):
+    e = torch.empty((0, 16), dtype=torch.float32, device="cuda")
+    assert H.fused_add_mul(e, e).shape == (0, 16)
+    a, b = O.gen_c1((1, 4099))
+    da, db = dev(np.concatenate([[0], a.ravel()]).astype(np.float32)), \
+        dev(np.concatenate([[0], b.ravel()]).astype(np.float32))
+    ua, ub = da[1:].view(1, -1), db[1:].view(1, -1)       # 4-byte aligned only
+    out = H.fused_add_mul(ua, ub).cpu().numpy()
+    assert out.tobytes() == O.golden_c1(a, b).tobytes()
+    a, b = O.gen_c1((512, 1000))
+    for bd in (1, 7, 40):                                   # reference-style block_dim
+        out = H.fused_add_mul(dev(a), dev(b), block_dim=bd).cpu().numpy()
+        assert out.tobytes() == O.golden_c1(a, b).tobytes()
+
+
+def test_c1_special_values(H):
+    a = np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, 3e38, 1.0], np.float32)
+    b = np.array([0.0, 0.0, 1.0, np.inf, 1.0, 1e-45, 3e38, -1.0], np.float32)
+    with np.errstate(all="ignore"):
+        want = O.golden_c1(a, b)
+    out = H.fused_add_mul(dev(a.reshape(1, -1)), dev(b.reshape(1, -1))).cpu().numpy().ravel()
+    assert np.array_equal(np.isnan(out), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert out[ok].tobytes() == want[ok].tobytes()       # denormals are kept
+
+
+# ---------------------------------------------------------------- C2 --------
+
+def _check_rowsum(x, bias, y):
+    want = O.golden_c2(x, bias)
+    scale = np.abs(x.astype(np.float64) + bias.astype(np.float64)).sum(axis=1)
+    err = np.abs(y.astype(np.float64) - want.astype(np.float64))
+    tol = 1e-5 * np.abs(want.astype(np.float64)) + 1e-7 * scale
+    assert np.all(err <= tol), (err.max(), (err / np.maximum(tol, 1e-300)).max())
+    # and against exact arithmetic: well inside f32 accumulation error
+    exact = x.astype(np.float64).sum(axis=1) + bias.astype(np.float64).sum()
+    assert np.all(np.abs(y - exact) <= 2e-6 * scale + 1e-30)
+
+
+@pytest.mark.parametrize("m,n", [(1, 4), (7, 5), (33, 4096), (64, 512), (5, 1000),
+                                 (130, 1028), (3, 8192), (2, 100000)])
+def test_c2_small(H, m, n):
+    x, bias = O.gen_c2(m, n)
+    y = H.broadcast_add_reducesum(dev(x), dev(bias)).cpu().numpy()
+    _check_rowsum(x, bias, y)
+
+
+def test_c2_full_size(H):
+    x, bias = O.gen_c2()
+    y = H.broadcast_add_reducesum(dev(x), dev(bias)).cpu().numpy()
+    _check_rowsum(x, bias, y)
+
+
+def test_c2_exact_integer_rows_and_blockdim(H):
+    ones = np.ones((16, 4096), np.float32)
+    z = np.zeros(4096, np.float32)
+    y = H.broadcast_add_reducesum(dev(ones), dev(z)).cpu().numpy()
+    assert np.array_equal(y, np.full(16, 4096, np.float32))
+    onehot = np.zeros((4, 128), np.float32)
+    onehot[np.arange(4), [0, 5, 77, 127]] = 3.0
+    y = H.broadcast_add_reducesum(dev(onehot), dev(np.ones(128, np.float32))).cpu().numpy()
+    assert np.array_equal(y, np.full(4, 131, np.float32))
+    x, bias = O.gen_c2(100, 640)
+    for bd in (1, 40):
+        y = H.broadcast_add_reducesum(dev(x), dev(bias), block_dim=bd).cpu().numpy()
+        _check_rowsum(x, bias, y)
+    e = torch.empty((0, 8), dtype=torch.float32, device="cuda")
+    assert H.broadcast_add_reducesum(e, dev(z[:8])).shape == (0,)
+    # zero columns: every row sums to 0
+    y = H.broadcast_add_reducesum(torch.empty((3, 0), dtype=torch.float32, device="cuda"),
+                                  torch.empty((0,), dtype=torch.float32, device="cuda"))
+    assert np.array_equal(y.cpu().numpy(), np.zeros(3, np.float32))
+
+
+# ---------------------------------------------------------------- C3 --------
+
+@pytest.mark.parametrize("b,m,n", [(2, 3, 5), (1, 128, 128), (3, 256, 128), (2, 128, 384),
+                                   (3, 70, 36), (1, 1, 1), (2, 129, 128), (1, 33, 250)])
+def test_c3_small_bit_exact(H, b, m, n):
+    x, c = O.gen_c3(b, m, n)
+    out = H.relu_broadcast_add_transpose(dev(x), dev(c)).cpu().numpy()
+    assert out.shape == (b, n, m)
+    assert out.tobytes() == O.golden_c3(x, c).tobytes()
+    assert out.tobytes() == C.relu_bcast_add_transpose_f16(x, c).tobytes()
+
+
+def test_c3_full_size_bit_exact(H):
+    x, c = O.gen_c3()
+    out = H.relu_broadcast_add_transpose(dev(x), dev(c)).cpu().numpy()
+    assert out.tobytes() == O.golden_c3(x, c).tobytes()
+
+
+def test_c3_involution_and_blockdim(H):
+    x, _ = O.gen_c3(4, 256, 384)
+    pos = np.abs(x)
+    z1 = dev(np.zeros(384, np.float16))
+    z2 = dev(np.zeros(256, np.float16))
+    once = H.relu_broadcast_add_transpose(dev(pos), z1)
+    twice = H.relu_broadcast_add_transpose(once, z2).cpu().numpy()
+    assert twice.tobytes() == pos.tobytes()
+    x, c = O.gen_c3(2, 256, 256)
+    for bd in (1, 5):
+        out = H.relu_broadcast_add_transpose(dev(x), dev(c), block_dim=bd).cpu().numpy()
+        assert out.tobytes() == O.golden_c3(x, c).tobytes()
+    e = torch.empty((0, 4, 4), dtype=torch.float16, device="cuda")
+    assert H.relu_broadcast_add_transpose(e, dev(np.zeros(4, np.float16))).shape == (0, 4, 4)
+
+
+def test_c3_special_values(H):
+    x = np.zeros((1, 128, 128), np.float16)
+    x[0, 0, :8] = [np.nan, -np.inf, np.inf, -0.0, 6e-8, -6e-8, 65504, -65504]
+    c = np.zeros(128, np.float16)
+    c[3] = -0.0
+    with np.errstate(all="ignore"):
+        want = O.golden_c3(x, c)
+    out = H.relu_broadcast_add_transpose(dev(x), dev(c)).cpu().numpy()
+    assert np.array_equal(np.isnan(out), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert out[ok].tobytes() == want[ok].tobytes()
+
+
+# ---------------------------------------------------------------- C4 --------
+
+@pytest.mark.parametrize("rows,dim,nidx", [(512, 64, 256), (1000, 1024, 513), (100, 136, 77),
+                                           (64, 8, 5), (300, 2048, 40), (50, 100, 33),
+                                           (10, 1, 7), (128, 1536, 19)])
+def test_c4_small_bit_exact(H, rows, dim, nidx):
+    table, idx, scale, shift = O.gen_c4(rows, dim, nidx)
+    idx[:3] = [0, rows - 1, rows - 1]
+    out = H.gather_scale_shift(dev(table), dev(idx), dev(scale), dev(shift)).cpu().numpy()
+    assert out.tobytes() == O.golden_c4(table, idx, scale, shift).tobytes()
+    assert out.tobytes() == C.gather_scale_shift_f16(table, idx, scale, shift).tobytes()
+
+
+def test_c4_identity_rows_are_byte_identical(H):
+    table, idx, _, _ = O.gen_c4(4096, 1024, 2048)
+    one = np.ones(1024, np.float16)
+    zero = np.zeros(1024, np.float16)
+    out = H.gather_scale_shift(dev(table), dev(idx), dev(one), dev(zero)).cpu().numpy()
+    assert out.tobytes() == table[idx].tobytes()
+
+
+def test_c4_full_size_bit_exact(H):
+    table, idx, scale, shift = O.gen_c4()
+    idx[:4] = [0, 131071, 131071, 0]
+    out = H.gather_scale_shift(dev(table), dev(idx), dev(scale), dev(shift)).cpu().numpy()
+    assert out.tobytes() == O.golden_c4(table, idx, scale, shift).tobytes()
+
+
+def test_c4_out_of_range_index_is_flagged_not_read(H):
+    table, idx, scale, shift = O.gen_c4(64, 128, 16)
+    idx[5] = 64
+    idx[9] = -1
+    ws = torch.zeros(2, dtype=torch.int32, device="cuda")
+    out = H.gather_scale_shift(dev(table), dev(idx), dev(scale), dev(shift),
+                               workspace=ws).cpu().numpy()
+    assert int(ws[0].item()) != 0
+    assert np.isnan(out[5]).all() and np.isnan(out[9]).all()
+    good = np.ones(16, bool)
+    good[[5, 9]] = False
+    idx2 = idx.copy()
+    idx2[[5, 9]] = 0
+    want = O.golden_c4(table, idx2, scale, shift)
+    assert out[good].tobytes() == want[good].tobytes()
+    ws.zero_()
+    H.gather_scale_shift(dev(table), dev(idx2), dev(scale), dev(shift), workspace=ws)
+    assert int(ws[0].item()) == 0
+    e = torch.empty((0,), dtype=torch.int32, device="cuda")
+    assert H.gather_scale_shift(dev(table), e, dev(scale), dev(shift)).shape == (0, 128)
+
+
+def test_c4_blockdim(H):
+    table, idx, scale, shift = O.gen_c4(777, 1024, 1000)
+    want = O.golden_c4(table, idx, scale, shift)
+    for bd in (1, 3, 40):
+        out = H.gather_scale_shift(dev(table), dev(idx), dev(scale), dev(shift),
+                                   block_dim=bd).cpu().numpy()
+        assert out.tobytes() == want.tobytes()
+
+
+# ---------------------------------------------------------------- C5 --------
+
+C5_ATOL, C5_RTOL = 1e-5, 1e-2
+
+
+def _check_c5(got_bits, want_bits):
+    r = O.compare_outputs([(got_bits, "bf16")], [(want_bits, "bf16")], C5_ATOL, C5_RTOL)
+    assert r["passed"], r
+    assert (got_bits == want_bits).mean() > 0.97
+
+
+@pytest.mark.parametrize("m,k,n", [(256, 256, 256), (512, 128, 768), (128, 64, 128),
+                                   (384, 192, 128), (48, 1024, 80), (1, 1, 1), (17, 33, 65),
+                                   (256, 100, 256)])
+def test_c5_small(H, m, k, n):
+    a, b, bias = O.gen_c5(m, k, n)
+    out = H.matmul_add_leakyrelu(dev_bf16(a), dev_bf16(b), dev_bf16(bias), 0.01)
+    _check_c5(host_bf16(out), O.golden_c5(a, b, bias, 0.01))
+
+
+def test_c5_integer_known_answer_exact(H):
+    # the reference's trick: small integers make f32 accumulation exact, so any
+    # summation order must give the same bits
+    r = np.random.default_rng(42)
+    for (m, k, n) in [(128, 256, 128), (256, 512, 512)]:
+        A = r.integers(-10, 10, (m, k)).astype(np.float32)
+        B = r.integers(-10, 10, (k, n)).astype(np.float32)
+        bias = r.integers(1, 10, (n,)).astype(np.float32)
+        bits = [O.f32_to_bf16_bits(v) for v in (A, B, bias)]
+        out = H.matmul_add_leakyrelu(dev_bf16(bits[0]), dev_bf16(bits[1]), dev_bf16(bits[2]), 0.01)
+        assert np.array_equal(host_bf16(out), O.golden_c5(*bits, 0.01))
+
+
+def test_c5_identity_and_alpha(H):
+    n = 256
+    eye = O.f32_to_bf16_bits(np.eye(n, dtype=np.float32))
+    a, _, _ = O.gen_c5(n, n, n)
+    zero = np.zeros(n, np.uint16)
+    out = H.matmul_add_leakyrelu(dev_bf16(a), dev_bf16(eye), dev_bf16(zero), 1.0)
+    assert np.array_equal(host_bf16(out), a)                 # alpha=1: identity
+    out = H.matmul_add_leakyrelu(dev_bf16(a), dev_bf16(eye), dev_bf16(zero), 0.0)
+    want = O.f32_to_bf16_bits(np.maximum(O.bf16_bits_to_f32(a), 0))
+    got = host_bf16(out)
+    assert np.array_equal(O.bf16_bits_to_f32(got), O.bf16_bits_to_f32(want))   # relu (-0 == 0)
+
+
+def test_c5_full_size(H):
+    a, b, bias = O.gen_c5()
+    out = H.matmul_add_leakyrelu(dev_bf16(a), dev_bf16(b), dev_bf16(bias), 0.01)
+    got = host_bf16(out)
+    want = O.golden_c5(a, b, bias, 0.01)
+    _check_c5(got, want)
+
+
+def test_c5_empty_and_blockdim(H):
+    a, b, bias = O.gen_c5(512, 128, 512)
+    want = O.golden_c5(a, b, bias, 0.01)
+    for bd in (1, 3):
+        out = H.matmul_add_leakyrelu(dev_bf16(a), dev_bf16(b), dev_bf16(bias), 0.01, block_dim=bd)
+        _check_c5(host_bf16(out), want)
+    e = torch.empty((0, 128), dtype=torch.bfloat16, device="cuda")
+    out = H.matmul_add_leakyrelu(e, dev_bf16(b), dev_bf16(bias), 0.01)
+    assert out.shape == (0, 512)
+
+
+# ------------------------------------------------------- dispatch by name ----
+
+def test_launch_by_name_and_errors(H):
+    import ctypes
+    L = H.load()
+    a, b = O.gen_c1((64, 64))
+    da, db = dev(a), dev(b)
+    out = torch.empty_like(da)
+    args = (ctypes.c_void_p * 3)(da.data_ptr(), db.data_ptr(), out.data_ptr())
+    til = H.pack_tiling(64, 64)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rc = L.afir_hip_launch(b"fused_add_mul", 0, stream, 3, args, None, til, len(til))
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert out.cpu().numpy().tobytes() == O.golden_c1(a, b).tobytes()
+    assert L.afir_hip_launch(b"no_such_kernel", 0, stream, 3, args, None, til, len(til)) == 3
+    assert b"no_such_kernel" in L.afir_hip_last_error()
+    assert L.afir_hip_launch(b"fused_add_mul", 0, stream, 2, args, None, til, len(til)) == 1
+    assert L.afir_hip_launch(b"fused_add_mul", 0, stream, 3, args, None, til, 8) == 1
+    assert b"tiling" in L.afir_hip_last_error()
+    bad = H.pack_tiling(-1, 64)
+    assert L.afir_hip_launch(b"fused_add_mul", 0, stream, 3, args, None, bad, len(bad)) == 1
