@@ -27,7 +27,8 @@ constexpr int kThreads = 256;
 constexpr int kTile = 128;               // elements per tile edge
 constexpr int kChunksPerRow = kTile / 8;  // 16-byte chunks per LDS row
 
-__device__ __forceinline__ float relu_keep_nan(float v) { return (v < 0.f) ? 0.f : v; }
+// max(v, +0) with IEEE-754 maximum semantics: NaN propagates, -0 gives +0.
+__device__ __forceinline__ float relu_keep_nan(float v) { return (v > 0.f) ? v : ((v != v) ? v : 0.f); }
 
 __device__ __forceinline__ uint32_t relu_add_pack(uint32_t packed, float c_lo, float c_hi) {
   float lo = relu_keep_nan(f16_lo(packed)) + c_lo;
