@@ -35,6 +35,7 @@ KERNEL_SOURCES = [
     ("kernels/transpose.hip", STRICT),
     ("kernels/gather.hip", STRICT),
     ("kernels/matmul.hip", []),
+    ("kernels/matmul_dma.hip", []),
     ("capi/afir_hip_kernels.cpp", []),
 ]
 

@@ -18,8 +18,15 @@ namespace afir {
 
 namespace {
 
+#ifndef AFIR_GATHER_RIF
+#define AFIR_GATHER_RIF 1
+#endif
+#ifndef AFIR_GATHER_PASSES
+#define AFIR_GATHER_PASSES 4
+#endif
 constexpr int kThreads = 256;
-constexpr int kRowsInFlight = 4;
+constexpr int kRowsInFlight = AFIR_GATHER_RIF;
+constexpr int kPassesPerBlock = AFIR_GATHER_PASSES;
 
 __device__ __forceinline__ u32x4 scale_shift(u32x4 t, const float *s, const float *h) {
   u32x4 r;
@@ -41,8 +48,10 @@ __global__ __launch_bounds__(kThreads) void gather_scale_shift_f16_vec(
     uint16_t *__restrict__ out, int32_t *__restrict__ error_flag, uint32_t rows, int chunks,
     int64_t nidx, int lanes_per_row, int64_t rows_per_block) {
   const int rows_per_pass = kThreads / lanes_per_row;
-  const int slot = threadIdx.x / lanes_per_row;  // wave-uniform
-  const int lane_col = threadIdx.x % lanes_per_row;
+  // a wave never straddles two rows, so the row slot is wave-uniform: say so,
+  // and the index fetch becomes a scalar load
+  const int slot = __builtin_amdgcn_readfirstlane(threadIdx.x / lanes_per_row);
+  const int lane_col = threadIdx.x - slot * lanes_per_row;
   const int64_t dim = (int64_t)chunks * 8;
   const u32x4 nan_row = {0x7e007e00u, 0x7e007e00u, 0x7e007e00u, 0x7e007e00u};
 
@@ -61,24 +70,28 @@ __global__ __launch_bounds__(kThreads) void gather_scale_shift_f16_vec(
         h[2 * d + 1] = f16_hi(hraw[d]);
       }
       for (int64_t r = r_begin + slot; r < r_end; r += (int64_t)rows_per_pass * kRowsInFlight) {
+        // Branch-free fetch: rows past the end re-read the last row, indices
+        // outside the table read row 0; both are discarded below.  All index
+        // loads are issued first, then all row loads, so kRowsInFlight rows
+        // are in flight per lane.
+        uint32_t src[kRowsInFlight];
+        bool good[kRowsInFlight];
         u32x4 v[kRowsInFlight];
-        bool live[kRowsInFlight], good[kRowsInFlight];
 #pragma unroll
         for (int u = 0; u < kRowsInFlight; ++u) {
           const int64_t rr = r + (int64_t)u * rows_per_pass;
-          live[u] = rr < r_end;
-          good[u] = false;
-          if (live[u]) {
-            const uint32_t src = (uint32_t)idx[rr];
-            good[u] = src < rows;
-            if (good[u])
-              v[u] = load_nt(reinterpret_cast<const u32x4 *>(table + (int64_t)src * dim) + col);
-          }
+          src[u] = (uint32_t)idx[rr < r_end ? rr : r_end - 1];
+        }
+#pragma unroll
+        for (int u = 0; u < kRowsInFlight; ++u) {
+          good[u] = src[u] < rows;
+          const uint32_t safe = good[u] ? src[u] : 0u;
+          v[u] = load_nt(reinterpret_cast<const u32x4 *>(table + (int64_t)safe * dim) + col);
         }
 #pragma unroll
         for (int u = 0; u < kRowsInFlight; ++u) {
           const int64_t rr = r + (int64_t)u * rows_per_pass;
-          if (live[u]) {
+          if (rr < r_end) {
             u32x4 res = good[u] ? scale_shift(v[u], s, h) : nan_row;
             store_nt(reinterpret_cast<u32x4 *>(out + rr * dim) + col, res);
             if (!good[u] && error_flag && col == 0) atomicOr(error_flag, 1);
@@ -130,7 +143,8 @@ LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx
   if (dim > 0x7fffffffLL || nidx > INT64_MAX / dim / 4 || (rows && rows > INT64_MAX / dim / 4))
     return invalid("gather_scale_shift: extent overflow");
 
-  const bool vec = (dim % 8 == 0) && aligned16(table) && aligned16(scale) && aligned16(shift) &&
+  // (an empty table has no row to fall back on: the scalar kernel never reads it)
+  const bool vec = rows > 0 && (dim % 8 == 0) && aligned16(table) && aligned16(scale) && aligned16(shift) &&
                    aligned16(out);
   if (vec) {
     const int chunks = (int)(dim / 8);
@@ -140,7 +154,7 @@ LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx
     const int rows_per_pass = kThreads / lanes_per_row;
     // rows handled by one workgroup before it moves on: enough to amortise the
     // scale/shift registers, small enough to spread over all CUs
-    int64_t rows_per_block = (int64_t)rows_per_pass * kRowsInFlight * 2;
+    int64_t rows_per_block = (int64_t)rows_per_pass * kRowsInFlight * kPassesPerBlock;
     int64_t blocks = (nidx + rows_per_block - 1) / rows_per_block;
     if (block_dim) blocks = block_dim;
     if (blocks > 0x7fffffff) blocks = 0x7fffffff;

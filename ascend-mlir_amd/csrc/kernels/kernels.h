@@ -38,6 +38,12 @@ LaunchStatus launch_matmul_add_leakyrelu(const uint16_t *a, const uint16_t *b,
                                          int64_t k, int64_t n, float alpha,
                                          uint32_t block_dim, hipStream_t stream);
 
+// Fast path of the matmul for tile-aligned shapes (matmul_dma.hip).
+bool matmul_dma_supported(int64_t m, int64_t k, int64_t n);
+LaunchStatus launch_matmul_dma(const uint16_t *a, const uint16_t *b, const uint16_t *bias,
+                               uint16_t *out, int m, int k, int n, float alpha,
+                               uint32_t block_dim, hipStream_t stream);
+
 inline LaunchStatus ok_status() { return LaunchStatus{0u, ""}; }
 inline LaunchStatus invalid(const char *msg) { return LaunchStatus{1u, msg}; }
 inline LaunchStatus after_launch() {

@@ -265,6 +265,8 @@ LaunchStatus launch_matmul_add_leakyrelu(const uint16_t *a, const uint16_t *b,
 
   const bool al = aligned16(a) && aligned16(b) && aligned16(out) &&
                   ((reinterpret_cast<uintptr_t>(bias) & 7u) == 0);
+  if (al && matmul_dma_supported(m, k, n))
+    return launch_matmul_dma(a, b, bias, out, (int)m, (int)k, (int)n, alpha, block_dim, stream);
   if (al && k >= kBK && k % kBK == 0 && m % 256 == 0 && n % 256 == 0)
     return launch_mfma<2, 4, 4, 2>(a, b, bias, out, (int)m, (int)k, (int)n, alpha, block_dim, stream);
   if (al && k >= kBK && k % kBK == 0 && m % 128 == 0 && n % 128 == 0)

@@ -1,0 +1,389 @@
+// Matmul + bias + leaky relu for large, tile-aligned shapes (M, N multiples of
+// 256, K a multiple of 64): the MFMA-bound fast path.
+//
+// The feed is the bottleneck of a bf16 GEMM on this chip: one K step of 32 is
+// ~0.4 us of MFMA work per CU while a global load takes ~2 us to come back
+// under load, so several K steps have to be in flight.  Registers cannot hold
+// them, LDS can: tiles are copied global -> LDS directly (global_load_lds, 16
+// bytes per lane, no VGPR staging) into two rings that together fill the
+// 160 KiB of LDS:
+//
+//   A ring: 3 slots of [256 m][64 k] bf16 (128-byte rows, 32 KiB): 64 k at a
+//           time so that every row segment is a full 128-byte line -- with
+//           64-byte segments the feed alone took 30 % longer;
+//   B ring: 4 slots of [32 k][256 n] bf16 (512-byte rows, 16 KiB).
+//
+// A direct-to-LDS load writes lane l's 16 bytes at base + 16*l, so a wave
+// fills 1 KiB of contiguous LDS; which 16-byte chunk of global memory a lane
+// fetches is free, and that is where the bank swizzle goes:
+//   A: chunk c of row r lands at chunk position c ^ ((r>>1)&7);
+//   B: chunk c of row k lands at chunk position c ^ ((k&3)<<2).
+// The A operand of an MFMA is one 128-bit LDS read per lane (8 consecutive k
+// of one m).  The B operand needs 8 consecutive k of one n from a tile whose
+// rows run along n: ds_read_b64_tr_b16 does that transpose in the LDS unit
+// (within 16 lanes, lanes 4r..4r+3 address row r, lane i receives column i of
+// the four rows).  With the swizzles above both reads are bank-conflict free.
+//
+// The compiler cannot be trusted to wait for exactly the right stage (it
+// drains every outstanding direct-to-LDS load before any LDS read that might
+// alias one), so the operand reads are issued from inline asm and the waits
+// are explicit: s_waitcnt vmcnt(n) + s_barrier once per K step of 32, which
+// leaves the two youngest B stages and the youngest A slice in flight.
+// Operand reads are software-pipelined one k16 substep ahead of the MFMAs.
+//
+// Every tile starts its walk over K at a different offset and wraps around
+// (K-stagger): the row pitch of A and B is a large power of two, so without it
+// all workgroups of the chip ask the same few L2 / memory channels for the
+// same K offset at the same time.
+//
+// 8 waves as 2(m) x 4(n), wave tile 128 x 64 = 4 x 2 MFMA tiles of 32x32,
+// v_mfma_f32_32x32x16_bf16 with the operands swapped (B as the row operand) so
+// that a lane holds four consecutive n of one m for the fused epilogue.
+#include "kernels.h"
+
+namespace afir {
+
+namespace {
+
+#ifndef AFIR_MM_KSTAGGER_M
+#define AFIR_MM_KSTAGGER_M 2
+#endif
+#ifndef AFIR_MM_KSTAGGER_N
+#define AFIR_MM_KSTAGGER_N 1
+#endif
+constexpr int kBK = 32;                   // K per B stage
+constexpr int kBM = 256, kBN = 256;
+constexpr int kASlots = 3, kBSlots = 4;
+constexpr int kSlotA = kBM * 64 * 2;      // 32 KiB: 64 k per A slice
+constexpr int kSlotB = kBK * kBN * 2;     // 16 KiB
+constexpr int kRingB = kASlots * kSlotA;  // byte offset of the B ring
+constexpr int kLdsBytes = kASlots * kSlotA + kBSlots * kSlotB;  // 160 KiB
+
+typedef __attribute__((address_space(3))) unsigned char lds_byte;
+typedef __attribute__((address_space(3))) void lds_void;
+typedef __attribute__((address_space(1))) const void gbl_void;
+
+__device__ __forceinline__ void map_tile_dma(int p, int tiles_m, int tiles_n, int &tm, int &tn) {
+  const int ntiles = tiles_m * tiles_n;
+  int q = p;
+  if ((ntiles % kNumXCD) == 0) q = (p % kNumXCD) * (ntiles / kNumXCD) + p / kNumXCD;
+  constexpr int kGroupM = 4;
+  const int per_group = kGroupM * tiles_n;
+  const int group = q / per_group, within = q % per_group;
+  const int first_m = group * kGroupM;
+  const int gsize = (tiles_m - first_m < kGroupM) ? tiles_m - first_m : kGroupM;
+  tm = first_m + within % gsize;
+  tn = within / gsize;
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+}
+
+// Operands of one k16 substep: four A fragments (m tiles 0..3, 4 KiB apart)
+// and two B fragments (n tiles 0..1, each two transposing 64-bit reads 4 rows
+// apart).  issue_reads only issues; the registers must not be touched until
+// settle_reads, which waits for the LDS unit and hands the same registers back
+// as fresh values.
+template <int TMW>
+struct Operands {
+  u32x4 a[TMW];
+  u32x2 b[2][2];
+};
+
+template <int KS>  // k16 substep within the B stage (0 or 1)
+__device__ __forceinline__ void issue_reads(uint32_t a_addr, uint32_t b_addr0, uint32_t b_addr1,
+                                            Operands<4> &o) {
+  constexpr int kOff = KS * 16 * 512;  // 16 rows of B
+  asm volatile(
+      "ds_read_b128 %0, %8\n\t"
+      "ds_read_b128 %1, %8 offset:4096\n\t"
+      "ds_read_b128 %2, %8 offset:8192\n\t"
+      "ds_read_b128 %3, %8 offset:12288\n\t"
+      "ds_read_b64_tr_b16 %4, %9 offset:%11\n\t"
+      "ds_read_b64_tr_b16 %5, %9 offset:%12\n\t"
+      "ds_read_b64_tr_b16 %6, %10 offset:%11\n\t"
+      "ds_read_b64_tr_b16 %7, %10 offset:%12"
+      : "=&v"(o.a[0]), "=&v"(o.a[1]), "=&v"(o.a[2]), "=&v"(o.a[3]), "=&v"(o.b[0][0]),
+        "=&v"(o.b[0][1]), "=&v"(o.b[1][0]), "=&v"(o.b[1][1])
+      : "v"(a_addr), "v"(b_addr0), "v"(b_addr1), "n"(kOff), "n"(kOff + 4 * 512)
+      : "memory");
+}
+
+template <int KS>
+__device__ __forceinline__ void issue_reads(uint32_t a_addr, uint32_t b_addr0, uint32_t b_addr1,
+                                            Operands<2> &o) {
+  constexpr int kOff = KS * 16 * 512;
+  asm volatile(
+      "ds_read_b128 %0, %6\n\t"
+      "ds_read_b128 %1, %6 offset:4096\n\t"
+      "ds_read_b64_tr_b16 %2, %7 offset:%9\n\t"
+      "ds_read_b64_tr_b16 %3, %7 offset:%10\n\t"
+      "ds_read_b64_tr_b16 %4, %8 offset:%9\n\t"
+      "ds_read_b64_tr_b16 %5, %8 offset:%10"
+      : "=&v"(o.a[0]), "=&v"(o.a[1]), "=&v"(o.b[0][0]), "=&v"(o.b[0][1]), "=&v"(o.b[1][0]),
+        "=&v"(o.b[1][1])
+      : "v"(a_addr), "v"(b_addr0), "v"(b_addr1), "n"(kOff), "n"(kOff + 4 * 512)
+      : "memory");
+}
+
+__device__ __forceinline__ void settle_reads(Operands<4> &o) {
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(o.a[0]), "+v"(o.a[1]), "+v"(o.a[2]), "+v"(o.a[3]), "+v"(o.b[0][0]),
+                 "+v"(o.b[0][1]), "+v"(o.b[1][0]), "+v"(o.b[1][1])
+               :
+               : "memory");
+}
+__device__ __forceinline__ void settle_reads(Operands<2> &o) {
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(o.a[0]), "+v"(o.a[1]), "+v"(o.b[0][0]), "+v"(o.b[0][1]), "+v"(o.b[1][0]),
+                 "+v"(o.b[1][1])
+               :
+               : "memory");
+}
+
+struct Par0 { static constexpr int value = 0; };
+struct Par1 { static constexpr int value = 1; };
+struct Steady { static constexpr bool value = true; };
+struct Drain { static constexpr bool value = false; };
+
+// WM = waves along m (2 or 4); 4 waves along n.  Wave tile (256/WM) x 64.
+template <int WM>
+__global__ __launch_bounds__(WM * 4 * 64) void matmul_bias_leakyrelu_bf16_dma(
+    const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
+    const uint16_t *__restrict__ bias, uint16_t *__restrict__ out, int M, int K, int N,
+    float alpha, int tiles_m, int tiles_n) {
+  extern __shared__ __align__(1024) unsigned char smem[];
+  lds_byte *const lds = (lds_byte *)smem;
+  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+
+  const int t = threadIdx.x, lane = t & 63;
+  constexpr int TMW = 8 / WM;            // 32-row MFMA tiles per wave along m
+  constexpr int NWAVES = WM * 4;
+  constexpr int A_REG = 32 / NWAVES;     // 1 KiB direct-to-LDS regions per wave per A slice
+  constexpr int B_REG = 16 / NWAVES;     // ... per B stage
+  constexpr int kSteadyVm = 2 * B_REG + A_REG;  // loads younger than what the next stage needs
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int wm = wave >> 2, wn = wave & 3;
+  const int KT = K / kBK;   // B stages; even, the launcher requires K % 64 == 0
+  const int KT2 = KT >> 1;  // A slices
+
+  // ---- per-lane operand read addresses, relative to a ring slot ----
+  const int lrow = lane & 31, lk = lane >> 5;
+  // substep ks (0..3) of the slice reads chunk 2*ks + lk:  a_rd ^ (ks * 32)
+  const uint32_t a_rd =
+      (uint32_t)((wm * TMW * 32 + lrow) * 128 + (lk ^ ((lrow >> 1) & 7)) * 16);
+  const int g = lane >> 4, li = lane & 15;
+  uint32_t b_rd[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int ntile = wn * 2 + j;
+    const int c16 = ntile * 4 + (g & 1) * 2 + ((li & 3) >> 1);
+    const int phys = c16 ^ ((li >> 2) << 2);
+    b_rd[j] = (uint32_t)(kRingB + ((g >> 1) * 8 + (li >> 2)) * 512 + phys * 16 + (li & 1) * 8);
+  }
+
+  for (int p = blockIdx.x; p < tiles_m * tiles_n; p += gridDim.x) {
+    int tile_m, tile_n;
+    map_tile_dma(p, tiles_m, tiles_n, tile_m, tile_n);
+    const int m0 = tile_m * kBM, n0 = tile_n * kBN;
+
+    // K-stagger: this tile walks stages kfirst, kfirst+1, ..., wrapping at KT.
+    // kfirst is even so that A slices (two stages) stay aligned.
+    const int kfirst =
+        (int)(((unsigned)(tile_m * AFIR_MM_KSTAGGER_M + tile_n * AFIR_MM_KSTAGGER_N) * 2u) %
+              (unsigned)KT);
+
+    // ---- per-lane global sources of the direct-to-LDS loads ----
+    // A slice: 32 regions of 1 KiB (8 rows x 128 B), A_REG per wave.
+    // B stage: 16 regions of 1 KiB (2 rows x 512 B), B_REG per wave.
+    const uint16_t *ga[A_REG], *gb[B_REG];
+#pragma unroll
+    for (int q = 0; q < A_REG; ++q) {
+      const int arow = (wave * A_REG + q) * 8 + (lane >> 3);
+      const int ac = (lane & 7) ^ ((arow >> 1) & 7);
+      ga[q] = A + (int64_t)(m0 + arow) * K + ac * 8 + (int64_t)kfirst * kBK;
+    }
+#pragma unroll
+    for (int q = 0; q < B_REG; ++q) {
+      const int bk = (wave * B_REG + q) * 2 + (lane >> 5);
+      const int bc = (lane & 31) ^ ((bk & 3) << 2);
+      gb[q] = B + (int64_t)(bk + kfirst * kBK) * N + n0 + bc * 8;
+    }
+    int ka_next = kfirst >> 1;  // slice (64 k) the next A issue fetches
+    int kb_next = kfirst;       // stage (32 k) the next B issue fetches
+
+    auto issue_a = [&](int slot) {
+      lds_byte *dst = lds + slot * kSlotA + wave * (A_REG * 1024);
+#pragma unroll
+      for (int q = 0; q < A_REG; ++q)
+        __builtin_amdgcn_global_load_lds((gbl_void *)ga[q], (lds_void *)(dst + q * 1024), 16, 0, 0);
+      ka_next = (ka_next + 1 == KT2) ? 0 : ka_next + 1;
+      const int64_t step = (ka_next == 0) ? -(int64_t)(KT2 - 1) * 64 : (int64_t)64;
+#pragma unroll
+      for (int q = 0; q < A_REG; ++q) ga[q] += step;
+    };
+    auto issue_b = [&](int slot) {
+      lds_byte *dst = lds + kRingB + slot * kSlotB + wave * (B_REG * 1024);
+#pragma unroll
+      for (int q = 0; q < B_REG; ++q)
+        __builtin_amdgcn_global_load_lds((gbl_void *)gb[q], (lds_void *)(dst + q * 1024), 16, 0, 0);
+      kb_next = (kb_next + 1 == KT) ? 0 : kb_next + 1;
+      const int64_t step = (kb_next == 0) ? -(int64_t)(KT - 1) * kBK * N : (int64_t)kBK * N;
+#pragma unroll
+      for (int q = 0; q < B_REG; ++q) gb[q] += step;
+    };
+
+    f32x16 acc[TMW][2];
+#pragma unroll
+    for (int i = 0; i < TMW; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+
+    auto multiply = [&](const Operands<TMW> &o) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const u32x4 bw = {o.b[j][0].x, o.b[j][0].y, o.b[j][1].x, o.b[j][1].y};
+#pragma unroll
+        for (int i = 0; i < TMW; ++i)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+              __builtin_bit_cast(bf16x8, bw), __builtin_bit_cast(bf16x8, o.a[i]), acc[i][j], 0, 0,
+              0);
+      }
+    };
+    // operand reads for a stage held in A slot sa / B slot sbk; the stage is the
+    // first (par 0) or second (par 1) half of its A slice; h = k16 substep
+    auto reads = [&](int sa, int sbk, int par, int h, Operands<TMW> &o) {
+      const uint32_t aa =
+          lds_base + (uint32_t)(sa * kSlotA) + (a_rd ^ (uint32_t)((par * 2 + h) * 32));
+      const uint32_t bb = lds_base + (uint32_t)(sbk * kSlotB);
+      if (h == 0)
+        issue_reads<0>(aa, bb + b_rd[0], bb + b_rd[1], o);
+      else
+        issue_reads<1>(aa, bb + b_rd[0], bb + b_rd[1], o);
+    };
+
+    // prologue (the launcher guarantees KT >= 8): fill both rings, oldest first
+    issue_a(0);
+    issue_b(0);
+    issue_b(1);
+    issue_a(1);
+    issue_b(2);
+    issue_b(3);
+    issue_a(2);
+    wait_vmcnt<3 * B_REG + 2 * A_REG>();  // everything younger than A(0), B(0)
+    __builtin_amdgcn_s_barrier();
+    Operands<TMW> even, odd;
+    reads(0, 0, 0, 0, even);
+    settle_reads(even);
+
+    // One step of the pipeline for stage s of parity PAR:
+    //   reads(s, substep 1) in flight | MFMAs(s, substep 0)
+    //   wait until stage s+1 has landed, barrier: everyone is done reading s
+    //   reads(s+1, substep 0) in flight, refill the freed slots | MFMAs(s, substep 1)
+    // Refill after stage s: B(s+4) into s's B slot; after an odd s also the A
+    // slice (s+5)/2 into the slot of the slice just finished.  In the steady
+    // state both exist and the vmcnt is exact: younger than what stage s+1 needs
+    // are exactly 2 B stages and 1 A slice.  Otherwise drain.
+    int sa = 0, sb = 0;  // ring slots of the stage being multiplied
+    auto step = [&](auto par_tag, auto mode_tag, bool has_next, bool refill_b, bool refill_a) {
+      constexpr int PAR = decltype(par_tag)::value;
+      constexpr bool STEADY = decltype(mode_tag)::value;
+      const int sb_next = (sb + 1 == kBSlots) ? 0 : sb + 1;
+      const int sa_next = PAR ? ((sa + 1 == kASlots) ? 0 : sa + 1) : sa;
+      reads(sa, sb, PAR, 1, odd);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(even);
+      __builtin_amdgcn_sched_barrier(0);
+      settle_reads(odd);
+      if (STEADY || has_next) {
+        if (STEADY)
+          wait_vmcnt<kSteadyVm>();
+        else
+          wait_vmcnt<0>();
+        __builtin_amdgcn_s_barrier();
+        reads(sa_next, sb_next, PAR ^ 1, 0, even);
+        if (PAR && (STEADY || refill_a)) issue_a(sa);
+        if (STEADY || refill_b) issue_b(sb);
+      }
+      multiply(odd);
+      __builtin_amdgcn_sched_barrier(0);
+      if (STEADY || has_next) settle_reads(even);
+      sa = sa_next;
+      sb = sb_next;
+    };
+
+    int s = 0;
+    for (; s + 6 < KT; s += 2) {  // both refills exist: B(s+4), B(s+5), A((s+6)/2)
+      step(Par0{}, Steady{}, true, true, true);
+      step(Par1{}, Steady{}, true, true, true);
+    }
+    for (; s < KT; s += 2) {
+      step(Par0{}, Drain{}, true, s + 4 < KT, false);
+      step(Par1{}, Drain{}, s + 2 < KT, s + 5 < KT, s + 6 < KT);
+    }
+
+    // epilogue: lane holds m = lane%32, n = 8q + 4*(lane/32) + e
+    const int lm = lane & 31, lq = lane >> 5;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + (wn * 2 + j) * 32 + 8 * q + 4 * lq;
+        const u32x2 braw = *reinterpret_cast<const u32x2 *>(bias + n);
+        const float b0 = bf16_lo(braw.x), b1 = bf16_hi(braw.x);
+        const float b2 = bf16_lo(braw.y), b3 = bf16_hi(braw.y);
+#pragma unroll
+        for (int i = 0; i < TMW; ++i) {
+          const int m = m0 + (wm * TMW + i) * 32 + lm;
+          float v0 = acc[i][j][4 * q + 0] + b0;
+          float v1 = acc[i][j][4 * q + 1] + b1;
+          float v2 = acc[i][j][4 * q + 2] + b2;
+          float v3 = acc[i][j][4 * q + 3] + b3;
+          v0 = fmaxf(v0, v0 * alpha);
+          v1 = fmaxf(v1, v1 * alpha);
+          v2 = fmaxf(v2, v2 * alpha);
+          v3 = fmaxf(v3, v3 * alpha);
+          u32x2 w;
+          w.x = pack_bf16(v0, v1);
+          w.y = pack_bf16(v2, v3);
+          *reinterpret_cast<u32x2 *>(out + (int64_t)m * N + n) = w;
+        }
+      }
+    }
+    // every wave must be done reading the rings before the next tile refills them
+    __builtin_amdgcn_s_barrier();
+  }
+}
+
+}  // namespace
+
+bool matmul_dma_supported(int64_t m, int64_t k, int64_t n) {
+  return m % kBM == 0 && n % kBN == 0 && k % 64 == 0 && k >= 8 * kBK;
+}
+
+#ifndef AFIR_MM_WAVES_M
+#define AFIR_MM_WAVES_M 2
+#endif
+
+LaunchStatus launch_matmul_dma(const uint16_t *a, const uint16_t *b, const uint16_t *bias,
+                               uint16_t *out, int m, int k, int n, float alpha,
+                               uint32_t block_dim, hipStream_t stream) {
+  constexpr int WM = AFIR_MM_WAVES_M;
+  auto kernel = matmul_bias_leakyrelu_bf16_dma<WM>;
+  static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                                               kLdsBytes);
+  if (attr != hipSuccess) return LaunchStatus{2u, hipGetErrorString(attr)};
+  const int tiles_m = m / kBM, tiles_n = n / kBN;
+  int64_t blocks = (int64_t)tiles_m * tiles_n;
+  if (block_dim) blocks = block_dim;
+  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(WM * 4 * 64), kLdsBytes, stream, a, b,
+                     bias, out, m, k, n, alpha, tiles_m, tiles_n);
+  return after_launch();
+}
+
+}  // namespace afir

@@ -17,9 +17,50 @@ namespace afir {
 
 namespace {
 
-constexpr int kThreads = 256;
+#ifndef AFIR_ROWSUM_THREADS
+#define AFIR_ROWSUM_THREADS 512
+#endif
+#ifndef AFIR_ROWSUM_UNROLL
+#define AFIR_ROWSUM_UNROLL 8
+#endif
+#ifndef AFIR_ROWSUM_WAVES_PER_CU
+#define AFIR_ROWSUM_WAVES_PER_CU 16
+#endif
+constexpr int kThreads = AFIR_ROWSUM_THREADS;
 constexpr int kWavesPerBlock = kThreads / kWave;
-constexpr int kUnroll = 8;
+constexpr int kUnroll = AFIR_ROWSUM_UNROLL;
+constexpr int kWavesPerCU = AFIR_ROWSUM_WAVES_PER_CU;
+
+// Rows of at most 64*CH 128-bit chunks: the wave keeps its CH chunks of bias
+// in registers for all the rows it walks, and has a whole row in flight.
+template <int CH>
+__global__ __launch_bounds__(kThreads) void bcast_add_rowsum_f32_resident(
+    const float *__restrict__ x, const float *__restrict__ bias, float *__restrict__ y,
+    int64_t m, int64_t n) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t wave = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
+  const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
+  const int n4 = (int)(n >> 2);
+  const f32x4 *b4 = reinterpret_cast<const f32x4 *>(bias);
+  const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+  f32x4 vb[CH];
+#pragma unroll
+  for (int u = 0; u < CH; ++u) vb[u] = (lane + u * kWave < n4) ? b4[lane + u * kWave] : zero;
+
+  for (int64_t row = wave; row < m; row += nwaves) {
+    const f32x4 *x4 = reinterpret_cast<const f32x4 *>(x + row * n);
+    f32x4 vx[CH];
+#pragma unroll
+    for (int u = 0; u < CH; ++u)
+      vx[u] = (lane + u * kWave < n4) ? load_nt(x4 + lane + u * kWave) : zero;
+    f32x4 acc = zero;
+#pragma unroll
+    for (int u = 0; u < CH; ++u) acc += vx[u] + vb[u];
+    float s = (acc.x + acc.y) + (acc.z + acc.w);
+    s = wave_sum(s);
+    if (lane == 0) y[row] = s;
+  }
+}
 
 __global__ __launch_bounds__(kThreads) void bcast_add_rowsum_f32_vec(
     const float *__restrict__ x, const float *__restrict__ bias, float *__restrict__ y,
@@ -82,7 +123,24 @@ LaunchStatus launch_broadcast_add_reducesum(const float *x, const float *bias, f
   if (block_dim) blocks = block_dim;
   if (blocks > 0x7fffffff) blocks = 0x7fffffff;
   const bool vec = n > 0 && (n % 4 == 0) && aligned16(x) && aligned16(bias);
-  if (vec) {
+  if (vec && n / 4 <= 16 * kWave) {
+    // persistent waves: each keeps its bias chunks resident and walks several rows
+    const int64_t n4 = n / 4;
+    int64_t pblocks = (int64_t)kNumCU * kWavesPerCU / kWavesPerBlock;
+    if (pblocks * kWavesPerBlock > m) pblocks = (m + kWavesPerBlock - 1) / kWavesPerBlock;
+    if (block_dim) pblocks = block_dim;
+    const dim3 grid((unsigned)pblocks), block(kThreads);
+    if (n4 <= 1 * kWave)
+      hipLaunchKernelGGL(bcast_add_rowsum_f32_resident<1>, grid, block, 0, stream, x, bias, y, m, n);
+    else if (n4 <= 2 * kWave)
+      hipLaunchKernelGGL(bcast_add_rowsum_f32_resident<2>, grid, block, 0, stream, x, bias, y, m, n);
+    else if (n4 <= 4 * kWave)
+      hipLaunchKernelGGL(bcast_add_rowsum_f32_resident<4>, grid, block, 0, stream, x, bias, y, m, n);
+    else if (n4 <= 8 * kWave)
+      hipLaunchKernelGGL(bcast_add_rowsum_f32_resident<8>, grid, block, 0, stream, x, bias, y, m, n);
+    else
+      hipLaunchKernelGGL(bcast_add_rowsum_f32_resident<16>, grid, block, 0, stream, x, bias, y, m, n);
+  } else if (vec) {
     hipLaunchKernelGGL(bcast_add_rowsum_f32_vec, dim3((unsigned)blocks), dim3(kThreads), 0,
                        stream, x, bias, y, m, n);
   } else {

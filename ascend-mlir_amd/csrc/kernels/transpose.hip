@@ -17,12 +17,21 @@
 // The LDS tile is 128 rows x 256 B with no padding; the 16-byte chunk column
 // is XOR-ed with (row/8)%16, which makes both the row-wise writes and the
 // block-column reads hit 16 distinct bank groups per 16 lanes.
+// The grid is persistent (a few workgroups per CU); each workgroup issues the
+// loads of its next tile before it stores the current one, so HBM reads and
+// writes overlap instead of alternating in phases.
 #include "kernels.h"
 
 namespace afir {
 
 namespace {
 
+#ifndef AFIR_TR_EXTRA_LDS
+#define AFIR_TR_EXTRA_LDS 0
+#endif
+#ifndef AFIR_TR_BLOCKS_PER_CU
+#define AFIR_TR_BLOCKS_PER_CU 5
+#endif
 constexpr int kThreads = 256;
 constexpr int kTile = 128;               // elements per tile edge
 constexpr int kChunksPerRow = kTile / 8;  // 16-byte chunks per LDS row
@@ -49,26 +58,38 @@ __global__ __launch_bounds__(kThreads) void relu_bcast_add_transpose_f16_tiled(
   const int iblk = t & 15;     // 8-row block (along M) in the store phase
   const int jblk = t >> 4;     // 8-col block (along N) in the store phase
 
-  for (int64_t tile_id = blockIdx.x; tile_id < ntiles; tile_id += gridDim.x) {
+  // Software pipeline over the tiles of this workgroup: the global loads of
+  // the next tile are issued before the current tile is read back from LDS and
+  // stored, so reads and writes to HBM overlap instead of alternating.
+  auto decode = [&](int64_t tile_id, int &b, int &m0, int &n0) {
     const int tn = (int)(tile_id % tiles_n);
     const int tm = (int)((tile_id / tiles_n) % tiles_m);
-    const int b = (int)(tile_id / ((int64_t)tiles_n * tiles_m));
-    const int m0 = tm * kTile, n0 = tn * kTile;
+    b = (int)(tile_id / ((int64_t)tiles_n * tiles_m));
+    m0 = tm * kTile;
+    n0 = tn * kTile;
+  };
+  u32x4 v[8], craw;
+  auto fetch = [&](int64_t tile_id) {
+    int b, m0, n0;
+    decode(tile_id, b, m0, n0);
+    craw = *reinterpret_cast<const u32x4 *>(c + n0 + cc * 8);
+    const uint16_t *xin = x + ((int64_t)b * m + m0) * n + n0 + cc * 8;
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      v[k] = load_nt(reinterpret_cast<const u32x4 *>(xin + (int64_t)(row0 + 16 * k) * n));
+  };
 
-    // this lane's eight values of c
-    u32x4 craw = *reinterpret_cast<const u32x4 *>(c + n0 + cc * 8);
+  int64_t tile_id = blockIdx.x;
+  if (tile_id < ntiles) fetch(tile_id);
+  for (; tile_id < ntiles; tile_id += gridDim.x) {
+    int b, m0, n0;
+    decode(tile_id, b, m0, n0);
     float cf[8];
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
       cf[2 * d] = f16_lo(craw[d]);
       cf[2 * d + 1] = f16_hi(craw[d]);
     }
-
-    const uint16_t *xin = x + ((int64_t)b * m + m0) * n + n0 + cc * 8;
-    u32x4 v[8];
-#pragma unroll
-    for (int k = 0; k < 8; ++k)
-      v[k] = load_nt(reinterpret_cast<const u32x4 *>(xin + (int64_t)(row0 + 16 * k) * n));
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
       const int row = row0 + 16 * k;
@@ -78,6 +99,7 @@ __global__ __launch_bounds__(kThreads) void relu_bcast_add_transpose_f16_tiled(
       tile[row * kChunksPerRow + (cc ^ ((row >> 3) & 15))] = r;
     }
     __syncthreads();
+    if (tile_id + gridDim.x < ntiles) fetch(tile_id + gridDim.x);
 
     u32x4 in[8];
 #pragma unroll
@@ -148,11 +170,13 @@ LaunchStatus launch_relu_broadcast_add_transpose(const uint16_t *x, const uint16
   int64_t tiles = tiled ? nb * (m / kTile) * (n / kTile)
                         : nb * ((m + 31) / 32) * ((n + 31) / 32);
   int64_t blocks = tiles;
+  if (AFIR_TR_BLOCKS_PER_CU && tiled && blocks > (int64_t)kNumCU * AFIR_TR_BLOCKS_PER_CU)
+    blocks = (int64_t)kNumCU * AFIR_TR_BLOCKS_PER_CU;
   if (block_dim) blocks = block_dim;
   if (blocks > 0x7fffffff) blocks = 0x7fffffff;
   if (tiled) {
     hipLaunchKernelGGL(relu_bcast_add_transpose_f16_tiled, dim3((unsigned)blocks), dim3(kThreads),
-                       0, stream, x, c, out, (int)nb, (int)m, (int)n);
+                       AFIR_TR_EXTRA_LDS, stream, x, c, out, (int)nb, (int)m, (int)n);
   } else {
     hipLaunchKernelGGL(relu_bcast_add_transpose_f16_any, dim3((unsigned)blocks), dim3(kThreads),
                        0, stream, x, c, out, (int)nb, (int)m, (int)n);
