@@ -67,8 +67,40 @@ def build_kernels():
     return out
 
 
+RUNTIME_SOURCES = ["runtime/support.cpp", "runtime/artifact.cpp", "runtime/session.cpp",
+                   "runtime/hip_runner.cpp", "capi/afirt_runtime.cpp"]
+HOST = ["-std=c++17", "-O2", "-fPIC", "-Wall", "-Wno-unused-result",
+        "-D__HIP_PLATFORM_AMD__", "-I", "/opt/rocm/include", "-I", os.path.join(ROOT, "include")]
+CXX = os.environ.get("CXX", "g++")
+
+
+def _compile_host(src):
+    obj = os.path.join(OBJ, "host_" + src.replace("/", "_") + ".o")
+    _run([CXX, *HOST, "-c", os.path.join(CSRC, src), "-o", obj])
+    return obj
+
+
+def build_runtime():
+    """libAFIRRuntimeCAPI.so (afirt_* C API + host runtime) and the
+    runtime-session CLI.  Host code only: compiled with g++ against the HIP
+    runtime API; the kernels are reached through dlopen of the kernel library."""
+    os.makedirs(LIB, exist_ok=True)
+    os.makedirs(OBJ, exist_ok=True)
+    os.makedirs(os.path.join(HERE, "bin"), exist_ok=True)
+    with cf.ThreadPoolExecutor(max_workers=6) as ex:
+        objs = list(ex.map(_compile_host, RUNTIME_SOURCES))
+    lib = os.path.join(LIB, "libAFIRRuntimeCAPI.so")
+    _run([CXX, "-shared", "-fPIC", "-o", lib, *objs, "-L/opt/rocm/lib", "-lamdhip64", "-ldl",
+          "-Wl,-rpath,/opt/rocm/lib"])
+    main_obj = _compile_host("tools/runtime_session_main.cpp")
+    exe = os.path.join(HERE, "bin", "runtime-session")
+    _run([CXX, "-o", exe, main_obj, "-L" + LIB, "-lAFIRRuntimeCAPI", "-L/opt/rocm/lib",
+          "-lamdhip64", "-ldl", "-Wl,-rpath,$ORIGIN/../lib", "-Wl,-rpath,/opt/rocm/lib"])
+    return [lib, exe]
+
+
 def build_all():
-    return [build_kernels()]
+    return [build_kernels(), *build_runtime()]
 
 
 if __name__ == "__main__":

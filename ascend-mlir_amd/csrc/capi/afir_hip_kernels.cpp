@@ -137,6 +137,47 @@ const AfirHipKernelInfo *afir_hip_find_kernel(const char *name) {
   return nullptr;
 }
 
+uint32_t afir_hip_argument_bytes(const char *kernel_name, const void *tiling, size_t tiling_len,
+                                 size_t *bytes, int max_args) {
+  const AfirHipKernelInfo *info = afir_hip_find_kernel(kernel_name);
+  if (!info)
+    return fail(AFIR_HIP_E_UNKNOWN,
+                std::string("no fused kernel named '") + (kernel_name ? kernel_name : "") + "'");
+  const int nargs = info->num_inputs + info->num_outputs;
+  if (!bytes || max_args < nargs) return fail(AFIR_HIP_E_INVALID, "argument_bytes: output array too small");
+  const size_t want_len = sizeof(int64_t) * (size_t)info->num_tiling_fields;
+  if (!tiling || tiling_len != want_len) {
+    char buf[160];
+    std::snprintf(buf, sizeof buf, "%s: tiling data must be %zu bytes (%d int64 fields), got %zu",
+                  info->name, want_len, info->num_tiling_fields, tiling_len);
+    return fail(AFIR_HIP_E_INVALID, buf);
+  }
+  int64_t f[4] = {0, 0, 0, 0};
+  std::memcpy(f, tiling, want_len);
+  const int dims = info->num_tiling_fields - ((info - kKernels) == 4 ? 1 : 0);
+  for (int i = 0; i < dims; ++i)
+    if (f[i] < 0 || f[i] > (int64_t)1 << 40)
+      return fail(AFIR_HIP_E_INVALID, std::string(info->name) + ": extent out of range in tiling data");
+  auto sz = [](int64_t a, int64_t b, int64_t c, int64_t elem) {
+    return (size_t)((unsigned __int128)a * (unsigned __int128)b * (unsigned __int128)c * (unsigned __int128)elem);
+  };
+  switch ((int)(info - kKernels)) {
+    case 0: bytes[0] = bytes[1] = bytes[2] = sz(f[0], f[1], 1, 4); break;
+    case 1: bytes[0] = sz(f[0], f[1], 1, 4); bytes[1] = sz(f[1], 1, 1, 4); bytes[2] = sz(f[0], 1, 1, 4); break;
+    case 2: bytes[0] = bytes[2] = sz(f[0], f[1], f[2], 2); bytes[1] = sz(f[2], 1, 1, 2); break;
+    case 3:
+      bytes[0] = sz(f[0], f[1], 1, 2); bytes[1] = sz(f[2], 1, 1, 4);
+      bytes[2] = bytes[3] = sz(f[1], 1, 1, 2); bytes[4] = sz(f[2], f[1], 1, 2);
+      break;
+    case 4:
+      bytes[0] = sz(f[0], f[1], 1, 2); bytes[1] = sz(f[1], f[2], 1, 2);
+      bytes[2] = sz(f[2], 1, 1, 2); bytes[3] = sz(f[0], f[2], 1, 2);
+      break;
+  }
+  g_last_error.clear();
+  return AFIR_HIP_OK;
+}
+
 uint32_t afir_hip_launch(const char *kernel_name, uint32_t block_dim, void *stream, int num_args,
                          void *const *args, void *workspace, const void *tiling,
                          size_t tiling_len) {

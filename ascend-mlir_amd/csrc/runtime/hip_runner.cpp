@@ -1,0 +1,258 @@
+// The MI355X execution runner and the single-task session.
+//
+// Runner sequence (shape of the reference's NativeExecutionRunner::runWithHandle
+// and ::runDynamicLibraryArtifact, lib/Runtime/Execution/NativeExecutionRunner.cpp:
+// 372-528, 616-802): allocate inputs / outputs / workspace on the device, copy
+// the inputs in, call the artifact's launcher symbol with
+// [inputs..., outputs..., workspace, tiling] in sixteen pointer slots, wait for
+// the stream, copy the outputs back, free.  The tiling pointer handed to the
+// launcher is the host copy: HIP kernels take their arguments by value.
+//
+// Before anything is launched the caller's byte counts are checked against the
+// sizes the tiling implies (afir_hip_argument_bytes), because the C API above
+// carries no shapes and a short buffer would otherwise be read past its end on
+// the device.
+#include <dlfcn.h>
+#include <hip/hip_runtime.h>
+
+#include <chrono>
+#include <cstring>
+
+#include "runtime.h"
+
+namespace afirt {
+
+namespace {
+
+struct KernelInfoView {  // layout of AfirHipKernelInfo (include/afir_hip_kernels.h)
+  const char *name;
+  const char *symbol;
+  int num_inputs;
+  int num_outputs;
+  int num_tiling_fields;
+  const char *const *tiling_fields;
+  const char *signature;
+};
+
+using LaunchFn16 = uint32_t (*)(uint32_t, void *, void *, void *, void *, void *, void *, void *,
+                                void *, void *, void *, void *, void *, void *, void *, void *,
+                                void *, void *);
+using LastErrorFn = const char *(*)();
+using KernelCountFn = int (*)();
+using KernelInfoFn = const KernelInfoView *(*)(int);
+using ArgBytesFn = uint32_t (*)(const char *, const void *, size_t, size_t *, int);
+
+std::string hipErr(const char *what, hipError_t e) {
+  return std::string(what) + " failed: " + hipGetErrorString(e);
+}
+
+class HipExecutionRunner final : public ExecutionRunner {
+ public:
+  ~HipExecutionRunner() override {
+    if (stream_) (void)hipStreamDestroy(stream_);
+    if (ev0_) (void)hipEventDestroy(ev0_);
+    if (ev1_) (void)hipEventDestroy(ev1_);
+  }
+
+  ExecutionRunnerMode mode() const override { return ExecutionRunnerMode::RealDevice; }
+
+  Status initialize(int deviceId) override {
+    if (deviceId < 0) return Status::error("device id must be non-negative");
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess) return Status::error(hipErr("hipGetDeviceCount", e));
+    if (deviceId >= count)
+      return Status::error(format("device %d is not present (%d HIP device(s) visible)", deviceId, count));
+    e = hipSetDevice(deviceId);
+    if (e != hipSuccess) return Status::error(hipErr("hipSetDevice", e));
+    if (!stream_) {
+      e = hipStreamCreate(&stream_);  // default priority
+      if (e != hipSuccess) return Status::error(hipErr("hipStreamCreate", e));
+      e = hipEventCreate(&ev0_);
+      if (e == hipSuccess) e = hipEventCreate(&ev1_);
+      if (e != hipSuccess) return Status::error(hipErr("hipEventCreate", e));
+    }
+    deviceId_ = deviceId;
+    initialized_ = true;
+    return Status::success();
+  }
+
+  Status runFile(const FileExecutionLaunch &launch, RunArgs &args) override {
+    if (launch.magic != kMagicAIVec && launch.magic != kMagicAICube)
+      return Status::error(format("unsupported kernel magic: 0x%08x", launch.magic));
+    auto text = readTextFile(launch.binaryPath);
+    if (!text) return Status::error("cannot open " + launch.binaryPath);
+    auto d = parseDescriptor(*text);
+    if (!d) return Status::error(d.error());
+    DynamicLibraryExecutionLaunch dl;
+    dl.sharedLibraryPath = d->library.empty() ? defaultKernelLibraryPath() : d->library;
+    dl.symbolName = d->symbol;
+    return runDynamicLibraryArtifact(dl, args);
+  }
+
+  Status runDynamicLibraryArtifact(const DynamicLibraryExecutionLaunch &launch,
+                                   RunArgs &args) override {
+    lastKernelUs_ = -1.0;
+    if (!initialized_) return Status::error("execution runner has not been initialized");
+    if (args.inputs.size() + args.outputs.size() + 2 > 16)
+      return Status::error("too many tensor arguments for a launcher call (16 pointer slots)");
+
+    void *lib = dlopen(launch.sharedLibraryPath.c_str(), RTLD_NOW | RTLD_LOCAL);
+    if (!lib)
+      return Status::error("dlopen dynamic library artifact failed (" + launch.sharedLibraryPath +
+                           "): " + dlerror());
+    struct LibGuard {
+      void *h;
+      ~LibGuard() { dlclose(h); }
+    } libGuard{lib};
+
+    auto launchFn = reinterpret_cast<LaunchFn16>(dlsym(lib, launch.symbolName.c_str()));
+    if (!launchFn) {
+      const char *err = dlerror();
+      return Status::error("dlsym " + launch.symbolName + " failed: " + (err ? err : "unknown"));
+    }
+    auto lastError = reinterpret_cast<LastErrorFn>(dlsym(lib, "afir_hip_last_error"));
+
+    // ---- host-side validation against the shapes in the tiling bytes ----
+    if (Status st = validate(lib, launch.symbolName, args); !st.ok()) return st;
+
+    // ---- device buffers ----
+    std::vector<void *> allocs;
+    auto cleanup = [&]() {
+      for (auto it = allocs.rbegin(); it != allocs.rend(); ++it)
+        if (*it) (void)hipFree(*it);
+      allocs.clear();
+    };
+    auto devAlloc = [&](size_t bytes, void **out) -> hipError_t {
+      // an empty tensor still gets a valid, distinct pointer
+      hipError_t e = hipMalloc(out, bytes ? bytes : 16);
+      if (e == hipSuccess) allocs.push_back(*out);
+      return e;
+    };
+
+    void *slots[16] = {};
+    size_t idx = 0;
+    std::vector<void *> outDev;
+    for (auto &in : args.inputs) {
+      void *dev = nullptr;
+      hipError_t e = devAlloc(in.nbytes(), &dev);
+      if (e != hipSuccess) { cleanup(); return Status::error(hipErr("hipMalloc input", e)); }
+      if (in.nbytes()) {
+        e = hipMemcpyAsync(dev, in.data, in.nbytes(), hipMemcpyHostToDevice, stream_);
+        if (e != hipSuccess) { cleanup(); return Status::error(hipErr("hipMemcpy input", e)); }
+      }
+      slots[idx++] = dev;
+    }
+    for (auto &out : args.outputs) {
+      void *dev = nullptr;
+      hipError_t e = devAlloc(out.nbytes(), &dev);
+      if (e != hipSuccess) { cleanup(); return Status::error(hipErr("hipMalloc output", e)); }
+      outDev.push_back(dev);
+      slots[idx++] = dev;
+    }
+    void *workspace = nullptr;
+    {
+      const size_t ws = args.workspace_size < 16 ? 16 : args.workspace_size;
+      hipError_t e = devAlloc(ws, &workspace);
+      if (e != hipSuccess) { cleanup(); return Status::error(hipErr("hipMalloc workspace", e)); }
+      e = hipMemsetAsync(workspace, 0, 16, stream_);  // error flag words start at zero
+      if (e != hipSuccess) { cleanup(); return Status::error(hipErr("hipMemset workspace", e)); }
+    }
+    slots[idx++] = workspace;
+    slots[idx++] = args.tiling.empty() ? nullptr : args.tiling.data();
+
+    // ---- launch ----
+    (void)hipEventRecord(ev0_, stream_);
+    const uint32_t rc = launchFn((uint32_t)(args.block_dim < 0 ? 0 : args.block_dim), stream_,
+                                 slots[0], slots[1], slots[2], slots[3], slots[4], slots[5],
+                                 slots[6], slots[7], slots[8], slots[9], slots[10], slots[11],
+                                 slots[12], slots[13], slots[14], slots[15]);
+    if (rc != 0) {
+      std::string why = lastError ? lastError() : "";
+      (void)hipStreamSynchronize(stream_);
+      cleanup();
+      return Status::error(format("dynamic library artifact launch failed: rc=%u", rc) +
+                           (why.empty() ? "" : " (" + why + ")"));
+    }
+    (void)hipEventRecord(ev1_, stream_);
+    hipError_t e = hipStreamSynchronize(stream_);
+    if (e != hipSuccess) { cleanup(); return Status::error(hipErr("hipStreamSynchronize", e)); }
+    float ms = 0.f;
+    if (hipEventElapsedTime(&ms, ev0_, ev1_) == hipSuccess) lastKernelUs_ = (double)ms * 1e3;
+
+    // ---- data errors reported through the workspace ----
+    int32_t flag = 0;
+    e = hipMemcpy(&flag, workspace, sizeof flag, hipMemcpyDeviceToHost);
+    if (e != hipSuccess) { cleanup(); return Status::error(hipErr("hipMemcpy workspace", e)); }
+    if (flag != 0) {
+      cleanup();
+      return Status::error("kernel reported a data error: index out of range in gather");
+    }
+
+    for (size_t i = 0; i < args.outputs.size(); ++i) {
+      if (!args.outputs[i].nbytes()) continue;
+      e = hipMemcpy(args.outputs[i].data, outDev[i], args.outputs[i].nbytes(), hipMemcpyDeviceToHost);
+      if (e != hipSuccess) { cleanup(); return Status::error(hipErr("hipMemcpy output", e)); }
+    }
+    cleanup();
+    return Status::success();
+  }
+
+  double lastKernelMicroseconds() const override { return lastKernelUs_; }
+
+ private:
+  Status validate(void *lib, const std::string &symbol, const RunArgs &args) {
+    auto countFn = reinterpret_cast<KernelCountFn>(dlsym(lib, "afir_hip_kernel_count"));
+    auto infoFn = reinterpret_cast<KernelInfoFn>(dlsym(lib, "afir_hip_kernel_info"));
+    auto bytesFn = reinterpret_cast<ArgBytesFn>(dlsym(lib, "afir_hip_argument_bytes"));
+    auto lastError = reinterpret_cast<LastErrorFn>(dlsym(lib, "afir_hip_last_error"));
+    if (!countFn || !infoFn || !bytesFn)
+      return Status::error("library exports no kernel registry (afir_hip_kernel_info): cannot "
+                           "validate buffers for " + symbol);
+    const KernelInfoView *info = nullptr;
+    for (int i = 0; i < countFn(); ++i) {
+      const KernelInfoView *k = infoFn(i);
+      if (k && symbol == k->symbol) info = k;
+    }
+    if (!info) return Status::error("launcher symbol is not in the kernel registry: " + symbol);
+    if ((int)args.inputs.size() != info->num_inputs)
+      return Status::error(format("%s expects %d inputs, got %zu", info->name, info->num_inputs,
+                                  args.inputs.size()));
+    if ((int)args.outputs.size() != info->num_outputs)
+      return Status::error(format("%s expects %d outputs, got %zu", info->name, info->num_outputs,
+                                  args.outputs.size()));
+    size_t want[16] = {};
+    if (bytesFn(info->name, args.tiling.data(), args.tiling.size(), want, 16) != 0)
+      return Status::error(std::string("invalid tiling data: ") + (lastError ? lastError() : ""));
+    for (size_t i = 0; i < args.inputs.size(); ++i) {
+      if (args.inputs[i].nbytes() != want[i])
+        return Status::error(format("%s: input %zu holds %zu bytes, the tiling data implies %zu",
+                                    info->name, i, args.inputs[i].nbytes(), want[i]));
+      if (want[i] && !args.inputs[i].data)
+        return Status::error(format("%s: input %zu has no data", info->name, i));
+    }
+    for (size_t i = 0; i < args.outputs.size(); ++i) {
+      const size_t w = want[args.inputs.size() + i];
+      if (args.outputs[i].nbytes() != w)
+        return Status::error(format("%s: output %zu holds %zu bytes, the tiling data implies %zu",
+                                    info->name, i, args.outputs[i].nbytes(), w));
+      if (w && !args.outputs[i].data)
+        return Status::error(format("%s: output %zu has no buffer", info->name, i));
+    }
+    return Status::success();
+  }
+
+  bool initialized_ = false;
+  int deviceId_ = 0;
+  hipStream_t stream_ = nullptr;
+  hipEvent_t ev0_ = nullptr, ev1_ = nullptr;
+  double lastKernelUs_ = -1.0;
+};
+
+}  // namespace
+
+std::unique_ptr<ExecutionRunner> createHipExecutionRunner() {
+  return std::make_unique<HipExecutionRunner>();
+}
+
+}  // namespace afirt

@@ -37,6 +37,7 @@ EXPORTED_SYMBOLS = [
     "afir_hip_kernel_info",
     "afir_hip_find_kernel",
     "afir_hip_launch",
+    "afir_hip_argument_bytes",
 ]
 
 _lib = None

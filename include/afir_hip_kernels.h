@@ -139,6 +139,14 @@ int afir_hip_kernel_count(void);
 const AfirHipKernelInfo *afir_hip_kernel_info(int index);
 const AfirHipKernelInfo *afir_hip_find_kernel(const char *name);
 
+/* Byte sizes of the tensor arguments [inputs..., outputs...] that a tiling
+ * implies, so that a runner can check the caller's buffers on the host before
+ * it launches (the C API above it carries byte counts but no shapes,
+ * lib/CAPI/Runtime/Runtime.cpp:122-134).  Writes num_inputs + num_outputs
+ * entries; max_args is the capacity of `bytes`. */
+uint32_t afir_hip_argument_bytes(const char *kernel_name, const void *tiling, size_t tiling_len,
+                                 size_t *bytes, int max_args);
+
 /* Launch by name.  args = [inputs..., outputs...] device pointers
  * (num_args must equal num_inputs + num_outputs of the kernel); tiling_len is
  * checked against 8 * num_tiling_fields. */

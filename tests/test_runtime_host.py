@@ -1,0 +1,251 @@
+"""Host-side runtime: formats, C API error behaviour, CLI contract.  CPU only."""
+import ctypes
+import json
+import os
+import re
+import struct
+import subprocess
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+PKG = os.path.join(ROOT, "ascend-mlir_amd")
+RS = os.path.join(PKG, "bin", "runtime-session")
+
+EXAMPLE_MLIR = """func.func @example(%arg0: tensor<4x4xf32>, %arg1: tensor<4x4xf32>) -> tensor<4x4xf32> {
+  %0 = afir.add %arg0, %arg1 : (tensor<4x4xf32>, tensor<4x4xf32>) -> tensor<4x4xf32>
+  %1 = afir.mul %0, %arg1 : (tensor<4x4xf32>, tensor<4x4xf32>) -> tensor<4x4xf32>
+  return %1 : tensor<4x4xf32>
+}
+"""
+
+
+def test_cpp_host_tests(tmp_path):
+    exe = tmp_path / "test_runtime_host"
+    src = [os.path.join(ROOT, "tests", "cpp", "test_runtime_host.cpp"),
+           os.path.join(PKG, "csrc", "runtime", "support.cpp"),
+           os.path.join(PKG, "csrc", "runtime", "artifact.cpp")]
+    subprocess.run(["g++", "-std=c++17", "-O1", "-Wall", "-I", os.path.join(PKG, "csrc", "runtime"),
+                    "-I", os.path.join(ROOT, "include"), *src, "-ldl", "-o", str(exe)], check=True)
+    work = tmp_path / "w"
+    work.mkdir()
+    p = subprocess.run([str(exe), str(work)], capture_output=True, text=True)
+    assert p.returncode == 0, p.stdout + p.stderr
+    assert " 0 failed" in p.stdout
+
+
+def _declared(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(afirt_[a-z_]+)\s*\(", text)))
+
+
+def test_capi_exports_every_declared_symbol(pkg):
+    from ascend_mlir_amd.runtime import capi
+    L = capi.load_capi()
+    names = _declared("afirt_runtime.h")
+    assert sorted(capi.EXPORTED_SYMBOLS) == names
+    for n in names:
+        assert hasattr(L, n), n
+
+
+def test_capi_error_behaviour_without_gpu(pkg, tmp_path):
+    from ascend_mlir_amd.runtime import capi
+    L = capi.load_capi()
+    err = ctypes.create_string_buffer(256)
+    # null / uninitialised handles are errors, not crashes
+    assert L.afirt_executor_initialize(None, 0, err, len(err)) == 1
+    assert err.value == b"executor handle is null"
+    h = L.afirt_executor_create()
+    assert h
+    assert L.afirt_executor_initialize(h, -1, err, len(err)) == 1
+    assert err.value == b"device id must be non-negative"
+    vp, sz = ctypes.c_void_p, ctypes.c_size_t
+    ptrs, sizes = (vp * 1)(0), (sz * 1)(0)
+    rc = L.afirt_executor_run(h, None, 0, b"k", 0, ptrs, sizes, 1, ptrs, sizes, None, 0, 1,
+                              capi.MAGIC_ELF_AIVEC, err, len(err))
+    assert rc == 1 and err.value == b"executor has not been initialized"
+    rc = L.afirt_executor_run_file(h, b"/x", b"k", 0, ptrs, sizes, 1, ptrs, sizes, None, 0, 1,
+                                   capi.MAGIC_ELF_AIVEC, err, len(err))
+    assert rc == 1 and err.value == b"executor has not been initialized"
+    # message is truncated into the caller's buffer and NUL-terminated
+    small = ctypes.create_string_buffer(8)
+    assert L.afirt_executor_initialize(None, 0, small, len(small)) == 1
+    assert small.value == b"executo"
+    L.afirt_executor_destroy(h)
+    # compiler
+    buf = ctypes.create_string_buffer(512)
+    assert L.afirt_compiler_compile(None, b"a", b"b", b"c", buf, len(buf)) == 1
+    assert buf.value == b"compiler handle is null"
+    c = L.afirt_compiler_create(b"gfx950", b"gfx950-vec", 3)
+    assert L.afirt_compiler_compile(c, b"/no/such/file.mlir", str(tmp_path).encode(), b"k", buf,
+                                    len(buf)) == 1
+    assert b"cannot read kernel source" in buf.value
+    src = tmp_path / "example.mlir"
+    src.write_text(EXAMPLE_MLIR)
+    assert L.afirt_compiler_compile(c, str(src).encode(), str(tmp_path / "art").encode(), b"example",
+                                    buf, len(buf)) == 0
+    assert buf.value.decode().endswith("art/example.hipk")
+    assert os.path.exists(buf.value.decode())
+    bad = tmp_path / "bad.mlir"
+    bad.write_text("func.func @unknown_thing() { return }\n")
+    assert L.afirt_compiler_compile(c, str(bad).encode(), str(tmp_path / "art2").encode(), b"", buf,
+                                    len(buf)) == 1
+    assert b"cannot map kernel source" in buf.value
+    L.afirt_compiler_destroy(c)
+    L.afirt_compiler_destroy(None)
+    L.afirt_executor_destroy(None)
+
+
+def test_python_runtime_mirror(pkg, tmp_path):
+    from ascend_mlir_amd import runtime as R
+    src = tmp_path / "k.mlir"
+    src.write_text(EXAMPLE_MLIR)
+    path = R.compile_kernel(src, tmp_path / "art", "example")
+    text = R.read_binary(path).decode()
+    assert text.startswith("afir-hip-artifact 1\n") and "hip_kernel=fused_add_mul" in text
+    manifest = (tmp_path / "art" / "out" / "manifest.txt").read_text()
+    assert "kernel_name=example" in manifest and "kernel_so_symbol=afir_hip_launch_fused_add_mul" in manifest
+    with pytest.raises(R.CompilerError):
+        R.compile_kernel(tmp_path / "missing.mlir", tmp_path / "a2", "x")
+    ex = R.KernelExecutor()
+    with pytest.raises(R.ExecutorError):   # no device in this container
+        ex.initialize()
+
+
+# --- the reference's Python tiling-schema tests, restated --------------------
+
+@pytest.fixture()
+def schema_file(tmp_path):
+    p = tmp_path / "tiling_space.json"
+    p.write_text(json.dumps({"tiling_params": [
+        {"name": "TB_M", "type": "int64"}, {"name": "TB_N", "type": "int64"},
+        {"name": "M", "type": "int64"}, {"name": "N", "type": "int32"}]}))
+    return p
+
+
+def test_tiling_schema_python(pkg, schema_file, tmp_path):
+    from ascend_mlir_amd.runtime import TilingSchema
+    s = TilingSchema.from_json(schema_file)
+    assert len(s) == 4 and s.field_names == ["TB_M", "TB_N", "M", "N"]
+    b = s.pack(TB_M=16, TB_N=4, M=64, N=64)
+    assert len(b) == 28 and struct.unpack("<qqqi", b) == (16, 4, 64, 64)
+    assert s.pack(N=64, M=64, TB_N=4, TB_M=16) == b          # keyword order is irrelevant
+    with pytest.raises(ValueError, match="missing tiling fields"):
+        s.pack(TB_M=16)
+    with pytest.raises(ValueError, match="unexpected tiling fields"):
+        s.pack(TB_M=16, TB_N=4, M=64, N=64, K=1)
+    with pytest.raises(FileNotFoundError):
+        TilingSchema.from_json(tmp_path / "none.json")
+    bad = tmp_path / "bad.json"
+    bad.write_text("{ nope")
+    with pytest.raises(ValueError, match="JSON parse error"):
+        TilingSchema.from_json(bad)
+    bad.write_text("{}")
+    with pytest.raises(ValueError, match="missing 'tiling_params'"):
+        TilingSchema.from_json(bad)
+    bad.write_text('{"tiling_params": [{"type": "int64"}]}')
+    with pytest.raises(ValueError, match="missing 'name'"):
+        TilingSchema.from_json(bad)
+    assert TilingSchema.for_kernel("matmul_add_leakyrelu").field_names == [
+        "dim_arg0_0", "dim_arg0_1", "dim_arg1_1", "alpha_f32_bits"]
+
+
+# --- runtime-session CLI contract --------------------------------------------
+
+def _rs(*args, cwd=None):
+    return subprocess.run([RS, *args], capture_output=True, text=True, cwd=cwd)
+
+
+def _manifest(tmp_path, expected=True, **over):
+    a = np.arange(16, dtype=np.float32).reshape(4, 4)
+    np.save(tmp_path / "a.npy", a)
+    np.save(tmp_path / "b.npy", np.ones((4, 4), np.float32))
+    np.save(tmp_path / "exp.npy", np.zeros((4, 4), np.float32))
+    (tmp_path / "ts.json").write_text(json.dumps(
+        {"tiling_params": [{"name": "dim_arg0_0"}, {"name": "dim_arg0_1"}]}))
+    m = {"task_id": "main", "backend": "hip", "artifact_root": str(tmp_path / "art"),
+         "inputs": [{"name": "a", "path": str(tmp_path / "a.npy")},
+                    {"name": "b", "path": str(tmp_path / "b.npy")}],
+         "outputs": [{"name": "out", "path": str(tmp_path / "out.npy")}],
+         "tiling": {"schema": str(tmp_path / "ts.json"), "params": "dim_arg0_0=4,dim_arg0_1=4"},
+         "block_dim": 0, "atol": 0, "rtol": 0}
+    if expected:
+        m["expected_outputs"] = [{"name": "out", "path": str(tmp_path / "exp.npy")}]
+    else:
+        m["outputs"][0].update({"shape": [4, 4], "dtype": "f32"})
+    m.update(over)
+    (tmp_path / "m.json").write_text(json.dumps(m))
+    return str(tmp_path / "m.json")
+
+
+def test_cli_compile_plan_and_exit_codes(tmp_path):
+    src = tmp_path / "example.mlir"
+    src.write_text(EXAMPLE_MLIR)
+    p = _rs("--kernel", str(src), "--kernel-kind", "vec", "--output", str(tmp_path / "art"),
+            "--name", "example")
+    assert p.returncode == 0, p.stderr
+    out = p.stdout.splitlines()
+    assert "artifact.kernel_name=example" in out and f"artifact.root={tmp_path / 'art'}" in out
+    assert "artifact.soc=gfx950" in out and "session.plan.tasks=1" in out and "session.plan[0]=main" in out
+    assert _rs("--artifact-root", str(tmp_path / "art")).returncode == 0
+    assert _rs().returncode == 4
+    assert _rs("--kernel", str(src), "--artifact-root", str(tmp_path / "art")).returncode == 4
+    assert _rs("--kernel", str(src), "--kernel-kind", "weird", "--output", str(tmp_path / "x")).returncode == 4
+    assert _rs("--run-manifest", str(tmp_path / "none.json"), "--run").returncode == 4
+    assert _rs("--artifact-root", str(tmp_path / "nope")).returncode == 4
+    assert _rs("--bogus").returncode == 4
+
+
+def test_cli_run_with_testing_driver(tmp_path):
+    src = tmp_path / "example.mlir"
+    src.write_text(EXAMPLE_MLIR)
+    assert _rs("--kernel", str(src), "--output", str(tmp_path / "art"), "--name", "example").returncode == 0
+    m = _manifest(tmp_path)
+    p = _rs("--run-manifest", m, "--run", "--testing-driver=hip-success")
+    assert p.returncode == 0, p.stderr
+    lines = p.stdout.splitlines()
+    for want in ("session.backend=hip", "session.result=success", "session.validation=pass",
+                 "session.profile.count=0", "session.runtime.counter.tiling_bytes=16"):
+        assert want in lines, p.stdout
+    assert np.array_equal(np.load(tmp_path / "out.npy"), np.zeros((4, 4), np.float32))
+    # no expected outputs: no validation line, shapes come from the output binding
+    p = _rs("--run-manifest", _manifest(tmp_path, expected=False), "--run", "--testing-driver=hip-success")
+    assert p.returncode == 0 and "session.validation=pass" not in p.stdout
+    # validation failure: exit 2, stage 'validate', lines on stderr
+    m = _manifest(tmp_path)
+    np.save(tmp_path / "exp.npy", np.ones((4, 4), np.float32))
+    p = _rs("--run-manifest", m, "--run", "--testing-driver=hip-success")
+    assert p.returncode == 2
+    err = p.stderr.splitlines()
+    assert "session.result=error" in err and "session.validation=fail" in err
+    assert "session.error_stage=validate" in err
+    assert any(l.startswith("Error: [hip:validate] output comparison failed") for l in err)
+
+
+def test_cli_error_stages(tmp_path):
+    src = tmp_path / "example.mlir"
+    src.write_text(EXAMPLE_MLIR)
+    assert _rs("--kernel", str(src), "--output", str(tmp_path / "art"), "--name", "example").returncode == 0
+    # without a GPU the real runner fails at executor_initialize, and says so
+    p = _rs("--run-manifest", _manifest(tmp_path), "--run")
+    assert p.returncode == 2
+    assert "session.error_stage=executor_initialize" in p.stderr.splitlines()
+    # missing input file -> bindings
+    m = _manifest(tmp_path, inputs=[{"name": "a", "path": str(tmp_path / "gone.npy")}])
+    p = _rs("--run-manifest", m, "--run", "--testing-driver=hip-success")
+    assert p.returncode == 2 and "session.error_stage=bindings" in p.stderr
+    # tiling params that do not match the schema -> bindings
+    m = _manifest(tmp_path, tiling={"schema": str(tmp_path / "ts.json"), "params": "dim_arg0_0=4"})
+    p = _rs("--run-manifest", m, "--run", "--testing-driver=hip-success")
+    assert p.returncode == 2 and "missing field" in p.stderr
+    # bad artifact root -> artifact
+    m = _manifest(tmp_path, artifact_root=str(tmp_path / "nowhere"))
+    p = _rs("--run-manifest", m, "--run", "--testing-driver=hip-success")
+    assert p.returncode == 2 and "session.error_stage=artifact" in p.stderr
+    # a manifest written for the reference's simulator still runs, and says what it asked for
+    m = _manifest(tmp_path, backend="sim")
+    np.save(tmp_path / "exp.npy", np.zeros((4, 4), np.float32))
+    p = _rs("--run-manifest", m, "--run", "--testing-driver=hip-success")
+    assert p.returncode == 0 and "session.backend_requested=sim" in p.stdout
