@@ -36,6 +36,7 @@ KERNEL_SOURCES = [
     ("kernels/gather.hip", STRICT),
     ("kernels/matmul.hip", []),
     ("kernels/matmul_dma.hip", []),
+    ("kernels/probe.hip", []),
     ("capi/afir_hip_kernels.cpp", []),
 ]
 

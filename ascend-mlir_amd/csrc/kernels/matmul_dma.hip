@@ -326,31 +326,58 @@ __global__ __launch_bounds__(WM * 4 * 64) void matmul_bias_leakyrelu_bf16_dma(
       step(Par1{}, Drain{}, s + 2 < KT, s + 5 < KT, s + 6 < KT);
     }
 
-    // epilogue: lane holds m = lane%32, n = 8q + 4*(lane/32) + e
-    const int lm = lane & 31, lq = lane >> 5;
+    // Epilogue.  A lane holds m = lane%32, n = 8q + 4*(lane/32) + e of each
+    // 32x32 block, i.e. 8 bytes of an output row per store: written straight
+    // to memory that is 16 bytes per row per instruction, and the partial
+    // lines cost three times the write traffic.  So each wave stages 32 rows
+    // of its tile (64 n = one 128-byte line per row) in LDS and stores them as
+    // full lines, eight rows per instruction.  The rings are free once every
+    // wave has left the K loop; a wave's 4 KiB staging area is private, and
+    // the LDS unit keeps a wave's accesses in order, so no further barrier is
+    // needed until the next tile refills the rings.  The 16-byte chunk column
+    // is XOR-ed with (row/2)%8: conflict-free for the 8-byte writes (32 rows
+    // x 2 halves) and for the 16-byte row reads.
+    __builtin_amdgcn_s_barrier();
+    {
+      unsigned char *const stage = smem + wave * 4096;
+      const int lm = lane & 31, lq = lane >> 5;
+      const int rr = lane >> 3, cc = lane & 7;
+      u32x2 braw[2][4];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < 2; ++j)
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int n = n0 + (wn * 2 + j) * 32 + 8 * q + 4 * lq;
-        const u32x2 braw = *reinterpret_cast<const u32x2 *>(bias + n);
-        const float b0 = bf16_lo(braw.x), b1 = bf16_hi(braw.x);
-        const float b2 = bf16_lo(braw.y), b3 = bf16_hi(braw.y);
+        for (int q = 0; q < 4; ++q)
+          braw[j][q] = *reinterpret_cast<const u32x2 *>(bias + n0 + (wn * 2 + j) * 32 + 8 * q + 4 * lq);
 #pragma unroll
-        for (int i = 0; i < TMW; ++i) {
-          const int m = m0 + (wm * TMW + i) * 32 + lm;
-          float v0 = acc[i][j][4 * q + 0] + b0;
-          float v1 = acc[i][j][4 * q + 1] + b1;
-          float v2 = acc[i][j][4 * q + 2] + b2;
-          float v3 = acc[i][j][4 * q + 3] + b3;
-          v0 = fmaxf(v0, v0 * alpha);
-          v1 = fmaxf(v1, v1 * alpha);
-          v2 = fmaxf(v2, v2 * alpha);
-          v3 = fmaxf(v3, v3 * alpha);
-          u32x2 w;
-          w.x = pack_bf16(v0, v1);
-          w.y = pack_bf16(v2, v3);
-          *reinterpret_cast<u32x2 *>(out + (int64_t)m * N + n) = w;
+      for (int i = 0; i < TMW; ++i) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const float b0 = bf16_lo(braw[j][q].x), b1 = bf16_hi(braw[j][q].x);
+            const float b2 = bf16_lo(braw[j][q].y), b3 = bf16_hi(braw[j][q].y);
+            float v0 = acc[i][j][4 * q + 0] + b0;
+            float v1 = acc[i][j][4 * q + 1] + b1;
+            float v2 = acc[i][j][4 * q + 2] + b2;
+            float v3 = acc[i][j][4 * q + 3] + b3;
+            v0 = fmaxf(v0, v0 * alpha);
+            v1 = fmaxf(v1, v1 * alpha);
+            v2 = fmaxf(v2, v2 * alpha);
+            v3 = fmaxf(v3, v3 * alpha);
+            u32x2 w;
+            w.x = pack_bf16(v0, v1);
+            w.y = pack_bf16(v2, v3);
+            const int chunk = (j * 4 + q) ^ ((lm >> 1) & 7);
+            *reinterpret_cast<u32x2 *>(stage + lm * 128 + chunk * 16 + lq * 8) = w;
+          }
+        }
+#pragma unroll
+        for (int tq = 0; tq < 4; ++tq) {
+          const int r = rr + 8 * tq;
+          const u32x4 line =
+              *reinterpret_cast<const u32x4 *>(stage + r * 128 + ((cc ^ ((r >> 1) & 7)) * 16));
+          const int m = m0 + (wm * TMW + i) * 32 + r;
+          *reinterpret_cast<u32x4 *>(out + (int64_t)m * N + n0 + wn * 64 + cc * 8) = line;
         }
       }
     }
@@ -368,6 +395,9 @@ bool matmul_dma_supported(int64_t m, int64_t k, int64_t n) {
 #ifndef AFIR_MM_WAVES_M
 #define AFIR_MM_WAVES_M 2
 #endif
+#ifndef AFIR_MM_GRID
+#define AFIR_MM_GRID kNumCU
+#endif
 
 LaunchStatus launch_matmul_dma(const uint16_t *a, const uint16_t *b, const uint16_t *bias,
                                uint16_t *out, int m, int k, int n, float alpha,
@@ -379,7 +409,10 @@ LaunchStatus launch_matmul_dma(const uint16_t *a, const uint16_t *b, const uint1
                                                kLdsBytes);
   if (attr != hipSuccess) return LaunchStatus{2u, hipGetErrorString(attr)};
   const int tiles_m = m / kBM, tiles_n = n / kBN;
+  // One workgroup fills a CU's LDS, so the grid is persistent: one workgroup
+  // per CU, each walking its share of the tiles.
   int64_t blocks = (int64_t)tiles_m * tiles_n;
+  if (blocks > AFIR_MM_GRID) blocks = AFIR_MM_GRID;
   if (block_dim) blocks = block_dim;
   hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(WM * 4 * 64), kLdsBytes, stream, a, b,
                      bias, out, m, k, n, alpha, tiles_m, tiles_n);

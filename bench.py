@@ -256,6 +256,33 @@ def make_workload(key, torch, H, O, C):
             return (2.0 * rows * 8192 * 8192) / dt / 1e12, \
                 f"{rows} of 8192 output rows (full K and N), one run"
         w.cpu = cpu
+
+        def power_evidence():
+            """Why the fraction of the published MFMA peak is what it is: the
+            board power limit sets the clock, and the power an MFMA draws
+            depends on its operand values.  Three figures: the register-only
+            MFMA rate on this workload's operands and on constant ones, and
+            this same matmul kernel on constant matrices."""
+            ev = {"mfma_only_workload_operands_tflops":
+                  round(H.probe_mfma_rate(sets[0][0]), 1)}
+            ones = torch.ones((8192, 8192), dtype=torch.bfloat16, device="cuda")
+            ev["mfma_only_constant_operands_tflops"] = round(H.probe_mfma_rate(ones), 1)
+            launch = H.prepare(w.symbol, [ones.data_ptr(), ones.data_ptr(), sets[0][2].data_ptr(),
+                                          sets[1][3].data_ptr(), 0],
+                               H.pack_tiling(8192, 8192, 8192, H.f32_bits(0.01)))
+            for _ in range(3):
+                launch()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(20):
+                launch()
+            e1.record()
+            torch.cuda.synchronize()
+            ev["kernel_constant_operands_tflops"] = round(
+                w.work() * 20 / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
+            return ev
+        w.power_evidence = power_evidence
     else:
         raise SystemExit(f"unknown workload {key}")
     return w
@@ -305,6 +332,9 @@ def main():
     ap.add_argument("--no-all", dest="all", action="store_false")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three plain 256 MiB device copies, so that a counter run "
+                         "(rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) holds a kernel of known traffic")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs the fused-kernel path on ONE GPU; "
@@ -338,9 +368,12 @@ def main():
         wall, ev_ms = run_workload(w, torch, steps, warmup)
         value, unit, roof = summarize(w, wall, ev_ms, steps)
         par = w.parity()
+        extra = w.power_evidence() if hasattr(w, "power_evidence") else None
         entry = {"workload": w.title, "value": round(value, 2), "unit": unit, "steps": steps,
                  "warmup": warmup, "ms_per_step": round(wall * 1e3 / steps, 5), "dtype": w.dtype,
                  "buffer_sets": w.nsets, "roofline": roof, "parity": par}
+        if extra is not None:
+            entry["power_limit_evidence"] = extra
         if not args.no_cpu_baseline:
             budget = args.cpu_seconds if key == args.workload else min(3.0, args.cpu_seconds)
             v, sample = w.cpu(budget)
@@ -350,6 +383,14 @@ def main():
         results.append(entry)
         del w
         torch.cuda.empty_cache()
+
+    if args.copy_calibration:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     main_e = results[0]
     line = {
