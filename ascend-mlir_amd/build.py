@@ -37,6 +37,8 @@ KERNEL_SOURCES = [
     ("kernels/matmul.hip", []),
     ("kernels/matmul_dma.hip", []),
     ("kernels/probe.hip", []),
+    ("kernels/region.hip", STRICT),
+    ("target/region_program.cpp", []),
     ("capi/afir_hip_kernels.cpp", []),
 ]
 

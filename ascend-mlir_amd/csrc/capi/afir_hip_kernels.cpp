@@ -8,7 +8,14 @@
 #include <cstring>
 #include <string>
 
+#include <map>
+#include <memory>
+#include <mutex>
+#include <vector>
+
 #include "../kernels/kernels.h"
+#include "../kernels/region_launch.h"
+#include "../target/region_program.h"
 
 namespace {
 
@@ -55,6 +62,67 @@ const AfirHipKernelInfo kKernels[] = {
      "(A bf16[M,K], B bf16[K,N], bias bf16[N]) -> out bf16[M,N] = leakyrelu(A@B + bias, alpha)"},
 };
 constexpr int kNumKernels = (int)(sizeof(kKernels) / sizeof(kKernels[0]));
+
+
+// ---- registered region programs ----
+
+struct RegisteredRegion {
+  afir_region::Program program;
+  std::vector<std::string> fields;
+};
+std::mutex g_region_mutex;
+std::map<uint64_t, std::shared_ptr<RegisteredRegion>> g_regions;
+uint64_t g_next_region = 1;
+
+std::shared_ptr<RegisteredRegion> find_region(uint64_t handle) {
+  std::lock_guard<std::mutex> lock(g_region_mutex);
+  auto it = g_regions.find(handle);
+  return it == g_regions.end() ? nullptr : it->second;
+}
+
+int region_type_code(afir_region::ElemType t) {
+  switch (t) {
+    case afir_region::ElemType::F16: return afir::kRegionF16;
+    case afir_region::ElemType::BF16: return afir::kRegionBF16;
+    case afir_region::ElemType::F32: return afir::kRegionF32;
+    case afir_region::ElemType::I32: return afir::kRegionI32;
+    case afir_region::ElemType::I64: return afir::kRegionI64;
+  }
+  return afir::kRegionF32;
+}
+
+int region_op_code(afir_region::OpCode c) {
+  using afir_region::OpCode;
+  switch (c) {
+    case OpCode::Push: return afir::kRegionPush;
+    case OpCode::Const: return afir::kRegionConst;
+    case OpCode::Add: return afir::kRegionAdd;
+    case OpCode::Sub: return afir::kRegionSub;
+    case OpCode::Mul: return afir::kRegionMul;
+    case OpCode::Div: return afir::kRegionDiv;
+    case OpCode::Max: return afir::kRegionMax;
+    case OpCode::Min: return afir::kRegionMin;
+    case OpCode::Relu: return afir::kRegionRelu;
+    case OpCode::Leaky: return afir::kRegionLeaky;
+    case OpCode::Neg: return afir::kRegionNeg;
+    case OpCode::Dup: return afir::kRegionDup;
+    default: return -1;  // ReduceSum / Store are not interpreted per element
+  }
+}
+
+std::string resolve_region(const RegisteredRegion &r, const void *tiling, size_t tiling_len,
+                           afir_region::Resolved *out) {
+  const size_t want = r.fields.size() * sizeof(int64_t);
+  if ((!tiling && want) || tiling_len != want) {
+    char buf[160];
+    std::snprintf(buf, sizeof buf, "region: tiling data must be %zu bytes (%zu int64 fields), got %zu",
+                  want, r.fields.size(), tiling_len);
+    return buf;
+  }
+  std::vector<int64_t> dims(r.fields.size());
+  if (want) std::memcpy(dims.data(), tiling, want);
+  return afir_region::resolve(r.program, dims, out);
+}
 
 }  // namespace
 
@@ -127,6 +195,125 @@ uint32_t afir_hip_probe_mfma_rate(void *stream, const void *operands, void *sink
                                   uint64_t *flops) {
   return finish(afir::launch_mfma_rate_probe(operands, static_cast<float *>(sink), iters, flops,
                                              static_cast<hipStream_t>(stream)));
+}
+
+uint32_t afir_hip_region_register(const char *program_text, size_t program_len, uint64_t *handle) {
+  if (!program_text || !handle) return fail(AFIR_HIP_E_INVALID, "region_register: null argument");
+  auto r = std::make_shared<RegisteredRegion>();
+  std::string why = afir_region::parse(std::string(program_text, program_len), &r->program);
+  if (!why.empty()) return fail(AFIR_HIP_E_INVALID, why);
+  r->fields = afir_region::tilingFieldNames(r->program);
+  std::lock_guard<std::mutex> lock(g_region_mutex);
+  *handle = g_next_region++;
+  g_regions[*handle] = std::move(r);
+  g_last_error.clear();
+  return AFIR_HIP_OK;
+}
+
+uint32_t afir_hip_region_unregister(uint64_t handle) {
+  std::lock_guard<std::mutex> lock(g_region_mutex);
+  if (!g_regions.erase(handle)) return fail(AFIR_HIP_E_UNKNOWN, "no region program with that handle");
+  return AFIR_HIP_OK;
+}
+
+uint32_t afir_hip_region_info(uint64_t handle, int *num_inputs, int *num_outputs,
+                              int *num_tiling_fields) {
+  auto r = find_region(handle);
+  if (!r) return fail(AFIR_HIP_E_UNKNOWN, "no region program with that handle");
+  if (num_inputs) *num_inputs = r->program.numInputs();
+  if (num_outputs) *num_outputs = 1;
+  if (num_tiling_fields) *num_tiling_fields = (int)r->fields.size();
+  return AFIR_HIP_OK;
+}
+
+const char *afir_hip_region_tiling_field(uint64_t handle, int index) {
+  auto r = find_region(handle);
+  if (!r || index < 0 || index >= (int)r->fields.size()) return "";
+  return r->fields[index].c_str();  // owned by the registry entry
+}
+
+uint32_t afir_hip_region_argument_bytes(uint64_t handle, const void *tiling, size_t tiling_len,
+                                        size_t *bytes, int max_args) {
+  auto r = find_region(handle);
+  if (!r) return fail(AFIR_HIP_E_UNKNOWN, "no region program with that handle");
+  if (!bytes || max_args < (int)r->program.args.size())
+    return fail(AFIR_HIP_E_INVALID, "region_argument_bytes: output array too small");
+  afir_region::Resolved res;
+  std::string why = resolve_region(*r, tiling, tiling_len, &res);
+  if (!why.empty()) return fail(AFIR_HIP_E_INVALID, why);
+  for (size_t i = 0; i < res.bytes.size(); ++i) bytes[i] = res.bytes[i];
+  g_last_error.clear();
+  return AFIR_HIP_OK;
+}
+
+uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *stream, int num_args,
+                                void *const *args, void *workspace, const void *tiling,
+                                size_t tiling_len) {
+  auto r = find_region(handle);
+  if (!r) return fail(AFIR_HIP_E_UNKNOWN, "no region program with that handle");
+  const int want = (int)r->program.args.size();
+  if (num_args != want || !args) {
+    char buf[128];
+    std::snprintf(buf, sizeof buf, "region: expected %d tensor arguments, got %d", want, num_args);
+    return fail(AFIR_HIP_E_INVALID, buf);
+  }
+  afir_region::Resolved res;
+  std::string why = resolve_region(*r, tiling, tiling_len, &res);
+  if (!why.empty()) return fail(AFIR_HIP_E_INVALID, why);
+  for (int i = 0; i < want; ++i)
+    if (res.bytes[i] && !args[i]) return fail(AFIR_HIP_E_INVALID, "region: null tensor pointer");
+
+  auto aligned = [](const void *p, int64_t bytes) {
+    return ((reinterpret_cast<uintptr_t>(p) + (uintptr_t)bytes) & 15u) == 0;
+  };
+  for (const afir_region::ResolvedSegment &seg : res.segments) {
+    afir::RegionArgs a;
+    std::memset(&a, 0, sizeof a);
+    a.rank = seg.rank;
+    for (int k = 0; k < 3; ++k) a.size[k] = k < seg.rank ? seg.size[k] : 1;
+    a.reduce = seg.reduce ? 1 : 0;
+    a.out_type = region_type_code(seg.outType);
+    const int64_t oes = (int64_t)afir_region::elemTypeBytes(seg.outType);
+    a.out = static_cast<char *>(args[want - 1]) + seg.outOffsetElems * oes;
+    a.error_flag = static_cast<int32_t *>(workspace);
+    const int last = seg.rank - 1;
+    int64_t rows = 1;
+    for (int k = 0; k < last; ++k) rows *= seg.size[k];
+    a.out_vec = !seg.reduce && aligned(a.out, 0) && (rows <= 1 || (seg.size[last] * oes) % 16 == 0);
+    a.ninputs = (int)seg.inputs.size();
+    for (int i = 0; i < a.ninputs; ++i) {
+      const afir_region::ResolvedInput &in = seg.inputs[i];
+      afir::RegionInput &d = a.in[i];
+      const int64_t es = (int64_t)afir_region::elemTypeBytes(in.type);
+      d.base = args[in.arg];
+      d.type = region_type_code(in.type);
+      for (int k = 0; k < 3; ++k) d.stride[k] = in.iterStride[k];
+      d.offset = in.offset;
+      d.gdim = in.gatherIterDim;
+      d.index = in.gatherIterDim >= 0 ? args[in.gatherIndexArg] : nullptr;
+      d.gtype = region_type_code(in.gatherIndexType);
+      d.gstride = in.gatherStride;
+      d.gextent = in.gatherExtent;
+      bool vec = aligned(d.base, in.offset * es);
+      for (int k = 0; k < last; ++k)
+        if (seg.size[k] > 1 && (in.iterStride[k] * es) % 16 != 0) vec = false;
+      d.vec = vec ? 1 : 0;
+      d.gvec = (in.gatherStride * es) % 16 == 0 ? 1 : 0;
+    }
+    a.nops = 0;
+    for (const afir_region::ResolvedOp &op : seg.ops) {
+      const int code = region_op_code(op.code);
+      if (code < 0) continue;
+      afir::RegionOp &d = a.ops[a.nops++];
+      d.code = code;
+      d.input = op.input;
+      d.constant = op.constant;
+      d.depth = op.depth;
+    }
+    uint32_t rc = finish(afir::launch_fused_region(a, block_dim, static_cast<hipStream_t>(stream)));
+    if (rc != AFIR_HIP_OK) return rc;
+  }
+  return AFIR_HIP_OK;
 }
 
 int afir_hip_kernel_count(void) { return kNumKernels; }

@@ -1,0 +1,59 @@
+// Kernel-argument form of one segment of a fused-region program (see
+// ../target/region_program.h for the program, region.hip for the kernel).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "common.h"
+
+namespace afir {
+
+constexpr int kRegionMaxInputs = 8;
+constexpr int kRegionMaxOps = 32;
+
+enum RegionType : int { kRegionF16 = 0, kRegionBF16 = 1, kRegionF32 = 2, kRegionI32 = 3, kRegionI64 = 4 };
+enum RegionOpCode : int {
+  kRegionPush = 0, kRegionConst, kRegionAdd, kRegionSub, kRegionMul, kRegionDiv, kRegionMax,
+  kRegionMin, kRegionRelu, kRegionLeaky, kRegionNeg, kRegionDup
+};
+
+struct RegionInput {
+  const void *base;    // device pointer of the tensor
+  const void *index;   // device pointer of the index tensor (gather), else null
+  int64_t stride[3];   // elements per step of each iteration dim
+  int64_t offset;      // constant element offset
+  int64_t gstride;     // elements per index step
+  int64_t gextent;     // valid indices are [0, gextent)
+  int type;            // RegionType of the tensor
+  int gdim;            // iteration dim that indexes the index tensor, -1 = no gather
+  int gtype;           // kRegionI32 / kRegionI64
+  int vec;             // 128-bit loads along the innermost dim are aligned
+  int gvec;            // ... also after adding any multiple of gstride
+  int pad;
+};
+
+struct RegionOp {
+  int code;
+  int input;
+  float constant;
+  int depth;
+};
+
+struct RegionArgs {
+  int64_t size[3];
+  void *out;            // first element this segment writes
+  int32_t *error_flag;  // set to 1 when a gathered index is out of range (may be null)
+  int out_type;
+  int out_vec;          // 128-bit stores are aligned for every full vector
+  int rank;
+  int nops;
+  int ninputs;
+  int reduce;
+  RegionInput in[kRegionMaxInputs];
+  RegionOp ops[kRegionMaxOps];
+};
+
+LaunchStatus launch_fused_region(const RegionArgs &args, uint32_t block_dim, hipStream_t stream);
+
+}  // namespace afir

@@ -39,6 +39,12 @@ EXPORTED_SYMBOLS = [
     "afir_hip_launch",
     "afir_hip_argument_bytes",
     "afir_hip_probe_mfma_rate",
+    "afir_hip_region_register",
+    "afir_hip_region_unregister",
+    "afir_hip_region_info",
+    "afir_hip_region_tiling_field",
+    "afir_hip_region_argument_bytes",
+    "afir_hip_launch_region",
 ]
 
 _lib = None
@@ -265,3 +271,86 @@ def probe_mfma_rate(operands, iters=20000, repeats=3):
         torch.cuda.synchronize()
         best = max(best, flops.value / (e0.elapsed_time(e1) * 1e-3) / 1e12)
     return best
+
+
+# ---- fused-region programs ---------------------------------------------------
+
+_TORCH_TYPES = None
+
+
+def _torch_type(name):
+    global _TORCH_TYPES
+    import torch
+    if _TORCH_TYPES is None:
+        _TORCH_TYPES = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32,
+                        "i32": torch.int32, "i64": torch.int64}
+    return _TORCH_TYPES[name]
+
+
+class Region:
+    """A registered fused-region program (afir_hip_region_register)."""
+
+    def __init__(self, text: str):
+        L = load()
+        u64 = ctypes.c_uint64
+        L.afir_hip_region_register.restype = ctypes.c_uint32
+        L.afir_hip_region_register.argtypes = [ctypes.c_char_p, ctypes.c_size_t, ctypes.POINTER(u64)]
+        L.afir_hip_region_unregister.argtypes = [u64]
+        L.afir_hip_region_info.argtypes = [u64] + [ctypes.POINTER(ctypes.c_int)] * 3
+        L.afir_hip_region_tiling_field.restype = ctypes.c_char_p
+        L.afir_hip_region_tiling_field.argtypes = [u64, ctypes.c_int]
+        L.afir_hip_region_argument_bytes.argtypes = [u64, ctypes.c_void_p, ctypes.c_size_t,
+                                                    ctypes.POINTER(ctypes.c_size_t), ctypes.c_int]
+        L.afir_hip_launch_region.restype = ctypes.c_uint32
+        L.afir_hip_launch_region.argtypes = [u64, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_int,
+                                             ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p,
+                                             ctypes.c_void_p, ctypes.c_size_t]
+        data = text.encode()
+        h = u64(0)
+        _check(L.afir_hip_region_register(data, len(data), ctypes.byref(h)))
+        self.handle = h.value
+        ni, no, nf = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+        _check(L.afir_hip_region_info(u64(self.handle), ctypes.byref(ni), ctypes.byref(no), ctypes.byref(nf)))
+        self.num_inputs, self.num_outputs = ni.value, no.value
+        self.tiling_fields = [L.afir_hip_region_tiling_field(u64(self.handle), i).decode()
+                              for i in range(nf.value)]
+        self.arg_types = [l.split()[2] for l in text.splitlines() if l.split()[:1] == ["arg"]]
+
+    def close(self):
+        if self.handle:
+            load().afir_hip_region_unregister(ctypes.c_uint64(self.handle))
+            self.handle = 0
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def argument_bytes(self, tiling: bytes):
+        n = self.num_inputs + self.num_outputs
+        out = (ctypes.c_size_t * n)()
+        buf = ctypes.create_string_buffer(tiling, len(tiling))
+        _check(load().afir_hip_region_argument_bytes(ctypes.c_uint64(self.handle), buf, len(tiling), out, n))
+        return list(out)
+
+    def launch_raw(self, ptrs, tiling: bytes, workspace=0, block_dim=0, stream=None):
+        arr = (ctypes.c_void_p * len(ptrs))(*[ctypes.c_void_p(p) for p in ptrs])
+        buf = ctypes.create_string_buffer(tiling, len(tiling))
+        return load().afir_hip_launch_region(ctypes.c_uint64(self.handle), block_dim, _stream(stream),
+                                             len(ptrs), arr, ctypes.c_void_p(workspace), buf, len(tiling))
+
+    def __call__(self, *inputs, out_shape, workspace=None, block_dim=0, stream=None):
+        """inputs: device tensors in argument order; returns the output tensor."""
+        import torch
+        if len(inputs) != self.num_inputs:
+            raise AfirHipError(f"region expects {self.num_inputs} inputs, got {len(inputs)}")
+        for i, t in enumerate(inputs):
+            _dev(t, _torch_type(self.arg_types[i]), f"region input {i}")
+        out = torch.empty(tuple(out_shape), dtype=_torch_type(self.arg_types[-1]), device=inputs[0].device)
+        dims = [d for t in inputs for d in t.shape] + list(out.shape)
+        tiling = pack_tiling(*dims)
+        ws = workspace.data_ptr() if workspace is not None else 0
+        _check(self.launch_raw([t.data_ptr() for t in inputs] + [out.data_ptr()], tiling, ws,
+                               block_dim, stream))
+        return out

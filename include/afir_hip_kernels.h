@@ -154,6 +154,34 @@ uint32_t afir_hip_launch(const char *kernel_name, uint32_t block_dim, void *stre
                          int num_args, void *const *args, void *workspace,
                          const void *tiling, size_t tiling_len);
 
+/* ---- fused-region programs -----------------------------------------------------
+ * A fused region that is none of the families above (any chain of
+ * add/sub/mul/div/max/min/relu/leaky_relu over inputs read through broadcast,
+ * transposed, constant or gathered index maps, optionally summed over the last
+ * dim, optionally concatenated along dim 0) runs on one generic kernel that
+ * executes a region PROGRAM -- the text a translator derives from the region's
+ * IR (grammar: csrc/target/region_program.h).  The program stands where the
+ * reference has a device binary: it is registered once and launched by handle,
+ * the shape of rtDevBinaryRegister / rtFunctionRegister followed by
+ * rtKernelLaunch(handle, block_dim, args...)
+ * (lib/Runtime/Execution/NativeExecutionRunner.cpp:332-369,476-488).
+ *
+ * TilingData of a program: one int64 per dimension of every argument,
+ * dim_arg<A>_<D>, arguments in declaration order (inputs..., output);
+ * afir_hip_region_tiling_field names them.  args = device pointers in the same
+ * order.  workspace as for the launchers (int32 error flag for gathers). */
+uint32_t afir_hip_region_register(const char *program_text, size_t program_len, uint64_t *handle);
+uint32_t afir_hip_region_unregister(uint64_t handle);
+uint32_t afir_hip_region_info(uint64_t handle, int *num_inputs, int *num_outputs,
+                              int *num_tiling_fields);
+/* Name of tiling field `index` ("" if out of range); valid until unregister. */
+const char *afir_hip_region_tiling_field(uint64_t handle, int index);
+uint32_t afir_hip_region_argument_bytes(uint64_t handle, const void *tiling, size_t tiling_len,
+                                        size_t *bytes, int max_args);
+uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *stream, int num_args,
+                                void *const *args, void *workspace, const void *tiling,
+                                size_t tiling_len);
+
 /* ---- measurement aid ----------------------------------------------------------
  * No counterpart in the reference.  Launches a kernel that does nothing but
  * issue v_mfma_f32_32x32x16_bf16 from registers on every CU (8 waves per

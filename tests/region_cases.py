@@ -1,0 +1,302 @@
+"""Region programs used by the CPU and GPU tests: the reference's example
+graphs and the benchmark configurations, written in the region-program text
+form, each with a seeded input generator and the closed-form golden it must
+reproduce (formulas: examples/*/gen_data.py, gen_inputs.py of the reference)."""
+import numpy as np
+
+from oracle import afir_oracle as O
+
+HEADER = "afir-hip-region 1\n"
+
+
+def _u(rng, shape, lo=-1.0, hi=1.0, dt=np.float16):
+    return rng.uniform(lo, hi, shape).astype(np.float32).astype(dt)
+
+
+# c[m] = f16(sum_n (a[m] + b[m,n]))        examples/broadcast-add-reduce
+REDUCE_ROWBIAS = HEADER + """
+arg in f16 1
+arg in f16 2
+arg out f16 1
+segment 2
+  size arg1.0 arg1.1
+  outoff 0
+  push arg0 d0
+  push arg1 d0 d1
+  add
+  reduce sum
+  store
+end
+"""
+
+# out[n,m] = f16(relu(data0[m,0]) + data1[n,m])   examples/relu-broadcast-transpose
+RELU_COL_ADD = HEADER + """
+arg in f16 2
+arg in f16 2
+arg out f16 2
+segment 2
+  size arg1.0 arg1.1
+  outoff 0
+  push arg0 d1 0
+  relu
+  push arg1 d0 d1
+  add
+  store
+end
+"""
+
+# out[i,j] = f16(relu(data[i, idx[j]]) + bias[j])   examples/gather-elementwise-fusion
+RELU_COLGATHER_ADD = HEADER + """
+arg in f16 2
+arg in i64 1
+arg in f16 1
+arg out f16 2
+segment 2
+  size arg0.0 arg1.0
+  outoff 0
+  push arg0 d0 g1:arg1
+  relu
+  push arg2 d1
+  add
+  store
+end
+"""
+
+# rows [0,M): a[m] + b[m,n]; rows [M,2M): c[m] * d[m,n]   examples/add-broadcast-concat
+ADD_BROADCAST_CONCAT = HEADER + """
+arg in f16 1
+arg in f16 2
+arg in f16 1
+arg in f16 2
+arg out f16 2
+segment 2
+  size arg1.0 arg1.1
+  outoff 0
+  push arg0 d0
+  push arg1 d0 d1
+  add
+  store
+end
+segment 2
+  size arg3.0 arg3.1
+  outoff arg1.0
+  push arg2 d0
+  push arg3 d0 d1
+  mul
+  store
+end
+"""
+
+# halves of a: (relu(a_h) + bias_h[m]) * scale_h[n]        examples/split-relu-brc-add-mul
+SPLIT_RELU_BRC_ADD_MUL = HEADER + """
+arg in f16 2
+arg in f16 1
+arg in f16 1
+arg in f16 1
+arg in f16 1
+arg out f16 2
+segment 2
+  size arg1.0 arg0.1
+  outoff 0
+  push arg0 d0 d1
+  relu
+  push arg1 d0
+  add
+  push arg3 d1
+  mul
+  store
+end
+segment 2
+  size arg2.0 arg0.1
+  outoff arg1.0
+  push arg0 d0 d1 slice arg1.0 0
+  relu
+  push arg2 d0
+  add
+  push arg4 d1
+  mul
+  store
+end
+"""
+
+# the benchmark configurations as programs
+C1_ADD_MUL = HEADER + """
+arg in f32 2
+arg in f32 2
+arg out f32 2
+segment 2
+  size arg0.0 arg0.1
+  outoff 0
+  push arg0 d0 d1
+  push arg1 d0 d1
+  add
+  push arg1 d0 d1
+  mul
+  store
+end
+"""
+
+C2_BCAST_ADD_ROWSUM = HEADER + """
+arg in f32 2
+arg in f32 1
+arg out f32 1
+segment 2
+  size arg0.0 arg0.1
+  outoff 0
+  push arg0 d0 d1
+  push arg1 d1
+  add
+  reduce sum
+  store
+end
+"""
+
+# out[b,j,i] = f16(relu(x[b,i,j]) + c[j]): iteration space = output (b, j, i)
+C3_RELU_BCAST_TRANSPOSE = HEADER + """
+arg in f16 3
+arg in f16 1
+arg out f16 3
+segment 3
+  size arg0.0 arg0.2 arg0.1
+  outoff 0
+  push arg0 d0 d2 d1
+  relu
+  push arg1 d1
+  add
+  store
+end
+"""
+
+C4_GATHER_SCALE_SHIFT = HEADER + """
+arg in f16 2
+arg in i32 1
+arg in f16 1
+arg in f16 1
+arg out f16 2
+segment 2
+  size arg1.0 arg0.1
+  outoff 0
+  push arg0 g0:arg1 d1
+  push arg2 d1
+  mul
+  push arg3 d1
+  add
+  store
+end
+"""
+
+# torch_e2e graphs (examples/torch_e2e/test_elementwise.py): (a + b) * c, and an
+# AFIR-only chain with sub / div / leaky relu and a dup
+ADD_MUL_3 = HEADER + """
+arg in f32 2
+arg in f32 2
+arg in f32 2
+arg out f32 2
+segment 2
+  size arg0.0 arg0.1
+  outoff 0
+  push arg0 d0 d1
+  push arg1 d0 d1
+  add
+  push arg2 d0 d1
+  mul
+  store
+end
+"""
+
+SUB_DIV_LEAKY = HEADER + """
+arg in f32 2
+arg in f32 1
+arg out bf16 2
+segment 2
+  size arg0.0 arg0.1
+  outoff 0
+  push arg0 d0 d1
+  push arg1 d1
+  sub
+  dup 0
+  const 1.5
+  add
+  div
+  leaky 0.01
+  neg
+  push arg1 d1
+  min
+  store
+end
+"""
+
+
+def case_reduce_rowbias(m=640, n=512, seed=42):
+    rng = np.random.default_rng(seed)
+    a, b = _u(rng, (m,)), _u(rng, (m, n))
+    return REDUCE_ROWBIAS, [a, b], O.reduce_rowbias_f16(a, b)
+
+
+def case_relu_col_add(m=640, n=500, seed=42):
+    rng = np.random.default_rng(seed)
+    d0, d1 = _u(rng, (m, 1)), _u(rng, (n, m))
+    return RELU_COL_ADD, [d0, d1], O.relu_col_add_f16(d0, d1)
+
+
+def case_relu_colgather_add(m=16, n=640, k=128, seed=42):
+    rng = np.random.default_rng(seed)
+    data, bias = _u(rng, (m, n)), _u(rng, (k,))
+    idx = rng.integers(0, n, k, dtype=np.int64)
+    return RELU_COLGATHER_ADD, [data, idx, bias], O.relu_colgather_add_f16(data, idx, bias)
+
+
+def case_add_broadcast_concat(m=320, n=512, seed=42):
+    rng = np.random.default_rng(seed)
+    a, b, c, d = _u(rng, (m,)), _u(rng, (m, n)), _u(rng, (m,)), _u(rng, (m, n))
+    want = np.concatenate([(a[:, None].astype(np.float32) + b.astype(np.float32)),
+                           (c[:, None].astype(np.float32) * d.astype(np.float32))],
+                          axis=0).astype(np.float16)
+    return ADD_BROADCAST_CONCAT, [a, b, c, d], want
+
+
+def case_split_relu_brc_add_mul(m=640, n=512, seed=42):
+    rng = np.random.default_rng(seed)
+    hm = m // 2
+    a = _u(rng, (m, n))
+    b0, b1, s0, s1 = _u(rng, (hm,)), _u(rng, (hm,)), _u(rng, (n,)), _u(rng, (n,))
+    f = np.float32
+    o0 = (np.maximum(a[:hm].astype(f), f(0)) + b0[:, None].astype(f)) * s0[None, :].astype(f)
+    o1 = (np.maximum(a[hm:].astype(f), f(0)) + b1[:, None].astype(f)) * s1[None, :].astype(f)
+    return SPLIT_RELU_BRC_ADD_MUL, [a, b0, b1, s0, s1], np.concatenate([o0, o1], 0).astype(np.float16)
+
+
+def case_c1(shape=(96, 1000)):
+    a, b = O.gen_c1(shape)
+    return C1_ADD_MUL, [a, b], O.golden_c1(a, b)
+
+
+def case_c2(m=64, n=4096):
+    x, bias = O.gen_c2(m, n)
+    return C2_BCAST_ADD_ROWSUM, [x, bias], O.golden_c2(x, bias)
+
+
+def case_c3(b=2, m=96, n=64):
+    x, c = O.gen_c3(b, m, n)
+    return C3_RELU_BCAST_TRANSPOSE, [x, c], O.golden_c3(x, c)
+
+
+def case_c4(rows=512, dim=264, nidx=300):
+    table, idx, scale, shift = O.gen_c4(rows, dim, nidx)
+    return C4_GATHER_SCALE_SHIFT, [table, idx, scale, shift], O.golden_c4(table, idx, scale, shift)
+
+
+def case_add_mul_3(shape=(33, 77), seed=5):
+    rng = np.random.default_rng(seed)
+    a, b, c = (_u(rng, shape, dt=np.float32) for _ in range(3))
+    return ADD_MUL_3, [a, b, c], ((a + b) * c).astype(np.float32)
+
+
+EXACT_CASES = {
+    "relu_col_add": case_relu_col_add,
+    "relu_colgather_add": case_relu_colgather_add,
+    "add_broadcast_concat": case_add_broadcast_concat,
+    "split_relu_brc_add_mul": case_split_relu_brc_add_mul,
+    "c1": case_c1, "c3": case_c3, "c4": case_c4, "add_mul_3": case_add_mul_3,
+}
+REDUCE_CASES = {"reduce_rowbias": case_reduce_rowbias, "c2": case_c2}

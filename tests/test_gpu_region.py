@@ -1,0 +1,182 @@
+"""The generic fused-region kernel against the region oracle: the reference's
+example graphs at their own shapes, the benchmark configurations as programs,
+ragged / unaligned shapes, and seeded random op chains.  Needs a GPU."""
+import numpy as np
+import pytest
+
+from oracle import afir_oracle as O
+from oracle import region_oracle as RO
+from tests import region_cases as RC
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def H(pkg):
+    import torch
+    from ascend_mlir_amd import hip_kernels
+    hip_kernels.load()
+    assert torch.cuda.is_available()
+    return hip_kernels
+
+
+def _dev(x, t):
+    import torch
+    if t == "bf16":
+        return torch.from_numpy(x.view(np.int16)).cuda().view(torch.bfloat16)
+    return torch.from_numpy(np.ascontiguousarray(x)).cuda()
+
+
+def _host(t, ty):
+    import torch
+    if ty == "bf16":
+        return t.view(torch.int16).cpu().numpy().view(np.uint16)
+    return t.cpu().numpy()
+
+
+def run(H, text, inputs, out_shape, workspace=None, block_dim=0):
+    r = H.Region(text)
+    dev = [_dev(x, r.arg_types[i]) for i, x in enumerate(inputs)]
+    out = r(*dev, out_shape=out_shape, workspace=workspace, block_dim=block_dim)
+    res = _host(out, r.arg_types[-1])
+    r.close()
+    return res
+
+
+@pytest.mark.parametrize("name", sorted(RC.EXACT_CASES))
+def test_reference_examples_and_configs_bit_exact(H, name):
+    text, inputs, want = RC.EXACT_CASES[name]()
+    got = run(H, text, inputs, want.shape)
+    assert got.tobytes() == want.tobytes()
+
+
+@pytest.mark.parametrize("name", sorted(RC.REDUCE_CASES))
+def test_reductions_within_tolerance(H, name):
+    text, inputs, want = RC.REDUCE_CASES[name]()
+    got = run(H, text, inputs, want.shape).astype(np.float64)
+    terms = (inputs[0].astype(np.float64)[:, None] + inputs[1].astype(np.float64)
+             if inputs[0].ndim == 1 else inputs[0].astype(np.float64) + inputs[1].astype(np.float64))
+    scale = np.abs(terms).sum(axis=1)
+    ulp = 2.0 ** -10 if want.dtype == np.float16 else 0.0      # one f16 rounding of the result
+    tol = 1e-5 * np.abs(want.astype(np.float64)) + 1e-6 * scale + ulp * np.abs(want.astype(np.float64))
+    assert np.all(np.abs(got - want.astype(np.float64)) <= tol)
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (3, 5), (7, 8), (5, 9), (64, 1000), (2, 4099), (0, 8), (4, 0)])
+def test_ragged_shapes_and_block_dim(H, shape):
+    rng = np.random.default_rng(11)
+    a = rng.uniform(-2, 2, shape).astype(np.float32)
+    b = rng.uniform(-2, 2, shape).astype(np.float32)
+    want = RO.evaluate(RC.C1_ADD_MUL, [a, b])
+    for bd in (0, 1, 7):
+        got = run(H, RC.C1_ADD_MUL, [a, b], shape, block_dim=bd)
+        assert got.tobytes() == want.tobytes()
+
+
+def test_unaligned_bases_take_the_element_path(H):
+    import torch
+    rng = np.random.default_rng(12)
+    a = rng.uniform(-2, 2, (17, 40)).astype(np.float16)
+    c = rng.uniform(-2, 2, (40,)).astype(np.float16)
+    text = RC.HEADER + ("arg in f16 2\narg in f16 1\narg out f16 2\nsegment 2\n size arg0.0 arg0.1\n"
+                        " outoff 0\n push arg0 d0 d1\n push arg1 d1\n mul\n store\nend\n")
+    want = RO.evaluate(text, [a, c])
+    r = H.Region(text)
+    # same data at odd element offsets: neither operand is 16-byte aligned
+    abuf = torch.zeros(a.size + 8, dtype=torch.float16, device="cuda")
+    cbuf = torch.zeros(c.size + 8, dtype=torch.float16, device="cuda")
+    obuf = torch.zeros(a.size + 8, dtype=torch.float16, device="cuda")
+    abuf[3:3 + a.size] = torch.from_numpy(a.ravel()).cuda()
+    cbuf[1:1 + c.size] = torch.from_numpy(c).cuda()
+    rc = r.launch_raw([abuf.data_ptr() + 6, cbuf.data_ptr() + 2, obuf.data_ptr() + 10],
+                      H.pack_tiling(17, 40, 40, 17, 40))
+    assert rc == 0
+    torch.cuda.synchronize()
+    got = obuf[5:5 + a.size].cpu().numpy().reshape(17, 40)
+    assert got.tobytes() == want.tobytes()
+    assert float(obuf[:5].abs().sum()) == 0 and float(obuf[5 + a.size:].abs().sum()) == 0
+    r.close()
+
+
+def test_special_values_match_the_oracle(H):
+    nan, inf = np.float32("nan"), np.float32("inf")
+    a = np.array([[-0.0, 0.0, nan, 1.0, -inf, -2.0, inf, 1e-40, -1e-40, 3.0]], dtype=np.float32)
+    b = np.array([0.0, -0.0, 1.0, nan, 3.0, -1.0, inf, 2.0, 0.5, 0.0], dtype=np.float32)
+    head = RC.HEADER + "arg in f32 2\narg in f32 1\narg out f32 2\nsegment 2\n size arg0.0 arg0.1\n outoff 0\n"
+    for body in ("push arg0 d0 d1\n push arg1 d1\n max\n", "push arg0 d0 d1\n push arg1 d1\n min\n",
+                 "push arg0 d0 d1\n relu\n", "push arg0 d0 d1\n leaky 0.01\n",
+                 "push arg0 d0 d1\n push arg1 d1\n div\n", "push arg0 d0 d1\n push arg1 d1\n mul\n",
+                 "push arg0 d0 d1\n push arg1 d1\n sub\n neg\n"):
+        text = head + body + " store\nend\n"
+        want = RO.evaluate(text, [a, b])
+        got = run(H, text, [a, b], a.shape)
+        same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))
+        assert same.all(), (body, got, want)
+
+
+def test_gather_out_of_range_sets_the_flag_and_reads_nothing_outside(H):
+    import torch
+    text, inputs, _ = RC.case_relu_colgather_add(8, 64, 24)
+    idx = inputs[1].copy()
+    idx[5] = 64
+    idx[9] = -1
+    ws = torch.zeros(4, dtype=torch.int32, device="cuda")
+    got = run(H, text, [inputs[0], idx, inputs[2]], (8, 24), workspace=ws)
+    assert int(ws[0]) != 0
+    assert np.isnan(got[:, 5]).all() and np.isnan(got[:, 9]).all()
+    good = [j for j in range(24) if j not in (5, 9)]
+    ref = O.relu_colgather_add_f16(inputs[0], np.where((idx < 0) | (idx >= 64), 0, idx), inputs[2])
+    assert got[:, good].tobytes() == ref[:, good].tobytes()
+
+
+OPS2 = ["add", "sub", "mul", "div", "max", "min"]
+OPS1 = ["relu", "leaky 0.125", "neg"]
+
+
+def _random_program(rng, ty):
+    """A random chain over x[d0,d1] (identity), r[d0] (row broadcast), c[d1]
+    (column broadcast) and t[d1,d0] (transposed)."""
+    lines = ["push arg0 d0 d1"]
+    depth = 1
+    for _ in range(int(rng.integers(2, 9))):
+        k = rng.integers(0, 4)
+        if depth < 3 and k == 0:
+            lines.append(["push arg1 d0", "push arg2 d1", "push arg3 d1 d0", "const 0.75",
+                          "dup 0"][int(rng.integers(0, 5))])
+            depth += 1
+        elif depth >= 2 and k in (1, 2):
+            lines.append(OPS2[int(rng.integers(0, len(OPS2)))])
+            depth -= 1
+        else:
+            lines.append(OPS1[int(rng.integers(0, len(OPS1)))])
+    while depth > 1:
+        lines.append(OPS2[int(rng.integers(0, 3))])
+        depth -= 1
+    return (RC.HEADER + f"arg in {ty} 2\narg in {ty} 1\narg in {ty} 1\narg in {ty} 2\narg out {ty} 2\n"
+            "segment 2\n size arg0.0 arg0.1\n outoff 0\n " + "\n ".join(lines) + "\n store\nend\n")
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_chains_bit_exact(H, seed):
+    rng = np.random.default_rng(1000 + seed)
+    ty = ["f32", "f16", "bf16"][seed % 3]
+    m, n = int(rng.integers(1, 70)), int(rng.integers(1, 200))
+    text = _random_program(rng, ty)
+
+    def gen(shape):
+        x = rng.uniform(-3, 3, shape).astype(np.float32)
+        if ty == "f16":
+            return x.astype(np.float16)
+        if ty == "bf16":
+            return O.f32_to_bf16_bits(x)
+        return x
+    inputs = [gen((m, n)), gen((m,)), gen((n,)), gen((n, m))]
+    want = RO.evaluate(text, inputs)
+    got = run(H, text, inputs, (m, n))
+    if ty == "bf16":
+        wf, gf = O.bf16_bits_to_f32(want), O.bf16_bits_to_f32(got)
+    else:
+        wf, gf = want.astype(np.float32), got.astype(np.float32)
+    same = (got.view(np.uint16 if ty != "f32" else np.uint32) ==
+            want.view(np.uint16 if ty != "f32" else np.uint32)) | (np.isnan(wf) & np.isnan(gf))
+    assert same.all(), text

@@ -1,0 +1,147 @@
+"""The region-program oracle against the closed-form goldens of the reference's
+examples and of the benchmark configurations, and the host side of the region
+C ABI (parse / validate / resolve) -- CPU only."""
+import ctypes
+import struct
+
+import numpy as np
+import pytest
+
+from oracle import region_oracle as RO
+from tests import region_cases as RC
+
+
+@pytest.mark.parametrize("name", sorted(RC.EXACT_CASES))
+def test_program_reproduces_closed_form_golden(name):
+    text, inputs, want = RC.EXACT_CASES[name]()
+    got = RO.evaluate(text, inputs)
+    assert got.dtype == want.dtype and got.shape == want.shape
+    assert got.tobytes() == want.tobytes()
+
+
+@pytest.mark.parametrize("name", sorted(RC.REDUCE_CASES))
+def test_reduce_program_reproduces_golden(name):
+    text, inputs, want = RC.REDUCE_CASES[name]()
+    got = RO.evaluate(text, inputs)
+    # same numpy pairwise float32 sum as the golden: identical
+    assert got.tobytes() == want.tobytes()
+
+
+def _py(op, a, b):
+    """One float32 operation through Python doubles, rounded with struct
+    (a double holds the exact sum / product / difference of two floats, and
+    the correctly rounded quotient rounds to the same float)."""
+    r = {"add": a + b, "sub": a - b, "mul": a * b, "div": a / b}[op]
+    return struct.unpack("<f", struct.pack("<f", r))[0]
+
+
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div"])
+def test_single_ops_against_python_floats(op):
+    rng = np.random.default_rng(3)
+    a = rng.uniform(-4, 4, (5, 7)).astype(np.float32)
+    b = rng.uniform(0.5, 4, (7,)).astype(np.float32)
+    text = RC.HEADER + f"""
+arg in f32 2
+arg in f32 1
+arg out f32 2
+segment 2
+  size arg0.0 arg0.1
+  outoff 0
+  push arg0 d0 d1
+  push arg1 d1
+  {op}
+  store
+end
+"""
+    got = RO.evaluate(text, [a, b])
+    for i in range(5):
+        for j in range(7):
+            assert got[i, j] == np.float32(_py(op, float(a[i, j]), float(b[j])))
+
+
+def test_max_min_relu_special_values():
+    nan, inf = np.float32("nan"), np.float32("inf")
+    a = np.array([[-0.0, 0.0, nan, 1.0, -inf, -2.0]], dtype=np.float32)
+    b = np.array([0.0, -0.0, 1.0, nan, 3.0, -1.0], dtype=np.float32)
+    body = "push arg0 d0 d1\n  push arg1 d1\n  {}\n  store"
+    head = RC.HEADER + "arg in f32 2\narg in f32 1\narg out f32 2\nsegment 2\n  size arg0.0 arg0.1\n  outoff 0\n  "
+    mx = RO.evaluate(head + body.format("max") + "\nend\n", [a, b])[0]
+    mn = RO.evaluate(head + body.format("min") + "\nend\n", [a, b])[0]
+    assert not np.signbit(mx[0]) and not np.signbit(mx[1])       # max(-0, +0) = +0 either way
+    assert np.signbit(mn[0]) and np.signbit(mn[1])               # min(-0, +0) = -0 either way
+    assert np.isnan(mx[2]) and np.isnan(mx[3]) and np.isnan(mn[2]) and np.isnan(mn[3])
+    assert mx[4] == 3.0 and mn[4] == -inf and mx[5] == -1.0 and mn[5] == -2.0
+    relu = RO.evaluate(head + "push arg0 d0 d1\n  relu\n  store\nend\n", [a, b])[0]
+    assert not np.signbit(relu[0]) and relu[0] == 0 and np.isnan(relu[2]) and relu[4] == 0 and relu[5] == 0
+
+
+def test_gather_out_of_range_is_an_error():
+    text, inputs, _ = RC.case_relu_colgather_add(4, 10, 6)
+    inputs[1] = inputs[1].copy()
+    inputs[1][2] = 10
+    with pytest.raises(RO.RegionError):
+        RO.evaluate(text, inputs)
+
+
+# ---- the C ABI's host side: parse / validate / resolve, no GPU needed --------
+
+@pytest.fixture(scope="module")
+def H(pkg):
+    from ascend_mlir_amd import hip_kernels
+    hip_kernels.load()
+    return hip_kernels
+
+
+ALL_TEXTS = {k: getattr(RC, k) for k in dir(RC) if k.isupper() and k != "HEADER"
+             and isinstance(getattr(RC, k), str)}
+
+
+@pytest.mark.parametrize("name", sorted(ALL_TEXTS))
+def test_library_accepts_every_case_program(H, name):
+    r = H.Region(ALL_TEXTS[name])
+    prog = RO.parse(ALL_TEXTS[name])
+    assert r.num_inputs == len(prog["args"]) - 1 and r.num_outputs == 1
+    want = [f"dim_arg{a}_{d}" for a, (_, _, rank) in enumerate(prog["args"]) for d in range(rank)]
+    assert r.tiling_fields == want
+    r.close()
+
+
+def test_library_resolves_shapes_and_rejects_inconsistent_ones(H):
+    r = H.Region(RC.SPLIT_RELU_BRC_ADD_MUL)
+    ok = H.pack_tiling(640, 512, 320, 320, 512, 512, 640, 512)
+    assert r.argument_bytes(ok) == [640 * 512 * 2, 640, 640, 1024, 1024, 640 * 512 * 2]
+    with pytest.raises(H.AfirHipError, match="cover|tile|beyond"):     # halves do not add up
+        r.argument_bytes(H.pack_tiling(640, 512, 320, 300, 512, 512, 640, 512))
+    with pytest.raises(H.AfirHipError, match="runs past"):             # scale shorter than N
+        r.argument_bytes(H.pack_tiling(640, 512, 320, 320, 100, 512, 640, 512))
+    with pytest.raises(H.AfirHipError, match="tiling data must be"):
+        r.argument_bytes(b"\0" * 8)
+    r.close()
+    g = H.Region(RC.RELU_COLGATHER_ADD)
+    with pytest.raises(H.AfirHipError, match="does not match the output"):
+        g.argument_bytes(H.pack_tiling(16, 640, 100, 128, 16, 128))
+    with pytest.raises(H.AfirHipError, match="argument 2 runs past"):
+        g.argument_bytes(H.pack_tiling(16, 640, 128, 100, 16, 128))
+    g.close()
+
+
+@pytest.mark.parametrize("bad,why", [
+    ("", "header"),
+    (RC.HEADER + "arg out f32 2\n", "no segment"),
+    (RC.HEADER + "arg in f32 2\narg out f32 2\nsegment 2\n size arg0.0 arg0.1\n push arg0 d0 d1\n add\n store\nend\n",
+     "fewer than two"),
+    (RC.HEADER + "arg in f32 2\narg out f32 2\nsegment 2\n size arg0.0 arg0.1\n push arg0 d0 d1\nend\n", "end with 'store'"),
+    (RC.HEADER + "arg in f32 2\narg out f32 2\nsegment 2\n size arg0.0 arg0.1\n push arg0 d0 d5\n store\nend\n",
+     "missing iteration dim"),
+    (RC.HEADER + "arg in f32 2\narg in f32 1\narg out f32 2\nsegment 2\n size arg0.0 arg0.1\n push arg0 d0 g1:arg1\n store\nend\n",
+     "index tensor must be"),
+    (RC.HEADER + "arg in f32 2\narg out f32 2\nsegment 2\n size arg0.0 arg0.1\n push arg0 d0 d1\n frobnicate\n store\nend\n",
+     "unknown operation"),
+    (RC.HEADER + "arg in f32 2\narg out f32 2\nsegment 2\n size arg0.0 arg0.1\n" + " push arg0 d0 d1\n" * 5 + " store\nend\n",
+     "more than 4 live"),
+    (RC.HEADER + "arg in f32 2\narg out f32 2\nsegment 2\n size arg0.0 arg0.1\n push arg0 d0 d1\n reduce sum\n store\nend\n",
+     "output rank"),
+])
+def test_library_rejects_malformed_programs(H, bad, why):
+    with pytest.raises(H.AfirHipError, match=why):
+        H.Region(bad)
