@@ -71,7 +71,8 @@ def build_kernels():
 
 
 RUNTIME_SOURCES = ["runtime/support.cpp", "runtime/artifact.cpp", "runtime/session.cpp",
-                   "runtime/hip_runner.cpp", "capi/afirt_runtime.cpp"]
+                   "runtime/hip_runner.cpp", "capi/afirt_runtime.cpp",
+                   "target/region_program.cpp", "target/mlir_translate.cpp"]
 HOST = ["-std=c++17", "-O2", "-fPIC", "-Wall", "-Wno-unused-result",
         "-D__HIP_PLATFORM_AMD__", "-I", "/opt/rocm/include", "-I", os.path.join(ROOT, "include")]
 CXX = os.environ.get("CXX", "g++")
@@ -99,7 +100,11 @@ def build_runtime():
     exe = os.path.join(HERE, "bin", "runtime-session")
     _run([CXX, "-o", exe, main_obj, "-L" + LIB, "-lAFIRRuntimeCAPI", "-L/opt/rocm/lib",
           "-lamdhip64", "-ldl", "-Wl,-rpath,$ORIGIN/../lib", "-Wl,-rpath,/opt/rocm/lib"])
-    return [lib, exe]
+    # afir-translate -mlir-to-hip: host-only, no HIP runtime needed
+    tr_obj = _compile_host("tools/afir_translate_main.cpp")
+    tr_exe = os.path.join(HERE, "bin", "afir-translate")
+    _run([CXX, "-o", tr_exe, tr_obj, *[o for o in objs if "target_" in o]])
+    return [lib, exe, tr_exe]
 
 
 def build_all():

@@ -5,6 +5,7 @@
 #include "afir_hip_kernels.h"
 
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <string>
 
@@ -66,10 +67,113 @@ constexpr int kNumKernels = (int)(sizeof(kKernels) / sizeof(kKernels[0]));
 
 // ---- registered region programs ----
 
+// Programs that are exactly one of the hand-tuned kernels are routed to it
+// (same arithmetic, faster data movement); everything else runs on the generic
+// region kernel.  Matmul programs have no generic form: they must match.
+enum class FastPath { None, AddMul, BcastAddRowsum, ReluBcastTranspose, GatherScaleShift, MatmulBiasLeaky };
+
 struct RegisteredRegion {
   afir_region::Program program;
   std::vector<std::string> fields;
+  FastPath fast = FastPath::None;
+  int fastArgs[4] = {-1, -1, -1, -1};  // argument index of each kernel operand
+  float alpha = 0.f;
 };
+
+bool is_push(const afir_region::Op &o, int rank, std::initializer_list<int> dims) {
+  using afir_region::MapResult;
+  if (o.code != afir_region::OpCode::Push || !o.slice.empty() || (int)o.map.size() != (int)dims.size()) return false;
+  (void)rank;
+  size_t i = 0;
+  for (int d : dims) {
+    if (o.map[i].kind != MapResult::IterDim || o.map[i].iterDim != d) return false;
+    ++i;
+  }
+  return true;
+}
+
+// Recognises the five hand-tuned kernels among region programs.  Returns a
+// diagnostic for matmul programs that match none.
+std::string detect_fast_path(RegisteredRegion *r) {
+  using afir_region::ElemType;
+  using afir_region::MapResult;
+  using afir_region::OpCode;
+  const afir_region::Program &p = r->program;
+  if (p.segments.size() != 1) return "";
+  const afir_region::Segment &g = p.segments[0];
+  if (g.outOffset.arg >= 0 || g.outOffset.constant != 0) return "";
+  const std::vector<afir_region::Op> &ops = g.ops;
+  auto type = [&](int a) { return p.args[a].type; };
+  const ElemType out = p.output().type;
+  const bool hasMatmul = !ops.empty() && ops[0].code == OpCode::Matmul;
+
+  if (hasMatmul) {
+    // [matmul A B, push bias (d1), add, leaky alpha, store]
+    if (ops.size() == 5 && is_push(ops[1], 2, {1}) && ops[2].code == OpCode::Add &&
+        ops[3].code == OpCode::Leaky && ops[4].code == OpCode::Store) {
+      const int a = ops[0].arg, b = ops[0].arg2, bias = ops[1].arg;
+      if (type(a) == ElemType::BF16 && type(b) == ElemType::BF16 && type(bias) == ElemType::BF16 &&
+          out == ElemType::BF16) {
+        r->fast = FastPath::MatmulBiasLeaky;
+        r->fastArgs[0] = a; r->fastArgs[1] = b; r->fastArgs[2] = bias;
+        r->alpha = ops[3].constant;
+        return "";
+      }
+      return "matmul regions are implemented for bf16 A, B, bias and output; this one has other types";
+    }
+    return "a matmul region must be matmul -> bias add (per column) -> leaky relu; other epilogues are not implemented";
+  }
+  if (g.rank == 2 && ops.size() == 6 && out == ElemType::F32 && is_push(ops[0], 2, {0, 1}) &&
+      is_push(ops[1], 2, {0, 1}) && ops[2].code == OpCode::Add && is_push(ops[3], 2, {0, 1}) &&
+      ops[4].code == OpCode::Mul && type(ops[0].arg) == ElemType::F32 && type(ops[1].arg) == ElemType::F32 &&
+      (ops[3].arg == ops[0].arg || ops[3].arg == ops[1].arg) && ops[0].arg != ops[1].arg) {
+    // (x + y) * z with z one of x, y: out = (a + b) * b with b the repeated operand
+    r->fast = FastPath::AddMul;
+    r->fastArgs[1] = ops[3].arg;
+    r->fastArgs[0] = ops[3].arg == ops[0].arg ? ops[1].arg : ops[0].arg;
+    return "";
+  }
+  if (g.rank == 2 && ops.size() == 5 && out == ElemType::F32 && ops[2].code == OpCode::Add &&
+      ops[3].code == OpCode::ReduceSum) {
+    for (int swap = 0; swap < 2; ++swap) {
+      const afir_region::Op &x = ops[swap], &b = ops[1 - swap];
+      if (is_push(x, 2, {0, 1}) && is_push(b, 2, {1}) && type(x.arg) == ElemType::F32 &&
+          type(b.arg) == ElemType::F32) {
+        r->fast = FastPath::BcastAddRowsum;
+        r->fastArgs[0] = x.arg; r->fastArgs[1] = b.arg;
+        return "";
+      }
+    }
+  }
+  if (g.rank == 3 && ops.size() == 5 && out == ElemType::F16 && ops[3].code == OpCode::Add) {
+    // out[b,j,i] = relu(x[b,i,j]) + c[j]: x through (d0,d2,d1), c through (d1)
+    const afir_region::Op *x = nullptr, *c = nullptr;
+    if (is_push(ops[0], 3, {0, 2, 1}) && ops[1].code == OpCode::Relu && is_push(ops[2], 3, {1})) { x = &ops[0]; c = &ops[2]; }
+    if (is_push(ops[0], 3, {1}) && is_push(ops[1], 3, {0, 2, 1}) && ops[2].code == OpCode::Relu) { x = &ops[1]; c = &ops[0]; }
+    if (x && type(x->arg) == ElemType::F16 && type(c->arg) == ElemType::F16) {
+      r->fast = FastPath::ReluBcastTranspose;
+      r->fastArgs[0] = x->arg; r->fastArgs[1] = c->arg;
+      return "";
+    }
+  }
+  if (g.rank == 2 && ops.size() == 6 && out == ElemType::F16 && ops[2].code == OpCode::Mul &&
+      ops[4].code == OpCode::Add && is_push(ops[3], 2, {1})) {
+    for (int swap = 0; swap < 2; ++swap) {
+      const afir_region::Op &t = ops[swap], &sc = ops[1 - swap];
+      if (t.code == OpCode::Push && t.slice.empty() && t.map.size() == 2 &&
+          t.map[0].kind == MapResult::Gather && t.map[0].iterDim == 0 &&
+          t.map[1].kind == MapResult::IterDim && t.map[1].iterDim == 1 && is_push(sc, 2, {1}) &&
+          type(t.arg) == ElemType::F16 && type(sc.arg) == ElemType::F16 &&
+          type(ops[3].arg) == ElemType::F16 && type(t.map[0].indexArg) == ElemType::I32) {
+        r->fast = FastPath::GatherScaleShift;
+        r->fastArgs[0] = t.arg; r->fastArgs[1] = t.map[0].indexArg;
+        r->fastArgs[2] = sc.arg; r->fastArgs[3] = ops[3].arg;
+        return "";
+      }
+    }
+  }
+  return "";
+}
 std::mutex g_region_mutex;
 std::map<uint64_t, std::shared_ptr<RegisteredRegion>> g_regions;
 uint64_t g_next_region = 1;
@@ -203,6 +307,10 @@ uint32_t afir_hip_region_register(const char *program_text, size_t program_len, 
   std::string why = afir_region::parse(std::string(program_text, program_len), &r->program);
   if (!why.empty()) return fail(AFIR_HIP_E_INVALID, why);
   r->fields = afir_region::tilingFieldNames(r->program);
+  why = detect_fast_path(r.get());
+  if (!why.empty()) return fail(AFIR_HIP_E_INVALID, why);
+  if (const char *env = std::getenv("AFIR_HIP_REGION_GENERIC"))
+    if (*env && *env != '0' && r->fast != FastPath::MatmulBiasLeaky) r->fast = FastPath::None;
   std::lock_guard<std::mutex> lock(g_region_mutex);
   *handle = g_next_region++;
   g_regions[*handle] = std::move(r);
@@ -224,6 +332,20 @@ uint32_t afir_hip_region_info(uint64_t handle, int *num_inputs, int *num_outputs
   if (num_outputs) *num_outputs = 1;
   if (num_tiling_fields) *num_tiling_fields = (int)r->fields.size();
   return AFIR_HIP_OK;
+}
+
+const char *afir_hip_region_kernel(uint64_t handle) {
+  auto r = find_region(handle);
+  if (!r) return "";
+  switch (r->fast) {
+    case FastPath::AddMul: return "fused_add_mul";
+    case FastPath::BcastAddRowsum: return "broadcast_add_reducesum";
+    case FastPath::ReluBcastTranspose: return "relu_broadcast_add_transpose";
+    case FastPath::GatherScaleShift: return "gather_scale_shift";
+    case FastPath::MatmulBiasLeaky: return "matmul_add_leakyrelu";
+    case FastPath::None: break;
+  }
+  return "fused_region";
 }
 
 const char *afir_hip_region_tiling_field(uint64_t handle, int index) {
@@ -262,6 +384,41 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
   if (!why.empty()) return fail(AFIR_HIP_E_INVALID, why);
   for (int i = 0; i < want; ++i)
     if (res.bytes[i] && !args[i]) return fail(AFIR_HIP_E_INVALID, "region: null tensor pointer");
+
+  if (r->fast != FastPath::None) {
+    const afir_region::ResolvedSegment &seg = res.segments[0];
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int *fa = r->fastArgs;
+    void *out = args[want - 1];
+    switch (r->fast) {
+      case FastPath::AddMul:
+        return finish(afir::launch_fused_add_mul(static_cast<const float *>(args[fa[0]]),
+                                                 static_cast<const float *>(args[fa[1]]),
+                                                 static_cast<float *>(out), seg.size[0], seg.size[1],
+                                                 block_dim, st));
+      case FastPath::BcastAddRowsum:
+        return finish(afir::launch_broadcast_add_reducesum(
+            static_cast<const float *>(args[fa[0]]), static_cast<const float *>(args[fa[1]]),
+            static_cast<float *>(out), seg.size[0], seg.size[1], block_dim, st));
+      case FastPath::ReluBcastTranspose:
+        // iteration space (b, j, i) = output; x is [b, i, j]
+        return finish(afir::launch_relu_broadcast_add_transpose(
+            static_cast<const uint16_t *>(args[fa[0]]), static_cast<const uint16_t *>(args[fa[1]]),
+            static_cast<uint16_t *>(out), seg.size[0], seg.size[2], seg.size[1], block_dim, st));
+      case FastPath::GatherScaleShift:
+        return finish(afir::launch_gather_scale_shift(
+            static_cast<const uint16_t *>(args[fa[0]]), static_cast<const int32_t *>(args[fa[1]]),
+            static_cast<const uint16_t *>(args[fa[2]]), static_cast<const uint16_t *>(args[fa[3]]),
+            static_cast<uint16_t *>(out), static_cast<int32_t *>(workspace), res.shapes[fa[0]][0],
+            seg.size[1], seg.size[0], block_dim, st));
+      case FastPath::MatmulBiasLeaky:
+        return finish(afir::launch_matmul_add_leakyrelu(
+            static_cast<const uint16_t *>(args[fa[0]]), static_cast<const uint16_t *>(args[fa[1]]),
+            static_cast<const uint16_t *>(args[fa[2]]), static_cast<uint16_t *>(out), seg.size[0],
+            res.shapes[fa[0]][1], seg.size[1], r->alpha, block_dim, st));
+      case FastPath::None: break;
+    }
+  }
 
   auto aligned = [](const void *p, int64_t bytes) {
     return ((reinterpret_cast<uintptr_t>(p) + (uintptr_t)bytes) & 15u) == 0;

@@ -73,6 +73,7 @@ afirt::Status runDescriptor(ExecutorHandle *h, const std::string &descriptorText
   afirt::DynamicLibraryExecutionLaunch launch;
   launch.sharedLibraryPath = d->library.empty() ? afirt::defaultKernelLibraryPath() : d->library;
   launch.symbolName = d->symbol;
+  launch.regionProgram = d->program;
   return h->runner->runDynamicLibraryArtifact(launch, args);
 }
 

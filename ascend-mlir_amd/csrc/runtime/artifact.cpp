@@ -1,9 +1,11 @@
 // Artifact directories and run manifests.
 //
-// On this backend the fused kernels are precompiled in the kernel library, so
-// "compiling" a fused region means recognising which kernel family it is and
-// writing an artifact that names it:
-//     <root>/<kernel_name>.hipk      descriptor (key=value text)
+// On this backend the device code is precompiled in the kernel library, so
+// "compiling" a fused region means translating its IR to a region program
+// (csrc/target/mlir_translate.h) -- or taking an explicit request for one of
+// the hand-tuned kernel families -- and writing an artifact that carries it:
+//     <root>/<kernel_name>.hipk      descriptor (key=value text, then the
+//                                    region program after a "program:" line)
 //     <root>/out/manifest.txt        kernel_name= soc_version= kernel_kind=
 //                                    device_binary_path= manifest_path=
 //                                    kernel_so_path= kernel_so_symbol=
@@ -18,6 +20,7 @@
 #include <fstream>
 #include <sstream>
 
+#include "../target/mlir_translate.h"
 #include "runtime.h"
 
 namespace afirt {
@@ -53,6 +56,7 @@ const KnownKernel kKnown[] = {
     {"relu_broadcast_add_transpose", "afir_hip_launch_relu_broadcast_add_transpose", KernelKind::Vec},
     {"gather_scale_shift", "afir_hip_launch_gather_scale_shift", KernelKind::Vec},
     {"matmul_add_leakyrelu", "afir_hip_launch_matmul_add_leakyrelu", KernelKind::Mix},
+    {"fused_region", "afir_hip_launch_region", KernelKind::Vec},
 };
 
 const KnownKernel *findKnown(const std::string &name) {
@@ -123,75 +127,6 @@ std::string firstFuncName(const std::string &text) {
   return "";
 }
 
-// argument names of the first func.func, in order: (%a: ..., %b: ...) -> {"%a", "%b"}
-std::vector<std::string> firstFuncArgs(const std::string &text) {
-  std::vector<std::string> args;
-  size_t p = text.find("func.func");
-  if (p == std::string::npos) return args;
-  size_t open = text.find('(', p);
-  if (open == std::string::npos) return args;
-  int depth = 0;
-  size_t i = open;
-  std::string cur;
-  for (; i < text.size(); ++i) {
-    char c = text[i];
-    if (c == '(' || c == '<' || c == '[' || c == '{') {
-      if (depth++ > 0) cur += c;
-    } else if (c == ')' || c == '>' || c == ']' || c == '}') {
-      if (--depth == 0) break;
-      cur += c;
-    } else if (c == ',' && depth == 1) {
-      args.push_back(cur);
-      cur.clear();
-    } else {
-      cur += c;
-    }
-  }
-  if (!trim(cur).empty()) args.push_back(cur);
-  for (auto &a : args) {
-    size_t c = a.find("//");
-    while (c != std::string::npos) {  // drop trailing comments inside the signature
-      size_t nl = a.find('\n', c);
-      a.erase(c, nl == std::string::npos ? std::string::npos : nl - c);
-      c = a.find("//");
-    }
-    size_t colon = a.find(':');
-    a = trim(colon == std::string::npos ? a : a.substr(0, colon));
-  }
-  return args;
-}
-
-// %r = afir.<op> %x, %y ...   ->   (result, op, lhs, rhs)
-struct AfirBinary {
-  std::string result, op, lhs, rhs;
-};
-std::vector<AfirBinary> afirBinaries(const std::string &text) {
-  std::vector<AfirBinary> ops;
-  std::istringstream ss(text);
-  std::string line;
-  while (std::getline(ss, line)) {
-    size_t c = line.find("//");
-    if (c != std::string::npos) line = line.substr(0, c);
-    size_t p = line.find("afir.");
-    size_t eq = line.find('=');
-    if (p == std::string::npos || eq == std::string::npos || eq > p) continue;
-    AfirBinary b;
-    b.result = trim(line.substr(0, eq));
-    size_t e = p + 5;
-    while (e < line.size() && (isalnum((unsigned char)line[e]) || line[e] == '_')) ++e;
-    b.op = line.substr(p + 5, e - p - 5);
-    std::string rest = line.substr(e);
-    size_t stop = rest.find_first_of("{:");
-    if (stop != std::string::npos) rest = rest.substr(0, stop);
-    size_t comma = rest.find(',');
-    if (comma == std::string::npos) continue;
-    b.lhs = trim(rest.substr(0, comma));
-    b.rhs = trim(rest.substr(comma + 1));
-    if (!b.result.empty() && b.result[0] == '%' && !b.lhs.empty() && !b.rhs.empty()) ops.push_back(b);
-  }
-  return ops;
-}
-
 }  // namespace
 
 std::string defaultKernelLibraryPath() {
@@ -215,58 +150,78 @@ std::string serializeDescriptor(const HipKernelDescriptor &d) {
   s += "hip_kernel=" + d.hipKernel + "\n";
   s += "library=" + d.library + "\n";
   s += "symbol=" + d.symbol + "\n";
+  if (!d.program.empty()) s += "program:\n" + d.program;
   return s;
 }
 
 Expected<HipKernelDescriptor> parseDescriptor(const std::string &text) {
   if (text.compare(0, 17, "afir-hip-artifact") != 0)
     return Status::error("not an afir-hip artifact descriptor (missing 'afir-hip-artifact' header)");
-  auto kv = parseKeyValues(text.substr(text.find('\n') == std::string::npos ? text.size()
-                                                                           : text.find('\n') + 1));
+  std::string head = text, program;
+  const size_t mark = text.find("\nprogram:\n");
+  if (mark != std::string::npos) {
+    head = text.substr(0, mark + 1);
+    program = text.substr(mark + 10);
+  }
+  auto kv = parseKeyValues(head.substr(head.find('\n') == std::string::npos ? head.size()
+                                                                           : head.find('\n') + 1));
   HipKernelDescriptor d;
   d.kernelName = kv["kernel_name"];
   d.hipKernel = kv["hip_kernel"];
   d.library = kv["library"];
   d.symbol = kv["symbol"];
+  d.program = program;
   if (d.hipKernel.empty()) return Status::error("artifact descriptor names no hip_kernel");
   const KnownKernel *k = findKnown(d.hipKernel);
   if (!k) return Status::error("artifact descriptor names an unknown hip_kernel: " + d.hipKernel);
+  if ((d.hipKernel == "fused_region") != !d.program.empty())
+    return Status::error("artifact descriptor: a region program is required for fused_region and only there");
   if (d.symbol.empty()) d.symbol = k->symbol;
   if (d.kernelName.empty()) d.kernelName = d.hipKernel;
   return d;
 }
 
-Expected<std::string> selectHipKernel(const std::string &text, const std::string &nameHint) {
-  // 1. an explicit request
+Expected<HipKernelDescriptor> compileSourceText(const std::string &text, const std::string &nameHint) {
+  HipKernelDescriptor d;
+  // 1. an explicit request for a hand-tuned family
   for (const auto &kv : parseKeyValues(text))
     if (kv.first == "hip_kernel") {
-      if (!findKnown(kv.second)) return Status::error("unknown hip_kernel: " + kv.second);
-      return kv.second;
+      const KnownKernel *k = findKnown(kv.second);
+      if (!k || kv.second == "fused_region") return Status::error("unknown hip_kernel: " + kv.second);
+      d.hipKernel = kv.second;
+      d.symbol = k->symbol;
+      return d;
     }
-  // 2. the AFIR elementwise chain %1 = afir.mul(afir.add(%a, %b), %b)
-  //    (README.md:191-197 of the reference)
-  auto ops = afirBinaries(text);
-  if (ops.size() == 2 && ops[0].op == "add" && ops[1].op == "mul") {
-    // The kernel computes (in0 + in1) * in1 with inputs bound in function
-    // argument order, so the factor the product repeats must be the second
-    // argument (the sum itself commutes bit-exactly).
-    const auto &add = ops[0], &mul = ops[1];
-    const auto args = firstFuncArgs(text);
-    const std::string factor = mul.lhs == add.result ? mul.rhs : (mul.rhs == add.result ? mul.lhs : "");
-    const bool sum_of_args = args.size() == 2 && ((add.lhs == args[0] && add.rhs == args[1]) ||
-                                                  (add.lhs == args[1] && add.rhs == args[0]));
-    if (sum_of_args && factor == args[1]) return std::string("fused_add_mul");
-    return Status::error("afir add->mul chain is not of the form (arg0 + arg1) * arg1");
+  const std::string fn = firstFuncName(text);
+  // 2. a function with an empty or opaque body that is named after a family
+  // 3. MLIR text: translate the function to a region program
+  if (text.find("func.func") != std::string::npos) {
+    afir_target::Translation tr;
+    const std::string why = afir_target::translateMlirToRegion(text, &tr);
+    if (why.empty()) {
+      d.kernelName = tr.functionName;
+      d.hipKernel = "fused_region";
+      d.symbol = findKnown("fused_region")->symbol;
+      d.program = afir_region::serialize(tr.program);
+      return d;
+    }
+    if (const KnownKernel *k = findKnown(fn)) {
+      d.kernelName = fn;
+      d.hipKernel = fn;
+      d.symbol = k->symbol;
+      return d;
+    }
+    return Status::error("cannot lower kernel source to a fused HIP kernel: " + why);
   }
-  if (!ops.empty())
-    return Status::error("unsupported AFIR elementwise chain (" + std::to_string(ops.size()) +
-                         " ops); only afir.add -> afir.mul as (a + b) * b is lowered");
-  // 3. a function named after a kernel family
-  std::string fn = firstFuncName(text);
-  if (!fn.empty() && findKnown(fn)) return fn;
-  if (!nameHint.empty() && findKnown(nameHint)) return nameHint;
-  return Status::error("cannot map kernel source to a fused HIP kernel (function '" + fn +
-                       "'); known kernels: fused_add_mul, broadcast_add_reducesum, "
+  if (const KnownKernel *k = findKnown(nameHint)) {
+    if (nameHint != "fused_region") {
+      d.hipKernel = nameHint;
+      d.symbol = k->symbol;
+      return d;
+    }
+  }
+  return Status::error("cannot map kernel source to a fused HIP kernel: expected MLIR text (func.func) or "
+                       "'hip_kernel=<family>' with one of fused_add_mul, broadcast_add_reducesum, "
                        "relu_broadcast_add_transpose, gather_scale_shift, matmul_add_leakyrelu");
 }
 
@@ -275,22 +230,21 @@ Expected<KernelArtifact> compileArtifact(const CompileRequest &request) {
   if (request.outputDir.empty()) return Status::error("output directory is required");
   auto text = readTextFile(request.kernelSource);
   if (!text) return Status::error("cannot read kernel source: " + request.kernelSource);
-  auto family = selectHipKernel(*text, request.kernelName);
-  if (!family) return Status::error(family.error());
-  const KnownKernel *known = findKnown(*family);
+  auto compiled = compileSourceText(*text, request.kernelName);
+  if (!compiled) return Status::error(compiled.error());
+  const KnownKernel *known = findKnown(compiled->hipKernel);
 
   std::string name = request.kernelName;
+  if (name.empty()) name = compiled->kernelName;
   if (name.empty()) name = firstFuncName(*text);
-  if (name.empty()) name = *family;
+  if (name.empty()) name = compiled->hipKernel;
 
   if (!makeDirs(joinPath(request.outputDir, "out")))
     return Status::error("cannot create artifact manifest directory");
 
-  HipKernelDescriptor d;
+  HipKernelDescriptor d = *compiled;
   d.kernelName = name;
-  d.hipKernel = *family;
   d.library = defaultKernelLibraryPath();
-  d.symbol = known->symbol;
   const std::string binRel = name + ".hipk";
   const std::string binPath = joinPath(request.outputDir, binRel);
   {
@@ -300,7 +254,9 @@ Expected<KernelArtifact> compileArtifact(const CompileRequest &request) {
   }
   KernelArtifact a;
   a.kernelName = name;
-  a.kernelKind = request.kernelKind ? *request.kernelKind : known->kind;
+  a.kernelKind = request.kernelKind ? *request.kernelKind
+                 : (d.program.find("\nmatmul ") != std::string::npos ? KernelKind::Mix : known->kind);
+  a.regionProgram = d.program;
   a.socVersion = request.socVersion.empty() ? "gfx950" : request.socVersion;
   a.artifactRoot = request.outputDir;
   a.deviceBinaryPath = binPath;
@@ -352,6 +308,7 @@ Expected<KernelArtifact> loadArtifactFromRoot(const std::string &root) {
   if (a.sharedLibraryPath.empty()) a.sharedLibraryPath = d->library;
   if (a.sharedLibraryPath.empty()) a.sharedLibraryPath = defaultKernelLibraryPath();
   if (a.sharedLibrarySymbol.empty()) a.sharedLibrarySymbol = d->symbol;
+  a.regionProgram = d->program;
   return a;
 }
 

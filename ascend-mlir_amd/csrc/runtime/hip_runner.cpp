@@ -41,6 +41,12 @@ using LastErrorFn = const char *(*)();
 using KernelCountFn = int (*)();
 using KernelInfoFn = const KernelInfoView *(*)(int);
 using ArgBytesFn = uint32_t (*)(const char *, const void *, size_t, size_t *, int);
+using RegionRegisterFn = uint32_t (*)(const char *, size_t, uint64_t *);
+using RegionUnregisterFn = uint32_t (*)(uint64_t);
+using RegionInfoFn = uint32_t (*)(uint64_t, int *, int *, int *);
+using RegionBytesFn = uint32_t (*)(uint64_t, const void *, size_t, size_t *, int);
+using RegionLaunchFn = uint32_t (*)(uint64_t, uint32_t, void *, int, void *const *, void *,
+                                    const void *, size_t);
 
 std::string hipErr(const char *what, hipError_t e) {
   return std::string(what) + " failed: " + hipGetErrorString(e);
@@ -87,6 +93,7 @@ class HipExecutionRunner final : public ExecutionRunner {
     DynamicLibraryExecutionLaunch dl;
     dl.sharedLibraryPath = d->library.empty() ? defaultKernelLibraryPath() : d->library;
     dl.symbolName = d->symbol;
+    dl.regionProgram = d->program;
     return runDynamicLibraryArtifact(dl, args);
   }
 
@@ -106,15 +113,38 @@ class HipExecutionRunner final : public ExecutionRunner {
       ~LibGuard() { dlclose(h); }
     } libGuard{lib};
 
-    auto launchFn = reinterpret_cast<LaunchFn16>(dlsym(lib, launch.symbolName.c_str()));
-    if (!launchFn) {
-      const char *err = dlerror();
-      return Status::error("dlsym " + launch.symbolName + " failed: " + (err ? err : "unknown"));
-    }
     auto lastError = reinterpret_cast<LastErrorFn>(dlsym(lib, "afir_hip_last_error"));
-
-    // ---- host-side validation against the shapes in the tiling bytes ----
-    if (Status st = validate(lib, launch.symbolName, args); !st.ok()) return st;
+    LaunchFn16 launchFn = nullptr;
+    RegionLaunchFn regionLaunch = nullptr;
+    uint64_t region = 0;
+    struct RegionGuard {  // the registration lives for one run, like the library handle
+      RegionUnregisterFn fn = nullptr;
+      uint64_t handle = 0;
+      ~RegionGuard() { if (fn && handle) fn(handle); }
+    } regionGuard;
+    if (launch.regionProgram.empty()) {
+      launchFn = reinterpret_cast<LaunchFn16>(dlsym(lib, launch.symbolName.c_str()));
+      if (!launchFn) {
+        const char *err = dlerror();
+        return Status::error("dlsym " + launch.symbolName + " failed: " + (err ? err : "unknown"));
+      }
+      // ---- host-side validation against the shapes in the tiling bytes ----
+      if (Status st = validate(lib, launch.symbolName, args); !st.ok()) return st;
+    } else {
+      // A region program stands where the reference has a device binary:
+      // register it, check the buffers against the shapes, launch by handle.
+      auto reg = reinterpret_cast<RegionRegisterFn>(dlsym(lib, "afir_hip_region_register"));
+      auto unreg = reinterpret_cast<RegionUnregisterFn>(dlsym(lib, "afir_hip_region_unregister"));
+      regionLaunch = reinterpret_cast<RegionLaunchFn>(dlsym(lib, "afir_hip_launch_region"));
+      if (!reg || !unreg || !regionLaunch)
+        return Status::error("library has no fused-region entry points (afir_hip_region_register)");
+      auto why = [&]() { return std::string(lastError ? lastError() : ""); };
+      if (reg(launch.regionProgram.data(), launch.regionProgram.size(), &region) != 0)
+        return Status::error("invalid region program in artifact: " + why());
+      regionGuard.fn = unreg;
+      regionGuard.handle = region;
+      if (Status st = validateRegion(lib, region, args, why); !st.ok()) return st;
+    }
 
     // ---- device buffers ----
     std::vector<void *> allocs;
@@ -163,10 +193,17 @@ class HipExecutionRunner final : public ExecutionRunner {
 
     // ---- launch ----
     (void)hipEventRecord(ev0_, stream_);
-    const uint32_t rc = launchFn((uint32_t)(args.block_dim < 0 ? 0 : args.block_dim), stream_,
-                                 slots[0], slots[1], slots[2], slots[3], slots[4], slots[5],
-                                 slots[6], slots[7], slots[8], slots[9], slots[10], slots[11],
-                                 slots[12], slots[13], slots[14], slots[15]);
+    const uint32_t bd = (uint32_t)(args.block_dim < 0 ? 0 : args.block_dim);
+    uint32_t rc;
+    if (regionLaunch) {
+      const int nargs = (int)(args.inputs.size() + args.outputs.size());
+      rc = regionLaunch(region, bd, stream_, nargs, slots, workspace, args.tiling.data(),
+                        args.tiling.size());
+    } else {
+      rc = launchFn(bd, stream_, slots[0], slots[1], slots[2], slots[3], slots[4], slots[5],
+                    slots[6], slots[7], slots[8], slots[9], slots[10], slots[11], slots[12],
+                    slots[13], slots[14], slots[15]);
+    }
     if (rc != 0) {
       std::string why = lastError ? lastError() : "";
       (void)hipStreamSynchronize(stream_);
@@ -238,6 +275,36 @@ class HipExecutionRunner final : public ExecutionRunner {
                                     info->name, i, args.outputs[i].nbytes(), w));
       if (w && !args.outputs[i].data)
         return Status::error(format("%s: output %zu has no buffer", info->name, i));
+    }
+    return Status::success();
+  }
+
+  template <typename Why>
+  Status validateRegion(void *lib, uint64_t region, const RunArgs &args, Why why) {
+    auto infoFn = reinterpret_cast<RegionInfoFn>(dlsym(lib, "afir_hip_region_info"));
+    auto bytesFn = reinterpret_cast<RegionBytesFn>(dlsym(lib, "afir_hip_region_argument_bytes"));
+    if (!infoFn || !bytesFn) return Status::error("library cannot describe region programs");
+    int nin = 0, nout = 0, nfields = 0;
+    if (infoFn(region, &nin, &nout, &nfields) != 0) return Status::error(why());
+    if ((int)args.inputs.size() != nin)
+      return Status::error(format("region expects %d inputs, got %zu", nin, args.inputs.size()));
+    if ((int)args.outputs.size() != nout)
+      return Status::error(format("region expects %d outputs, got %zu", nout, args.outputs.size()));
+    size_t want[16] = {};
+    if (bytesFn(region, args.tiling.data(), args.tiling.size(), want, 16) != 0)
+      return Status::error("invalid tiling data: " + why());
+    for (size_t i = 0; i < args.inputs.size(); ++i) {
+      if (args.inputs[i].nbytes() != want[i])
+        return Status::error(format("region: input %zu holds %zu bytes, the tiling data implies %zu",
+                                    i, args.inputs[i].nbytes(), want[i]));
+      if (want[i] && !args.inputs[i].data) return Status::error(format("region: input %zu has no data", i));
+    }
+    for (size_t i = 0; i < args.outputs.size(); ++i) {
+      const size_t w = want[args.inputs.size() + i];
+      if (args.outputs[i].nbytes() != w)
+        return Status::error(format("region: output %zu holds %zu bytes, the tiling data implies %zu",
+                                    i, args.outputs[i].nbytes(), w));
+      if (w && !args.outputs[i].data) return Status::error(format("region: output %zu has no buffer", i));
     }
     return Status::success();
   }

@@ -180,6 +180,7 @@ struct KernelArtifact {
   std::string sharedLibraryPath;    // library exporting the launcher
   std::string sharedLibrarySymbol;  // launcher symbol
   std::string manifestPath;         // <root>/out/manifest.txt
+  std::string regionProgram;        // fused_region artifacts: the program text
 };
 
 // The descriptor a "compiled" fused region consists of on this backend: the
@@ -189,6 +190,7 @@ struct HipKernelDescriptor {
   std::string hipKernel;    // family name in the kernel library's registry
   std::string library;      // path or soname of the kernel library ("" = default)
   std::string symbol;       // launcher symbol
+  std::string program;      // hip_kernel == "fused_region": the region program text
 };
 std::string serializeDescriptor(const HipKernelDescriptor &d);
 Expected<HipKernelDescriptor> parseDescriptor(const std::string &text);
@@ -203,8 +205,11 @@ struct CompileRequest {
 // Source -> artifact directory: <out>/<name>.hipk + <out>/out/manifest.txt.
 Expected<KernelArtifact> compileArtifact(const CompileRequest &request);
 Expected<KernelArtifact> loadArtifactFromRoot(const std::string &artifactRoot);
-// Which fused-kernel family a source text asks for (see artifact.cpp).
-Expected<std::string> selectHipKernel(const std::string &sourceText, const std::string &nameHint);
+// What a kernel source compiles to: an explicit `hip_kernel=<family>` request
+// or a function named after a family gives that family; MLIR text (linalg /
+// AFIR) is translated to a fused-region program (csrc/target/mlir_translate.h).
+Expected<HipKernelDescriptor> compileSourceText(const std::string &sourceText,
+                                                const std::string &nameHint);
 
 // Location of libafir_hip_kernels.so: $AFIR_HIP_KERNELS_LIB, else next to this
 // library, else the bare soname for the dynamic loader to resolve.
@@ -254,6 +259,10 @@ struct FileExecutionLaunch {
 struct DynamicLibraryExecutionLaunch {
   std::string sharedLibraryPath;
   std::string symbolName;
+  // Non-empty: the artifact is a fused-region program.  It is registered with
+  // the library (afir_hip_region_register) and launched by handle instead of
+  // through a 16-slot launcher symbol.
+  std::string regionProgram;
 };
 
 class ExecutionRunner {

@@ -90,6 +90,7 @@ SessionSummary runSingleTask(const RunTaskSpec &task, RunnerFactory factory, int
   DynamicLibraryExecutionLaunch launch;
   launch.sharedLibraryPath = artifact->sharedLibraryPath;
   launch.symbolName = artifact->sharedLibrarySymbol;
+  launch.regionProgram = artifact->regionProgram;
   if (Status st = runner->runDynamicLibraryArtifact(launch, args); !st.ok())
     return fail(summary, "kernel_launch", st.message);
   const double us = runner->lastKernelMicroseconds();

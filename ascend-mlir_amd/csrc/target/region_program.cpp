@@ -132,6 +132,9 @@ std::string serialize(const Program &p) {
           s += "\n";
           break;
         }
+        case OpCode::Matmul:
+          s += "matmul arg" + std::to_string(o.arg) + " arg" + std::to_string(o.arg2) + "\n";
+          break;
         case OpCode::Const: s += "const " + floatText(o.constant) + "\n"; break;
         case OpCode::Leaky: s += "leaky " + floatText(o.constant) + "\n"; break;
         case OpCode::Dup: s += "dup " + std::to_string(o.depth) + "\n"; break;
@@ -233,6 +236,12 @@ std::string parse(const std::string &text, Program *out) {
         }
       }
       seg->ops.push_back(o);
+    } else if (k == "matmul") {
+      Op o;
+      o.code = OpCode::Matmul;
+      if (tok.size() != 3 || !parseArgName(tok[1], &o.arg) || !parseArgName(tok[2], &o.arg2))
+        return err(lineno, "expected 'matmul arg<A> arg<B>'");
+      seg->ops.push_back(o);
     } else if (k == "const" || k == "leaky") {
       Op o;
       o.code = k == "const" ? OpCode::Const : OpCode::Leaky;
@@ -331,6 +340,15 @@ std::string validate(const Program &p) {
           ++pushes;
           break;
         }
+        case OpCode::Matmul: {
+          if (i != 0 || g.rank != 2) return "region program: 'matmul' must open a rank-2 segment";
+          for (int a : {o.arg, o.arg2}) {
+            if (a < 0 || a >= p.numInputs()) return "region program: matmul of a non-input argument";
+            if (p.args[a].rank != 2 || !isFloat(p.args[a].type)) return "region program: matmul operands must be rank-2 float tensors";
+          }
+          ++depth;
+          break;
+        }
         case OpCode::Const: ++depth; break;
         case OpCode::Dup:
           if (o.depth < 0 || o.depth >= depth) return "region program: dup beyond the stack";
@@ -417,6 +435,14 @@ std::string resolve(const Program &p, const std::vector<int64_t> &dims, Resolved
       ro.code = o.code;
       ro.constant = o.constant;
       ro.depth = o.depth;
+      if (o.code == OpCode::Matmul) {
+        const std::vector<int64_t> &sa = r.shapes[o.arg], &sb = r.shapes[o.arg2];
+        if (sa[0] != s.size[0] || sb[1] != s.size[1] || sa[1] != sb[0])
+          return "region: matmul operand shapes do not agree with the segment";
+        ro.arg = o.arg;
+        ro.arg2 = o.arg2;
+        ro.k = sa[1];
+      }
       if (o.code == OpCode::Push) {
         const std::vector<int64_t> &shape = r.shapes[o.arg];
         ResolvedInput in;

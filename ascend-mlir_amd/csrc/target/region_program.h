@@ -31,6 +31,8 @@
 //                               integer constant, or g<k>:argI (dim r is indexed
 //                               by the rank-1 index tensor I at iteration dim k)
 //                               slice: per-dim start offsets of an extract_slice
+//     matmul argA argB          push sum_k A[d0,k] * B[k,d1] (float32 accumulation);
+//                               only as the first operation of a rank-2 segment
 //     const <float>             push a constant
 //     add | sub | mul | div | max | min      pop b, pop a, push a op b
 //     relu | leaky <alpha> | neg             on the top of the stack
@@ -72,7 +74,7 @@ struct Ref {
   static Ref value(int64_t c) { Ref r; r.constant = c; return r; }
 };
 
-enum class OpCode { Push, Const, Add, Sub, Mul, Div, Max, Min, Relu, Leaky, Neg, Dup, ReduceSum, Store };
+enum class OpCode { Push, Const, Add, Sub, Mul, Div, Max, Min, Relu, Leaky, Neg, Dup, ReduceSum, Store, Matmul };
 
 struct MapResult {
   enum Kind { IterDim, Constant, Gather } kind = IterDim;
@@ -83,7 +85,8 @@ struct MapResult {
 
 struct Op {
   OpCode code = OpCode::Add;
-  int arg = -1;                     // Push
+  int arg = -1;                     // Push; Matmul: the [M,K] operand
+  int arg2 = -1;                    // Matmul: the [K,N] operand
   std::vector<MapResult> map;       // Push: one per dim of the input
   std::vector<Ref> slice;           // Push: start offset per dim (empty = none)
   float constant = 0.f;             // Const, Leaky
@@ -134,6 +137,8 @@ struct ResolvedInput {
 struct ResolvedOp {
   OpCode code = OpCode::Add;
   int input = -1;      // Push: index into ResolvedSegment::inputs
+  int arg = -1, arg2 = -1;  // Matmul: argument indices
+  int64_t k = 0;            // Matmul: contraction extent
   float constant = 0.f;
   int depth = 0;
 };

@@ -1,0 +1,90 @@
+// afir-translate -mlir-to-hip: prints the fused-region program a function of
+// MLIR text lowers to on the HIP backend -- the sibling of the reference's
+// `afir-translate -mlir-to-cann <step7.mlir> -o kernel.cpp --tiling-space-out
+// tiling_space.json` (tools/afir-translate/afir-translate.cpp:19-41), which
+// prints AscendC kernel source.  Same flags; the output is the program text
+// that `runtime-session --kernel` stores in the artifact.
+//
+//   afir-translate -mlir-to-hip input.mlir [-o program.txt] [--tiling-space-out tiling_space.json]
+//
+// Exit codes: 0 ok, 1 the input cannot be lowered (diagnostic on stderr),
+// 2 usage / file errors.
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <iostream>
+#include <iterator>
+#include <string>
+
+#include "../target/mlir_translate.h"
+
+int main(int argc, char **argv) {
+  std::string input, output, tilingOut;
+  bool toHip = false;
+  for (int i = 1; i < argc; ++i) {
+    const std::string a = argv[i];
+    auto value = [&](const char *flag) -> const char * {
+      const size_t n = std::strlen(flag);
+      if (a.compare(0, n, flag) == 0 && a.size() > n && a[n] == '=') return argv[i] + n + 1;
+      if (a == flag && i + 1 < argc) return argv[++i];
+      return nullptr;
+    };
+    if (a == "-mlir-to-hip" || a == "--mlir-to-hip") {
+      toHip = true;
+    } else if (a == "-mlir-to-cann" || a == "--mlir-to-cann") {
+      std::fprintf(stderr, "afir-translate: this build emits for gfx950 only; use -mlir-to-hip\n");
+      return 2;
+    } else if (a == "-o" || a.compare(0, 3, "-o=") == 0) {
+      const char *v = value("-o");
+      if (!v) { std::fprintf(stderr, "afir-translate: -o needs a file name\n"); return 2; }
+      output = v;
+    } else if (a.compare(0, 18, "--tiling-space-out") == 0) {
+      const char *v = value("--tiling-space-out");
+      if (!v) { std::fprintf(stderr, "afir-translate: --tiling-space-out needs a file name\n"); return 2; }
+      tilingOut = v;
+    } else if (a == "-h" || a == "--help") {
+      std::printf("usage: afir-translate -mlir-to-hip <input.mlir> [-o <file>] [--tiling-space-out <file>]\n");
+      return 0;
+    } else if (!a.empty() && a[0] == '-' && a != "-") {
+      std::fprintf(stderr, "afir-translate: unknown option %s\n", a.c_str());
+      return 2;
+    } else if (input.empty()) {
+      input = a;
+    } else {
+      std::fprintf(stderr, "afir-translate: more than one input file\n");
+      return 2;
+    }
+  }
+  if (!toHip) {
+    std::fprintf(stderr, "afir-translate: no translation requested (-mlir-to-hip)\n");
+    return 2;
+  }
+  std::string text;
+  if (input.empty() || input == "-") {
+    text.assign(std::istreambuf_iterator<char>(std::cin), std::istreambuf_iterator<char>());
+  } else {
+    std::ifstream f(input, std::ios::binary);
+    if (!f) { std::fprintf(stderr, "afir-translate: cannot open %s\n", input.c_str()); return 2; }
+    text.assign(std::istreambuf_iterator<char>(f), std::istreambuf_iterator<char>());
+  }
+  afir_target::Translation tr;
+  const std::string why = afir_target::translateMlirToRegion(text, &tr);
+  if (!why.empty()) {
+    std::fprintf(stderr, "%s: error: %s\n", input.empty() ? "<stdin>" : input.c_str(), why.c_str());
+    return 1;
+  }
+  const std::string program = "# kernel " + tr.functionName + "\n" + afir_region::serialize(tr.program);
+  if (output.empty() || output == "-") {
+    std::fputs(program.c_str(), stdout);
+  } else {
+    std::ofstream f(output, std::ios::trunc);
+    if (!f) { std::fprintf(stderr, "afir-translate: cannot write %s\n", output.c_str()); return 2; }
+    f << program;
+  }
+  if (!tilingOut.empty()) {
+    std::ofstream f(tilingOut, std::ios::trunc);
+    if (!f) { std::fprintf(stderr, "afir-translate: cannot write %s\n", tilingOut.c_str()); return 2; }
+    f << afir_target::tilingSpaceJson(tr.program, tr.functionName);
+  }
+  return 0;
+}

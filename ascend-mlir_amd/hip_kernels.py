@@ -43,6 +43,7 @@ EXPORTED_SYMBOLS = [
     "afir_hip_region_unregister",
     "afir_hip_region_info",
     "afir_hip_region_tiling_field",
+    "afir_hip_region_kernel",
     "afir_hip_region_argument_bytes",
     "afir_hip_launch_region",
 ]
@@ -314,6 +315,9 @@ class Region:
         self.num_inputs, self.num_outputs = ni.value, no.value
         self.tiling_fields = [L.afir_hip_region_tiling_field(u64(self.handle), i).decode()
                               for i in range(nf.value)]
+        L.afir_hip_region_kernel.restype = ctypes.c_char_p
+        L.afir_hip_region_kernel.argtypes = [u64]
+        self.kernel = L.afir_hip_region_kernel(u64(self.handle)).decode()
         self.arg_types = [l.split()[2] for l in text.splitlines() if l.split()[:1] == ["arg"]]
 
     def close(self):

@@ -174,6 +174,12 @@ uint32_t afir_hip_region_register(const char *program_text, size_t program_len, 
 uint32_t afir_hip_region_unregister(uint64_t handle);
 uint32_t afir_hip_region_info(uint64_t handle, int *num_inputs, int *num_outputs,
                               int *num_tiling_fields);
+/* Which kernel runs the program: one of the family names above when the
+ * program is exactly that family (it is then routed to the hand-tuned kernel),
+ * else "fused_region" (the generic kernel).  Setting the environment variable
+ * AFIR_HIP_REGION_GENERIC=1 before registering keeps every non-matmul program
+ * on the generic kernel. */
+const char *afir_hip_region_kernel(uint64_t handle);
 /* Name of tiling field `index` ("" if out of range); valid until unregister. */
 const char *afir_hip_region_tiling_field(uint64_t handle, int index);
 uint32_t afir_hip_region_argument_bytes(uint64_t handle, const void *tiling, size_t tiling_len,

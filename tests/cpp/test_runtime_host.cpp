@@ -307,7 +307,8 @@ static void testArtifactsAndManifests() {
   auto a = compileArtifact(req);
   EXPECT((bool)a, "afir add->mul chain compiles");
   if (a) {
-    EXPECT(a->kernelName == "example" && a->sharedLibrarySymbol == "afir_hip_launch_fused_add_mul", "artifact fields");
+    EXPECT(a->kernelName == "example" && a->sharedLibrarySymbol == "afir_hip_launch_region" &&
+               a->regionProgram.find("push arg1 d0 d1\nmul\n") != std::string::npos, "artifact fields");
     auto text = readTextFile(a->manifestPath);
     EXPECT((bool)text && text->find("kernel_name=example\n") != std::string::npos &&
                text->find("kernel_kind=vec\n") != std::string::npos &&
@@ -315,25 +316,36 @@ static void testArtifactsAndManifests() {
                text->find("manifest_path=out/manifest.txt\n") != std::string::npos,
            "manifest keys");
     auto back = loadArtifactFromRoot(g_tmp + "/art");
-    EXPECT((bool)back && back->kernelName == "example" && back->sharedLibrarySymbol == a->sharedLibrarySymbol,
+    EXPECT((bool)back && back->kernelName == "example" && back->sharedLibrarySymbol == a->sharedLibrarySymbol &&
+               back->regionProgram == a->regionProgram,
            "artifact reloads");
   }
-  // (a + b) * a multiplies by the wrong argument: must be rejected, not mis-lowered
-  auto wrong = selectHipKernel("func.func @f(%a: tensor<4xf32>, %b: tensor<4xf32>) -> tensor<4xf32> {\n"
-                               "%0 = afir.add %a, %b : (tensor<4xf32>, tensor<4xf32>) -> tensor<4xf32>\n"
-                               "%1 = afir.mul %0, %a : (tensor<4xf32>, tensor<4xf32>) -> tensor<4xf32>\n}", "");
-  EXPECT(!wrong, "(a+b)*a is rejected");
-  auto three = selectHipKernel("func.func @f(%a: tensor<4xf32>, %b: tensor<4xf32>, %c: tensor<4xf32>) -> tensor<4xf32> {\n"
-                               "%0 = afir.add %a, %b : (tensor<4xf32>, tensor<4xf32>) -> tensor<4xf32>\n"
-                               "%1 = afir.mul %0, %c : (tensor<4xf32>, tensor<4xf32>) -> tensor<4xf32>\n}", "");
-  EXPECT(!three, "(a+b)*c is rejected");
-  auto commuted = selectHipKernel("func.func @f(%a: tensor<4xf32>, %b: tensor<4xf32>) -> tensor<4xf32> {\n"
-                                  "%0 = afir.add %b, %a : (tensor<4xf32>, tensor<4xf32>) -> tensor<4xf32>\n"
-                                  "%1 = afir.mul %b, %0 : (tensor<4xf32>, tensor<4xf32>) -> tensor<4xf32>\n}", "");
-  EXPECT((bool)commuted && *commuted == "fused_add_mul", "b*(b+a) is the same chain");
-  EXPECT((bool)selectHipKernel("hip_kernel=gather_scale_shift\n", ""), "explicit family");
-  EXPECT(!selectHipKernel("hip_kernel=nope\n", ""), "unknown family rejected");
-  EXPECT(!selectHipKernel("func.func @mystery() { return }", ""), "unknown function rejected");
+  // any AFIR chain lowers to a program; (a + b) * a keeps its own operand order
+  auto other = compileSourceText("func.func @f(%a: tensor<4xf32>, %b: tensor<4xf32>) -> tensor<4xf32> {\n"
+                                 "%0 = afir.add %a, %b : (tensor<4xf32>, tensor<4xf32>) -> tensor<4xf32>\n"
+                                 "%1 = afir.mul %0, %a : (tensor<4xf32>, tensor<4xf32>) -> tensor<4xf32>\n"
+                                 "return %1 : tensor<4xf32>\n}", "");
+  EXPECT((bool)other && other->hipKernel == "fused_region" &&
+             other->program.find("push arg0 d0\npush arg1 d0\nadd\npush arg0 d0\nmul\n") != std::string::npos,
+         "(a+b)*a lowers as written");
+  auto explicitFamily = compileSourceText("hip_kernel=gather_scale_shift\n", "");
+  EXPECT((bool)explicitFamily && explicitFamily->hipKernel == "gather_scale_shift" &&
+             explicitFamily->symbol == "afir_hip_launch_gather_scale_shift" && explicitFamily->program.empty(),
+         "explicit family");
+  EXPECT(!compileSourceText("hip_kernel=nope\n", ""), "unknown family rejected");
+  EXPECT(!compileSourceText("hip_kernel=fused_region\n", ""), "a region needs a program, not a name");
+  EXPECT(!compileSourceText("func.func @mystery() { return }", ""), "function without a tensor result rejected");
+  auto unsupported = compileSourceText("func.func @f(%a: tensor<4xf32>) -> tensor<4xf32> {\n"
+                                       "%0 = afir.exp %a : tensor<4xf32> -> tensor<4xf32>\nreturn %0 : tensor<4xf32>\n}", "");
+  EXPECT(!unsupported && unsupported.error().find("line 2") != std::string::npos &&
+             unsupported.error().find("afir.exp has no HIP lowering") != std::string::npos,
+         "unsupported op is named with its line");
+  {  // descriptor round trip with a program
+    HipKernelDescriptor d = *other;
+    d.kernelName = "k";
+    auto back = parseDescriptor(serializeDescriptor(d));
+    EXPECT((bool)back && back->program == d.program && back->hipKernel == "fused_region", "descriptor round trip");
+  }
   EXPECT(!loadArtifactFromRoot(g_tmp + "/no_such_root"), "missing artifact root");
   EXPECT(!parseDescriptor("ELF..."), "foreign binary rejected");
 

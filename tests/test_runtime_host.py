@@ -25,7 +25,9 @@ def test_cpp_host_tests(tmp_path):
     exe = tmp_path / "test_runtime_host"
     src = [os.path.join(ROOT, "tests", "cpp", "test_runtime_host.cpp"),
            os.path.join(PKG, "csrc", "runtime", "support.cpp"),
-           os.path.join(PKG, "csrc", "runtime", "artifact.cpp")]
+           os.path.join(PKG, "csrc", "runtime", "artifact.cpp"),
+           os.path.join(PKG, "csrc", "target", "region_program.cpp"),
+           os.path.join(PKG, "csrc", "target", "mlir_translate.cpp")]
     subprocess.run(["g++", "-std=c++17", "-O1", "-Wall", "-I", os.path.join(PKG, "csrc", "runtime"),
                     "-I", os.path.join(ROOT, "include"), *src, "-ldl", "-o", str(exe)], check=True)
     work = tmp_path / "w"
@@ -92,7 +94,7 @@ def test_capi_error_behaviour_without_gpu(pkg, tmp_path):
     bad.write_text("func.func @unknown_thing() { return }\n")
     assert L.afirt_compiler_compile(c, str(bad).encode(), str(tmp_path / "art2").encode(), b"", buf,
                                     len(buf)) == 1
-    assert b"cannot map kernel source" in buf.value
+    assert b"cannot lower kernel source" in buf.value
     L.afirt_compiler_destroy(c)
     L.afirt_compiler_destroy(None)
     L.afirt_executor_destroy(None)
@@ -104,9 +106,13 @@ def test_python_runtime_mirror(pkg, tmp_path):
     src.write_text(EXAMPLE_MLIR)
     path = R.compile_kernel(src, tmp_path / "art", "example")
     text = R.read_binary(path).decode()
-    assert text.startswith("afir-hip-artifact 1\n") and "hip_kernel=fused_add_mul" in text
+    assert text.startswith("afir-hip-artifact 1\n") and "hip_kernel=fused_region" in text
+    # the AFIR chain became a region program: (arg0 + arg1) * arg1
+    program = text.split("\nprogram:\n", 1)[1].split()
+    assert program[:3] == ["afir-hip-region", "1", "arg"]
+    assert " ".join(program).endswith("push arg0 d0 d1 push arg1 d0 d1 add push arg1 d0 d1 mul store end")
     manifest = (tmp_path / "art" / "out" / "manifest.txt").read_text()
-    assert "kernel_name=example" in manifest and "kernel_so_symbol=afir_hip_launch_fused_add_mul" in manifest
+    assert "kernel_name=example" in manifest and "kernel_so_symbol=afir_hip_launch_region" in manifest
     with pytest.raises(R.CompilerError):
         R.compile_kernel(tmp_path / "missing.mlir", tmp_path / "a2", "x")
     ex = R.KernelExecutor()
@@ -154,6 +160,11 @@ def test_tiling_schema_python(pkg, schema_file, tmp_path):
 
 # --- runtime-session CLI contract --------------------------------------------
 
+# TilingData of the compiled example: every dim of every argument (a, b, out)
+TILING_FIELDS = ["dim_arg0_0", "dim_arg0_1", "dim_arg1_0", "dim_arg1_1", "dim_arg2_0", "dim_arg2_1"]
+TILING_PARAMS = ",".join(f"{n}=4" for n in TILING_FIELDS)
+
+
 def _rs(*args, cwd=None):
     return subprocess.run([RS, *args], capture_output=True, text=True, cwd=cwd)
 
@@ -164,12 +175,12 @@ def _manifest(tmp_path, expected=True, **over):
     np.save(tmp_path / "b.npy", np.ones((4, 4), np.float32))
     np.save(tmp_path / "exp.npy", np.zeros((4, 4), np.float32))
     (tmp_path / "ts.json").write_text(json.dumps(
-        {"tiling_params": [{"name": "dim_arg0_0"}, {"name": "dim_arg0_1"}]}))
+        {"tiling_params": [{"name": n} for n in TILING_FIELDS]}))
     m = {"task_id": "main", "backend": "hip", "artifact_root": str(tmp_path / "art"),
          "inputs": [{"name": "a", "path": str(tmp_path / "a.npy")},
                     {"name": "b", "path": str(tmp_path / "b.npy")}],
          "outputs": [{"name": "out", "path": str(tmp_path / "out.npy")}],
-         "tiling": {"schema": str(tmp_path / "ts.json"), "params": "dim_arg0_0=4,dim_arg0_1=4"},
+         "tiling": {"schema": str(tmp_path / "ts.json"), "params": TILING_PARAMS},
          "block_dim": 0, "atol": 0, "rtol": 0}
     if expected:
         m["expected_outputs"] = [{"name": "out", "path": str(tmp_path / "exp.npy")}]
@@ -207,7 +218,7 @@ def test_cli_run_with_testing_driver(tmp_path):
     assert p.returncode == 0, p.stderr
     lines = p.stdout.splitlines()
     for want in ("session.backend=hip", "session.result=success", "session.validation=pass",
-                 "session.profile.count=0", "session.runtime.counter.tiling_bytes=16"):
+                 "session.profile.count=0", "session.runtime.counter.tiling_bytes=48"):
         assert want in lines, p.stdout
     assert np.array_equal(np.load(tmp_path / "out.npy"), np.zeros((4, 4), np.float32))
     # no expected outputs: no validation line, shapes come from the output binding
