@@ -70,7 +70,7 @@ constexpr int kNumKernels = (int)(sizeof(kKernels) / sizeof(kKernels[0]));
 // Programs that are exactly one of the hand-tuned kernels are routed to it
 // (same arithmetic, faster data movement); everything else runs on the generic
 // region kernel.  Matmul programs have no generic form: they must match.
-enum class FastPath { None, AddMul, BcastAddRowsum, ReluBcastTranspose, GatherScaleShift, MatmulBiasLeaky };
+enum class FastPath { None, AddMul, BcastAddRowsum, ReluBcastTranspose, GatherScaleShift, MatmulBiasLeaky, MatmulBiasLeakyF16 };
 
 struct RegisteredRegion {
   afir_region::Program program;
@@ -119,7 +119,15 @@ std::string detect_fast_path(RegisteredRegion *r) {
         r->alpha = ops[3].constant;
         return "";
       }
-      return "matmul regions are implemented for bf16 A, B, bias and output; this one has other types";
+      if (type(a) == ElemType::F16 && type(b) == ElemType::F16 && type(bias) == ElemType::F32 &&
+          out == ElemType::F32) {
+        r->fast = FastPath::MatmulBiasLeakyF16;
+        r->fastArgs[0] = a; r->fastArgs[1] = b; r->fastArgs[2] = bias;
+        r->alpha = ops[3].constant;
+        return "";
+      }
+      return "matmul regions are implemented for bf16 A, B, bias, out and for f16 A, B with f32 bias, out; "
+             "this one has other types";
     }
     return "a matmul region must be matmul -> bias add (per column) -> leaky relu; other epilogues are not implemented";
   }
@@ -310,7 +318,8 @@ uint32_t afir_hip_region_register(const char *program_text, size_t program_len, 
   why = detect_fast_path(r.get());
   if (!why.empty()) return fail(AFIR_HIP_E_INVALID, why);
   if (const char *env = std::getenv("AFIR_HIP_REGION_GENERIC"))
-    if (*env && *env != '0' && r->fast != FastPath::MatmulBiasLeaky) r->fast = FastPath::None;
+    if (*env && *env != '0' && r->fast != FastPath::MatmulBiasLeaky && r->fast != FastPath::MatmulBiasLeakyF16)
+      r->fast = FastPath::None;
   std::lock_guard<std::mutex> lock(g_region_mutex);
   *handle = g_next_region++;
   g_regions[*handle] = std::move(r);
@@ -343,6 +352,7 @@ const char *afir_hip_region_kernel(uint64_t handle) {
     case FastPath::ReluBcastTranspose: return "relu_broadcast_add_transpose";
     case FastPath::GatherScaleShift: return "gather_scale_shift";
     case FastPath::MatmulBiasLeaky: return "matmul_add_leakyrelu";
+    case FastPath::MatmulBiasLeakyF16: return "matmul_add_leakyrelu_f16";
     case FastPath::None: break;
   }
   return "fused_region";
@@ -415,6 +425,11 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
         return finish(afir::launch_matmul_add_leakyrelu(
             static_cast<const uint16_t *>(args[fa[0]]), static_cast<const uint16_t *>(args[fa[1]]),
             static_cast<const uint16_t *>(args[fa[2]]), static_cast<uint16_t *>(out), seg.size[0],
+            res.shapes[fa[0]][1], seg.size[1], r->alpha, block_dim, st));
+      case FastPath::MatmulBiasLeakyF16:
+        return finish(afir::launch_matmul_add_leakyrelu_f16(
+            static_cast<const uint16_t *>(args[fa[0]]), static_cast<const uint16_t *>(args[fa[1]]),
+            static_cast<const float *>(args[fa[2]]), static_cast<float *>(out), seg.size[0],
             res.shapes[fa[0]][1], seg.size[1], r->alpha, block_dim, st));
       case FastPath::None: break;
     }

@@ -38,6 +38,12 @@ LaunchStatus launch_matmul_add_leakyrelu(const uint16_t *a, const uint16_t *b,
                                          int64_t k, int64_t n, float alpha,
                                          uint32_t block_dim, hipStream_t stream);
 
+// The same with f16 A, B and f32 bias, out (the types of the reference's matmul
+// example, examples/matmul-add-leakyrelu/step0_input.mlir:10-15).
+LaunchStatus launch_matmul_add_leakyrelu_f16(const uint16_t *a, const uint16_t *b, const float *bias,
+                                             float *out, int64_t m, int64_t k, int64_t n,
+                                             float alpha, uint32_t block_dim, hipStream_t stream);
+
 // Fast path of the matmul for tile-aligned shapes (matmul_dma.hip).
 bool matmul_dma_supported(int64_t m, int64_t k, int64_t n);
 LaunchStatus launch_matmul_dma(const uint16_t *a, const uint16_t *b, const uint16_t *bias,

@@ -52,10 +52,14 @@ __device__ __forceinline__ void map_tile(int p, int tiles_m, int tiles_n, int &t
   tn = within / gsize;
 }
 
-template <int WAVES_M, int WAVES_N, int TM, int TN>
-__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void matmul_bias_leakyrelu_bf16_mfma(
+// F16IO = false: A, B, bias, out are bf16.  F16IO = true: A, B are f16, bias
+// and out are f32 -- the types of the reference's own matmul example
+// (examples/matmul-add-leakyrelu/step0_input.mlir:10-15); same tiling, the
+// f16 MFMA, and an epilogue that stores the float32 value unrounded.
+template <int WAVES_M, int WAVES_N, int TM, int TN, bool F16IO>
+__global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void matmul_bias_leakyrelu_mfma(
     const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
-    const uint16_t *__restrict__ bias, uint16_t *__restrict__ out, int M, int K, int N,
+    const void *__restrict__ bias_v, void *__restrict__ out_v, int M, int K, int N,
     float alpha, int tiles_m, int tiles_n) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int BM = WAVES_M * TM * 32, BN = WAVES_N * TN * 32;
@@ -142,20 +146,26 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void matmul_bias_leakyrelu_b
       const int lrow = lane & 31, lk = lane >> 5;
 #pragma unroll
       for (int ks = 0; ks < kBK / 16; ++ks) {
-        bf16x8 fa[TM], fb[TN];
+        u32x4 fa[TM], fb[TN];
 #pragma unroll
         for (int i = 0; i < TM; ++i)
-          fa[i] = *reinterpret_cast<const bf16x8 *>(As + ((wm * TM + i) * 32 + lrow) * kPitch +
-                                                    (ks * 2 + lk) * 16);
+          fa[i] = *reinterpret_cast<const u32x4 *>(As + ((wm * TM + i) * 32 + lrow) * kPitch +
+                                                   (ks * 2 + lk) * 16);
 #pragma unroll
         for (int j = 0; j < TN; ++j)
-          fb[j] = *reinterpret_cast<const bf16x8 *>(Bs + ((wn * TN + j) * 32 + lrow) * kPitch +
-                                                    (ks * 2 + lk) * 16);
+          fb[j] = *reinterpret_cast<const u32x4 *>(Bs + ((wn * TN + j) * 32 + lrow) * kPitch +
+                                                   (ks * 2 + lk) * 16);
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
-          for (int j = 0; j < TN; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+          for (int j = 0; j < TN; ++j) {
+            if constexpr (F16IO)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                  __builtin_bit_cast(f16x8, fb[j]), __builtin_bit_cast(f16x8, fa[i]), acc[i][j], 0, 0, 0);
+            else
+              acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                  __builtin_bit_cast(bf16x8, fb[j]), __builtin_bit_cast(bf16x8, fa[i]), acc[i][j], 0, 0, 0);
+          }
       }
     };
 
@@ -177,9 +187,15 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void matmul_bias_leakyrelu_b
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int n = n0 + (wn * TN + j) * 32 + 8 * q + 4 * lq;
-        const u32x2 braw = *reinterpret_cast<const u32x2 *>(bias + n);
-        const float b0 = bf16_lo(braw.x), b1 = bf16_hi(braw.x);
-        const float b2 = bf16_lo(braw.y), b3 = bf16_hi(braw.y);
+        float b0, b1, b2, b3;
+        if constexpr (F16IO) {
+          const f32x4 bf = *reinterpret_cast<const f32x4 *>(static_cast<const float *>(bias_v) + n);
+          b0 = bf[0]; b1 = bf[1]; b2 = bf[2]; b3 = bf[3];
+        } else {
+          const u32x2 braw = *reinterpret_cast<const u32x2 *>(static_cast<const uint16_t *>(bias_v) + n);
+          b0 = bf16_lo(braw.x); b1 = bf16_hi(braw.x);
+          b2 = bf16_lo(braw.y); b3 = bf16_hi(braw.y);
+        }
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
           const int m = m0 + (wm * TM + i) * 32 + lm;
@@ -191,10 +207,15 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void matmul_bias_leakyrelu_b
           v1 = fmaxf(v1, v1 * alpha);
           v2 = fmaxf(v2, v2 * alpha);
           v3 = fmaxf(v3, v3 * alpha);
-          u32x2 w;
-          w.x = pack_bf16(v0, v1);
-          w.y = pack_bf16(v2, v3);
-          *reinterpret_cast<u32x2 *>(out + (int64_t)m * N + n) = w;
+          if constexpr (F16IO) {
+            const f32x4 w = {v0, v1, v2, v3};
+            *reinterpret_cast<f32x4 *>(static_cast<float *>(out_v) + (int64_t)m * N + n) = w;
+          } else {
+            u32x2 w;
+            w.x = pack_bf16(v0, v1);
+            w.y = pack_bf16(v2, v3);
+            *reinterpret_cast<u32x2 *>(static_cast<uint16_t *>(out_v) + (int64_t)m * N + n) = w;
+          }
         }
       }
     }
@@ -202,10 +223,15 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void matmul_bias_leakyrelu_b
 }
 
 // Any shape: 16x16 output tile per workgroup, f32 FMAs, bounds-checked.
-__global__ __launch_bounds__(256) void matmul_bias_leakyrelu_bf16_any(
+template <bool F16IO>
+__global__ __launch_bounds__(256) void matmul_bias_leakyrelu_any(
     const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
-    const uint16_t *__restrict__ bias, uint16_t *__restrict__ out, int M, int K, int N,
+    const void *__restrict__ bias_v, void *__restrict__ out_v, int M, int K, int N,
     float alpha, int tiles_m, int tiles_n) {
+  auto widen = [](uint16_t h) {
+    if constexpr (F16IO) return (float)__builtin_bit_cast(_Float16, h);
+    else return __uint_as_float((uint32_t)h << 16);
+  };
   __shared__ float As[16][17], Bs[16][17];
   const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
   for (int p = blockIdx.x; p < tiles_m * tiles_n; p += gridDim.x) {
@@ -213,29 +239,33 @@ __global__ __launch_bounds__(256) void matmul_bias_leakyrelu_bf16_any(
     float acc = 0.f;
     for (int k0 = 0; k0 < K; k0 += 16) {
       const int ka = k0 + tx, kb = k0 + ty;
-      As[ty][tx] = (m < M && ka < K) ? __uint_as_float((uint32_t)A[(int64_t)m * K + ka] << 16) : 0.f;
-      Bs[ty][tx] = (kb < K && n < N) ? __uint_as_float((uint32_t)B[(int64_t)kb * N + n] << 16) : 0.f;
+      As[ty][tx] = (m < M && ka < K) ? widen(A[(int64_t)m * K + ka]) : 0.f;
+      Bs[ty][tx] = (kb < K && n < N) ? widen(B[(int64_t)kb * N + n]) : 0.f;
       __syncthreads();
 #pragma unroll
       for (int kk = 0; kk < 16; ++kk) acc += As[ty][kk] * Bs[kk][tx];
       __syncthreads();
     }
     if (m < M && n < N) {
-      float v = acc + __uint_as_float((uint32_t)bias[n] << 16);
-      v = fmaxf(v, v * alpha);
-      out[(int64_t)m * N + n] = (uint16_t)f32_to_bf16_rne(v);
+      if constexpr (F16IO) {
+        float v = acc + static_cast<const float *>(bias_v)[n];
+        static_cast<float *>(out_v)[(int64_t)m * N + n] = fmaxf(v, v * alpha);
+      } else {
+        float v = acc + __uint_as_float((uint32_t) static_cast<const uint16_t *>(bias_v)[n] << 16);
+        v = fmaxf(v, v * alpha);
+        static_cast<uint16_t *>(out_v)[(int64_t)m * N + n] = (uint16_t)f32_to_bf16_rne(v);
+      }
     }
   }
 }
 
-template <int WAVES_M, int WAVES_N, int TM, int TN>
-LaunchStatus launch_mfma(const uint16_t *a, const uint16_t *b, const uint16_t *bias,
-                         uint16_t *out, int m, int k, int n, float alpha, uint32_t block_dim,
-                         hipStream_t stream) {
+template <int WAVES_M, int WAVES_N, int TM, int TN, bool F16IO>
+LaunchStatus launch_mfma(const uint16_t *a, const uint16_t *b, const void *bias, void *out, int m,
+                         int k, int n, float alpha, uint32_t block_dim, hipStream_t stream) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int BM = WAVES_M * TM * 32, BN = WAVES_N * TN * 32;
   constexpr size_t kLds = 2 * (size_t)(BM + BN) * kPitch;
-  auto kernel = matmul_bias_leakyrelu_bf16_mfma<WAVES_M, WAVES_N, TM, TN>;
+  auto kernel = matmul_bias_leakyrelu_mfma<WAVES_M, WAVES_N, TM, TN, F16IO>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize,
                                                (int)kLds);
@@ -250,10 +280,12 @@ LaunchStatus launch_mfma(const uint16_t *a, const uint16_t *b, const uint16_t *b
 
 }  // namespace
 
-LaunchStatus launch_matmul_add_leakyrelu(const uint16_t *a, const uint16_t *b,
-                                         const uint16_t *bias, uint16_t *out, int64_t m,
-                                         int64_t k, int64_t n, float alpha, uint32_t block_dim,
-                                         hipStream_t stream) {
+namespace {
+
+template <bool F16IO>
+LaunchStatus launch_matmul_any_io(const uint16_t *a, const uint16_t *b, const void *bias, void *out,
+                                  int64_t m, int64_t k, int64_t n, float alpha, uint32_t block_dim,
+                                  hipStream_t stream) {
   if (m < 0 || k < 0 || n < 0) return invalid("matmul_add_leakyrelu: negative extent");
   if (m == 0 || n == 0) return ok_status();
   if (!out || !bias) return invalid("matmul_add_leakyrelu: null tensor pointer");
@@ -264,21 +296,39 @@ LaunchStatus launch_matmul_add_leakyrelu(const uint16_t *a, const uint16_t *b,
     return invalid("matmul_add_leakyrelu: extent overflow");
 
   const bool al = aligned16(a) && aligned16(b) && aligned16(out) &&
-                  ((reinterpret_cast<uintptr_t>(bias) & 7u) == 0);
-  if (al && matmul_dma_supported(m, k, n))
-    return launch_matmul_dma(a, b, bias, out, (int)m, (int)k, (int)n, alpha, block_dim, stream);
+                  ((reinterpret_cast<uintptr_t>(bias) & (F16IO ? 15u : 7u)) == 0);
+  if constexpr (!F16IO) {
+    if (al && matmul_dma_supported(m, k, n))
+      return launch_matmul_dma(a, b, static_cast<const uint16_t *>(bias), static_cast<uint16_t *>(out),
+                               (int)m, (int)k, (int)n, alpha, block_dim, stream);
+  }
   if (al && k >= kBK && k % kBK == 0 && m % 256 == 0 && n % 256 == 0)
-    return launch_mfma<2, 4, 4, 2>(a, b, bias, out, (int)m, (int)k, (int)n, alpha, block_dim, stream);
+    return launch_mfma<2, 4, 4, 2, F16IO>(a, b, bias, out, (int)m, (int)k, (int)n, alpha, block_dim, stream);
   if (al && k >= kBK && k % kBK == 0 && m % 128 == 0 && n % 128 == 0)
-    return launch_mfma<2, 2, 2, 2>(a, b, bias, out, (int)m, (int)k, (int)n, alpha, block_dim, stream);
+    return launch_mfma<2, 2, 2, 2, F16IO>(a, b, bias, out, (int)m, (int)k, (int)n, alpha, block_dim, stream);
 
   const int tiles_m = (int)((m + 15) / 16), tiles_n = (int)((n + 15) / 16);
   int64_t blocks = (int64_t)tiles_m * tiles_n;
   if (block_dim) blocks = block_dim;
   if (blocks > 0x7fffffff) blocks = 0x7fffffff;
-  hipLaunchKernelGGL(matmul_bias_leakyrelu_bf16_any, dim3((unsigned)blocks), dim3(256), 0, stream,
+  hipLaunchKernelGGL(matmul_bias_leakyrelu_any<F16IO>, dim3((unsigned)blocks), dim3(256), 0, stream,
                      a, b, bias, out, (int)m, (int)k, (int)n, alpha, tiles_m, tiles_n);
   return after_launch();
+}
+
+}  // namespace
+
+LaunchStatus launch_matmul_add_leakyrelu(const uint16_t *a, const uint16_t *b,
+                                         const uint16_t *bias, uint16_t *out, int64_t m,
+                                         int64_t k, int64_t n, float alpha, uint32_t block_dim,
+                                         hipStream_t stream) {
+  return launch_matmul_any_io<false>(a, b, bias, out, m, k, n, alpha, block_dim, stream);
+}
+
+LaunchStatus launch_matmul_add_leakyrelu_f16(const uint16_t *a, const uint16_t *b, const float *bias,
+                                             float *out, int64_t m, int64_t k, int64_t n,
+                                             float alpha, uint32_t block_dim, hipStream_t stream) {
+  return launch_matmul_any_io<true>(a, b, bias, out, m, k, n, alpha, block_dim, stream);
 }
 
 }  // namespace afir

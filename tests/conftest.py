@@ -4,6 +4,15 @@ import sys
 
 import pytest
 
+# PyTorch ships its own copy of the HIP runtime under the same soname as the
+# system one the C-ABI libraries are linked against; whichever is loaded first
+# serves the whole process.  Tests use torch for device memory, so its copy has
+# to be the one: import it before any test loads a library.
+try:
+    import torch  # noqa: F401
+except ImportError:      # the CPU-only checks do not need it
+    torch = None
+
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)

@@ -1,0 +1,151 @@
+"""The reference's example graphs end to end on the GPU, the way its
+examples/*/run.sh drive them: kernel source (MLIR) -> runtime-session --kernel
+-> artifact; seeded .npy inputs + golden -> run manifest -> runtime-session
+--run-manifest --run; pass = the three session lines.  Shapes and tolerances
+are the examples' own (run.sh atol / rtol lines); the MLIR is this repository's
+text in the same syntax (tests/mlir_cases.py).  Needs a GPU."""
+import json
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from oracle import afir_oracle as O
+from tests import mlir_cases as MC
+from tests import region_cases as RC
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+RS = os.path.join(ROOT, "ascend-mlir_amd", "bin", "runtime-session")
+TR = os.path.join(ROOT, "ascend-mlir_amd", "bin", "afir-translate")
+
+
+def _matmul_f16_case(m=128, k=256, n=128, seed=42):
+    """Small integers: every product and partial sum is exact in float32, so
+    the golden is independent of the summation order
+    (examples/matmul-add-leakyrelu/gen_data.py:29-31)."""
+    rng = np.random.default_rng(seed)
+    a = rng.integers(-3, 4, (m, k)).astype(np.float16)
+    b = rng.integers(-3, 4, (k, n)).astype(np.float16)
+    bias = rng.integers(-8, 9, (n,)).astype(np.float32)
+    init = np.zeros((m, n), np.float32)
+    return None, [a, b, bias, init], O.matmul_bias_leakyrelu_f16(a, b, bias, 0.001)
+
+
+# (mlir, case, kernel kind, atol, rtol of the example's run.sh, bit-exact expected)
+EXAMPLES = {
+    "broadcast-add-reduce": (MC.ROW_BIAS_REDUCE, RC.case_reduce_rowbias, "vec", 10.0, 1e-2, False),
+    "relu-broadcast-transpose": (MC.RELU_COLUMN_ADD, RC.case_relu_col_add, "vec", 1e-2, 1e-2, True),
+    "gather-elementwise-fusion": (MC.RELU_GATHER_COLUMNS_ADD, RC.case_relu_colgather_add, "vec", 10.0, 1e-2, True),
+    "matmul-add-leakyrelu": (MC.MATMUL_BIAS_LEAKY_F16, _matmul_f16_case, "mix", 1.0, 1e-2, True),
+    "add-broadcast-concat": (MC.TWO_CHAINS_CONCAT, RC.case_add_broadcast_concat, "vec", 1e-3, 1e-3, True),
+    "split-relu-brc-add-mul": (MC.SPLIT_HALVES, RC.case_split_relu_brc_add_mul, "vec", 1e-3, 1e-3, True),
+}
+
+
+def _rs(*args):
+    return subprocess.run([RS, *args], capture_output=True, text=True, timeout=100)
+
+
+@pytest.mark.parametrize("example", sorted(EXAMPLES))
+def test_example_pipeline(tmp_path, example):
+    mlir, case, kind, atol, rtol, exact = EXAMPLES[example]
+    src = tmp_path / "step0_input.mlir"
+    src.write_text(mlir)
+    art = tmp_path / "artifact"
+    p = _rs("--kernel", str(src), "--kernel-kind", kind, "--output", str(art), "--name", "kernel0")
+    assert p.returncode == 0, p.stderr
+    assert f"kernel_kind={kind}" in (art / "out" / "manifest.txt").read_text().splitlines()
+    ts = tmp_path / "tiling_space.json"
+    assert subprocess.run([TR, "-mlir-to-hip", str(src), "-o", str(tmp_path / "program.txt"),
+                           "--tiling-space-out", str(ts)]).returncode == 0
+    _, inputs, want = case()
+    want = np.ascontiguousarray(want)     # fancy indexing may hand back Fortran order
+    bind = []
+    for i, x in enumerate(inputs):
+        np.save(tmp_path / f"input_{i}.npy", x)
+        bind.append({"name": f"in{i}", "path": str(tmp_path / f"input_{i}.npy")})
+    np.save(tmp_path / "output_expected.npy", want)
+    fields = [f["name"] for f in json.loads(ts.read_text())["tiling_params"]]
+    dims = [d for x in inputs for d in x.shape] + list(want.shape)
+    assert len(fields) == len(dims)
+    manifest = {
+        "task_id": "main", "backend": "hip", "artifact_root": str(art), "inputs": bind,
+        "outputs": [{"name": "out", "path": str(tmp_path / "output_actual.npy")}],
+        "expected_outputs": [{"name": "out", "path": str(tmp_path / "output_expected.npy")}],
+        "tiling": {"schema": str(ts), "params": ",".join(f"{k}={v}" for k, v in zip(fields, dims))},
+        "block_dim": 0, "workspace_size": 8192, "profiling": False, "atol": atol, "rtol": rtol}
+    (tmp_path / "run_manifest.json").write_text(json.dumps(manifest))
+    p = _rs("--run-manifest", str(tmp_path / "run_manifest.json"), "--run")
+    assert p.returncode == 0, p.stdout + p.stderr
+    lines = p.stdout.splitlines()
+    for line in ("session.backend=hip", "session.result=success", "session.validation=pass"):
+        assert line in lines, p.stdout
+    got = np.load(tmp_path / "output_actual.npy")
+    if exact:
+        assert got.tobytes() == want.tobytes()
+    else:   # float32 row sums in another order, rounded to f16: within one f16 ulp
+        assert np.all(np.abs(got.astype(np.float64) - want.astype(np.float64))
+                      <= 2.0 ** -10 * np.abs(want.astype(np.float64)) + 1e-3)
+
+
+def test_capi_runs_a_compiled_mlir_kernel(pkg, tmp_path):
+    """compile_kernel on MLIR text, then execute_kernel on host arrays: the
+    reference's python/test/test_runtime_e2e.py flow."""
+    from ascend_mlir_amd import runtime as R
+    src = tmp_path / "k.mlir"
+    src.write_text(MC.SPLIT_HALVES)
+    path = R.compile_kernel(src, tmp_path / "art", "split_halves")
+    _, inputs, want = RC.case_split_relu_brc_add_mul(64, 40)
+    dims = [d for x in inputs for d in x.shape] + list(want.shape)
+    import struct
+    tiling = struct.pack("<%dq" % len(dims), *dims)
+    ex = R.KernelExecutor(device_id=0)
+    out = ex.execute(R.read_binary(path), "split_halves", inputs, [np.empty_like(want)], tiling)
+    assert out[0].tobytes() == want.tobytes()
+    with pytest.raises(R.ExecutorError, match="tiling data implies"):
+        ex.execute(R.read_binary(path), "split_halves", inputs, [np.empty((10, 40), np.float16)], tiling)
+
+
+def test_fast_paths_and_generic_kernel_agree(pkg, monkeypatch):
+    """A program that is one of the hand-tuned kernels gives the same bits on
+    that kernel and on the generic one (row sums: same tolerance both ways)."""
+    import torch
+    from ascend_mlir_amd import hip_kernels as H
+    H.load()
+    for name, case in [("c1", RC.case_c1), ("c3", RC.case_c3), ("c4", RC.case_c4), ("c2", RC.case_c2)]:
+        text, inputs, want = case()
+        outs = {}
+        for generic in ("0", "1"):
+            monkeypatch.setenv("AFIR_HIP_REGION_GENERIC", generic)
+            r = H.Region(text)
+            assert (r.kernel == "fused_region") == (generic == "1")
+            dev = [torch.from_numpy(x).cuda() for x in inputs]
+            outs[generic] = r(*dev, out_shape=want.shape).cpu().numpy()
+            r.close()
+        if name == "c2":
+            assert np.allclose(outs["0"], outs["1"], rtol=1e-5, atol=1e-3)
+        else:
+            assert outs["0"].tobytes() == outs["1"].tobytes() == want.tobytes()
+
+
+def test_matmul_bf16_program_runs_on_the_mfma_kernel(pkg):
+    import torch
+    from ascend_mlir_amd import hip_kernels as H
+    H.load()
+    p = subprocess.run([TR, "-mlir-to-hip", "-"], input=MC.MATMUL_BIAS_LEAKY_BF16, capture_output=True, text=True)
+    assert p.returncode == 0, p.stderr
+    r = H.Region(p.stdout)
+    assert r.kernel == "matmul_add_leakyrelu"
+    a, b, bias = O.gen_c5(256, 512, 256)
+
+    def dev(bits):
+        return torch.from_numpy(bits.view(np.int16)).cuda().view(torch.bfloat16)
+    init = torch.zeros((256, 256), dtype=torch.bfloat16, device="cuda")
+    out = r(dev(a), dev(b), dev(bias), init, out_shape=(256, 256))
+    got = out.view(torch.int16).cpu().numpy().view(np.uint16)
+    res = O.compare_outputs([(got, "bf16")], [(O.golden_c5(a, b, bias, 0.01), "bf16")], 1e-5, 1e-2)
+    assert res["passed"], res
+    r.close()
