@@ -13,9 +13,14 @@
 // is broadcast along it, element loads for transposed or gathered operands),
 // evaluates the chain in float32 registers and rounds once to the output
 // type.  The program is wave-uniform (it lives in the kernel argument
-// segment), so interpreting it costs scalar branches only; the value stack is
-// four register vectors that are shifted on push and pop, which keeps every
-// register index static.
+// segment), so interpreting it costs scalar branches only.  The value stack is
+// four register vectors; the launcher resolves every operation's stack slot on
+// the host, so the kernel never shifts the stack: an operation is a scalar
+// switch on its slot and then straight-line vector code.  Rows and 8-element
+// chunks are assigned to lanes without a division (a row of at most 256
+// chunks takes a power-of-two group of lanes, longer rows take the whole
+// workgroup), and positions are 32-bit when every tensor is below 2^31
+// elements.
 #include "kernels.h"
 #include "region_launch.h"
 
@@ -54,163 +59,164 @@ __device__ __forceinline__ int64_t load_index(const void *base, int type, int64_
                             : static_cast<const int64_t *>(base)[i];
 }
 
-// One operand for the 8 elements j0..j0+7 of the innermost dim at outer
-// position (i0, i1).  `full`: all 8 elements exist.
-__device__ __forceinline__ void read_operand(const RegionInput &in, int last, int64_t i0,
-                                             int64_t i1, int64_t j0, int nvalid, bool full,
-                                             int32_t *error_flag, float (&v)[kVec]) {
-  // iteration position of element j0: the innermost dim is `last`
-  const int64_t x0 = last == 0 ? j0 : i0;
-  const int64_t x1 = last == 1 ? j0 : i1;
-  const int64_t x2 = last == 2 ? j0 : 0;
+// Iteration position of the first of a lane's 8 elements.
+template <typename I>
+struct Position {
+  I x0, x1, x2;  // index along iteration dims 0..2 (the innermost one holds j0)
+};
+
+// One operand for the 8 elements at `at`.  `full`: all 8 elements exist.
+template <typename I>
+__device__ __forceinline__ void read_operand(const RegionInput &in, int last, const Position<I> &at,
+                                             int nvalid, bool full, int32_t *error_flag,
+                                             float (&v)[kVec]) {
   // element position without the gathered dim
-  const int64_t pos0 = in.offset + x0 * in.stride[0] + x1 * in.stride[1] + x2 * in.stride[2];
-  int64_t pos = pos0;
-  const int64_t step = last == 0 ? in.stride[0] : (last == 1 ? in.stride[1] : in.stride[2]);
+  I pos = (I)in.offset + at.x0 * (I)in.stride[0] + at.x1 * (I)in.stride[1] + at.x2 * (I)in.stride[2];
+  const I step = (I)(last == 0 ? in.stride[0] : (last == 1 ? in.stride[1] : in.stride[2]));
   const float nan = __uint_as_float(0x7fc00000u);
 
-  if (in.gdim < 0) {
-    if (step == 1 && full && in.vec) {
-      load_vec(in.base, in.type, pos, v);
-    } else if (step == 0) {
-      const float x = load_elem(in.base, in.type, pos);
+  if (in.gdim >= 0 && in.gdim == last) {
+    // gathered along the innermost dim: one index per element
+    const I j0 = last == 0 ? at.x0 : (last == 1 ? at.x1 : at.x2);
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) v[e] = x;
-    } else {
-#pragma unroll
-      for (int e = 0; e < kVec; ++e) v[e] = (e < nvalid) ? load_elem(in.base, in.type, pos + e * step) : 0.f;
+    for (int e = 0; e < kVec; ++e) {
+      float x = 0.f;
+      if (e < nvalid) {
+        const int64_t g = load_index(in.index, in.gtype, (int64_t)j0 + e);
+        if (g < 0 || g >= in.gextent) {
+          if (error_flag) *error_flag = 1;
+          x = nan;
+        } else {
+          x = load_elem(in.base, in.type, (int64_t)pos + (int64_t)e * step + g * in.gstride);
+        }
+      }
+      v[e] = x;
     }
     return;
   }
-  if (in.gdim != last) {
+  bool vec = in.vec != 0;
+  int64_t p64 = (int64_t)pos;
+  if (in.gdim >= 0) {
     // the index is the same for the whole vector
-    const int64_t g = load_index(in.index, in.gtype, in.gdim == 0 ? x0 : (in.gdim == 1 ? x1 : x2));
+    const int64_t g = load_index(in.index, in.gtype,
+                                 (int64_t)(in.gdim == 0 ? at.x0 : (in.gdim == 1 ? at.x1 : at.x2)));
     if (g < 0 || g >= in.gextent) {
       if (error_flag) *error_flag = 1;
 #pragma unroll
       for (int e = 0; e < kVec; ++e) v[e] = nan;
       return;
     }
-    pos += g * in.gstride;
-    if (step == 1 && full && in.vec && in.gvec) {
-      load_vec(in.base, in.type, pos, v);
-    } else if (step == 0) {
-      const float x = load_elem(in.base, in.type, pos);
-#pragma unroll
-      for (int e = 0; e < kVec; ++e) v[e] = x;
-    } else {
-#pragma unroll
-      for (int e = 0; e < kVec; ++e) v[e] = (e < nvalid) ? load_elem(in.base, in.type, pos + e * step) : 0.f;
-    }
-    return;
+    p64 += g * in.gstride;
+    vec = vec && in.gvec;
   }
-  // gathered along the innermost dim: one index per element
+  if (step == 1 && full && vec) {
+    load_vec(in.base, in.type, p64, v);
+  } else if (step == 0) {
+    const float x = load_elem(in.base, in.type, p64);
 #pragma unroll
-  for (int e = 0; e < kVec; ++e) {
-    float x = 0.f;
-    if (e < nvalid) {
-      const int64_t g = load_index(in.index, in.gtype, j0 + e);
-      if (g < 0 || g >= in.gextent) {
-        if (error_flag) *error_flag = 1;
-        x = nan;
-      } else {
-        x = load_elem(in.base, in.type, pos + e * step + g * in.gstride);
-      }
-    }
-    v[e] = x;
+    for (int e = 0; e < kVec; ++e) v[e] = x;
+  } else {
+#pragma unroll
+    for (int e = 0; e < kVec; ++e)
+      v[e] = (e < nvalid) ? load_elem(in.base, in.type, p64 + (int64_t)e * step) : 0.f;
   }
 }
 
-// max / min with IEEE-754 maximum / minimum semantics (NaN propagates), as
-// arith.maximumf / numpy.maximum define them.
-__device__ __forceinline__ float fmax_nan(float a, float b) {
-  return (a != a) ? a : ((b != b) ? b : ((a > b) ? a : ((b > a) ? b : ((__float_as_uint(a) & 0x80000000u) ? b : a))));
-}
-__device__ __forceinline__ float fmin_nan(float a, float b) {
-  return (a != a) ? a : ((b != b) ? b : ((a < b) ? a : ((b < a) ? b : ((__float_as_uint(a) & 0x80000000u) ? a : b))));
+// max / min with IEEE-754 maximum / minimum semantics (NaN propagates, -0 < +0),
+// as arith.maximumf / arith.minimumf define them: v_maximum3_f32 / v_minimum3_f32.
+__device__ __forceinline__ float fmax_nan(float a, float b) { return __builtin_elementwise_maximum(a, b); }
+__device__ __forceinline__ float fmin_nan(float a, float b) { return __builtin_elementwise_minimum(a, b); }
+
+__device__ __forceinline__ void binary(int code, float (&a)[kVec], const float (&b)[kVec]) {
+  switch (code) {
+    case kRegionAdd:
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) a[e] = a[e] + b[e];
+      break;
+    case kRegionSub:
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) a[e] = a[e] - b[e];
+      break;
+    case kRegionMul:
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) a[e] = a[e] * b[e];
+      break;
+    case kRegionDiv:
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) a[e] = a[e] / b[e];
+      break;
+    case kRegionMax:
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) a[e] = fmax_nan(a[e], b[e]);
+      break;
+    default:
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) a[e] = fmin_nan(a[e], b[e]);
+      break;
+  }
 }
 
-// Evaluates the expression for 8 elements; the result is s0.
-__device__ __forceinline__ void evaluate(const RegionArgs &R, int last, int64_t i0, int64_t i1,
-                                         int64_t j0, int nvalid, bool full, float (&s0)[kVec]) {
+__device__ __forceinline__ void unary(int code, float c, float (&a)[kVec]) {
+  switch (code) {
+    case kRegionRelu:
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) a[e] = fmax_nan(a[e], 0.f);
+      break;
+    case kRegionLeaky:
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) a[e] = fmax_nan(a[e], a[e] * c);
+      break;
+    default:
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) a[e] = -a[e];
+      break;
+  }
+}
+
+__device__ __forceinline__ void assign(float (&d)[kVec], const float (&s)[kVec]) {
+#pragma unroll
+  for (int e = 0; e < kVec; ++e) d[e] = s[e];
+}
+
+// Evaluates the expression for 8 elements; the result ends up in slot 0.
+template <typename I>
+__device__ __forceinline__ void evaluate(const RegionArgs &R, int last, const Position<I> &at,
+                                         int nvalid, bool full, float (&s0)[kVec]) {
   float s1[kVec], s2[kVec], s3[kVec];
 #pragma unroll
   for (int e = 0; e < kVec; ++e) s0[e] = s1[e] = s2[e] = s3[e] = 0.f;
-  auto push = [&]() {
-#pragma unroll
-    for (int e = 0; e < kVec; ++e) { s3[e] = s2[e]; s2[e] = s1[e]; s1[e] = s0[e]; }
-  };
-  auto pop_below = [&]() {  // drop s1, shifting the rest up
-#pragma unroll
-    for (int e = 0; e < kVec; ++e) { s1[e] = s2[e]; s2[e] = s3[e]; }
-  };
   for (int pc = 0; pc < R.nops; ++pc) {
     const RegionOp op = R.ops[pc];
-    switch (op.code) {
-      case kRegionPush: {
-        push();
-        read_operand(R.in[op.input], last, i0, i1, j0, nvalid, full, R.error_flag, s0);
-        break;
+    if (op.code == kRegionPush || op.code == kRegionConst || op.code == kRegionDup) {
+      float t[kVec];
+      if (op.code == kRegionPush) {
+        read_operand<I>(R.in[op.input], last, at, nvalid, full, R.error_flag, t);
+      } else if (op.code == kRegionConst) {
+#pragma unroll
+        for (int e = 0; e < kVec; ++e) t[e] = op.constant;
+      } else {
+        const int src = op.dst - 1 - op.depth;
+        assign(t, src == 0 ? s0 : (src == 1 ? s1 : s2));
       }
-      case kRegionConst:
-        push();
-#pragma unroll
-        for (int e = 0; e < kVec; ++e) s0[e] = op.constant;
-        break;
-      case kRegionDup: {
-        float t[kVec];
-#pragma unroll
-        for (int e = 0; e < kVec; ++e)
-          t[e] = op.depth == 0 ? s0[e] : (op.depth == 1 ? s1[e] : (op.depth == 2 ? s2[e] : s3[e]));
-        push();
-#pragma unroll
-        for (int e = 0; e < kVec; ++e) s0[e] = t[e];
-        break;
+      switch (op.dst) {
+        case 0: assign(s0, t); break;
+        case 1: assign(s1, t); break;
+        case 2: assign(s2, t); break;
+        default: assign(s3, t); break;
       }
-      case kRegionAdd:
-#pragma unroll
-        for (int e = 0; e < kVec; ++e) s0[e] = s1[e] + s0[e];
-        pop_below();
-        break;
-      case kRegionSub:
-#pragma unroll
-        for (int e = 0; e < kVec; ++e) s0[e] = s1[e] - s0[e];
-        pop_below();
-        break;
-      case kRegionMul:
-#pragma unroll
-        for (int e = 0; e < kVec; ++e) s0[e] = s1[e] * s0[e];
-        pop_below();
-        break;
-      case kRegionDiv:
-#pragma unroll
-        for (int e = 0; e < kVec; ++e) s0[e] = s1[e] / s0[e];
-        pop_below();
-        break;
-      case kRegionMax:
-#pragma unroll
-        for (int e = 0; e < kVec; ++e) s0[e] = fmax_nan(s1[e], s0[e]);
-        pop_below();
-        break;
-      case kRegionMin:
-#pragma unroll
-        for (int e = 0; e < kVec; ++e) s0[e] = fmin_nan(s1[e], s0[e]);
-        pop_below();
-        break;
-      case kRegionRelu:
-#pragma unroll
-        for (int e = 0; e < kVec; ++e) s0[e] = fmax_nan(s0[e], 0.f);
-        break;
-      case kRegionLeaky:
-#pragma unroll
-        for (int e = 0; e < kVec; ++e) s0[e] = fmax_nan(s0[e], s0[e] * op.constant);
-        break;
-      case kRegionNeg:
-#pragma unroll
-        for (int e = 0; e < kVec; ++e) s0[e] = -s0[e];
-        break;
-      default:
-        break;
+    } else if (op.code <= kRegionMin) {   // binary: slot dst (op) slot dst + 1
+      switch (op.dst) {
+        case 0: binary(op.code, s0, s1); break;
+        case 1: binary(op.code, s1, s2); break;
+        default: binary(op.code, s2, s3); break;
+      }
+    } else {
+      switch (op.dst) {
+        case 0: unary(op.code, op.constant, s0); break;
+        case 1: unary(op.code, op.constant, s1); break;
+        case 2: unary(op.code, op.constant, s2); break;
+        default: unary(op.code, op.constant, s3); break;
+      }
     }
   }
 }
@@ -221,44 +227,65 @@ __device__ __forceinline__ void store_elem(void *out, int type, int64_t i, float
   else static_cast<uint16_t *>(out)[i] = (uint16_t)f32_to_bf16_rne(x);
 }
 
-__global__ __launch_bounds__(kThreads) void fused_region_parallel(const RegionArgs R) {
+template <typename I>
+__device__ __forceinline__ Position<I> position(const RegionArgs &R, I row, I j0) {
+  Position<I> p;
+  if (R.rank == 1) { p.x0 = j0; p.x1 = 0; p.x2 = 0; }
+  else if (R.rank == 2) { p.x0 = row; p.x1 = j0; p.x2 = 0; }
+  else {
+    // unsigned 32-bit division where it fits: an order of magnitude cheaper
+    // than the 64-bit one
+    if (sizeof(I) == 4) p.x0 = (I)((uint32_t)row / (uint32_t)R.size[1]);
+    else p.x0 = row / (I)R.size[1];
+    p.x1 = row - p.x0 * (I)R.size[1];
+    p.x2 = j0;
+  }
+  return p;
+}
+
+// lanes_log2: a row's chunks are spread over 2^lanes_log2 lanes of the
+// workgroup (8 = the whole workgroup walks one row at a time).
+template <typename I>
+__global__ __launch_bounds__(kThreads) void fused_region_parallel(const RegionArgs R, int lanes_log2) {
   const int last = R.rank - 1;
-  const int64_t n = R.size[last];
-  const int64_t chunks = (n + kVec - 1) / kVec;
-  const int64_t rows = (R.rank == 1) ? 1 : ((R.rank == 2) ? R.size[0] : R.size[0] * R.size[1]);
-  const int64_t items = rows * chunks;
-  const int64_t stride = (int64_t)gridDim.x * kThreads;
-  for (int64_t item = (int64_t)blockIdx.x * kThreads + threadIdx.x; item < items; item += stride) {
-    const int64_t row = item / chunks;
-    const int64_t j0 = (item - row * chunks) * kVec;
-    int64_t i0 = 0, i1 = 0;
-    if (R.rank == 2) i0 = row;
-    else if (R.rank == 3) { i0 = row / R.size[1]; i1 = row - i0 * R.size[1]; }
-    const int64_t left = n - j0;
-    const int nvalid = left >= kVec ? kVec : (int)left;
-    const bool full = nvalid == kVec;
-    float v[kVec];
-    evaluate(R, last, i0, i1, j0, nvalid, full, v);
-    const int64_t o = row * n + j0;
-    if (full && R.out_vec) {
-      if (R.out_type == kRegionF32) {
-        f32x4 a, b;
+  const I n = (I)R.size[last];
+  const I chunks = (n + kVec - 1) / kVec;
+  const I rows = (I)((R.rank == 1) ? 1 : ((R.rank == 2) ? R.size[0] : R.size[0] * R.size[1]));
+  const int lanes = 1 << lanes_log2;
+  const int rows_per_pass = kThreads >> lanes_log2;
+  const I local_row = (I)(threadIdx.x >> lanes_log2);
+  const I first_chunk = (I)(threadIdx.x & (lanes - 1));
+  for (I row0 = (I)blockIdx.x * rows_per_pass; row0 < rows; row0 += (I)gridDim.x * rows_per_pass) {
+    const I row = row0 + local_row;
+    if (row >= rows) continue;
+    for (I chunk = first_chunk; chunk < chunks; chunk += lanes) {
+      const I j0 = chunk * kVec;
+      const I left = n - j0;
+      const int nvalid = left >= kVec ? kVec : (int)left;
+      const bool full = nvalid == kVec;
+      float v[kVec];
+      evaluate<I>(R, last, position<I>(R, row, j0), nvalid, full, v);
+      const int64_t o = (int64_t)row * n + j0;
+      if (full && R.out_vec) {
+        if (R.out_type == kRegionF32) {
+          f32x4 a, b;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) { a[e] = v[e]; b[e] = v[4 + e]; }
-        f32x4 *p = reinterpret_cast<f32x4 *>(static_cast<float *>(R.out) + o);
-        p[0] = a;
-        p[1] = b;
+          for (int e = 0; e < 4; ++e) { a[e] = v[e]; b[e] = v[4 + e]; }
+          f32x4 *p = reinterpret_cast<f32x4 *>(static_cast<float *>(R.out) + o);
+          p[0] = a;
+          p[1] = b;
+        } else {
+          u32x4 w;
+#pragma unroll
+          for (int d = 0; d < 4; ++d)
+            w[d] = R.out_type == kRegionF16 ? pack_f16(v[2 * d], v[2 * d + 1]) : pack_bf16(v[2 * d], v[2 * d + 1]);
+          *reinterpret_cast<u32x4 *>(static_cast<uint16_t *>(R.out) + o) = w;
+        }
       } else {
-        u32x4 w;
 #pragma unroll
-        for (int d = 0; d < 4; ++d)
-          w[d] = R.out_type == kRegionF16 ? pack_f16(v[2 * d], v[2 * d + 1]) : pack_bf16(v[2 * d], v[2 * d + 1]);
-        *reinterpret_cast<u32x4 *>(static_cast<uint16_t *>(R.out) + o) = w;
+        for (int e = 0; e < kVec; ++e)
+          if (e < nvalid) store_elem(R.out, R.out_type, o + e, v[e]);
       }
-    } else {
-#pragma unroll
-      for (int e = 0; e < kVec; ++e)
-        if (e < nvalid) store_elem(R.out, R.out_type, o + e, v[e]);
     }
   }
 }
@@ -266,38 +293,38 @@ __global__ __launch_bounds__(kThreads) void fused_region_parallel(const RegionAr
 // Row sum over the innermost dim: one wavefront per output element, lanes
 // stride over the row in vectors of 8, float32 partial sums per vector slot,
 // fixed-order combination and a DPP wave reduction: deterministic.
+template <typename I>
 __global__ __launch_bounds__(kThreads) void fused_region_rowsum(const RegionArgs R) {
   const int last = R.rank - 1;
-  const int64_t n = R.size[last];
-  const int64_t chunks = (n + kVec - 1) / kVec;
-  const int64_t rows = (R.rank == 2) ? R.size[0] : R.size[0] * R.size[1];
+  const I n = (I)R.size[last];
+  const I chunks = (n + kVec - 1) / kVec;
+  const I rows = (I)((R.rank == 2) ? R.size[0] : R.size[0] * R.size[1]);
   const int lane = threadIdx.x & (kWave - 1);
-  const int64_t wave = (int64_t)blockIdx.x * (kThreads / kWave) + (threadIdx.x >> 6);
-  const int64_t nwaves = (int64_t)gridDim.x * (kThreads / kWave);
-  for (int64_t row = wave; row < rows; row += nwaves) {
-    int64_t i0 = row, i1 = 0;
-    if (R.rank == 3) { i0 = row / R.size[1]; i1 = row - i0 * R.size[1]; }
+  const I wave = (I)blockIdx.x * (kThreads / kWave) + (I)(threadIdx.x >> 6);
+  const I nwaves = (I)gridDim.x * (kThreads / kWave);
+  for (I row = wave; row < rows; row += nwaves) {
     float acc[kVec];
 #pragma unroll
     for (int e = 0; e < kVec; ++e) acc[e] = 0.f;
-    for (int64_t c = lane; c < chunks; c += kWave) {
-      const int64_t j0 = c * kVec;
-      const int64_t left = n - j0;
+    for (I c = lane; c < chunks; c += kWave) {
+      const I j0 = c * kVec;
+      const I left = n - j0;
       const int nvalid = left >= kVec ? kVec : (int)left;
       float v[kVec];
-      evaluate(R, last, i0, i1, j0, nvalid, nvalid == kVec, v);
+      evaluate<I>(R, last, position<I>(R, row, j0), nvalid, nvalid == kVec, v);
 #pragma unroll
       for (int e = 0; e < kVec; ++e) acc[e] += (e < nvalid) ? v[e] : 0.f;
     }
     float s = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
     s = wave_sum(s);
-    if (lane == 0) store_elem(R.out, R.out_type, row, s);
+    if (lane == 0) store_elem(R.out, R.out_type, (int64_t)row, s);
   }
 }
 
 }  // namespace
 
-LaunchStatus launch_fused_region(const RegionArgs &args, uint32_t block_dim, hipStream_t stream) {
+LaunchStatus launch_fused_region(const RegionArgs &args_in, uint32_t block_dim, hipStream_t stream) {
+  RegionArgs args = args_in;
   if (args.rank < 1 || args.rank > 3) return invalid("fused_region: bad iteration rank");
   if (args.nops < 0 || args.nops > kRegionMaxOps || args.ninputs < 0 || args.ninputs > kRegionMaxInputs)
     return invalid("fused_region: program too large");
@@ -308,6 +335,40 @@ LaunchStatus launch_fused_region(const RegionArgs &args, uint32_t block_dim, hip
     total *= args.size[k];
     if (k + 1 < args.rank) rows *= args.size[k];
   }
+  // stack slots: the interpreter does not shift values, every operation is
+  // told where its operands live
+  int depth = 0;
+  for (int i = 0; i < args.nops; ++i) {
+    RegionOp &op = args.ops[i];
+    if (op.code == kRegionPush || op.code == kRegionConst || op.code == kRegionDup) {
+      if (op.code == kRegionDup && (op.depth < 0 || op.depth >= depth)) return invalid("fused_region: dup beyond the stack");
+      op.dst = depth++;
+      if (depth > 4) return invalid("fused_region: more than 4 live values");
+      if (op.code == kRegionPush && (op.input < 0 || op.input >= args.ninputs)) return invalid("fused_region: bad operand");
+    } else if (op.code >= kRegionAdd && op.code <= kRegionMin) {
+      if (depth < 2) return invalid("fused_region: binary operation on fewer than two values");
+      op.dst = depth - 2;
+      --depth;
+    } else if (op.code == kRegionRelu || op.code == kRegionLeaky || op.code == kRegionNeg) {
+      if (depth < 1) return invalid("fused_region: unary operation on an empty stack");
+      op.dst = depth - 1;
+    } else {
+      return invalid("fused_region: unknown operation code");
+    }
+  }
+  if (depth != 1) return invalid("fused_region: the program must leave exactly one value");
+
+  // 32-bit positions when every operand and the output stay below 2^31 elements
+  bool idx32 = total < ((int64_t)1 << 31);
+  for (int i = 0; i < args.ninputs && idx32; ++i) {
+    int64_t reach = args.in[i].offset < 0 ? -args.in[i].offset : args.in[i].offset;
+    for (int k = 0; k < args.rank; ++k) {
+      const int64_t st = args.in[i].stride[k] < 0 ? -args.in[i].stride[k] : args.in[i].stride[k];
+      if (args.size[k] > 0 && st > (((int64_t)1 << 31) - 1 - reach) / args.size[k]) { idx32 = false; break; }
+      reach += st * (args.size[k] > 0 ? args.size[k] - 1 : 0);
+    }
+  }
+
   if (args.reduce) {
     if (args.rank < 2) return invalid("fused_region: reduction needs rank >= 2");
     if (rows == 0) return ok_status();
@@ -315,17 +376,26 @@ LaunchStatus launch_fused_region(const RegionArgs &args, uint32_t block_dim, hip
     int64_t blocks = (rows + (kThreads / kWave) - 1) / (kThreads / kWave);
     if (blocks > (int64_t)kNumCU * 8) blocks = (int64_t)kNumCU * 8;
     if (block_dim) blocks = block_dim;
-    hipLaunchKernelGGL(fused_region_rowsum, dim3((unsigned)blocks), dim3(kThreads), 0, stream, args);
+    if (idx32)
+      hipLaunchKernelGGL(fused_region_rowsum<int>, dim3((unsigned)blocks), dim3(kThreads), 0, stream, args);
+    else
+      hipLaunchKernelGGL(fused_region_rowsum<int64_t>, dim3((unsigned)blocks), dim3(kThreads), 0, stream, args);
     return after_launch();
   }
   if (total == 0) return ok_status();
   if (!args.out) return invalid("fused_region: null output pointer");
   const int64_t n = args.size[args.rank - 1];
-  const int64_t items = rows * ((n + kVec - 1) / kVec);
-  int64_t blocks = (items + kThreads - 1) / kThreads;
+  const int64_t chunks = (n + kVec - 1) / kVec;
+  int lanes_log2 = 0;
+  while (lanes_log2 < 8 && ((int64_t)1 << lanes_log2) < chunks) ++lanes_log2;
+  const int rows_per_pass = kThreads >> lanes_log2;
+  int64_t blocks = (rows + rows_per_pass - 1) / rows_per_pass;
   if (blocks > (int64_t)kNumCU * 16) blocks = (int64_t)kNumCU * 16;
   if (block_dim) blocks = block_dim;
-  hipLaunchKernelGGL(fused_region_parallel, dim3((unsigned)blocks), dim3(kThreads), 0, stream, args);
+  if (idx32)
+    hipLaunchKernelGGL(fused_region_parallel<int>, dim3((unsigned)blocks), dim3(kThreads), 0, stream, args, lanes_log2);
+  else
+    hipLaunchKernelGGL(fused_region_parallel<int64_t>, dim3((unsigned)blocks), dim3(kThreads), 0, stream, args, lanes_log2);
   return after_launch();
 }
 

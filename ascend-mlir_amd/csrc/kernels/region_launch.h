@@ -37,7 +37,11 @@ struct RegionOp {
   int code;
   int input;
   float constant;
-  int depth;
+  int depth;   // Dup: entries below the top
+  int dst;     // stack slot the operation writes, filled in by the launcher:
+               // push / const / dup write a new top, a binary operation
+               // combines slot dst with slot dst + 1, a unary one works in place
+  int pad[3];
 };
 
 struct RegionArgs {
