@@ -344,6 +344,20 @@ class Region:
         return load().afir_hip_launch_region(ctypes.c_uint64(self.handle), block_dim, _stream(stream),
                                              len(ptrs), arr, ctypes.c_void_p(workspace), buf, len(tiling))
 
+    def prepare(self, ptrs, tiling: bytes, workspace=0, block_dim=0, stream=None):
+        """Pre-marshal one launch; returns a zero-argument callable."""
+        L = load()
+        arr = (ctypes.c_void_p * len(ptrs))(*[ctypes.c_void_p(p) for p in ptrs])
+        buf = ctypes.create_string_buffer(tiling, len(tiling))
+        args = (ctypes.c_uint64(self.handle), ctypes.c_uint32(block_dim), _stream(stream), len(ptrs),
+                arr, ctypes.c_void_p(workspace), ctypes.cast(buf, ctypes.c_void_p), len(tiling))
+
+        def call(_fn=L.afir_hip_launch_region, _args=args, _keep=(arr, buf)):
+            rc = _fn(*_args)
+            if rc:
+                _check(rc)
+        return call
+
     def __call__(self, *inputs, out_shape, workspace=None, block_dim=0, stream=None):
         """inputs: device tensors in argument order; returns the output tensor."""
         import torch

@@ -41,6 +41,55 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 MEASURED_TRAFFIC = {"c1": None, "c2": None, "c3": None, "c4": None, "c5": None}
 
 
+# Region programs of the two generic-kernel workloads (grammar:
+# ascend-mlir_amd/csrc/target/region_program.h)
+REGION_ADD_MUL = """afir-hip-region 1
+arg in f32 2
+arg in f32 2
+arg out f32 2
+segment 2
+size arg0.0 arg0.1
+outoff 0
+push arg0 d0 d1
+push arg1 d0 d1
+add
+push arg1 d0 d1
+mul
+store
+end
+"""
+REGION_SPLIT_RELU_BRC_ADD_MUL = """afir-hip-region 1
+arg in f16 2
+arg in f16 1
+arg in f16 1
+arg in f16 1
+arg in f16 1
+arg out f16 2
+segment 2
+size arg1.0 arg0.1
+outoff 0
+push arg0 d0 d1
+relu
+push arg1 d0
+add
+push arg3 d1
+mul
+store
+end
+segment 2
+size arg2.0 arg0.1
+outoff arg1.0
+push arg0 d0 d1 slice arg1.0 0
+relu
+push arg2 d0
+add
+push arg4 d1
+mul
+store
+end
+"""
+
+
 def load_package():
     name = "ascend_mlir_amd"
     if name in sys.modules:
@@ -283,6 +332,62 @@ def make_workload(key, torch, H, O, C):
                 w.work() * 20 / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
             return ev
         w.power_evidence = power_evidence
+    elif key in ("g1", "g2"):
+        # The generic region kernel (any fused chain) next to the hand-tuned
+        # ones: g1 = the c1 chain kept off its fast path, g2 = the reference's
+        # split / relu / broadcast-add / broadcast-mul / concat graph
+        # (examples/split-relu-brc-add-mul) at [8192, 4096] f16.
+        from oracle import region_oracle as RO
+        os.environ["AFIR_HIP_REGION_GENERIC"] = "1"
+        if key == "g1":
+            text = REGION_ADD_MUL
+            a, b = O.gen_c1()
+            inputs, out_shape, out_dt = [a, b], (4096, 4096), torch.float32
+            w.title = "g1 generic region kernel: (a+b)*b f32 [4096,4096] as a region program"
+            w.dtype = "f32"
+            work = O.algorithmic_bytes("c1", m=4096, n=4096)
+        else:
+            text = REGION_SPLIT_RELU_BRC_ADD_MUL
+            rng = np.random.default_rng(42)
+            m, n = 8192, 4096
+            f16 = lambda shape: rng.uniform(-1, 1, shape).astype(np.float32).astype(np.float16)
+            inputs = [f16((m, n)), f16((m // 2,)), f16((m // 2,)), f16((n,)), f16((n,))]
+            out_shape, out_dt = (m, n), torch.float16
+            w.title = ("g2 generic region kernel: split/relu/bcast-add/bcast-mul/concat f16 [8192,4096] "
+                       "(two segments)")
+            w.dtype = "f16"
+            work = 2 * m * n * 2 + 2 * (m // 2) * 2 + 2 * n * 2
+        region = H.Region(text)
+        del os.environ["AFIR_HIP_REGION_GENERIC"]
+        assert region.kernel == "fused_region"
+        w.work = lambda: work
+        w.nsets = 3 if key == "g1" else 4
+        dev0 = [_dev(torch, x) for x in inputs]
+        sets = []
+        for i in range(w.nsets):
+            ins = dev0 if i == 0 else [dev0[0].clone()] + ([dev0[1].clone()] if key == "g1" else dev0[1:])
+            sets.append((ins, torch.empty(out_shape, dtype=out_dt, device="cuda")))
+        w.sets = sets
+        dims = [d for x in inputs for d in x.shape] + list(out_shape)
+        w.launches = [region.prepare([t.data_ptr() for t in s[0]] + [s[1].data_ptr()],
+                                     H.pack_tiling(*dims)) for s in sets]
+        w.region = region
+
+        def parity():
+            want = RO.evaluate(text, inputs)
+            got = sets[0][1].cpu().numpy()
+            return {"bar": "bit-exact vs the region oracle", "passed": got.tobytes() == want.tobytes(),
+                    "mismatches": int((got.view(np.uint16 if key == "g2" else np.uint32) !=
+                                       want.view(np.uint16 if key == "g2" else np.uint32)).sum())}
+        w.parity = parity
+
+        def cpu(budget_s):
+            t0 = time.perf_counter()
+            RO.evaluate(text, inputs)
+            dt = time.perf_counter() - t0
+            return w.work() / dt / 1e9, "full workload, numpy region oracle (1 thread), one run"
+        w.cpu = cpu
+        w.cpu_cores = 1
     else:
         raise SystemExit(f"unknown workload {key}")
     return w
@@ -327,7 +432,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "g1", "g2"])
     ap.add_argument("--all", dest="all", action="store_true", default=True)
     ap.add_argument("--no-all", dest="all", action="store_false")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -359,8 +464,8 @@ def main():
             return args.warmup
         return 5 if key == "c5" else 30
 
-    order = [args.workload] + ([k for k in ["c1", "c2", "c3", "c4", "c5"] if k != args.workload]
-                               if args.all else [])
+    order = [args.workload] + ([k for k in ["c1", "c2", "c3", "c4", "c5", "g1", "g2"]
+                                if k != args.workload] if args.all else [])
     results = []
     for key in order:
         w = make_workload(key, torch, H, O, C)
@@ -377,7 +482,8 @@ def main():
         if not args.no_cpu_baseline:
             budget = args.cpu_seconds if key == args.workload else min(3.0, args.cpu_seconds)
             v, sample = w.cpu(budget)
-            entry["cpu_baseline"] = {"value": round(v, 4), "unit": unit, "cores": C.threads(),
+            entry["cpu_baseline"] = {"value": round(v, 4), "unit": unit,
+                                     "cores": getattr(w, "cpu_cores", None) or C.threads(),
                                      "kind": "port", "sample": sample,
                                      "host_cpus": os.cpu_count()}
         results.append(entry)
