@@ -35,10 +35,11 @@ METRIC = "fused-kernel HBM GB/s (% of peak); matmul+epilogue TFLOP/s; 1 GPU"
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 
-# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (two runs), scaled by the same counters' reading for a plain copy kernel of
-# known size; None until measured.  Source: profiles/*_pmc.txt.
-MEASURED_TRAFFIC = {"c1": None, "c2": None, "c3": None, "c4": None, "c5": None}
+# HBM bytes per step measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (two runs), scaled by the same counters' reading for a plain 256 MiB copy
+# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Source: profiles/*.txt, section (2).
+MEASURED_TRAFFIC = {"c1": 201364275, "c2": 134441381, "c3": 134502809, "c4": 134574489,
+                    "c5": 1869395968, "g1": 201536102, "g2": 134893568}
 
 
 # Region programs of the two generic-kernel workloads (grammar:
@@ -436,6 +437,9 @@ def main():
     ap.add_argument("--all", dest="all", action="store_true", default=True)
     ap.add_argument("--no-all", dest="all", action="store_false")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-power-evidence", action="store_true",
+                    help="c5: skip the extra launches on constant operands and the MFMA rate probe "
+                         "(keeps a profiler's per-kernel averages to the timed steps)")
     ap.add_argument("--cpu-seconds", type=float, default=10.0)
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three plain 256 MiB device copies, so that a counter run "
@@ -473,7 +477,8 @@ def main():
         wall, ev_ms = run_workload(w, torch, steps, warmup)
         value, unit, roof = summarize(w, wall, ev_ms, steps)
         par = w.parity()
-        extra = w.power_evidence() if hasattr(w, "power_evidence") else None
+        extra = (w.power_evidence() if hasattr(w, "power_evidence") and not args.no_power_evidence
+                 else None)
         entry = {"workload": w.title, "value": round(value, 2), "unit": unit, "steps": steps,
                  "warmup": warmup, "ms_per_step": round(wall * 1e3 / steps, 5), "dtype": w.dtype,
                  "buffer_sets": w.nsets, "roofline": roof, "parity": par}
