@@ -21,6 +21,15 @@
 // chunks takes a power-of-two group of lanes, longer rows take the whole
 // workgroup), and positions are 32-bit when every tensor is below 2^31
 // elements.
+//
+// Most fused regions are chains -- a running value combined with one new
+// operand per step, activations in between (every example graph of the
+// reference is one).  The launcher recognises that shape and hands the kernel
+// the linear form: one accumulator vector and one operand vector are the only
+// live values, no stack and no moves, which leaves registers for eight waves
+// per SIMD.  Expressions that are not chains run on the stack interpreter.
+#include <cstdlib>
+
 #include "kernels.h"
 #include "region_launch.h"
 
@@ -127,6 +136,9 @@ __device__ __forceinline__ void read_operand(const RegionInput &in, int last, co
 __device__ __forceinline__ float fmax_nan(float a, float b) { return __builtin_elementwise_maximum(a, b); }
 __device__ __forceinline__ float fmin_nan(float a, float b) { return __builtin_elementwise_minimum(a, b); }
 
+// Every operation has its own case and the default does nothing: with the
+// last operation as the default, hipcc 7.2 lost the eighth element of a
+// negation that followed a binary step in the chain evaluator.
 __device__ __forceinline__ void binary(int code, float (&a)[kVec], const float (&b)[kVec]) {
   switch (code) {
     case kRegionAdd:
@@ -149,9 +161,11 @@ __device__ __forceinline__ void binary(int code, float (&a)[kVec], const float (
 #pragma unroll
       for (int e = 0; e < kVec; ++e) a[e] = fmax_nan(a[e], b[e]);
       break;
-    default:
+    case kRegionMin:
 #pragma unroll
       for (int e = 0; e < kVec; ++e) a[e] = fmin_nan(a[e], b[e]);
+      break;
+    default:
       break;
   }
 }
@@ -166,9 +180,11 @@ __device__ __forceinline__ void unary(int code, float c, float (&a)[kVec]) {
 #pragma unroll
       for (int e = 0; e < kVec; ++e) a[e] = fmax_nan(a[e], a[e] * c);
       break;
-    default:
+    case kRegionNeg:
 #pragma unroll
       for (int e = 0; e < kVec; ++e) a[e] = -a[e];
+      break;
+    default:
       break;
   }
 }
@@ -221,6 +237,51 @@ __device__ __forceinline__ void evaluate(const RegionArgs &R, int last, const Po
   }
 }
 
+__device__ __forceinline__ void apply_unaries(const RegionUnary &u, float (&a)[kVec]) {
+  if (u.count > 0) unary(u.code[0], u.alpha[0], a);
+  if (u.count > 1) unary(u.code[1], u.alpha[1], a);
+}
+
+// Linear form: acc = u0(x0); acc = u_k(acc (op_k) x_k).
+template <typename I>
+__device__ __forceinline__ void evaluate_chain(const RegionArgs &R, int last, const Position<I> &at,
+                                               int nvalid, bool full, float (&acc)[kVec]) {
+  if (R.chain_first >= 0) {
+    read_operand<I>(R.in[R.chain_first], last, at, nvalid, full, R.error_flag, acc);
+  } else {
+#pragma unroll
+    for (int e = 0; e < kVec; ++e) acc[e] = R.chain_constant;
+  }
+  apply_unaries(R.chain_after_first, acc);
+  for (int k = 0; k < R.nsteps; ++k) {
+    const RegionStep &st = R.steps[k];
+    float x[kVec];
+    if (st.input >= 0) {
+      read_operand<I>(R.in[st.input], last, at, nvalid, full, R.error_flag, x);
+    } else {
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) x[e] = st.constant;
+    }
+    if (st.bop == kChainRSub) {
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) acc[e] = x[e] - acc[e];
+    } else if (st.bop == kChainRDiv) {
+#pragma unroll
+      for (int e = 0; e < kVec; ++e) acc[e] = x[e] / acc[e];
+    } else {
+      binary(st.bop, acc, x);
+    }
+    apply_unaries(st.after, acc);
+  }
+}
+
+template <typename I, bool CHAIN>
+__device__ __forceinline__ void evaluate_any(const RegionArgs &R, int last, const Position<I> &at,
+                                             int nvalid, bool full, float (&v)[kVec]) {
+  if (CHAIN) evaluate_chain<I>(R, last, at, nvalid, full, v);
+  else evaluate<I>(R, last, at, nvalid, full, v);
+}
+
 __device__ __forceinline__ void store_elem(void *out, int type, int64_t i, float x) {
   if (type == kRegionF32) static_cast<float *>(out)[i] = x;
   else if (type == kRegionF16) static_cast<uint16_t *>(out)[i] = __builtin_bit_cast(uint16_t, (_Float16)x);
@@ -245,7 +306,7 @@ __device__ __forceinline__ Position<I> position(const RegionArgs &R, I row, I j0
 
 // lanes_log2: a row's chunks are spread over 2^lanes_log2 lanes of the
 // workgroup (8 = the whole workgroup walks one row at a time).
-template <typename I>
+template <typename I, bool CHAIN>
 __global__ __launch_bounds__(kThreads) void fused_region_parallel(const RegionArgs R, int lanes_log2) {
   const int last = R.rank - 1;
   const I n = (I)R.size[last];
@@ -264,7 +325,7 @@ __global__ __launch_bounds__(kThreads) void fused_region_parallel(const RegionAr
       const int nvalid = left >= kVec ? kVec : (int)left;
       const bool full = nvalid == kVec;
       float v[kVec];
-      evaluate<I>(R, last, position<I>(R, row, j0), nvalid, full, v);
+      evaluate_any<I, CHAIN>(R, last, position<I>(R, row, j0), nvalid, full, v);
       const int64_t o = (int64_t)row * n + j0;
       if (full && R.out_vec) {
         if (R.out_type == kRegionF32) {
@@ -293,7 +354,7 @@ __global__ __launch_bounds__(kThreads) void fused_region_parallel(const RegionAr
 // Row sum over the innermost dim: one wavefront per output element, lanes
 // stride over the row in vectors of 8, float32 partial sums per vector slot,
 // fixed-order combination and a DPP wave reduction: deterministic.
-template <typename I>
+template <typename I, bool CHAIN>
 __global__ __launch_bounds__(kThreads) void fused_region_rowsum(const RegionArgs R) {
   const int last = R.rank - 1;
   const I n = (I)R.size[last];
@@ -311,7 +372,7 @@ __global__ __launch_bounds__(kThreads) void fused_region_rowsum(const RegionArgs
       const I left = n - j0;
       const int nvalid = left >= kVec ? kVec : (int)left;
       float v[kVec];
-      evaluate<I>(R, last, position<I>(R, row, j0), nvalid, nvalid == kVec, v);
+      evaluate_any<I, CHAIN>(R, last, position<I>(R, row, j0), nvalid, nvalid == kVec, v);
 #pragma unroll
       for (int e = 0; e < kVec; ++e) acc[e] += (e < nvalid) ? v[e] : 0.f;
     }
@@ -319,6 +380,91 @@ __global__ __launch_bounds__(kThreads) void fused_region_rowsum(const RegionArgs
     s = wave_sum(s);
     if (lane == 0) store_elem(R.out, R.out_type, (int64_t)row, s);
   }
+}
+
+// Postfix program -> linear chain, where the expression is one: at most one
+// partial result is alive at any time and every other stack entry is a leaf
+// (an operand read or a constant, with activations only on the leaf the chain
+// starts from).  Returns false for anything else (two partial results, dup).
+bool linearize(RegionArgs &a) {
+  struct Entry {
+    bool chain = false;
+    int input = -1;          // leaf: operand, or -1 = constant
+    float constant = 0.f;
+    RegionUnary un = {};
+  };
+  Entry stack[4];
+  int depth = 0;
+  bool started = false;
+  a.nsteps = 0;
+  a.chain_after_first = RegionUnary{};
+  auto reversed = [](int code) {
+    return code == kRegionSub ? (int)kChainRSub : (code == kRegionDiv ? (int)kChainRDiv : code);
+  };
+  auto add_unary = [](RegionUnary &u, int code, float alpha) {
+    if (u.count >= 2) return false;
+    u.code[u.count] = code;
+    u.alpha[u.count] = alpha;
+    ++u.count;
+    return true;
+  };
+  auto add_step = [&](int bop, const Entry &leaf) {
+    if (a.nsteps >= kRegionMaxSteps) return false;
+    RegionStep &st = a.steps[a.nsteps++];
+    st = RegionStep{};
+    st.bop = bop;
+    st.input = leaf.input;
+    st.constant = leaf.constant;
+    return true;
+  };
+  auto start = [&](const Entry &leaf) {
+    started = true;
+    a.chain_first = leaf.input;
+    a.chain_constant = leaf.constant;
+    a.chain_after_first = leaf.un;
+  };
+  for (int i = 0; i < a.nops; ++i) {
+    const RegionOp &op = a.ops[i];
+    if (op.code == kRegionPush || op.code == kRegionConst) {
+      Entry e;
+      e.input = op.code == kRegionPush ? op.input : -1;
+      e.constant = op.constant;
+      stack[depth++] = e;
+    } else if (op.code == kRegionDup) {
+      return false;
+    } else if (op.code >= kRegionAdd && op.code <= kRegionMin) {
+      Entry &x = stack[depth - 2], &y = stack[depth - 1];
+      if (x.chain && y.chain) return false;
+      if (x.chain) {
+        if (y.un.count || !add_step(op.code, y)) return false;
+      } else if (y.chain) {
+        if (x.un.count || !add_step(reversed(op.code), x)) return false;
+        x = y;
+      } else {
+        if (started) return false;          // a second partial result
+        if (x.un.count && y.un.count) return false;
+        if (y.un.count) {
+          start(y);
+          if (!add_step(reversed(op.code), x)) return false;
+        } else {
+          start(x);
+          if (!add_step(op.code, y)) return false;
+        }
+        x = Entry{};
+        x.chain = true;
+      }
+      --depth;
+    } else {   // unary
+      Entry &x = stack[depth - 1];
+      RegionUnary &u = x.chain ? (a.nsteps ? a.steps[a.nsteps - 1].after : a.chain_after_first) : x.un;
+      if (!add_unary(u, op.code, op.constant)) return false;
+    }
+  }
+  if (!stack[0].chain) {   // a single leaf: x0 with its activations, no steps
+    if (started) return false;
+    start(stack[0]);
+  }
+  return true;
 }
 
 }  // namespace
@@ -357,6 +503,11 @@ LaunchStatus launch_fused_region(const RegionArgs &args_in, uint32_t block_dim, 
     }
   }
   if (depth != 1) return invalid("fused_region: the program must leave exactly one value");
+  args.chain = linearize(args) ? 1 : 0;
+  // AFIR_HIP_REGION_STACK=1 keeps chains on the stack interpreter (the tests
+  // run every program both ways)
+  if (const char *env = std::getenv("AFIR_HIP_REGION_STACK"))
+    if (*env && *env != '0') args.chain = 0;
 
   // 32-bit positions when every operand and the output stay below 2^31 elements
   bool idx32 = total < ((int64_t)1 << 31);
@@ -376,10 +527,9 @@ LaunchStatus launch_fused_region(const RegionArgs &args_in, uint32_t block_dim, 
     int64_t blocks = (rows + (kThreads / kWave) - 1) / (kThreads / kWave);
     if (blocks > (int64_t)kNumCU * 8) blocks = (int64_t)kNumCU * 8;
     if (block_dim) blocks = block_dim;
-    if (idx32)
-      hipLaunchKernelGGL(fused_region_rowsum<int>, dim3((unsigned)blocks), dim3(kThreads), 0, stream, args);
-    else
-      hipLaunchKernelGGL(fused_region_rowsum<int64_t>, dim3((unsigned)blocks), dim3(kThreads), 0, stream, args);
+    auto kernel = args.chain ? (idx32 ? fused_region_rowsum<int, true> : fused_region_rowsum<int64_t, true>)
+                             : (idx32 ? fused_region_rowsum<int, false> : fused_region_rowsum<int64_t, false>);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), 0, stream, args);
     return after_launch();
   }
   if (total == 0) return ok_status();
@@ -392,10 +542,9 @@ LaunchStatus launch_fused_region(const RegionArgs &args_in, uint32_t block_dim, 
   int64_t blocks = (rows + rows_per_pass - 1) / rows_per_pass;
   if (blocks > (int64_t)kNumCU * 16) blocks = (int64_t)kNumCU * 16;
   if (block_dim) blocks = block_dim;
-  if (idx32)
-    hipLaunchKernelGGL(fused_region_parallel<int>, dim3((unsigned)blocks), dim3(kThreads), 0, stream, args, lanes_log2);
-  else
-    hipLaunchKernelGGL(fused_region_parallel<int64_t>, dim3((unsigned)blocks), dim3(kThreads), 0, stream, args, lanes_log2);
+  auto kernel = args.chain ? (idx32 ? fused_region_parallel<int, true> : fused_region_parallel<int64_t, true>)
+                           : (idx32 ? fused_region_parallel<int, false> : fused_region_parallel<int64_t, false>);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), 0, stream, args, lanes_log2);
   return after_launch();
 }
 

@@ -44,6 +44,25 @@ struct RegionOp {
   int pad[3];
 };
 
+// Linear form of a program, derived by the launcher where the expression is a
+// chain: acc = u0(x0); acc = u_k(acc (op_k) x_k) for each step.  Reversed
+// operands (x - acc, x / acc) have their own codes.
+constexpr int kRegionMaxSteps = 8;
+enum RegionChainCode : int { kChainRSub = 32, kChainRDiv = 33 };
+struct RegionUnary {
+  int code[2];      // kRegionRelu / kRegionLeaky / kRegionNeg
+  float alpha[2];
+  int count;
+  int pad;
+};
+struct RegionStep {
+  int bop;          // RegionOpCode of a binary operation, or a RegionChainCode
+  int input;        // operand: index into RegionArgs::in, or -1 for `constant`
+  float constant;
+  int pad;
+  RegionUnary after;
+};
+
 struct RegionArgs {
   int64_t size[3];
   void *out;            // first element this segment writes
@@ -56,6 +75,13 @@ struct RegionArgs {
   int reduce;
   RegionInput in[kRegionMaxInputs];
   RegionOp ops[kRegionMaxOps];
+  // filled in by the launcher
+  int chain;              // 1: the fields below describe the whole expression
+  int chain_first;        // x0: index into `in`, or -1 for chain_constant
+  float chain_constant;
+  int nsteps;
+  RegionUnary chain_after_first;
+  RegionStep steps[kRegionMaxSteps];
 };
 
 LaunchStatus launch_fused_region(const RegionArgs &args, uint32_t block_dim, hipStream_t stream);

@@ -34,6 +34,16 @@ def _host(t, ty):
     return t.cpu().numpy()
 
 
+@pytest.fixture(params=["chain", "stack"], autouse=True)
+def evaluator(request, monkeypatch):
+    """Every test runs twice: expressions that are chains on the linear form,
+    and everything on the stack interpreter."""
+    monkeypatch.setenv("AFIR_HIP_REGION_GENERIC", "1")
+    if request.param == "stack":
+        monkeypatch.setenv("AFIR_HIP_REGION_STACK", "1")
+    return request.param
+
+
 def run(H, text, inputs, out_shape, workspace=None, block_dim=0):
     r = H.Region(text)
     dev = [_dev(x, r.arg_types[i]) for i, x in enumerate(inputs)]
@@ -180,3 +190,23 @@ def test_random_chains_bit_exact(H, seed):
     same = (got.view(np.uint16 if ty != "f32" else np.uint32) ==
             want.view(np.uint16 if ty != "f32" else np.uint32)) | (np.isnan(wf) & np.isnan(gf))
     assert same.all(), text
+
+
+def test_every_operation_pair_at_every_vector_position(H):
+    """binary step followed by up to two activations, all combinations, on rows
+    of 19 elements (two full vectors and a tail): every position of the result
+    must match the oracle."""
+    rng = np.random.default_rng(77)
+    a = rng.uniform(-3, 3, (3, 19)).astype(np.float32)
+    b = rng.uniform(-3, 3, (19,)).astype(np.float32)
+    head = RC.HEADER + "arg in f32 2\narg in f32 1\narg out f32 2\nsegment 2\n size arg0.0 arg0.1\n outoff 0\n"
+    unaries = ["", "relu\n", "leaky 0.25\n", "neg\n"]
+    for first in (" push arg0 d0 d1\n push arg1 d1\n", " push arg1 d1\n push arg0 d0 d1\n"):
+        for op in OPS2:
+            for u1 in unaries:
+                for u2 in unaries:
+                    text = head + first + f" {op}\n {u1} {u2} store\nend\n"
+                    want = RO.evaluate(text, [a, b])
+                    got = run(H, text, [a, b], a.shape)
+                    same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))
+                    assert same.all(), (text, np.argwhere(~same))
