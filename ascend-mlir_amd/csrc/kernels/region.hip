@@ -7,7 +7,7 @@
 // generics :246-750; the fused gather loop :828-1272) is here one interpreter
 // whose program arrives as a kernel argument.
 //
-// HBM-bound by construction: a lane owns 8 consecutive elements of the
+// HBM-bound by construction: a lane owns 8 (or 16) consecutive elements of the
 // innermost iteration dim, reads each operand once (128-bit loads where the
 // operand is contiguous and aligned along that dim, one scalar load where it
 // is broadcast along it, element loads for transposed or gathered operands),
@@ -37,7 +37,6 @@ namespace afir {
 
 namespace {
 
-constexpr int kVec = 8;
 constexpr int kThreads = 256;
 
 __device__ __forceinline__ float load_elem(const void *base, int type, int64_t i) {
@@ -47,18 +46,26 @@ __device__ __forceinline__ float load_elem(const void *base, int type, int64_t i
   return __uint_as_float(h << 16);
 }
 
-__device__ __forceinline__ void load_vec(const void *base, int type, int64_t i, float (&v)[kVec]) {
+template <int V>
+__device__ __forceinline__ void load_vec(const void *base, int type, int64_t i, float (&v)[V]) {
   if (type == kRegionF32) {
     const f32x4 *p = reinterpret_cast<const f32x4 *>(static_cast<const float *>(base) + i);
-    const f32x4 a = p[0], b = p[1];
 #pragma unroll
-    for (int e = 0; e < 4; ++e) { v[e] = a[e]; v[4 + e] = b[e]; }
+    for (int q = 0; q < V / 4; ++q) {
+      const f32x4 a = p[q];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[4 * q + e] = a[e];
+    }
   } else {
-    const u32x4 raw = *reinterpret_cast<const u32x4 *>(static_cast<const uint16_t *>(base) + i);
+    const u32x4 *p = reinterpret_cast<const u32x4 *>(static_cast<const uint16_t *>(base) + i);
 #pragma unroll
-    for (int d = 0; d < 4; ++d) {
-      if (type == kRegionF16) { v[2 * d] = f16_lo(raw[d]); v[2 * d + 1] = f16_hi(raw[d]); }
-      else { v[2 * d] = bf16_lo(raw[d]); v[2 * d + 1] = bf16_hi(raw[d]); }
+    for (int q = 0; q < V / 8; ++q) {
+      const u32x4 raw = p[q];
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        if (type == kRegionF16) { v[8 * q + 2 * d] = f16_lo(raw[d]); v[8 * q + 2 * d + 1] = f16_hi(raw[d]); }
+        else { v[8 * q + 2 * d] = bf16_lo(raw[d]); v[8 * q + 2 * d + 1] = bf16_hi(raw[d]); }
+      }
     }
   }
 }
@@ -68,17 +75,17 @@ __device__ __forceinline__ int64_t load_index(const void *base, int type, int64_
                             : static_cast<const int64_t *>(base)[i];
 }
 
-// Iteration position of the first of a lane's 8 elements.
+// Iteration position of the first of a lane's V elements.
 template <typename I>
 struct Position {
   I x0, x1, x2;  // index along iteration dims 0..2 (the innermost one holds j0)
 };
 
-// One operand for the 8 elements at `at`.  `full`: all 8 elements exist.
-template <typename I>
+// One operand for the V elements at `at`.  `full`: all V elements exist.
+template <typename I, int V>
 __device__ __forceinline__ void read_operand(const RegionInput &in, int last, const Position<I> &at,
                                              int nvalid, bool full, int32_t *error_flag,
-                                             float (&v)[kVec]) {
+                                             float (&v)[V]) {
   // element position without the gathered dim
   I pos = (I)in.offset + at.x0 * (I)in.stride[0] + at.x1 * (I)in.stride[1] + at.x2 * (I)in.stride[2];
   const I step = (I)(last == 0 ? in.stride[0] : (last == 1 ? in.stride[1] : in.stride[2]));
@@ -88,7 +95,7 @@ __device__ __forceinline__ void read_operand(const RegionInput &in, int last, co
     // gathered along the innermost dim: one index per element
     const I j0 = last == 0 ? at.x0 : (last == 1 ? at.x1 : at.x2);
 #pragma unroll
-    for (int e = 0; e < kVec; ++e) {
+    for (int e = 0; e < V; ++e) {
       float x = 0.f;
       if (e < nvalid) {
         const int64_t g = load_index(in.index, in.gtype, (int64_t)j0 + e);
@@ -112,7 +119,7 @@ __device__ __forceinline__ void read_operand(const RegionInput &in, int last, co
     if (g < 0 || g >= in.gextent) {
       if (error_flag) *error_flag = 1;
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) v[e] = nan;
+      for (int e = 0; e < V; ++e) v[e] = nan;
       return;
     }
     p64 += g * in.gstride;
@@ -123,10 +130,10 @@ __device__ __forceinline__ void read_operand(const RegionInput &in, int last, co
   } else if (step == 0) {
     const float x = load_elem(in.base, in.type, p64);
 #pragma unroll
-    for (int e = 0; e < kVec; ++e) v[e] = x;
+    for (int e = 0; e < V; ++e) v[e] = x;
   } else {
 #pragma unroll
-    for (int e = 0; e < kVec; ++e)
+    for (int e = 0; e < V; ++e)
       v[e] = (e < nvalid) ? load_elem(in.base, in.type, p64 + (int64_t)e * step) : 0.f;
   }
 }
@@ -139,77 +146,80 @@ __device__ __forceinline__ float fmin_nan(float a, float b) { return __builtin_e
 // Every operation has its own case and the default does nothing: with the
 // last operation as the default, hipcc 7.2 lost the eighth element of a
 // negation that followed a binary step in the chain evaluator.
-__device__ __forceinline__ void binary(int code, float (&a)[kVec], const float (&b)[kVec]) {
+template <int V>
+__device__ __forceinline__ void binary(int code, float (&a)[V], const float (&b)[V]) {
   switch (code) {
     case kRegionAdd:
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) a[e] = a[e] + b[e];
+      for (int e = 0; e < V; ++e) a[e] = a[e] + b[e];
       break;
     case kRegionSub:
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) a[e] = a[e] - b[e];
+      for (int e = 0; e < V; ++e) a[e] = a[e] - b[e];
       break;
     case kRegionMul:
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) a[e] = a[e] * b[e];
+      for (int e = 0; e < V; ++e) a[e] = a[e] * b[e];
       break;
     case kRegionDiv:
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) a[e] = a[e] / b[e];
+      for (int e = 0; e < V; ++e) a[e] = a[e] / b[e];
       break;
     case kRegionMax:
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) a[e] = fmax_nan(a[e], b[e]);
+      for (int e = 0; e < V; ++e) a[e] = fmax_nan(a[e], b[e]);
       break;
     case kRegionMin:
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) a[e] = fmin_nan(a[e], b[e]);
+      for (int e = 0; e < V; ++e) a[e] = fmin_nan(a[e], b[e]);
       break;
     default:
       break;
   }
 }
 
-__device__ __forceinline__ void unary(int code, float c, float (&a)[kVec]) {
+template <int V>
+__device__ __forceinline__ void unary(int code, float c, float (&a)[V]) {
   switch (code) {
     case kRegionRelu:
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) a[e] = fmax_nan(a[e], 0.f);
+      for (int e = 0; e < V; ++e) a[e] = fmax_nan(a[e], 0.f);
       break;
     case kRegionLeaky:
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) a[e] = fmax_nan(a[e], a[e] * c);
+      for (int e = 0; e < V; ++e) a[e] = fmax_nan(a[e], a[e] * c);
       break;
     case kRegionNeg:
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) a[e] = -a[e];
+      for (int e = 0; e < V; ++e) a[e] = -a[e];
       break;
     default:
       break;
   }
 }
 
-__device__ __forceinline__ void assign(float (&d)[kVec], const float (&s)[kVec]) {
+template <int V>
+__device__ __forceinline__ void assign(float (&d)[V], const float (&s)[V]) {
 #pragma unroll
-  for (int e = 0; e < kVec; ++e) d[e] = s[e];
+  for (int e = 0; e < V; ++e) d[e] = s[e];
 }
 
-// Evaluates the expression for 8 elements; the result ends up in slot 0.
-template <typename I>
+// Evaluates the expression for V elements; the result ends up in slot 0.
+template <typename I, int V>
 __device__ __forceinline__ void evaluate(const RegionArgs &R, int last, const Position<I> &at,
-                                         int nvalid, bool full, float (&s0)[kVec]) {
-  float s1[kVec], s2[kVec], s3[kVec];
+                                         int nvalid, bool full, float (&s0)[V]) {
+  float s1[V], s2[V], s3[V];
 #pragma unroll
-  for (int e = 0; e < kVec; ++e) s0[e] = s1[e] = s2[e] = s3[e] = 0.f;
+  for (int e = 0; e < V; ++e) s0[e] = s1[e] = s2[e] = s3[e] = 0.f;
   for (int pc = 0; pc < R.nops; ++pc) {
     const RegionOp op = R.ops[pc];
     if (op.code == kRegionPush || op.code == kRegionConst || op.code == kRegionDup) {
-      float t[kVec];
+      float t[V];
       if (op.code == kRegionPush) {
-        read_operand<I>(R.in[op.input], last, at, nvalid, full, R.error_flag, t);
+        read_operand<I, V>(R.in[op.input], last, at, nvalid, full, R.error_flag, t);
       } else if (op.code == kRegionConst) {
 #pragma unroll
-        for (int e = 0; e < kVec; ++e) t[e] = op.constant;
+        for (int e = 0; e < V; ++e) t[e] = op.constant;
       } else {
         const int src = op.dst - 1 - op.depth;
         assign(t, src == 0 ? s0 : (src == 1 ? s1 : s2));
@@ -237,37 +247,38 @@ __device__ __forceinline__ void evaluate(const RegionArgs &R, int last, const Po
   }
 }
 
-__device__ __forceinline__ void apply_unaries(const RegionUnary &u, float (&a)[kVec]) {
+template <int V>
+__device__ __forceinline__ void apply_unaries(const RegionUnary &u, float (&a)[V]) {
   if (u.count > 0) unary(u.code[0], u.alpha[0], a);
   if (u.count > 1) unary(u.code[1], u.alpha[1], a);
 }
 
 // Linear form: acc = u0(x0); acc = u_k(acc (op_k) x_k).
-template <typename I>
+template <typename I, int V>
 __device__ __forceinline__ void evaluate_chain(const RegionArgs &R, int last, const Position<I> &at,
-                                               int nvalid, bool full, float (&acc)[kVec]) {
+                                               int nvalid, bool full, float (&acc)[V]) {
   if (R.chain_first >= 0) {
-    read_operand<I>(R.in[R.chain_first], last, at, nvalid, full, R.error_flag, acc);
+    read_operand<I, V>(R.in[R.chain_first], last, at, nvalid, full, R.error_flag, acc);
   } else {
 #pragma unroll
-    for (int e = 0; e < kVec; ++e) acc[e] = R.chain_constant;
+    for (int e = 0; e < V; ++e) acc[e] = R.chain_constant;
   }
   apply_unaries(R.chain_after_first, acc);
   for (int k = 0; k < R.nsteps; ++k) {
     const RegionStep &st = R.steps[k];
-    float x[kVec];
+    float x[V];
     if (st.input >= 0) {
-      read_operand<I>(R.in[st.input], last, at, nvalid, full, R.error_flag, x);
+      read_operand<I, V>(R.in[st.input], last, at, nvalid, full, R.error_flag, x);
     } else {
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) x[e] = st.constant;
+      for (int e = 0; e < V; ++e) x[e] = st.constant;
     }
     if (st.bop == kChainRSub) {
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) acc[e] = x[e] - acc[e];
+      for (int e = 0; e < V; ++e) acc[e] = x[e] - acc[e];
     } else if (st.bop == kChainRDiv) {
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) acc[e] = x[e] / acc[e];
+      for (int e = 0; e < V; ++e) acc[e] = x[e] / acc[e];
     } else {
       binary(st.bop, acc, x);
     }
@@ -275,11 +286,11 @@ __device__ __forceinline__ void evaluate_chain(const RegionArgs &R, int last, co
   }
 }
 
-template <typename I, bool CHAIN>
+template <typename I, bool CHAIN, int V>
 __device__ __forceinline__ void evaluate_any(const RegionArgs &R, int last, const Position<I> &at,
-                                             int nvalid, bool full, float (&v)[kVec]) {
-  if (CHAIN) evaluate_chain<I>(R, last, at, nvalid, full, v);
-  else evaluate<I>(R, last, at, nvalid, full, v);
+                                             int nvalid, bool full, float (&v)[V]) {
+  if (CHAIN) evaluate_chain<I, V>(R, last, at, nvalid, full, v);
+  else evaluate<I, V>(R, last, at, nvalid, full, v);
 }
 
 __device__ __forceinline__ void store_elem(void *out, int type, int64_t i, float x) {
@@ -306,11 +317,11 @@ __device__ __forceinline__ Position<I> position(const RegionArgs &R, I row, I j0
 
 // lanes_log2: a row's chunks are spread over 2^lanes_log2 lanes of the
 // workgroup (8 = the whole workgroup walks one row at a time).
-template <typename I, bool CHAIN>
+template <typename I, bool CHAIN, int V>
 __global__ __launch_bounds__(kThreads) void fused_region_parallel(const RegionArgs R, int lanes_log2) {
   const int last = R.rank - 1;
   const I n = (I)R.size[last];
-  const I chunks = (n + kVec - 1) / kVec;
+  const I chunks = (n + V - 1) / V;
   const I rows = (I)((R.rank == 1) ? 1 : ((R.rank == 2) ? R.size[0] : R.size[0] * R.size[1]));
   const int lanes = 1 << lanes_log2;
   const int rows_per_pass = kThreads >> lanes_log2;
@@ -320,31 +331,38 @@ __global__ __launch_bounds__(kThreads) void fused_region_parallel(const RegionAr
     const I row = row0 + local_row;
     if (row >= rows) continue;
     for (I chunk = first_chunk; chunk < chunks; chunk += lanes) {
-      const I j0 = chunk * kVec;
+      const I j0 = chunk * V;
       const I left = n - j0;
-      const int nvalid = left >= kVec ? kVec : (int)left;
-      const bool full = nvalid == kVec;
-      float v[kVec];
-      evaluate_any<I, CHAIN>(R, last, position<I>(R, row, j0), nvalid, full, v);
+      const int nvalid = left >= V ? V : (int)left;
+      const bool full = nvalid == V;
+      float v[V];
+      evaluate_any<I, CHAIN, V>(R, last, position<I>(R, row, j0), nvalid, full, v);
       const int64_t o = (int64_t)row * n + j0;
       if (full && R.out_vec) {
         if (R.out_type == kRegionF32) {
-          f32x4 a, b;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) { a[e] = v[e]; b[e] = v[4 + e]; }
           f32x4 *p = reinterpret_cast<f32x4 *>(static_cast<float *>(R.out) + o);
-          p[0] = a;
-          p[1] = b;
-        } else {
-          u32x4 w;
 #pragma unroll
-          for (int d = 0; d < 4; ++d)
-            w[d] = R.out_type == kRegionF16 ? pack_f16(v[2 * d], v[2 * d + 1]) : pack_bf16(v[2 * d], v[2 * d + 1]);
-          *reinterpret_cast<u32x4 *>(static_cast<uint16_t *>(R.out) + o) = w;
+          for (int q = 0; q < V / 4; ++q) {
+            f32x4 a;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) a[e] = v[4 * q + e];
+            p[q] = a;
+          }
+        } else {
+          u32x4 *p = reinterpret_cast<u32x4 *>(static_cast<uint16_t *>(R.out) + o);
+#pragma unroll
+          for (int q = 0; q < V / 8; ++q) {
+            u32x4 w;
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+              w[d] = R.out_type == kRegionF16 ? pack_f16(v[8 * q + 2 * d], v[8 * q + 2 * d + 1])
+                                              : pack_bf16(v[8 * q + 2 * d], v[8 * q + 2 * d + 1]);
+            p[q] = w;
+          }
         }
       } else {
 #pragma unroll
-        for (int e = 0; e < kVec; ++e)
+        for (int e = 0; e < V; ++e)
           if (e < nvalid) store_elem(R.out, R.out_type, o + e, v[e]);
       }
     }
@@ -354,29 +372,34 @@ __global__ __launch_bounds__(kThreads) void fused_region_parallel(const RegionAr
 // Row sum over the innermost dim: one wavefront per output element, lanes
 // stride over the row in vectors of 8, float32 partial sums per vector slot,
 // fixed-order combination and a DPP wave reduction: deterministic.
-template <typename I, bool CHAIN>
+template <typename I, bool CHAIN, int V>
 __global__ __launch_bounds__(kThreads) void fused_region_rowsum(const RegionArgs R) {
   const int last = R.rank - 1;
   const I n = (I)R.size[last];
-  const I chunks = (n + kVec - 1) / kVec;
+  const I chunks = (n + V - 1) / V;
   const I rows = (I)((R.rank == 2) ? R.size[0] : R.size[0] * R.size[1]);
   const int lane = threadIdx.x & (kWave - 1);
   const I wave = (I)blockIdx.x * (kThreads / kWave) + (I)(threadIdx.x >> 6);
   const I nwaves = (I)gridDim.x * (kThreads / kWave);
   for (I row = wave; row < rows; row += nwaves) {
-    float acc[kVec];
+    float acc[V];
 #pragma unroll
-    for (int e = 0; e < kVec; ++e) acc[e] = 0.f;
+    for (int e = 0; e < V; ++e) acc[e] = 0.f;
     for (I c = lane; c < chunks; c += kWave) {
-      const I j0 = c * kVec;
+      const I j0 = c * V;
       const I left = n - j0;
-      const int nvalid = left >= kVec ? kVec : (int)left;
-      float v[kVec];
-      evaluate_any<I, CHAIN>(R, last, position<I>(R, row, j0), nvalid, nvalid == kVec, v);
+      const int nvalid = left >= V ? V : (int)left;
+      float v[V];
+      evaluate_any<I, CHAIN, V>(R, last, position<I>(R, row, j0), nvalid, nvalid == V, v);
 #pragma unroll
-      for (int e = 0; e < kVec; ++e) acc[e] += (e < nvalid) ? v[e] : 0.f;
+      for (int e = 0; e < V; ++e) acc[e] += (e < nvalid) ? v[e] : 0.f;
     }
-    float s = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
+    // fixed-order pairwise combination of the per-slot partial sums
+#pragma unroll
+    for (int w = V / 2; w >= 1; w >>= 1)
+#pragma unroll
+      for (int e = 0; e < w; ++e) acc[e] = acc[2 * e] + acc[2 * e + 1];
+    float s = acc[0];
     s = wave_sum(s);
     if (lane == 0) store_elem(R.out, R.out_type, (int64_t)row, s);
   }
@@ -520,6 +543,12 @@ LaunchStatus launch_fused_region(const RegionArgs &args_in, uint32_t block_dim, 
     }
   }
 
+  // 32 bytes per lane and operand: 8 elements, or 16 when every tensor of a
+  // chain is 16-bit (twice the bytes per interpreted step)
+  bool wide = args.chain && args.out_type != kRegionF32;
+  for (int i = 0; i < args.ninputs; ++i) wide = wide && args.in[i].type != kRegionF32;
+  const int vec = wide ? 16 : 8;
+
   if (args.reduce) {
     if (args.rank < 2) return invalid("fused_region: reduction needs rank >= 2");
     if (rows == 0) return ok_status();
@@ -527,23 +556,25 @@ LaunchStatus launch_fused_region(const RegionArgs &args_in, uint32_t block_dim, 
     int64_t blocks = (rows + (kThreads / kWave) - 1) / (kThreads / kWave);
     if (blocks > (int64_t)kNumCU * 8) blocks = (int64_t)kNumCU * 8;
     if (block_dim) blocks = block_dim;
-    auto kernel = args.chain ? (idx32 ? fused_region_rowsum<int, true> : fused_region_rowsum<int64_t, true>)
-                             : (idx32 ? fused_region_rowsum<int, false> : fused_region_rowsum<int64_t, false>);
+    auto kernel = wide ? (idx32 ? fused_region_rowsum<int, true, 16> : fused_region_rowsum<int64_t, true, 16>)
+                  : args.chain ? (idx32 ? fused_region_rowsum<int, true, 8> : fused_region_rowsum<int64_t, true, 8>)
+                               : (idx32 ? fused_region_rowsum<int, false, 8> : fused_region_rowsum<int64_t, false, 8>);
     hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), 0, stream, args);
     return after_launch();
   }
   if (total == 0) return ok_status();
   if (!args.out) return invalid("fused_region: null output pointer");
   const int64_t n = args.size[args.rank - 1];
-  const int64_t chunks = (n + kVec - 1) / kVec;
+  const int64_t chunks = (n + vec - 1) / vec;
   int lanes_log2 = 0;
   while (lanes_log2 < 8 && ((int64_t)1 << lanes_log2) < chunks) ++lanes_log2;
   const int rows_per_pass = kThreads >> lanes_log2;
   int64_t blocks = (rows + rows_per_pass - 1) / rows_per_pass;
   if (blocks > (int64_t)kNumCU * 16) blocks = (int64_t)kNumCU * 16;
   if (block_dim) blocks = block_dim;
-  auto kernel = args.chain ? (idx32 ? fused_region_parallel<int, true> : fused_region_parallel<int64_t, true>)
-                           : (idx32 ? fused_region_parallel<int, false> : fused_region_parallel<int64_t, false>);
+  auto kernel = wide ? (idx32 ? fused_region_parallel<int, true, 16> : fused_region_parallel<int64_t, true, 16>)
+                : args.chain ? (idx32 ? fused_region_parallel<int, true, 8> : fused_region_parallel<int64_t, true, 8>)
+                             : (idx32 ? fused_region_parallel<int, false, 8> : fused_region_parallel<int64_t, false, 8>);
   hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), 0, stream, args, lanes_log2);
   return after_launch();
 }
