@@ -330,8 +330,13 @@ Expected<std::vector<TensorBinding>> parseBindings(const Json &root, const char 
     if (source == "external_file") {
       if (auto p = v.getString("path")) b.path = *p;
     } else if (source == "task_output") {
-      return Status::error("tensor binding source 'task_output' needs a multi-task session, which "
-                           "this runtime does not run");
+      auto task = v.getString("upstream_task");
+      if (!task) return Status::error("missing required string field: upstream_task");
+      auto output = v.getString("upstream_output");
+      if (!output) return Status::error("missing required string field: upstream_output");
+      b.fromTaskOutput = true;
+      b.upstreamTask = *task;
+      b.upstreamOutput = *output;
     } else {
       return Status::error("unsupported tensor binding source: " + source);
     }

@@ -222,6 +222,10 @@ struct TensorBinding {
   std::string path;
   std::vector<int64_t> shape;
   std::optional<DType> dtype;
+  // source = "task_output": the tensor is output `upstreamOutput` of task
+  // `upstreamTask` of the same manifest (lib/Runtime/Artifact/RunManifest.cpp:107-118)
+  bool fromTaskOutput = false;
+  std::string upstreamTask, upstreamOutput;
 };
 
 struct ExecutionInvocation {
@@ -303,8 +307,24 @@ struct SessionSummary {
   OutputComparisonResult comparison;
 };
 
-// Runs the (single) task of a manifest: load artifact, bind inputs, allocate
-// outputs from expected shapes, launch, validate, write outputs.
+// Runs one task: load artifact, bind inputs, allocate outputs from expected
+// shapes, launch, validate, write outputs.
 SessionSummary runSingleTask(const RunTaskSpec &task, RunnerFactory factory, int deviceId);
+
+// Execution order of a manifest's tasks: Kahn's algorithm over `dependencies`,
+// ready tasks in manifest order (lib/Runtime/Execution/TaskGraph.cpp:33-79).
+// Errors: "empty task id", "duplicate task id", "unknown task dependency",
+// "task graph contains a cycle".
+Expected<std::vector<size_t>> planTasks(const RunManifestSpec &manifest);
+
+// Serial session over all tasks in plan order.  An input bound to a task
+// output reads the file that task wrote; outputs without a path are
+// materialised as <workingDirectory>/<task>__<name>.npy
+// (lib/Runtime/Execution/ExecutionSession.cpp:62-134,511-559).  Stops at the
+// first failing task; the summary is the failing task's, or the merged one
+// (validation passed = every validating task passed; counters carry a
+// "<task>." prefix when there is more than one task).
+SessionSummary runSession(const RunManifestSpec &manifest, RunnerFactory factory, int deviceId,
+                          const std::string &workingDirectory);
 
 }  // namespace afirt

@@ -3,6 +3,9 @@
 // load artifact -> pack tiling -> load input .npy -> allocate outputs from the
 // expected shapes -> launch -> compare -> save outputs.  Errors carry the
 // stage they happened in, as "[hip:<stage>] message".
+#include <deque>
+#include <map>
+
 #include "runtime.h"
 
 namespace afirt {
@@ -116,6 +119,91 @@ SessionSummary runSingleTask(const RunTaskSpec &task, RunnerFactory factory, int
   }
   summary.success = true;
   return summary;
+}
+
+Expected<std::vector<size_t>> planTasks(const RunManifestSpec &manifest) {
+  const auto &tasks = manifest.tasks;
+  std::map<std::string, size_t> indexById;
+  for (size_t i = 0; i < tasks.size(); ++i) {
+    if (tasks[i].taskId.empty()) return Status::error("empty task id");
+    if (!indexById.emplace(tasks[i].taskId, i).second) return Status::error("duplicate task id");
+  }
+  std::vector<size_t> indegree(tasks.size(), 0);
+  std::vector<std::vector<size_t>> outgoing(tasks.size());
+  for (size_t i = 0; i < tasks.size(); ++i)
+    for (const std::string &dep : tasks[i].dependencies) {
+      auto it = indexById.find(dep);
+      if (it == indexById.end()) return Status::error("unknown task dependency");
+      outgoing[it->second].push_back(i);
+      ++indegree[i];
+    }
+  std::deque<size_t> ready;
+  for (size_t i = 0; i < tasks.size(); ++i)
+    if (indegree[i] == 0) ready.push_back(i);
+  std::vector<size_t> order;
+  while (!ready.empty()) {
+    const size_t i = ready.front();
+    ready.pop_front();
+    order.push_back(i);
+    for (size_t next : outgoing[i])
+      if (--indegree[next] == 0) ready.push_back(next);
+  }
+  if (order.size() != tasks.size()) return Status::error("task graph contains a cycle");
+  return order;
+}
+
+SessionSummary runSession(const RunManifestSpec &manifest, RunnerFactory factory, int deviceId,
+                          const std::string &workingDirectory) {
+  SessionSummary merged;
+  auto order = planTasks(manifest);
+  if (!order) return fail(merged, "driver", order.error());
+  const bool many = manifest.tasks.size() > 1;
+  std::map<std::string, TensorBinding> produced;   // "<task>::<output>" -> where it was written
+  merged.validationPassed = true;
+  for (size_t index : *order) {
+    RunTaskSpec task = manifest.tasks[index];
+    for (TensorBinding &b : task.invocation.inputs) {
+      if (!b.fromTaskOutput) continue;
+      const std::string key = b.upstreamTask + "::" + b.upstreamOutput;
+      auto it = produced.find(key);
+      if (it == produced.end())
+        return fail(merged, "bindings", "task input binding cannot resolve upstream output " + key +
+                                            " for task " + task.taskId);
+      b.path = it->second.path;
+      if (b.shape.empty()) b.shape = it->second.shape;
+      if (!b.dtype) b.dtype = it->second.dtype;
+      b.fromTaskOutput = false;
+    }
+    for (size_t i = 0; i < task.invocation.outputs.size(); ++i) {
+      TensorBinding &b = task.invocation.outputs[i];
+      if (b.name.empty()) b.name = "output" + std::to_string(i);
+      if (b.path.empty()) {
+        if (workingDirectory.empty())
+          return fail(merged, "bindings", "output '" + b.name + "' of task " + task.taskId +
+                                              " has no path and the session has no working directory");
+        b.path = workingDirectory + "/" + task.taskId + "__" + b.name + ".npy";
+      }
+    }
+    SessionSummary s = runSingleTask(task, factory, deviceId);
+    if (!s.success) {
+      if (many) s.errorMessage = "task " + task.taskId + ": " + s.errorMessage;
+      if (many) s.rawErrorMessage = std::string("[hip:") + s.errorStage + "] " + s.errorMessage;
+      return s;
+    }
+    for (const TensorBinding &b : task.invocation.outputs) produced[task.taskId + "::" + b.name] = b;
+    merged.validationRan = merged.validationRan || s.validationRan;
+    if (s.validationRan) {
+      merged.validationPassed = merged.validationPassed && s.validationPassed;
+      if (s.comparison.maxAbsDiff > merged.comparison.maxAbsDiff) merged.comparison = s.comparison;
+    }
+    const std::string prefix = many ? task.taskId + "." : "";
+    for (const auto &kv : s.runtimeAttributes) merged.runtimeAttributes[prefix + kv.first] = kv.second;
+    for (const auto &kv : s.runtimeCounters) merged.runtimeCounters[prefix + kv.first] = kv.second;
+    merged.producedFiles.insert(merged.producedFiles.end(), s.producedFiles.begin(), s.producedFiles.end());
+  }
+  merged.success = true;
+  if (!merged.validationRan) merged.validationPassed = false;
+  return merged;
 }
 
 }  // namespace afirt

@@ -92,6 +92,7 @@ int main(int argc, char **argv) {
   }
 
   RunTaskSpec task;
+  RunManifestSpec session;   // every task of the manifest (or the one implied by the flags)
   task.taskId = opt.count("task-id") ? opt["task-id"] : "main";
   std::string backend = "hip";
   if (opt.count("run-manifest")) {
@@ -100,13 +101,9 @@ int main(int argc, char **argv) {
       std::fprintf(stderr, "Error: %s\n", manifest.error().c_str());
       return 4;
     }
-    if (manifest->tasks.size() != 1) {
-      std::fprintf(stderr, "Error: this session runs single-task manifests; got %zu tasks\n",
-                   manifest->tasks.size());
-      return 4;
-    }
     if (manifest->backend != "hip")
       std::printf("session.backend_requested=%s\n", manifest->backend.c_str());
+    session = *manifest;
     task = manifest->tasks[0];
   } else {
     const bool hasRoot = opt.count("artifact-root") != 0, hasKernel = opt.count("kernel") != 0;
@@ -159,8 +156,15 @@ int main(int argc, char **argv) {
     factory = &makeTestingRunner;
   }
 
-  std::printf("session.plan.tasks=1\n");
-  std::printf("session.plan[0]=%s\n", task.taskId.c_str());
+  if (session.tasks.empty()) session.tasks.push_back(task);
+  auto plan = planTasks(session);
+  if (!plan) {
+    std::fprintf(stderr, "Error: %s\n", plan.error().c_str());
+    return 4;
+  }
+  std::printf("session.plan.tasks=%zu\n", plan->size());
+  for (size_t i = 0; i < plan->size(); ++i)
+    std::printf("session.plan[%zu]=%s\n", i, session.tasks[(*plan)[i]].taskId.c_str());
   std::fflush(stdout);
   if (!run) return 0;
 
@@ -173,7 +177,11 @@ int main(int argc, char **argv) {
   }
 
   const int device = opt.count("device") ? std::atoi(opt["device"].c_str()) : 0;
-  SessionSummary s = runSingleTask(task, factory, device);
+  // outputs without a path go to a directory next to the manifest
+  std::string workdir = opt["run-manifest"];
+  const size_t slash = workdir.rfind('/');
+  workdir = slash == std::string::npos ? "." : workdir.substr(0, slash);
+  SessionSummary s = runSession(session, factory, device, workdir);
   if (!s.success) {
     printErrorSummary(s);
     return 2;

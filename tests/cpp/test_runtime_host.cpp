@@ -15,6 +15,9 @@
 
 using namespace afirt;
 
+// The GPU runner is not linked into this host-only binary; nothing here runs a kernel.
+std::unique_ptr<ExecutionRunner> afirt::createHipExecutionRunner() { return nullptr; }
+
 static int g_pass = 0, g_fail = 0;
 #define EXPECT(cond, msg)                                   \
   do {                                                      \
@@ -383,6 +386,35 @@ static void testArtifactsAndManifests() {
          "tasks array with default artifact root");
 }
 
+// Task ordering (reference: lib/Runtime/Execution/TaskGraph.cpp:33-79 and its
+// tests in test/tools/runtime/test_taskgraph_runtime.cpp): dependencies first,
+// ready tasks in manifest order, unknown / duplicate / cyclic graphs rejected.
+static void testPlan() {
+  auto task = [](const char *id, std::vector<std::string> deps) {
+    RunTaskSpec t;
+    t.taskId = id;
+    t.dependencies = std::move(deps);
+    return t;
+  };
+  RunManifestSpec m;
+  m.tasks = {task("d", {"b", "c"}), task("b", {"a"}), task("c", {"a"}), task("a", {}), task("e", {})};
+  auto order = planTasks(m);
+  EXPECT((bool)order, "diamond plans");
+  if (order) {
+    std::string ids;
+    for (size_t i : *order) ids += m.tasks[i].taskId;
+    EXPECT(ids == "aebcd", "ready tasks in manifest order, dependencies first");
+  }
+  m.tasks = {task("a", {"zz"})};
+  EXPECT(!planTasks(m) && planTasks(m).error() == "unknown task dependency", "unknown dependency");
+  m.tasks = {task("a", {}), task("a", {})};
+  EXPECT(!planTasks(m) && planTasks(m).error() == "duplicate task id", "duplicate id");
+  m.tasks = {task("a", {"b"}), task("b", {"a"})};
+  EXPECT(!planTasks(m) && planTasks(m).error() == "task graph contains a cycle", "cycle");
+  m.tasks = {task("", {})};
+  EXPECT(!planTasks(m) && planTasks(m).error() == "empty task id", "empty id");
+}
+
 int main(int argc, char **argv) {
   if (argc < 2) {
     std::printf("usage: %s <tmpdir>\n", argv[0]);
@@ -393,6 +425,7 @@ int main(int argc, char **argv) {
   testTiling();
   testComparator();
   testArtifactsAndManifests();
+  testPlan();
   std::printf("%d passed, %d failed\n", g_pass, g_fail);
   return g_fail ? 1 : 0;
 }

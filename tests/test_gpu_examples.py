@@ -149,3 +149,49 @@ def test_matmul_bf16_program_runs_on_the_mfma_kernel(pkg):
     res = O.compare_outputs([(got, "bf16")], [(O.golden_c5(a, b, bias, 0.01), "bf16")], 1e-5, 1e-2)
     assert res["passed"], res
     r.close()
+
+
+def test_two_kernel_session_feeds_one_kernel_into_the_next(tmp_path):
+    """A two-task manifest (the shape of examples/real-npu-multikernel): t = (a + b) * b on the first
+    kernel, y[i] = sum_j (t[i,j] + bias[j]) on the second, the intermediate tensor bound as a task output."""
+    k1, k2 = tmp_path / "k1.mlir", tmp_path / "k2.mlir"
+    k1.write_text(MC.C1_AFIR)
+    k2.write_text(MC.C2_LINALG)
+    for src, name in ((k1, "add_mul"), (k2, "rowsum")):
+        assert _rs("--kernel", str(src), "--output", str(tmp_path / name), "--name", name).returncode == 0
+        assert subprocess.run([TR, "-mlir-to-hip", str(src), "-o", str(tmp_path / (name + ".txt")),
+                               "--tiling-space-out", str(tmp_path / (name + ".json"))]).returncode == 0
+    rng = np.random.default_rng(3)
+    m, n = 300, 1000
+    a = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+    b = rng.uniform(-1, 1, (m, n)).astype(np.float32)
+    bias = rng.uniform(-1, 1, (n,)).astype(np.float32)
+    t = (a + b) * b
+    want = (t + bias[None, :]).sum(axis=1, dtype=np.float32)
+    for name, arr in (("a", a), ("b", b), ("bias", bias), ("want", want)):
+        np.save(tmp_path / f"{name}.npy", arr)
+
+    def params(path, dims):
+        fields = [f["name"] for f in json.loads(open(path).read())["tiling_params"]]
+        return ",".join(f"{k}={v}" for k, v in zip(fields, dims))
+    manifest = {"backend": "hip", "tasks": [
+        {"task_id": "reduce", "artifact_root": str(tmp_path / "rowsum"), "dependencies": ["chain"],
+         "inputs": [{"name": "x", "source": "task_output", "upstream_task": "chain", "upstream_output": "t"},
+                    {"name": "bias", "path": str(tmp_path / "bias.npy")}],
+         "outputs": [{"name": "y", "path": str(tmp_path / "y.npy")}],
+         "expected_outputs": [{"name": "y", "path": str(tmp_path / "want.npy")}],
+         "tiling": {"schema": str(tmp_path / "rowsum.json"), "params": params(tmp_path / "rowsum.json", [m, n, n, m])},
+         "atol": 1e-3, "rtol": 1e-5},
+        {"task_id": "chain", "artifact_root": str(tmp_path / "add_mul"),
+         "inputs": [{"name": "a", "path": str(tmp_path / "a.npy")}, {"name": "b", "path": str(tmp_path / "b.npy")}],
+         "outputs": [{"name": "t", "shape": [m, n], "dtype": "f32"}],
+         "tiling": {"schema": str(tmp_path / "add_mul.json"),
+                    "params": params(tmp_path / "add_mul.json", [m, n, m, n, m, n])}}]}
+    (tmp_path / "m.json").write_text(json.dumps(manifest))
+    p = _rs("--run-manifest", str(tmp_path / "m.json"), "--run")
+    assert p.returncode == 0, p.stdout + p.stderr
+    lines = p.stdout.splitlines()
+    assert "session.plan[0]=chain" in lines and "session.plan[1]=reduce" in lines
+    assert "session.result=success" in lines and "session.validation=pass" in lines
+    assert np.load(tmp_path / "chain__t.npy").tobytes() == t.tobytes()      # the intermediate is bit-exact
+    assert np.allclose(np.load(tmp_path / "y.npy"), want, rtol=1e-5, atol=1e-3)

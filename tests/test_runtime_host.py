@@ -26,6 +26,7 @@ def test_cpp_host_tests(tmp_path):
     src = [os.path.join(ROOT, "tests", "cpp", "test_runtime_host.cpp"),
            os.path.join(PKG, "csrc", "runtime", "support.cpp"),
            os.path.join(PKG, "csrc", "runtime", "artifact.cpp"),
+           os.path.join(PKG, "csrc", "runtime", "session.cpp"),
            os.path.join(PKG, "csrc", "target", "region_program.cpp"),
            os.path.join(PKG, "csrc", "target", "mlir_translate.cpp")]
     subprocess.run(["g++", "-std=c++17", "-O1", "-Wall", "-I", os.path.join(PKG, "csrc", "runtime"),
@@ -260,3 +261,68 @@ def test_cli_error_stages(tmp_path):
     np.save(tmp_path / "exp.npy", np.zeros((4, 4), np.float32))
     p = _rs("--run-manifest", m, "--run", "--testing-driver=hip-success")
     assert p.returncode == 0 and "session.backend_requested=sim" in p.stdout
+
+
+# --- multi-task manifests: plan order, task-output bindings (CPU, testing driver) ---
+
+def _two_task_manifest(tmp_path, **second):
+    src = tmp_path / "example.mlir"
+    src.write_text(EXAMPLE_MLIR)
+    assert _rs("--kernel", str(src), "--output", str(tmp_path / "art"), "--name", "example").returncode == 0
+    np.save(tmp_path / "a.npy", np.zeros((4, 4), np.float32))
+    np.save(tmp_path / "b.npy", np.ones((4, 4), np.float32))
+    (tmp_path / "ts.json").write_text(json.dumps({"tiling_params": [{"name": n} for n in TILING_FIELDS]}))
+    tiling = {"schema": str(tmp_path / "ts.json"), "params": TILING_PARAMS}
+    first = {"task_id": "first", "inputs": [{"name": "a", "path": str(tmp_path / "a.npy")},
+                                           {"name": "b", "path": str(tmp_path / "b.npy")}],
+             "outputs": [{"name": "t", "shape": [4, 4], "dtype": "f32"}], "tiling": tiling}
+    then = {"task_id": "then", "dependencies": ["first"],
+            "inputs": [{"name": "x", "source": "task_output", "upstream_task": "first", "upstream_output": "t"},
+                       {"name": "b", "path": str(tmp_path / "b.npy")}],
+            "outputs": [{"name": "y", "path": str(tmp_path / "y.npy"), "shape": [4, 4], "dtype": "f32"}],
+            "tiling": tiling}
+    then.update(second)
+    m = {"backend": "hip", "artifact_root": str(tmp_path / "art"), "tasks": [then, first]}
+    (tmp_path / "m.json").write_text(json.dumps(m))
+    return str(tmp_path / "m.json")
+
+
+def test_cli_multi_task_plan_and_task_output_binding(tmp_path):
+    m = _two_task_manifest(tmp_path)
+    p = _rs("--run-manifest", m)
+    assert p.returncode == 0, p.stderr
+    lines = p.stdout.splitlines()
+    # dependencies first, whatever the order in the file
+    assert "session.plan.tasks=2" in lines and "session.plan[0]=first" in lines and "session.plan[1]=then" in lines
+    p = _rs("--run-manifest", m, "--run", "--testing-driver=hip-success")
+    assert p.returncode == 0, p.stderr
+    assert "session.result=success" in p.stdout.splitlines()
+    # the intermediate tensor was materialised next to the manifest and fed to the second task
+    assert (tmp_path / "first__t.npy").exists() and (tmp_path / "y.npy").exists()
+    assert "session.runtime.counter.first.tiling_bytes=48" in p.stdout.splitlines()
+    assert "session.runtime.counter.then.tiling_bytes=48" in p.stdout.splitlines()
+
+
+def test_cli_multi_task_errors(tmp_path):
+    m = _two_task_manifest(tmp_path, dependencies=["nowhere"])
+    p = _rs("--run-manifest", m)
+    assert p.returncode == 4 and "unknown task dependency" in p.stderr
+    m = _two_task_manifest(tmp_path, inputs=[{"name": "x", "source": "task_output", "upstream_task": "first",
+                                              "upstream_output": "missing"},
+                                             {"name": "b", "path": str(tmp_path / "b.npy")}])
+    p = _rs("--run-manifest", m, "--run", "--testing-driver=hip-success")
+    assert p.returncode == 2 and "cannot resolve upstream output first::missing for task then" in p.stderr
+    assert "session.error_stage=bindings" in p.stderr
+    m = _two_task_manifest(tmp_path, inputs=[{"name": "x", "source": "task_output", "upstream_task": "first"}])
+    assert _rs("--run-manifest", m).returncode == 4
+    # a cycle
+    d = json.loads(open(_two_task_manifest(tmp_path)).read())
+    d["tasks"][1]["dependencies"] = ["then"]
+    (tmp_path / "cycle.json").write_text(json.dumps(d))
+    p = _rs("--run-manifest", str(tmp_path / "cycle.json"))
+    assert p.returncode == 4 and "task graph contains a cycle" in p.stderr
+    d["tasks"][1]["dependencies"] = []
+    d["tasks"][1]["task_id"] = "then"
+    (tmp_path / "dup.json").write_text(json.dumps(d))
+    p = _rs("--run-manifest", str(tmp_path / "dup.json"))
+    assert p.returncode == 4 and "duplicate task id" in p.stderr
