@@ -28,8 +28,10 @@ program must reproduce the closed-form golden of that example
 (afir_oracle.reduce_rowbias_f16, relu_col_add_f16, relu_colgather_add_f16 and
 the concat / split formulas written out with numpy in the test), the five
 benchmark configurations as programs must reproduce golden_c1..c4 bit for bit,
-and single-op programs are checked against Python float arithmetic rounded
-through struct.  max / min follow IEEE-754 maximum / minimum (-0 < +0, NaN
+single-op programs are checked against Python float arithmetic rounded
+through struct, and the graphs of the reference's examples, translated from
+MLIR, must turn the reference's own input vectors into its own expected
+outputs (tests/golden/reference_examples.npz, tests/test_golden_fixtures.py).  max / min follow IEEE-754 maximum / minimum (-0 < +0, NaN
 propagates), which is what arith.maximumf specifies.
 """
 from __future__ import annotations
@@ -91,6 +93,8 @@ def parse(text: str) -> dict:
                 else:
                     m.append(("const", int(t)))
             seg["ops"].append(("push", arg, m, sl))
+        elif k == "matmul":
+            seg["ops"].append(("matmul", int(tok[1][3:]), int(tok[2][3:])))
         elif k in ("const", "leaky"):
             seg["ops"].append((k, np.float32(float(tok[1]))))
         elif k == "dup":
@@ -160,6 +164,12 @@ def evaluate(text: str, inputs):
                         idx.append(g.reshape(shape) + start)
                 v = _widen(src, args[a][1])[tuple(idx)] if src.ndim else _widen(src, args[a][1])
                 stack.append(np.broadcast_to(v, size).astype(np.float32))
+            elif k == "matmul":
+                # float32 product as the reference golden computes it
+                # (examples/matmul-add-leakyrelu/gen_data.py:33: A.f32 @ B.f32)
+                a = _widen(inputs[op[1]], args[op[1]][1])
+                b = _widen(inputs[op[2]], args[op[2]][1])
+                stack.append((a @ b).astype(np.float32))
             elif k == "const":
                 stack.append(np.full(size, op[1], dtype=np.float32))
             elif k == "dup":

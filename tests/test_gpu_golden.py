@@ -1,0 +1,40 @@
+"""The GPU path on the reference's own vectors (inputs and expected outputs
+written by the reference's golden scripts, tests/golden/reference_examples.npz):
+MLIR graph -> region program -> kernel, compared with the reference's output.
+Needs a GPU."""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from tests import golden_cases as GC
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+TR = os.path.join(ROOT, "ascend-mlir_amd", "bin", "afir-translate")
+CASES = list(GC.cases())
+
+
+@pytest.mark.parametrize("generic", ["routed", "generic"])
+@pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
+def test_kernel_reproduces_the_reference_output(pkg, monkeypatch, case, generic):
+    import torch
+    from ascend_mlir_amd import hip_kernels as H
+    H.load()
+    name, mlir, program, inputs, want, exact = case
+    if program is None:
+        p = subprocess.run([TR, "-mlir-to-hip", "-"], input=mlir, capture_output=True, text=True)
+        assert p.returncode == 0, p.stderr
+        program = p.stdout
+    monkeypatch.setenv("AFIR_HIP_REGION_GENERIC", "1" if generic == "generic" else "0")
+    r = H.Region(program)
+    dev = [torch.from_numpy(x).cuda() for x in inputs]
+    got = r(*dev, out_shape=want.shape).cpu().numpy()
+    r.close()
+    if exact:
+        assert got.tobytes() == want.tobytes()
+    else:   # f32 row sum in another order, one rounding to f16
+        assert np.all(np.abs(got.astype(np.float64) - want.astype(np.float64))
+                      <= 2.0 ** -10 * np.abs(want.astype(np.float64)) + 1e-3)
