@@ -32,11 +32,19 @@ constexpr int kUnroll = AFIR_ROWSUM_UNROLL;
 constexpr int kWavesPerCU = AFIR_ROWSUM_WAVES_PER_CU;
 
 // Rows of at most 64*CH 128-bit chunks: the wave keeps its CH chunks of bias
-// in registers for all the rows it walks, and has a whole row in flight.
-template <int CH>
+// in registers for all the rows it walks.  The row is requested in batches of
+// kBatch chunks per lane (a batch is summed while the next is in flight): the
+// memory system sustains more with a few KiB outstanding per wave than with a
+// whole row.  EXACT: the row is exactly 64*CH chunks, no lane is ever idle and
+// the loads carry no predicate.
+#ifndef AFIR_ROWSUM_BATCH
+#define AFIR_ROWSUM_BATCH 4
+#endif
+template <int CH, bool EXACT>
 __global__ __launch_bounds__(kThreads) void bcast_add_rowsum_f32_resident(
     const float *__restrict__ x, const float *__restrict__ bias, float *__restrict__ y,
     int64_t m, int64_t n) {
+  constexpr int kBatch = CH < AFIR_ROWSUM_BATCH ? CH : AFIR_ROWSUM_BATCH;
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t wave = (int64_t)blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
   const int64_t nwaves = (int64_t)gridDim.x * kWavesPerBlock;
@@ -45,20 +53,71 @@ __global__ __launch_bounds__(kThreads) void bcast_add_rowsum_f32_resident(
   const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
   f32x4 vb[CH];
 #pragma unroll
-  for (int u = 0; u < CH; ++u) vb[u] = (lane + u * kWave < n4) ? b4[lane + u * kWave] : zero;
+  for (int u = 0; u < CH; ++u) vb[u] = (EXACT || lane + u * kWave < n4) ? b4[lane + u * kWave] : zero;
 
   for (int64_t row = wave; row < m; row += nwaves) {
     const f32x4 *x4 = reinterpret_cast<const f32x4 *>(x + row * n);
-    f32x4 vx[CH];
-#pragma unroll
-    for (int u = 0; u < CH; ++u)
-      vx[u] = (lane + u * kWave < n4) ? load_nt(x4 + lane + u * kWave) : zero;
     f32x4 acc = zero;
 #pragma unroll
-    for (int u = 0; u < CH; ++u) acc += vx[u] + vb[u];
+    for (int g = 0; g < CH; g += kBatch) {
+      f32x4 vx[kBatch];
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u)
+        vx[u] = (EXACT || lane + (g + u) * kWave < n4) ? load_nt(x4 + lane + (g + u) * kWave) : zero;
+#pragma unroll
+      for (int u = 0; u < kBatch; ++u) acc += vx[u] + vb[g + u];
+    }
     float s = (acc.x + acc.y) + (acc.z + acc.w);
     s = wave_sum(s);
     if (lane == 0) y[row] = s;
+  }
+}
+
+// Rows of exactly 256*U chunks: a workgroup of four waves owns a row, so that
+// the grid walks x like a linear stream -- every load instruction of a
+// workgroup covers 4 KiB of contiguous memory and the whole grid a window of
+// a few MiB -- which this memory system serves ~8 % faster than one wave per
+// row.  A lane's U chunks of bias stay in registers.  The next row is
+// requested before the current one is reduced (DPP inside the waves, one LDS
+// word per wave, one barrier per row: the partial sums are double-buffered by
+// row parity).
+#ifndef AFIR_ROWSUM_WG_PER_CU
+#define AFIR_ROWSUM_WG_PER_CU 2
+#endif
+constexpr int kRowThreads = 256;
+template <int U>
+__global__ __launch_bounds__(kRowThreads) void bcast_add_rowsum_f32_wgrow(
+    const float *__restrict__ x, const float *__restrict__ bias, float *__restrict__ y,
+    int64_t m, int64_t n) {
+  __shared__ float part[2][kRowThreads / kWave];
+  const int t = threadIdx.x, lane = t & (kWave - 1), wave = t >> 6;
+  const f32x4 *b4 = reinterpret_cast<const f32x4 *>(bias);
+  f32x4 vb[U], vx[U];
+#pragma unroll
+  for (int u = 0; u < U; ++u) vb[u] = b4[t + u * kRowThreads];
+  int64_t row = blockIdx.x;
+  if (row < m) {
+    const f32x4 *x4 = reinterpret_cast<const f32x4 *>(x + row * n);
+#pragma unroll
+    for (int u = 0; u < U; ++u) vx[u] = load_nt(x4 + t + u * kRowThreads);
+  }
+  int parity = 0;
+  for (; row < m; row += gridDim.x) {
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc += vx[u] + vb[u];
+    const int64_t next = row + gridDim.x;
+    if (next < m) {
+      const f32x4 *x4 = reinterpret_cast<const f32x4 *>(x + next * n);
+#pragma unroll
+      for (int u = 0; u < U; ++u) vx[u] = load_nt(x4 + t + u * kRowThreads);
+    }
+    float s = (acc.x + acc.y) + (acc.z + acc.w);
+    s = wave_sum(s);
+    if (lane == 0) part[parity][wave] = s;
+    __syncthreads();
+    if (t == 0) y[row] = (part[parity][0] + part[parity][1]) + (part[parity][2] + part[parity][3]);
+    parity ^= 1;
   }
 }
 
@@ -123,23 +182,37 @@ LaunchStatus launch_broadcast_add_reducesum(const float *x, const float *bias, f
   if (block_dim) blocks = block_dim;
   if (blocks > 0x7fffffff) blocks = 0x7fffffff;
   const bool vec = n > 0 && (n % 4 == 0) && aligned16(x) && aligned16(bias);
-  if (vec && n / 4 <= 16 * kWave) {
+  if (vec && (n / 4) % kRowThreads == 0 && n / 4 <= 8 * kRowThreads && aligned16(x) &&
+      ((n / 4 / kRowThreads) & (n / 4 / kRowThreads - 1)) == 0) {
+    // a workgroup per row
+    int64_t wblocks = (int64_t)kNumCU * AFIR_ROWSUM_WG_PER_CU;
+    if (wblocks > m) wblocks = m;
+    if (block_dim) wblocks = block_dim;
+    const dim3 grid((unsigned)wblocks), block(kRowThreads);
+    switch ((int)(n / 4 / kRowThreads)) {
+      case 1: hipLaunchKernelGGL(bcast_add_rowsum_f32_wgrow<1>, grid, block, 0, stream, x, bias, y, m, n); break;
+      case 2: hipLaunchKernelGGL(bcast_add_rowsum_f32_wgrow<2>, grid, block, 0, stream, x, bias, y, m, n); break;
+      case 4: hipLaunchKernelGGL(bcast_add_rowsum_f32_wgrow<4>, grid, block, 0, stream, x, bias, y, m, n); break;
+      default: hipLaunchKernelGGL(bcast_add_rowsum_f32_wgrow<8>, grid, block, 0, stream, x, bias, y, m, n); break;
+    }
+  } else if (vec && n / 4 <= 16 * kWave) {
     // persistent waves: each keeps its bias chunks resident and walks several rows
     const int64_t n4 = n / 4;
     int64_t pblocks = (int64_t)kNumCU * kWavesPerCU / kWavesPerBlock;
     if (pblocks * kWavesPerBlock > m) pblocks = (m + kWavesPerBlock - 1) / kWavesPerBlock;
     if (block_dim) pblocks = block_dim;
     const dim3 grid((unsigned)pblocks), block(kThreads);
-    if (n4 <= 1 * kWave)
-      hipLaunchKernelGGL(bcast_add_rowsum_f32_resident<1>, grid, block, 0, stream, x, bias, y, m, n);
-    else if (n4 <= 2 * kWave)
-      hipLaunchKernelGGL(bcast_add_rowsum_f32_resident<2>, grid, block, 0, stream, x, bias, y, m, n);
-    else if (n4 <= 4 * kWave)
-      hipLaunchKernelGGL(bcast_add_rowsum_f32_resident<4>, grid, block, 0, stream, x, bias, y, m, n);
-    else if (n4 <= 8 * kWave)
-      hipLaunchKernelGGL(bcast_add_rowsum_f32_resident<8>, grid, block, 0, stream, x, bias, y, m, n);
-    else
-      hipLaunchKernelGGL(bcast_add_rowsum_f32_resident<16>, grid, block, 0, stream, x, bias, y, m, n);
+    auto launch = [&](auto kernel) {
+      hipLaunchKernelGGL(kernel, grid, block, 0, stream, x, bias, y, m, n);
+    };
+    if (n4 == 16 * kWave) launch(bcast_add_rowsum_f32_resident<16, true>);
+    else if (n4 == 8 * kWave) launch(bcast_add_rowsum_f32_resident<8, true>);
+    else if (n4 == 4 * kWave) launch(bcast_add_rowsum_f32_resident<4, true>);
+    else if (n4 <= 1 * kWave) launch(bcast_add_rowsum_f32_resident<1, false>);
+    else if (n4 <= 2 * kWave) launch(bcast_add_rowsum_f32_resident<2, false>);
+    else if (n4 <= 4 * kWave) launch(bcast_add_rowsum_f32_resident<4, false>);
+    else if (n4 <= 8 * kWave) launch(bcast_add_rowsum_f32_resident<8, false>);
+    else launch(bcast_add_rowsum_f32_resident<16, false>);
   } else if (vec) {
     hipLaunchKernelGGL(bcast_add_rowsum_f32_vec, dim3((unsigned)blocks), dim3(kThreads), 0,
                        stream, x, bias, y, m, n);
