@@ -100,11 +100,15 @@ def build_runtime():
     exe = os.path.join(HERE, "bin", "runtime-session")
     _run([CXX, "-o", exe, main_obj, "-L" + LIB, "-lAFIRRuntimeCAPI", "-L/opt/rocm/lib",
           "-lamdhip64", "-ldl", "-Wl,-rpath,$ORIGIN/../lib", "-Wl,-rpath,/opt/rocm/lib"])
+    at_obj = _compile_host("tools/autotuner_main.cpp")
+    at_exe = os.path.join(HERE, "bin", "autotuner")
+    _run([CXX, "-o", at_exe, at_obj, "-L" + LIB, "-lAFIRRuntimeCAPI", "-L/opt/rocm/lib",
+          "-lamdhip64", "-ldl", "-Wl,-rpath,$ORIGIN/../lib", "-Wl,-rpath,/opt/rocm/lib"])
     # afir-translate -mlir-to-hip: host-only, no HIP runtime needed
     tr_obj = _compile_host("tools/afir_translate_main.cpp")
     tr_exe = os.path.join(HERE, "bin", "afir-translate")
     _run([CXX, "-o", tr_exe, tr_obj, *[o for o in objs if "target_" in o]])
-    return [lib, exe, tr_exe]
+    return [lib, exe, at_exe, tr_exe]
 
 
 def build_all():

@@ -1,0 +1,93 @@
+"""Host-side checks of the autotuner CLI: reading a tiling space in the
+reference's format (tools/autotuner/autotuner_main.cpp:28-50 flags, :348-470
+space parsing), enumerating candidates, and the keys of best_config.json
+(:557-595).  The testing driver stands in for the GPU: it runs nothing and
+reports a kernel time that falls as block_dim grows."""
+import json
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+AT = os.path.join(ROOT, "ascend-mlir_amd", "bin", "autotuner")
+
+from mlir_cases import ROW_BIAS_REDUCE  # noqa: E402
+
+
+def _at(*args):
+    return subprocess.run([AT, *args], capture_output=True, text=True)
+
+
+def _setup(tmp_path, space):
+    (tmp_path / "k.mlir").write_text(ROW_BIAS_REDUCE)
+    np.save(tmp_path / "a.npy", np.ones(8, np.float16))
+    np.save(tmp_path / "b.npy", np.ones((8, 32), np.float16))
+    np.save(tmp_path / "e.npy", np.zeros(8, np.float16))
+    (tmp_path / "space.json").write_text(json.dumps(space))
+    return ["--space", str(tmp_path / "space.json"), "--kernel", str(tmp_path / "k.mlir"),
+            "--inputs", f"{tmp_path / 'a.npy'},{tmp_path / 'b.npy'}", "--expected", str(tmp_path / "e.npy"),
+            "--output", str(tmp_path / "best.json"), "--build-dir", str(tmp_path / "art"),
+            "--testing-driver=hip-success"]
+
+
+DIMS = [{"name": "dim_arg0_0", "type": "int64", "fixed": True, "shape_key": "M"},
+        {"name": "dim_arg1_0", "type": "int64", "fixed": True, "shape_key": "M"},
+        {"name": "dim_arg1_1", "type": "int64", "fixed": True, "shape_key": "N"},
+        {"name": "dim_arg2_0", "type": "int64"}]          # taken from e.npy
+
+
+def test_block_dim_candidates_and_best_config(tmp_path):
+    space = {"kernel": "rowbias_reduce", "kernel_file": "k.mlir", "soc": "gfx950",
+             "block_dim_values": [0, 64, 256, 128], "tiling_params": DIMS}
+    p = _at(*_setup(tmp_path, space), "--shape", "M=8,N=32", "--repeats", "2")
+    assert p.returncode == 0, p.stderr + p.stdout
+    lines = [l for l in p.stdout.splitlines() if l.startswith("[")]
+    assert len(lines) == 4 and lines[0].startswith("[1/4] block_dim=0 ...") and all(" OK " in l for l in lines)
+    best = json.loads((tmp_path / "best.json").read_text())
+    # every key the reference writes
+    for key in ("kernel_name", "kernel_type", "soc", "artifact_root", "manifest_path", "device_binary_path",
+                "kernel_file", "best", "config", "shape"):
+        assert key in best, key
+    assert set(best["best"]) >= {"block_dim", "cycle_count", "score", "max_abs_diff"}
+    assert best["best"]["block_dim"] == 256               # the testing driver's fastest
+    assert best["kernel_name"] == "rowbias_reduce" and best["soc"] == "gfx950"
+    assert best["kernel_file"] == "k.mlir" and best["shape"] == {"M": 8, "N": 32}
+    assert best["config"] == {"dim_arg0_0": 8, "dim_arg1_0": 8, "dim_arg1_1": 32, "dim_arg2_0": 8}
+    assert best["candidates"] == 4
+    assert os.path.exists(best["manifest_path"]) and os.path.exists(best["device_binary_path"])
+
+
+def test_search_parameters_and_block_dim_expr(tmp_path):
+    # a searched parameter in both notations; block_dim follows from it
+    space = {"block_dim_expr": "ceil(M / tile_m)",
+             "tiling_params": [{"name": "tile_m", "type": "int64", "values": [1, 2, 4]},
+                               {"name": "tile_n", "type": "int32", "min": 16, "max": 32, "step": 16},
+                               {"name": "m", "type": "int64", "fixed": True, "shape_key": "M"}]}
+    p = _at(*_setup(tmp_path, space), "--shape", "M=8,N=32")
+    assert p.returncode == 0, p.stderr + p.stdout
+    lines = [l for l in p.stdout.splitlines() if l.startswith("[")]
+    assert len(lines) == 6
+    assert any("tile_m=1" in l and "tile_n=32" in l and "block_dim=8 " in l for l in lines)
+    assert any("tile_m=4" in l and "block_dim=2 " in l for l in lines)
+    best = json.loads((tmp_path / "best.json").read_text())
+    assert best["best"]["block_dim"] == 8 and best["config"]["tile_m"] == 1 and best["config"]["m"] == 8
+
+
+def test_bad_invocations(tmp_path):
+    base = _setup(tmp_path, {"tiling_params": DIMS})
+    assert _at().returncode == 4
+    assert _at(*base).returncode == 4                                    # --shape missing
+    p = _at(*base, "--shape", "M=8")                                     # N missing
+    assert p.returncode == 4 and "shape key 'N'" in p.stderr
+    p = _at(*base, "--shape", "M=8,N=32", "--artifact-root", str(tmp_path / "art"))
+    assert p.returncode == 4 and "exactly one" in p.stderr
+    (tmp_path / "space.json").write_text(json.dumps({"tiling_params": [{"name": "tile"}]}))
+    p = _at(*base, "--shape", "M=8,N=32")
+    assert p.returncode == 4 and "no shape_key, value or candidates" in p.stderr
+    (tmp_path / "space.json").write_text(json.dumps(
+        {"block_dim_expr": "ceil(M / nope)", "tiling_params": DIMS}))
+    p = _at(*base, "--shape", "M=8,N=32")
+    assert p.returncode == 4 and "unknown name 'nope'" in p.stderr
+    (tmp_path / "space.json").write_text("[1, 2]")
+    assert _at(*base, "--shape", "M=8,N=32").returncode == 4

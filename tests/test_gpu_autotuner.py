@@ -1,0 +1,59 @@
+"""The autotuner on a real GPU: every candidate is launched, validated against
+the expected output and scored by its measured kernel time
+(reference flow: tools/autotuner/autotuner_main.cpp:700-860)."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+from mlir_cases import ROW_BIAS_REDUCE  # noqa: E402
+
+AT = os.path.join(ROOT, "ascend-mlir_amd", "bin", "autotuner")
+pytestmark = pytest.mark.gpu
+
+SPACE = {"kernel": "rowbias_reduce", "kernel_file": "k.mlir", "soc": "gfx950",
+         "block_dim_values": [0, 256, 1024, 4096],
+         "tiling_params": [{"name": "dim_arg0_0", "fixed": True, "shape_key": "M"},
+                           {"name": "dim_arg1_0", "fixed": True, "shape_key": "M"},
+                           {"name": "dim_arg1_1", "fixed": True, "shape_key": "N"},
+                           {"name": "dim_arg2_0", "fixed": True, "shape_key": "M"}]}
+
+
+def _run(tmp_path, expected, *extra):
+    (tmp_path / "k.mlir").write_text(ROW_BIAS_REDUCE)
+    (tmp_path / "space.json").write_text(json.dumps(SPACE))
+    np.save(tmp_path / "e.npy", expected)
+    return subprocess.run(
+        [AT, "--space", str(tmp_path / "space.json"), "--kernel", str(tmp_path / "k.mlir"),
+         "--inputs", f"{tmp_path / 'a.npy'},{tmp_path / 'b.npy'}", "--expected", str(tmp_path / "e.npy"),
+         "--shape", "M=2048,N=1024", "--output", str(tmp_path / "best.json"),
+         "--build-dir", str(tmp_path / "art"), *extra], capture_output=True, text=True, timeout=110)
+
+
+def test_autotune_row_bias_reduce(tmp_path):
+    rng = np.random.default_rng(5)
+    a = rng.standard_normal(2048).astype(np.float16)
+    b = rng.standard_normal((2048, 1024)).astype(np.float16)
+    np.save(tmp_path / "a.npy", a)
+    np.save(tmp_path / "b.npy", b)
+    want = (a[:, None].astype(np.float32) + b.astype(np.float32)).sum(axis=1).astype(np.float16)
+    p = _run(tmp_path, want, "--atol", "0.25", "--rtol", "0.01")
+    assert p.returncode == 0, p.stdout + p.stderr
+    lines = [l for l in p.stdout.splitlines() if l.startswith("[")]
+    assert len(lines) == 4 and all(" OK " in l for l in lines), p.stdout
+    best = json.loads((tmp_path / "best.json").read_text())
+    assert best["best"]["block_dim"] in (0, 256, 1024, 4096)
+    assert 0 < best["best"]["score"] < 5_000_000          # ns: a 4 MiB pass takes microseconds
+    assert best["best"]["max_abs_diff"] <= 0.25
+    scores = [float(l.split("score=")[1].split()[0]) for l in lines]
+    assert best["best"]["score"] == round(min(scores))
+
+    # an expected output no candidate can match: every candidate FAILs, exit 1
+    p = _run(tmp_path, want + np.float16(3.0), "--atol", "0.25", "--rtol", "0.01")
+    assert p.returncode == 1, p.stdout + p.stderr
+    assert p.stdout.count(" FAIL ") == 4 and "no candidate passed" in p.stderr
