@@ -38,8 +38,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # HBM bytes per step measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (two runs), scaled by the same counters' reading for a plain 256 MiB copy
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Source: profiles/*.txt, section (2).
-MEASURED_TRAFFIC = {"c1": 201364275, "c2": 134441381, "c3": 134502809, "c4": 134574489,
-                    "c5": 1869395968, "g1": 201536102, "g2": 134893568}
+MEASURED_TRAFFIC = {"c1": 201364070, "c2": 134645390, "c3": 134496358, "c4": 134578995,
+                    "c5": 1862780928, "g1": 201559961, "g2": 134977945}
 
 
 # Region programs of the two generic-kernel workloads (grammar:
