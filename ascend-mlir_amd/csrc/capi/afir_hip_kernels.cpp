@@ -16,6 +16,7 @@
 
 #include "../kernels/kernels.h"
 #include "../kernels/region_launch.h"
+#include "../target/hip_emitter.h"
 #include "../target/region_program.h"
 
 namespace {
@@ -72,13 +73,60 @@ constexpr int kNumKernels = (int)(sizeof(kKernels) / sizeof(kKernels[0]));
 // region kernel.  Matmul programs have no generic form: they must match.
 enum class FastPath { None, AddMul, BcastAddRowsum, ReluBcastTranspose, GatherScaleShift, MatmulBiasLeaky, MatmulBiasLeakyF16 };
 
+// A code object compiled for one program (afir_target::emitHipSource), loaded
+// on first launch.
+struct CompiledRegion {
+  std::vector<char> image;
+  std::mutex mutex;
+  bool loaded = false;
+  hipModule_t module = nullptr;
+  std::map<std::string, hipFunction_t> functions;
+  ~CompiledRegion() {
+    if (!loaded) return;
+    (void)hipDeviceSynchronize();   // no launch of this module may still be running
+    (void)hipModuleUnload(module);
+  }
+};
+
 struct RegisteredRegion {
   afir_region::Program program;
   std::vector<std::string> fields;
   FastPath fast = FastPath::None;
   int fastArgs[4] = {-1, -1, -1, -1};  // argument index of each kernel operand
   float alpha = 0.f;
+  std::shared_ptr<CompiledRegion> compiled;   // null: the interpreter kernel runs the program
 };
+
+// Loads the module if needed and looks a kernel up.  "" on success.
+std::string compiled_function(CompiledRegion *c, const afir_region::Program &program, const std::string &name,
+                              hipFunction_t *fn) {
+  std::lock_guard<std::mutex> lock(c->mutex);
+  if (!c->loaded) {
+    hipModule_t m = nullptr;
+    hipError_t e = hipModuleLoadData(&m, c->image.data());
+    if (e != hipSuccess) return std::string("code object does not load: ") + hipGetErrorString(e);
+    hipDeviceptr_t sym = nullptr;
+    size_t bytes = 0;
+    unsigned long long hash = 0;
+    e = hipModuleGetGlobal(&sym, &bytes, m, "afir_region_program_hash");
+    if (e == hipSuccess && bytes == sizeof hash) e = hipMemcpyDtoH(&hash, sym, sizeof hash);
+    if (e != hipSuccess || bytes != sizeof hash || hash != afir_target::programHash(program)) {
+      (void)hipModuleUnload(m);
+      return "code object was not built from this program";
+    }
+    c->module = m;
+    c->loaded = true;
+  }
+  auto it = c->functions.find(name);
+  if (it == c->functions.end()) {
+    hipFunction_t f = nullptr;
+    const hipError_t e = hipModuleGetFunction(&f, c->module, name.c_str());
+    if (e != hipSuccess) return "code object lacks kernel " + name + ": " + hipGetErrorString(e);
+    it = c->functions.emplace(name, f).first;
+  }
+  *fn = it->second;
+  return "";
+}
 
 bool is_push(const afir_region::Op &o, int rank, std::initializer_list<int> dims) {
   using afir_region::MapResult;
@@ -355,7 +403,39 @@ const char *afir_hip_region_kernel(uint64_t handle) {
     case FastPath::MatmulBiasLeakyF16: return "matmul_add_leakyrelu_f16";
     case FastPath::None: break;
   }
-  return "fused_region";
+  return r->compiled ? "fused_region_compiled" : "fused_region";
+}
+
+uint32_t afir_hip_region_emit_source(uint64_t handle, char *buffer, size_t capacity, size_t *length) {
+  auto r = find_region(handle);
+  if (!r) return fail(AFIR_HIP_E_UNKNOWN, "no region program with that handle");
+  if (!length) return fail(AFIR_HIP_E_INVALID, "region_emit_source: null length pointer");
+  std::string source;
+  const std::string why = afir_target::emitHipSource(r->program, "region", &source);
+  if (!why.empty()) return fail(AFIR_HIP_E_INVALID, "no specialised kernel: " + why);
+  *length = source.size();
+  if (buffer && capacity) {
+    const size_t n = source.size() < capacity - 1 ? source.size() : capacity - 1;
+    std::memcpy(buffer, source.data(), n);
+    buffer[n] = 0;
+  }
+  g_last_error.clear();
+  return AFIR_HIP_OK;
+}
+
+uint32_t afir_hip_region_attach_code_object(uint64_t handle, const void *image, size_t image_len) {
+  auto r = find_region(handle);
+  if (!r) return fail(AFIR_HIP_E_UNKNOWN, "no region program with that handle");
+  if (!image || image_len < 8) return fail(AFIR_HIP_E_INVALID, "region_attach_code_object: empty image");
+  for (const afir_region::Segment &g : r->program.segments)
+    if (!g.ops.empty() && g.ops[0].code == afir_region::OpCode::Matmul)
+      return fail(AFIR_HIP_E_INVALID, "matmul regions run on the hand-written kernels and take no code object");
+  auto c = std::make_shared<CompiledRegion>();
+  c->image.assign(static_cast<const char *>(image), static_cast<const char *>(image) + image_len);
+  std::lock_guard<std::mutex> lock(g_region_mutex);
+  r->compiled = std::move(c);
+  g_last_error.clear();
+  return AFIR_HIP_OK;
 }
 
 const char *afir_hip_region_tiling_field(uint64_t handle, int index) {
@@ -438,6 +518,15 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
   auto aligned = [](const void *p, int64_t bytes) {
     return ((reinterpret_cast<uintptr_t>(p) + (uintptr_t)bytes) & 15u) == 0;
   };
+  std::shared_ptr<CompiledRegion> compiled;
+  {
+    std::lock_guard<std::mutex> lock(g_region_mutex);
+    compiled = r->compiled;
+  }
+  // AFIR_HIP_REGION_INTERPRET=1 keeps programs with a code object on the
+  // interpreter kernel (the tests compare the two)
+  if (const char *env = std::getenv("AFIR_HIP_REGION_INTERPRET"))
+    if (*env && *env != '0') compiled.reset();
   for (const afir_region::ResolvedSegment &seg : res.segments) {
     afir::RegionArgs a;
     std::memset(&a, 0, sizeof a);
@@ -482,9 +571,55 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
       d.constant = op.constant;
       d.depth = op.depth;
     }
+    if (compiled) {
+      const int segment = (int)(&seg - res.segments.data());
+      const afir_target::SpecShape shape = afir_target::specShape(r->program, segment);
+      const int W = shape.width, U = shape.unroll;
+      afir::RegionGeometry g;
+      uint32_t rc = finish(afir::plan_fused_region(a, W * U, block_dim, &g));
+      if (rc != AFIR_HIP_OK) return rc;
+      if (g.empty) continue;
+      afir_target::SpecArgs sa;
+      std::memset(&sa, 0, sizeof sa);
+      for (int k = 0; k < 3; ++k) sa.size[k] = a.size[k];
+      sa.out = a.out;
+      sa.error_flag = a.error_flag;
+      sa.out_vec = a.out_vec;
+      sa.lanes_log2 = g.lanes_log2;
+      sa.grid = (int)g.blocks;
+      // the aligned variant has no tail handling: whole groups, whole passes
+      const int64_t groups = seg.size[last] / W;
+      const int64_t per_pass = (seg.reduce ? (int64_t)64 : ((int64_t)1 << g.lanes_log2)) * U;
+      bool all_aligned = seg.size[last] % W == 0 && groups % per_pass == 0 && (seg.reduce || a.out_vec);
+      for (int i = 0; i < a.ninputs; ++i) {
+        const afir::RegionInput &d = a.in[i];
+        afir_target::SpecInput &t = sa.in[i];
+        t.base = d.base;
+        t.index = d.index;
+        for (int k = 0; k < 3; ++k) t.stride[k] = d.stride[k];
+        t.offset = d.offset;
+        t.gstride = d.gstride;
+        t.gextent = d.gextent;
+        t.vec = d.vec;
+        t.gvec = d.gvec;
+        // operands that are contiguous along the innermost dim are read with
+        // 128-bit loads by the aligned variant
+        if (d.stride[last] == 1 && d.gdim != last && (!d.vec || (d.gdim >= 0 && !d.gvec))) all_aligned = false;
+      }
+      hipFunction_t fn = nullptr;
+      why = compiled_function(compiled.get(), r->program, afir_target::specKernelName(segment, g.idx32, all_aligned), &fn);
+      if (!why.empty()) return fail(AFIR_HIP_E_LAUNCH, why);
+      size_t bytes = sizeof sa;
+      void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &sa, HIP_LAUNCH_PARAM_BUFFER_SIZE, &bytes, HIP_LAUNCH_PARAM_END};
+      const hipError_t e = hipModuleLaunchKernel(fn, (unsigned)g.blocks, 1, 1, 256, 1, 1, 0,
+                                                 static_cast<hipStream_t>(stream), nullptr, config);
+      if (e != hipSuccess) return fail(AFIR_HIP_E_LAUNCH, std::string("compiled region kernel: ") + hipGetErrorString(e));
+      continue;
+    }
     uint32_t rc = finish(afir::launch_fused_region(a, block_dim, static_cast<hipStream_t>(stream)));
     if (rc != AFIR_HIP_OK) return rc;
   }
+  g_last_error.clear();
   return AFIR_HIP_OK;
 }
 

@@ -31,7 +31,7 @@ void writeErr(char *buf, size_t len, const std::string &msg) {
   buf[len - 1] = '\0';
 }
 
-afirt::Status runDescriptor(ExecutorHandle *h, const std::string &descriptorText,
+afirt::Status runDescriptor(ExecutorHandle *h, const std::string &descriptorText, const std::string &descriptorDir,
                             const char *function_name, int num_inputs, const void **input_ptrs,
                             const size_t *input_bytes, int num_outputs, void **output_ptrs,
                             const size_t *output_bytes, const uint8_t *tiling_data,
@@ -74,6 +74,7 @@ afirt::Status runDescriptor(ExecutorHandle *h, const std::string &descriptorText
   launch.sharedLibraryPath = d->library.empty() ? afirt::defaultKernelLibraryPath() : d->library;
   launch.symbolName = d->symbol;
   launch.regionProgram = d->program;
+  launch.codeObjectPath = afirt::resolveCodeObject(*d, descriptorDir);
   return h->runner->runDynamicLibraryArtifact(launch, args);
 }
 
@@ -159,7 +160,7 @@ int afirt_executor_run(AfirtExecutor executor, const uint8_t *binary_data, size_
     return 1;
   }
   std::string text(reinterpret_cast<const char *>(binary_data), binary_len);
-  afirt::Status st = runDescriptor(h, text, function_name, num_inputs, input_ptrs, input_bytes,
+  afirt::Status st = runDescriptor(h, text, "", function_name, num_inputs, input_ptrs, input_bytes,
                                    num_outputs, output_ptrs, output_bytes, tiling_data, tiling_len,
                                    block_dim, magic);
   if (!st.ok()) {
@@ -190,7 +191,9 @@ int afirt_executor_run_file(AfirtExecutor executor, const char *binary_path,
     return 1;
   }
   std::string text((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
-  afirt::Status st = runDescriptor(h, text, function_name, num_inputs, input_ptrs, input_bytes,
+  const std::string path = binary_path;
+  const size_t slash = path.find_last_of('/');
+  afirt::Status st = runDescriptor(h, text, slash == std::string::npos ? "." : path.substr(0, slash), function_name, num_inputs, input_ptrs, input_bytes,
                                    num_outputs, output_ptrs, output_bytes, tiling_data, tiling_len,
                                    block_dim, magic);
   if (!st.ok()) {

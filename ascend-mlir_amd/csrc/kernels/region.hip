@@ -492,11 +492,9 @@ bool linearize(RegionArgs &a) {
 
 }  // namespace
 
-LaunchStatus launch_fused_region(const RegionArgs &args_in, uint32_t block_dim, hipStream_t stream) {
-  RegionArgs args = args_in;
+LaunchStatus plan_fused_region(const RegionArgs &args, int vec, uint32_t block_dim, RegionGeometry *g) {
   if (args.rank < 1 || args.rank > 3) return invalid("fused_region: bad iteration rank");
-  if (args.nops < 0 || args.nops > kRegionMaxOps || args.ninputs < 0 || args.ninputs > kRegionMaxInputs)
-    return invalid("fused_region: program too large");
+  if (args.ninputs < 0 || args.ninputs > kRegionMaxInputs) return invalid("fused_region: program too large");
   int64_t rows = 1, total = 1;
   for (int k = 0; k < args.rank; ++k) {
     if (args.size[k] < 0) return invalid("fused_region: negative extent");
@@ -504,6 +502,52 @@ LaunchStatus launch_fused_region(const RegionArgs &args_in, uint32_t block_dim, 
     total *= args.size[k];
     if (k + 1 < args.rank) rows *= args.size[k];
   }
+  // 32-bit positions when every operand and the output stay below 2^31 elements
+  // (with room for the positions of a last, partly empty pass)
+  bool idx32 = total < ((int64_t)1 << 31) - 65536;
+  for (int i = 0; i < args.ninputs && idx32; ++i) {
+    int64_t reach = args.in[i].offset < 0 ? -args.in[i].offset : args.in[i].offset;
+    for (int k = 0; k < args.rank; ++k) {
+      const int64_t st = args.in[i].stride[k] < 0 ? -args.in[i].stride[k] : args.in[i].stride[k];
+      if (args.size[k] > 0 && st > (((int64_t)1 << 31) - 1 - reach) / args.size[k]) { idx32 = false; break; }
+      reach += st * (args.size[k] > 0 ? args.size[k] - 1 : 0);
+    }
+  }
+  g->idx32 = idx32;
+  g->lanes_log2 = 0;
+  g->blocks = 0;
+  if (args.reduce) {
+    if (args.rank < 2) return invalid("fused_region: reduction needs rank >= 2");
+    g->empty = rows == 0;
+    if (g->empty) return ok_status();
+    if (!args.out) return invalid("fused_region: null output pointer");
+    int64_t blocks = (rows + (kThreads / kWave) - 1) / (kThreads / kWave);
+    if (blocks > (int64_t)kNumCU * 8) blocks = (int64_t)kNumCU * 8;
+    if (block_dim) blocks = block_dim;
+    g->blocks = blocks;
+    return ok_status();
+  }
+  g->empty = total == 0;
+  if (g->empty) return ok_status();
+  if (!args.out) return invalid("fused_region: null output pointer");
+  const int64_t n = args.size[args.rank - 1];
+  const int64_t chunks = (n + vec - 1) / vec;
+  int lanes_log2 = 0;
+  while (lanes_log2 < 8 && ((int64_t)1 << lanes_log2) < chunks) ++lanes_log2;
+  const int rows_per_pass = kThreads >> lanes_log2;
+  int64_t blocks = (rows + rows_per_pass - 1) / rows_per_pass;
+  if (blocks > (int64_t)kNumCU * 16) blocks = (int64_t)kNumCU * 16;
+  if (block_dim) blocks = block_dim;
+  g->blocks = blocks;
+  g->lanes_log2 = lanes_log2;
+  return ok_status();
+}
+
+LaunchStatus launch_fused_region(const RegionArgs &args_in, uint32_t block_dim, hipStream_t stream) {
+  RegionArgs args = args_in;
+  if (args.rank < 1 || args.rank > 3) return invalid("fused_region: bad iteration rank");
+  if (args.nops < 0 || args.nops > kRegionMaxOps || args.ninputs < 0 || args.ninputs > kRegionMaxInputs)
+    return invalid("fused_region: program too large");
   // stack slots: the interpreter does not shift values, every operation is
   // told where its operands live
   int depth = 0;
@@ -532,50 +576,27 @@ LaunchStatus launch_fused_region(const RegionArgs &args_in, uint32_t block_dim, 
   if (const char *env = std::getenv("AFIR_HIP_REGION_STACK"))
     if (*env && *env != '0') args.chain = 0;
 
-  // 32-bit positions when every operand and the output stay below 2^31 elements
-  bool idx32 = total < ((int64_t)1 << 31);
-  for (int i = 0; i < args.ninputs && idx32; ++i) {
-    int64_t reach = args.in[i].offset < 0 ? -args.in[i].offset : args.in[i].offset;
-    for (int k = 0; k < args.rank; ++k) {
-      const int64_t st = args.in[i].stride[k] < 0 ? -args.in[i].stride[k] : args.in[i].stride[k];
-      if (args.size[k] > 0 && st > (((int64_t)1 << 31) - 1 - reach) / args.size[k]) { idx32 = false; break; }
-      reach += st * (args.size[k] > 0 ? args.size[k] - 1 : 0);
-    }
-  }
-
   // 32 bytes per lane and operand: 8 elements, or 16 when every tensor of a
   // chain is 16-bit (twice the bytes per interpreted step)
   bool wide = args.chain && args.out_type != kRegionF32;
   for (int i = 0; i < args.ninputs; ++i) wide = wide && args.in[i].type != kRegionF32;
   const int vec = wide ? 16 : 8;
 
+  RegionGeometry g;
+  const LaunchStatus planned = plan_fused_region(args, vec, block_dim, &g);
+  if (planned.code != 0 || g.empty) return planned;
+  const bool idx32 = g.idx32;
   if (args.reduce) {
-    if (args.rank < 2) return invalid("fused_region: reduction needs rank >= 2");
-    if (rows == 0) return ok_status();
-    if (!args.out) return invalid("fused_region: null output pointer");
-    int64_t blocks = (rows + (kThreads / kWave) - 1) / (kThreads / kWave);
-    if (blocks > (int64_t)kNumCU * 8) blocks = (int64_t)kNumCU * 8;
-    if (block_dim) blocks = block_dim;
     auto kernel = wide ? (idx32 ? fused_region_rowsum<int, true, 16> : fused_region_rowsum<int64_t, true, 16>)
                   : args.chain ? (idx32 ? fused_region_rowsum<int, true, 8> : fused_region_rowsum<int64_t, true, 8>)
                                : (idx32 ? fused_region_rowsum<int, false, 8> : fused_region_rowsum<int64_t, false, 8>);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), 0, stream, args);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)g.blocks), dim3(kThreads), 0, stream, args);
     return after_launch();
   }
-  if (total == 0) return ok_status();
-  if (!args.out) return invalid("fused_region: null output pointer");
-  const int64_t n = args.size[args.rank - 1];
-  const int64_t chunks = (n + vec - 1) / vec;
-  int lanes_log2 = 0;
-  while (lanes_log2 < 8 && ((int64_t)1 << lanes_log2) < chunks) ++lanes_log2;
-  const int rows_per_pass = kThreads >> lanes_log2;
-  int64_t blocks = (rows + rows_per_pass - 1) / rows_per_pass;
-  if (blocks > (int64_t)kNumCU * 16) blocks = (int64_t)kNumCU * 16;
-  if (block_dim) blocks = block_dim;
   auto kernel = wide ? (idx32 ? fused_region_parallel<int, true, 16> : fused_region_parallel<int64_t, true, 16>)
                 : args.chain ? (idx32 ? fused_region_parallel<int, true, 8> : fused_region_parallel<int64_t, true, 8>)
                              : (idx32 ? fused_region_parallel<int, false, 8> : fused_region_parallel<int64_t, false, 8>);
-  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kThreads), 0, stream, args, lanes_log2);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)g.blocks), dim3(kThreads), 0, stream, args, g.lanes_log2);
   return after_launch();
 }
 

@@ -86,4 +86,14 @@ struct RegionArgs {
 
 LaunchStatus launch_fused_region(const RegionArgs &args, uint32_t block_dim, hipStream_t stream);
 
+// Launch geometry of a segment for `vec` elements per lane and step: shared by
+// the interpreter kernels and by kernels compiled for one program.
+struct RegionGeometry {
+  int64_t blocks = 0;    // workgroups of 256 lanes
+  int lanes_log2 = 0;    // parallel segments: 2^lanes_log2 lanes share a row
+  bool idx32 = false;    // every position fits 32 bits
+  bool empty = false;    // nothing to compute
+};
+LaunchStatus plan_fused_region(const RegionArgs &args, int vec, uint32_t block_dim, RegionGeometry *geometry);
+
 }  // namespace afir

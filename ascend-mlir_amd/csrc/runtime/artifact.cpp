@@ -1,11 +1,14 @@
 // Artifact directories and run manifests.
 //
-// On this backend the device code is precompiled in the kernel library, so
-// "compiling" a fused region means translating its IR to a region program
+// "Compiling" a fused region means translating its IR to a region program
 // (csrc/target/mlir_translate.h) -- or taking an explicit request for one of
-// the hand-tuned kernel families -- and writing an artifact that carries it:
+// the hand-tuned kernel families of the kernel library -- emitting HIP source
+// specialised for the program (csrc/target/hip_emitter.h), compiling that with
+// hipcc and writing an artifact that carries it all:
 //     <root>/<kernel_name>.hipk      descriptor (key=value text, then the
 //                                    region program after a "program:" line)
+//     <root>/<kernel_name>.hip       emitted kernel source    } region programs,
+//     <root>/<kernel_name>.hsaco     its gfx950 code object   } when hipcc is there
 //     <root>/out/manifest.txt        kernel_name= soc_version= kernel_kind=
 //                                    device_binary_path= manifest_path=
 //                                    kernel_so_path= kernel_so_symbol=
@@ -14,13 +17,23 @@
 // the key its mix artifacts use for a launcher library
 // (lib/Runtime/Artifact/RuntimeSessionRequestBuilder.cpp:374-455).
 #include <dlfcn.h>
+#include <fcntl.h>
+#include <spawn.h>
 #include <sys/stat.h>
+#include <sys/wait.h>
+#include <unistd.h>
 
+#include <cerrno>
+#include <climits>
+#include <cstdlib>
 #include <cstring>
 #include <fstream>
 #include <sstream>
 
+#include "../target/hip_emitter.h"
 #include "../target/mlir_translate.h"
+
+extern char **environ;
 #include "runtime.h"
 
 namespace afirt {
@@ -150,6 +163,10 @@ std::string serializeDescriptor(const HipKernelDescriptor &d) {
   s += "hip_kernel=" + d.hipKernel + "\n";
   s += "library=" + d.library + "\n";
   s += "symbol=" + d.symbol + "\n";
+  if (!d.codeObject.empty()) {
+    s += "code_object=" + d.codeObject + "\n";
+    s += "code_object_dir=" + d.codeObjectDir + "\n";
+  }
   if (!d.program.empty()) s += "program:\n" + d.program;
   return s;
 }
@@ -171,6 +188,8 @@ Expected<HipKernelDescriptor> parseDescriptor(const std::string &text) {
   d.library = kv["library"];
   d.symbol = kv["symbol"];
   d.program = program;
+  d.codeObject = kv["code_object"];
+  d.codeObjectDir = kv["code_object_dir"];
   if (d.hipKernel.empty()) return Status::error("artifact descriptor names no hip_kernel");
   const KnownKernel *k = findKnown(d.hipKernel);
   if (!k) return Status::error("artifact descriptor names an unknown hip_kernel: " + d.hipKernel);
@@ -179,6 +198,76 @@ Expected<HipKernelDescriptor> parseDescriptor(const std::string &text) {
   if (d.symbol.empty()) d.symbol = k->symbol;
   if (d.kernelName.empty()) d.kernelName = d.hipKernel;
   return d;
+}
+
+namespace {
+std::string absolutePath(const std::string &path) {
+  char buf[PATH_MAX];
+  return realpath(path.c_str(), buf) ? std::string(buf) : path;
+}
+}  // namespace
+
+std::string resolveCodeObject(const HipKernelDescriptor &d, const std::string &descriptorDir) {
+  if (d.codeObject.empty()) return "";
+  if (!descriptorDir.empty() && fileExists(joinPath(descriptorDir, d.codeObject)))
+    return joinPath(descriptorDir, d.codeObject);
+  if (!d.codeObjectDir.empty() && fileExists(joinPath(d.codeObjectDir, d.codeObject)))
+    return joinPath(d.codeObjectDir, d.codeObject);
+  return "";
+}
+
+Expected<std::string> compileRegionCodeObject(const std::string &programText, const std::string &dir,
+                                              const std::string &name) {
+  if (const char *env = std::getenv("AFIR_HIP_CODEGEN"))
+    if (*env == '0') return Status::error("disabled by AFIR_HIP_CODEGEN=0");
+  afir_region::Program program;
+  if (std::string why = afir_region::parse(programText, &program); !why.empty()) return Status::error(why);
+  std::string source;
+  if (std::string why = afir_target::emitHipSource(program, name, &source); !why.empty()) return Status::error(why);
+  const std::string srcPath = joinPath(dir, name + ".hip"), objName = name + ".hsaco",
+                    objPath = joinPath(dir, objName), logPath = joinPath(dir, name + ".hipcc.log");
+  {
+    std::ofstream f(srcPath, std::ios::trunc);
+    if (!f) return Status::error("cannot write " + srcPath);
+    f << source;
+  }
+  std::string hipcc;
+  if (const char *env = std::getenv("HIPCC")) hipcc = env;
+  if (hipcc.empty()) {
+    const char *path = std::getenv("PATH");
+    std::istringstream dirs(path ? path : "");
+    for (std::string d; std::getline(dirs, d, ':');)
+      if (!d.empty() && access(joinPath(d, "hipcc").c_str(), X_OK) == 0) {
+        hipcc = joinPath(d, "hipcc");
+        break;
+      }
+  }
+  if (hipcc.empty() && access("/opt/rocm/bin/hipcc", X_OK) == 0) hipcc = "/opt/rocm/bin/hipcc";
+  if (hipcc.empty()) return Status::error("hipcc not found (set HIPCC); the source is kept at " + srcPath);
+  std::vector<std::string> argv = {hipcc, "--genco", "--offload-arch=gfx950", "-O3", "-nogpuinc", "-ffp-contract=off",
+                                   "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-o", objPath, srcPath};
+  std::vector<char *> cargv;
+  for (std::string &a : argv) cargv.push_back(a.data());
+  cargv.push_back(nullptr);
+  posix_spawn_file_actions_t actions;
+  posix_spawn_file_actions_init(&actions);
+  posix_spawn_file_actions_addopen(&actions, 1, logPath.c_str(), O_WRONLY | O_CREAT | O_TRUNC, 0644);
+  posix_spawn_file_actions_adddup2(&actions, 1, 2);
+  pid_t pid = 0;
+  const int rc = posix_spawn(&pid, hipcc.c_str(), &actions, nullptr, cargv.data(), environ);
+  posix_spawn_file_actions_destroy(&actions);
+  if (rc != 0) return Status::error("cannot start " + hipcc + ": " + std::strerror(rc));
+  int status = 0;
+  while (waitpid(pid, &status, 0) < 0)
+    if (errno != EINTR) return Status::error("waitpid failed for hipcc");
+  if (!WIFEXITED(status) || WEXITSTATUS(status) != 0 || !fileExists(objPath)) {
+    auto log = readTextFile(logPath);
+    std::string tail = log ? *log : "";
+    if (tail.size() > 1500) tail = tail.substr(tail.size() - 1500);
+    return Status::error("hipcc rejected " + srcPath + ":\n" + tail);
+  }
+  std::remove(logPath.c_str());
+  return objName;
 }
 
 Expected<HipKernelDescriptor> compileSourceText(const std::string &text, const std::string &nameHint) {
@@ -245,6 +334,18 @@ Expected<KernelArtifact> compileArtifact(const CompileRequest &request) {
   HipKernelDescriptor d = *compiled;
   d.kernelName = name;
   d.library = defaultKernelLibraryPath();
+  std::string codegenNote;
+  if (!d.program.empty()) {
+    // kernels specialised for the program; without them the interpreter
+    // kernel of the library runs it
+    auto object = compileRegionCodeObject(d.program, request.outputDir, name);
+    if (object) {
+      d.codeObject = *object;
+      d.codeObjectDir = absolutePath(request.outputDir);
+    } else {
+      codegenNote = object.error();
+    }
+  }
   const std::string binRel = name + ".hipk";
   const std::string binPath = joinPath(request.outputDir, binRel);
   {
@@ -257,6 +358,8 @@ Expected<KernelArtifact> compileArtifact(const CompileRequest &request) {
   a.kernelKind = request.kernelKind ? *request.kernelKind
                  : (d.program.find("\nmatmul ") != std::string::npos ? KernelKind::Mix : known->kind);
   a.regionProgram = d.program;
+  a.codeObjectPath = resolveCodeObject(d, request.outputDir);
+  a.codegenNote = codegenNote;
   a.socVersion = request.socVersion.empty() ? "gfx950" : request.socVersion;
   a.artifactRoot = request.outputDir;
   a.deviceBinaryPath = binPath;
@@ -273,6 +376,11 @@ Expected<KernelArtifact> compileArtifact(const CompileRequest &request) {
     f << "manifest_path=out/manifest.txt\n";
     f << "kernel_so_path=" << a.sharedLibraryPath << "\n";
     f << "kernel_so_symbol=" << a.sharedLibrarySymbol << "\n";
+    if (!d.codeObject.empty()) f << "code_object_path=" << d.codeObject << "\n";
+    if (!codegenNote.empty()) {
+      std::string oneLine = codegenNote.substr(0, codegenNote.find('\n'));
+      f << "code_object_note=" << oneLine << "\n";
+    }
   }
   return a;
 }
@@ -309,6 +417,8 @@ Expected<KernelArtifact> loadArtifactFromRoot(const std::string &root) {
   if (a.sharedLibraryPath.empty()) a.sharedLibraryPath = defaultKernelLibraryPath();
   if (a.sharedLibrarySymbol.empty()) a.sharedLibrarySymbol = d->symbol;
   a.regionProgram = d->program;
+  a.codeObjectPath = resolveCodeObject(*d, root);
+  a.codegenNote = kv["code_object_note"];
   return a;
 }
 

@@ -13,6 +13,9 @@
 // carries no shapes and a short buffer would otherwise be read past its end on
 // the device.
 #include <dlfcn.h>
+
+#include <fstream>
+#include <iterator>
 #include <hip/hip_runtime.h>
 
 #include <chrono>
@@ -94,6 +97,8 @@ class HipExecutionRunner final : public ExecutionRunner {
     dl.sharedLibraryPath = d->library.empty() ? defaultKernelLibraryPath() : d->library;
     dl.symbolName = d->symbol;
     dl.regionProgram = d->program;
+    const size_t slash = launch.binaryPath.find_last_of('/');
+    dl.codeObjectPath = resolveCodeObject(*d, slash == std::string::npos ? "." : launch.binaryPath.substr(0, slash));
     return runDynamicLibraryArtifact(dl, args);
   }
 
@@ -143,6 +148,16 @@ class HipExecutionRunner final : public ExecutionRunner {
         return Status::error("invalid region program in artifact: " + why());
       regionGuard.fn = unreg;
       regionGuard.handle = region;
+      if (!launch.codeObjectPath.empty()) {
+        // kernels compiled for this program run in place of the interpreter
+        using AttachFn = uint32_t (*)(uint64_t, const void *, size_t);
+        auto attach = reinterpret_cast<AttachFn>(dlsym(lib, "afir_hip_region_attach_code_object"));
+        std::ifstream f(launch.codeObjectPath, std::ios::binary);
+        if (!attach || !f) return Status::error("cannot attach code object " + launch.codeObjectPath);
+        const std::string image((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+        if (attach(region, image.data(), image.size()) != 0)
+          return Status::error("code object " + launch.codeObjectPath + " rejected: " + why());
+      }
       if (Status st = validateRegion(lib, region, args, why); !st.ok()) return st;
     }
 

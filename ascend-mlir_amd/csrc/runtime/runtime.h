@@ -181,6 +181,8 @@ struct KernelArtifact {
   std::string sharedLibrarySymbol;  // launcher symbol
   std::string manifestPath;         // <root>/out/manifest.txt
   std::string regionProgram;        // fused_region artifacts: the program text
+  std::string codeObjectPath;       // fused_region artifacts: kernels compiled for the program ("" = none)
+  std::string codegenNote;          // why there is no code object, when there is none
 };
 
 // The descriptor a "compiled" fused region consists of on this backend: the
@@ -191,7 +193,20 @@ struct HipKernelDescriptor {
   std::string library;      // path or soname of the kernel library ("" = default)
   std::string symbol;       // launcher symbol
   std::string program;      // hip_kernel == "fused_region": the region program text
+  // Kernels compiled for the program (hipcc --genco of the emitted source):
+  // file name beside the descriptor, and the directory it was written to.
+  std::string codeObject;
+  std::string codeObjectDir;
 };
+// Path of the descriptor's code object: beside the descriptor when its
+// directory is known and the file is there, else where it was compiled; ""
+// when there is none.
+std::string resolveCodeObject(const HipKernelDescriptor &d, const std::string &descriptorDir);
+// Emits the HIP source of a region program to <dir>/<name>.hip and compiles it
+// to <dir>/<name>.hsaco with hipcc ($HIPCC, PATH, /opt/rocm/bin).  Returns the
+// code object's file name, or an error saying why there is none.
+Expected<std::string> compileRegionCodeObject(const std::string &programText, const std::string &dir,
+                                              const std::string &name);
 std::string serializeDescriptor(const HipKernelDescriptor &d);
 Expected<HipKernelDescriptor> parseDescriptor(const std::string &text);
 
@@ -267,6 +282,9 @@ struct DynamicLibraryExecutionLaunch {
   // the library (afir_hip_region_register) and launched by handle instead of
   // through a 16-slot launcher symbol.
   std::string regionProgram;
+  // Optional code object compiled for that program; attached after
+  // registration so the launch runs the compiled kernels.
+  std::string codeObjectPath;
 };
 
 class ExecutionRunner {

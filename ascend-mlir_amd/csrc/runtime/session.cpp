@@ -94,6 +94,7 @@ SessionSummary runSingleTask(const RunTaskSpec &task, RunnerFactory factory, int
   launch.sharedLibraryPath = artifact->sharedLibraryPath;
   launch.symbolName = artifact->sharedLibrarySymbol;
   launch.regionProgram = artifact->regionProgram;
+  launch.codeObjectPath = artifact->codeObjectPath;
   if (Status st = runner->runDynamicLibraryArtifact(launch, args); !st.ok())
     return fail(summary, "kernel_launch", st.message);
   const double us = runner->lastKernelMicroseconds();

@@ -1,0 +1,665 @@
+#include "hip_emitter.h"
+
+#include <cstddef>
+#include <cstdio>
+#include <cstring>
+#include <sstream>
+#include <vector>
+
+namespace afir_target {
+
+using namespace afir_region;
+
+namespace {
+
+// Device helpers of every emitted file.  Builtins only: the file compiles with
+// -nogpuinc.
+const char *const kPrelude = R"HIP(
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+#define DEV static __attribute__((device)) inline __attribute__((always_inline))
+#define KERNEL extern "C" __attribute__((global)) __attribute__((amdgpu_flat_work_group_size(256, 256)))
+
+struct SpecInput {
+  const void *base;
+  const void *index;
+  long long stride[3];
+  long long offset;
+  long long gstride;
+  long long gextent;
+  int vec;
+  int gvec;
+};
+struct SpecArgs {
+  long long size[3];
+  void *out;
+  int *error_flag;
+  int out_vec;
+  int lanes_log2;
+  int grid;
+  int pad;
+  SpecInput in[8];
+};
+
+DEV float as_f32(unsigned u) { return __builtin_bit_cast(float, u); }
+DEV unsigned as_u32(float f) { return __builtin_bit_cast(unsigned, f); }
+DEV float fmax_ieee(float a, float b) { return __builtin_elementwise_maximum(a, b); }
+DEV float fmin_ieee(float a, float b) { return __builtin_elementwise_minimum(a, b); }
+
+// ---- element access: float32 in registers, one round-to-nearest-even on store
+DEV float ld_f32(const void *b, long long i) { return ((const float *)b)[i]; }
+DEV float ld_f16(const void *b, long long i) {
+  return (float)__builtin_bit_cast(_Float16, ((const unsigned short *)b)[i]);
+}
+DEV float ld_bf16(const void *b, long long i) { return as_f32((unsigned)((const unsigned short *)b)[i] << 16); }
+DEV long long ld_i32(const void *b, long long i) { return ((const int *)b)[i]; }
+DEV long long ld_i64(const void *b, long long i) { return ((const long long *)b)[i]; }
+DEV unsigned bf16_rne(float f) {
+  const unsigned u = as_u32(f);
+  const unsigned r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+  return (f != f) ? ((u >> 16) | 0x40u) : r;
+}
+DEV void st_f32(void *o, long long i, float x) { ((float *)o)[i] = x; }
+DEV void st_f16(void *o, long long i, float x) {
+  ((unsigned short *)o)[i] = __builtin_bit_cast(unsigned short, (_Float16)x);
+}
+DEV void st_bf16(void *o, long long i, float x) { ((unsigned short *)o)[i] = (unsigned short)bf16_rne(x); }
+
+// ---- 128-bit access; NT: the tensor is read exactly once by the launch
+template <bool NT> DEV f32x4 ld128(const f32x4 *p) { return NT ? __builtin_nontemporal_load(p) : *p; }
+template <bool NT> DEV u32x4 ld128(const u32x4 *p) { return NT ? __builtin_nontemporal_load(p) : *p; }
+template <int V, bool NT> DEV void ldv_f32(const void *b, long long i, float (&v)[V]) {
+  const f32x4 *p = (const f32x4 *)((const float *)b + i);
+#pragma unroll
+  for (int q = 0; q < V / 4; ++q) {
+    const f32x4 a = ld128<NT>(p + q);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[4 * q + e] = a[e];
+  }
+}
+template <int V, bool NT> DEV void ldv_f16(const void *b, long long i, float (&v)[V]) {
+  const u32x4 *p = (const u32x4 *)((const unsigned short *)b + i);
+#pragma unroll
+  for (int q = 0; q < V / 8; ++q) {
+    const u32x4 raw = ld128<NT>(p + q);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const unsigned word = raw[d];   // a copy: bit_cast of a vector element reads element 0
+      const f16x2 h = __builtin_bit_cast(f16x2, word);
+      v[8 * q + 2 * d] = (float)h.x;
+      v[8 * q + 2 * d + 1] = (float)h.y;
+    }
+  }
+}
+template <int V, bool NT> DEV void ldv_bf16(const void *b, long long i, float (&v)[V]) {
+  const u32x4 *p = (const u32x4 *)((const unsigned short *)b + i);
+#pragma unroll
+  for (int q = 0; q < V / 8; ++q) {
+    const u32x4 raw = ld128<NT>(p + q);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      v[8 * q + 2 * d] = as_f32(raw[d] << 16);
+      v[8 * q + 2 * d + 1] = as_f32(raw[d] & 0xffff0000u);
+    }
+  }
+}
+template <int V> DEV void stv_f32(void *o, long long i, const float (&v)[V]) {
+  f32x4 *p = (f32x4 *)((float *)o + i);
+#pragma unroll
+  for (int q = 0; q < V / 4; ++q) {
+    f32x4 a;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) a[e] = v[4 * q + e];
+    __builtin_nontemporal_store(a, p + q);
+  }
+}
+template <int V> DEV void stv_f16(void *o, long long i, const float (&v)[V]) {
+  u32x4 *p = (u32x4 *)((unsigned short *)o + i);
+#pragma unroll
+  for (int q = 0; q < V / 8; ++q) {
+    u32x4 w;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      f16x2 h;
+      h.x = (_Float16)v[8 * q + 2 * d];
+      h.y = (_Float16)v[8 * q + 2 * d + 1];
+      w[d] = __builtin_bit_cast(unsigned, h);
+    }
+    __builtin_nontemporal_store(w, p + q);
+  }
+}
+template <int V> DEV void stv_bf16(void *o, long long i, const float (&v)[V]) {
+  u32x4 *p = (u32x4 *)((unsigned short *)o + i);
+#pragma unroll
+  for (int q = 0; q < V / 8; ++q) {
+    u32x4 w;
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+      w[d] = (bf16_rne(v[8 * q + 2 * d]) & 0xffffu) | (bf16_rne(v[8 * q + 2 * d + 1]) << 16);
+    __builtin_nontemporal_store(w, p + q);
+  }
+}
+
+// ---- sum over the 64 lanes of a wavefront, fixed order: quad butterflies,
+// half-row and row mirrors, then the four row totals
+template <int C> DEV float dpp_add(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), C, 0xf, 0xf, true);
+  return v + __builtin_bit_cast(float, moved);
+}
+DEV float wave_sum(float v) {
+  v = dpp_add<0xB1>(v);
+  v = dpp_add<0x4E>(v);
+  v = dpp_add<0x141>(v);
+  v = dpp_add<0x140>(v);
+  const int iv = __builtin_bit_cast(int, v);
+  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 0));
+  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 16));
+  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 32));
+  const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 48));
+  return (r0 + r1) + (r2 + r3);
+}
+)HIP";
+
+const char *typeTag(ElemType t) {
+  switch (t) {
+    case ElemType::F16: return "f16";
+    case ElemType::BF16: return "bf16";
+    case ElemType::F32: return "f32";
+    case ElemType::I32: return "i32";
+    case ElemType::I64: return "i64";
+  }
+  return "f32";
+}
+
+std::string floatLiteral(float f) {
+  uint32_t u;
+  std::memcpy(&u, &f, 4);
+  char buf[64];
+  std::snprintf(buf, sizeof buf, "as_f32(0x%08xu) /* %g */", u, (double)f);
+  return buf;
+}
+
+// One distinct operand read of a segment.
+struct Operand {
+  int slot = 0;            // index into SpecArgs::in (the first push that reads it)
+  ElemType type = ElemType::F32;
+  enum Step { Broadcast, Contiguous, Strided } step = Broadcast;
+  int gatherDim = -1;      // iteration dim that indexes the index tensor
+  ElemType gatherType = ElemType::I64;
+  bool usesDim[kMaxRank] = {false, false, false};
+  bool readOnce = false;   // every iteration dim addresses it: no reuse across the launch
+};
+
+bool sameRead(const Op &a, const Op &b) {
+  if (a.arg != b.arg || a.map.size() != b.map.size() || a.slice.size() != b.slice.size()) return false;
+  for (size_t i = 0; i < a.map.size(); ++i) {
+    const MapResult &x = a.map[i], &y = b.map[i];
+    if (x.kind != y.kind || x.iterDim != y.iterDim || x.constant != y.constant || x.indexArg != y.indexArg)
+      return false;
+  }
+  for (size_t i = 0; i < a.slice.size(); ++i)
+    if (a.slice[i].arg != b.slice[i].arg || a.slice[i].dim != b.slice[i].dim ||
+        a.slice[i].constant != b.slice[i].constant)
+      return false;
+  return true;
+}
+
+struct Value {
+  std::string name;
+  bool scalar = false;
+  std::string at() const { return scalar ? name : name + "[u][e]"; }
+};
+
+// A lane's share of one pass over a row: U groups of W consecutive elements,
+// the groups 2^lanes_log2 * W elements apart, so that every load or store
+// instruction of a wavefront covers one contiguous run of memory.
+class SegmentEmitter {
+ public:
+  SegmentEmitter(const Program &p, int index, std::ostringstream &os)
+      : p_(p), seg_(p.segments[index]), index_(index), os_(os) {}
+
+  std::string run() {
+    if (!seg_.ops.empty() && seg_.ops[0].code == OpCode::Matmul)
+      return "matmul segments run on the hand-written MFMA kernels";
+    rank_ = seg_.rank;
+    last_ = rank_ - 1;
+    reduce_ = seg_.reduces();
+    const SpecShape shape = specShape(p_, index_);
+    W_ = shape.width;
+    U_ = shape.unroll;
+    collectOperands();
+    if ((int)pushSlot_.size() > kSpecMaxInputs) return "more than 8 operand reads in a segment";
+    emitBody();
+    emitWrappers();
+    return "";
+  }
+
+ private:
+  void collectOperands() {
+    int slot = 0;
+    std::vector<const Op *> firsts;
+    for (const Op &op : seg_.ops) {
+      if (op.code != OpCode::Push) continue;
+      int found = -1;
+      for (size_t i = 0; i < firsts.size(); ++i)
+        if (sameRead(*firsts[i], op)) found = (int)i;
+      if (found < 0) {
+        Operand o;
+        o.slot = slot;
+        o.type = p_.args[op.arg].type;
+        int lastHits = 0;
+        bool lastInnermost = false;
+        for (size_t d = 0; d < op.map.size(); ++d) {
+          const MapResult &m = op.map[d];
+          if (m.kind == MapResult::IterDim) {
+            o.usesDim[m.iterDim] = true;
+            if (m.iterDim == last_) {
+              ++lastHits;
+              lastInnermost = d + 1 == op.map.size();
+            }
+          } else if (m.kind == MapResult::Gather) {
+            o.gatherDim = m.iterDim;
+            o.gatherType = p_.args[m.indexArg].type;
+          }
+        }
+        o.step = lastHits == 0 ? Operand::Broadcast
+                               : (lastHits == 1 && lastInnermost ? Operand::Contiguous : Operand::Strided);
+        o.readOnce = true;
+        for (int k = 0; k < rank_; ++k)
+          if (!o.usesDim[k] && o.gatherDim != k) o.readOnce = false;
+        if (o.gatherDim >= 0) o.readOnce = false;   // gathered rows may repeat
+        found = (int)firsts.size();
+        firsts.push_back(&op);
+        operands_.push_back(o);
+      }
+      pushSlot_.push_back(found);
+      ++slot;
+    }
+  }
+
+  std::string in(const Operand &o) const { return "R.in[" + std::to_string(o.slot) + "]"; }
+  std::string id(const Operand &o) const { return std::to_string(o.slot); }
+  void line(int depth, const std::string &text) { os_ << std::string(2 * depth, ' ') << text << "\n"; }
+  void unroll() { os_ << "#pragma unroll\n"; }
+
+  // Row-invariant part of every operand: its position without the innermost
+  // dim, the index of a gather along an outer dim, the value of an operand that
+  // is broadcast along the innermost dim.
+  void emitRowInvariants(int d) {
+    for (const Operand &o : operands_) {
+      const std::string u = id(o), r = in(o);
+      std::string pos = "(I)" + r + ".offset";
+      for (int k = 0; k < last_; ++k)
+        if (o.usesDim[k]) pos += " + x" + std::to_string(k) + " * (I)" + r + ".stride[" + std::to_string(k) + "]";
+      const bool outerGather = o.gatherDim >= 0 && o.gatherDim != last_;
+      if (outerGather) {
+        line(d, "const long long g" + u + " = ld_" + typeTag(o.gatherType) + "(" + r + ".index, x" +
+                    std::to_string(o.gatherDim) + ");");
+        line(d, "const bool bad" + u + " = g" + u + " < 0 || g" + u + " >= " + r + ".gextent;");
+        line(d, "if (bad" + u + " && R.error_flag) *R.error_flag = 1;");
+        line(d, "const long long q" + u + " = (long long)(" + pos + ") + (bad" + u + " ? 0 : g" + u + " * " + r +
+                    ".gstride);");
+      } else {
+        line(d, "const long long q" + u + " = (long long)(" + pos + ");");
+      }
+      if (o.step == Operand::Broadcast && o.gatherDim != last_)
+        line(d, "const float s" + u + " = " + (outerGather ? "bad" + u + " ? as_f32(0x7fc00000u) : " : "") + "ld_" +
+                    typeTag(o.type) + "(" + r + ".base, q" + u + ");");
+    }
+  }
+
+  // Operand values for the U groups of this pass; returns the value name.
+  Value emitRead(const Operand &o, int d) {
+    const std::string u = id(o), r = in(o), tag = typeTag(o.type);
+    Value v;
+    if (o.step == Operand::Broadcast && o.gatherDim != last_) {
+      v.name = "s" + u;
+      v.scalar = true;
+      return v;
+    }
+    v.name = "v" + u;
+    line(d, "float v" + u + "[U][W];");
+    const std::string nan = "as_f32(0x7fc00000u)";
+    if (o.gatherDim == last_) {
+      // one index per element
+      line(d, "{");
+      line(d + 1, std::string("const long long step = ") +
+                      (o.step == Operand::Broadcast ? "0" : r + ".stride[" + std::to_string(last_) + "]") + ";");
+      unroll();
+      line(d + 1, "for (int u = 0; u < U; ++u) {");
+      unroll();
+      line(d + 2, "for (int e = 0; e < W; ++e) {");
+      line(d + 3, "float x = 0.f;");
+      line(d + 3, "if (e < nvalid[u]) {");
+      line(d + 4, "const long long g = ld_" + std::string(typeTag(o.gatherType)) + "(" + r + ".index, (long long)j0[u] + e);");
+      line(d + 4, "if (g < 0 || g >= " + r + ".gextent) {");
+      line(d + 5, "if (R.error_flag) *R.error_flag = 1;");
+      line(d + 5, "x = " + nan + ";");
+      line(d + 4, "} else {");
+      line(d + 5, "x = ld_" + tag + "(" + r + ".base, q" + u + " + ((long long)j0[u] + e) * step + g * " + r + ".gstride);");
+      line(d + 4, "}");
+      line(d + 3, "}");
+      line(d + 3, "v" + u + "[u][e] = x;");
+      line(d + 2, "}");
+      line(d + 1, "}");
+      line(d, "}");
+      return v;
+    }
+    const bool outerGather = o.gatherDim >= 0;
+    const std::string nt = o.readOnce ? "true" : "false";
+    if (o.step == Operand::Contiguous) {
+      unroll();
+      line(d, "for (int u = 0; u < U; ++u) {");
+      line(d + 1, "if (A || (full[u] && vec" + u + ")) {");
+      line(d + 2, "ldv_" + tag + "<W, " + nt + ">(" + r + ".base, q" + u + " + j0[u], v" + u + "[u]);");
+      line(d + 1, "} else {");
+      unroll();
+      line(d + 2, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = e < nvalid[u] ? ld_" + tag + "(" + r + ".base, q" + u +
+                      " + j0[u] + e) : 0.f;");
+      line(d + 1, "}");
+      line(d, "}");
+    } else {
+      // the stride along the innermost dim is a launch argument; a stride of
+      // one (a trailing extent of 1) still takes the 128-bit path
+      line(d, "{");
+      line(d + 1, "const long long step = " + r + ".stride[" + std::to_string(last_) + "];");
+      unroll();
+      line(d + 1, "for (int u = 0; u < U; ++u) {");
+      line(d + 2, "if (step == 1 && (A || (full[u] && vec" + u + "))) {");
+      line(d + 3, "ldv_" + tag + "<W, " + nt + ">(" + r + ".base, q" + u + " + j0[u], v" + u + "[u]);");
+      line(d + 2, "} else {");
+      unroll();
+      line(d + 3, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = e < nvalid[u] ? ld_" + tag + "(" + r + ".base, q" + u +
+                      " + ((long long)j0[u] + e) * step) : 0.f;");
+      line(d + 2, "}");
+      line(d + 1, "}");
+      line(d, "}");
+    }
+    if (outerGather) {
+      line(d, "if (bad" + u + ") {");
+      unroll();
+      line(d + 1, "for (int u = 0; u < U; ++u)");
+      unroll();
+      line(d + 2, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = " + nan + ";");
+      line(d, "}");
+    }
+    return v;
+  }
+
+  // The expression for the U groups of this pass; returns the value to store.
+  Value emitExpression(int d) {
+    std::vector<Value> stack;
+    std::vector<Value> read(operands_.size());
+    std::vector<bool> have(operands_.size(), false);
+    int push = 0, temp = 0;
+    auto fresh = [&](bool scalar) {
+      Value v;
+      v.name = "t" + std::to_string(temp++);
+      v.scalar = scalar;
+      return v;
+    };
+    auto define = [&](const Value &v, const std::string &expr) {
+      if (v.scalar) {
+        line(d, "const float " + v.name + " = " + expr + ";");
+      } else {
+        line(d, "float " + v.name + "[U][W];");
+        unroll();
+        line(d, "for (int u = 0; u < U; ++u)");
+        unroll();
+        line(d + 1, "for (int e = 0; e < W; ++e) " + v.name + "[u][e] = " + expr + ";");
+      }
+    };
+    // every operand is requested before the first use of any
+    for (const Op &op : seg_.ops)
+      if (op.code == OpCode::Push) {
+        const int k = pushSlot_[push++];
+        if (!have[k]) {
+          read[k] = emitRead(operands_[k], d);
+          have[k] = true;
+        }
+      }
+    push = 0;
+    for (const Op &op : seg_.ops) {
+      switch (op.code) {
+        case OpCode::Push:
+          stack.push_back(read[pushSlot_[push++]]);
+          break;
+        case OpCode::Const: {
+          Value v = fresh(true);
+          define(v, floatLiteral(op.constant));
+          stack.push_back(v);
+          break;
+        }
+        case OpCode::Dup:
+          stack.push_back(stack[stack.size() - 1 - op.depth]);
+          break;
+        case OpCode::Add: case OpCode::Sub: case OpCode::Mul: case OpCode::Div:
+        case OpCode::Max: case OpCode::Min: {
+          const Value b = stack.back();
+          stack.pop_back();
+          const Value a = stack.back();
+          stack.pop_back();
+          Value v = fresh(a.scalar && b.scalar);
+          std::string expr;
+          switch (op.code) {
+            case OpCode::Add: expr = a.at() + " + " + b.at(); break;
+            case OpCode::Sub: expr = a.at() + " - " + b.at(); break;
+            case OpCode::Mul: expr = a.at() + " * " + b.at(); break;
+            case OpCode::Div: expr = a.at() + " / " + b.at(); break;
+            case OpCode::Max: expr = "fmax_ieee(" + a.at() + ", " + b.at() + ")"; break;
+            default: expr = "fmin_ieee(" + a.at() + ", " + b.at() + ")"; break;
+          }
+          define(v, expr);
+          stack.push_back(v);
+          break;
+        }
+        case OpCode::Relu: case OpCode::Leaky: case OpCode::Neg: {
+          const Value a = stack.back();
+          stack.pop_back();
+          Value v = fresh(a.scalar);
+          if (op.code == OpCode::Relu) define(v, "fmax_ieee(" + a.at() + ", 0.f)");
+          else if (op.code == OpCode::Leaky)
+            define(v, "fmax_ieee(" + a.at() + ", " + a.at() + " * " + floatLiteral(op.constant) + ")");
+          else define(v, "-" + a.at());
+          stack.push_back(v);
+          break;
+        }
+        case OpCode::ReduceSum: case OpCode::Store: case OpCode::Matmul:
+          break;
+      }
+    }
+    return stack.back();
+  }
+
+  void emitPositionOfRow(int d) {
+    if (rank_ == 2) {
+      line(d, "const I x0 = row;");
+    } else if (rank_ == 3) {
+      line(d, "const I x0 = sizeof(I) == 4 ? (I)((unsigned)row / (unsigned)R.size[1]) : (I)(row / (I)R.size[1]);");
+      line(d, "const I x1 = row - x0 * (I)R.size[1];");
+    }
+  }
+
+  // j0 / nvalid / full of the U groups of a pass that starts at group `first`
+  // with `lanes` lanes on the row.
+  void emitGroups(int d, const std::string &first, const std::string &lanes) {
+    line(d, "I j0[U];");
+    line(d, "int nvalid[U];");
+    line(d, "bool full[U];");
+    unroll();
+    line(d, "for (int u = 0; u < U; ++u) {");
+    line(d + 1, "j0[u] = (" + first + " + (I)u * " + lanes + ") * W;");
+    line(d + 1, "const I left = n - j0[u];");
+    line(d + 1, "nvalid[u] = (A || left >= W) ? W : (left > 0 ? (int)left : 0);");
+    line(d + 1, "full[u] = A || nvalid[u] == W;");
+    line(d, "}");
+  }
+
+  void emitBody() {
+    const std::string otag = typeTag(p_.output().type);
+    os_ << "\n// ---- segment " << index_ << ": iteration rank " << rank_
+        << (reduce_ ? ", row sum over the innermost dim" : ", parallel") << "; a lane takes " << U_ << " groups of " << W_
+        << " elements per pass ----\n";
+    os_ << "// I: position type.  A: every 128-bit access is aligned and every pass is whole (no tail).\n";
+    os_ << "template <typename I, bool A>\nDEV void segment" << index_ << "(const SpecArgs &R) {\n";
+    line(1, "constexpr int W = " + std::to_string(W_) + ", U = " + std::to_string(U_) + ";");
+    line(1, "const int tid = (int)__builtin_amdgcn_workitem_id_x();");
+    line(1, "const I bid = (I)__builtin_amdgcn_workgroup_id_x();");
+    line(1, "const I n = (I)R.size[" + std::to_string(last_) + "];");
+    line(1, "const I groups = (n + (W - 1)) / W;");
+    if (rank_ == 1) line(1, "const I rows = 1;");
+    else if (rank_ == 2) line(1, "const I rows = (I)R.size[0];");
+    else line(1, "const I rows = (I)(R.size[0] * R.size[1]);");
+    for (const Operand &o : operands_)
+      if (o.step != Operand::Broadcast && o.gatherDim != last_)
+        line(1, "const bool vec" + id(o) + " = " + in(o) + ".vec != 0" + (o.gatherDim >= 0 ? " && " + in(o) + ".gvec != 0" : "") + ";");
+    if (reduce_) {
+      line(1, "const int lane = tid & 63;");
+      line(1, "const I wave = bid * 4 + (I)(tid >> 6);");
+      line(1, "const I nwaves = (I)R.grid * 4;");
+      line(1, "for (I row = wave; row < rows; row += nwaves) {");
+      emitPositionOfRow(2);
+      emitRowInvariants(2);
+      line(2, "float acc[U][W];");
+      unroll();
+      line(2, "for (int u = 0; u < U; ++u)");
+      unroll();
+      line(3, "for (int e = 0; e < W; ++e) acc[u][e] = 0.f;");
+      line(2, "for (I first = (I)lane; first < groups; first += 64 * U) {");
+      emitGroups(3, "first", "(I)64");
+      const Value v = emitExpression(3);
+      unroll();
+      line(3, "for (int u = 0; u < U; ++u)");
+      unroll();
+      line(4, "for (int e = 0; e < W; ++e) acc[u][e] += (e < nvalid[u]) ? " + v.at() + " : 0.f;");
+      line(2, "}");
+      line(2, "// fixed-order combination: groups, then element slots pairwise, then the wavefront");
+      unroll();
+      line(2, "for (int w = U / 2; w >= 1; w >>= 1)");
+      unroll();
+      line(3, "for (int u = 0; u < w; ++u)");
+      unroll();
+      line(4, "for (int e = 0; e < W; ++e) acc[u][e] = acc[2 * u][e] + acc[2 * u + 1][e];");
+      unroll();
+      line(2, "for (int w = W / 2; w >= 1; w >>= 1)");
+      unroll();
+      line(3, "for (int e = 0; e < w; ++e) acc[0][e] = acc[0][2 * e] + acc[0][2 * e + 1];");
+      line(2, "const float s = wave_sum(acc[0][0]);");
+      line(2, "if (lane == 0) st_" + otag + "(R.out, (long long)row, s);");
+      line(1, "}");
+      os_ << "}\n";
+      return;
+    }
+    line(1, "const I lanes = (I)1 << R.lanes_log2;");
+    line(1, "const I rows_per_pass = (I)(256 >> R.lanes_log2);");
+    line(1, "const I local_row = (I)(tid >> R.lanes_log2);");
+    line(1, "const I first_group = (I)tid & (lanes - 1);");
+    line(1, "for (I row0 = bid * rows_per_pass; row0 < rows; row0 += (I)R.grid * rows_per_pass) {");
+    line(2, "const I row = row0 + local_row;");
+    line(2, "if (row >= rows) continue;");
+    emitPositionOfRow(2);
+    emitRowInvariants(2);
+    line(2, "for (I first = first_group; first < groups; first += lanes * U) {");
+    emitGroups(3, "first", "lanes");
+    const Value v = emitExpression(3);
+    std::string res = v.name;
+    if (v.scalar) {
+      line(3, "float splat[U][W];");
+      unroll();
+      line(3, "for (int u = 0; u < U; ++u)");
+      unroll();
+      line(4, "for (int e = 0; e < W; ++e) splat[u][e] = " + v.name + ";");
+      res = "splat";
+    }
+    unroll();
+    line(3, "for (int u = 0; u < U; ++u) {");
+    line(4, "const long long o = (long long)row * (long long)n + (long long)j0[u];");
+    line(4, "if (A || (full[u] && R.out_vec)) {");
+    line(5, "stv_" + otag + "<W>(R.out, o, " + res + "[u]);");
+    line(4, "} else {");
+    unroll();
+    line(5, "for (int e = 0; e < W; ++e)");
+    line(6, "if (e < nvalid[u]) st_" + otag + "(R.out, o + e, " + res + "[u][e]);");
+    line(4, "}");
+    line(3, "}");
+    line(2, "}");
+    line(1, "}");
+    os_ << "}\n";
+  }
+
+  void emitWrappers() {
+    for (int i32 = 1; i32 >= 0; --i32)
+      for (int a = 1; a >= 0; --a)
+        os_ << "KERNEL void " << specKernelName(index_, i32 != 0, a != 0) << "(const SpecArgs R) { segment" << index_
+            << "<" << (i32 ? "int" : "long long") << ", " << (a ? "true" : "false") << ">(R); }\n";
+  }
+
+  const Program &p_;
+  const Segment &seg_;
+  int index_;
+  std::ostringstream &os_;
+  int rank_ = 0, last_ = 0, W_ = 8, U_ = 2;
+  bool reduce_ = false;
+  std::vector<Operand> operands_;
+  std::vector<int> pushSlot_;   // per push, in order: index into operands_
+};
+
+}  // namespace
+
+SpecShape specShape(const Program &p, int segment) {
+  const Segment &g = p.segments[segment];
+  bool any16 = p.output().type != ElemType::F32, any32 = p.output().type == ElemType::F32;
+  for (const Op &op : g.ops)
+    if (op.code == OpCode::Push) (p.args[op.arg].type == ElemType::F32 ? any32 : any16) = true;
+  SpecShape s;
+  s.width = any16 ? 8 : 4;            // 16 bytes of the narrowest tensor
+  s.unroll = (any16 && any32) ? 2 : 4;
+  return s;
+}
+
+uint64_t programHash(const Program &p) {
+  uint64_t h = 0xcbf29ce484222325ull;
+  for (unsigned char c : serialize(p)) {
+    h ^= c;
+    h *= 0x100000001b3ull;
+  }
+  return h;
+}
+
+std::string specKernelName(int segment, bool idx32, bool aligned) {
+  return "afir_region_s" + std::to_string(segment) + (idx32 ? "_i32" : "_i64") + (aligned ? "_a" : "_g");
+}
+
+std::string emitHipSource(const Program &p, const std::string &title, std::string *source) {
+  if (std::string why = validate(p); !why.empty()) return why;
+  std::ostringstream os;
+  os << "// HIP kernels for the fused region '" << title << "' (gfx950), generated from this program:\n";
+  {
+    std::istringstream lines(serialize(p));
+    for (std::string line; std::getline(lines, line);) os << "//   " << line << "\n";
+  }
+  os << "// Build: hipcc --genco --offload-arch=gfx950 -O3 -nogpuinc -ffp-contract=off \\\n"
+        "//          -Xclang -target-feature -Xclang -packed-fp32-ops -o region.hsaco region.hip\n";
+  os << kPrelude;
+  os << "static_assert(sizeof(SpecInput) == " << sizeof(SpecInput) << " && sizeof(SpecArgs) == " << sizeof(SpecArgs)
+     << " && __builtin_offsetof(SpecArgs, in) == " << offsetof(SpecArgs, in)
+     << " && __builtin_offsetof(SpecInput, vec) == " << offsetof(SpecInput, vec)
+     << ", \"launch argument layout differs from the kernel library's\");\n";
+  char hash[32];
+  std::snprintf(hash, sizeof hash, "0x%016llxull", (unsigned long long)programHash(p));
+  os << "extern \"C\" __attribute__((device)) __attribute__((used)) const unsigned long long afir_region_program_hash = " << hash << ";\n";
+  for (int s = 0; s < (int)p.segments.size(); ++s) {
+    SegmentEmitter e(p, s, os);
+    if (std::string why = e.run(); !why.empty()) return why;
+  }
+  *source = os.str();
+  return "";
+}
+
+std::string hipccCommandLine(const std::string &sourcePath, const std::string &outputPath) {
+  return "hipcc --genco --offload-arch=gfx950 -O3 -nogpuinc -ffp-contract=off -Xclang -target-feature -Xclang "
+         "-packed-fp32-ops -o " + outputPath + " " + sourcePath;
+}
+
+}  // namespace afir_target

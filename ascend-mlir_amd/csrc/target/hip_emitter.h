@@ -1,0 +1,76 @@
+// Fused-region program -> HIP source of a kernel specialised for it: what the
+// reference's emitter does for AscendC (lib/Target/CannKernel/CannTranslation.cpp:2487-2694
+// prints one C++ kernel per fused region; the compute bodies come from
+// lib/Conversion/LinalgToAscendC/ComputeConversion.cpp:1290-1640 for parallel
+// generics, :246-750 for reductions, :828-1272 for the fused gather loop).
+//
+// The emitted source needs no headers (it uses compiler builtins only), so
+// compiling it to a code object takes a fraction of a second:
+//   hipcc --genco --offload-arch=gfx950 -O3 -nogpuinc -ffp-contract=off
+//         -Xclang -target-feature -Xclang -packed-fp32-ops -o region.hsaco region.hip
+// The code object is attached to the registered program
+// (afir_hip_region_attach_code_object) and launched in place of the generic
+// interpreter kernel; results are bit-identical to it.
+//
+// What is fixed at emission: the iteration rank, the operation sequence, the
+// element types, which operands are broadcast / contiguous / strided / gathered
+// along the innermost dim.  What stays a launch argument: pointers, extents,
+// strides, offsets, alignment of this particular launch.
+#pragma once
+
+#include <cstdint>
+#include <string>
+
+#include "region_program.h"
+
+namespace afir_target {
+
+// Launch argument of every emitted kernel.  The emitted source carries the same
+// declaration and static_asserts its size and field offsets against this one.
+struct SpecInput {
+  const void *base;    // device pointer of the tensor
+  const void *index;   // device pointer of the index tensor (gather), else null
+  long long stride[3]; // elements per step of each iteration dim
+  long long offset;    // constant element offset
+  long long gstride;   // elements per index step
+  long long gextent;   // valid indices are [0, gextent)
+  int vec;             // 128-bit loads along the innermost dim are aligned
+  int gvec;            // ... also after adding any multiple of gstride
+};
+constexpr int kSpecMaxInputs = 8;
+struct SpecArgs {
+  long long size[3];
+  void *out;
+  int *error_flag;     // set to 1 when a gathered index is out of range (may be null)
+  int out_vec;         // 128-bit stores are aligned for every full vector
+  int lanes_log2;      // parallel segments: lanes of the workgroup that share a row
+  int grid;            // number of workgroups launched
+  int pad;
+  SpecInput in[kSpecMaxInputs];
+};
+
+// A lane's share of one pass over a row: `unroll` groups of `width` consecutive
+// elements (16 bytes of the narrowest tensor), the groups one lane-set apart.
+struct SpecShape {
+  int width = 8;
+  int unroll = 2;
+};
+SpecShape specShape(const afir_region::Program &p, int segment);
+
+// FNV-1a of the serialized program: the emitted code object exports it as
+// `afir_region_program_hash`, checked when the code object is attached.
+uint64_t programHash(const afir_region::Program &p);
+
+// Kernel symbol of a segment: idx32 = positions fit 32 bits, aligned = every
+// vector access of the launch is 16-byte aligned and rows are whole vectors.
+std::string specKernelName(int segment, bool idx32, bool aligned);
+
+// Emits the source for every segment.  Returns "" on success, else why the
+// program has no specialised form (matmul segments: those run on the
+// hand-written kernels).
+std::string emitHipSource(const afir_region::Program &p, const std::string &title, std::string *source);
+
+// The compiler invocation for a source file (argv, no shell).
+std::string hipccCommandLine(const std::string &sourcePath, const std::string &outputPath);
+
+}  // namespace afir_target

@@ -6,6 +6,12 @@
 // that `runtime-session --kernel` stores in the artifact.
 //
 //   afir-translate -mlir-to-hip input.mlir [-o program.txt] [--tiling-space-out tiling_space.json]
+//                  [--emit-hip-source]
+//
+// --emit-hip-source prints, instead of the program, the HIP source of the
+// kernels specialised for it (what `runtime-session --kernel` compiles into the
+// artifact's code object); an input that starts with "afir-hip-region" is taken
+// as a program rather than MLIR.
 //
 // Exit codes: 0 ok, 1 the input cannot be lowered (diagnostic on stderr),
 // 2 usage / file errors.
@@ -16,11 +22,12 @@
 #include <iterator>
 #include <string>
 
+#include "../target/hip_emitter.h"
 #include "../target/mlir_translate.h"
 
 int main(int argc, char **argv) {
   std::string input, output, tilingOut;
-  bool toHip = false;
+  bool toHip = false, emitSource = false;
   for (int i = 1; i < argc; ++i) {
     const std::string a = argv[i];
     auto value = [&](const char *flag) -> const char * {
@@ -31,6 +38,8 @@ int main(int argc, char **argv) {
     };
     if (a == "-mlir-to-hip" || a == "--mlir-to-hip") {
       toHip = true;
+    } else if (a == "--emit-hip-source") {
+      emitSource = true;
     } else if (a == "-mlir-to-cann" || a == "--mlir-to-cann") {
       std::fprintf(stderr, "afir-translate: this build emits for gfx950 only; use -mlir-to-hip\n");
       return 2;
@@ -43,7 +52,7 @@ int main(int argc, char **argv) {
       if (!v) { std::fprintf(stderr, "afir-translate: --tiling-space-out needs a file name\n"); return 2; }
       tilingOut = v;
     } else if (a == "-h" || a == "--help") {
-      std::printf("usage: afir-translate -mlir-to-hip <input.mlir> [-o <file>] [--tiling-space-out <file>]\n");
+      std::printf("usage: afir-translate -mlir-to-hip <input.mlir> [-o <file>] [--tiling-space-out <file>] [--emit-hip-source]\n");
       return 0;
     } else if (!a.empty() && a[0] == '-' && a != "-") {
       std::fprintf(stderr, "afir-translate: unknown option %s\n", a.c_str());
@@ -68,12 +77,33 @@ int main(int argc, char **argv) {
     text.assign(std::istreambuf_iterator<char>(f), std::istreambuf_iterator<char>());
   }
   afir_target::Translation tr;
-  const std::string why = afir_target::translateMlirToRegion(text, &tr);
+  std::string why;
+  {
+    size_t at = 0;
+    while (at < text.size() && (text[at] == '#' || isspace((unsigned char)text[at]))) {
+      if (text[at] == '#') while (at < text.size() && text[at] != '\n') ++at;
+      else ++at;
+    }
+    if (text.compare(at, 15, "afir-hip-region") == 0) {
+      tr.functionName = "region";
+      why = afir_region::parse(text, &tr.program);
+      if (why.empty()) why = afir_region::validate(tr.program);
+    } else {
+      why = afir_target::translateMlirToRegion(text, &tr);
+    }
+  }
   if (!why.empty()) {
     std::fprintf(stderr, "%s: error: %s\n", input.empty() ? "<stdin>" : input.c_str(), why.c_str());
     return 1;
   }
-  const std::string program = "# kernel " + tr.functionName + "\n" + afir_region::serialize(tr.program);
+  std::string program = "# kernel " + tr.functionName + "\n" + afir_region::serialize(tr.program);
+  if (emitSource) {
+    const std::string no = afir_target::emitHipSource(tr.program, tr.functionName, &program);
+    if (!no.empty()) {
+      std::fprintf(stderr, "%s: error: no specialised kernel: %s\n", input.empty() ? "<stdin>" : input.c_str(), no.c_str());
+      return 1;
+    }
+  }
   if (output.empty() || output == "-") {
     std::fputs(program.c_str(), stdout);
   } else {

@@ -263,6 +263,7 @@ int main(int argc, char **argv) {
   launch.sharedLibraryPath = artifact.sharedLibraryPath;
   launch.symbolName = artifact.sharedLibrarySymbol;
   launch.regionProgram = artifact.regionProgram;
+  launch.codeObjectPath = artifact.codeObjectPath;
 
   struct Best {
     bool found = false;

@@ -13,6 +13,8 @@ import struct
 
 from . import KERNELS_LIB
 
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
 
 class AfirHipError(RuntimeError):
     pass
@@ -44,6 +46,8 @@ EXPORTED_SYMBOLS = [
     "afir_hip_region_info",
     "afir_hip_region_tiling_field",
     "afir_hip_region_kernel",
+    "afir_hip_region_emit_source",
+    "afir_hip_region_attach_code_object",
     "afir_hip_region_argument_bytes",
     "afir_hip_launch_region",
 ]
@@ -288,6 +292,45 @@ def _torch_type(name):
     return _TORCH_TYPES[name]
 
 
+HIPCC_REGION_FLAGS = ["--genco", "--offload-arch=gfx950", "-O3", "-nogpuinc", "-ffp-contract=off",
+                      "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def compile_region_source(source: str, cache_dir: str = None) -> bytes:
+    """HIP source of a region (Region.emit_source, afir-translate
+    --emit-hip-source) -> code object bytes.  Raises AfirHipError when hipcc is
+    missing or rejects the source."""
+    import hashlib
+    import shutil
+    import subprocess
+    import tempfile
+    cache_dir = cache_dir or os.path.join(_HERE, "lib", "region_cache")
+    key = hashlib.sha256(("\n".join(HIPCC_REGION_FLAGS) + "\n" + source).encode()).hexdigest()[:24]
+    path = os.path.join(cache_dir, key + ".hsaco")
+    if os.path.exists(path):
+        with open(path, "rb") as f:
+            return f.read()
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        raise AfirHipError("hipcc not found: cannot compile a region kernel")
+    os.makedirs(cache_dir, exist_ok=True)
+    with tempfile.TemporaryDirectory() as tmp:
+        src = os.path.join(tmp, "region.hip")
+        obj = os.path.join(tmp, "region.hsaco")
+        with open(src, "w") as f:
+            f.write(source)
+        p = subprocess.run([hipcc, *HIPCC_REGION_FLAGS, "-o", obj, src], capture_output=True, text=True)
+        if p.returncode != 0:
+            raise AfirHipError("hipcc rejected the region source:\n" + p.stderr[-2000:])
+        with open(obj, "rb") as f:
+            image = f.read()
+    tmp_path = path + f".{os.getpid()}.tmp"
+    with open(tmp_path, "wb") as f:
+        f.write(image)
+    os.replace(tmp_path, path)
+    return image
+
+
 class Region:
     """A registered fused-region program (afir_hip_region_register)."""
 
@@ -319,6 +362,34 @@ class Region:
         L.afir_hip_region_kernel.argtypes = [u64]
         self.kernel = L.afir_hip_region_kernel(u64(self.handle)).decode()
         self.arg_types = [l.split()[2] for l in text.splitlines() if l.split()[:1] == ["arg"]]
+
+    # ---- kernels compiled for this program ----
+
+    def emit_source(self) -> str:
+        """HIP source of the kernels specialised for this program."""
+        L = load()
+        L.afir_hip_region_emit_source.argtypes = [ctypes.c_uint64, ctypes.c_char_p, ctypes.c_size_t,
+                                                  ctypes.POINTER(ctypes.c_size_t)]
+        n = ctypes.c_size_t(0)
+        _check(L.afir_hip_region_emit_source(ctypes.c_uint64(self.handle), None, 0, ctypes.byref(n)))
+        buf = ctypes.create_string_buffer(n.value + 1)
+        _check(L.afir_hip_region_emit_source(ctypes.c_uint64(self.handle), buf, n.value + 1, ctypes.byref(n)))
+        return buf.value.decode()
+
+    def attach_code_object(self, image: bytes):
+        L = load()
+        L.afir_hip_region_attach_code_object.argtypes = [ctypes.c_uint64, ctypes.c_char_p, ctypes.c_size_t]
+        _check(L.afir_hip_region_attach_code_object(ctypes.c_uint64(self.handle), image, len(image)))
+        L.afir_hip_region_kernel.restype = ctypes.c_char_p
+        self.kernel = L.afir_hip_region_kernel(ctypes.c_uint64(self.handle)).decode()
+
+    def compile(self, cache_dir: str = None):
+        """Emit, compile with hipcc and attach; the code object is kept in
+        `cache_dir` (default: lib/region_cache beside the libraries) under the
+        hash of its source, so a program is compiled once."""
+        source = self.emit_source()
+        self.attach_code_object(compile_region_source(source, cache_dir))
+        return self
 
     def close(self):
         if self.handle:

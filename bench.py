@@ -39,7 +39,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # (two runs), scaled by the same counters' reading for a plain 256 MiB copy
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Source: profiles/*.txt, section (2).
 MEASURED_TRAFFIC = {"c1": 201364070, "c2": 134645390, "c3": 134496358, "c4": 134578995,
-                    "c5": 1862780928, "g1": 201559961, "g2": 134977945}
+                    "c5": 1862780928, "i1": 201559961, "i2": 134977945}
 
 
 # Region programs of the two generic-kernel workloads (grammar:
@@ -333,18 +333,22 @@ def make_workload(key, torch, H, O, C):
                 w.work() * 20 / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
             return ev
         w.power_evidence = power_evidence
-    elif key in ("g1", "g2"):
-        # The generic region kernel (any fused chain) next to the hand-tuned
-        # ones: g1 = the c1 chain kept off its fast path, g2 = the reference's
-        # split / relu / broadcast-add / broadcast-mul / concat graph
-        # (examples/split-relu-brc-add-mul) at [8192, 4096] f16.
+    elif key in ("g1", "g2", "i1", "i2"):
+        # Region programs (any fused chain) next to the hand-tuned kernels:
+        # g1 / i1 = the c1 chain kept off its fast path, g2 / i2 = the
+        # reference's split / relu / broadcast-add / broadcast-mul / concat
+        # graph (examples/split-relu-brc-add-mul) at [8192, 4096] f16.
+        # g: kernels emitted and compiled for the program; i: the interpreter
+        # kernel of the library.
         from oracle import region_oracle as RO
+        compiled = key[0] == "g"
+        how = "compiled region kernel" if compiled else "region interpreter kernel"
         os.environ["AFIR_HIP_REGION_GENERIC"] = "1"
-        if key == "g1":
+        if key[1] == "1":
             text = REGION_ADD_MUL
             a, b = O.gen_c1()
             inputs, out_shape, out_dt = [a, b], (4096, 4096), torch.float32
-            w.title = "g1 generic region kernel: (a+b)*b f32 [4096,4096] as a region program"
+            w.title = f"{key} {how}: (a+b)*b f32 [4096,4096] as a region program"
             w.dtype = "f32"
             work = O.algorithmic_bytes("c1", m=4096, n=4096)
         else:
@@ -354,19 +358,22 @@ def make_workload(key, torch, H, O, C):
             f16 = lambda shape: rng.uniform(-1, 1, shape).astype(np.float32).astype(np.float16)
             inputs = [f16((m, n)), f16((m // 2,)), f16((m // 2,)), f16((n,)), f16((n,))]
             out_shape, out_dt = (m, n), torch.float16
-            w.title = ("g2 generic region kernel: split/relu/bcast-add/bcast-mul/concat f16 [8192,4096] "
+            w.title = (f"{key} {how}: split/relu/bcast-add/bcast-mul/concat f16 [8192,4096] "
                        "(two segments)")
             w.dtype = "f16"
             work = 2 * m * n * 2 + 2 * (m // 2) * 2 + 2 * n * 2
         region = H.Region(text)
         del os.environ["AFIR_HIP_REGION_GENERIC"]
         assert region.kernel == "fused_region"
+        if compiled:
+            region.compile()     # from lib/region_cache when build() left it there
+            assert region.kernel == "fused_region_compiled"
         w.work = lambda: work
-        w.nsets = 3 if key == "g1" else 4
+        w.nsets = 3 if key[1] == "1" else 4
         dev0 = [_dev(torch, x) for x in inputs]
         sets = []
         for i in range(w.nsets):
-            ins = dev0 if i == 0 else [dev0[0].clone()] + ([dev0[1].clone()] if key == "g1" else dev0[1:])
+            ins = dev0 if i == 0 else [dev0[0].clone()] + ([dev0[1].clone()] if key[1] == "1" else dev0[1:])
             sets.append((ins, torch.empty(out_shape, dtype=out_dt, device="cuda")))
         w.sets = sets
         dims = [d for x in inputs for d in x.shape] + list(out_shape)
@@ -378,8 +385,8 @@ def make_workload(key, torch, H, O, C):
             want = RO.evaluate(text, inputs)
             got = sets[0][1].cpu().numpy()
             return {"bar": "bit-exact vs the region oracle", "passed": got.tobytes() == want.tobytes(),
-                    "mismatches": int((got.view(np.uint16 if key == "g2" else np.uint32) !=
-                                       want.view(np.uint16 if key == "g2" else np.uint32)).sum())}
+                    "mismatches": int((got.view(np.uint16 if key[1] == "2" else np.uint32) !=
+                                       want.view(np.uint16 if key[1] == "2" else np.uint32)).sum())}
         w.parity = parity
 
         def cpu(budget_s):
@@ -433,7 +440,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "g1", "g2"])
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "g1", "g2", "i1", "i2"])
     ap.add_argument("--all", dest="all", action="store_true", default=True)
     ap.add_argument("--no-all", dest="all", action="store_false")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -468,7 +475,7 @@ def main():
             return args.warmup
         return 5 if key == "c5" else 30
 
-    order = [args.workload] + ([k for k in ["c1", "c2", "c3", "c4", "c5", "g1", "g2"]
+    order = [args.workload] + ([k for k in ["c1", "c2", "c3", "c4", "c5", "g1", "g2", "i1", "i2"]
                                 if k != args.workload] if args.all else [])
     results = []
     for key in order:

@@ -180,6 +180,23 @@ uint32_t afir_hip_region_info(uint64_t handle, int *num_inputs, int *num_outputs
  * AFIR_HIP_REGION_GENERIC=1 before registering keeps every non-matmul program
  * on the generic kernel. */
 const char *afir_hip_region_kernel(uint64_t handle);
+/* Kernels compiled for one program, the counterpart of the reference's
+ * generated kernel source and device binary
+ * (lib/Target/CannKernel/CannTranslation.cpp:2487-2694 prints the source,
+ * lib/Runtime/Execution/NativeExecutionRunner.cpp:332-369 registers the
+ * binary).  emit_source writes the HIP source for the program (NUL-terminated,
+ * truncated to `capacity`; *length = full length, so call with a null buffer
+ * first).  It is compiled with
+ *   hipcc --genco --offload-arch=gfx950 -O3 -nogpuinc -ffp-contract=off
+ *         -Xclang -target-feature -Xclang -packed-fp32-ops -o region.hsaco region.hip
+ * and the resulting file's bytes are handed to attach_code_object; the launches
+ * of that handle then run the compiled kernels ("fused_region_compiled")
+ * instead of the interpreter, with bit-identical results.  The image is checked
+ * against the program when it is first launched (AFIR_HIP_E_LAUNCH if it was
+ * built from another program).  Programs routed to a hand-tuned family keep
+ * that kernel.  Matmul programs have no source form (AFIR_HIP_E_INVALID). */
+uint32_t afir_hip_region_emit_source(uint64_t handle, char *buffer, size_t capacity, size_t *length);
+uint32_t afir_hip_region_attach_code_object(uint64_t handle, const void *image, size_t image_len);
 /* Name of tiling field `index` ("" if out of range); valid until unregister. */
 const char *afir_hip_region_tiling_field(uint64_t handle, int index);
 uint32_t afir_hip_region_argument_bytes(uint64_t handle, const void *tiling, size_t tiling_len,

@@ -58,6 +58,10 @@ def test_example_pipeline(tmp_path, example):
     p = _rs("--kernel", str(src), "--kernel-kind", kind, "--output", str(art), "--name", "kernel0")
     assert p.returncode == 0, p.stderr
     assert f"kernel_kind={kind}" in (art / "out" / "manifest.txt").read_text().splitlines()
+    if kind != "mix":
+        # the region was also emitted as HIP source and compiled for gfx950
+        assert "code_object_path=kernel0.hsaco" in (art / "out" / "manifest.txt").read_text().splitlines()
+        assert (art / "kernel0.hip").stat().st_size > 0 and (art / "kernel0.hsaco").stat().st_size > 0
     ts = tmp_path / "tiling_space.json"
     assert subprocess.run([TR, "-mlir-to-hip", str(src), "-o", str(tmp_path / "program.txt"),
                            "--tiling-space-out", str(ts)]).returncode == 0
@@ -89,6 +93,20 @@ def test_example_pipeline(tmp_path, example):
     else:   # float32 row sums in another order, rounded to f16: within one f16 ulp
         assert np.all(np.abs(got.astype(np.float64) - want.astype(np.float64))
                       <= 2.0 ** -10 * np.abs(want.astype(np.float64)) + 1e-3)
+    if kind != "mix":
+        # the same artifact on the interpreter kernel instead of its code object
+        manifest["outputs"][0]["path"] = str(tmp_path / "output_interpreted.npy")
+        (tmp_path / "run_manifest2.json").write_text(json.dumps(manifest))
+        p = subprocess.run([RS, "--run-manifest", str(tmp_path / "run_manifest2.json"), "--run"],
+                           capture_output=True, text=True, timeout=100,
+                           env=dict(os.environ, AFIR_HIP_REGION_INTERPRET="1"))
+        assert p.returncode == 0, p.stdout + p.stderr
+        other = np.load(tmp_path / "output_interpreted.npy")
+        if exact:
+            assert other.tobytes() == got.tobytes()
+        else:
+            assert np.all(np.abs(other.astype(np.float64) - got.astype(np.float64))
+                          <= 2.0 ** -9 * np.abs(want.astype(np.float64)) + 2e-3)
 
 
 def test_capi_runs_a_compiled_mlir_kernel(pkg, tmp_path):

@@ -17,9 +17,9 @@ TR = os.path.join(ROOT, "ascend-mlir_amd", "bin", "afir-translate")
 CASES = list(GC.cases())
 
 
-@pytest.mark.parametrize("generic", ["routed", "generic"])
+@pytest.mark.parametrize("generic", ["routed", "generic", "compiled"])
 @pytest.mark.parametrize("case", CASES, ids=[c[0] for c in CASES])
-def test_kernel_reproduces_the_reference_output(pkg, monkeypatch, case, generic):
+def test_kernel_reproduces_the_reference_output(pkg, monkeypatch, tmp_path_factory, case, generic):
     import torch
     from ascend_mlir_amd import hip_kernels as H
     H.load()
@@ -28,8 +28,11 @@ def test_kernel_reproduces_the_reference_output(pkg, monkeypatch, case, generic)
         p = subprocess.run([TR, "-mlir-to-hip", "-"], input=mlir, capture_output=True, text=True)
         assert p.returncode == 0, p.stderr
         program = p.stdout
-    monkeypatch.setenv("AFIR_HIP_REGION_GENERIC", "1" if generic == "generic" else "0")
+    monkeypatch.setenv("AFIR_HIP_REGION_GENERIC", "0" if generic == "routed" else "1")
     r = H.Region(program)
+    if generic == "compiled" and "matmul" not in program:
+        r.compile(cache_dir=str(tmp_path_factory.mktemp("region_cache")))
+        assert r.kernel == "fused_region_compiled"
     dev = [torch.from_numpy(x).cuda() for x in inputs]
     got = r(*dev, out_shape=want.shape).cpu().numpy()
     r.close()

@@ -1,6 +1,8 @@
-"""The generic fused-region kernel against the region oracle: the reference's
-example graphs at their own shapes, the benchmark configurations as programs,
-ragged / unaligned shapes, and seeded random op chains.  Needs a GPU."""
+"""Fused-region programs against the region oracle, on the interpreter kernel
+(chain and stack evaluators) and on kernels compiled for each program: the
+reference's example graphs at their own shapes, the benchmark configurations as
+programs, ragged / unaligned shapes, and seeded random op chains.  Needs a GPU
+(and hipcc for the compiled mode)."""
 import numpy as np
 import pytest
 
@@ -34,18 +36,34 @@ def _host(t, ty):
     return t.cpu().numpy()
 
 
-@pytest.fixture(params=["chain", "stack"], autouse=True)
-def evaluator(request, monkeypatch):
-    """Every test runs twice: expressions that are chains on the linear form,
-    and everything on the stack interpreter."""
+MODE = {"compiled": False, "cache": None}
+
+
+@pytest.fixture(params=["chain", "stack", "compiled"], autouse=True)
+def evaluator(request, monkeypatch, tmp_path_factory):
+    """Every test runs three times: expressions that are chains on the linear
+    form of the interpreter, everything on its stack form, and everything on
+    kernels emitted and compiled for the program."""
     monkeypatch.setenv("AFIR_HIP_REGION_GENERIC", "1")
     if request.param == "stack":
         monkeypatch.setenv("AFIR_HIP_REGION_STACK", "1")
-    return request.param
+    MODE["compiled"] = request.param == "compiled"
+    if MODE["cache"] is None:
+        MODE["cache"] = str(tmp_path_factory.mktemp("region_cache"))
+    yield request.param
+    MODE["compiled"] = False
+
+
+def region(H, text):
+    r = H.Region(text)
+    if MODE["compiled"]:
+        r.compile(cache_dir=MODE["cache"])
+        assert r.kernel == "fused_region_compiled"
+    return r
 
 
 def run(H, text, inputs, out_shape, workspace=None, block_dim=0):
-    r = H.Region(text)
+    r = region(H, text)
     dev = [_dev(x, r.arg_types[i]) for i, x in enumerate(inputs)]
     out = r(*dev, out_shape=out_shape, workspace=workspace, block_dim=block_dim)
     res = _host(out, r.arg_types[-1])
@@ -91,7 +109,7 @@ def test_unaligned_bases_take_the_element_path(H):
     text = RC.HEADER + ("arg in f16 2\narg in f16 1\narg out f16 2\nsegment 2\n size arg0.0 arg0.1\n"
                         " outoff 0\n push arg0 d0 d1\n push arg1 d1\n mul\n store\nend\n")
     want = RO.evaluate(text, [a, c])
-    r = H.Region(text)
+    r = region(H, text)
     # same data at odd element offsets: neither operand is 16-byte aligned
     abuf = torch.zeros(a.size + 8, dtype=torch.float16, device="cuda")
     cbuf = torch.zeros(c.size + 8, dtype=torch.float16, device="cuda")
@@ -210,3 +228,20 @@ def test_every_operation_pair_at_every_vector_position(H):
                     got = run(H, text, [a, b], a.shape)
                     same = (got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))
                     assert same.all(), (text, np.argwhere(~same))
+
+
+def test_code_object_of_another_program_is_rejected(H, evaluator, tmp_path):
+    """A code object carries the hash of the program it was emitted from; the
+    first launch checks it and runs nothing when it does not match."""
+    import torch
+    if evaluator != "compiled":
+        pytest.skip("one run is enough")
+    other = H.Region(RC.RELU_COL_ADD)
+    image = H.compile_region_source(other.emit_source(), str(tmp_path))
+    other.close()
+    r = H.Region(RC.C1_ADD_MUL)
+    r.attach_code_object(image)
+    a = torch.ones(4, 8, device="cuda")
+    with pytest.raises(H.AfirHipError, match="not built from this program"):
+        r(a, a, out_shape=(4, 8))
+    r.close()

@@ -1,0 +1,143 @@
+"""Region program -> HIP source -> gfx950 code object, without a GPU: the
+emitter accepts every program the translator produces, the source carries the
+program and its hash, hipcc accepts it, and the artifact layer stores it
+(reference counterpart: the kernel source `afir-translate -mlir-to-cann` prints,
+lib/Target/CannKernel/CannTranslation.cpp:2487-2694, compiled by
+lib/Runtime/Compilation/KernelCompiler.cpp into the artifact's device binary)."""
+import ctypes
+import os
+import shutil
+import subprocess
+
+import pytest
+
+from tests import mlir_cases as MC
+from tests import region_cases as RC
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "ascend-mlir_amd", "bin")
+TR = os.path.join(BIN, "afir-translate")
+RS = os.path.join(BIN, "runtime-session")
+HIPCC = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+FLAGS = ["--genco", "--offload-arch=gfx950", "-O3", "-nogpuinc", "-ffp-contract=off",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+PROGRAMS = {n: getattr(RC, n) for n in dir(RC)
+            if n.isupper() and isinstance(getattr(RC, n), str) and "segment" in getattr(RC, n)}
+
+
+def _emit(text):
+    return subprocess.run([TR, "-mlir-to-hip", "-", "--emit-hip-source"], input=text, capture_output=True, text=True)
+
+
+def _fnv1a(data: bytes) -> int:
+    h = 0xcbf29ce484222325
+    for c in data:
+        h = ((h ^ c) * 0x100000001b3) & 0xFFFFFFFFFFFFFFFF
+    return h
+
+
+@pytest.mark.parametrize("name", sorted(PROGRAMS))
+def test_every_program_emits_and_compiles(tmp_path, name):
+    p = _emit(PROGRAMS[name])
+    assert p.returncode == 0, p.stderr
+    src = p.stdout
+    # the program it was generated from, line by line, and its hash
+    canonical = subprocess.run([TR, "-mlir-to-hip", "-"], input=PROGRAMS[name], capture_output=True, text=True).stdout
+    body = "".join(l + "\n" for l in canonical.splitlines() if not l.startswith("#"))
+    for line in body.splitlines():
+        assert "//   " + line in src
+    assert "afir_region_program_hash = 0x%016xull" % _fnv1a(body.encode()) in src
+    nseg = body.count("\nsegment ")
+    for k in range(nseg):
+        for variant in ("i32_a", "i32_g", "i64_a", "i64_g"):
+            assert f"afir_region_s{k}_{variant}(" in src
+    assert "#include" not in src            # builtins only: compiles with -nogpuinc
+    (tmp_path / "k.hip").write_text(src)
+    q = subprocess.run([HIPCC, *FLAGS, "-o", str(tmp_path / "k.hsaco"), str(tmp_path / "k.hip")],
+                       capture_output=True, text=True)
+    assert q.returncode == 0, q.stderr[-3000:]
+    image = (tmp_path / "k.hsaco").read_bytes()
+    assert b"afir_region_s0_i32_a" in image and b"afir_region_program_hash" in image
+
+
+def test_lane_shapes_follow_the_element_types():
+    assert "a lane takes 4 groups of 4 elements per pass" in _emit(RC.C1_ADD_MUL).stdout       # all f32
+    assert "a lane takes 4 groups of 8 elements per pass" in _emit(RC.RELU_COL_ADD).stdout     # all f16
+    mixed = RC.HEADER + ("arg in f16 2\narg in f32 1\narg out f16 2\nsegment 2\n size arg0.0 arg0.1\n outoff 0\n"
+                         " push arg0 d0 d1\n push arg1 d1\n add\n store\nend\n")
+    assert "a lane takes 2 groups of 8 elements per pass" in _emit(mixed).stdout
+
+
+def test_identical_reads_are_loaded_once():
+    src = _emit(RC.C1_ADD_MUL).stdout           # (a + b) * b reads b twice
+    assert src.count("ldv_f32<W, true>(R.in[1].base") == 1 and "R.in[2]" not in src
+
+
+def test_matmul_programs_have_no_source_form():
+    prog = subprocess.run([TR, "-mlir-to-hip", "-"], input=MC.MATMUL_BIAS_LEAKY_BF16, capture_output=True, text=True)
+    assert prog.returncode == 0
+    p = _emit(prog.stdout)
+    assert p.returncode == 1 and "hand-written MFMA kernels" in p.stderr
+    # MLIR input works as well as a program
+    p = subprocess.run([TR, "-mlir-to-hip", "-", "--emit-hip-source"], input=MC.SPLIT_HALVES,
+                       capture_output=True, text=True)
+    assert p.returncode == 0 and "afir_region_s1_i32_a" in p.stdout
+
+
+def _compile(tmp_path, env=None, mlir=MC.SPLIT_HALVES):
+    src = tmp_path / "k.mlir"
+    src.write_text(mlir)
+    p = subprocess.run([RS, "--kernel", str(src), "--output", str(tmp_path / "art"), "--name", "k"],
+                       capture_output=True, text=True, env=dict(os.environ, **(env or {})))
+    assert p.returncode == 0, p.stderr
+    return (tmp_path / "art" / "out" / "manifest.txt").read_text().splitlines(), tmp_path / "art"
+
+
+def test_artifact_holds_source_and_code_object(tmp_path):
+    manifest, art = _compile(tmp_path)
+    assert "code_object_path=k.hsaco" in manifest
+    assert (art / "k.hip").read_text().startswith("// HIP kernels for the fused region 'k'")
+    assert b"afir_region_s1_i64_g" in (art / "k.hsaco").read_bytes()
+    desc = (art / "k.hipk").read_text()
+    assert "code_object=k.hsaco\n" in desc and f"code_object_dir={art}\n" in desc
+    assert not (art / "k.hipcc.log").exists()
+    # the artifact loads again from its root
+    assert subprocess.run([RS, "--artifact-root", str(art)], capture_output=True).returncode == 0
+
+
+def test_artifact_without_compiler_keeps_the_program(tmp_path):
+    manifest, art = _compile(tmp_path, env={"AFIR_HIP_CODEGEN": "0"})
+    assert not any(l.startswith("code_object_path=") for l in manifest)
+    assert "code_object_note=disabled by AFIR_HIP_CODEGEN=0" in manifest
+    assert "program:\nafir-hip-region 1" in (art / "k.hipk").read_text()
+    sub = tmp_path / "b"
+    sub.mkdir()
+    manifest, art = _compile(sub, env={"HIPCC": "/nonexistent/hipcc"})
+    assert any(l.startswith("code_object_note=cannot start /nonexistent/hipcc") for l in manifest)
+    assert (art / "k.hip").exists() and not (art / "k.hsaco").exists()
+
+
+def test_capi_emit_and_attach_without_gpu(pkg):
+    from ascend_mlir_amd import hip_kernels as H
+    L = H.load()
+    r = H.Region(RC.RELU_COL_ADD)
+    src = r.emit_source()
+    assert src == _emit(RC.RELU_COL_ADD).stdout.replace("fused region 'region'", "fused region 'region'")
+    u64 = ctypes.c_uint64
+    L.afir_hip_region_attach_code_object.argtypes = [u64, ctypes.c_char_p, ctypes.c_size_t]
+    assert L.afir_hip_region_attach_code_object(u64(r.handle), None, 0) != 0
+    assert b"empty image" in L.afir_hip_last_error()
+    assert L.afir_hip_region_attach_code_object(u64(999999), b"x" * 16, 16) != 0
+    assert b"no region program" in L.afir_hip_last_error()
+    # an image is accepted as bytes here; it is checked against the program when first launched
+    r.attach_code_object(b"\x7fELF" + b"\0" * 60)
+    assert r.kernel == "fused_region_compiled"
+    r.close()
+    prog = subprocess.run([TR, "-mlir-to-hip", "-"], input=MC.MATMUL_BIAS_LEAKY_BF16, capture_output=True, text=True).stdout
+    m = H.Region(prog)
+    with pytest.raises(H.AfirHipError, match="no specialised kernel"):
+        m.emit_source()
+    with pytest.raises(H.AfirHipError, match="take no code object"):
+        m.attach_code_object(b"\x7fELF" + b"\0" * 60)
+    m.close()
