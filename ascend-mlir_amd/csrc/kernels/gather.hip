@@ -102,6 +102,54 @@ __global__ __launch_bounds__(kThreads) void gather_scale_shift_f16_vec(
   }
 }
 
+// Rows of exactly lanes * 4 chunks (lanes a power of two <= 256): a row is
+// spread over `lanes` lanes, each taking four 16-byte chunks `lanes` chunks
+// apart, so a wave-level load covers contiguous runs of whole rows and every
+// lane has four loads in flight; 256 / lanes rows per workgroup pass.  The
+// lane's four scale / shift chunks stay in registers.
+constexpr int kGroups = 4;
+__global__ __launch_bounds__(kThreads) void gather_scale_shift_f16_grouped(
+    const uint16_t *__restrict__ table, const int32_t *__restrict__ idx,
+    const uint16_t *__restrict__ scale, const uint16_t *__restrict__ shift,
+    uint16_t *__restrict__ out, int32_t *__restrict__ error_flag, uint32_t rows, int lanes_log2,
+    int64_t nidx) {
+  const int lanes = 1 << lanes_log2;
+  const int rows_per_pass = kThreads >> lanes_log2;
+  const int local_row = threadIdx.x >> lanes_log2;
+  const int col0 = threadIdx.x & (lanes - 1);
+  const int64_t dim = (int64_t)lanes * kGroups * 8;
+  const u32x4 nan_row = {0x7e007e00u, 0x7e007e00u, 0x7e007e00u, 0x7e007e00u};
+  float s[kGroups][8], h[kGroups][8];
+#pragma unroll
+  for (int u = 0; u < kGroups; ++u) {
+    const int col = col0 + u * lanes;
+    const u32x4 sraw = *reinterpret_cast<const u32x4 *>(scale + (int64_t)col * 8);
+    const u32x4 hraw = *reinterpret_cast<const u32x4 *>(shift + (int64_t)col * 8);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      s[u][2 * d] = f16_lo(sraw[d]);
+      s[u][2 * d + 1] = f16_hi(sraw[d]);
+      h[u][2 * d] = f16_lo(hraw[d]);
+      h[u][2 * d + 1] = f16_hi(hraw[d]);
+    }
+  }
+  for (int64_t r0 = (int64_t)blockIdx.x * rows_per_pass; r0 < nidx; r0 += (int64_t)gridDim.x * rows_per_pass) {
+    const int64_t r = r0 + local_row;
+    if (r >= nidx) continue;
+    const uint32_t src = (uint32_t)idx[r];
+    const bool good = src < rows;
+    const u32x4 *row = reinterpret_cast<const u32x4 *>(table + (int64_t)(good ? src : 0u) * dim);
+    u32x4 v[kGroups];
+#pragma unroll
+    for (int u = 0; u < kGroups; ++u) v[u] = row[col0 + u * lanes];
+    u32x4 *dst = reinterpret_cast<u32x4 *>(out + r * dim);
+#pragma unroll
+    for (int u = 0; u < kGroups; ++u)
+      store_nt(dst + col0 + u * lanes, good ? scale_shift(v[u], s[u], h[u]) : nan_row);
+    if (!good && error_flag && col0 == 0) atomicOr(error_flag, 1);
+  }
+}
+
 // Any dim / alignment: one wave per row, 2-byte accesses.
 __global__ __launch_bounds__(kThreads) void gather_scale_shift_f16_any(
     const uint16_t *__restrict__ table, const int32_t *__restrict__ idx,
@@ -146,7 +194,18 @@ LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx
   // (an empty table has no row to fall back on: the scalar kernel never reads it)
   const bool vec = rows > 0 && (dim % 8 == 0) && aligned16(table) && aligned16(scale) && aligned16(shift) &&
                    aligned16(out);
-  if (vec) {
+  const int64_t chunks64 = dim / 8;
+  int lanes_log2 = 0;
+  while (lanes_log2 < 8 && ((int64_t)kGroups << lanes_log2) < chunks64) ++lanes_log2;
+  if (vec && ((int64_t)kGroups << lanes_log2) == chunks64) {
+    const int rows_per_pass = kThreads >> lanes_log2;
+    int64_t blocks = (nidx + rows_per_pass - 1) / rows_per_pass;
+    if (blocks > (int64_t)kNumCU * 64) blocks = (int64_t)kNumCU * 64;
+    if (block_dim) blocks = block_dim;
+    hipLaunchKernelGGL(gather_scale_shift_f16_grouped, dim3((unsigned)blocks), dim3(kThreads), 0,
+                       stream, table, idx, scale, shift, out, error_flag, (uint32_t)rows, lanes_log2,
+                       nidx);
+  } else if (vec) {
     const int chunks = (int)(dim / 8);
     int lanes_per_row = ((chunks + kWave - 1) / kWave) * kWave;
     if (lanes_per_row > kThreads) lanes_per_row = kThreads;

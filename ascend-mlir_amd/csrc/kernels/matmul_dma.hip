@@ -39,6 +39,11 @@
 // 8 waves as 2(m) x 4(n), wave tile 128 x 64 = 4 x 2 MFMA tiles of 32x32,
 // v_mfma_f32_32x32x16_bf16 with the operands swapped (B as the row operand) so
 // that a lane holds four consecutive n of one m for the fused epilogue.
+// (AFIR_MM_WAVES_N=2 builds 4 waves of 128 x 128 instead: a third fewer LDS
+// operand bytes per MFMA, but one wave per SIMD leaves the matrix unit idle
+// around every barrier; measured on MI355X it is 11 % slower on constant
+// operands and equal, within 1 %, on N(0, 1/sqrt(K)) operands, where the board
+// power limit sets the pace.)
 #include "kernels.h"
 
 namespace afir {
@@ -81,66 +86,55 @@ __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-// Operands of one k16 substep: four A fragments (m tiles 0..3, 4 KiB apart)
-// and two B fragments (n tiles 0..1, each two transposing 64-bit reads 4 rows
-// apart).  issue_reads only issues; the registers must not be touched until
+// Operands of one k16 substep: TMW A fragments (m tiles, 4 KiB apart) and TNW
+// B fragments (n tiles, each two transposing 64-bit reads 4 rows apart).
+// issue_reads only issues; the registers must not be touched until
 // settle_reads, which waits for the LDS unit and hands the same registers back
 // as fresh values.
-template <int TMW>
+template <int TMW, int TNW>
 struct Operands {
   u32x4 a[TMW];
-  u32x2 b[2][2];
+  u32x2 b[TNW][2];
 };
 
-template <int KS>  // k16 substep within the B stage (0 or 1)
-__device__ __forceinline__ void issue_reads(uint32_t a_addr, uint32_t b_addr0, uint32_t b_addr1,
-                                            Operands<4> &o) {
+template <int OFF>
+__device__ __forceinline__ void read_a(uint32_t addr, u32x4 &dst) {
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(dst) : "v"(addr), "n"(OFF) : "memory");
+}
+template <int OFF>
+__device__ __forceinline__ void read_b(uint32_t addr, u32x2 &dst) {
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=&v"(dst) : "v"(addr), "n"(OFF) : "memory");
+}
+
+template <int KS, int TMW, int TNW>  // KS: k16 substep within the B stage (0 or 1)
+__device__ __forceinline__ void issue_reads(uint32_t a_addr, const uint32_t (&b_addr)[TNW],
+                                            Operands<TMW, TNW> &o) {
   constexpr int kOff = KS * 16 * 512;  // 16 rows of B
-  asm volatile(
-      "ds_read_b128 %0, %8\n\t"
-      "ds_read_b128 %1, %8 offset:4096\n\t"
-      "ds_read_b128 %2, %8 offset:8192\n\t"
-      "ds_read_b128 %3, %8 offset:12288\n\t"
-      "ds_read_b64_tr_b16 %4, %9 offset:%11\n\t"
-      "ds_read_b64_tr_b16 %5, %9 offset:%12\n\t"
-      "ds_read_b64_tr_b16 %6, %10 offset:%11\n\t"
-      "ds_read_b64_tr_b16 %7, %10 offset:%12"
-      : "=&v"(o.a[0]), "=&v"(o.a[1]), "=&v"(o.a[2]), "=&v"(o.a[3]), "=&v"(o.b[0][0]),
-        "=&v"(o.b[0][1]), "=&v"(o.b[1][0]), "=&v"(o.b[1][1])
-      : "v"(a_addr), "v"(b_addr0), "v"(b_addr1), "n"(kOff), "n"(kOff + 4 * 512)
-      : "memory");
+  read_a<0>(a_addr, o.a[0]);
+  read_a<4096>(a_addr, o.a[1]);
+  if constexpr (TMW == 4) {
+    read_a<8192>(a_addr, o.a[2]);
+    read_a<12288>(a_addr, o.a[3]);
+  }
+#pragma unroll
+  for (int j = 0; j < TNW; ++j) {
+    read_b<kOff>(b_addr[j], o.b[j][0]);
+    read_b<kOff + 4 * 512>(b_addr[j], o.b[j][1]);
+  }
 }
 
-template <int KS>
-__device__ __forceinline__ void issue_reads(uint32_t a_addr, uint32_t b_addr0, uint32_t b_addr1,
-                                            Operands<2> &o) {
-  constexpr int kOff = KS * 16 * 512;
-  asm volatile(
-      "ds_read_b128 %0, %6\n\t"
-      "ds_read_b128 %1, %6 offset:4096\n\t"
-      "ds_read_b64_tr_b16 %2, %7 offset:%9\n\t"
-      "ds_read_b64_tr_b16 %3, %7 offset:%10\n\t"
-      "ds_read_b64_tr_b16 %4, %8 offset:%9\n\t"
-      "ds_read_b64_tr_b16 %5, %8 offset:%10"
-      : "=&v"(o.a[0]), "=&v"(o.a[1]), "=&v"(o.b[0][0]), "=&v"(o.b[0][1]), "=&v"(o.b[1][0]),
-        "=&v"(o.b[1][1])
-      : "v"(a_addr), "v"(b_addr0), "v"(b_addr1), "n"(kOff), "n"(kOff + 4 * 512)
-      : "memory");
-}
-
-__device__ __forceinline__ void settle_reads(Operands<4> &o) {
-  asm volatile("s_waitcnt lgkmcnt(0)"
-               : "+v"(o.a[0]), "+v"(o.a[1]), "+v"(o.a[2]), "+v"(o.a[3]), "+v"(o.b[0][0]),
-                 "+v"(o.b[0][1]), "+v"(o.b[1][0]), "+v"(o.b[1][1])
-               :
-               : "memory");
-}
-__device__ __forceinline__ void settle_reads(Operands<2> &o) {
-  asm volatile("s_waitcnt lgkmcnt(0)"
-               : "+v"(o.a[0]), "+v"(o.a[1]), "+v"(o.b[0][0]), "+v"(o.b[0][1]), "+v"(o.b[1][0]),
-                 "+v"(o.b[1][1])
-               :
-               : "memory");
+template <int TMW, int TNW>
+__device__ __forceinline__ void settle_reads(Operands<TMW, TNW> &o) {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  // volatile asm statements keep their order: every register counts as
+  // rewritten after the wait, so no use can move above it
+#pragma unroll
+  for (int i = 0; i < TMW; ++i) asm volatile("" : "+v"(o.a[i]));
+#pragma unroll
+  for (int j = 0; j < TNW; ++j) {
+    asm volatile("" : "+v"(o.b[j][0]));
+    asm volatile("" : "+v"(o.b[j][1]));
+  }
 }
 
 struct Par0 { static constexpr int value = 0; };
@@ -148,9 +142,11 @@ struct Par1 { static constexpr int value = 1; };
 struct Steady { static constexpr bool value = true; };
 struct Drain { static constexpr bool value = false; };
 
-// WM = waves along m (2 or 4); 4 waves along n.  Wave tile (256/WM) x 64.
-template <int WM>
-__global__ __launch_bounds__(WM * 4 * 64) void matmul_bias_leakyrelu_bf16_dma(
+// WM x WN waves (m x n), wave tile (256/WM) x (256/WN): 2 x 4 waves of
+// 128 x 64, or 2 x 2 waves of 128 x 128 (one wave per SIMD, two thirds of the
+// LDS operand bytes per MFMA).
+template <int WM, int WN>
+__global__ __launch_bounds__(WM * WN * 64) void matmul_bias_leakyrelu_bf16_dma(
     const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
     const uint16_t *__restrict__ bias, uint16_t *__restrict__ out, int M, int K, int N,
     float alpha, int tiles_m, int tiles_n) {
@@ -160,12 +156,13 @@ __global__ __launch_bounds__(WM * 4 * 64) void matmul_bias_leakyrelu_bf16_dma(
 
   const int t = threadIdx.x, lane = t & 63;
   constexpr int TMW = 8 / WM;            // 32-row MFMA tiles per wave along m
-  constexpr int NWAVES = WM * 4;
+  constexpr int TNW = 8 / WN;            // 32-column MFMA tiles per wave along n
+  constexpr int NWAVES = WM * WN;
   constexpr int A_REG = 32 / NWAVES;     // 1 KiB direct-to-LDS regions per wave per A slice
   constexpr int B_REG = 16 / NWAVES;     // ... per B stage
   constexpr int kSteadyVm = 2 * B_REG + A_REG;  // loads younger than what the next stage needs
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-  const int wm = wave >> 2, wn = wave & 3;
+  const int wm = wave / WN, wn = wave % WN;
   const int KT = K / kBK;   // B stages; even, the launcher requires K % 64 == 0
   const int KT2 = KT >> 1;  // A slices
 
@@ -175,10 +172,10 @@ __global__ __launch_bounds__(WM * 4 * 64) void matmul_bias_leakyrelu_bf16_dma(
   const uint32_t a_rd =
       (uint32_t)((wm * TMW * 32 + lrow) * 128 + (lk ^ ((lrow >> 1) & 7)) * 16);
   const int g = lane >> 4, li = lane & 15;
-  uint32_t b_rd[2];
+  uint32_t b_rd[TNW];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int ntile = wn * 2 + j;
+  for (int j = 0; j < TNW; ++j) {
+    const int ntile = wn * TNW + j;
     const int c16 = ntile * 4 + (g & 1) * 2 + ((li & 3) >> 1);
     const int phys = c16 ^ ((li >> 2) << 2);
     b_rd[j] = (uint32_t)(kRingB + ((g >> 1) * 8 + (li >> 2)) * 512 + phys * 16 + (li & 1) * 8);
@@ -235,17 +232,17 @@ __global__ __launch_bounds__(WM * 4 * 64) void matmul_bias_leakyrelu_bf16_dma(
       for (int q = 0; q < B_REG; ++q) gb[q] += step;
     };
 
-    f32x16 acc[TMW][2];
+    f32x16 acc[TMW][TNW];
 #pragma unroll
     for (int i = 0; i < TMW; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < TNW; ++j)
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-    auto multiply = [&](const Operands<TMW> &o) {
+    auto multiply = [&](const Operands<TMW, TNW> &o) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < TNW; ++j) {
         const u32x4 bw = {o.b[j][0].x, o.b[j][0].y, o.b[j][1].x, o.b[j][1].y};
 #pragma unroll
         for (int i = 0; i < TMW; ++i)
@@ -256,14 +253,17 @@ __global__ __launch_bounds__(WM * 4 * 64) void matmul_bias_leakyrelu_bf16_dma(
     };
     // operand reads for a stage held in A slot sa / B slot sbk; the stage is the
     // first (par 0) or second (par 1) half of its A slice; h = k16 substep
-    auto reads = [&](int sa, int sbk, int par, int h, Operands<TMW> &o) {
+    auto reads = [&](int sa, int sbk, int par, int h, Operands<TMW, TNW> &o) {
       const uint32_t aa =
           lds_base + (uint32_t)(sa * kSlotA) + (a_rd ^ (uint32_t)((par * 2 + h) * 32));
       const uint32_t bb = lds_base + (uint32_t)(sbk * kSlotB);
+      uint32_t ba[TNW];
+#pragma unroll
+      for (int j = 0; j < TNW; ++j) ba[j] = bb + b_rd[j];
       if (h == 0)
-        issue_reads<0>(aa, bb + b_rd[0], bb + b_rd[1], o);
+        issue_reads<0>(aa, ba, o);
       else
-        issue_reads<1>(aa, bb + b_rd[0], bb + b_rd[1], o);
+        issue_reads<1>(aa, ba, o);
     };
 
     // prologue (the launcher guarantees KT >= 8): fill both rings, oldest first
@@ -276,7 +276,7 @@ __global__ __launch_bounds__(WM * 4 * 64) void matmul_bias_leakyrelu_bf16_dma(
     issue_a(2);
     wait_vmcnt<3 * B_REG + 2 * A_REG>();  // everything younger than A(0), B(0)
     __builtin_amdgcn_s_barrier();
-    Operands<TMW> even, odd;
+    Operands<TMW, TNW> even, odd;
     reads(0, 0, 0, 0, even);
     settle_reads(even);
 
@@ -339,19 +339,25 @@ __global__ __launch_bounds__(WM * 4 * 64) void matmul_bias_leakyrelu_bf16_dma(
     // x 2 halves) and for the 16-byte row reads.
     __builtin_amdgcn_s_barrier();
     {
-      unsigned char *const stage = smem + wave * 4096;
+      constexpr int CH = TNW * 4;              // 16-byte chunks per staged row
+      constexpr int kRowBytes = CH * 16;       // 128 or 256
+      constexpr int kRowsPerPass = 64 / CH;    // rows one store instruction covers
+      unsigned char *const stage = smem + wave * (32 * kRowBytes);
       const int lm = lane & 31, lq = lane >> 5;
-      const int rr = lane >> 3, cc = lane & 7;
-      u32x2 braw[2][4];
+      const int rr = lane / CH, cc = lane % CH;
+      // two 128-byte rows share a swizzle value (they span the same banks as
+      // one 256-byte row)
+      auto swz = [](int r) { return CH == 8 ? ((r >> 1) & 7) : (r & 15); };
+      u32x2 braw[TNW][4];
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < TNW; ++j)
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-          braw[j][q] = *reinterpret_cast<const u32x2 *>(bias + n0 + (wn * 2 + j) * 32 + 8 * q + 4 * lq);
+          braw[j][q] = *reinterpret_cast<const u32x2 *>(bias + n0 + (wn * TNW + j) * 32 + 8 * q + 4 * lq);
 #pragma unroll
       for (int i = 0; i < TMW; ++i) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
+        for (int j = 0; j < TNW; ++j) {
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             const float b0 = bf16_lo(braw[j][q].x), b1 = bf16_hi(braw[j][q].x);
@@ -367,17 +373,17 @@ __global__ __launch_bounds__(WM * 4 * 64) void matmul_bias_leakyrelu_bf16_dma(
             u32x2 w;
             w.x = pack_bf16(v0, v1);
             w.y = pack_bf16(v2, v3);
-            const int chunk = (j * 4 + q) ^ ((lm >> 1) & 7);
-            *reinterpret_cast<u32x2 *>(stage + lm * 128 + chunk * 16 + lq * 8) = w;
+            const int chunk = (j * 4 + q) ^ swz(lm);
+            *reinterpret_cast<u32x2 *>(stage + lm * kRowBytes + chunk * 16 + lq * 8) = w;
           }
         }
 #pragma unroll
-        for (int tq = 0; tq < 4; ++tq) {
-          const int r = rr + 8 * tq;
+        for (int tq = 0; tq < 32 / kRowsPerPass; ++tq) {
+          const int r = rr + kRowsPerPass * tq;
           const u32x4 line =
-              *reinterpret_cast<const u32x4 *>(stage + r * 128 + ((cc ^ ((r >> 1) & 7)) * 16));
+              *reinterpret_cast<const u32x4 *>(stage + r * kRowBytes + ((cc ^ swz(r)) * 16));
           const int m = m0 + (wm * TMW + i) * 32 + r;
-          *reinterpret_cast<u32x4 *>(out + (int64_t)m * N + n0 + wn * 64 + cc * 8) = line;
+          *reinterpret_cast<u32x4 *>(out + (int64_t)m * N + n0 + wn * (TNW * 32) + cc * 8) = line;
         }
       }
     }
@@ -395,6 +401,9 @@ bool matmul_dma_supported(int64_t m, int64_t k, int64_t n) {
 #ifndef AFIR_MM_WAVES_M
 #define AFIR_MM_WAVES_M 2
 #endif
+#ifndef AFIR_MM_WAVES_N
+#define AFIR_MM_WAVES_N 4
+#endif
 #ifndef AFIR_MM_GRID
 #define AFIR_MM_GRID kNumCU
 #endif
@@ -402,8 +411,8 @@ bool matmul_dma_supported(int64_t m, int64_t k, int64_t n) {
 LaunchStatus launch_matmul_dma(const uint16_t *a, const uint16_t *b, const uint16_t *bias,
                                uint16_t *out, int m, int k, int n, float alpha,
                                uint32_t block_dim, hipStream_t stream) {
-  constexpr int WM = AFIR_MM_WAVES_M;
-  auto kernel = matmul_bias_leakyrelu_bf16_dma<WM>;
+  constexpr int WM = AFIR_MM_WAVES_M, WN = AFIR_MM_WAVES_N;
+  auto kernel = matmul_bias_leakyrelu_bf16_dma<WM, WN>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize,
                                                kLdsBytes);
@@ -414,7 +423,7 @@ LaunchStatus launch_matmul_dma(const uint16_t *a, const uint16_t *b, const uint1
   int64_t blocks = (int64_t)tiles_m * tiles_n;
   if (blocks > AFIR_MM_GRID) blocks = AFIR_MM_GRID;
   if (block_dim) blocks = block_dim;
-  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(WM * 4 * 64), kLdsBytes, stream, a, b,
+  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(WM * WN * 64), kLdsBytes, stream, a, b,
                      bias, out, m, k, n, alpha, tiles_m, tiles_n);
   return after_launch();
 }
