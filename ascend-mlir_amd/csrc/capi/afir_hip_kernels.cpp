@@ -4,6 +4,7 @@
 // include/afir_hip_kernels.h.
 #include "afir_hip_kernels.h"
 
+#include <cstddef>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -527,6 +528,12 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
   // interpreter kernel (the tests compare the two)
   if (const char *env = std::getenv("AFIR_HIP_REGION_INTERPRET"))
     if (*env && *env != '0') compiled.reset();
+  struct PendingSegment {
+    int segment;
+    afir_target::SpecArgs args;
+    bool idx32, aligned;
+  };
+  std::vector<PendingSegment> pending;   // compiled kernels to launch, non-empty segments only
   for (const afir_region::ResolvedSegment &seg : res.segments) {
     afir::RegionArgs a;
     std::memset(&a, 0, sizeof a);
@@ -606,18 +613,56 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
         // 128-bit loads by the aligned variant
         if (d.stride[last] == 1 && d.gdim != last && (!d.vec || (d.gdim >= 0 && !d.gvec))) all_aligned = false;
       }
-      hipFunction_t fn = nullptr;
-      why = compiled_function(compiled.get(), r->program, afir_target::specKernelName(segment, g.idx32, all_aligned), &fn);
-      if (!why.empty()) return fail(AFIR_HIP_E_LAUNCH, why);
-      size_t bytes = sizeof sa;
-      void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, &sa, HIP_LAUNCH_PARAM_BUFFER_SIZE, &bytes, HIP_LAUNCH_PARAM_END};
-      const hipError_t e = hipModuleLaunchKernel(fn, (unsigned)g.blocks, 1, 1, 256, 1, 1, 0,
-                                                 static_cast<hipStream_t>(stream), nullptr, config);
-      if (e != hipSuccess) return fail(AFIR_HIP_E_LAUNCH, std::string("compiled region kernel: ") + hipGetErrorString(e));
+      pending.push_back({segment, sa, g.idx32, all_aligned});
       continue;
     }
     uint32_t rc = finish(afir::launch_fused_region(a, block_dim, static_cast<hipStream_t>(stream)));
     if (rc != AFIR_HIP_OK) return rc;
+  }
+  if (!pending.empty()) {
+    auto launch = [&](const std::string &name, void *args, size_t bytes, unsigned blocks) -> uint32_t {
+      hipFunction_t fn = nullptr;
+      const std::string no = compiled_function(compiled.get(), r->program, name, &fn);
+      if (!no.empty()) return fail(AFIR_HIP_E_LAUNCH, no);
+      void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &bytes, HIP_LAUNCH_PARAM_END};
+      const hipError_t e = hipModuleLaunchKernel(fn, blocks, 1, 1, 256, 1, 1, 0, static_cast<hipStream_t>(stream),
+                                                 nullptr, config);
+      if (e != hipSuccess) return fail(AFIR_HIP_E_LAUNCH, std::string("compiled region kernel: ") + hipGetErrorString(e));
+      return AFIR_HIP_OK;
+    };
+    // segments that agree on the kernel variant go out as one launch
+    const int nseg = (int)res.segments.size();
+    bool together = pending.size() > 1 && nseg <= afir_target::kSpecMaxSegments;
+    int64_t total = 0;
+    for (const PendingSegment &p : pending) {
+      together = together && p.idx32 == pending[0].idx32 && p.aligned == pending[0].aligned;
+      total += p.args.grid;
+    }
+    if (together && total <= 0x7fffffff) {
+      afir_target::SpecAll all;
+      std::memset(&all, 0, sizeof all);
+      int next = 0;
+      size_t at = 0;
+      for (int k = 0; k < nseg; ++k) {
+        all.first[k] = next;
+        if (at < pending.size() && pending[at].segment == k) {
+          all.seg[k] = pending[at].args;
+          next += pending[at].args.grid;
+          ++at;
+        }
+      }
+      for (int k = nseg; k <= afir_target::kSpecMaxSegments; ++k) all.first[k] = next;
+      const uint32_t rc = launch(afir_target::specAllKernelName(pending[0].idx32, pending[0].aligned), &all,
+                                 offsetof(afir_target::SpecAll, seg) + (size_t)nseg * sizeof(afir_target::SpecArgs),
+                                 (unsigned)next);
+      if (rc != AFIR_HIP_OK) return rc;
+    } else {
+      for (PendingSegment &p : pending) {
+        const uint32_t rc = launch(afir_target::specKernelName(p.segment, p.idx32, p.aligned), &p.args,
+                                   sizeof p.args, (unsigned)p.args.grid);
+        if (rc != AFIR_HIP_OK) return rc;
+      }
+    }
   }
   g_last_error.clear();
   return AFIR_HIP_OK;

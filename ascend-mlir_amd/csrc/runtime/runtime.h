@@ -323,11 +323,25 @@ struct SessionSummary {
   std::map<std::string, std::string> runtimeAttributes;
   std::map<std::string, int64_t> runtimeCounters;
   OutputComparisonResult comparison;
+  // Profiling (tasks with "profiling": true): one trace.json per task, schema
+  // version 1 of lib/Runtime/Execution/SimBackend.cpp:314-374; score =
+  // cycle_count = the kernel's duration in nanoseconds.
+  struct ProfileArtifact {
+    std::string taskId;
+    std::string path;
+    int64_t score = 0;
+    int64_t cycleCount = 0;
+  };
+  std::string sessionId;
+  std::vector<ProfileArtifact> profileArtifacts;
+  std::string retainedSummaryPath;   // session_summary.json, when profiles were retained
 };
 
 // Runs one task: load artifact, bind inputs, allocate outputs from expected
 // shapes, launch, validate, write outputs.
-SessionSummary runSingleTask(const RunTaskSpec &task, RunnerFactory factory, int deviceId);
+// profileDirectory: where a profiling task writes its trace.json ("" = nowhere).
+SessionSummary runSingleTask(const RunTaskSpec &task, RunnerFactory factory, int deviceId,
+                             const std::string &profileDirectory = "", const std::string &sessionId = "");
 
 // Execution order of a manifest's tasks: Kahn's algorithm over `dependencies`,
 // ready tasks in manifest order (lib/Runtime/Execution/TaskGraph.cpp:33-79).
@@ -342,7 +356,17 @@ Expected<std::vector<size_t>> planTasks(const RunManifestSpec &manifest);
 // first failing task; the summary is the failing task's, or the merged one
 // (validation passed = every validating task passed; counters carry a
 // "<task>." prefix when there is more than one task).
+// Profiling tasks write <workingDirectory>/opprof/hip/<task>/trace.json.
 SessionSummary runSession(const RunManifestSpec &manifest, RunnerFactory factory, int deviceId,
                           const std::string &workingDirectory);
+
+// Copies a session's profile artifacts to <root>/<session id>/tasks/<task>.json,
+// writes <root>/<session id>/session_summary.json (schema version 1 of
+// lib/Runtime/Profile/ProfileUtils.cpp:134-345: session_id, backend,
+// task_count, successful_task_count, failed_task_count, tasks[{task_id,
+// profile_path, score, cycle_count}], runtime{attributes, counters},
+// total_score, total_cycle_count) and keeps the `keep` newest sessions under
+// root.  Rewrites the summary's artifact paths to the retained copies.
+Status retainProfileArtifacts(SessionSummary &summary, const std::string &root, size_t keep = 20);
 
 }  // namespace afirt

@@ -502,10 +502,10 @@ class SegmentEmitter {
         << (reduce_ ? ", row sum over the innermost dim" : ", parallel") << "; a lane takes " << U_ << " groups of " << W_
         << " elements per pass ----\n";
     os_ << "// I: position type.  A: every 128-bit access is aligned and every pass is whole (no tail).\n";
-    os_ << "template <typename I, bool A>\nDEV void segment" << index_ << "(const SpecArgs &R) {\n";
+    os_ << "template <typename I, bool A>\nDEV void segment" << index_
+        << "(const SpecArgs &R, const I bid, const I nblocks) {\n";
     line(1, "constexpr int W = " + std::to_string(W_) + ", U = " + std::to_string(U_) + ";");
     line(1, "const int tid = (int)__builtin_amdgcn_workitem_id_x();");
-    line(1, "const I bid = (I)__builtin_amdgcn_workgroup_id_x();");
     line(1, "const I n = (I)R.size[" + std::to_string(last_) + "];");
     line(1, "const I groups = (n + (W - 1)) / W;");
     if (rank_ == 1) line(1, "const I rows = 1;");
@@ -517,7 +517,7 @@ class SegmentEmitter {
     if (reduce_) {
       line(1, "const int lane = tid & 63;");
       line(1, "const I wave = bid * 4 + (I)(tid >> 6);");
-      line(1, "const I nwaves = (I)R.grid * 4;");
+      line(1, "const I nwaves = nblocks * 4;");
       line(1, "for (I row = wave; row < rows; row += nwaves) {");
       emitPositionOfRow(2);
       emitRowInvariants(2);
@@ -555,7 +555,7 @@ class SegmentEmitter {
     line(1, "const I rows_per_pass = (I)(256 >> R.lanes_log2);");
     line(1, "const I local_row = (I)(tid >> R.lanes_log2);");
     line(1, "const I first_group = (I)tid & (lanes - 1);");
-    line(1, "for (I row0 = bid * rows_per_pass; row0 < rows; row0 += (I)R.grid * rows_per_pass) {");
+    line(1, "for (I row0 = bid * rows_per_pass; row0 < rows; row0 += nblocks * rows_per_pass) {");
     line(2, "const I row = row0 + local_row;");
     line(2, "if (row >= rows) continue;");
     emitPositionOfRow(2);
@@ -592,7 +592,9 @@ class SegmentEmitter {
     for (int i32 = 1; i32 >= 0; --i32)
       for (int a = 1; a >= 0; --a)
         os_ << "KERNEL void " << specKernelName(index_, i32 != 0, a != 0) << "(const SpecArgs R) { segment" << index_
-            << "<" << (i32 ? "int" : "long long") << ", " << (a ? "true" : "false") << ">(R); }\n";
+            << "<" << (i32 ? "int" : "long long") << ", " << (a ? "true" : "false")
+            << ">(R, (" << (i32 ? "int" : "long long") << ")__builtin_amdgcn_workgroup_id_x(), ("
+            << (i32 ? "int" : "long long") << ")R.grid); }\n";
   }
 
   const Program &p_;
@@ -627,6 +629,10 @@ uint64_t programHash(const Program &p) {
   return h;
 }
 
+std::string specAllKernelName(bool idx32, bool aligned) {
+  return std::string("afir_region_all") + (idx32 ? "_i32" : "_i64") + (aligned ? "_a" : "_g");
+}
+
 std::string specKernelName(int segment, bool idx32, bool aligned) {
   return "afir_region_s" + std::to_string(segment) + (idx32 ? "_i32" : "_i64") + (aligned ? "_a" : "_g");
 }
@@ -652,6 +658,26 @@ std::string emitHipSource(const Program &p, const std::string &title, std::strin
   for (int s = 0; s < (int)p.segments.size(); ++s) {
     SegmentEmitter e(p, s, os);
     if (std::string why = e.run(); !why.empty()) return why;
+  }
+  const int nseg = (int)p.segments.size();
+  if (nseg > 1 && nseg <= kSpecMaxSegments) {
+    // every segment in one launch: the workgroups are dealt out segment by segment
+    os << "\n// ---- all segments in one launch ----\n";
+    os << "struct SpecAll {\n  int first[" << kSpecMaxSegments + 1 << "];   // first workgroup of each segment, then the total\n"
+       << "  int pad;\n  SpecArgs seg[" << nseg << "];\n};\n";
+    os << "static_assert(__builtin_offsetof(SpecAll, seg) == " << offsetof(SpecAll, seg)
+       << ", \"launch argument layout differs from the kernel library's\");\n";
+    for (int i32 = 1; i32 >= 0; --i32)
+      for (int a = 1; a >= 0; --a) {
+        const char *I = i32 ? "int" : "long long";
+        os << "KERNEL void " << specAllKernelName(i32 != 0, a != 0) << "(const SpecAll M) {\n";
+        os << "  const int b = (int)__builtin_amdgcn_workgroup_id_x();\n";
+        for (int k = 0; k < nseg; ++k)
+          os << "  " << (k ? "else " : "") << (k + 1 < nseg ? "if (b < M.first[" + std::to_string(k + 1) + "]) " : "")
+             << "segment" << k << "<" << I << ", " << (a ? "true" : "false") << ">(M.seg[" << k << "], (" << I
+             << ")(b - M.first[" << k << "]), (" << I << ")(M.first[" << k + 1 << "] - M.first[" << k << "]));\n";
+        os << "}\n";
+      }
   }
   *source = os.str();
   return "";

@@ -49,6 +49,17 @@ struct SpecArgs {
   SpecInput in[kSpecMaxInputs];
 };
 
+// Programs of 2..kSpecMaxSegments segments also get one kernel that runs all
+// of them in a single launch (segments write disjoint row ranges of the
+// output); its argument:
+constexpr int kSpecMaxSegments = 4;
+struct SpecAll {
+  int first[kSpecMaxSegments + 1];   // first workgroup of each segment, then the total
+  int pad;
+  SpecArgs seg[kSpecMaxSegments];    // the emitted declaration holds the program's segment count
+};
+std::string specAllKernelName(bool idx32, bool aligned);
+
 // A lane's share of one pass over a row: `unroll` groups of `width` consecutive
 // elements (16 bytes of the narrowest tensor), the groups one lane-set apart.
 struct SpecShape {

@@ -27,6 +27,7 @@ class SuccessfulTestingRunner final : public ExecutionRunner {
   Status runDynamicLibraryArtifact(const DynamicLibraryExecutionLaunch &, RunArgs &) override {
     return Status::success();
   }
+  double lastKernelMicroseconds() const override { return 12.5; }   // a fixed figure for the profile tests
 };
 std::unique_ptr<ExecutionRunner> makeTestingRunner() {
   return std::make_unique<SuccessfulTestingRunner>();
@@ -189,8 +190,25 @@ int main(int argc, char **argv) {
   std::printf("session.backend=%s\n", s.backend.c_str());
   std::printf("session.result=success\n");
   if (s.validationRan && s.validationPassed) std::printf("session.validation=pass\n");
-  std::printf("session.profile.session_id=%s\n", task.taskId.c_str());
-  std::printf("session.profile.count=0\n");
+  if (!s.profileArtifacts.empty()) {
+    // profiles outlive the run directory: <tmp>/ascendc-runtime-profiles/<session id>/
+    // (tools/runtime-session/runtime_session_main.cpp:212-228)
+    const char *tmp = std::getenv("TMPDIR");
+    const std::string root = std::string(tmp && *tmp ? tmp : "/tmp") + "/ascendc-runtime-profiles";
+    if (Status st = retainProfileArtifacts(s, root); !st.ok()) {
+      s.success = false;
+      s.errorStage = "profiling";
+      s.errorMessage = st.message;
+      s.rawErrorMessage = "[hip:profiling] " + st.message;
+      printErrorSummary(s);
+      return 2;
+    }
+  }
+  std::printf("session.profile.session_id=%s\n", s.sessionId.c_str());
+  std::printf("session.profile.count=%zu\n", s.profileArtifacts.size());
+  for (size_t i = 0; i < s.profileArtifacts.size(); ++i)
+    std::printf("session.profile[%zu]=%s\n", i, s.profileArtifacts[i].path.c_str());
+  if (!s.retainedSummaryPath.empty()) std::printf("session.profile.summary=%s\n", s.retainedSummaryPath.c_str());
   if (s.validationRan) {
     std::printf("session.runtime.attribute.max_abs_diff=%g\n", s.comparison.maxAbsDiff);
     std::printf("session.runtime.attribute.mean_abs_diff=%g\n", s.comparison.meanAbsDiff);

@@ -199,17 +199,27 @@ def test_two_kernel_session_feeds_one_kernel_into_the_next(tmp_path):
          "outputs": [{"name": "y", "path": str(tmp_path / "y.npy")}],
          "expected_outputs": [{"name": "y", "path": str(tmp_path / "want.npy")}],
          "tiling": {"schema": str(tmp_path / "rowsum.json"), "params": params(tmp_path / "rowsum.json", [m, n, n, m])},
-         "atol": 1e-3, "rtol": 1e-5},
-        {"task_id": "chain", "artifact_root": str(tmp_path / "add_mul"),
+         "atol": 1e-3, "rtol": 1e-5, "profiling": True},
+        {"task_id": "chain", "artifact_root": str(tmp_path / "add_mul"), "profiling": True,
          "inputs": [{"name": "a", "path": str(tmp_path / "a.npy")}, {"name": "b", "path": str(tmp_path / "b.npy")}],
          "outputs": [{"name": "t", "shape": [m, n], "dtype": "f32"}],
          "tiling": {"schema": str(tmp_path / "add_mul.json"),
                     "params": params(tmp_path / "add_mul.json", [m, n, m, n, m, n])}}]}
     (tmp_path / "m.json").write_text(json.dumps(manifest))
-    p = _rs("--run-manifest", str(tmp_path / "m.json"), "--run")
+    (tmp_path / "tmp").mkdir()
+    p = subprocess.run([RS, "--run-manifest", str(tmp_path / "m.json"), "--run"], capture_output=True, text=True,
+                       timeout=100, env=dict(os.environ, TMPDIR=str(tmp_path / "tmp")))
     assert p.returncode == 0, p.stdout + p.stderr
     lines = p.stdout.splitlines()
     assert "session.plan[0]=chain" in lines and "session.plan[1]=reduce" in lines
+    # both tasks profiled: measured kernel times in the traces and the retained summary
+    kv = dict(l.split("=", 1) for l in lines if "=" in l)
+    assert kv["session.profile.count"] == "2"
+    traces = [json.loads(open(kv[f"session.profile[{i}]"]).read()) for i in range(2)]
+    assert [t_["task_id"] for t_ in traces] == ["chain", "reduce"]
+    assert all(t_["backend"] == "hip" and 0 < t_["score"] < 10_000_000 and t_["validation_passed"] for t_ in traces)
+    summary = json.loads(open(kv["session.profile.summary"]).read())
+    assert summary["task_count"] == 2 and summary["total_score"] == sum(t_["score"] for t_ in traces)
     assert "session.result=success" in lines and "session.validation=pass" in lines
     assert np.load(tmp_path / "chain__t.npy").tobytes() == t.tobytes()      # the intermediate is bit-exact
     assert np.allclose(np.load(tmp_path / "y.npy"), want, rtol=1e-5, atol=1e-3)

@@ -327,3 +327,52 @@ def test_cli_multi_task_errors(tmp_path):
     (tmp_path / "dup.json").write_text(json.dumps(d))
     p = _rs("--run-manifest", str(tmp_path / "dup.json"))
     assert p.returncode == 4 and "duplicate task id" in p.stderr
+
+
+def test_cli_profiling_writes_trace_and_retained_summary(tmp_path):
+    """"profiling": true -> trace.json per task (schema version 1 of
+    lib/Runtime/Execution/SimBackend.cpp:314-374) and a retained
+    session_summary.json (lib/Runtime/Profile/ProfileUtils.cpp:134-345),
+    announced on the session.profile.* lines
+    (tools/runtime-session/runtime_session_main.cpp:167-177)."""
+    src = tmp_path / "example.mlir"
+    src.write_text(EXAMPLE_MLIR)
+    assert _rs("--kernel", str(src), "--output", str(tmp_path / "art"), "--name", "example").returncode == 0
+    m = _manifest(tmp_path, profiling=True, block_dim=3, workspace_size=64)
+    tmp = tmp_path / "tmp"
+    tmp.mkdir()
+    p = subprocess.run([RS, "--run-manifest", m, "--run", "--testing-driver=hip-success"], capture_output=True,
+                       text=True, env=dict(os.environ, TMPDIR=str(tmp)))
+    assert p.returncode == 0, p.stderr
+    kv = dict(l.split("=", 1) for l in p.stdout.splitlines() if "=" in l)
+    sid = kv["session.profile.session_id"]
+    assert re.fullmatch(r"runtime-session-[a-z0-9]{6}", sid)
+    assert kv["session.profile.count"] == "1"
+    retained = kv["session.profile[0]"]
+    assert retained == str(tmp / "ascendc-runtime-profiles" / sid / "tasks" / "main.json")
+    trace = json.loads(open(retained).read())
+    assert trace == json.loads((tmp_path / "opprof" / "hip" / "main" / "trace.json").read_text())
+    for key in ("schema_version", "backend", "session_id", "task_id", "kernel_name", "kernel_kind", "soc_version",
+                "block_dim", "workspace_size", "cycle_count", "elapsed_us", "score", "validation_passed",
+                "artifact_root", "inputs", "outputs", "tiling"):
+        assert key in trace, key
+    assert trace["schema_version"] == 1 and trace["backend"] == "hip" and trace["session_id"] == sid
+    assert trace["task_id"] == "main" and trace["kernel_name"] == "example" and trace["kernel_kind"] == "vec"
+    assert trace["block_dim"] == 3 and trace["workspace_size"] == 64
+    assert trace["score"] == trace["cycle_count"] == 12500 and trace["elapsed_us"] == 13
+    assert trace["inputs"] == [{"name": "a", "shape": [4, 4], "dtype": "f32"},
+                               {"name": "b", "shape": [4, 4], "dtype": "f32"}]
+    assert trace["outputs"] == [{"name": "out", "shape": [4, 4], "dtype": "f32"}]
+    assert trace["tiling"]["present"] is True and trace["tiling"]["bytes"] == 48
+    assert open(trace["tiling"]["binary_path"], "rb").read() == struct.pack("<6q", *[4] * 6)
+    summary = json.loads(open(kv["session.profile.summary"]).read())
+    assert summary["schema_version"] == 1 and summary["session_id"] == sid and summary["backend"] == "hip"
+    assert summary["task_count"] == summary["successful_task_count"] == 1 and summary["failed_task_count"] == 0
+    assert summary["tasks"] == [{"task_id": "main", "profile_path": retained, "score": 12500, "cycle_count": 12500}]
+    assert summary["total_score"] == summary["total_cycle_count"] == 12500
+    assert summary["runtime"]["counters"]["kernel_ns"] == 12500
+    assert summary["runtime"]["attributes"]["kernel_name"] == "example"
+    # without "profiling" nothing is written
+    p = subprocess.run([RS, "--run-manifest", _manifest(tmp_path), "--run", "--testing-driver=hip-success"],
+                       capture_output=True, text=True, env=dict(os.environ, TMPDIR=str(tmp)))
+    assert "session.profile.count=0" in p.stdout.splitlines() and "session.profile.summary" not in p.stdout
