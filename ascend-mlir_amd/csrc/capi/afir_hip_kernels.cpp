@@ -581,6 +581,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
     if (compiled) {
       const int segment = (int)(&seg - res.segments.data());
       const afir_target::SpecShape shape = afir_target::specShape(r->program, segment);
+      const afir_target::SpecTile tile = afir_target::specTile(r->program, segment);
       const int W = shape.width, U = shape.unroll;
       afir::RegionGeometry g;
       uint32_t rc = finish(afir::plan_fused_region(a, W * U, block_dim, &g));
@@ -594,10 +595,25 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
       sa.out_vec = a.out_vec;
       sa.lanes_log2 = g.lanes_log2;
       sa.grid = (int)g.blocks;
-      // the aligned variant has no tail handling: whole groups, whole passes
-      const int64_t groups = seg.size[last] / W;
-      const int64_t per_pass = (seg.reduce ? (int64_t)64 : ((int64_t)1 << g.lanes_log2)) * U;
-      bool all_aligned = seg.size[last] % W == 0 && groups % per_pass == 0 && (seg.reduce || a.out_vec);
+      bool all_aligned;
+      if (tile.tiled) {
+        // one workgroup pass per tile of kTileP x kTileQ
+        const int64_t tq = (seg.size[last] + afir_target::kTileQ - 1) / afir_target::kTileQ;
+        const int64_t tp = (seg.size[tile.dim] + afir_target::kTileP - 1) / afir_target::kTileP;
+        int64_t tiles = tq * tp;
+        for (int k = 0; k < last; ++k)
+          if (k != tile.dim) tiles *= seg.size[k];
+        int64_t blocks = tiles < (int64_t)afir::kNumCU * 8 ? tiles : (int64_t)afir::kNumCU * 8;
+        if (block_dim) blocks = block_dim;
+        sa.grid = (int)blocks;
+        all_aligned = seg.size[last] % afir_target::kTileQ == 0 && seg.size[tile.dim] % afir_target::kTileP == 0 &&
+                      a.out_vec;
+      } else {
+        // the aligned variant has no tail handling: whole groups, whole passes
+        const int64_t groups = seg.size[last] / W;
+        const int64_t per_pass = (seg.reduce ? (int64_t)64 : ((int64_t)1 << g.lanes_log2)) * U;
+        all_aligned = seg.size[last] % W == 0 && groups % per_pass == 0 && (seg.reduce || a.out_vec);
+      }
       for (int i = 0; i < a.ninputs; ++i) {
         const afir::RegionInput &d = a.in[i];
         afir_target::SpecInput &t = sa.in[i];
@@ -609,6 +625,16 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
         t.gextent = d.gextent;
         t.vec = d.vec;
         t.gvec = d.gvec;
+        if (tile.tiled && ((tile.inputs >> i) & 1u)) {
+          // staged through LDS: 128-bit loads run along the tile dim
+          const int64_t es = (int64_t)afir_region::elemTypeBytes(seg.inputs[i].type);
+          bool tvec = aligned(d.base, d.offset * es);
+          for (int k = 0; k < seg.rank; ++k)
+            if (k != tile.dim && seg.size[k] > 1 && (d.stride[k] * es) % 16 != 0) tvec = false;
+          t.vec = tvec ? 1 : 0;
+          if (!tvec) all_aligned = false;
+          continue;
+        }
         // operands that are contiguous along the innermost dim are read with
         // 128-bit loads by the aligned variant
         if (d.stride[last] == 1 && d.gdim != last && (!d.vec || (d.gdim >= 0 && !d.gvec))) all_aligned = false;

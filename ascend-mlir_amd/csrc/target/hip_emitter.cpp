@@ -189,6 +189,11 @@ struct Operand {
   ElemType gatherType = ElemType::I64;
   bool usesDim[kMaxRank] = {false, false, false};
   bool readOnce = false;   // every iteration dim addresses it: no reuse across the launch
+  // Strided along the innermost iteration dim but contiguous along another one
+  // (a transposed read): staged through an LDS tile when the segment is tiled.
+  int contiguousDim = -1;  // the iteration dim the operand's innermost dim follows, else -1
+  bool tiled = false;
+  int tileSlot = 0;        // which LDS tile
 };
 
 bool sameRead(const Op &a, const Op &b) {
@@ -204,6 +209,8 @@ bool sameRead(const Op &a, const Op &b) {
       return false;
   return true;
 }
+
+constexpr int kMaxTiles = 2;
 
 struct Value {
   std::string name;
@@ -222,15 +229,17 @@ class SegmentEmitter {
   std::string run() {
     if (!seg_.ops.empty() && seg_.ops[0].code == OpCode::Matmul)
       return "matmul segments run on the hand-written MFMA kernels";
-    rank_ = seg_.rank;
-    last_ = rank_ - 1;
-    reduce_ = seg_.reduces();
     const SpecShape shape = specShape(p_, index_);
     W_ = shape.width;
     U_ = shape.unroll;
-    collectOperands();
+    analyze();
     if ((int)pushSlot_.size() > kSpecMaxInputs) return "more than 8 operand reads in a segment";
-    emitBody();
+    if (tiled()) {
+      U_ = kTileQ / 8 / W_;   // eight lanes cover a tile row
+      emitBodyTiled();
+    } else {
+      emitBody();
+    }
     emitWrappers();
     return "";
   }
@@ -265,6 +274,13 @@ class SegmentEmitter {
         }
         o.step = lastHits == 0 ? Operand::Broadcast
                                : (lastHits == 1 && lastInnermost ? Operand::Contiguous : Operand::Strided);
+        if (o.step == Operand::Strided && lastHits == 1 && o.gatherDim < 0 && !op.map.empty() &&
+            op.map.back().kind == MapResult::IterDim && op.map.back().iterDim != last_) {
+          int hits = 0;
+          for (const MapResult &m : op.map)
+            if (m.kind == MapResult::IterDim && m.iterDim == op.map.back().iterDim) ++hits;
+          if (hits == 1) o.contiguousDim = op.map.back().iterDim;
+        }
         o.readOnce = true;
         for (int k = 0; k < rank_; ++k)
           if (!o.usesDim[k] && o.gatherDim != k) o.readOnce = false;
@@ -276,8 +292,38 @@ class SegmentEmitter {
       pushSlot_.push_back(found);
       ++slot;
     }
+    // a parallel segment with transposed reads is walked in tiles of
+    // kTileP x kTileQ over (that dim, innermost dim); up to two such operands
+    // go through LDS, all along the same dim
+    tileDim_ = -1;
+    int tiles = 0;
+    if (!reduce_)
+      for (Operand &o : operands_)
+        if (o.contiguousDim >= 0 && (tileDim_ < 0 || tileDim_ == o.contiguousDim) && tiles < kMaxTiles) {
+          tileDim_ = o.contiguousDim;
+          o.tiled = true;
+          o.tileSlot = tiles++;
+        }
+    numTiles_ = tiles;
   }
 
+ public:
+  bool tiled() const { return tileDim_ >= 0; }
+  int tileDim() const { return tileDim_; }
+  unsigned tiledInputs() const {
+    unsigned mask = 0;
+    for (const Operand &o : operands_)
+      if (o.tiled) mask |= 1u << o.slot;
+    return mask;
+  }
+  void analyze() {
+    rank_ = seg_.rank;
+    last_ = rank_ - 1;
+    reduce_ = seg_.reduces();
+    collectOperands();
+  }
+
+ private:
   std::string in(const Operand &o) const { return "R.in[" + std::to_string(o.slot) + "]"; }
   std::string id(const Operand &o) const { return std::to_string(o.slot); }
   void line(int depth, const std::string &text) { os_ << std::string(2 * depth, ' ') << text << "\n"; }
@@ -320,6 +366,15 @@ class SegmentEmitter {
     }
     v.name = "v" + u;
     line(d, "float v" + u + "[U][W];");
+    if (o.tiled) {
+      unroll();
+      line(d, "for (int u = 0; u < U; ++u)");
+      unroll();
+      line(d + 1, "for (int e = 0; e < W; ++e)");
+      line(d + 2, "v" + u + "[u][e] = e < nvalid[u] ? tile[" + std::to_string(o.tileSlot) +
+                      "][((int)(j0[u] - tile_q) + e) * PITCH + pl] : 0.f;");
+      return v;
+    }
     const std::string nan = "as_f32(0x7fc00000u)";
     if (o.gatherDim == last_) {
       // one index per element
@@ -483,13 +538,13 @@ class SegmentEmitter {
 
   // j0 / nvalid / full of the U groups of a pass that starts at group `first`
   // with `lanes` lanes on the row.
-  void emitGroups(int d, const std::string &first, const std::string &lanes) {
+  void emitGroups(int d, const std::string &first, const std::string &lanes, const std::string &base = "") {
     line(d, "I j0[U];");
     line(d, "int nvalid[U];");
     line(d, "bool full[U];");
     unroll();
     line(d, "for (int u = 0; u < U; ++u) {");
-    line(d + 1, "j0[u] = (" + first + " + (I)u * " + lanes + ") * W;");
+    line(d + 1, "j0[u] = " + (base.empty() ? std::string() : base + " + ") + "(" + first + " + (I)u * " + lanes + ") * W;");
     line(d + 1, "const I left = n - j0[u];");
     line(d + 1, "nvalid[u] = (A || left >= W) ? W : (left > 0 ? (int)left : 0);");
     line(d + 1, "full[u] = A || nvalid[u] == W;");
@@ -588,6 +643,108 @@ class SegmentEmitter {
     os_ << "}\n";
   }
 
+  // Parallel segment with transposed reads: a workgroup takes a tile of kTileP
+  // (the dim those operands are contiguous along) x kTileQ (the innermost
+  // iteration dim).  Phase 1 loads each transposed operand's tile with 128-bit
+  // loads along ITS contiguous dim and writes it to LDS as float32, rows padded
+  // by one word; phase 2 is the ordinary row code, 8 lanes per row, reading
+  // those operands from LDS column-wise (conflict-free with the odd pitch).
+  void emitBodyTiled() {
+    const std::string otag = typeTag(p_.output().type);
+    const int p = tileDim_, r = rank_ == 3 ? (p == 0 ? 1 : 0) : -1;
+    const std::string P = std::to_string(p), L = std::to_string(last_);
+    os_ << "\n// ---- segment " << index_ << ": iteration rank " << rank_ << ", parallel, tiles of " << kTileP
+        << " (dim " << p << ") x " << kTileQ << " (dim " << last_ << ") through LDS; a lane takes " << U_
+        << " groups of " << W_ << " elements per row ----\n";
+    os_ << "// I: position type.  A: every 128-bit access is aligned and every tile is whole.\n";
+    os_ << "template <typename I, bool A>\nDEV void segment" << index_
+        << "(const SpecArgs &R, const I bid, const I nblocks) {\n";
+    line(1, "constexpr int W = " + std::to_string(W_) + ", U = " + std::to_string(U_) + ";");
+    line(1, "constexpr int TP = " + std::to_string(kTileP) + ", TQ = " + std::to_string(kTileQ) + ", PITCH = TP + 1;");
+    line(1, "static_assert(8 * U * W == TQ, \"eight lanes cover a tile row\");");
+    line(1, "__attribute__((shared)) static float tile[" + std::to_string(numTiles_) + "][TQ * PITCH];");
+    line(1, "const int tid = (int)__builtin_amdgcn_workitem_id_x();");
+    line(1, "const I n = (I)R.size[" + L + "];");
+    line(1, "const I np = (I)R.size[" + P + "];");
+    line(1, "const I tiles_q = (n + (TQ - 1)) / TQ, tiles_p = (np + (TP - 1)) / TP;");
+    line(1, std::string("const I ntiles = tiles_q * tiles_p") + (r >= 0 ? " * (I)R.size[" + std::to_string(r) + "]" : "") + ";");
+    for (const Operand &o : operands_)
+      if (o.step != Operand::Broadcast && o.gatherDim != last_)
+        line(1, "const bool vec" + id(o) + " = " + in(o) + ".vec != 0" + (o.gatherDim >= 0 ? " && " + in(o) + ".gvec != 0" : "") + ";");
+    line(1, "for (I t = bid; t < ntiles; t += nblocks) {");
+    line(2, "const I tq = t % tiles_q, rest = t / tiles_q;");
+    line(2, "const I tp = rest % tiles_p;");
+    if (r >= 0) line(2, "const I x" + std::to_string(r) + " = rest / tiles_p;");
+    line(2, "const I tile_p = tp * TP, tile_q = tq * TQ;");
+    for (const Operand &o : operands_) {
+      if (!o.tiled) continue;
+      const std::string u = id(o), rr = in(o), tag = typeTag(o.type);
+      const int el = o.type == ElemType::F32 ? 4 : 8;
+      line(2, "{  // operand " + u + ": " + std::to_string(kTileQ) + " runs of " + std::to_string(kTileP) + " elements along dim " + P);
+      line(3, "constexpr int EL = " + std::to_string(el) + ", LPR = TP / EL, RPP = 256 / LPR, NP = TQ / RPP;");
+      line(3, "const int lp = (tid % LPR) * EL, lq = tid / LPR;");
+      line(3, "const long long pos = (long long)" + rr + ".offset" +
+                  (r >= 0 && o.usesDim[r] ? " + (long long)x" + std::to_string(r) + " * " + rr + ".stride[" + std::to_string(r) + "]" : "") +
+                  " + (long long)(tile_p + lp);");
+      line(3, "const long long sq = " + rr + ".stride[" + L + "];");
+      line(3, "float vals[NP][EL];");
+      unroll();
+      line(3, "for (int s = 0; s < NP; ++s) {");
+      line(4, "const I q = tile_q + (I)(lq + s * RPP);");
+      line(4, "if (A || (vec" + u + " && q < n && tile_p + (I)(lp + EL) <= np)) {");
+      line(5, "ldv_" + tag + "<EL, " + (o.readOnce ? "true" : "false") + ">(" + rr + ".base, pos + (long long)q * sq, vals[s]);");
+      line(4, "} else {");
+      unroll();
+      line(5, "for (int e = 0; e < EL; ++e)");
+      line(6, "vals[s][e] = (q < n && tile_p + (I)(lp + e) < np) ? ld_" + tag + "(" + rr + ".base, pos + (long long)q * sq + e) : 0.f;");
+      line(4, "}");
+      line(3, "}");
+      unroll();
+      line(3, "for (int s = 0; s < NP; ++s)");
+      unroll();
+      line(4, "for (int e = 0; e < EL; ++e) tile[" + std::to_string(o.tileSlot) + "][(lq + s * RPP) * PITCH + lp + e] = vals[s][e];");
+      line(2, "}");
+    }
+    line(2, "__builtin_amdgcn_fence(__ATOMIC_RELEASE, \"workgroup\");");
+    line(2, "__builtin_amdgcn_s_barrier();");
+    line(2, "__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, \"workgroup\");");
+    unroll();
+    line(2, "for (int pp = 0; pp < TP / 32; ++pp) {");
+    line(3, "const int pl = (tid >> 3) + 32 * pp;");
+    line(3, "const I x" + P + " = tile_p + (I)pl;");
+    line(3, "if (A || x" + P + " < np) {");
+    if (rank_ == 2) line(4, "const I row = x0;");
+    else line(4, "const I row = x0 * (I)R.size[1] + x1;");
+    emitRowInvariants(4);
+    emitGroups(4, "(I)(tid & 7)", "(I)8", "tile_q");
+    const Value v = emitExpression(4);
+    std::string res = v.name;
+    if (v.scalar) {
+      line(4, "float splat[U][W];");
+      unroll();
+      line(4, "for (int u = 0; u < U; ++u)");
+      unroll();
+      line(5, "for (int e = 0; e < W; ++e) splat[u][e] = " + v.name + ";");
+      res = "splat";
+    }
+    unroll();
+    line(4, "for (int u = 0; u < U; ++u) {");
+    line(5, "const long long o = (long long)row * (long long)n + (long long)j0[u];");
+    line(5, "if (A || (full[u] && R.out_vec)) {");
+    line(6, "stv_" + otag + "<W>(R.out, o, " + res + "[u]);");
+    line(5, "} else {");
+    unroll();
+    line(6, "for (int e = 0; e < W; ++e)");
+    line(7, "if (e < nvalid[u]) st_" + otag + "(R.out, o + e, " + res + "[u][e]);");
+    line(5, "}");
+    line(4, "}");
+    line(3, "}");
+    line(2, "}");
+    line(2, "__builtin_amdgcn_s_barrier();   // the tile is reused by the next iteration");
+    line(1, "}");
+    os_ << "}\n";
+  }
+
   void emitWrappers() {
     for (int i32 = 1; i32 >= 0; --i32)
       for (int a = 1; a >= 0; --a)
@@ -602,6 +759,7 @@ class SegmentEmitter {
   int index_;
   std::ostringstream &os_;
   int rank_ = 0, last_ = 0, W_ = 8, U_ = 2;
+  int tileDim_ = -1, numTiles_ = 0;
   bool reduce_ = false;
   std::vector<Operand> operands_;
   std::vector<int> pushSlot_;   // per push, in order: index into operands_
@@ -618,6 +776,28 @@ SpecShape specShape(const Program &p, int segment) {
   s.width = any16 ? 8 : 4;            // 16 bytes of the narrowest tensor
   s.unroll = (any16 && any32) ? 2 : 4;
   return s;
+}
+
+SpecTile specTile(const Program &p, int segment) {
+  std::ostringstream sink;
+  SegmentEmitter e(p, segment, sink);
+  e.analyze();
+  SpecTile t;
+  t.tiled = e.tiled();
+  t.dim = e.tileDim();
+  t.inputs = e.tiledInputs();
+  return t;
+}
+
+bool specAllSegments(const Program &p) {
+  const int nseg = (int)p.segments.size();
+  if (nseg < 2 || nseg > kSpecMaxSegments) return false;
+  for (int s = 0; s < nseg; ++s) {
+    const Segment &g = p.segments[s];
+    if (!g.ops.empty() && g.ops[0].code == OpCode::Matmul) return false;
+    if (specTile(p, s).tiled) return false;   // LDS tiles of several segments would add up
+  }
+  return true;
 }
 
 uint64_t programHash(const Program &p) {
@@ -660,7 +840,7 @@ std::string emitHipSource(const Program &p, const std::string &title, std::strin
     if (std::string why = e.run(); !why.empty()) return why;
   }
   const int nseg = (int)p.segments.size();
-  if (nseg > 1 && nseg <= kSpecMaxSegments) {
+  if (specAllSegments(p)) {
     // every segment in one launch: the workgroups are dealt out segment by segment
     os << "\n// ---- all segments in one launch ----\n";
     os << "struct SpecAll {\n  int first[" << kSpecMaxSegments + 1 << "];   // first workgroup of each segment, then the total\n"

@@ -59,6 +59,20 @@ struct SpecAll {
   SpecArgs seg[kSpecMaxSegments];    // the emitted declaration holds the program's segment count
 };
 std::string specAllKernelName(bool idx32, bool aligned);
+bool specAllSegments(const afir_region::Program &p);   // whether that kernel is emitted
+
+// A parallel segment that reads an operand transposed (contiguous along an
+// outer iteration dim `dim`, strided along the innermost one) is walked in
+// tiles of kTileP (dim) x kTileQ (innermost dim), the transposed operands
+// staged through LDS; the launch then has one workgroup pass per tile.
+constexpr int kTileP = 64, kTileQ = 128;
+struct SpecTile {
+  bool tiled = false;
+  int dim = -1;
+  unsigned inputs = 0;   // bit i: SpecArgs::in[i] is staged through LDS; its `vec` flag then
+                         // means "128-bit loads along `dim` are aligned"
+};
+SpecTile specTile(const afir_region::Program &p, int segment);
 
 // A lane's share of one pass over a row: `unroll` groups of `width` consecutive
 // elements (16 bytes of the narrowest tensor), the groups one lane-set apart.
