@@ -157,28 +157,34 @@ std::string detect_fast_path(RegisteredRegion *r) {
   const bool hasMatmul = !ops.empty() && ops[0].code == OpCode::Matmul;
 
   if (hasMatmul) {
-    // [matmul A B, push bias (d1), add, leaky alpha, store]
-    if (ops.size() == 5 && is_push(ops[1], 2, {1}) && ops[2].code == OpCode::Add &&
-        ops[3].code == OpCode::Leaky && ops[4].code == OpCode::Store) {
-      const int a = ops[0].arg, b = ops[0].arg2, bias = ops[1].arg;
-      if (type(a) == ElemType::BF16 && type(b) == ElemType::BF16 && type(bias) == ElemType::BF16 &&
+    // [matmul A B, (push bias (d1), add)?, (leaky alpha)?, store]: the epilogue kinds None, BiasAdd and
+    // BiasAddLeakyRelu of lib/Conversion/MarkStructuredOps/AnnotateMixMatmulSemanticsPass.cpp:319-323
+    // (and leaky relu without a bias)
+    size_t at = 1;
+    int bias = -1;
+    float alpha = 1.f;   // max(v, v * 1) is v
+    if (at + 1 < ops.size() && is_push(ops[at], 2, {1}) && ops[at + 1].code == OpCode::Add) {
+      bias = ops[at].arg;
+      at += 2;
+    }
+    if (at < ops.size() && ops[at].code == OpCode::Leaky) alpha = ops[at++].constant;
+    if (at + 1 == ops.size() && ops[at].code == OpCode::Store) {
+      const int a = ops[0].arg, b = ops[0].arg2;
+      if (type(a) == ElemType::BF16 && type(b) == ElemType::BF16 && (bias < 0 || type(bias) == ElemType::BF16) &&
           out == ElemType::BF16) {
         r->fast = FastPath::MatmulBiasLeaky;
-        r->fastArgs[0] = a; r->fastArgs[1] = b; r->fastArgs[2] = bias;
-        r->alpha = ops[3].constant;
-        return "";
-      }
-      if (type(a) == ElemType::F16 && type(b) == ElemType::F16 && type(bias) == ElemType::F32 &&
-          out == ElemType::F32) {
+      } else if (type(a) == ElemType::F16 && type(b) == ElemType::F16 && (bias < 0 || type(bias) == ElemType::F32) &&
+                 out == ElemType::F32) {
         r->fast = FastPath::MatmulBiasLeakyF16;
-        r->fastArgs[0] = a; r->fastArgs[1] = b; r->fastArgs[2] = bias;
-        r->alpha = ops[3].constant;
-        return "";
+      } else {
+        return "matmul regions are implemented for bf16 A, B, bias, out and for f16 A, B with f32 bias, out; "
+               "this one has other types";
       }
-      return "matmul regions are implemented for bf16 A, B, bias, out and for f16 A, B with f32 bias, out; "
-             "this one has other types";
+      r->fastArgs[0] = a; r->fastArgs[1] = b; r->fastArgs[2] = bias;
+      r->alpha = alpha;
+      return "";
     }
-    return "a matmul region must be matmul -> bias add (per column) -> leaky relu; other epilogues are not implemented";
+    return "a matmul region must be matmul [-> bias add (per column)] [-> leaky relu]; other epilogues are not implemented";
   }
   if (g.rank == 2 && ops.size() == 6 && out == ElemType::F32 && is_push(ops[0], 2, {0, 1}) &&
       is_push(ops[1], 2, {0, 1}) && ops[2].code == OpCode::Add && is_push(ops[3], 2, {0, 1}) &&
@@ -343,6 +349,8 @@ uint32_t afir_hip_launch_matmul_add_leakyrelu(uint32_t block_dim, void *stream, 
   int64_t f[4];
   if (!read_fields(tiling, 4, f))
     return fail(AFIR_HIP_E_INVALID, "matmul_add_leakyrelu: null tiling");
+  if (!bias && f[0] != 0 && f[2] != 0)   // (the region route takes a null bias as "no bias")
+    return fail(AFIR_HIP_E_INVALID, "matmul_add_leakyrelu: null tensor pointer");
   const uint32_t bits = (uint32_t)((uint64_t)f[3] & 0xffffffffu);
   float alpha;
   std::memcpy(&alpha, &bits, 4);
@@ -505,13 +513,13 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
       case FastPath::MatmulBiasLeaky:
         return finish(afir::launch_matmul_add_leakyrelu(
             static_cast<const uint16_t *>(args[fa[0]]), static_cast<const uint16_t *>(args[fa[1]]),
-            static_cast<const uint16_t *>(args[fa[2]]), static_cast<uint16_t *>(out), seg.size[0],
-            res.shapes[fa[0]][1], seg.size[1], r->alpha, block_dim, st));
+            fa[2] >= 0 ? static_cast<const uint16_t *>(args[fa[2]]) : nullptr, static_cast<uint16_t *>(out),
+            seg.size[0], res.shapes[fa[0]][1], seg.size[1], r->alpha, block_dim, st));
       case FastPath::MatmulBiasLeakyF16:
         return finish(afir::launch_matmul_add_leakyrelu_f16(
             static_cast<const uint16_t *>(args[fa[0]]), static_cast<const uint16_t *>(args[fa[1]]),
-            static_cast<const float *>(args[fa[2]]), static_cast<float *>(out), seg.size[0],
-            res.shapes[fa[0]][1], seg.size[1], r->alpha, block_dim, st));
+            fa[2] >= 0 ? static_cast<const float *>(args[fa[2]]) : nullptr, static_cast<float *>(out),
+            seg.size[0], res.shapes[fa[0]][1], seg.size[1], r->alpha, block_dim, st));
       case FastPath::None: break;
     }
   }

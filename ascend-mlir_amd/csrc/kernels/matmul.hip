@@ -188,7 +188,9 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void matmul_bias_leakyrelu_m
       for (int q = 0; q < 4; ++q) {
         const int n = n0 + (wn * TN + j) * 32 + 8 * q + 4 * lq;
         float b0, b1, b2, b3;
-        if constexpr (F16IO) {
+        if (!bias_v) {
+          b0 = b1 = b2 = b3 = -0.f;   // no bias: x + (-0) is x for every x, signed zeros included
+        } else if constexpr (F16IO) {
           const f32x4 bf = *reinterpret_cast<const f32x4 *>(static_cast<const float *>(bias_v) + n);
           b0 = bf[0]; b1 = bf[1]; b2 = bf[2]; b3 = bf[3];
         } else {
@@ -248,10 +250,10 @@ __global__ __launch_bounds__(256) void matmul_bias_leakyrelu_any(
     }
     if (m < M && n < N) {
       if constexpr (F16IO) {
-        float v = acc + static_cast<const float *>(bias_v)[n];
+        float v = acc + (bias_v ? static_cast<const float *>(bias_v)[n] : -0.f);
         static_cast<float *>(out_v)[(int64_t)m * N + n] = fmaxf(v, v * alpha);
       } else {
-        float v = acc + __uint_as_float((uint32_t) static_cast<const uint16_t *>(bias_v)[n] << 16);
+        float v = acc + (bias_v ? __uint_as_float((uint32_t) static_cast<const uint16_t *>(bias_v)[n] << 16) : -0.f);
         v = fmaxf(v, v * alpha);
         static_cast<uint16_t *>(out_v)[(int64_t)m * N + n] = (uint16_t)f32_to_bf16_rne(v);
       }
@@ -288,7 +290,7 @@ LaunchStatus launch_matmul_any_io(const uint16_t *a, const uint16_t *b, const vo
                                   hipStream_t stream) {
   if (m < 0 || k < 0 || n < 0) return invalid("matmul_add_leakyrelu: negative extent");
   if (m == 0 || n == 0) return ok_status();
-  if (!out || !bias) return invalid("matmul_add_leakyrelu: null tensor pointer");
+  if (!out) return invalid("matmul_add_leakyrelu: null tensor pointer");   // a null bias means "no bias"
   if (k > 0 && (!a || !b)) return invalid("matmul_add_leakyrelu: null input matrix");
   if (m > 0x7fffffff || n > 0x7fffffff || k > 0x7fffffff)
     return invalid("matmul_add_leakyrelu: extent exceeds 2^31-1");

@@ -353,7 +353,8 @@ __global__ __launch_bounds__(WM * WN * 64) void matmul_bias_leakyrelu_bf16_dma(
       for (int j = 0; j < TNW; ++j)
 #pragma unroll
         for (int q = 0; q < 4; ++q)
-          braw[j][q] = *reinterpret_cast<const u32x2 *>(bias + n0 + (wn * TNW + j) * 32 + 8 * q + 4 * lq);
+          braw[j][q] = bias ? *reinterpret_cast<const u32x2 *>(bias + n0 + (wn * TNW + j) * 32 + 8 * q + 4 * lq)
+                            : u32x2{0x80008000u, 0x80008000u};   // no bias: -0, the identity of the add
 #pragma unroll
       for (int i = 0; i < TMW; ++i) {
 #pragma unroll

@@ -142,6 +142,38 @@ func.func @mm_bias_leaky(%a : tensor<?x?xf16>, %b : tensor<?x?xf16>, %bias : ten
 MATMUL_BIAS_LEAKY_BF16 = MATMUL_BIAS_LEAKY_F16.replace("xf16", "xbf16").replace("f32", "bf16") \
     .replace("1.0e-3", "1.0e-2").replace("@mm_bias_leaky", "@mm_bias_leaky_bf16")
 
+# The other epilogue kinds the reference's matmul annotation knows
+# (test/Conversion/annotate-mix-matmul-semantics.mlir:3-25: "None", "BiasAdd").
+MATMUL_PLAIN_F16 = """
+func.func @mm_plain(%a : tensor<?x?xf16>, %b : tensor<?x?xf16>, %init : tensor<?x?xf32>) -> tensor<?x?xf32> {
+  %c = linalg.matmul ins(%a, %b : tensor<?x?xf16>, tensor<?x?xf16>) outs(%init : tensor<?x?xf32>) -> tensor<?x?xf32>
+  return %c : tensor<?x?xf32>
+}
+"""
+
+MATMUL_BIAS_F16 = """
+#bias = affine_map<(d0, d1) -> (d1)>
+#all = affine_map<(d0, d1) -> (d0, d1)>
+func.func @mm_bias(%a : tensor<?x?xf16>, %b : tensor<?x?xf16>, %bias : tensor<?xf32>,
+                   %init : tensor<?x?xf32>) -> tensor<?x?xf32> {
+  %c0 = arith.constant 0 : index
+  %c1 = arith.constant 1 : index
+  %m = tensor.dim %init, %c0 : tensor<?x?xf32>
+  %n = tensor.dim %init, %c1 : tensor<?x?xf32>
+  %c = linalg.matmul ins(%a, %b : tensor<?x?xf16>, tensor<?x?xf16>) outs(%init : tensor<?x?xf32>) -> tensor<?x?xf32>
+  %e0 = tensor.empty(%m, %n) : tensor<?x?xf32>
+  %d = linalg.generic {indexing_maps = [#all, #bias, #all], iterator_types = ["parallel", "parallel"]}
+      ins(%c, %bias : tensor<?x?xf32>, tensor<?xf32>) outs(%e0 : tensor<?x?xf32>) {
+    ^bb0(%x: f32, %y: f32, %o: f32):
+      %s = arith.addf %x, %y : f32
+      linalg.yield %s : f32
+  } -> tensor<?x?xf32>
+  return %d : tensor<?x?xf32>
+}
+"""
+MATMUL_PLAIN_BF16 = MATMUL_PLAIN_F16.replace("xf16", "xbf16").replace("f32", "bf16").replace("@mm_plain", "@mm_plain_bf16")
+MATMUL_BIAS_BF16 = MATMUL_BIAS_F16.replace("xf16", "xbf16").replace("f32", "bf16").replace("@mm_bias", "@mm_bias_bf16")
+
 TWO_CHAINS_CONCAT = """
 #row = affine_map<(d0, d1) -> (d0)>
 #all = affine_map<(d0, d1) -> (d0, d1)>

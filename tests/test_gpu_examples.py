@@ -223,3 +223,45 @@ def test_two_kernel_session_feeds_one_kernel_into_the_next(tmp_path):
     assert "session.result=success" in lines and "session.validation=pass" in lines
     assert np.load(tmp_path / "chain__t.npy").tobytes() == t.tobytes()      # the intermediate is bit-exact
     assert np.allclose(np.load(tmp_path / "y.npy"), want, rtol=1e-5, atol=1e-3)
+
+
+@pytest.mark.parametrize("kind", ["none", "bias"])
+@pytest.mark.parametrize("ty", ["f16", "bf16"])
+def test_matmul_epilogue_kinds(pkg, kind, ty):
+    """matmul with no epilogue and with a bias add only (the reference's epilogue
+    kinds "None" and "BiasAdd") on the MFMA kernels.  Small-integer operands:
+    every product and partial sum is exact in float32
+    (examples/matmul-add-leakyrelu/gen_data.py:29-31), so the result does not
+    depend on the order of accumulation; negative sums keep their sign without a
+    leaky relu.  bf16 at 512x512x256 takes the direct-to-LDS kernel."""
+    import torch
+    from ascend_mlir_amd import hip_kernels as H
+    from oracle import region_oracle as RO
+    H.load()
+    mlir = {("none", "f16"): MC.MATMUL_PLAIN_F16, ("bias", "f16"): MC.MATMUL_BIAS_F16,
+            ("none", "bf16"): MC.MATMUL_PLAIN_BF16, ("bias", "bf16"): MC.MATMUL_BIAS_BF16}[(kind, ty)]
+    p = subprocess.run([TR, "-mlir-to-hip", "-"], input=mlir, capture_output=True, text=True)
+    assert p.returncode == 0, p.stderr
+    for (m, k, n) in ((512, 256, 512), (96, 64, 40)):
+        rng = np.random.default_rng(7)
+        a = rng.integers(-3, 4, (m, k)).astype(np.float32)
+        b = rng.integers(-3, 4, (k, n)).astype(np.float32)
+        bias = rng.integers(-8, 9, (n,)).astype(np.float32)
+        exact = a @ b + (bias[None, :] if kind == "bias" else 0.0)      # integers: exact in float32
+        assert np.abs(exact).max() < 2 ** 24
+        if ty == "f16":
+            ins = [a.astype(np.float16), b.astype(np.float16)] + ([bias] if kind == "bias" else [])
+            init = np.zeros((m, n), np.float32)
+            want = exact.astype(np.float32)
+            dev = [torch.from_numpy(x).cuda() for x in ins + [init]]
+        else:
+            ins = [O.f32_to_bf16_bits(a), O.f32_to_bf16_bits(b)] + ([O.f32_to_bf16_bits(bias)] if kind == "bias" else [])
+            init = O.f32_to_bf16_bits(np.zeros((m, n), np.float32))
+            want = O.f32_to_bf16_bits(exact.astype(np.float32))
+            dev = [torch.from_numpy(x.view(np.int16)).cuda().view(torch.bfloat16) for x in ins + [init]]
+        assert RO.evaluate(p.stdout, ins + [init]).tobytes() == want.tobytes()      # the oracle agrees with the closed form
+        r = H.Region(p.stdout)
+        out = r(*dev, out_shape=(m, n))
+        got = out.cpu().numpy() if ty == "f16" else out.view(torch.int16).cpu().numpy().view(np.uint16)
+        r.close()
+        assert got.tobytes() == want.tobytes(), (kind, ty, m, k, n)

@@ -63,6 +63,28 @@ def test_benchmark_graphs_route_to_the_hand_tuned_kernels(pkg):
         r.close()
 
 
+def test_matmul_epilogue_kinds_none_and_bias_add(pkg):
+    """The reference annotates matmul regions with the epilogue kinds None,
+    BiasAdd and BiasAddLeakyRelu
+    (lib/Conversion/MarkStructuredOps/AnnotateMixMatmulSemanticsPass.cpp:319-323);
+    all three become a matmul program on the MFMA kernels."""
+    from ascend_mlir_amd import hip_kernels as H
+    for mlir, tail in ((MC.MATMUL_PLAIN_F16, ["matmul arg0 arg1", "store", "end"]),
+                       (MC.MATMUL_BIAS_F16, ["matmul arg0 arg1", "push arg2 d1", "add", "store", "end"]),
+                       (MC.MATMUL_PLAIN_BF16, ["matmul arg0 arg1", "store", "end"]),
+                       (MC.MATMUL_BIAS_BF16, ["matmul arg0 arg1", "push arg2 d1", "add", "store", "end"])):
+        out = program_of(mlir)
+        body = [l.strip() for l in out.splitlines() if l.strip() and not l.startswith("#")]
+        assert body[-len(tail):] == tail, out
+        r = H.Region(out)
+        assert r.kernel == ("matmul_add_leakyrelu" if "bf16" in mlir else "matmul_add_leakyrelu_f16")
+        r.close()
+    # an epilogue outside the vocabulary is refused at registration
+    odd = program_of(MC.MATMUL_BIAS_F16).replace("add\n", "mul\n")
+    with pytest.raises(H.AfirHipError, match="other epilogues are not implemented"):
+        H.Region(odd)
+
+
 def test_matmul_epilogue_program_and_alpha():
     out = program_of(MC.MATMUL_BIAS_LEAKY_F16)
     body = [l for l in out.splitlines() if l and not l.startswith(("#", "afir-hip", "arg"))]
