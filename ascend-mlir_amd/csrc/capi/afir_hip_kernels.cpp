@@ -611,7 +611,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
         int64_t tiles = tq * tp;
         for (int k = 0; k < last; ++k)
           if (k != tile.dim) tiles *= seg.size[k];
-        int64_t blocks = tiles < (int64_t)afir::kNumCU * 8 ? tiles : (int64_t)afir::kNumCU * 8;
+        int64_t blocks = tiles < (int64_t)afir::kNumCU * 256 ? tiles : (int64_t)afir::kNumCU * 256;
         if (block_dim) blocks = block_dim;
         sa.grid = (int)blocks;
         all_aligned = seg.size[last] % afir_target::kTileQ == 0 && seg.size[tile.dim] % afir_target::kTileP == 0 &&

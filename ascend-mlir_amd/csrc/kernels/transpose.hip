@@ -5,117 +5,69 @@
 // 1290-1640; golden style examples/relu-broadcast-transpose/gen_inputs.py:34-35:
 // f32 arithmetic, one round-to-nearest-even to f16).
 //
-// HBM-bound: 2 bytes in + 2 bytes out per element.  A workgroup of 256 lanes
-// moves one 128x128 tile:
-//   1. 128-bit global loads along N (16 lanes cover 256 contiguous bytes),
-//      relu + c applied in registers (a lane's column chunk is the same for
-//      all its rows, so its 8 values of c are loaded once), 128-bit LDS
-//      writes;
-//   2. every lane reads one 8x8 block back as eight 128-bit LDS reads,
-//      transposes it in registers with byte permutes, and issues eight
-//      128-bit global stores along M (16 lanes cover 256 contiguous bytes).
-// The LDS tile is 128 rows x 256 B with no padding; the 16-byte chunk column
-// is XOR-ed with (row/8)%16, which makes both the row-wise writes and the
-// block-column reads hit 16 distinct bank groups per 16 lanes.
-// The grid is persistent (a few workgroups per CU); each workgroup issues the
-// loads of its next tile before it stores the current one, so HBM reads and
-// writes overlap instead of alternating in phases.
+// HBM-bound: 2 bytes in + 2 bytes out per element; the kernel for aligned
+// shapes is described at its definition below.
 #include "kernels.h"
 
 namespace afir {
 
 namespace {
 
-#ifndef AFIR_TR_EXTRA_LDS
-#define AFIR_TR_EXTRA_LDS 0
-#endif
-#ifndef AFIR_TR_BLOCKS_PER_CU
-#define AFIR_TR_BLOCKS_PER_CU 5
-#endif
 constexpr int kThreads = 256;
-constexpr int kTile = 128;               // elements per tile edge
-constexpr int kChunksPerRow = kTile / 8;  // 16-byte chunks per LDS row
 
 // max(v, +0) with IEEE-754 maximum semantics: NaN propagates, -0 gives +0.
 __device__ __forceinline__ float relu_keep_nan(float v) { return (v > 0.f) ? v : ((v != v) ? v : 0.f); }
 
-__device__ __forceinline__ uint32_t relu_add_pack(uint32_t packed, float c_lo, float c_hi) {
-  float lo = relu_keep_nan(f16_lo(packed)) + c_lo;
-  float hi = relu_keep_nan(f16_hi(packed)) + c_hi;
-  return pack_f16(lo, hi);
-}
-
-__global__ __launch_bounds__(kThreads) void relu_bcast_add_transpose_f16_tiled(
+// One 64x64 tile per workgroup, one workgroup pass per tile, float32 in LDS:
+// 16.6 KiB of LDS and few registers, so eight workgroups fit a CU and the
+// chip holds 2048 tiles at once.  Phase 1: a lane loads two 16-byte chunks of
+// x rows (a wave covers eight 128-byte runs per load), applies relu and + c
+// (its eight columns are fixed, so c is read once) and writes the float32
+// results to tile[i][j], rows padded to 65 words.  Phase 2: a lane reads eight
+// consecutive i of one j (a column of the padded tile: conflict-free), rounds
+// them to f16 and writes one 16-byte chunk of an output row; eight lanes cover
+// a 128-byte run along M.  Tiles are numbered along M first, so neighbouring
+// workgroups write neighbouring runs of the same output rows.
+constexpr int kSmallTile = 64, kSmallPitch = kSmallTile + 1;
+__global__ __launch_bounds__(kThreads) void relu_bcast_add_transpose_f16_tile64(
     const uint16_t *__restrict__ x, const uint16_t *__restrict__ c, uint16_t *__restrict__ out,
     int nb, int m, int n) {
-  __shared__ u32x4 tile[kTile * kChunksPerRow];  // 32 KiB
-
-  const int tiles_m = m / kTile, tiles_n = n / kTile;
-  const int64_t ntiles = (int64_t)nb * tiles_m * tiles_n;
+  __shared__ float tile[kSmallTile * kSmallPitch];
   const int t = threadIdx.x;
-  const int cc = t & 15;       // chunk column of this lane in the load phase
-  const int row0 = t >> 4;     // first row of this lane in the load phase
-  const int iblk = t & 15;     // 8-row block (along M) in the store phase
-  const int jblk = t >> 4;     // 8-col block (along N) in the store phase
-
-  // Software pipeline over the tiles of this workgroup: the global loads of
-  // the next tile are issued before the current tile is read back from LDS and
-  // stored, so reads and writes to HBM overlap instead of alternating.
-  auto decode = [&](int64_t tile_id, int &b, int &m0, int &n0) {
-    const int tn = (int)(tile_id % tiles_n);
-    const int tm = (int)((tile_id / tiles_n) % tiles_m);
-    b = (int)(tile_id / ((int64_t)tiles_n * tiles_m));
-    m0 = tm * kTile;
-    n0 = tn * kTile;
-  };
-  u32x4 v[8], craw;
-  auto fetch = [&](int64_t tile_id) {
-    int b, m0, n0;
-    decode(tile_id, b, m0, n0);
-    craw = *reinterpret_cast<const u32x4 *>(c + n0 + cc * 8);
-    const uint16_t *xin = x + ((int64_t)b * m + m0) * n + n0 + cc * 8;
+  // 32-bit tile numbers (the launcher checks that they fit): a 64-bit
+  // division costs hundreds of instructions before the first load
+  const unsigned tiles_m = (unsigned)(m / kSmallTile), tiles_n = (unsigned)(n / kSmallTile);
+  const unsigned ntiles = (unsigned)nb * tiles_m * tiles_n;
+  const int lj = (t & 7) * 8, li = t >> 3;        // phase 1: first column, row within a pass of 32
+  const int oi = (t & 7) * 8, oj = t >> 3;        // phase 2: first i of the chunk, j within a pass of 32
+  for (unsigned tile_id = blockIdx.x; tile_id < ntiles; tile_id += gridDim.x) {
+    const unsigned rest = tile_id / tiles_m;
+    const int tm = (int)(tile_id - rest * tiles_m);
+    const int b = (int)(rest / tiles_n);
+    const int tn = (int)(rest - (unsigned)b * tiles_n);
+    const int m0 = tm * kSmallTile, n0 = tn * kSmallTile;
+    const u32x4 craw = *reinterpret_cast<const u32x4 *>(c + n0 + lj);
+    const uint16_t *xin = x + ((int64_t)b * m + m0 + li) * n + n0 + lj;
+    u32x4 v[2];
 #pragma unroll
-    for (int k = 0; k < 8; ++k)
-      v[k] = load_nt(reinterpret_cast<const u32x4 *>(xin + (int64_t)(row0 + 16 * k) * n));
-  };
-
-  int64_t tile_id = blockIdx.x;
-  if (tile_id < ntiles) fetch(tile_id);
-  for (; tile_id < ntiles; tile_id += gridDim.x) {
-    int b, m0, n0;
-    decode(tile_id, b, m0, n0);
-    float cf[8];
+    for (int k = 0; k < 2; ++k) v[k] = load_nt(reinterpret_cast<const u32x4 *>(xin + (int64_t)(32 * k) * n));
 #pragma unroll
-    for (int d = 0; d < 4; ++d) {
-      cf[2 * d] = f16_lo(craw[d]);
-      cf[2 * d + 1] = f16_hi(craw[d]);
-    }
+    for (int k = 0; k < 2; ++k)
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      const int row = row0 + 16 * k;
-      u32x4 r;
-#pragma unroll
-      for (int d = 0; d < 4; ++d) r[d] = relu_add_pack(v[k][d], cf[2 * d], cf[2 * d + 1]);
-      tile[row * kChunksPerRow + (cc ^ ((row >> 3) & 15))] = r;
-    }
+      for (int d = 0; d < 4; ++d) {
+        float *dst = tile + (li + 32 * k) * kSmallPitch + lj + 2 * d;
+        dst[0] = relu_keep_nan(f16_lo(v[k][d])) + f16_lo(craw[d]);
+        dst[1] = relu_keep_nan(f16_hi(v[k][d])) + f16_hi(craw[d]);
+      }
     __syncthreads();
-    if (tile_id + gridDim.x < ntiles) fetch(tile_id + gridDim.x);
-
-    u32x4 in[8];
 #pragma unroll
-    for (int r = 0; r < 8; ++r) in[r] = tile[(iblk * 8 + r) * kChunksPerRow + (jblk ^ iblk)];
-
-    uint16_t *o = out + ((int64_t)b * n + n0 + jblk * 8) * m + m0 + iblk * 8;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
+    for (int k = 0; k < 2; ++k) {
+      const int j = oj + 32 * k;
       u32x4 w;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        uint32_t xlo = in[2 * q][j >> 1], xhi = in[2 * q + 1][j >> 1];
-        w[q] = (j & 1) ? __builtin_amdgcn_perm(xhi, xlo, 0x07060302u)
-                       : __builtin_amdgcn_perm(xhi, xlo, 0x05040100u);
-      }
-      store_nt(reinterpret_cast<u32x4 *>(o + (int64_t)j * m), w);
+      for (int d = 0; d < 4; ++d)
+        w[d] = pack_f16(tile[(oi + 2 * d) * kSmallPitch + j], tile[(oi + 2 * d + 1) * kSmallPitch + j]);
+      store_nt(reinterpret_cast<u32x4 *>(out + ((int64_t)b * n + n0 + j) * m + m0 + oi), w);
     }
     __syncthreads();
   }
@@ -165,19 +117,17 @@ LaunchStatus launch_relu_broadcast_add_transpose(const uint16_t *x, const uint16
     return invalid("relu_broadcast_add_transpose: extent exceeds 2^31-1");
   if (nb > INT64_MAX / m / n / 4) return invalid("relu_broadcast_add_transpose: extent overflow");
 
-  const bool tiled = (m % kTile == 0) && (n % kTile == 0) && aligned16(x) && aligned16(c) &&
-                     aligned16(out);
-  int64_t tiles = tiled ? nb * (m / kTile) * (n / kTile)
-                        : nb * ((m + 31) / 32) * ((n + 31) / 32);
-  int64_t blocks = tiles;
-  if (AFIR_TR_BLOCKS_PER_CU && tiled && blocks > (int64_t)kNumCU * AFIR_TR_BLOCKS_PER_CU)
-    blocks = (int64_t)kNumCU * AFIR_TR_BLOCKS_PER_CU;
-  if (block_dim) blocks = block_dim;
-  if (blocks > 0x7fffffff) blocks = 0x7fffffff;
-  if (tiled) {
-    hipLaunchKernelGGL(relu_bcast_add_transpose_f16_tiled, dim3((unsigned)blocks), dim3(kThreads),
-                       AFIR_TR_EXTRA_LDS, stream, x, c, out, (int)nb, (int)m, (int)n);
+  if ((m % kSmallTile == 0) && (n % kSmallTile == 0) && aligned16(x) && aligned16(c) && aligned16(out) &&
+      nb * (m / kSmallTile) * (n / kSmallTile) < ((int64_t)1 << 31)) {
+    int64_t blocks = nb * (m / kSmallTile) * (n / kSmallTile);   // one tile per workgroup
+    if (blocks > (int64_t)kNumCU * 256) blocks = (int64_t)kNumCU * 256;
+    if (block_dim) blocks = block_dim;
+    hipLaunchKernelGGL(relu_bcast_add_transpose_f16_tile64, dim3((unsigned)blocks), dim3(kThreads), 0, stream,
+                       x, c, out, (int)nb, (int)m, (int)n);
   } else {
+    int64_t blocks = nb * ((m + 31) / 32) * ((n + 31) / 32);
+    if (block_dim) blocks = block_dim;
+    if (blocks > 0x7fffffff) blocks = 0x7fffffff;
     hipLaunchKernelGGL(relu_bcast_add_transpose_f16_any, dim3((unsigned)blocks), dim3(kThreads),
                        0, stream, x, c, out, (int)nb, (int)m, (int)n);
   }

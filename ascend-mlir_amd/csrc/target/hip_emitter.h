@@ -65,7 +65,7 @@ bool specAllSegments(const afir_region::Program &p);   // whether that kernel is
 // outer iteration dim `dim`, strided along the innermost one) is walked in
 // tiles of kTileP (dim) x kTileQ (innermost dim), the transposed operands
 // staged through LDS; the launch then has one workgroup pass per tile.
-constexpr int kTileP = 64, kTileQ = 128;
+constexpr int kTileP = 64, kTileQ = 64;
 struct SpecTile {
   bool tiled = false;
   int dim = -1;
