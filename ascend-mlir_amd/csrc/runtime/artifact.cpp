@@ -281,6 +281,26 @@ Expected<HipKernelDescriptor> compileSourceText(const std::string &text, const s
       d.symbol = k->symbol;
       return d;
     }
+  // 1b. a hand-written region program (the counterpart of the reference's
+  // hand-written kernel sources, examples/real-npu-microcases/kernels/*.cpp)
+  {
+    size_t at = 0;
+    while (at < text.size() && (text[at] == '#' || isspace((unsigned char)text[at]))) {
+      if (text[at] == '#') while (at < text.size() && text[at] != '\n') ++at;
+      else ++at;
+    }
+    if (text.compare(at, 15, "afir-hip-region") == 0) {
+      afir_region::Program program;
+      std::string why = afir_region::parse(text, &program);
+      if (why.empty()) why = afir_region::validate(program);
+      if (!why.empty()) return Status::error("invalid region program: " + why);
+      d.kernelName = nameHint;
+      d.hipKernel = "fused_region";
+      d.symbol = findKnown("fused_region")->symbol;
+      d.program = afir_region::serialize(program);
+      return d;
+    }
+  }
   const std::string fn = firstFuncName(text);
   // 2. a function with an empty or opaque body that is named after a family
   // 3. MLIR text: translate the function to a region program
@@ -309,7 +329,7 @@ Expected<HipKernelDescriptor> compileSourceText(const std::string &text, const s
       return d;
     }
   }
-  return Status::error("cannot map kernel source to a fused HIP kernel: expected MLIR text (func.func) or "
+  return Status::error("cannot map kernel source to a fused HIP kernel: expected MLIR text (func.func), a region program or "
                        "'hip_kernel=<family>' with one of fused_add_mul, broadcast_add_reducesum, "
                        "relu_broadcast_add_transpose, gather_scale_shift, matmul_add_leakyrelu");
 }

@@ -10,6 +10,7 @@
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <ctime>
 #include <deque>
 #include <fstream>
@@ -173,6 +174,19 @@ SessionSummary runSingleTask(const RunTaskSpec &task, RunnerFactory factory, int
     }
     out.allocate();
     args.outputs.push_back(std::move(out));
+  }
+
+  // A region program takes its extents from TilingData (dim_arg<A>_<D> for
+  // every dimension of every argument).  A task without a tiling binding --
+  // the reference's hand-written static kernels have none,
+  // examples/real-npu-multikernel/prepare.sh:74-176 -- gets them from the
+  // tensors it binds.
+  if (!inv.tiling && !artifact->regionProgram.empty()) {
+    std::vector<int64_t> dims;
+    for (const NDArray &a : args.inputs) dims.insert(dims.end(), a.shape.begin(), a.shape.end());
+    for (const NDArray &a : args.outputs) dims.insert(dims.end(), a.shape.begin(), a.shape.end());
+    args.tiling.resize(dims.size() * sizeof(int64_t));
+    std::memcpy(args.tiling.data(), dims.data(), args.tiling.size());
   }
 
   // ---- executor ----

@@ -300,3 +300,15 @@ EXACT_CASES = {
     "c1": case_c1, "c3": case_c3, "c4": case_c4, "add_mul_3": case_add_mul_3,
 }
 REDUCE_CASES = {"reduce_rowbias": case_reduce_rowbias, "c2": case_c2}
+
+
+# Hand-written static kernels of the reference's multi-kernel examples
+# (examples/real-npu-microcases/kernels/const640.cpp: every element 1,
+# const_with_input640.cpp: every element 2, its input ignored,
+# copy_scalar640.cpp: a copy; examples/real-npu-multikernel/kernels/add_wait640.cpp:
+# lhs + rhs), as region programs.
+CONST_ONE = HEADER + "arg out f16 1\nsegment 1\n size arg0.0\n outoff 0\n const 1\n store\nend\n"
+CONST_TWO_IGNORING_INPUT = HEADER + "arg in f16 1\narg out f16 1\nsegment 1\n size arg1.0\n outoff 0\n const 2\n store\nend\n"
+COPY_1D = HEADER + "arg in f16 1\narg out f16 1\nsegment 1\n size arg1.0\n outoff 0\n push arg0 d0\n store\nend\n"
+ADD_1D = (HEADER + "arg in f16 1\narg in f16 1\narg out f16 1\nsegment 1\n size arg2.0\n outoff 0\n"
+          " push arg0 d0\n push arg1 d0\n add\n store\nend\n")

@@ -265,3 +265,59 @@ def test_matmul_epilogue_kinds(pkg, kind, ty):
         got = out.cpu().numpy() if ty == "f16" else out.view(torch.int16).cpu().numpy().view(np.uint16)
         r.close()
         assert got.tobytes() == want.tobytes(), (kind, ty, m, k, n)
+
+
+def _multikernel_artifacts(tmp_path):
+    for name, text in (("const640", RC.CONST_ONE), ("const_with_input640", RC.CONST_TWO_IGNORING_INPUT),
+                       ("copy_scalar640", RC.COPY_1D), ("add_wait640", RC.ADD_1D)):
+        src = tmp_path / f"{name}.region"
+        src.write_text(text)
+        p = _rs("--kernel", str(src), "--output", str(tmp_path / "artifacts" / name / "artifact"), "--name", name)
+        assert p.returncode == 0, p.stderr
+    return tmp_path / "artifacts"
+
+
+@pytest.mark.parametrize("case", ["serial-two-kernel", "fork-join"])
+def test_reference_multikernel_manifests(tmp_path, case):
+    """The two task graphs of examples/real-npu-multikernel (prepare.sh:74-176) with their own
+    shapes, bindings and goldens (gen_data.py:17-33: 640 x 1.0 after const -> copy, 640 x 3.0
+    after const(1) + const(2)); the kernels are hand-written there and region programs here.
+    No task has a tiling binding: extents come from the bound tensors."""
+    arts = _multikernel_artifacts(tmp_path)
+    common = {"block_dim": 1, "workspace_size": 16384, "atol": 0, "rtol": 0}
+    out = tmp_path / case
+    out.mkdir()
+    if case == "serial-two-kernel":
+        np.save(out / "expected.npy", np.full((640,), 1.0, np.float16))
+        tasks = [
+            dict(task_id="producer", artifact_root=str(arts / "const640" / "artifact"),
+                 outputs=[{"name": "mid", "shape": [640], "dtype": "f16"}], **common),
+            dict(task_id="consumer", artifact_root=str(arts / "copy_scalar640" / "artifact"), dependencies=["producer"],
+                 inputs=[{"name": "input", "source": "task_output", "upstream_task": "producer", "upstream_output": "mid"}],
+                 outputs=[{"name": "out", "path": str(out / "output.npy"), "shape": [640], "dtype": "f16"}],
+                 expected_outputs=[{"name": "out", "path": str(out / "expected.npy")}], **common)]
+        plan = ["producer", "consumer"]
+    else:
+        np.save(out / "expected.npy", np.full((640,), 3.0, np.float16))
+        np.save(out / "input.npy", (np.arange(640) / 17.0).astype(np.float16))
+        tasks = [
+            dict(task_id="producer_a", artifact_root=str(arts / "const640" / "artifact"),
+                 outputs=[{"name": "a", "shape": [640], "dtype": "f16"}], **common),
+            dict(task_id="producer_b", artifact_root=str(arts / "const_with_input640" / "artifact"),
+                 inputs=[{"name": "input", "path": str(out / "input.npy")}],
+                 outputs=[{"name": "b", "shape": [640], "dtype": "f16"}], **common),
+            dict(task_id="consumer", artifact_root=str(arts / "add_wait640" / "artifact"),
+                 dependencies=["producer_a", "producer_b"],
+                 inputs=[{"name": "lhs", "source": "task_output", "upstream_task": "producer_a", "upstream_output": "a"},
+                         {"name": "rhs", "source": "task_output", "upstream_task": "producer_b", "upstream_output": "b"}],
+                 outputs=[{"name": "out", "path": str(out / "output.npy"), "shape": [640], "dtype": "f16"}],
+                 expected_outputs=[{"name": "out", "path": str(out / "expected.npy")}], **common)]
+        plan = ["producer_a", "producer_b", "consumer"]
+    (out / "run_manifest.json").write_text(json.dumps({"backend": "hip", "tasks": tasks}))
+    p = _rs("--run-manifest", str(out / "run_manifest.json"), "--run")
+    assert p.returncode == 0, p.stdout + p.stderr
+    lines = p.stdout.splitlines()
+    assert [l.split("=")[1] for l in lines if l.startswith("session.plan[")] == plan
+    for line in ("session.backend=hip", "session.result=success", "session.validation=pass"):
+        assert line in lines, p.stdout
+    assert np.load(out / "output.npy").tobytes() == np.load(out / "expected.npy").tobytes()
