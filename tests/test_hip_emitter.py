@@ -71,7 +71,7 @@ def test_lane_shapes_follow_the_element_types():
 
 def test_transposed_reads_go_through_lds_tiles():
     src = _emit(RC.C3_RELU_BCAST_TRANSPOSE).stdout      # x[b, i, j] read over the space (b, j, i)
-    assert "tiles of 64 (dim 1) x 128 (dim 2) through LDS; a lane takes 2 groups of 8 elements per row" in src
+    assert "tiles of 64 (dim 1) x 64 (dim 2) through LDS; a lane takes 1 groups of 8 elements per row" in src
     assert "__attribute__((shared)) static float tile[1][TQ * PITCH];" in src
     assert src.count("__builtin_amdgcn_s_barrier();") == 2          # after the tile is written, before it is reused
     # a program with transposed reads gets no all-segments kernel, others of 2..4 segments do
@@ -80,7 +80,7 @@ def test_transposed_reads_go_through_lds_tiles():
     two = RC.HEADER + ("arg in f32 2\narg in f32 2\narg in f32 2\narg out f32 2\nsegment 2\n size arg0.0 arg0.1\n outoff 0\n"
                        " push arg0 d0 d1\n push arg1 d1 d0\n add\n push arg2 d1 d0\n mul\n store\nend\n")
     src = _emit(two).stdout                             # two transposed operands, f32
-    assert "tiles of 64 (dim 0) x 128 (dim 1) through LDS; a lane takes 4 groups of 4 elements per row" in src
+    assert "tiles of 64 (dim 0) x 64 (dim 1) through LDS; a lane takes 2 groups of 4 elements per row" in src
     assert "static float tile[2][TQ * PITCH];" in src
 
 
