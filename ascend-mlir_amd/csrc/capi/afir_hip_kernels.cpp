@@ -80,6 +80,7 @@ struct CompiledRegion {
   std::vector<char> image;
   std::mutex mutex;
   bool loaded = false;
+  afir_target::EmitOptions options;   // read from the loaded module
   hipModule_t module = nullptr;
   std::map<std::string, hipFunction_t> functions;
   ~CompiledRegion() {
@@ -115,9 +116,22 @@ std::string compiled_function(CompiledRegion *c, const afir_region::Program &pro
       (void)hipModuleUnload(m);
       return "code object was not built from this program";
     }
+    // the tile / unroll choices the kernels were emitted with (older objects: the defaults)
+    int opts[3] = {0, 0, 0};
+    if (hipModuleGetGlobal(&sym, &bytes, m, "afir_region_emit_options") == hipSuccess && bytes == sizeof opts &&
+        hipMemcpyDtoH(opts, sym, sizeof opts) == hipSuccess) {
+      c->options.tileP = opts[0];
+      c->options.tileQ = opts[1];
+      c->options.unroll = opts[2];
+      if (!afir_target::checkEmitOptions(c->options).empty()) {
+        (void)hipModuleUnload(m);
+        return "code object carries unusable emit options";
+      }
+    }
     c->module = m;
     c->loaded = true;
   }
+  if (name.empty()) return "";   // load only
   auto it = c->functions.find(name);
   if (it == c->functions.end()) {
     hipFunction_t f = nullptr;
@@ -536,6 +550,14 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
   // interpreter kernel (the tests compare the two)
   if (const char *env = std::getenv("AFIR_HIP_REGION_INTERPRET"))
     if (*env && *env != '0') compiled.reset();
+  afir_target::EmitOptions emit;
+  if (compiled) {
+    // load the module now: the grids below depend on the options it was emitted with
+    hipFunction_t none = nullptr;
+    const std::string no = compiled_function(compiled.get(), r->program, "", &none);
+    if (!no.empty()) return fail(AFIR_HIP_E_LAUNCH, no);
+    emit = compiled->options;
+  }
   struct PendingSegment {
     int segment;
     afir_target::SpecArgs args;
@@ -588,7 +610,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
     }
     if (compiled) {
       const int segment = (int)(&seg - res.segments.data());
-      const afir_target::SpecShape shape = afir_target::specShape(r->program, segment);
+      const afir_target::SpecShape shape = afir_target::specShape(r->program, segment, emit);
       const afir_target::SpecTile tile = afir_target::specTile(r->program, segment);
       const int W = shape.width, U = shape.unroll;
       afir::RegionGeometry g;
@@ -605,16 +627,16 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
       sa.grid = (int)g.blocks;
       bool all_aligned;
       if (tile.tiled) {
-        // one workgroup pass per tile of kTileP x kTileQ
-        const int64_t tq = (seg.size[last] + afir_target::kTileQ - 1) / afir_target::kTileQ;
-        const int64_t tp = (seg.size[tile.dim] + afir_target::kTileP - 1) / afir_target::kTileP;
+        // one workgroup pass per tile of tile_p x tile_q
+        const int64_t tq = (seg.size[last] + emit.tileQ - 1) / emit.tileQ;
+        const int64_t tp = (seg.size[tile.dim] + emit.tileP - 1) / emit.tileP;
         int64_t tiles = tq * tp;
         for (int k = 0; k < last; ++k)
           if (k != tile.dim) tiles *= seg.size[k];
         int64_t blocks = tiles < (int64_t)afir::kNumCU * 256 ? tiles : (int64_t)afir::kNumCU * 256;
         if (block_dim) blocks = block_dim;
         sa.grid = (int)blocks;
-        all_aligned = seg.size[last] % afir_target::kTileQ == 0 && seg.size[tile.dim] % afir_target::kTileP == 0 &&
+        all_aligned = seg.size[last] % emit.tileQ == 0 && seg.size[tile.dim] % emit.tileP == 0 &&
                       a.out_vec;
       } else {
         // the aligned variant has no tail handling: whole groups, whole passes

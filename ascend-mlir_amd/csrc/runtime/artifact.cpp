@@ -217,13 +217,19 @@ std::string resolveCodeObject(const HipKernelDescriptor &d, const std::string &d
 }
 
 Expected<std::string> compileRegionCodeObject(const std::string &programText, const std::string &dir,
-                                              const std::string &name) {
+                                              const std::string &name,
+                                              const std::map<std::string, int64_t> &emitOptions) {
   if (const char *env = std::getenv("AFIR_HIP_CODEGEN"))
     if (*env == '0') return Status::error("disabled by AFIR_HIP_CODEGEN=0");
   afir_region::Program program;
   if (std::string why = afir_region::parse(programText, &program); !why.empty()) return Status::error(why);
+  afir_target::EmitOptions options;
+  for (const auto &kv : emitOptions)
+    if (!afir_target::setEmitOption(&options, kv.first, kv.second))
+      return Status::error("unknown emit option '" + kv.first + "' (tile_p, tile_q, unroll)");
   std::string source;
-  if (std::string why = afir_target::emitHipSource(program, name, &source); !why.empty()) return Status::error(why);
+  if (std::string why = afir_target::emitHipSource(program, name, &source, options); !why.empty())
+    return Status::error(why);
   const std::string srcPath = joinPath(dir, name + ".hip"), objName = name + ".hsaco",
                     objPath = joinPath(dir, objName), logPath = joinPath(dir, name + ".hipcc.log");
   {
@@ -358,10 +364,13 @@ Expected<KernelArtifact> compileArtifact(const CompileRequest &request) {
   if (!d.program.empty()) {
     // kernels specialised for the program; without them the interpreter
     // kernel of the library runs it
-    auto object = compileRegionCodeObject(d.program, request.outputDir, name);
+    auto object = compileRegionCodeObject(d.program, request.outputDir, name, request.emitOptions);
     if (object) {
       d.codeObject = *object;
       d.codeObjectDir = absolutePath(request.outputDir);
+    } else if (!request.emitOptions.empty() && object.error().find("hipcc") == std::string::npos &&
+               object.error().find("AFIR_HIP_CODEGEN") == std::string::npos) {
+      return Status::error("emit options: " + object.error());   // asked-for choices must not be dropped silently
     } else {
       codegenNote = object.error();
     }

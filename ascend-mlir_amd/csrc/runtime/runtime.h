@@ -206,7 +206,8 @@ std::string resolveCodeObject(const HipKernelDescriptor &d, const std::string &d
 // to <dir>/<name>.hsaco with hipcc ($HIPCC, PATH, /opt/rocm/bin).  Returns the
 // code object's file name, or an error saying why there is none.
 Expected<std::string> compileRegionCodeObject(const std::string &programText, const std::string &dir,
-                                              const std::string &name);
+                                              const std::string &name,
+                                              const std::map<std::string, int64_t> &emitOptions = {});
 std::string serializeDescriptor(const HipKernelDescriptor &d);
 Expected<HipKernelDescriptor> parseDescriptor(const std::string &text);
 
@@ -216,6 +217,9 @@ struct CompileRequest {
   std::string kernelName;    // optional override
   std::string socVersion = "gfx950";
   std::optional<KernelKind> kernelKind;
+  // Compile-time choices of the emitted region kernels: "tile_p", "tile_q",
+  // "unroll" (csrc/target/hip_emitter.h: EmitOptions); absent = defaults.
+  std::map<std::string, int64_t> emitOptions;
 };
 // Source -> artifact directory: <out>/<name>.hipk + <out>/out/manifest.txt.
 Expected<KernelArtifact> compileArtifact(const CompileRequest &request);

@@ -223,19 +223,19 @@ struct Value {
 // instruction of a wavefront covers one contiguous run of memory.
 class SegmentEmitter {
  public:
-  SegmentEmitter(const Program &p, int index, std::ostringstream &os)
-      : p_(p), seg_(p.segments[index]), index_(index), os_(os) {}
+  SegmentEmitter(const Program &p, int index, std::ostringstream &os, const EmitOptions &options = EmitOptions())
+      : p_(p), seg_(p.segments[index]), index_(index), os_(os), opt_(options) {}
 
   std::string run() {
     if (!seg_.ops.empty() && seg_.ops[0].code == OpCode::Matmul)
       return "matmul segments run on the hand-written MFMA kernels";
-    const SpecShape shape = specShape(p_, index_);
+    const SpecShape shape = specShape(p_, index_, opt_);
     W_ = shape.width;
     U_ = shape.unroll;
     analyze();
     if ((int)pushSlot_.size() > kSpecMaxInputs) return "more than 8 operand reads in a segment";
     if (tiled()) {
-      U_ = kTileQ / 8 / W_;   // eight lanes cover a tile row
+      U_ = opt_.tileQ / 8 / W_;   // eight lanes cover a tile row
       emitBodyTiled();
     } else {
       emitBody();
@@ -653,6 +653,7 @@ class SegmentEmitter {
     const std::string otag = typeTag(p_.output().type);
     const int p = tileDim_, r = rank_ == 3 ? (p == 0 ? 1 : 0) : -1;
     const std::string P = std::to_string(p), L = std::to_string(last_);
+    const int kTileP = opt_.tileP, kTileQ = opt_.tileQ;
     os_ << "\n// ---- segment " << index_ << ": iteration rank " << rank_ << ", parallel, tiles of " << kTileP
         << " (dim " << p << ") x " << kTileQ << " (dim " << last_ << ") through LDS; a lane takes " << U_
         << " groups of " << W_ << " elements per row ----\n";
@@ -758,6 +759,7 @@ class SegmentEmitter {
   const Segment &seg_;
   int index_;
   std::ostringstream &os_;
+  EmitOptions opt_;
   int rank_ = 0, last_ = 0, W_ = 8, U_ = 2;
   int tileDim_ = -1, numTiles_ = 0;
   bool reduce_ = false;
@@ -767,14 +769,31 @@ class SegmentEmitter {
 
 }  // namespace
 
-SpecShape specShape(const Program &p, int segment) {
+std::string checkEmitOptions(const EmitOptions &o) {
+  if (o.tileP < 32 || o.tileP > 256 || o.tileP % 32 != 0) return "tile_p must be a multiple of 32 in 32..256";
+  if (o.tileQ != 64 && o.tileQ != 128 && o.tileQ != 256) return "tile_q must be 64, 128 or 256";
+  if ((long long)o.tileQ * (o.tileP + 1) * 4 * kMaxTiles > 160 * 1024) return "tile_p x tile_q does not fit the LDS";
+  if (o.unroll != 0 && o.unroll != 1 && o.unroll != 2 && o.unroll != 4 && o.unroll != 8)
+    return "unroll must be 0 (by element types), 1, 2, 4 or 8";
+  return "";
+}
+
+bool setEmitOption(EmitOptions *o, const std::string &name, long long value) {
+  if (name == "tile_p") o->tileP = (int)value;
+  else if (name == "tile_q") o->tileQ = (int)value;
+  else if (name == "unroll") o->unroll = (int)value;
+  else return false;
+  return true;
+}
+
+SpecShape specShape(const Program &p, int segment, const EmitOptions &options) {
   const Segment &g = p.segments[segment];
   bool any16 = p.output().type != ElemType::F32, any32 = p.output().type == ElemType::F32;
   for (const Op &op : g.ops)
     if (op.code == OpCode::Push) (p.args[op.arg].type == ElemType::F32 ? any32 : any16) = true;
   SpecShape s;
   s.width = any16 ? 8 : 4;            // 16 bytes of the narrowest tensor
-  s.unroll = (any16 && any32) ? 2 : 4;
+  s.unroll = options.unroll ? options.unroll : ((any16 && any32) ? 2 : 4);
   return s;
 }
 
@@ -817,8 +836,10 @@ std::string specKernelName(int segment, bool idx32, bool aligned) {
   return "afir_region_s" + std::to_string(segment) + (idx32 ? "_i32" : "_i64") + (aligned ? "_a" : "_g");
 }
 
-std::string emitHipSource(const Program &p, const std::string &title, std::string *source) {
+std::string emitHipSource(const Program &p, const std::string &title, std::string *source,
+                          const EmitOptions &options) {
   if (std::string why = validate(p); !why.empty()) return why;
+  if (std::string why = checkEmitOptions(options); !why.empty()) return why;
   std::ostringstream os;
   os << "// HIP kernels for the fused region '" << title << "' (gfx950), generated from this program:\n";
   {
@@ -835,8 +856,10 @@ std::string emitHipSource(const Program &p, const std::string &title, std::strin
   char hash[32];
   std::snprintf(hash, sizeof hash, "0x%016llxull", (unsigned long long)programHash(p));
   os << "extern \"C\" __attribute__((device)) __attribute__((used)) const unsigned long long afir_region_program_hash = " << hash << ";\n";
+  os << "extern \"C\" __attribute__((device)) __attribute__((used)) const int afir_region_emit_options[3] = {"
+     << options.tileP << ", " << options.tileQ << ", " << options.unroll << "};   // tile_p, tile_q, unroll\n";
   for (int s = 0; s < (int)p.segments.size(); ++s) {
-    SegmentEmitter e(p, s, os);
+    SegmentEmitter e(p, s, os, options);
     if (std::string why = e.run(); !why.empty()) return why;
   }
   const int nseg = (int)p.segments.size();

@@ -63,9 +63,8 @@ bool specAllSegments(const afir_region::Program &p);   // whether that kernel is
 
 // A parallel segment that reads an operand transposed (contiguous along an
 // outer iteration dim `dim`, strided along the innermost one) is walked in
-// tiles of kTileP (dim) x kTileQ (innermost dim), the transposed operands
-// staged through LDS; the launch then has one workgroup pass per tile.
-constexpr int kTileP = 64, kTileQ = 64;
+// tiles of EmitOptions::tileP (dim) x tileQ (innermost dim), the transposed
+// operands staged through LDS; the launch then has one workgroup pass per tile.
 struct SpecTile {
   bool tiled = false;
   int dim = -1;
@@ -74,13 +73,27 @@ struct SpecTile {
 };
 SpecTile specTile(const afir_region::Program &p, int segment);
 
+// Choices the emitter leaves open: the tile of segments that read an operand
+// transposed, and how many groups a lane takes per pass elsewhere.  They are
+// compile-time constants of the emitted kernels; the code object exports them
+// (`afir_region_emit_options`) so that the launcher sizes its grids to match.
+struct EmitOptions {
+  int tileP = 64;   // tile extent along the dim the transposed operands are contiguous in (multiple of 32)
+  int tileQ = 64;   // tile extent along the innermost iteration dim (64, 128 or 256)
+  int unroll = 0;   // groups per lane and pass in untiled segments; 0 = by element types (4, or 2 when mixed)
+};
+// "" if usable, else why not.
+std::string checkEmitOptions(const EmitOptions &o);
+// "tile_p" / "tile_q" / "unroll" = integer; returns false for an unknown name.
+bool setEmitOption(EmitOptions *o, const std::string &name, long long value);
+
 // A lane's share of one pass over a row: `unroll` groups of `width` consecutive
 // elements (16 bytes of the narrowest tensor), the groups one lane-set apart.
 struct SpecShape {
   int width = 8;
   int unroll = 2;
 };
-SpecShape specShape(const afir_region::Program &p, int segment);
+SpecShape specShape(const afir_region::Program &p, int segment, const EmitOptions &options = EmitOptions());
 
 // FNV-1a of the serialized program: the emitted code object exports it as
 // `afir_region_program_hash`, checked when the code object is attached.
@@ -93,7 +106,8 @@ std::string specKernelName(int segment, bool idx32, bool aligned);
 // Emits the source for every segment.  Returns "" on success, else why the
 // program has no specialised form (matmul segments: those run on the
 // hand-written kernels).
-std::string emitHipSource(const afir_region::Program &p, const std::string &title, std::string *source);
+std::string emitHipSource(const afir_region::Program &p, const std::string &title, std::string *source,
+                          const EmitOptions &options = EmitOptions());
 
 // The compiler invocation for a source file (argv, no shell).
 std::string hipccCommandLine(const std::string &sourcePath, const std::string &outputPath);

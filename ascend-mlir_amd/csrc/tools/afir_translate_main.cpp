@@ -16,6 +16,7 @@
 // Exit codes: 0 ok, 1 the input cannot be lowered (diagnostic on stderr),
 // 2 usage / file errors.
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <fstream>
 #include <iostream>
@@ -28,6 +29,7 @@
 int main(int argc, char **argv) {
   std::string input, output, tilingOut;
   bool toHip = false, emitSource = false;
+  afir_target::EmitOptions emitOptions;
   for (int i = 1; i < argc; ++i) {
     const std::string a = argv[i];
     auto value = [&](const char *flag) -> const char * {
@@ -40,6 +42,23 @@ int main(int argc, char **argv) {
       toHip = true;
     } else if (a == "--emit-hip-source") {
       emitSource = true;
+    } else if (a.compare(0, 14, "--emit-options") == 0) {
+      const char *v = value("--emit-options");
+      if (!v) { std::fprintf(stderr, "afir-translate: --emit-options needs name=value[,name=value]\n"); return 2; }
+      std::string items = v;
+      size_t at = 0;
+      while (at <= items.size()) {
+        const size_t comma = items.find(',', at);
+        const std::string kv = items.substr(at, comma == std::string::npos ? std::string::npos : comma - at);
+        const size_t eq = kv.find('=');
+        if (eq == std::string::npos || !afir_target::setEmitOption(&emitOptions, kv.substr(0, eq),
+                                                                   std::strtoll(kv.c_str() + eq + 1, nullptr, 10))) {
+          std::fprintf(stderr, "afir-translate: unknown emit option '%s' (tile_p, tile_q, unroll)\n", kv.c_str());
+          return 2;
+        }
+        if (comma == std::string::npos) break;
+        at = comma + 1;
+      }
     } else if (a == "-mlir-to-cann" || a == "--mlir-to-cann") {
       std::fprintf(stderr, "afir-translate: this build emits for gfx950 only; use -mlir-to-hip\n");
       return 2;
@@ -52,7 +71,7 @@ int main(int argc, char **argv) {
       if (!v) { std::fprintf(stderr, "afir-translate: --tiling-space-out needs a file name\n"); return 2; }
       tilingOut = v;
     } else if (a == "-h" || a == "--help") {
-      std::printf("usage: afir-translate -mlir-to-hip <input.mlir> [-o <file>] [--tiling-space-out <file>] [--emit-hip-source]\n");
+      std::printf("usage: afir-translate -mlir-to-hip <input.mlir> [-o <file>] [--tiling-space-out <file>] [--emit-hip-source [--emit-options tile_p=64,tile_q=64,unroll=0]]\n");
       return 0;
     } else if (!a.empty() && a[0] == '-' && a != "-") {
       std::fprintf(stderr, "afir-translate: unknown option %s\n", a.c_str());
@@ -98,7 +117,7 @@ int main(int argc, char **argv) {
   }
   std::string program = "# kernel " + tr.functionName + "\n" + afir_region::serialize(tr.program);
   if (emitSource) {
-    const std::string no = afir_target::emitHipSource(tr.program, tr.functionName, &program);
+    const std::string no = afir_target::emitHipSource(tr.program, tr.functionName, &program, emitOptions);
     if (!no.empty()) {
       std::fprintf(stderr, "%s: error: no specialised kernel: %s\n", input.empty() ? "<stdin>" : input.c_str(), no.c_str());
       return 1;

@@ -18,6 +18,10 @@
 //   "values": [..] | "min","max","step" | "fixed": true + "shape_key" | "value"}]}.
 // A parameter named dim_arg<A>_<D> with nothing else given takes dimension D
 // of argument A from the .npy files (inputs first, then the expected output).
+// A parameter named emit_tile_p / emit_tile_q / emit_unroll is a compile-time
+// choice of the emitted kernels (only with --kernel): every combination is
+// compiled into its own artifact under the build directory and is not part of
+// the TilingData bytes.
 //
 // Exit codes: 0 ok, 1 no candidate passed, 2 run error, 4 bad invocation.
 #include <cmath>
@@ -179,6 +183,7 @@ int main(int argc, char **argv) {
 
   // ---- artifact ----
   KernelArtifact artifact;
+  CompileRequest baseRequest;
   if (opt.count("artifact-root")) {
     auto a = loadArtifactFromRoot(opt["artifact-root"]);
     if (!a) return usage(a.error().c_str());
@@ -197,6 +202,7 @@ int main(int argc, char **argv) {
     auto a = compileArtifact(req);
     if (!a) return usage(a.error().c_str());
     artifact = *a;
+    baseRequest = req;
   }
 
   // ---- tensors ----
@@ -270,6 +276,7 @@ int main(int argc, char **argv) {
     double ns = 0, maxAbs = 0;
     int64_t blockDim = 0;
     std::map<std::string, int64_t> config;
+    KernelArtifact artifact;
   } best;
   size_t index = 0, total = 0;
   for (const auto &c : combos) {
@@ -293,10 +300,40 @@ int main(int argc, char **argv) {
     // tiling bytes in the order of the space
     std::vector<TilingField> fields;
     std::vector<std::pair<std::string, int64_t>> values;
+    std::map<std::string, int64_t> emitOptions;
     for (const Param &p : space) {
+      if (p.name.rfind("emit_", 0) == 0) {
+        emitOptions[p.name.substr(5)] = vars[p.name];
+        continue;
+      }
       fields.push_back({p.name, p.type});
       values.push_back({p.name, vars[p.name]});
     }
+    // kernels emitted with these choices: one artifact per combination
+    KernelArtifact candidateArtifact = artifact;
+    if (!emitOptions.empty()) {
+      if (baseRequest.kernelSource.empty())
+        return usage("emit_* parameters need --kernel (the kernels are compiled per candidate)");
+      CompileRequest req = baseRequest;
+      req.emitOptions = emitOptions;
+      req.outputDir = baseRequest.outputDir + "/emit";
+      for (const auto &kv : emitOptions) req.outputDir += "_" + kv.first + std::to_string(kv.second);
+      auto a = compileArtifact(req);
+      if (!a) {
+        for (int64_t bd : dims) {
+          ++index;
+          std::printf("[%zu/%zu]", index, total);
+          for (const auto &kv : combo) std::printf(" %s=%lld", kv.first.c_str(), (long long)kv.second);
+          std::printf(" block_dim=%lld ... FAIL  %s\n", (long long)bd, a.error().c_str());
+        }
+        continue;
+      }
+      candidateArtifact = *a;
+    }
+    launch.sharedLibraryPath = candidateArtifact.sharedLibraryPath;
+    launch.symbolName = candidateArtifact.sharedLibrarySymbol;
+    launch.regionProgram = candidateArtifact.regionProgram;
+    launch.codeObjectPath = candidateArtifact.codeObjectPath;
     auto packed = TilingSchema::fromFields(fields).pack(values);
     if (!packed) return usage(packed.error().c_str());
 
@@ -342,6 +379,7 @@ int main(int argc, char **argv) {
       }
       std::printf(" OK  score=%.0f max_abs_diff=%g\n", bestNs, cmp->maxAbsDiff);
       if (!best.found || bestNs < best.ns) {
+        best.artifact = candidateArtifact;
         best.found = true;
         best.ns = bestNs;
         best.maxAbs = cmp->maxAbsDiff;
@@ -362,12 +400,12 @@ int main(int argc, char **argv) {
     return 2;
   }
   f << "{\n";
-  f << "  \"kernel_name\": \"" << jsonEscape(artifact.kernelName) << "\",\n";
-  f << "  \"kernel_type\": \"" << kernelKindName(artifact.kernelKind) << "\",\n";
-  f << "  \"soc\": \"" << jsonEscape(artifact.socVersion) << "\",\n";
-  f << "  \"artifact_root\": \"" << jsonEscape(artifact.artifactRoot) << "\",\n";
-  f << "  \"manifest_path\": \"" << jsonEscape(artifact.manifestPath) << "\",\n";
-  f << "  \"device_binary_path\": \"" << jsonEscape(artifact.deviceBinaryPath) << "\",\n";
+  f << "  \"kernel_name\": \"" << jsonEscape(best.artifact.kernelName) << "\",\n";
+  f << "  \"kernel_type\": \"" << kernelKindName(best.artifact.kernelKind) << "\",\n";
+  f << "  \"soc\": \"" << jsonEscape(best.artifact.socVersion) << "\",\n";
+  f << "  \"artifact_root\": \"" << jsonEscape(best.artifact.artifactRoot) << "\",\n";
+  f << "  \"manifest_path\": \"" << jsonEscape(best.artifact.manifestPath) << "\",\n";
+  f << "  \"device_binary_path\": \"" << jsonEscape(best.artifact.deviceBinaryPath) << "\",\n";
   f << "  \"kernel_file\": \"" << jsonEscape(json->getString("kernel_file").value_or("")) << "\",\n";
   f << "  \"best\": {\"block_dim\": " << best.blockDim << ", \"cycle_count\": " << (long long)std::llround(best.ns)
     << ", \"score\": " << (long long)std::llround(best.ns) << ", \"score_unit\": \"ns\", \"max_abs_diff\": "

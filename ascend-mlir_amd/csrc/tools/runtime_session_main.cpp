@@ -9,6 +9,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <sstream>
 #include <string>
 
 #include "../runtime/runtime.h"
@@ -47,7 +48,7 @@ void printErrorSummary(const SessionSummary &s) {
 int main(int argc, char **argv) {
   std::map<std::string, std::string> opt;
   bool run = false;
-  const char *valued[] = {"kernel", "kernel-kind", "output", "name", "soc", "artifact-root",
+  const char *valued[] = {"emit-options", "kernel", "kernel-kind", "output", "name", "soc", "artifact-root",
                           "run-manifest", "task-id", "testing-driver", "device", "cann-mlir",
                           "npy-dir"};
   for (int i = 1; i < argc; ++i) {
@@ -73,6 +74,7 @@ int main(int argc, char **argv) {
     if (key == "help" || key == "h") {
       std::printf("task graph runtime planning and execution CLI for artifacts and session graphs (HIP backend)\n"
                   "  --kernel <file> --output <dir> [--name N] [--kernel-kind vec|cube|mix] [--soc S]\n"
+                  "           [--emit-options tile_p=64,tile_q=64,unroll=0]\n"
                   "  --artifact-root <dir>\n  --run-manifest <json>\n  --run\n  --device <n>\n");
       return 0;
     }
@@ -126,6 +128,17 @@ int main(int argc, char **argv) {
       req.outputDir = opt.count("output") ? opt["output"] : "./build/runtime-session-artifact";
       req.kernelName = opt.count("name") ? opt["name"] : "";
       req.socVersion = opt.count("soc") ? opt["soc"] : "gfx950";
+      if (opt.count("emit-options")) {   // --emit-options tile_p=64,tile_q=128,unroll=2
+        std::istringstream items(opt["emit-options"]);
+        for (std::string kv; std::getline(items, kv, ',');) {
+          const size_t eq = kv.find('=');
+          if (eq == std::string::npos || eq == 0) {
+            std::fprintf(stderr, "Error: --emit-options takes name=value pairs, got '%s'\n", kv.c_str());
+            return 4;
+          }
+          req.emitOptions[kv.substr(0, eq)] = std::strtoll(kv.c_str() + eq + 1, nullptr, 10);
+        }
+      }
       if (opt.count("kernel-kind")) {
         auto kind = parseKernelKind(opt["kernel-kind"]);
         if (!kind) {

@@ -91,3 +91,42 @@ def test_bad_invocations(tmp_path):
     assert p.returncode == 4 and "unknown name 'nope'" in p.stderr
     (tmp_path / "space.json").write_text("[1, 2]")
     assert _at(*base, "--shape", "M=8,N=32").returncode == 4
+
+
+def test_emit_parameters_compile_one_artifact_per_candidate(tmp_path):
+    """emit_* parameters are compile-time choices of the emitted kernels: every
+    combination gets its own artifact and stays out of the TilingData bytes."""
+    from tests import region_cases as RC
+    (tmp_path / "k.region").write_text(RC.C3_RELU_BCAST_TRANSPOSE)
+    np.save(tmp_path / "x.npy", np.ones((2, 64, 128), np.float16))
+    np.save(tmp_path / "c.npy", np.ones((128,), np.float16))
+    np.save(tmp_path / "e.npy", np.zeros((2, 128, 64), np.float16))
+    space = {"kernel": "c3", "kernel_file": "k.region", "block_dim_values": [0, 8],
+             "tiling_params": [{"name": "emit_tile_q", "values": [64, 128]},
+                               {"name": "emit_tile_p", "value": 32},
+                               {"name": "dim_arg0_0"}, {"name": "dim_arg0_1"}, {"name": "dim_arg0_2"},
+                               {"name": "dim_arg1_0"},
+                               {"name": "dim_arg2_0"}, {"name": "dim_arg2_1"}, {"name": "dim_arg2_2"}]}
+    (tmp_path / "space.json").write_text(json.dumps(space))
+    p = _at("--space", str(tmp_path / "space.json"), "--kernel", str(tmp_path / "k.region"),
+            "--inputs", f"{tmp_path / 'x.npy'},{tmp_path / 'c.npy'}", "--expected", str(tmp_path / "e.npy"),
+            "--shape", "B=2", "--output", str(tmp_path / "best.json"), "--build-dir", str(tmp_path / "art"),
+            "--testing-driver=hip-success")
+    assert p.returncode == 0, p.stderr + p.stdout
+    lines = [l for l in p.stdout.splitlines() if l.startswith("[")]
+    assert len(lines) == 4 and all(" OK " in l for l in lines)
+    for tq in (64, 128):
+        src = (tmp_path / "art" / f"emit_tile_p32_tile_q{tq}" / "c3.hip").read_text()
+        assert f"tiles of 32 (dim 1) x {tq} (dim 2)" in src
+        assert (tmp_path / "art" / f"emit_tile_p32_tile_q{tq}" / "c3.hsaco").stat().st_size > 0
+    best = json.loads((tmp_path / "best.json").read_text())
+    assert best["config"]["emit_tile_p"] == 32 and best["config"]["emit_tile_q"] in (64, 128)
+    assert best["artifact_root"].endswith(f"emit_tile_p32_tile_q{best['config']['emit_tile_q']}")
+    # a choice the emitter refuses fails that candidate only
+    space["tiling_params"][0]["values"] = [64, 100]
+    (tmp_path / "space.json").write_text(json.dumps(space))
+    p = _at("--space", str(tmp_path / "space.json"), "--kernel", str(tmp_path / "k.region"),
+            "--inputs", f"{tmp_path / 'x.npy'},{tmp_path / 'c.npy'}", "--expected", str(tmp_path / "e.npy"),
+            "--shape", "B=2", "--output", str(tmp_path / "best.json"), "--build-dir", str(tmp_path / "art2"),
+            "--testing-driver=hip-success")
+    assert p.returncode == 0 and p.stdout.count(" FAIL ") == 2 and "tile_q must be 64, 128 or 256" in p.stdout

@@ -57,3 +57,32 @@ def test_autotune_row_bias_reduce(tmp_path):
     p = _run(tmp_path, want + np.float16(3.0), "--atol", "0.25", "--rtol", "0.01")
     assert p.returncode == 1, p.stdout + p.stderr
     assert p.stdout.count(" FAIL ") == 4 and "no candidate passed" in p.stderr
+
+
+def test_autotune_tile_shapes_of_a_transposing_region(tmp_path):
+    """Tile shapes as searched parameters: each candidate is compiled, run and
+    validated bit-exactly (atol = rtol = 0) against the oracle's result."""
+    from tests import region_cases as RC
+    from oracle import region_oracle as RO
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((3, 200, 136)).astype(np.float16)       # ragged against every tile shape
+    c = rng.standard_normal((136,)).astype(np.float16)
+    want = RO.evaluate(RC.C3_RELU_BCAST_TRANSPOSE, [x, c])
+    (tmp_path / "k.region").write_text(RC.C3_RELU_BCAST_TRANSPOSE)
+    np.save(tmp_path / "x.npy", x)
+    np.save(tmp_path / "c.npy", c)
+    np.save(tmp_path / "e.npy", want)
+    space = {"kernel": "c3", "kernel_file": "k.region", "block_dim_values": [0],
+             "tiling_params": [{"name": "emit_tile_p", "values": [32, 64]}, {"name": "emit_tile_q", "values": [64, 128]},
+                               {"name": "dim_arg0_0"}, {"name": "dim_arg0_1"}, {"name": "dim_arg0_2"}, {"name": "dim_arg1_0"},
+                               {"name": "dim_arg2_0"}, {"name": "dim_arg2_1"}, {"name": "dim_arg2_2"}]}
+    (tmp_path / "space.json").write_text(json.dumps(space))
+    p = subprocess.run([AT, "--space", str(tmp_path / "space.json"), "--kernel", str(tmp_path / "k.region"),
+                        "--inputs", f"{tmp_path / 'x.npy'},{tmp_path / 'c.npy'}", "--expected", str(tmp_path / "e.npy"),
+                        "--shape", "B=3", "--output", str(tmp_path / "best.json"), "--build-dir", str(tmp_path / "art"),
+                        "--atol", "0", "--rtol", "0"], capture_output=True, text=True, timeout=110)
+    assert p.returncode == 0, p.stdout + p.stderr
+    lines = [l for l in p.stdout.splitlines() if l.startswith("[")]
+    assert len(lines) == 4 and all(" OK " in l and "max_abs_diff=0" in l for l in lines), p.stdout
+    best = json.loads((tmp_path / "best.json").read_text())
+    assert (best["config"]["emit_tile_p"], best["config"]["emit_tile_q"]) in [(32, 64), (32, 128), (64, 64), (64, 128)]

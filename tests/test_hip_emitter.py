@@ -156,3 +156,29 @@ def test_capi_emit_and_attach_without_gpu(pkg):
     with pytest.raises(H.AfirHipError, match="take no code object"):
         m.attach_code_object(b"\x7fELF" + b"\0" * 60)
     m.close()
+
+
+def test_emit_options_change_the_tile_and_the_unroll(tmp_path):
+    def emit(text, *flags):
+        return subprocess.run([TR, "-mlir-to-hip", "-", "--emit-hip-source", *flags], input=text, capture_output=True, text=True)
+    p = emit(RC.C3_RELU_BCAST_TRANSPOSE, "--emit-options", "tile_p=32,tile_q=128")
+    assert p.returncode == 0, p.stderr
+    assert "tiles of 32 (dim 1) x 128 (dim 2) through LDS; a lane takes 2 groups of 8 elements per row" in p.stdout
+    assert "afir_region_emit_options[3] = {32, 128, 0};" in p.stdout
+    assert "afir_region_emit_options[3] = {64, 64, 0};" in emit(RC.C3_RELU_BCAST_TRANSPOSE).stdout
+    p = emit(RC.C1_ADD_MUL, "--emit-options=unroll=2")
+    assert p.returncode == 0 and "a lane takes 2 groups of 4 elements per pass" in p.stdout
+    p = emit(RC.C1_ADD_MUL, "--emit-options", "tile_q=100")
+    assert p.returncode == 1 and "tile_q must be 64, 128 or 256" in p.stderr
+    p = emit(RC.C1_ADD_MUL, "--emit-options", "tiles=3")
+    assert p.returncode == 2 and "unknown emit option" in p.stderr
+    # through the artifact compiler
+    src = tmp_path / "k.region"
+    src.write_text(RC.C3_RELU_BCAST_TRANSPOSE)
+    q = subprocess.run([RS, "--kernel", str(src), "--output", str(tmp_path / "a"), "--name", "k",
+                        "--emit-options", "tile_q=128"], capture_output=True, text=True)
+    assert q.returncode == 0, q.stderr
+    assert "x 128 (dim 2) through LDS" in (tmp_path / "a" / "k.hip").read_text()
+    q = subprocess.run([RS, "--kernel", str(src), "--output", str(tmp_path / "b"), "--name", "k",
+                        "--emit-options", "tile_p=48"], capture_output=True, text=True)
+    assert q.returncode == 4 and "tile_p must be a multiple of 32" in q.stderr
