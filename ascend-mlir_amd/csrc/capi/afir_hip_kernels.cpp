@@ -97,6 +97,7 @@ struct RegisteredRegion {
   int fastArgs[4] = {-1, -1, -1, -1};  // argument index of each kernel operand
   float alpha = 0.f;
   std::shared_ptr<CompiledRegion> compiled;   // null: the interpreter kernel runs the program
+  bool preferCompiled = false;                // the attached code object outranks a hand-tuned family
 };
 
 // Loads the module if needed and looks a kernel up.  "" on success.
@@ -414,9 +415,20 @@ uint32_t afir_hip_region_info(uint64_t handle, int *num_inputs, int *num_outputs
   return AFIR_HIP_OK;
 }
 
+uint32_t afir_hip_region_prefer_code_object(uint64_t handle, int prefer) {
+  auto r = find_region(handle);
+  if (!r) return fail(AFIR_HIP_E_UNKNOWN, "no region program with that handle");
+  std::lock_guard<std::mutex> lock(g_region_mutex);
+  r->preferCompiled = prefer != 0;
+  g_last_error.clear();
+  return AFIR_HIP_OK;
+}
+
 const char *afir_hip_region_kernel(uint64_t handle) {
   auto r = find_region(handle);
   if (!r) return "";
+  const bool matmul = r->fast == FastPath::MatmulBiasLeaky || r->fast == FastPath::MatmulBiasLeakyF16;
+  if (r->preferCompiled && r->compiled && !matmul) return "fused_region_compiled";
   switch (r->fast) {
     case FastPath::AddMul: return "fused_add_mul";
     case FastPath::BcastAddRowsum: return "broadcast_add_reducesum";
@@ -498,7 +510,13 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
   for (int i = 0; i < want; ++i)
     if (res.bytes[i] && !args[i]) return fail(AFIR_HIP_E_INVALID, "region: null tensor pointer");
 
-  if (r->fast != FastPath::None) {
+  bool prefer_compiled;
+  {
+    std::lock_guard<std::mutex> lock(g_region_mutex);
+    prefer_compiled = r->preferCompiled && r->compiled != nullptr && r->fast != FastPath::MatmulBiasLeaky &&
+                      r->fast != FastPath::MatmulBiasLeakyF16;
+  }
+  if (r->fast != FastPath::None && !prefer_compiled) {
     const afir_region::ResolvedSegment &seg = res.segments[0];
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int *fa = r->fastArgs;

@@ -75,6 +75,7 @@ afirt::Status runDescriptor(ExecutorHandle *h, const std::string &descriptorText
   launch.symbolName = d->symbol;
   launch.regionProgram = d->program;
   launch.codeObjectPath = afirt::resolveCodeObject(*d, descriptorDir);
+  launch.preferCodeObject = d->codeObjectPreferred;
   return h->runner->runDynamicLibraryArtifact(launch, args);
 }
 

@@ -166,6 +166,7 @@ std::string serializeDescriptor(const HipKernelDescriptor &d) {
   if (!d.codeObject.empty()) {
     s += "code_object=" + d.codeObject + "\n";
     s += "code_object_dir=" + d.codeObjectDir + "\n";
+    if (d.codeObjectPreferred) s += "code_object_preferred=1\n";
   }
   if (!d.program.empty()) s += "program:\n" + d.program;
   return s;
@@ -190,6 +191,7 @@ Expected<HipKernelDescriptor> parseDescriptor(const std::string &text) {
   d.program = program;
   d.codeObject = kv["code_object"];
   d.codeObjectDir = kv["code_object_dir"];
+  d.codeObjectPreferred = kv["code_object_preferred"] == "1";
   if (d.hipKernel.empty()) return Status::error("artifact descriptor names no hip_kernel");
   const KnownKernel *k = findKnown(d.hipKernel);
   if (!k) return Status::error("artifact descriptor names an unknown hip_kernel: " + d.hipKernel);
@@ -368,6 +370,7 @@ Expected<KernelArtifact> compileArtifact(const CompileRequest &request) {
     if (object) {
       d.codeObject = *object;
       d.codeObjectDir = absolutePath(request.outputDir);
+      d.codeObjectPreferred = !request.emitOptions.empty();
     } else if (!request.emitOptions.empty() && object.error().find("hipcc") == std::string::npos &&
                object.error().find("AFIR_HIP_CODEGEN") == std::string::npos) {
       return Status::error("emit options: " + object.error());   // asked-for choices must not be dropped silently
@@ -388,6 +391,7 @@ Expected<KernelArtifact> compileArtifact(const CompileRequest &request) {
                  : (d.program.find("\nmatmul ") != std::string::npos ? KernelKind::Mix : known->kind);
   a.regionProgram = d.program;
   a.codeObjectPath = resolveCodeObject(d, request.outputDir);
+  a.codeObjectPreferred = d.codeObjectPreferred;
   a.codegenNote = codegenNote;
   a.socVersion = request.socVersion.empty() ? "gfx950" : request.socVersion;
   a.artifactRoot = request.outputDir;
@@ -447,6 +451,7 @@ Expected<KernelArtifact> loadArtifactFromRoot(const std::string &root) {
   if (a.sharedLibrarySymbol.empty()) a.sharedLibrarySymbol = d->symbol;
   a.regionProgram = d->program;
   a.codeObjectPath = resolveCodeObject(*d, root);
+  a.codeObjectPreferred = d->codeObjectPreferred;
   a.codegenNote = kv["code_object_note"];
   return a;
 }

@@ -99,6 +99,7 @@ class HipExecutionRunner final : public ExecutionRunner {
     dl.regionProgram = d->program;
     const size_t slash = launch.binaryPath.find_last_of('/');
     dl.codeObjectPath = resolveCodeObject(*d, slash == std::string::npos ? "." : launch.binaryPath.substr(0, slash));
+    dl.preferCodeObject = d->codeObjectPreferred;
     return runDynamicLibraryArtifact(dl, args);
   }
 
@@ -157,6 +158,11 @@ class HipExecutionRunner final : public ExecutionRunner {
         const std::string image((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
         if (attach(region, image.data(), image.size()) != 0)
           return Status::error("code object " + launch.codeObjectPath + " rejected: " + why());
+        if (launch.preferCodeObject) {
+          using PreferFn = uint32_t (*)(uint64_t, int);
+          auto prefer = reinterpret_cast<PreferFn>(dlsym(lib, "afir_hip_region_prefer_code_object"));
+          if (prefer) (void)prefer(region, 1);
+        }
       }
       if (Status st = validateRegion(lib, region, args, why); !st.ok()) return st;
     }
@@ -207,8 +213,10 @@ class HipExecutionRunner final : public ExecutionRunner {
     slots[idx++] = args.tiling.empty() ? nullptr : args.tiling.data();
 
     // ---- launch ----
-    (void)hipEventRecord(ev0_, stream_);
     const uint32_t bd = (uint32_t)(args.block_dim < 0 ? 0 : args.block_dim);
+    double bestUs = -1.0;
+    for (int rep = 0; rep <= (args.timing_repeats > 0 ? args.timing_repeats : 0); ++rep) {
+    (void)hipEventRecord(ev0_, stream_);
     uint32_t rc;
     if (regionLaunch) {
       const int nargs = (int)(args.inputs.size() + args.outputs.size());
@@ -230,11 +238,14 @@ class HipExecutionRunner final : public ExecutionRunner {
     hipError_t e = hipStreamSynchronize(stream_);
     if (e != hipSuccess) { cleanup(); return Status::error(hipErr("hipStreamSynchronize", e)); }
     float ms = 0.f;
-    if (hipEventElapsedTime(&ms, ev0_, ev1_) == hipSuccess) lastKernelUs_ = (double)ms * 1e3;
+    if (hipEventElapsedTime(&ms, ev0_, ev1_) == hipSuccess && (bestUs < 0 || (double)ms * 1e3 < bestUs))
+      bestUs = (double)ms * 1e3;
+    }
+    lastKernelUs_ = bestUs;
 
     // ---- data errors reported through the workspace ----
     int32_t flag = 0;
-    e = hipMemcpy(&flag, workspace, sizeof flag, hipMemcpyDeviceToHost);
+    hipError_t e = hipMemcpy(&flag, workspace, sizeof flag, hipMemcpyDeviceToHost);
     if (e != hipSuccess) { cleanup(); return Status::error(hipErr("hipMemcpy workspace", e)); }
     if (flag != 0) {
       cleanup();

@@ -94,6 +94,10 @@ struct RunArgs {
   std::vector<uint8_t> tiling;    // packed TilingData bytes (little-endian)
   int block_dim = 1;
   size_t workspace_size = 8192;
+  // Extra timed launches of the same kernel on the same device buffers (the
+  // kernels are pure functions of their inputs): the reported kernel time is the
+  // fastest of 1 + timing_repeats launches.  For searches that score by time.
+  int timing_repeats = 0;
 };
 
 // ------------------------------------------------------------------- npy ----
@@ -183,6 +187,7 @@ struct KernelArtifact {
   std::string regionProgram;        // fused_region artifacts: the program text
   std::string codeObjectPath;       // fused_region artifacts: kernels compiled for the program ("" = none)
   std::string codegenNote;          // why there is no code object, when there is none
+  bool codeObjectPreferred = false; // the code object outranks a matching hand-tuned family
 };
 
 // The descriptor a "compiled" fused region consists of on this backend: the
@@ -197,6 +202,7 @@ struct HipKernelDescriptor {
   // file name beside the descriptor, and the directory it was written to.
   std::string codeObject;
   std::string codeObjectDir;
+  bool codeObjectPreferred = false;   // compiled with explicit emit options: run it even where a hand-tuned family matches
 };
 // Path of the descriptor's code object: beside the descriptor when its
 // directory is known and the file is there, else where it was compiled; ""
@@ -289,6 +295,7 @@ struct DynamicLibraryExecutionLaunch {
   // Optional code object compiled for that program; attached after
   // registration so the launch runs the compiled kernels.
   std::string codeObjectPath;
+  bool preferCodeObject = false;
 };
 
 class ExecutionRunner {

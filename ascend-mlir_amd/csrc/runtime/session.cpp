@@ -201,6 +201,7 @@ SessionSummary runSingleTask(const RunTaskSpec &task, RunnerFactory factory, int
   launch.symbolName = artifact->sharedLibrarySymbol;
   launch.regionProgram = artifact->regionProgram;
   launch.codeObjectPath = artifact->codeObjectPath;
+  launch.preferCodeObject = artifact->codeObjectPreferred;
   if (Status st = runner->runDynamicLibraryArtifact(launch, args); !st.ok())
     return fail(summary, "kernel_launch", st.message);
   const double us = runner->lastKernelMicroseconds();

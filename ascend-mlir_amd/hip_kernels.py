@@ -48,6 +48,7 @@ EXPORTED_SYMBOLS = [
     "afir_hip_region_kernel",
     "afir_hip_region_emit_source",
     "afir_hip_region_attach_code_object",
+    "afir_hip_region_prefer_code_object",
     "afir_hip_region_argument_bytes",
     "afir_hip_launch_region",
 ]
@@ -382,6 +383,15 @@ class Region:
         _check(L.afir_hip_region_attach_code_object(ctypes.c_uint64(self.handle), image, len(image)))
         L.afir_hip_region_kernel.restype = ctypes.c_char_p
         self.kernel = L.afir_hip_region_kernel(ctypes.c_uint64(self.handle)).decode()
+
+    def prefer_code_object(self, prefer: bool = True):
+        """Run the attached code object even where a hand-tuned family matches."""
+        L = load()
+        L.afir_hip_region_prefer_code_object.argtypes = [ctypes.c_uint64, ctypes.c_int]
+        _check(L.afir_hip_region_prefer_code_object(ctypes.c_uint64(self.handle), 1 if prefer else 0))
+        L.afir_hip_region_kernel.restype = ctypes.c_char_p
+        self.kernel = L.afir_hip_region_kernel(ctypes.c_uint64(self.handle)).decode()
+        return self
 
     def compile(self, cache_dir: str = None):
         """Emit, compile with hipcc and attach; the code object is kept in

@@ -197,6 +197,12 @@ const char *afir_hip_region_kernel(uint64_t handle);
  * that kernel.  Matmul programs have no source form (AFIR_HIP_E_INVALID). */
 uint32_t afir_hip_region_emit_source(uint64_t handle, char *buffer, size_t capacity, size_t *length);
 uint32_t afir_hip_region_attach_code_object(uint64_t handle, const void *image, size_t image_len);
+/* prefer != 0: the attached code object runs even when the program is one of
+ * the hand-tuned families (which otherwise keep their kernel).  Used for
+ * artifacts compiled with explicit emit options and by tile searches, where
+ * the emitted kernel is the thing under test.  No counterpart in the
+ * reference, whose kernels are all generated. */
+uint32_t afir_hip_region_prefer_code_object(uint64_t handle, int prefer);
 /* Name of tiling field `index` ("" if out of range); valid until unregister. */
 const char *afir_hip_region_tiling_field(uint64_t handle, int index);
 uint32_t afir_hip_region_argument_bytes(uint64_t handle, const void *tiling, size_t tiling_len,

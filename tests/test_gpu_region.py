@@ -245,3 +245,24 @@ def test_code_object_of_another_program_is_rejected(H, evaluator, tmp_path):
     with pytest.raises(H.AfirHipError, match="not built from this program"):
         r(a, a, out_shape=(4, 8))
     r.close()
+
+
+def test_preferred_code_object_outranks_a_hand_tuned_family(H, evaluator, monkeypatch, tmp_path):
+    """A program that is exactly one of the hand-tuned families keeps that kernel
+    when a code object is attached, unless the code object is preferred."""
+    import torch
+    if evaluator != "compiled":
+        pytest.skip("one run is enough")
+    monkeypatch.setenv("AFIR_HIP_REGION_GENERIC", "0")
+    text, inputs, want = RC.case_c3()
+    r = H.Region(text)
+    assert r.kernel == "relu_broadcast_add_transpose"
+    r.compile(cache_dir=str(tmp_path))
+    assert r.kernel == "relu_broadcast_add_transpose"
+    r.prefer_code_object()
+    assert r.kernel == "fused_region_compiled"
+    got = r(*[torch.from_numpy(x).cuda() for x in inputs], out_shape=want.shape).cpu().numpy()
+    assert got.tobytes() == want.tobytes()
+    r.prefer_code_object(False)
+    assert r.kernel == "relu_broadcast_add_transpose"
+    r.close()
