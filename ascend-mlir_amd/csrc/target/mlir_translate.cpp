@@ -1135,7 +1135,7 @@ class Translator {
 
     static const struct { const char *n; OpCode c; } binary[] = {
         {"add", OpCode::Add}, {"sub", OpCode::Sub}, {"mul", OpCode::Mul}, {"div", OpCode::Div},
-        {"maximum", OpCode::Max}, {"minimum", OpCode::Min}};
+        {"maximum", OpCode::Max}, {"minimum", OpCode::Min}, {"truediv", OpCode::Div}};
     for (const auto &b : binary) {
       if (name != b.n) continue;
       if (in.size() != 2) r_.fail("afir." + name + " takes two operands");
@@ -1157,8 +1157,23 @@ class Translator {
       defineTensor(result, tv);
       return;
     }
+    {
+      static const char *const unary[] = {"load", "store", "abs", "relu", "neg", "leaky_relu", "broadcast", "sum"};
+      bool known = false;
+      for (const char *u : unary) known = known || name == u;
+      if (!known) r_.fail("afir." + name + " has no HIP lowering");
+    }
     if (in.size() != 1) r_.fail("afir." + name + " takes one operand");
-    if (name == "relu" || name == "neg" || name == "leaky_relu") {
+    if (name == "load" || name == "store") {
+      // data movement between global memory and the core in an AscGraph
+      // (include/Dialect/AFIR/Ops/Basic/data.td:31-32): the value itself
+      tv->shape = in[0]->shape;
+      tv->expr = in[0]->expr;
+    } else if (name == "abs") {
+      // |x| = maximum(x, -x): exact, +0 for both zeros, NaN stays NaN
+      tv->shape = in[0]->shape;
+      tv->expr = makeBinary(OpCode::Max, in[0]->expr, makeUnary(OpCode::Neg, in[0]->expr));
+    } else if (name == "relu" || name == "neg" || name == "leaky_relu") {
       tv->shape = in[0]->shape;
       if (name == "relu") tv->expr = makeUnary(OpCode::Relu, in[0]->expr);
       else if (name == "neg") tv->expr = makeUnary(OpCode::Neg, in[0]->expr);
@@ -1328,6 +1343,29 @@ class Translator {
 };
 
 }  // namespace
+
+std::string selectFunction(const std::string &text, const std::string &name) {
+  // positions of `func.func` outside of comments
+  std::vector<size_t> funcs;
+  for (size_t at = text.find("func.func"); at != std::string::npos; at = text.find("func.func", at + 9)) {
+    const size_t bol = text.rfind('\n', at);
+    const size_t comment = text.find("//", bol == std::string::npos ? 0 : bol);
+    if (comment == std::string::npos || comment > at) funcs.push_back(at);
+  }
+  if (funcs.empty()) return "";
+  for (size_t at : funcs) {
+    size_t p = at + 9;
+    auto skipSpace = [&]() { while (p < text.size() && isspace((unsigned char)text[p])) ++p; };
+    skipSpace();
+    for (const char *vis : {"private", "public"})
+      if (text.compare(p, std::strlen(vis), vis) == 0) { p += std::strlen(vis); skipSpace(); }
+    if (p >= text.size() || text[p] != '@') continue;
+    size_t e = p + 1;
+    while (e < text.size() && (isalnum((unsigned char)text[e]) || text[e] == '_' || text[e] == '.' || text[e] == '$')) ++e;
+    if (text.substr(p + 1, e - p - 1) == name) return text.substr(0, funcs[0]) + text.substr(at);
+  }
+  return "";
+}
 
 std::string translateMlirToRegion(const std::string &mlirText, Translation *out) {
   try {

@@ -28,7 +28,7 @@
 //     (examples/split-relu-brc-add-mul, examples/add-broadcast-concat);
 //   - AFIR ops in their custom syntax (afir.add / sub / mul / div / maximum /
 //     minimum with numpy-style broadcasting, relu, leaky_relu{negative_slop},
-//     neg, broadcast, sum{axis = last}; include/Dialect/AFIR/Ops/Basic/math.td:63-106,
+//     neg, broadcast, sum{axis = last}, load / store as the identity; include/Dialect/AFIR/Ops/Basic/math.td:63-106,
 //     lib/Dialect/AFIR/Ops/Basic/math.cpp:274-381).
 // Anything else is rejected with a diagnostic naming the construct.
 #pragma once
@@ -43,6 +43,12 @@ struct Translation {
   std::string functionName;
   afir_region::Program program;
 };
+
+// For files that hold several functions (the reference's lit tests do): the
+// text with everything between the leading aliases / module header and
+// `func.func @name` removed, so that it is the first function.  Returns "" when
+// there is no such function.
+std::string selectFunction(const std::string &mlirText, const std::string &name);
 
 // Translates the first func.func of `mlirText`.  Returns "" on success, else
 // the diagnostic ("line N: ...").

@@ -27,7 +27,7 @@
 #include "../target/mlir_translate.h"
 
 int main(int argc, char **argv) {
-  std::string input, output, tilingOut;
+  std::string input, output, tilingOut, function;
   bool toHip = false, emitSource = false;
   afir_target::EmitOptions emitOptions;
   for (int i = 1; i < argc; ++i) {
@@ -42,6 +42,10 @@ int main(int argc, char **argv) {
       toHip = true;
     } else if (a == "--emit-hip-source") {
       emitSource = true;
+    } else if (a.compare(0, 10, "--function") == 0) {
+      const char *v = value("--function");
+      if (!v) { std::fprintf(stderr, "afir-translate: --function needs a name\n"); return 2; }
+      function = v;
     } else if (a.compare(0, 14, "--emit-options") == 0) {
       const char *v = value("--emit-options");
       if (!v) { std::fprintf(stderr, "afir-translate: --emit-options needs name=value[,name=value]\n"); return 2; }
@@ -71,7 +75,7 @@ int main(int argc, char **argv) {
       if (!v) { std::fprintf(stderr, "afir-translate: --tiling-space-out needs a file name\n"); return 2; }
       tilingOut = v;
     } else if (a == "-h" || a == "--help") {
-      std::printf("usage: afir-translate -mlir-to-hip <input.mlir> [-o <file>] [--tiling-space-out <file>] [--emit-hip-source [--emit-options tile_p=64,tile_q=64,unroll=0]]\n");
+      std::printf("usage: afir-translate -mlir-to-hip <input.mlir> [-o <file>] [--tiling-space-out <file>] [--function NAME] [--emit-hip-source [--emit-options tile_p=64,tile_q=64,unroll=0]]\n");
       return 0;
     } else if (!a.empty() && a[0] == '-' && a != "-") {
       std::fprintf(stderr, "afir-translate: unknown option %s\n", a.c_str());
@@ -94,6 +98,13 @@ int main(int argc, char **argv) {
     std::ifstream f(input, std::ios::binary);
     if (!f) { std::fprintf(stderr, "afir-translate: cannot open %s\n", input.c_str()); return 2; }
     text.assign(std::istreambuf_iterator<char>(f), std::istreambuf_iterator<char>());
+  }
+  if (!function.empty()) {
+    text = afir_target::selectFunction(text, function);
+    if (text.empty()) {
+      std::fprintf(stderr, "%s: error: no function @%s\n", input.empty() ? "<stdin>" : input.c_str(), function.c_str());
+      return 1;
+    }
   }
   afir_target::Translation tr;
   std::string why;

@@ -174,6 +174,25 @@ func.func @mm_bias(%a : tensor<?x?xf16>, %b : tensor<?x?xf16>, %bias : tensor<?x
 MATMUL_PLAIN_BF16 = MATMUL_PLAIN_F16.replace("xf16", "xbf16").replace("f32", "bf16").replace("@mm_plain", "@mm_plain_bf16")
 MATMUL_BIAS_BF16 = MATMUL_BIAS_F16.replace("xf16", "xbf16").replace("f32", "bf16").replace("@mm_bias", "@mm_bias_bf16")
 
+# An AscGraph in AFIR form (the structure of python/afir-to-ascir/asc_graph.afir:1-13:
+# load, load, broadcast, add, mul, sub, store, every op with an attribute
+# dictionary): out = (x + y) - (x + y) * y with y broadcast over the rows.
+ASC_GRAPH_FORM = """
+#id = affine_map<(d0, d1) -> (d0, d1)>
+module attributes {afir.asc_graph_attr = #afir.asc_graph<axes = [<id = 0, name = "r", axis_type = Original, size = "12">, <id = 1, name = "c", axis_type = Original, size = "40">], type = Compute>} {
+  func.func @asc_graph(%x: tensor<12x40xf32>, %y: tensor<1x40xf32>) -> tensor<12x40xf32> {
+    %lx = afir.load %x {indexing_maps = [#id], ir_attr_def = {offset = "0"}, outputs = [#afir.asc_tensor<tensor_id = -1, position = <gm>>]} : tensor<12x40xf32> -> tensor<12x40xf32>
+    %ly = afir.load %y {indexing_maps = [#id], ir_attr_def = {offset = "0"}, outputs = [#afir.asc_tensor<tensor_id = -1, position = <gm>>]} : tensor<1x40xf32> -> tensor<1x40xf32>
+    %by = afir.broadcast %ly {indexing_maps = [#id], outputs = [#afir.asc_tensor<tensor_id = -1, position = <gm>>]} : tensor<1x40xf32> -> tensor<12x40xf32>
+    %s = afir.add %lx, %by {indexing_maps = [#id, #id, #id], outputs = [#afir.asc_tensor<tensor_id = -1, position = <gm>>]} : (tensor<12x40xf32>, tensor<12x40xf32>) -> tensor<12x40xf32>
+    %p = afir.mul %s, %by {indexing_maps = [#id, #id, #id], outputs = [#afir.asc_tensor<tensor_id = -1, position = <gm>>]} : (tensor<12x40xf32>, tensor<12x40xf32>) -> tensor<12x40xf32>
+    %d = afir.sub %s, %p {indexing_maps = [#id, #id, #id], outputs = [#afir.asc_tensor<tensor_id = -1, position = <gm>>]} : (tensor<12x40xf32>, tensor<12x40xf32>) -> tensor<12x40xf32>
+    %o = afir.store %d {indexing_maps = [#id], outputs = [#afir.asc_tensor<tensor_id = -1, position = <gm>>]} : tensor<12x40xf32> -> tensor<12x40xf32>
+    return %o : tensor<12x40xf32>
+  }
+}
+"""
+
 TWO_CHAINS_CONCAT = """
 #row = affine_map<(d0, d1) -> (d0)>
 #all = affine_map<(d0, d1) -> (d0, d1)>

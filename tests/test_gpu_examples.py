@@ -321,3 +321,25 @@ def test_reference_multikernel_manifests(tmp_path, case):
     for line in ("session.backend=hip", "session.result=success", "session.validation=pass"):
         assert line in lines, p.stdout
     assert np.load(out / "output.npy").tobytes() == np.load(out / "expected.npy").tobytes()
+
+
+def test_asc_graph_form_runs_interpreted_and_compiled(pkg, monkeypatch, tmp_path):
+    """The AscGraph form (load / broadcast / add / mul / sub / store) through the
+    translator onto the GPU, on the interpreter kernel and on its compiled kernel."""
+    import torch
+    from ascend_mlir_amd import hip_kernels as H
+    from oracle import region_oracle as RO
+    H.load()
+    p = subprocess.run([TR, "-mlir-to-hip", "-"], input=MC.ASC_GRAPH_FORM, capture_output=True, text=True)
+    assert p.returncode == 0, p.stderr
+    rng = np.random.default_rng(4)
+    x = rng.uniform(-2, 2, (12, 40)).astype(np.float32)
+    y = rng.uniform(-2, 2, (1, 40)).astype(np.float32)
+    want = RO.evaluate(p.stdout, [x, y])
+    r = H.Region(p.stdout)
+    dev = [torch.from_numpy(x).cuda(), torch.from_numpy(y).cuda()]
+    assert r(*dev, out_shape=(12, 40)).cpu().numpy().tobytes() == want.tobytes()
+    r.compile(cache_dir=str(tmp_path))
+    assert r.kernel == "fused_region_compiled"
+    assert r(*dev, out_shape=(12, 40)).cpu().numpy().tobytes() == want.tobytes()
+    r.close()

@@ -175,6 +175,65 @@ def test_reference_example_inputs_translate_and_evaluate(example, case):
     assert RO.evaluate(p.stdout, inputs).tobytes() == want.tobytes()
 
 
+def test_asc_graph_form_with_load_store_and_attribute_dictionaries():
+    out = program_of(MC.ASC_GRAPH_FORM)
+    body = [l.strip() for l in out.splitlines() if l.strip() and not l.startswith("#")]
+    assert body[body.index("outoff 0") + 1:] == [
+        "push arg0 d0 d1", "push arg1 0 d1", "add", "push arg0 d0 d1", "push arg1 0 d1", "add", "push arg1 0 d1",
+        "mul", "sub", "store", "end"]
+    rng = np.random.default_rng(4)
+    x = rng.uniform(-2, 2, (12, 40)).astype(np.float32)
+    y = rng.uniform(-2, 2, (1, 40)).astype(np.float32)
+    s = x + y
+    assert RO.evaluate(out, [x, y]).tobytes() == (s - s * y).astype(np.float32).tobytes()
+
+
+@pytest.mark.skipif(not os.path.isfile("/root/reference/python/afir-to-ascir/asc_graph.afir"),
+                    reason="reference tree not present")
+def test_reference_asc_graph_file_translates():
+    p = subprocess.run([TR, "-mlir-to-hip", "/root/reference/python/afir-to-ascir/asc_graph.afir"],
+                       capture_output=True, text=True)
+    assert p.returncode == 0, p.stderr
+    assert "# kernel HashCopyAscGraph" in p.stdout and p.stdout.rstrip().endswith("mul\nsub\nstore\nend")
+
+
+AFIR_LIT = "/root/reference/test/Dialect/AFIR/ops.mlir"
+
+
+@pytest.mark.skipif(not os.path.isfile(AFIR_LIT), reason="reference tree not present")
+def test_reference_afir_lit_functions_translate():
+    """The functions of the reference's AFIR round-trip test that use ops on this
+    path (binary math, relu / neg / leaky_relu / abs, broadcast, sum, load /
+    store, with their attribute dictionaries) translate one by one; an op
+    outside the path is refused by name."""
+    good = ["test_add", "test_sub", "test_mul", "test_div", "test_truediv", "test_minimum", "test_maximum",
+            "test_relu", "test_neg", "test_leaky_relu", "test_abs", "test_abs_f16", "test_broadcast", "test_load",
+            "test_store", "test_sum_reduce", "test_reduce_3d", "test_binary_1d", "test_binary_3d", "test_unary_1d",
+            "test_unary_3d", "test_add_output_double_buffer", "test_abs_output_vector_out"]
+    for fn in good:
+        p = subprocess.run([TR, "-mlir-to-hip", AFIR_LIT, "--function", fn], capture_output=True, text=True)
+        assert p.returncode == 0, (fn, p.stderr)
+        assert p.stdout.startswith(f"# kernel {fn}\nafir-hip-region 1\n") and p.stdout.rstrip().endswith("store\nend")
+    for fn, op in (("test_exp", "afir.exp"), ("test_eq", "afir.eq"), ("test_cast_f16_to_f32", "afir.cast")):
+        p = subprocess.run([TR, "-mlir-to-hip", AFIR_LIT, "--function", fn], capture_output=True, text=True)
+        assert p.returncode == 1 and f"{op} has no HIP lowering" in p.stderr, (fn, p.stderr)
+    p = subprocess.run([TR, "-mlir-to-hip", AFIR_LIT, "--function", "nope"], capture_output=True, text=True)
+    assert p.returncode == 1 and "no function @nope" in p.stderr
+
+
+def test_abs_is_maximum_of_x_and_minus_x():
+    text = """func.func @a(%x: tensor<2x5xf32>) -> tensor<2x5xf32> {
+  %0 = afir.abs %x : tensor<2x5xf32> -> tensor<2x5xf32>
+  return %0 : tensor<2x5xf32>
+}"""
+    out = program_of(text)
+    assert "push arg0 d0 d1\npush arg0 d0 d1\nneg\nmax\nstore" in out
+    x = np.array([[-0.0, 0.0, -1.5, 2.0, -np.inf], [np.nan, 1e-40, -1e-40, 3.0, -3.0]], np.float32)
+    got = RO.evaluate(out, [x])
+    want = np.abs(x)
+    assert ((got.view(np.uint32) == want.view(np.uint32)) | (np.isnan(got) & np.isnan(want))).all()
+
+
 @pytest.mark.skipif(not os.path.isdir(REF_EXAMPLES), reason="reference tree not present")
 def test_reference_matmul_example_translates():
     p = subprocess.run([TR, "-mlir-to-hip", os.path.join(REF_EXAMPLES, "matmul-add-leakyrelu", "step0_input.mlir")],
