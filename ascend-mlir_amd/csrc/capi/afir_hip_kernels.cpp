@@ -165,7 +165,7 @@ std::string detect_fast_path(RegisteredRegion *r) {
   const afir_region::Program &p = r->program;
   if (p.segments.size() != 1) return "";
   const afir_region::Segment &g = p.segments[0];
-  if (g.outOffset.arg >= 0 || g.outOffset.constant != 0) return "";
+  if (g.outOffset.arg >= 0 || g.outOffset.constant != 0 || !g.outOffsetMore.empty()) return "";
   const std::vector<afir_region::Op> &ops = g.ops;
   auto type = [&](int a) { return p.args[a].type; };
   const ElemType out = p.output().type;

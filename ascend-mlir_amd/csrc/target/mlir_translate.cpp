@@ -1065,6 +1065,8 @@ class Translator {
     int64_t axis = 0;
     bool hasSlope = false;
     double slope = 0.0;
+    bool hasConcatAxis = false;
+    int64_t concatAxis = 0;
   };
   AfirAttrs parseAfirAttrs() {
     AfirAttrs a;
@@ -1076,6 +1078,10 @@ class Translator {
       if (key == "axis") {
         a.hasAxis = true;
         a.axis = r_.integer();
+        if (r_.eat(':')) parseType();
+      } else if (key == "concat_axis") {
+        a.hasConcatAxis = true;
+        a.concatAxis = r_.integer();
         if (r_.eat(':')) parseType();
       } else if (key == "negative_slop" || key == "negative_slope") {
         a.hasSlope = true;
@@ -1114,6 +1120,24 @@ class Translator {
     do operands.push_back(r_.ssa()); while (r_.eat(','));
     AfirAttrs attrs = parseAfirAttrs();
     r_.expect(':');
+    if (name == "concat") {
+      // afir.concat %a, %b, ... {concat_axis = 0 : i32} : ta, tb, ... -> tr: along the
+      // rows it is the row-range segmentation of tensor.concat dim(0)
+      if (!attrs.hasConcatAxis || attrs.concatAxis != 0) r_.fail("afir.concat is supported along axis 0 only");
+      do parseType(); while (r_.eat(','));
+      if (!r_.eatArrow()) r_.fail("expected '->' in afir.concat");
+      TypeInfo rt = parseType();
+      auto tv = std::make_shared<Tensor>();
+      for (const std::string &o : operands) {
+        TensorP p = tensorOf(o);
+        if (!p->expr || p->reduced || !p->parts.empty()) r_.fail("afir.concat operand is not an elementwise value");
+        tv->parts.push_back(p);
+      }
+      tv->elem = rt.elemKnown ? rt.elem : tv->parts[0]->elem;
+      tv->shape = tv->parts[0]->shape;
+      defineTensor(result, tv);
+      return;
+    }
     std::vector<TypeInfo> inTypes;
     if (r_.eat('(')) {
       do inTypes.push_back(parseType()); while (r_.eat(','));
@@ -1314,16 +1338,23 @@ class Translator {
     if (!afir_region::isFloat(o.type)) r_.fail("the function must return a floating-point tensor");
     p.args.push_back(o);
     if (!result->parts.empty()) {
-      Ref offset = Ref::value(0);
+      // first row of each part: the sum of the parts before it (constants folded)
+      int64_t constant = 0;
+      std::vector<Ref> terms;
       for (size_t i = 0; i < result->parts.size(); ++i) {
         const TensorP &part = result->parts[i];
-        emitSegment(part, offset, &p);
-        const Ref &rows = part->shape[0];
-        if (i + 1 < result->parts.size()) {
-          if (offset.arg < 0 && offset.constant == 0) offset = rows;
-          else if (offset.arg < 0 && rows.arg < 0) offset = Ref::value(offset.constant + rows.constant);
-          else r_.fail("tensor.concat of more than two dynamically sized operands is not supported");
+        emitSegment(part, Ref::value(0), &p);
+        afir_region::Segment &g = p.segments.back();
+        if (terms.empty()) {
+          g.outOffset = Ref::value(constant);
+        } else {
+          g.outOffset = terms[0];
+          g.outOffsetMore.assign(terms.begin() + 1, terms.end());
+          if (constant) g.outOffsetMore.push_back(Ref::value(constant));
         }
+        const Ref &rows = part->shape[0];
+        if (rows.arg < 0) constant += rows.constant;
+        else terms.push_back(rows);
       }
     } else {
       if (!result->expr) r_.fail("the function returns an uninitialised tensor");

@@ -115,7 +115,9 @@ std::string serialize(const Program &p) {
     s += "segment " + std::to_string(g.rank) + "\n";
     s += "size";
     for (const Ref &r : g.sizes) s += " " + refText(r);
-    s += "\noutoff " + refText(g.outOffset) + "\n";
+    s += "\noutoff " + refText(g.outOffset);
+    for (const Ref &r : g.outOffsetMore) s += " " + refText(r);
+    s += "\n";
     for (const Op &o : g.ops) {
       switch (o.code) {
         case OpCode::Push: {
@@ -200,7 +202,12 @@ std::string parse(const std::string &text, Program *out) {
         seg->sizes.push_back(r);
       }
     } else if (k == "outoff") {
-      if (tok.size() != 2 || !parseRef(tok[1], &seg->outOffset)) return err(lineno, "expected 'outoff <ref>'");
+      if (tok.size() < 2 || !parseRef(tok[1], &seg->outOffset)) return err(lineno, "expected 'outoff <ref> [<ref> ...]'");
+      for (size_t i = 2; i < tok.size(); ++i) {
+        Ref r;
+        if (!parseRef(tok[i], &r)) return err(lineno, "bad output offset term '" + tok[i] + "'");
+        seg->outOffsetMore.push_back(r);
+      }
     } else if (k == "push") {
       Op o;
       o.code = OpCode::Push;
@@ -303,6 +310,8 @@ std::string validate(const Program &p) {
     for (const Ref &r : g.sizes)
       if (!refOk(r)) return "region program: bad extent reference";
     if (!refOk(g.outOffset)) return "region program: bad output offset reference";
+    for (const Ref &r : g.outOffsetMore)
+      if (!refOk(r)) return "region program: bad output offset reference";
     if (g.ops.empty() || g.ops.back().code != OpCode::Store) return "region program: a segment must end with 'store'";
     if ((int)g.ops.size() > kMaxOps) return "region program: too many operations in a segment";
     int depth = 0, pushes = 0;
@@ -421,7 +430,8 @@ std::string resolve(const Program &p, const std::vector<int64_t> &dims, Resolved
     s.outType = p.output().type;
     for (int k = 0; k < g.rank; ++k) s.size[k] = value(g.sizes[k]);
     const int outRank = g.rank - (s.reduce ? 1 : 0);
-    const int64_t off0 = value(g.outOffset);
+    int64_t off0 = value(g.outOffset);
+    for (const Ref &r : g.outOffsetMore) off0 += value(r);
     if (outRank == 0) return "region: scalar outputs are not supported";
     for (int d = 1; d < outRank; ++d)
       if (oshape[d] != s.size[d]) return "region: segment extent does not match the output shape";

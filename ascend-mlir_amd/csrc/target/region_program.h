@@ -25,7 +25,7 @@
 //   arg out <f16|bf16|f32> <rank>              inputs first, then the output
 //   segment <iteration rank>
 //     size <ref> <ref> ...      extent of each iteration dim: argA.D or a constant
-//     outoff <ref>              first output row (dim 0) this segment writes
+//     outoff <ref> [<ref> ...]  first output row (dim 0) this segment writes: the sum of the terms
 //     push argA <m0> <m1> ... [slice <ref> ...]
 //                               read input A; m_r is d<k> (iteration dim k), an
 //                               integer constant, or g<k>:argI (dim r is indexed
@@ -97,6 +97,7 @@ struct Segment {
   int rank = 0;
   std::vector<Ref> sizes;
   Ref outOffset = Ref::value(0);
+  std::vector<Ref> outOffsetMore;   // further terms added to outOffset (concat of 3+ dynamic parts)
   std::vector<Op> ops;
   bool reduces() const;
 };

@@ -67,14 +67,14 @@ def parse(text: str) -> dict:
         if k == "arg":
             args.append((tok[1], tok[2], int(tok[3])))
         elif k == "segment":
-            seg = {"rank": int(tok[1]), "size": [], "outoff": ("const", 0), "ops": []}
+            seg = {"rank": int(tok[1]), "size": [], "outoff": [("const", 0)], "ops": []}
             segments.append(seg)
         elif k == "end":
             seg = None
         elif k == "size":
             seg["size"] = [_ref(t) for t in tok[1:]]
         elif k == "outoff":
-            seg["outoff"] = _ref(tok[1])
+            seg["outoff"] = [_ref(t) for t in tok[1:]]      # terms, summed
         elif k == "push":
             arg = int(tok[1][3:])
             rest = tok[2:]
@@ -200,7 +200,7 @@ def evaluate(text: str, inputs):
                 raise RegionError(f"unknown op {k}")
         if len(stack) != 1:
             raise RegionError("stack does not hold exactly one value at store")
-        pieces.append((val(seg["outoff"]), stack[0], reduced))
+        pieces.append((sum(val(t) for t in seg["outoff"]), stack[0], reduced))
     pieces.sort(key=lambda p: p[0])
     res = np.concatenate([p[1] for p in pieces], axis=0)
     if res.ndim != out_rank:

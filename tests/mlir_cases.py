@@ -193,6 +193,17 @@ module attributes {afir.asc_graph_attr = #afir.asc_graph<axes = [<id = 0, name =
 }
 """
 
+# afir.concat of three parts along axis 0 (the op form of
+# test/Dialect/AFIR/ops.mlir:350-355), each part an elementwise value.
+THREE_PART_CONCAT = """
+func.func @concat3(%a: tensor<?x?xf32>, %b: tensor<?x?xf32>, %c: tensor<?x?xf32>) -> tensor<?x?xf32> {
+  %ra = afir.relu %a : tensor<?x?xf32> -> tensor<?x?xf32>
+  %nb = afir.neg %b : tensor<?x?xf32> -> tensor<?x?xf32>
+  %0 = afir.concat %ra, %nb, %c {concat_axis = 0 : i32} : tensor<?x?xf32>, tensor<?x?xf32>, tensor<?x?xf32> -> tensor<?x?xf32>
+  return %0 : tensor<?x?xf32>
+}
+"""
+
 TWO_CHAINS_CONCAT = """
 #row = affine_map<(d0, d1) -> (d0)>
 #all = affine_map<(d0, d1) -> (d0, d1)>

@@ -343,3 +343,21 @@ def test_asc_graph_form_runs_interpreted_and_compiled(pkg, monkeypatch, tmp_path
     assert r.kernel == "fused_region_compiled"
     assert r(*dev, out_shape=(12, 40)).cpu().numpy().tobytes() == want.tobytes()
     r.close()
+
+
+def test_concat_of_three_parts_runs_interpreted_and_compiled(pkg, tmp_path):
+    import torch
+    from ascend_mlir_amd import hip_kernels as H
+    H.load()
+    p = subprocess.run([TR, "-mlir-to-hip", "-"], input=MC.THREE_PART_CONCAT, capture_output=True, text=True)
+    assert p.returncode == 0, p.stderr
+    rng = np.random.default_rng(2)
+    a, b, c = (rng.uniform(-1, 1, (r, 70)).astype(np.float32) for r in (33, 5, 120))
+    want = np.concatenate([np.maximum(a, 0), -b, c], axis=0)
+    r = H.Region(p.stdout)
+    dev = [torch.from_numpy(x).cuda() for x in (a, b, c)]
+    assert r(*dev, out_shape=want.shape).cpu().numpy().tobytes() == want.tobytes()
+    r.compile(cache_dir=str(tmp_path))        # three segments in one launch
+    assert "afir_region_all_i32_g" in r.emit_source()
+    assert r(*dev, out_shape=want.shape).cpu().numpy().tobytes() == want.tobytes()
+    r.close()

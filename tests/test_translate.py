@@ -221,6 +221,16 @@ def test_reference_afir_lit_functions_translate():
     assert p.returncode == 1 and "no function @nope" in p.stderr
 
 
+def test_concat_of_three_parts_sums_the_row_offsets():
+    out = program_of(MC.THREE_PART_CONCAT)
+    offs = [l for l in out.splitlines() if l.startswith("outoff")]
+    assert offs == ["outoff 0", "outoff arg0.0", "outoff arg0.0 arg1.0"]
+    rng = np.random.default_rng(2)
+    a, b, c = (rng.uniform(-1, 1, (r, 7)).astype(np.float32) for r in (3, 5, 2))
+    want = np.concatenate([np.maximum(a, 0), -b, c], axis=0)
+    assert RO.evaluate(out, [a, b, c]).tobytes() == want.tobytes()
+
+
 def test_abs_is_maximum_of_x_and_minus_x():
     text = """func.func @a(%x: tensor<2x5xf32>) -> tensor<2x5xf32> {
   %0 = afir.abs %x : tensor<2x5xf32> -> tensor<2x5xf32>
