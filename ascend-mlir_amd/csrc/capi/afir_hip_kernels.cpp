@@ -269,12 +269,33 @@ int region_type_code(afir_region::ElemType t) {
     case afir_region::ElemType::F32: return afir::kRegionF32;
     case afir_region::ElemType::I32: return afir::kRegionI32;
     case afir_region::ElemType::I64: return afir::kRegionI64;
+    case afir_region::ElemType::I16: return afir::kRegionI16;
   }
   return afir::kRegionF32;
 }
 
-int region_op_code(afir_region::OpCode c) {
+int region_op_code(afir_region::OpCode c, bool integer, bool narrow = false) {
   using afir_region::OpCode;
+  if (integer && narrow) {
+    switch (c) {
+      case OpCode::Max: return afir::kRegionMaxI16;
+      case OpCode::Min: return afir::kRegionMinI16;
+      case OpCode::Relu: return afir::kRegionReluI16;
+      default: break;
+    }
+  }
+  if (integer) {
+    switch (c) {
+      case OpCode::Add: return afir::kRegionAddI;
+      case OpCode::Sub: return afir::kRegionSubI;
+      case OpCode::Mul: return afir::kRegionMulI;
+      case OpCode::Max: return afir::kRegionMaxI;
+      case OpCode::Min: return afir::kRegionMinI;
+      case OpCode::Relu: return afir::kRegionReluI;
+      case OpCode::Neg: return afir::kRegionNegI;
+      default: break;   // push, const, dup as below; the rest does not occur (validate)
+    }
+  }
   switch (c) {
     case OpCode::Push: return afir::kRegionPush;
     case OpCode::Const: return afir::kRegionConst;
@@ -618,12 +639,17 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
     }
     a.nops = 0;
     for (const afir_region::ResolvedOp &op : seg.ops) {
-      const int code = region_op_code(op.code);
+      const bool integer = afir_region::isRegionInt(seg.outType);
+      const int code = region_op_code(op.code, integer, seg.outType == afir_region::ElemType::I16);
       if (code < 0) continue;
       afir::RegionOp &d = a.ops[a.nops++];
       d.code = code;
       d.input = op.input;
       d.constant = op.constant;
+      if (integer && op.code == afir_region::OpCode::Const) {   // the integer, bit for bit
+        const int32_t iv = (int32_t)op.constant;
+        std::memcpy(&d.constant, &iv, sizeof iv);
+      }
       d.depth = op.depth;
     }
     if (compiled) {

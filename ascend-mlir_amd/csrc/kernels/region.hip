@@ -40,7 +40,8 @@ namespace {
 constexpr int kThreads = 256;
 
 __device__ __forceinline__ float load_elem(const void *base, int type, int64_t i) {
-  if (type == kRegionF32) return static_cast<const float *>(base)[i];
+  if (type == kRegionF32 || type == kRegionI32) return static_cast<const float *>(base)[i];   // i32: the bits
+  if (type == kRegionI16) return __int_as_float((int)static_cast<const int16_t *>(base)[i]);
   const uint32_t h = static_cast<const uint16_t *>(base)[i];
   if (type == kRegionF16) return (float)__builtin_bit_cast(_Float16, (uint16_t)h);
   return __uint_as_float(h << 16);
@@ -48,7 +49,7 @@ __device__ __forceinline__ float load_elem(const void *base, int type, int64_t i
 
 template <int V>
 __device__ __forceinline__ void load_vec(const void *base, int type, int64_t i, float (&v)[V]) {
-  if (type == kRegionF32) {
+  if (type == kRegionF32 || type == kRegionI32) {
     const f32x4 *p = reinterpret_cast<const f32x4 *>(static_cast<const float *>(base) + i);
 #pragma unroll
     for (int q = 0; q < V / 4; ++q) {
@@ -64,6 +65,10 @@ __device__ __forceinline__ void load_vec(const void *base, int type, int64_t i, 
 #pragma unroll
       for (int d = 0; d < 4; ++d) {
         if (type == kRegionF16) { v[8 * q + 2 * d] = f16_lo(raw[d]); v[8 * q + 2 * d + 1] = f16_hi(raw[d]); }
+        else if (type == kRegionI16) {   // sign-extended
+          v[8 * q + 2 * d] = __int_as_float((int)(raw[d] << 16) >> 16);
+          v[8 * q + 2 * d + 1] = __int_as_float((int)raw[d] >> 16);
+        }
         else { v[8 * q + 2 * d] = bf16_lo(raw[d]); v[8 * q + 2 * d + 1] = bf16_hi(raw[d]); }
       }
     }
@@ -89,7 +94,8 @@ __device__ __forceinline__ void read_operand(const RegionInput &in, int last, co
   // element position without the gathered dim
   I pos = (I)in.offset + at.x0 * (I)in.stride[0] + at.x1 * (I)in.stride[1] + at.x2 * (I)in.stride[2];
   const I step = (I)(last == 0 ? in.stride[0] : (last == 1 ? in.stride[1] : in.stride[2]));
-  const float nan = __uint_as_float(0x7fc00000u);
+  // what an out-of-range gather yields: NaN, or 0 in an integer region
+  const float nan = (in.type == kRegionI32 || in.type == kRegionI16) ? 0.f : __uint_as_float(0x7fc00000u);
 
   if (in.gdim >= 0 && in.gdim == last) {
     // gathered along the innermost dim: one index per element
@@ -173,6 +179,41 @@ __device__ __forceinline__ void binary(int code, float (&a)[V], const float (&b)
 #pragma unroll
       for (int e = 0; e < V; ++e) a[e] = fmin_nan(a[e], b[e]);
       break;
+    // 32-bit two's complement, wrapping (unsigned arithmetic)
+    case kRegionAddI:
+#pragma unroll
+      for (int e = 0; e < V; ++e) a[e] = __uint_as_float(__float_as_uint(a[e]) + __float_as_uint(b[e]));
+      break;
+    case kRegionSubI:
+#pragma unroll
+      for (int e = 0; e < V; ++e) a[e] = __uint_as_float(__float_as_uint(a[e]) - __float_as_uint(b[e]));
+      break;
+    case kRegionMulI:
+#pragma unroll
+      for (int e = 0; e < V; ++e) a[e] = __uint_as_float(__float_as_uint(a[e]) * __float_as_uint(b[e]));
+      break;
+    case kRegionMaxI:
+#pragma unroll
+      for (int e = 0; e < V; ++e) a[e] = __float_as_int(a[e]) > __float_as_int(b[e]) ? a[e] : b[e];
+      break;
+    case kRegionMinI:
+#pragma unroll
+      for (int e = 0; e < V; ++e) a[e] = __float_as_int(a[e]) < __float_as_int(b[e]) ? a[e] : b[e];
+      break;
+    case kRegionMaxI16:
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const int x = (short)__float_as_int(a[e]), y = (short)__float_as_int(b[e]);
+        a[e] = __int_as_float(x > y ? x : y);
+      }
+      break;
+    case kRegionMinI16:
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const int x = (short)__float_as_int(a[e]), y = (short)__float_as_int(b[e]);
+        a[e] = __int_as_float(x < y ? x : y);
+      }
+      break;
     default:
       break;
   }
@@ -192,6 +233,21 @@ __device__ __forceinline__ void unary(int code, float c, float (&a)[V]) {
     case kRegionNeg:
 #pragma unroll
       for (int e = 0; e < V; ++e) a[e] = -a[e];
+      break;
+    case kRegionReluI:
+#pragma unroll
+      for (int e = 0; e < V; ++e) a[e] = __float_as_int(a[e]) > 0 ? a[e] : 0.f;
+      break;
+    case kRegionNegI:
+#pragma unroll
+      for (int e = 0; e < V; ++e) a[e] = __uint_as_float(0u - __float_as_uint(a[e]));
+      break;
+    case kRegionReluI16:
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const int x = (short)__float_as_int(a[e]);
+        a[e] = __int_as_float(x > 0 ? x : 0);
+      }
       break;
     default:
       break;
@@ -230,7 +286,7 @@ __device__ __forceinline__ void evaluate(const RegionArgs &R, int last, const Po
         case 2: assign(s2, t); break;
         default: assign(s3, t); break;
       }
-    } else if (op.code <= kRegionMin) {   // binary: slot dst (op) slot dst + 1
+    } else if (region_is_binary(op.code)) {   // binary: slot dst (op) slot dst + 1
       switch (op.dst) {
         case 0: binary(op.code, s0, s1); break;
         case 1: binary(op.code, s1, s2); break;
@@ -279,6 +335,9 @@ __device__ __forceinline__ void evaluate_chain(const RegionArgs &R, int last, co
     } else if (st.bop == kChainRDiv) {
 #pragma unroll
       for (int e = 0; e < V; ++e) acc[e] = x[e] / acc[e];
+    } else if (st.bop == kChainRSubI) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] = __uint_as_float(__float_as_uint(x[e]) - __float_as_uint(acc[e]));
     } else {
       binary(st.bop, acc, x);
     }
@@ -294,7 +353,8 @@ __device__ __forceinline__ void evaluate_any(const RegionArgs &R, int last, cons
 }
 
 __device__ __forceinline__ void store_elem(void *out, int type, int64_t i, float x) {
-  if (type == kRegionF32) static_cast<float *>(out)[i] = x;
+  if (type == kRegionF32 || type == kRegionI32) static_cast<float *>(out)[i] = x;   // i32: the bits
+  else if (type == kRegionI16) static_cast<uint16_t *>(out)[i] = (uint16_t)__float_as_uint(x);
   else if (type == kRegionF16) static_cast<uint16_t *>(out)[i] = __builtin_bit_cast(uint16_t, (_Float16)x);
   else static_cast<uint16_t *>(out)[i] = (uint16_t)f32_to_bf16_rne(x);
 }
@@ -339,7 +399,7 @@ __global__ __launch_bounds__(kThreads) void fused_region_parallel(const RegionAr
       evaluate_any<I, CHAIN, V>(R, last, position<I>(R, row, j0), nvalid, full, v);
       const int64_t o = (int64_t)row * n + j0;
       if (full && R.out_vec) {
-        if (R.out_type == kRegionF32) {
+        if (R.out_type == kRegionF32 || R.out_type == kRegionI32) {
           f32x4 *p = reinterpret_cast<f32x4 *>(static_cast<float *>(R.out) + o);
 #pragma unroll
           for (int q = 0; q < V / 4; ++q) {
@@ -356,7 +416,9 @@ __global__ __launch_bounds__(kThreads) void fused_region_parallel(const RegionAr
 #pragma unroll
             for (int d = 0; d < 4; ++d)
               w[d] = R.out_type == kRegionF16 ? pack_f16(v[8 * q + 2 * d], v[8 * q + 2 * d + 1])
-                                              : pack_bf16(v[8 * q + 2 * d], v[8 * q + 2 * d + 1]);
+                     : R.out_type == kRegionI16
+                         ? ((__float_as_uint(v[8 * q + 2 * d]) & 0xffffu) | (__float_as_uint(v[8 * q + 2 * d + 1]) << 16))
+                         : pack_bf16(v[8 * q + 2 * d], v[8 * q + 2 * d + 1]);
             p[q] = w;
           }
         }
@@ -422,7 +484,8 @@ bool linearize(RegionArgs &a) {
   a.nsteps = 0;
   a.chain_after_first = RegionUnary{};
   auto reversed = [](int code) {
-    return code == kRegionSub ? (int)kChainRSub : (code == kRegionDiv ? (int)kChainRDiv : code);
+    return code == kRegionSub ? (int)kChainRSub
+                              : (code == kRegionDiv ? (int)kChainRDiv : (code == kRegionSubI ? (int)kChainRSubI : code));
   };
   auto add_unary = [](RegionUnary &u, int code, float alpha) {
     if (u.count >= 2) return false;
@@ -455,7 +518,7 @@ bool linearize(RegionArgs &a) {
       stack[depth++] = e;
     } else if (op.code == kRegionDup) {
       return false;
-    } else if (op.code >= kRegionAdd && op.code <= kRegionMin) {
+    } else if (region_is_binary(op.code)) {
       Entry &x = stack[depth - 2], &y = stack[depth - 1];
       if (x.chain && y.chain) return false;
       if (x.chain) {
@@ -558,11 +621,11 @@ LaunchStatus launch_fused_region(const RegionArgs &args_in, uint32_t block_dim, 
       op.dst = depth++;
       if (depth > 4) return invalid("fused_region: more than 4 live values");
       if (op.code == kRegionPush && (op.input < 0 || op.input >= args.ninputs)) return invalid("fused_region: bad operand");
-    } else if (op.code >= kRegionAdd && op.code <= kRegionMin) {
+    } else if (region_is_binary(op.code)) {
       if (depth < 2) return invalid("fused_region: binary operation on fewer than two values");
       op.dst = depth - 2;
       --depth;
-    } else if (op.code == kRegionRelu || op.code == kRegionLeaky || op.code == kRegionNeg) {
+    } else if (region_is_unary(op.code)) {
       if (depth < 1) return invalid("fused_region: unary operation on an empty stack");
       op.dst = depth - 1;
     } else {
@@ -578,8 +641,8 @@ LaunchStatus launch_fused_region(const RegionArgs &args_in, uint32_t block_dim, 
 
   // 32 bytes per lane and operand: 8 elements, or 16 when every tensor of a
   // chain is 16-bit (twice the bytes per interpreted step)
-  bool wide = args.chain && args.out_type != kRegionF32;
-  for (int i = 0; i < args.ninputs; ++i) wide = wide && args.in[i].type != kRegionF32;
+  bool wide = args.chain && region_is_16bit(args.out_type);
+  for (int i = 0; i < args.ninputs; ++i) wide = wide && region_is_16bit(args.in[i].type);
   const int vec = wide ? 16 : 8;
 
   RegionGeometry g;

@@ -12,11 +12,28 @@ namespace afir {
 constexpr int kRegionMaxInputs = 8;
 constexpr int kRegionMaxOps = 32;
 
-enum RegionType : int { kRegionF16 = 0, kRegionBF16 = 1, kRegionF32 = 2, kRegionI32 = 3, kRegionI64 = 4 };
+enum RegionType : int { kRegionF16 = 0, kRegionBF16 = 1, kRegionF32 = 2, kRegionI32 = 3, kRegionI64 = 4, kRegionI16 = 5 };
+// Values travel through float registers; an integer region keeps 32-bit two's
+// complement integers in them bit for bit and uses the *I operations.
 enum RegionOpCode : int {
   kRegionPush = 0, kRegionConst, kRegionAdd, kRegionSub, kRegionMul, kRegionDiv, kRegionMax,
-  kRegionMin, kRegionRelu, kRegionLeaky, kRegionNeg, kRegionDup
+  kRegionMin, kRegionRelu, kRegionLeaky, kRegionNeg, kRegionDup,
+  kRegionAddI = 16, kRegionSubI, kRegionMulI, kRegionMaxI, kRegionMinI, kRegionReluI, kRegionNegI,
+  // comparisons of an i16 region look at the low 16 bits of their operands (add, sub, mul
+  // and neg agree modulo 2^16 whatever the upper bits hold, and the store truncates)
+  kRegionMaxI16, kRegionMinI16, kRegionReluI16
 };
+__host__ __device__ inline bool region_is_binary(int code) {
+  return (code >= kRegionAdd && code <= kRegionMin) || (code >= kRegionAddI && code <= kRegionMinI) ||
+         code == kRegionMaxI16 || code == kRegionMinI16;
+}
+__host__ __device__ inline bool region_is_unary(int code) {
+  return code == kRegionRelu || code == kRegionLeaky || code == kRegionNeg || code == kRegionReluI ||
+         code == kRegionNegI || code == kRegionReluI16;
+}
+__host__ __device__ inline bool region_is_16bit(int type) {
+  return type == kRegionF16 || type == kRegionBF16 || type == kRegionI16;
+}
 
 struct RegionInput {
   const void *base;    // device pointer of the tensor
@@ -48,7 +65,7 @@ struct RegionOp {
 // chain: acc = u0(x0); acc = u_k(acc (op_k) x_k) for each step.  Reversed
 // operands (x - acc, x / acc) have their own codes.
 constexpr int kRegionMaxSteps = 8;
-enum RegionChainCode : int { kChainRSub = 32, kChainRDiv = 33 };
+enum RegionChainCode : int { kChainRSub = 32, kChainRDiv = 33, kChainRSubI = 34 };
 struct RegionUnary {
   int code[2];      // kRegionRelu / kRegionLeaky / kRegionNeg
   float alpha[2];

@@ -141,6 +141,56 @@ template <int V> DEV void stv_bf16(void *o, long long i, const float (&v)[V]) {
   }
 }
 
+// ---- integer regions: 32-bit two's complement values, i16 sign-extended on
+// load and truncated on store
+DEV int ldd_i32(const void *b, long long i) { return ((const int *)b)[i]; }
+DEV int ldd_i16(const void *b, long long i) { return (int)((const short *)b)[i]; }
+DEV void st_i32(void *o, long long i, int x) { ((int *)o)[i] = x; }
+DEV void st_i16(void *o, long long i, int x) { ((short *)o)[i] = (short)x; }
+template <int V, bool NT> DEV void ldv_i32(const void *b, long long i, int (&v)[V]) {
+  const u32x4 *p = (const u32x4 *)((const int *)b + i);
+#pragma unroll
+  for (int q = 0; q < V / 4; ++q) {
+    const u32x4 raw = ld128<NT>(p + q);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[4 * q + e] = (int)raw[e];
+  }
+}
+template <int V, bool NT> DEV void ldv_i16(const void *b, long long i, int (&v)[V]) {
+  const u32x4 *p = (const u32x4 *)((const short *)b + i);
+#pragma unroll
+  for (int q = 0; q < V / 8; ++q) {
+    const u32x4 raw = ld128<NT>(p + q);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const unsigned word = raw[d];
+      v[8 * q + 2 * d] = (int)(word << 16) >> 16;
+      v[8 * q + 2 * d + 1] = (int)word >> 16;
+    }
+  }
+}
+template <int V> DEV void stv_i32(void *o, long long i, const int (&v)[V]) {
+  u32x4 *p = (u32x4 *)((int *)o + i);
+#pragma unroll
+  for (int q = 0; q < V / 4; ++q) {
+    u32x4 a;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) a[e] = (unsigned)v[4 * q + e];
+    __builtin_nontemporal_store(a, p + q);
+  }
+}
+template <int V> DEV void stv_i16(void *o, long long i, const int (&v)[V]) {
+  u32x4 *p = (u32x4 *)((short *)o + i);
+#pragma unroll
+  for (int q = 0; q < V / 8; ++q) {
+    u32x4 w;
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+      w[d] = ((unsigned)v[8 * q + 2 * d] & 0xffffu) | ((unsigned)v[8 * q + 2 * d + 1] << 16);
+    __builtin_nontemporal_store(w, p + q);
+  }
+}
+
 // ---- sum over the 64 lanes of a wavefront, fixed order: quad butterflies,
 // half-row and row mirrors, then the four row totals
 template <int C> DEV float dpp_add(float v) {
@@ -168,6 +218,7 @@ const char *typeTag(ElemType t) {
     case ElemType::F32: return "f32";
     case ElemType::I32: return "i32";
     case ElemType::I64: return "i64";
+    case ElemType::I16: return "i16";
   }
   return "f32";
 }
@@ -178,6 +229,12 @@ std::string floatLiteral(float f) {
   char buf[64];
   std::snprintf(buf, sizeof buf, "as_f32(0x%08xu) /* %g */", u, (double)f);
   return buf;
+}
+
+// A constant of an integer region (validated to be a 32-bit integer).
+std::string intLiteral(float f) {
+  const long long v = (long long)f;
+  return v == -2147483648ll ? std::string("(-2147483647 - 1)") : "(" + std::to_string(v) + ")";
 }
 
 // One distinct operand read of a segment.
@@ -317,6 +374,8 @@ class SegmentEmitter {
     return mask;
   }
   void analyze() {
+    integer_ = isRegionInt(p_.output().type);
+    narrow_ = p_.output().type == ElemType::I16;
     rank_ = seg_.rank;
     last_ = rank_ - 1;
     reduce_ = seg_.reduces();
@@ -350,8 +409,8 @@ class SegmentEmitter {
         line(d, "const long long q" + u + " = (long long)(" + pos + ");");
       }
       if (o.step == Operand::Broadcast && o.gatherDim != last_)
-        line(d, "const float s" + u + " = " + (outerGather ? "bad" + u + " ? as_f32(0x7fc00000u) : " : "") + "ld_" +
-                    typeTag(o.type) + "(" + r + ".base, q" + u + ");");
+        line(d, "const " + ct() + " s" + u + " = " + (outerGather ? "bad" + u + " ? " + bad() + " : " : "") + ld(o.type) +
+                    "(" + r + ".base, q" + u + ");");
     }
   }
 
@@ -365,17 +424,17 @@ class SegmentEmitter {
       return v;
     }
     v.name = "v" + u;
-    line(d, "float v" + u + "[U][W];");
+    line(d, ct() + " v" + u + "[U][W];");
     if (o.tiled) {
       unroll();
       line(d, "for (int u = 0; u < U; ++u)");
       unroll();
       line(d + 1, "for (int e = 0; e < W; ++e)");
       line(d + 2, "v" + u + "[u][e] = e < nvalid[u] ? tile[" + std::to_string(o.tileSlot) +
-                      "][((int)(j0[u] - tile_q) + e) * PITCH + pl] : 0.f;");
+                      "][((int)(j0[u] - tile_q) + e) * PITCH + pl] : " + zero() + ";");
       return v;
     }
-    const std::string nan = "as_f32(0x7fc00000u)";
+    const std::string nan = bad();
     if (o.gatherDim == last_) {
       // one index per element
       line(d, "{");
@@ -385,14 +444,14 @@ class SegmentEmitter {
       line(d + 1, "for (int u = 0; u < U; ++u) {");
       unroll();
       line(d + 2, "for (int e = 0; e < W; ++e) {");
-      line(d + 3, "float x = 0.f;");
+      line(d + 3, ct() + " x = " + zero() + ";");
       line(d + 3, "if (e < nvalid[u]) {");
       line(d + 4, "const long long g = ld_" + std::string(typeTag(o.gatherType)) + "(" + r + ".index, (long long)j0[u] + e);");
       line(d + 4, "if (g < 0 || g >= " + r + ".gextent) {");
       line(d + 5, "if (R.error_flag) *R.error_flag = 1;");
       line(d + 5, "x = " + nan + ";");
       line(d + 4, "} else {");
-      line(d + 5, "x = ld_" + tag + "(" + r + ".base, q" + u + " + ((long long)j0[u] + e) * step + g * " + r + ".gstride);");
+      line(d + 5, "x = " + ld(o.type) + "(" + r + ".base, q" + u + " + ((long long)j0[u] + e) * step + g * " + r + ".gstride);");
       line(d + 4, "}");
       line(d + 3, "}");
       line(d + 3, "v" + u + "[u][e] = x;");
@@ -410,8 +469,8 @@ class SegmentEmitter {
       line(d + 2, "ldv_" + tag + "<W, " + nt + ">(" + r + ".base, q" + u + " + j0[u], v" + u + "[u]);");
       line(d + 1, "} else {");
       unroll();
-      line(d + 2, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = e < nvalid[u] ? ld_" + tag + "(" + r + ".base, q" + u +
-                      " + j0[u] + e) : 0.f;");
+      line(d + 2, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = e < nvalid[u] ? " + ld(o.type) + "(" + r + ".base, q" + u +
+                      " + j0[u] + e) : " + zero() + ";");
       line(d + 1, "}");
       line(d, "}");
     } else {
@@ -425,8 +484,8 @@ class SegmentEmitter {
       line(d + 3, "ldv_" + tag + "<W, " + nt + ">(" + r + ".base, q" + u + " + j0[u], v" + u + "[u]);");
       line(d + 2, "} else {");
       unroll();
-      line(d + 3, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = e < nvalid[u] ? ld_" + tag + "(" + r + ".base, q" + u +
-                      " + ((long long)j0[u] + e) * step) : 0.f;");
+      line(d + 3, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = e < nvalid[u] ? " + ld(o.type) + "(" + r + ".base, q" + u +
+                      " + ((long long)j0[u] + e) * step) : " + zero() + ";");
       line(d + 2, "}");
       line(d + 1, "}");
       line(d, "}");
@@ -456,9 +515,9 @@ class SegmentEmitter {
     };
     auto define = [&](const Value &v, const std::string &expr) {
       if (v.scalar) {
-        line(d, "const float " + v.name + " = " + expr + ";");
+        line(d, "const " + ct() + " " + v.name + " = " + expr + ";");
       } else {
-        line(d, "float " + v.name + "[U][W];");
+        line(d, ct() + " " + v.name + "[U][W];");
         unroll();
         line(d, "for (int u = 0; u < U; ++u)");
         unroll();
@@ -482,7 +541,7 @@ class SegmentEmitter {
           break;
         case OpCode::Const: {
           Value v = fresh(true);
-          define(v, floatLiteral(op.constant));
+          define(v, integer_ ? intLiteral(op.constant) : floatLiteral(op.constant));
           stack.push_back(v);
           break;
         }
@@ -497,6 +556,19 @@ class SegmentEmitter {
           stack.pop_back();
           Value v = fresh(a.scalar && b.scalar);
           std::string expr;
+          if (integer_) {
+            // wrapping 32-bit arithmetic: through unsigned, where overflow is defined
+            // an i16 region compares the low 16 bits; add, sub, mul agree modulo 2^16 anyway
+            const std::string ua = "(unsigned)" + a.at(), ub = "(unsigned)" + b.at();
+            const std::string ca = narrow_ ? "(int)(short)" + a.at() : a.at(), cb = narrow_ ? "(int)(short)" + b.at() : b.at();
+            switch (op.code) {
+              case OpCode::Add: expr = "(int)(" + ua + " + " + ub + ")"; break;
+              case OpCode::Sub: expr = "(int)(" + ua + " - " + ub + ")"; break;
+              case OpCode::Mul: expr = "(int)(" + ua + " * " + ub + ")"; break;
+              case OpCode::Max: expr = ca + " > " + cb + " ? " + ca + " : " + cb; break;
+              default: expr = ca + " < " + cb + " ? " + ca + " : " + cb; break;
+            }
+          } else
           switch (op.code) {
             case OpCode::Add: expr = a.at() + " + " + b.at(); break;
             case OpCode::Sub: expr = a.at() + " - " + b.at(); break;
@@ -513,7 +585,11 @@ class SegmentEmitter {
           const Value a = stack.back();
           stack.pop_back();
           Value v = fresh(a.scalar);
-          if (op.code == OpCode::Relu) define(v, "fmax_ieee(" + a.at() + ", 0.f)");
+          if (integer_) {
+            const std::string ca = narrow_ ? "(int)(short)" + a.at() : a.at();
+            define(v, op.code == OpCode::Relu ? ca + " > 0 ? " + ca + " : 0" : "(int)(0u - (unsigned)" + a.at() + ")");
+          }
+          else if (op.code == OpCode::Relu) define(v, "fmax_ieee(" + a.at() + ", 0.f)");
           else if (op.code == OpCode::Leaky)
             define(v, "fmax_ieee(" + a.at() + ", " + a.at() + " * " + floatLiteral(op.constant) + ")");
           else define(v, "-" + a.at());
@@ -620,7 +696,7 @@ class SegmentEmitter {
     const Value v = emitExpression(3);
     std::string res = v.name;
     if (v.scalar) {
-      line(3, "float splat[U][W];");
+      line(3, ct() + " splat[U][W];");
       unroll();
       line(3, "for (int u = 0; u < U; ++u)");
       unroll();
@@ -663,7 +739,7 @@ class SegmentEmitter {
     line(1, "constexpr int W = " + std::to_string(W_) + ", U = " + std::to_string(U_) + ";");
     line(1, "constexpr int TP = " + std::to_string(kTileP) + ", TQ = " + std::to_string(kTileQ) + ", PITCH = TP + 1;");
     line(1, "static_assert(8 * U * W == TQ, \"eight lanes cover a tile row\");");
-    line(1, "__attribute__((shared)) static float tile[" + std::to_string(numTiles_) + "][TQ * PITCH];");
+    line(1, "__attribute__((shared)) static " + ct() + " tile[" + std::to_string(numTiles_) + "][TQ * PITCH];");
     line(1, "const int tid = (int)__builtin_amdgcn_workitem_id_x();");
     line(1, "const I n = (I)R.size[" + L + "];");
     line(1, "const I np = (I)R.size[" + P + "];");
@@ -680,7 +756,7 @@ class SegmentEmitter {
     for (const Operand &o : operands_) {
       if (!o.tiled) continue;
       const std::string u = id(o), rr = in(o), tag = typeTag(o.type);
-      const int el = o.type == ElemType::F32 ? 4 : 8;
+      const int el = (o.type == ElemType::F32 || o.type == ElemType::I32) ? 4 : 8;
       line(2, "{  // operand " + u + ": " + std::to_string(kTileQ) + " runs of " + std::to_string(kTileP) + " elements along dim " + P);
       line(3, "constexpr int EL = " + std::to_string(el) + ", LPR = TP / EL, RPP = 256 / LPR, NP = TQ / RPP;");
       line(3, "const int lp = (tid % LPR) * EL, lq = tid / LPR;");
@@ -688,7 +764,7 @@ class SegmentEmitter {
                   (r >= 0 && o.usesDim[r] ? " + (long long)x" + std::to_string(r) + " * " + rr + ".stride[" + std::to_string(r) + "]" : "") +
                   " + (long long)(tile_p + lp);");
       line(3, "const long long sq = " + rr + ".stride[" + L + "];");
-      line(3, "float vals[NP][EL];");
+      line(3, ct() + " vals[NP][EL];");
       unroll();
       line(3, "for (int s = 0; s < NP; ++s) {");
       line(4, "const I q = tile_q + (I)(lq + s * RPP);");
@@ -697,7 +773,7 @@ class SegmentEmitter {
       line(4, "} else {");
       unroll();
       line(5, "for (int e = 0; e < EL; ++e)");
-      line(6, "vals[s][e] = (q < n && tile_p + (I)(lp + e) < np) ? ld_" + tag + "(" + rr + ".base, pos + (long long)q * sq + e) : 0.f;");
+      line(6, "vals[s][e] = (q < n && tile_p + (I)(lp + e) < np) ? " + ld(o.type) + "(" + rr + ".base, pos + (long long)q * sq + e) : " + zero() + ";");
       line(4, "}");
       line(3, "}");
       unroll();
@@ -721,7 +797,7 @@ class SegmentEmitter {
     const Value v = emitExpression(4);
     std::string res = v.name;
     if (v.scalar) {
-      line(4, "float splat[U][W];");
+      line(4, ct() + " splat[U][W];");
       unroll();
       line(4, "for (int u = 0; u < U; ++u)");
       unroll();
@@ -763,6 +839,14 @@ class SegmentEmitter {
   int rank_ = 0, last_ = 0, W_ = 8, U_ = 2;
   int tileDim_ = -1, numTiles_ = 0;
   bool reduce_ = false;
+  bool integer_ = false;   // 32-bit integers instead of float32 values
+  bool narrow_ = false;    // ... of which the low 16 bits are the value (i16 output)
+
+  // C type of a value, its zero, what an out-of-range gather yields, the scalar load of a tensor
+  std::string ct() const { return integer_ ? "int" : "float"; }
+  std::string zero() const { return integer_ ? "0" : "0.f"; }
+  std::string bad() const { return integer_ ? "0" : "as_f32(0x7fc00000u)"; }
+  std::string ld(ElemType t) const { return std::string(integer_ ? "ldd_" : "ld_") + typeTag(t); }
   std::vector<Operand> operands_;
   std::vector<int> pushSlot_;   // per push, in order: index into operands_
 };
@@ -788,9 +872,11 @@ bool setEmitOption(EmitOptions *o, const std::string &name, long long value) {
 
 SpecShape specShape(const Program &p, int segment, const EmitOptions &options) {
   const Segment &g = p.segments[segment];
-  bool any16 = p.output().type != ElemType::F32, any32 = p.output().type == ElemType::F32;
+  bool any16 = false, any32 = false;
+  auto note = [&](ElemType t) { (elemTypeBytes(t) == 4 ? any32 : any16) = true; };
+  note(p.output().type);
   for (const Op &op : g.ops)
-    if (op.code == OpCode::Push) (p.args[op.arg].type == ElemType::F32 ? any32 : any16) = true;
+    if (op.code == OpCode::Push) note(p.args[op.arg].type);
   SpecShape s;
   s.width = any16 ? 8 : 4;            // 16 bytes of the narrowest tensor
   s.unroll = options.unroll ? options.unroll : ((any16 && any32) ? 2 : 4);

@@ -379,6 +379,7 @@ bool elemFromName(const std::string &n, ElemType *t) {
   if (n == "f32") { *t = ElemType::F32; return true; }
   if (n == "i32") { *t = ElemType::I32; return true; }
   if (n == "i64") { *t = ElemType::I64; return true; }
+  if (n == "i16") { *t = ElemType::I16; return true; }
   return false;
 }
 
@@ -561,7 +562,9 @@ class Translator {
         tv->elem = t.elem;
         tv->directArg = argIndex;
         for (size_t d = 0; d < t.shape.size(); ++d) tv->shape.push_back(Ref::dimOf(argIndex, (int)d));
-        if (afir_region::isFloat(t.elem)) {
+        // i16 / i32 tensors are values to the afir integer ops (and i32 an index
+        // tensor to linalg.generic); i64 is an index type only
+        if (afir_region::isFloat(t.elem) || afir_region::isRegionInt(t.elem)) {
           auto e = std::make_shared<Expr>();
           e->kind = Expr::Input;
           e->arg = argIndex;
@@ -1156,6 +1159,15 @@ class Translator {
     }
     auto tv = std::make_shared<Tensor>();
     tv->elem = rt.elemKnown ? rt.elem : in[0]->elem;
+    // integer tensors (include/Dialect/AFIR/Ops/Basic/math.td:71-98): add, sub, mul, maximum,
+    // minimum, neg, relu, abs and the data movement ops; operands and result of one kind
+    const bool integer = afir_region::isRegionInt(tv->elem);
+    for (const TensorP &t : in)
+      if (afir_region::isRegionInt(t->elem) != integer)
+        r_.fail("afir." + name + ": integer and floating-point tensors in one operation");
+    if (!integer && !afir_region::isFloat(tv->elem)) r_.fail("afir." + name + ": unsupported result element type");
+    if (integer && (name == "div" || name == "truediv" || name == "leaky_relu" || name == "sum"))
+      r_.fail("afir." + name + " on integer tensors has no HIP lowering");
 
     static const struct { const char *n; OpCode c; } binary[] = {
         {"add", OpCode::Add}, {"sub", OpCode::Sub}, {"mul", OpCode::Mul}, {"div", OpCode::Div},
@@ -1335,7 +1347,8 @@ class Translator {
     o.isOutput = true;
     o.type = result->elem;
     o.rank = (int)result->shape.size();
-    if (!afir_region::isFloat(o.type)) r_.fail("the function must return a floating-point tensor");
+    if (!afir_region::isFloat(o.type) && !afir_region::isRegionInt(o.type))
+      r_.fail("the function must return an f16, bf16, f32, i16 or i32 tensor");
     p.args.push_back(o);
     if (!result->parts.empty()) {
       // first row of each part: the sum of the parts before it (constants folded)

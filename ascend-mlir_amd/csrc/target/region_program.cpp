@@ -18,6 +18,7 @@ const char *elemTypeName(ElemType t) {
     case ElemType::F32: return "f32";
     case ElemType::I32: return "i32";
     case ElemType::I64: return "i64";
+    case ElemType::I16: return "i16";
   }
   return "f32";
 }
@@ -29,6 +30,7 @@ size_t elemTypeBytes(ElemType t) {
     case ElemType::F32:
     case ElemType::I32: return 4;
     case ElemType::I64: return 8;
+    case ElemType::I16: return 2;
   }
   return 4;
 }
@@ -36,7 +38,7 @@ size_t elemTypeBytes(ElemType t) {
 bool parseElemType(const std::string &s, ElemType *out) {
   static const struct { const char *n; ElemType t; } table[] = {
       {"f16", ElemType::F16}, {"bf16", ElemType::BF16}, {"f32", ElemType::F32},
-      {"i32", ElemType::I32}, {"i64", ElemType::I64}};
+      {"i32", ElemType::I32}, {"i64", ElemType::I64}, {"i16", ElemType::I16}};
   for (const auto &e : table)
     if (s == e.n) { *out = e.t; return true; }
   return false;
@@ -298,7 +300,8 @@ std::string validate(const Program &p) {
     if (a.isOutput != (i + 1 == p.args.size()))
       return "region program: exactly one output, declared last, is supported";
   }
-  if (!isFloat(p.output().type)) return "region program: the output must be f16, bf16 or f32";
+  const bool integer = isRegionInt(p.output().type);
+  if (!isFloat(p.output().type) && !integer) return "region program: the output must be f16, bf16, f32, i16 or i32";
   if (p.segments.empty()) return "region program: no segment";
   auto refOk = [&](const Ref &r) {
     return r.arg < 0 ? r.constant >= 0
@@ -323,7 +326,9 @@ std::string validate(const Program &p) {
         case OpCode::Push: {
           if (o.arg < 0 || o.arg >= p.numInputs()) return "region program: push of a non-input argument";
           const Arg &a = p.args[o.arg];
-          if (!isFloat(a.type)) return "region program: pushed tensors must be f16, bf16 or f32";
+          if (integer ? !isRegionInt(a.type) : !isFloat(a.type))
+            return integer ? "region program: an integer region reads i16 / i32 tensors only"
+                           : "region program: pushed tensors must be f16, bf16 or f32";
           if ((int)o.map.size() != a.rank) return "region program: map needs one entry per dim of the input";
           if (!o.slice.empty() && (int)o.slice.size() != a.rank)
             return "region program: slice needs one offset per dim of the input";
@@ -350,6 +355,7 @@ std::string validate(const Program &p) {
           break;
         }
         case OpCode::Matmul: {
+          if (integer) return "region program: 'matmul' is not available in an integer region";
           if (i != 0 || g.rank != 2) return "region program: 'matmul' must open a rank-2 segment";
           for (int a : {o.arg, o.arg2}) {
             if (a < 0 || a >= p.numInputs()) return "region program: matmul of a non-input argument";
@@ -358,20 +364,27 @@ std::string validate(const Program &p) {
           ++depth;
           break;
         }
-        case OpCode::Const: ++depth; break;
+        case OpCode::Const:
+          if (integer && (o.constant != (float)(int32_t)o.constant || o.constant >= 2147483648.f || o.constant < -2147483648.f))
+            return "region program: a constant of an integer region must be a 32-bit integer";
+          ++depth;
+          break;
         case OpCode::Dup:
           if (o.depth < 0 || o.depth >= depth) return "region program: dup beyond the stack";
           ++depth;
           break;
         case OpCode::Add: case OpCode::Sub: case OpCode::Mul: case OpCode::Div:
         case OpCode::Max: case OpCode::Min:
+          if (integer && o.code == OpCode::Div) return "region program: 'div' is not available in an integer region";
           if (depth < 2) return "region program: binary operation on fewer than two values";
           --depth;
           break;
         case OpCode::Relu: case OpCode::Leaky: case OpCode::Neg:
+          if (integer && o.code == OpCode::Leaky) return "region program: 'leaky' is not available in an integer region";
           if (depth < 1) return "region program: unary operation on an empty stack";
           break;
         case OpCode::ReduceSum:
+          if (integer) return "region program: 'reduce sum' is not available in an integer region";
           if (depth != 1) return "region program: 'reduce sum' needs exactly one value";
           if (g.rank < 2) return "region program: a reduction needs an iteration rank of at least 2";
           reduced = true;

@@ -17,12 +17,17 @@
 // lib/Runtime/Execution/NativeExecutionRunner.cpp:332-369,476-488).
 //
 // Arithmetic is float32 with one round-to-nearest-even to the output type,
-// like the reference's numpy goldens (examples/*/gen_data.py).
+// like the reference's numpy goldens (examples/*/gen_data.py).  A region whose
+// output is i16 or i32 is an integer region (afir.add / sub / mul / maximum /
+// minimum / neg / relu on I16, I32: include/Dialect/AFIR/Ops/Basic/math.td:71-98):
+// every read is i16 or i32, arithmetic is 32-bit two's complement (wrapping),
+// the result is truncated to the output type; div, leaky relu, reductions and
+// matmul are float-only.
 //
 // Text form (one item per line, '#' starts a comment):
 //   afir-hip-region 1
-//   arg in  <f16|bf16|f32|i32|i64> <rank>      one line per function argument,
-//   arg out <f16|bf16|f32> <rank>              inputs first, then the output
+//   arg in  <f16|bf16|f32|i16|i32|i64> <rank>      one line per function argument,
+//   arg out <f16|bf16|f32|i16|i32> <rank>              inputs first, then the output
 //   segment <iteration rank>
 //     size <ref> <ref> ...      extent of each iteration dim: argA.D or a constant
 //     outoff <ref> [<ref> ...]  first output row (dim 0) this segment writes: the sum of the terms
@@ -48,11 +53,13 @@
 
 namespace afir_region {
 
-enum class ElemType { F16, BF16, F32, I32, I64 };
+enum class ElemType { F16, BF16, F32, I32, I64, I16 };
 const char *elemTypeName(ElemType t);
 size_t elemTypeBytes(ElemType t);
 bool parseElemType(const std::string &s, ElemType *out);
 inline bool isFloat(ElemType t) { return t == ElemType::F16 || t == ElemType::BF16 || t == ElemType::F32; }
+// Element types of integer regions (i64 serves as an index type only).
+inline bool isRegionInt(ElemType t) { return t == ElemType::I16 || t == ElemType::I32; }
 
 constexpr int kMaxRank = 3;       // iteration rank and tensor rank
 constexpr int kMaxArgs = 10;      // inputs + output

@@ -289,7 +289,7 @@ def _torch_type(name):
     import torch
     if _TORCH_TYPES is None:
         _TORCH_TYPES = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32,
-                        "i32": torch.int32, "i64": torch.int64}
+                        "i32": torch.int32, "i64": torch.int64, "i16": torch.int16}
     return _TORCH_TYPES[name]
 
 

@@ -33,6 +33,16 @@ through struct, and the graphs of the reference's examples, translated from
 MLIR, must turn the reference's own input vectors into its own expected
 outputs (tests/golden/reference_examples.npz, tests/test_golden_fixtures.py).  max / min follow IEEE-754 maximum / minimum (-0 < +0, NaN
 propagates), which is what arith.maximumf specifies.
+
+Integer regions (_evaluate_integer: afir.add / sub / mul / maximum / minimum /
+neg / relu on I16 and I32 tensors, include/Dialect/AFIR/Ops/Basic/math.td:71-98)
+are pinned against numpy's own int16 / int32 array arithmetic and against
+corner values written out by hand.  Where no intermediate overflows, the result
+is fixed by the mathematics.  Where one does, values wrap at the element width,
+as numpy (the language of the reference's golden generators) does; the
+reference holds no integer golden and lowers these ops to the device's vector
+instructions without stating their overflow behaviour, so for overflowing
+inputs this function is PARITY UNPINNED.
 """
 from __future__ import annotations
 
@@ -40,7 +50,7 @@ import numpy as np
 
 from . import afir_oracle as O
 
-_NP = {"f16": np.float16, "f32": np.float32, "i32": np.int32, "i64": np.int64}
+_NP = {"f16": np.float16, "f32": np.float32, "i32": np.int32, "i64": np.int64, "i16": np.int16}
 
 
 class RegionError(Exception):
@@ -122,6 +132,73 @@ def ieee_min(a, b):
     return np.where(np.isnan(a), a, np.where(np.isnan(b), b, r)).astype(np.float32)
 
 
+def _wrap(v, bits):
+    """int64 -> the value `bits`-wide two's complement arithmetic would hold."""
+    return ((v + (1 << (bits - 1))) % (1 << bits)) - (1 << (bits - 1))
+
+
+def _evaluate_integer(prog, inputs, val, out_type, out_rank):
+    """Integer regions (afir.add / sub / mul / maximum / minimum / neg / relu on
+    I16, I32; include/Dialect/AFIR/Ops/Basic/math.td:71-98): every read is
+    converted to the output type and every operation wraps at its width, as a
+    graph of afir ops on tensors of that type would."""
+    args = prog["args"]
+    bits = 16 if out_type == "i16" else 32
+    pieces = []
+    for seg in prog["segments"]:
+        size = [val(r) for r in seg["size"]]
+        rank = seg["rank"]
+        grids = np.ogrid[tuple(slice(0, s) for s in size)]
+        stack = []
+        for op in seg["ops"]:
+            k = op[0]
+            if k == "push":
+                _, a, m, sl = op
+                if args[a][1] not in ("i16", "i32"):
+                    raise RegionError("an integer region reads i16 / i32 tensors only")
+                src = np.asarray(inputs[a])
+                idx = []
+                for d, e in enumerate(m):
+                    start = val(sl[d]) if sl else 0
+                    if e[0] == "iter":
+                        idx.append(grids[e[1]] + start)
+                    elif e[0] == "const":
+                        idx.append(np.int64(e[1] + start))
+                    else:
+                        g = np.asarray(inputs[e[2]]).astype(np.int64)[:size[e[1]]]
+                        if g.size and (g.min() < 0 or g.max() + start >= src.shape[d]):
+                            raise RegionError("gather index out of range")
+                        shape = [1] * rank
+                        shape[e[1]] = size[e[1]]
+                        idx.append(g.reshape(shape) + start)
+                v = src[tuple(idx)] if src.ndim else src
+                stack.append(_wrap(np.broadcast_to(v, size).astype(np.int64), bits))
+            elif k == "const":
+                stack.append(_wrap(np.full(size, int(op[1]), dtype=np.int64), bits))
+            elif k == "dup":
+                stack.append(stack[-1 - op[1]])
+            elif k in ("add", "sub", "mul", "max", "min"):
+                b, a = stack.pop(), stack.pop()
+                stack.append(_wrap({"add": lambda: a + b, "sub": lambda: a - b, "mul": lambda: a * b,
+                                      "max": lambda: np.maximum(a, b), "min": lambda: np.minimum(a, b)}[k](), bits))
+            elif k == "relu":
+                stack.append(np.maximum(stack.pop(), 0))
+            elif k == "neg":
+                stack.append(_wrap(-stack.pop(), bits))
+            elif k == "store":
+                pass
+            else:
+                raise RegionError(f"'{k}' is not available in an integer region")
+        if len(stack) != 1:
+            raise RegionError("stack does not hold exactly one value at store")
+        pieces.append((sum(val(t) for t in seg["outoff"]), stack[0]))
+    pieces.sort(key=lambda p: p[0])
+    res = np.concatenate([p[1] for p in pieces], axis=0)
+    if res.ndim != out_rank:
+        raise RegionError("output rank mismatch")
+    return res.astype(np.int16 if out_type == "i16" else np.int32)
+
+
 def evaluate(text: str, inputs):
     """Runs the program on numpy inputs (bf16 tensors as uint16 bits).  Returns
     the output array in its storage type (bf16 as uint16 bits)."""
@@ -135,6 +212,9 @@ def evaluate(text: str, inputs):
 
     def val(ref):
         return shapes[ref[1]][ref[2]] if ref[0] == "dim" else ref[1]
+
+    if out_type in ("i16", "i32"):
+        return _evaluate_integer(prog, inputs, val, out_type, out_rank)
 
     pieces = []
     for seg in prog["segments"]:

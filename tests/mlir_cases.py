@@ -387,3 +387,17 @@ func.func @div_relu_sum(%arg0: tensor<6x40xf32>, %arg1: tensor<40xf32>) -> tenso
   return %3 : tensor<6xf32>
 }
 """
+
+
+# relu(a - b) * a + (-b) on i32 tensors: the integer side of the AFIR binary / unary math
+# ops (include/Dialect/AFIR/Ops/Basic/math.td:71-98), with dynamic shapes.
+INT_CHAIN_I32 = """
+func.func @int_chain(%a : tensor<?x?xi32>, %b : tensor<?x?xi32>) -> tensor<?x?xi32> {
+  %0 = afir.sub %a, %b : (tensor<?x?xi32>, tensor<?x?xi32>) -> tensor<?x?xi32>
+  %1 = afir.relu %0 : tensor<?x?xi32> -> tensor<?x?xi32>
+  %2 = afir.mul %1, %a : (tensor<?x?xi32>, tensor<?x?xi32>) -> tensor<?x?xi32>
+  %3 = afir.neg %b : tensor<?x?xi32> -> tensor<?x?xi32>
+  %4 = afir.add %2, %3 : (tensor<?x?xi32>, tensor<?x?xi32>) -> tensor<?x?xi32>
+  return %4 : tensor<?x?xi32>
+}
+"""

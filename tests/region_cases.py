@@ -312,3 +312,138 @@ CONST_TWO_IGNORING_INPUT = HEADER + "arg in f16 1\narg out f16 1\nsegment 1\n si
 COPY_1D = HEADER + "arg in f16 1\narg out f16 1\nsegment 1\n size arg1.0\n outoff 0\n push arg0 d0\n store\nend\n"
 ADD_1D = (HEADER + "arg in f16 1\narg in f16 1\narg out f16 1\nsegment 1\n size arg2.0\n outoff 0\n"
           " push arg0 d0\n push arg1 d0\n add\n store\nend\n")
+
+
+# Integer regions: afir.add / sub / mul / maximum / minimum / neg / relu on I16 and
+# I32 tensors (include/Dialect/AFIR/Ops/Basic/math.td:71-98; the reference's
+# convert_add_i32 and test_add_i16 functions, test/Conversion/afir_to_ascir.mlir:34-37,
+# test/Dialect/AFIR/ops.mlir:8-11).  Expected values come from numpy's own fixed
+# width integer arithmetic, which wraps like the kernels' 32-bit registers.
+INT_ADD_I32 = (HEADER + "arg in i32 2\narg in i32 2\narg out i32 2\nsegment 2\n size arg0.0 arg0.1\n outoff 0\n"
+               " push arg0 d0 d1\n push arg1 d0 d1\n add\n store\nend\n")
+INT_ADD_I16 = INT_ADD_I32.replace("i32", "i16")
+# relu(x - row) * col + min(x, -x), the transposed read included
+INT_CHAIN_I32 = HEADER + """
+arg in i32 2
+arg in i32 1
+arg in i32 1
+arg in i32 2
+arg out i32 2
+segment 2
+  size arg0.0 arg0.1
+  outoff 0
+  push arg0 d0 d1
+  push arg1 d0
+  sub
+  relu
+  push arg2 d1
+  mul
+  push arg0 d0 d1
+  dup 0
+  neg
+  min
+  add
+  push arg3 d1 d0
+  max
+  const -7
+  add
+  store
+end
+"""
+# the same on i16 tensors: comparisons see values wrapped to 16 bits
+INT_CHAIN_I16 = INT_CHAIN_I32.replace("i32", "i16")
+# i16 and i32 reads in one region, i16 result (every value taken modulo 2^16)
+INT_MIXED_TO_I16 = HEADER + """
+arg in i16 2
+arg in i32 1
+arg out i16 2
+segment 2
+  size arg0.0 arg0.1
+  outoff 0
+  push arg0 d0 d1
+  push arg1 d1
+  mul
+  push arg0 d0 d1
+  add
+  store
+end
+"""
+# rows of an i32 table picked by an index tensor, plus a per-column i16 term
+INT_GATHER_ROWS = HEADER + """
+arg in i32 2
+arg in i64 1
+arg in i16 1
+arg out i32 2
+segment 2
+  size arg1.0 arg0.1
+  outoff 0
+  push arg0 g0:arg1 d1
+  push arg2 d1
+  add
+  store
+end
+"""
+
+
+def _ints(rng, shape, dt):
+    """Full-range values with the overflow-prone ones seeded in."""
+    info = np.iinfo(dt)
+    x = rng.integers(info.min, info.max, shape, dtype=dt, endpoint=True)
+    flat = x.reshape(-1)
+    special = np.array([info.min, info.max, 0, -1, 1, info.min + 1], dtype=dt)
+    if flat.size:
+        where = rng.integers(0, flat.size, min(flat.size, 12))
+        flat[where] = special[np.arange(where.size) % special.size]
+    return x
+
+
+def case_int_add_i32(shape=(37, 203), seed=11):
+    rng = np.random.default_rng(seed)
+    a, b = _ints(rng, shape, np.int32), _ints(rng, shape, np.int32)
+    with np.errstate(over="ignore"):
+        return INT_ADD_I32, [a, b], a + b
+
+
+def case_int_add_i16(shape=(37, 203), seed=12):
+    rng = np.random.default_rng(seed)
+    a, b = _ints(rng, shape, np.int16), _ints(rng, shape, np.int16)
+    with np.errstate(over="ignore"):
+        return INT_ADD_I16, [a, b], a + b
+
+
+def case_int_chain_i32(m=70, n=130, seed=13, dt=np.int32, text=INT_CHAIN_I32):
+    rng = np.random.default_rng(seed)
+    x, r, c, t = _ints(rng, (m, n), dt), _ints(rng, (m,), dt), _ints(rng, (n,), dt), _ints(rng, (n, m), dt)
+    with np.errstate(over="ignore"):
+        v = np.maximum(x - r[:, None], dt(0)) * c[None, :]
+        v = v + np.minimum(x, -x)
+        v = np.maximum(v, t.T) + dt(-7)
+    assert v.dtype == dt
+    return text, [x, r, c, t], v
+
+
+def case_int_chain_i16(m=70, n=130, seed=16):
+    return case_int_chain_i32(m, n, seed, np.int16, INT_CHAIN_I16)
+
+
+def case_int_mixed_to_i16(m=33, n=77, seed=14):
+    rng = np.random.default_rng(seed)
+    x, c = _ints(rng, (m, n), np.int16), _ints(rng, (n,), np.int32)
+    with np.errstate(over="ignore"):
+        v = x * c.astype(np.int16)[None, :] + x            # numpy's narrowing cast keeps the low 16 bits
+    return INT_MIXED_TO_I16, [x, c], v
+
+
+def case_int_gather_rows(rows=300, n=96, nidx=45, seed=15):
+    rng = np.random.default_rng(seed)
+    table, col = _ints(rng, (rows, n), np.int32), _ints(rng, (n,), np.int16)
+    idx = rng.integers(0, rows, (nidx,), dtype=np.int64)
+    with np.errstate(over="ignore"):
+        return INT_GATHER_ROWS, [table, idx, col], table[idx] + col.astype(np.int32)[None, :]
+
+
+INT_CASES = {
+    "int_add_i32": case_int_add_i32, "int_add_i16": case_int_add_i16, "int_chain_i32": case_int_chain_i32,
+    "int_chain_i16": case_int_chain_i16,
+    "int_mixed_to_i16": case_int_mixed_to_i16, "int_gather_rows": case_int_gather_rows,
+}

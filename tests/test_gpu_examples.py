@@ -34,6 +34,15 @@ def _matmul_f16_case(m=128, k=256, n=128, seed=42):
     return None, [a, b, bias, init], O.matmul_bias_leakyrelu_f16(a, b, bias, 0.001)
 
 
+def _int_chain_case(m=640, n=500, seed=42):
+    """Full-range int32 values: every step wraps like numpy's int32 arrays."""
+    rng = np.random.default_rng(seed)
+    a = rng.integers(-2**31, 2**31 - 1, (m, n), dtype=np.int32)
+    b = rng.integers(-2**31, 2**31 - 1, (m, n), dtype=np.int32)
+    with np.errstate(over="ignore"):
+        return None, [a, b], np.maximum(a - b, np.int32(0)) * a + (-b)
+
+
 # (mlir, case, kernel kind, atol, rtol of the example's run.sh, bit-exact expected)
 EXAMPLES = {
     "broadcast-add-reduce": (MC.ROW_BIAS_REDUCE, RC.case_reduce_rowbias, "vec", 10.0, 1e-2, False),
@@ -42,6 +51,8 @@ EXAMPLES = {
     "matmul-add-leakyrelu": (MC.MATMUL_BIAS_LEAKY_F16, _matmul_f16_case, "mix", 1.0, 1e-2, True),
     "add-broadcast-concat": (MC.TWO_CHAINS_CONCAT, RC.case_add_broadcast_concat, "vec", 1e-3, 1e-3, True),
     "split-relu-brc-add-mul": (MC.SPLIT_HALVES, RC.case_split_relu_brc_add_mul, "vec", 1e-3, 1e-3, True),
+    # not one of the reference's examples: its integer element types through the same pipeline
+    "integer-chain": (MC.INT_CHAIN_I32, _int_chain_case, "vec", 0.0, 0.0, True),
 }
 
 

@@ -210,6 +210,72 @@ def test_random_chains_bit_exact(H, seed):
     assert same.all(), text
 
 
+@pytest.mark.parametrize("name", sorted(RC.INT_CASES))
+def test_integer_regions_bit_exact(H, name):
+    """i16 / i32 regions on full-range values (wraparound, 16-bit comparisons,
+    mixed widths, gathered rows, a transposed read): equal to numpy's fixed-width
+    arithmetic and to the region oracle."""
+    text, inputs, want = RC.INT_CASES[name]()
+    assert RO.evaluate(text, inputs).tobytes() == want.tobytes()
+    got = run(H, text, inputs, want.shape)
+    assert got.dtype == want.dtype and got.tobytes() == want.tobytes()
+
+
+INT_OPS2 = ["add", "sub", "mul", "max", "min"]
+INT_OPS1 = ["relu", "neg"]
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_integer_chains_bit_exact(H, seed):
+    """Seeded random integer programs over an identity read, a row and a column
+    broadcast and a transposed read, on ragged shapes."""
+    rng = np.random.default_rng(5000 + seed)
+    ty = ["i32", "i16"][seed % 2]
+    dt = np.int32 if ty == "i32" else np.int16
+    lines, depth = ["push arg0 d0 d1"], 1
+    for _ in range(int(rng.integers(2, 9))):
+        k = rng.integers(0, 4)
+        if depth < 3 and k == 0:
+            lines.append(["push arg1 d0", "push arg2 d1", "push arg3 d1 d0", "const -3", "dup 0"][int(rng.integers(0, 5))])
+            depth += 1
+        elif depth >= 2 and k in (1, 2):
+            lines.append(INT_OPS2[int(rng.integers(0, len(INT_OPS2)))])
+            depth -= 1
+        else:
+            lines.append(INT_OPS1[int(rng.integers(0, len(INT_OPS1)))])
+    while depth > 1:
+        lines.append(INT_OPS2[int(rng.integers(0, 3))])
+        depth -= 1
+    text = (RC.HEADER + f"arg in {ty} 2\narg in {ty} 1\narg in {ty} 1\narg in {ty} 2\narg out {ty} 2\n"
+            "segment 2\n size arg0.0 arg0.1\n outoff 0\n " + "\n ".join(lines) + "\n store\nend\n")
+    m, n = int(rng.integers(1, 70)), int(rng.integers(1, 200))
+    # small magnitudes half of the time so that comparisons are not all decided by overflow
+    lim = np.iinfo(dt).max if seed % 4 < 2 else 50
+    inputs = [rng.integers(-lim, lim, shape, dtype=dt, endpoint=True) for shape in ((m, n), (m,), (n,), (n, m))]
+    want = RO.evaluate(text, inputs)
+    got = run(H, text, inputs, (m, n))
+    assert got.dtype == want.dtype and got.tobytes() == want.tobytes(), text
+
+
+def test_integer_unaligned_views_and_tails(H):
+    """Integer tensors at odd element offsets (no 128-bit access possible) and rows
+    with tails, against the oracle."""
+    import torch
+    rng = np.random.default_rng(9)
+    for ty, dt in (("i32", np.int32), ("i16", np.int16)):
+        text = RC.INT_ADD_I32.replace("i32", ty)
+        for m, n in ((1, 1), (3, 19), (5, 64), (2, 4099)):
+            a = rng.integers(np.iinfo(dt).min, np.iinfo(dt).max, (m, n), dtype=dt)
+            b = rng.integers(np.iinfo(dt).min, np.iinfo(dt).max, (m, n), dtype=dt)
+            want = RO.evaluate(text, [a, b])
+            r = region(H, text)
+            da = torch.zeros(m * n + 1, dtype=getattr(torch, "int32" if ty == "i32" else "int16"), device="cuda")
+            da[1:] = torch.from_numpy(a.reshape(-1)).cuda()
+            got = r(da[1:].view(m, n), _dev(b, ty), out_shape=(m, n)).cpu().numpy()
+            r.close()
+            assert got.tobytes() == want.tobytes(), (ty, m, n)
+
+
 def test_every_operation_pair_at_every_vector_position(H):
     """binary step followed by up to two activations, all combinations, on rows
     of 19 elements (two full vectors and a tail): every position of the result

@@ -84,6 +84,21 @@ def test_transposed_reads_go_through_lds_tiles():
     assert "static float tile[2][TQ * PITCH];" in src
 
 
+def test_integer_regions_use_wrapping_integer_arithmetic():
+    src = _emit(RC.INT_CHAIN_I32).stdout
+    assert "a lane takes 2 groups of 4 elements per row" in src              # i32 everywhere, a transposed read
+    assert "static int tile[1][TQ * PITCH];" in src and "ldv_i32<EL, true>" in src
+    assert "(int)((unsigned)" in src and "stv_i32<W>(R.out" in src
+    body = src[src.index("// ---- segment 0"):]
+    assert "fmax_ieee" not in body and "float" not in body
+    narrow = _emit(RC.INT_CHAIN_I16).stdout
+    assert "(int)(short)" in narrow and "(int)(short)" not in src           # comparisons on 16-bit values
+    assert "stv_i16<W>(R.out" in narrow and "ldv_i16<W, " in narrow
+    mixed = _emit(RC.INT_MIXED_TO_I16).stdout
+    assert "a lane takes 2 groups of 8 elements per pass" in mixed          # 16 bytes of the i16 tensors
+    assert "ldv_i16<W, true>(R.in[0].base" in mixed and "ldd_i32(R.in[1].base" in mixed
+
+
 def test_identical_reads_are_loaded_once():
     src = _emit(RC.C1_ADD_MUL).stdout           # (a + b) * b reads b twice
     assert src.count("ldv_f32<W, true>(R.in[1].base") == 1 and "R.in[2]" not in src

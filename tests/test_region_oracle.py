@@ -83,6 +83,34 @@ def test_gather_out_of_range_is_an_error():
         RO.evaluate(text, inputs)
 
 
+@pytest.mark.parametrize("name", sorted(RC.INT_CASES))
+def test_integer_programs_reproduce_fixed_width_numpy(name):
+    """Integer regions against numpy's own int16 / int32 array arithmetic (which
+    wraps at the element width), on full-range values with the extremes seeded in."""
+    text, inputs, want = RC.INT_CASES[name]()
+    got = RO.evaluate(text, inputs)
+    assert got.dtype == want.dtype and got.tobytes() == want.tobytes()
+
+
+def test_integer_wraparound_by_hand():
+    """The corners a dropped wrap or a wrong width would miss, written out."""
+    head = RC.HEADER + "arg in {t} 1\narg in {t} 1\narg out {t} 1\nsegment 1\n size arg0.0\n outoff 0\n push arg0 d0\n push arg1 d0\n"
+    tail = " store\nend\n"
+    a32 = np.array([2147483647, -2147483648, 65536, -5], dtype=np.int32)
+    b32 = np.array([1, -1, 65536, 3], dtype=np.int32)
+    assert RO.evaluate(head.format(t="i32") + " add\n" + tail, [a32, b32]).tolist() == [-2147483648, 2147483647, 131072, -2]
+    assert RO.evaluate(head.format(t="i32") + " mul\n" + tail, [a32, b32]).tolist() == [2147483647, -2147483648, 0, -15]
+    assert RO.evaluate(head.format(t="i32") + " sub\n neg\n" + tail, [a32, b32]).tolist() == [-2147483646, 2147483647, 0, 8]
+    a16 = np.array([32767, -32768, 256, -5], dtype=np.int16)
+    b16 = np.array([1, -1, 256, 3], dtype=np.int16)
+    assert RO.evaluate(head.format(t="i16") + " add\n" + tail, [a16, b16]).tolist() == [-32768, 32767, 512, -2]
+    # the sum wraps to -32768 before the comparison sees it
+    assert RO.evaluate(head.format(t="i16") + " add\n relu\n" + tail, [a16, b16]).tolist() == [0, 32767, 512, 0]
+    assert RO.evaluate(head.format(t="i16") + " mul\n const 7\n max\n" + tail, [a16, b16]).tolist() == [32767, 7, 7, 7]
+    assert RO.evaluate(head.format(t="i16") + " neg\n" + tail.replace(" store", " add\n store"), [a16, b16]).tolist() == \
+        [32766, -32767, 0, -8]
+
+
 # ---- the C ABI's host side: parse / validate / resolve, no GPU needed --------
 
 @pytest.fixture(scope="module")
@@ -141,6 +169,13 @@ def test_library_resolves_shapes_and_rejects_inconsistent_ones(H):
      "more than 4 live"),
     (RC.HEADER + "arg in f32 2\narg out f32 2\nsegment 2\n size arg0.0 arg0.1\n push arg0 d0 d1\n reduce sum\n store\nend\n",
      "output rank"),
+    (RC.INT_ADD_I32.replace(" add\n", " div\n"), "'div' is not available in an integer region"),
+    (RC.INT_ADD_I32.replace(" add\n", " add\n leaky 0.1\n"), "'leaky' is not available in an integer region"),
+    (RC.INT_ADD_I32.replace(" add\n", " add\n reduce sum\n").replace("arg out i32 2", "arg out i32 1"),
+     "'reduce sum' is not available in an integer region"),
+    (RC.INT_ADD_I32.replace("arg in i32 2\narg in i32 2", "arg in i32 2\narg in f32 2"), "reads i16 / i32 tensors only"),
+    (RC.INT_ADD_I32.replace(" add\n", " add\n const 0.5\n mul\n"), "must be a 32-bit integer"),
+    (RC.C1_ADD_MUL.replace("arg in f32 2", "arg in i32 2", 1), "pushed tensors must be"),
 ])
 def test_library_rejects_malformed_programs(H, bad, why):
     with pytest.raises(H.AfirHipError, match=why):

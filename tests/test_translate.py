@@ -221,6 +221,50 @@ def test_reference_afir_lit_functions_translate():
     assert p.returncode == 1 and "no function @nope" in p.stderr
 
 
+AFIR_CONVERSION = "/root/reference/test/Conversion/afir_to_ascir.mlir"
+
+
+@pytest.mark.skipif(not os.path.isfile(AFIR_CONVERSION), reason="reference tree not present")
+def test_reference_afir_conversion_functions_translate():
+    """Every function of the reference's AFIR -> AscendC conversion test translates; its
+    i32 addition and the round-trip test's i16 addition become integer regions."""
+    import re
+    names = re.findall(r"^func\.func @(\w+)", open(AFIR_CONVERSION).read(), re.M)
+    assert "convert_add_i32" in names and len(names) >= 12
+    for fn in names:
+        p = subprocess.run([TR, "-mlir-to-hip", AFIR_CONVERSION, "--function", fn], capture_output=True, text=True)
+        assert p.returncode == 0, (fn, p.stderr)
+        assert p.stdout.startswith(f"# kernel {fn}\nafir-hip-region 1\n")
+    def body(text):
+        return [l.strip() for l in text.splitlines() if l.strip() and not l.startswith("#")]
+    p = subprocess.run([TR, "-mlir-to-hip", AFIR_CONVERSION, "--function", "convert_add_i32"], capture_output=True, text=True)
+    assert body(p.stdout) == body(RC.INT_ADD_I32)
+    p = subprocess.run([TR, "-mlir-to-hip", AFIR_LIT, "--function", "test_add_i16"], capture_output=True, text=True)
+    assert p.returncode == 0 and body(p.stdout) == body(RC.INT_ADD_I16)
+
+
+def test_integer_afir_graph_matches_numpy():
+    """relu(a - b) * a + (-b) on i32 tensors, against numpy's int32 arithmetic; ops that
+    exist for floating point only are refused on integer tensors."""
+    t = "tensor<?x?xi32>"
+    rc, program, err = translate(MC.INT_CHAIN_I32)
+    assert rc == 0, err
+    rng = np.random.default_rng(3)
+    a = rng.integers(-2**31, 2**31 - 1, (9, 21), dtype=np.int32)
+    b = rng.integers(-2**31, 2**31 - 1, (9, 21), dtype=np.int32)
+    with np.errstate(over="ignore"):
+        want = np.maximum(a - b, np.int32(0)) * a + (-b)
+    assert RO.evaluate(program, [a, b]).tobytes() == want.tobytes()
+    for op, form in (("div", f"%a, %b : ({t}, {t}) -> {t}"), ("leaky_relu", f"%a {{negative_slop = 0.1 : f32}} : {t} -> {t}")):
+        bad = f"func.func @f(%a : {t}, %b : {t}) -> {t} {{\n  %0 = afir.{op} {form}\n  return %0 : {t}\n}}\n"
+        rc, _, err = translate(bad)
+        assert rc == 1 and f"afir.{op} on integer tensors has no HIP lowering" in err, err
+    mixed = ("func.func @f(%a : tensor<4xi32>, %b : tensor<4xf32>) -> tensor<4xf32> {\n"
+             "  %0 = afir.add %a, %b : (tensor<4xi32>, tensor<4xf32>) -> tensor<4xf32>\n  return %0 : tensor<4xf32>\n}\n")
+    rc, _, err = translate(mixed)
+    assert rc == 1 and "integer and floating-point tensors in one operation" in err, err
+
+
 def test_concat_of_three_parts_sums_the_row_offsets():
     out = program_of(MC.THREE_PART_CONCAT)
     offs = [l for l in out.splitlines() if l.startswith("outoff")]
