@@ -38,9 +38,9 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # HBM bytes per step measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (two runs), scaled by the same counters' reading for a plain 256 MiB copy
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Source: profiles/*.txt, section (2).
-MEASURED_TRAFFIC = {"c1": 201364275, "c2": 134645378, "c3": 134506905, "c4": 134146150,
-                    "c5": 2678468608, "g1": 201360281, "g2": 134595481, "i1": 201564364,
-                    "i2": 134977945}
+MEASURED_TRAFFIC = {"c1": 201364377, "c2": 134645398, "c3": 134331904, "c4": 134146560,
+                    "c5": 2466480128, "g1": 201360588, "g2": 134597632, "i1": 201612185,
+                    "i2": 135318732}
 
 
 # Region programs of the two generic-kernel workloads (grammar:
