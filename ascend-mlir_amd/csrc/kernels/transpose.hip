@@ -24,7 +24,7 @@ __device__ __forceinline__ float relu_keep_nan(float v) { return (v > 0.f) ? v :
 // x rows (a wave covers eight 128-byte runs per load), applies relu and + c
 // (its eight columns are fixed, so c is read once) and writes the float32
 // results to tile[i][j], rows padded to 65 words.  Phase 2: a lane reads eight
-// consecutive i of one j (a column of the padded tile: conflict-free), rounds
+// consecutive i of one j (a column of the padded tile: at most two lanes per bank), rounds
 // them to f16 and writes one 16-byte chunk of an output row; eight lanes cover
 // a 128-byte run along M.  Tiles are numbered along M first, so neighbouring
 // workgroups write neighbouring runs of the same output rows.

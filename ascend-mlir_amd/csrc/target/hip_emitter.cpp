@@ -724,7 +724,7 @@ class SegmentEmitter {
   // iteration dim).  Phase 1 loads each transposed operand's tile with 128-bit
   // loads along ITS contiguous dim and writes it to LDS as float32, rows padded
   // by one word; phase 2 is the ordinary row code, 8 lanes per row, reading
-  // those operands from LDS column-wise (conflict-free with the odd pitch).
+  // those operands from LDS column-wise (at most two lanes per bank with the odd pitch).
   void emitBodyTiled() {
     const std::string otag = typeTag(p_.output().type);
     const int p = tileDim_, r = rank_ == 3 ? (p == 0 ? 1 : 0) : -1;
