@@ -96,6 +96,7 @@ struct RegisteredRegion {
   FastPath fast = FastPath::None;
   int fastArgs[4] = {-1, -1, -1, -1};  // argument index of each kernel operand
   float alpha = 0.f;
+  bool relu = false;   // matmul epilogue ends in max(v, 0) instead of max(v, v * alpha)
   std::shared_ptr<CompiledRegion> compiled;   // null: the interpreter kernel runs the program
   bool preferCompiled = false;                // the attached code object outranks a hand-tuned family
 };
@@ -172,9 +173,10 @@ std::string detect_fast_path(RegisteredRegion *r) {
   const bool hasMatmul = !ops.empty() && ops[0].code == OpCode::Matmul;
 
   if (hasMatmul) {
-    // [matmul A B, (push bias (d1), add)?, (leaky alpha)?, store]: the epilogue kinds None, BiasAdd and
-    // BiasAddLeakyRelu of lib/Conversion/MarkStructuredOps/AnnotateMixMatmulSemanticsPass.cpp:319-323
-    // (and leaky relu without a bias)
+    // [matmul A B, (push bias (d1), add)?, (leaky alpha | relu)?, store]: the epilogue kinds None, BiasAdd and
+    // BiasAddLeakyRelu of lib/Conversion/MarkStructuredOps/AnnotateMixMatmulSemanticsPass.cpp:319-323, the
+    // runtime's BiasAddRelu (include/Runtime/Mix/MatmulTilingTypes.h:13; the emitter tells Relu from LeakyRelu
+    // by the vector ops, test/Target/cann-translate-mix-relu.mlir:22-23), and either activation without a bias
     size_t at = 1;
     int bias = -1;
     float alpha = 1.f;   // max(v, v * 1) is v
@@ -182,7 +184,9 @@ std::string detect_fast_path(RegisteredRegion *r) {
       bias = ops[at].arg;
       at += 2;
     }
+    bool relu = false;
     if (at < ops.size() && ops[at].code == OpCode::Leaky) alpha = ops[at++].constant;
+    else if (at < ops.size() && ops[at].code == OpCode::Relu) { relu = true; ++at; }
     if (at + 1 == ops.size() && ops[at].code == OpCode::Store) {
       const int a = ops[0].arg, b = ops[0].arg2;
       if (type(a) == ElemType::BF16 && type(b) == ElemType::BF16 && (bias < 0 || type(bias) == ElemType::BF16) &&
@@ -197,9 +201,10 @@ std::string detect_fast_path(RegisteredRegion *r) {
       }
       r->fastArgs[0] = a; r->fastArgs[1] = b; r->fastArgs[2] = bias;
       r->alpha = alpha;
+      r->relu = relu;
       return "";
     }
-    return "a matmul region must be matmul [-> bias add (per column)] [-> leaky relu]; other epilogues are not implemented";
+    return "a matmul region must be matmul [-> bias add (per column)] [-> leaky relu | relu]; other epilogues are not implemented";
   }
   if (g.rank == 2 && ops.size() == 6 && out == ElemType::F32 && is_push(ops[0], 2, {0, 1}) &&
       is_push(ops[1], 2, {0, 1}) && ops[2].code == OpCode::Add && is_push(ops[3], 2, {0, 1}) &&
@@ -393,7 +398,7 @@ uint32_t afir_hip_launch_matmul_add_leakyrelu(uint32_t block_dim, void *stream, 
   return finish(afir::launch_matmul_add_leakyrelu(
       static_cast<const uint16_t *>(a), static_cast<const uint16_t *>(b),
       static_cast<const uint16_t *>(bias), static_cast<uint16_t *>(out), f[0], f[1], f[2], alpha,
-      block_dim, static_cast<hipStream_t>(stream)));
+      /*relu=*/false, block_dim, static_cast<hipStream_t>(stream)));
 }
 
 uint32_t afir_hip_probe_mfma_rate(void *stream, const void *operands, void *sink, uint32_t iters,
@@ -567,12 +572,12 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
         return finish(afir::launch_matmul_add_leakyrelu(
             static_cast<const uint16_t *>(args[fa[0]]), static_cast<const uint16_t *>(args[fa[1]]),
             fa[2] >= 0 ? static_cast<const uint16_t *>(args[fa[2]]) : nullptr, static_cast<uint16_t *>(out),
-            seg.size[0], res.shapes[fa[0]][1], seg.size[1], r->alpha, block_dim, st));
+            seg.size[0], res.shapes[fa[0]][1], seg.size[1], r->alpha, r->relu, block_dim, st));
       case FastPath::MatmulBiasLeakyF16:
         return finish(afir::launch_matmul_add_leakyrelu_f16(
             static_cast<const uint16_t *>(args[fa[0]]), static_cast<const uint16_t *>(args[fa[1]]),
             fa[2] >= 0 ? static_cast<const float *>(args[fa[2]]) : nullptr, static_cast<float *>(out),
-            seg.size[0], res.shapes[fa[0]][1], seg.size[1], r->alpha, block_dim, st));
+            seg.size[0], res.shapes[fa[0]][1], seg.size[1], r->alpha, r->relu, block_dim, st));
       case FastPath::None: break;
     }
   }

@@ -32,22 +32,23 @@ LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx
                                        int64_t dim, int64_t nidx, uint32_t block_dim,
                                        hipStream_t stream);
 
-// out = bf16(max(v, v*alpha)), v = A@B + bias, f32 accumulate.
+// out = bf16(max(v, v*alpha)), or bf16(max(v, 0)) with relu set; v = A@B + bias, f32 accumulate.
 LaunchStatus launch_matmul_add_leakyrelu(const uint16_t *a, const uint16_t *b,
                                          const uint16_t *bias, uint16_t *out, int64_t m,
-                                         int64_t k, int64_t n, float alpha,
+                                         int64_t k, int64_t n, float alpha, bool relu,
                                          uint32_t block_dim, hipStream_t stream);
 
 // The same with f16 A, B and f32 bias, out (the types of the reference's matmul
 // example, examples/matmul-add-leakyrelu/step0_input.mlir:10-15).
 LaunchStatus launch_matmul_add_leakyrelu_f16(const uint16_t *a, const uint16_t *b, const float *bias,
                                              float *out, int64_t m, int64_t k, int64_t n,
-                                             float alpha, uint32_t block_dim, hipStream_t stream);
+                                             float alpha, bool relu, uint32_t block_dim,
+                                             hipStream_t stream);
 
 // Fast path of the matmul for tile-aligned shapes (matmul_dma.hip).
 bool matmul_dma_supported(int64_t m, int64_t k, int64_t n);
 LaunchStatus launch_matmul_dma(const uint16_t *a, const uint16_t *b, const uint16_t *bias,
-                               uint16_t *out, int m, int k, int n, float alpha,
+                               uint16_t *out, int m, int k, int n, float alpha, bool relu,
                                uint32_t block_dim, hipStream_t stream);
 
 // Matrix-core issue rate from registers only (probe.hip).  operands: 64 KiB of

@@ -60,7 +60,7 @@ template <int WAVES_M, int WAVES_N, int TM, int TN, bool F16IO>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void matmul_bias_leakyrelu_mfma(
     const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
     const void *__restrict__ bias_v, void *__restrict__ out_v, int M, int K, int N,
-    float alpha, int tiles_m, int tiles_n) {
+    float alpha, int relu, int tiles_m, int tiles_n) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int BM = WAVES_M * TM * 32, BN = WAVES_N * TN * 32;
   constexpr int A_STAGE = BM * kPitch, B_STAGE = BN * kPitch, STAGE = A_STAGE + B_STAGE;
@@ -205,10 +205,10 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void matmul_bias_leakyrelu_m
           float v1 = acc[i][j][4 * q + 1] + b1;
           float v2 = acc[i][j][4 * q + 2] + b2;
           float v3 = acc[i][j][4 * q + 3] + b3;
-          v0 = fmaxf(v0, v0 * alpha);
-          v1 = fmaxf(v1, v1 * alpha);
-          v2 = fmaxf(v2, v2 * alpha);
-          v3 = fmaxf(v3, v3 * alpha);
+          v0 = fmaxf(v0, relu ? 0.f : v0 * alpha);
+          v1 = fmaxf(v1, relu ? 0.f : v1 * alpha);
+          v2 = fmaxf(v2, relu ? 0.f : v2 * alpha);
+          v3 = fmaxf(v3, relu ? 0.f : v3 * alpha);
           if constexpr (F16IO) {
             const f32x4 w = {v0, v1, v2, v3};
             *reinterpret_cast<f32x4 *>(static_cast<float *>(out_v) + (int64_t)m * N + n) = w;
@@ -229,7 +229,7 @@ template <bool F16IO>
 __global__ __launch_bounds__(256) void matmul_bias_leakyrelu_any(
     const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
     const void *__restrict__ bias_v, void *__restrict__ out_v, int M, int K, int N,
-    float alpha, int tiles_m, int tiles_n) {
+    float alpha, int relu, int tiles_m, int tiles_n) {
   auto widen = [](uint16_t h) {
     if constexpr (F16IO) return (float)__builtin_bit_cast(_Float16, h);
     else return __uint_as_float((uint32_t)h << 16);
@@ -251,10 +251,10 @@ __global__ __launch_bounds__(256) void matmul_bias_leakyrelu_any(
     if (m < M && n < N) {
       if constexpr (F16IO) {
         float v = acc + (bias_v ? static_cast<const float *>(bias_v)[n] : -0.f);
-        static_cast<float *>(out_v)[(int64_t)m * N + n] = fmaxf(v, v * alpha);
+        static_cast<float *>(out_v)[(int64_t)m * N + n] = fmaxf(v, relu ? 0.f : v * alpha);
       } else {
         float v = acc + (bias_v ? __uint_as_float((uint32_t) static_cast<const uint16_t *>(bias_v)[n] << 16) : -0.f);
-        v = fmaxf(v, v * alpha);
+        v = fmaxf(v, relu ? 0.f : v * alpha);
         static_cast<uint16_t *>(out_v)[(int64_t)m * N + n] = (uint16_t)f32_to_bf16_rne(v);
       }
     }
@@ -263,7 +263,7 @@ __global__ __launch_bounds__(256) void matmul_bias_leakyrelu_any(
 
 template <int WAVES_M, int WAVES_N, int TM, int TN, bool F16IO>
 LaunchStatus launch_mfma(const uint16_t *a, const uint16_t *b, const void *bias, void *out, int m,
-                         int k, int n, float alpha, uint32_t block_dim, hipStream_t stream) {
+                         int k, int n, float alpha, bool relu, uint32_t block_dim, hipStream_t stream) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int BM = WAVES_M * TM * 32, BN = WAVES_N * TN * 32;
   constexpr size_t kLds = 2 * (size_t)(BM + BN) * kPitch;
@@ -276,7 +276,7 @@ LaunchStatus launch_mfma(const uint16_t *a, const uint16_t *b, const void *bias,
   int64_t blocks = (int64_t)tiles_m * tiles_n;
   if (block_dim) blocks = block_dim;
   hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(NT), kLds, stream, a, b, bias, out, m, k,
-                     n, alpha, tiles_m, tiles_n);
+                     n, alpha, relu ? 1 : 0, tiles_m, tiles_n);
   return after_launch();
 }
 
@@ -286,8 +286,8 @@ namespace {
 
 template <bool F16IO>
 LaunchStatus launch_matmul_any_io(const uint16_t *a, const uint16_t *b, const void *bias, void *out,
-                                  int64_t m, int64_t k, int64_t n, float alpha, uint32_t block_dim,
-                                  hipStream_t stream) {
+                                  int64_t m, int64_t k, int64_t n, float alpha, bool relu,
+                                  uint32_t block_dim, hipStream_t stream) {
   if (m < 0 || k < 0 || n < 0) return invalid("matmul_add_leakyrelu: negative extent");
   if (m == 0 || n == 0) return ok_status();
   if (!out) return invalid("matmul_add_leakyrelu: null tensor pointer");   // a null bias means "no bias"
@@ -302,19 +302,19 @@ LaunchStatus launch_matmul_any_io(const uint16_t *a, const uint16_t *b, const vo
   if constexpr (!F16IO) {
     if (al && matmul_dma_supported(m, k, n))
       return launch_matmul_dma(a, b, static_cast<const uint16_t *>(bias), static_cast<uint16_t *>(out),
-                               (int)m, (int)k, (int)n, alpha, block_dim, stream);
+                               (int)m, (int)k, (int)n, alpha, relu, block_dim, stream);
   }
   if (al && k >= kBK && k % kBK == 0 && m % 256 == 0 && n % 256 == 0)
-    return launch_mfma<2, 4, 4, 2, F16IO>(a, b, bias, out, (int)m, (int)k, (int)n, alpha, block_dim, stream);
+    return launch_mfma<2, 4, 4, 2, F16IO>(a, b, bias, out, (int)m, (int)k, (int)n, alpha, relu, block_dim, stream);
   if (al && k >= kBK && k % kBK == 0 && m % 128 == 0 && n % 128 == 0)
-    return launch_mfma<2, 2, 2, 2, F16IO>(a, b, bias, out, (int)m, (int)k, (int)n, alpha, block_dim, stream);
+    return launch_mfma<2, 2, 2, 2, F16IO>(a, b, bias, out, (int)m, (int)k, (int)n, alpha, relu, block_dim, stream);
 
   const int tiles_m = (int)((m + 15) / 16), tiles_n = (int)((n + 15) / 16);
   int64_t blocks = (int64_t)tiles_m * tiles_n;
   if (block_dim) blocks = block_dim;
   if (blocks > 0x7fffffff) blocks = 0x7fffffff;
   hipLaunchKernelGGL(matmul_bias_leakyrelu_any<F16IO>, dim3((unsigned)blocks), dim3(256), 0, stream,
-                     a, b, bias, out, (int)m, (int)k, (int)n, alpha, tiles_m, tiles_n);
+                     a, b, bias, out, (int)m, (int)k, (int)n, alpha, relu ? 1 : 0, tiles_m, tiles_n);
   return after_launch();
 }
 
@@ -322,15 +322,16 @@ LaunchStatus launch_matmul_any_io(const uint16_t *a, const uint16_t *b, const vo
 
 LaunchStatus launch_matmul_add_leakyrelu(const uint16_t *a, const uint16_t *b,
                                          const uint16_t *bias, uint16_t *out, int64_t m,
-                                         int64_t k, int64_t n, float alpha, uint32_t block_dim,
-                                         hipStream_t stream) {
-  return launch_matmul_any_io<false>(a, b, bias, out, m, k, n, alpha, block_dim, stream);
+                                         int64_t k, int64_t n, float alpha, bool relu,
+                                         uint32_t block_dim, hipStream_t stream) {
+  return launch_matmul_any_io<false>(a, b, bias, out, m, k, n, alpha, relu, block_dim, stream);
 }
 
 LaunchStatus launch_matmul_add_leakyrelu_f16(const uint16_t *a, const uint16_t *b, const float *bias,
                                              float *out, int64_t m, int64_t k, int64_t n,
-                                             float alpha, uint32_t block_dim, hipStream_t stream) {
-  return launch_matmul_any_io<true>(a, b, bias, out, m, k, n, alpha, block_dim, stream);
+                                             float alpha, bool relu, uint32_t block_dim,
+                                             hipStream_t stream) {
+  return launch_matmul_any_io<true>(a, b, bias, out, m, k, n, alpha, relu, block_dim, stream);
 }
 
 }  // namespace afir

@@ -149,7 +149,7 @@ template <int WM, int WN>
 __global__ __launch_bounds__(WM * WN * 64) void matmul_bias_leakyrelu_bf16_dma(
     const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
     const uint16_t *__restrict__ bias, uint16_t *__restrict__ out, int M, int K, int N,
-    float alpha, int tiles_m, int tiles_n) {
+    float alpha, int relu, int tiles_m, int tiles_n) {
   extern __shared__ __align__(1024) unsigned char smem[];
   lds_byte *const lds = (lds_byte *)smem;
   const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
@@ -367,10 +367,10 @@ __global__ __launch_bounds__(WM * WN * 64) void matmul_bias_leakyrelu_bf16_dma(
             float v1 = acc[i][j][4 * q + 1] + b1;
             float v2 = acc[i][j][4 * q + 2] + b2;
             float v3 = acc[i][j][4 * q + 3] + b3;
-            v0 = fmaxf(v0, v0 * alpha);
-            v1 = fmaxf(v1, v1 * alpha);
-            v2 = fmaxf(v2, v2 * alpha);
-            v3 = fmaxf(v3, v3 * alpha);
+            v0 = fmaxf(v0, relu ? 0.f : v0 * alpha);
+            v1 = fmaxf(v1, relu ? 0.f : v1 * alpha);
+            v2 = fmaxf(v2, relu ? 0.f : v2 * alpha);
+            v3 = fmaxf(v3, relu ? 0.f : v3 * alpha);
             u32x2 w;
             w.x = pack_bf16(v0, v1);
             w.y = pack_bf16(v2, v3);
@@ -410,7 +410,7 @@ bool matmul_dma_supported(int64_t m, int64_t k, int64_t n) {
 #endif
 
 LaunchStatus launch_matmul_dma(const uint16_t *a, const uint16_t *b, const uint16_t *bias,
-                               uint16_t *out, int m, int k, int n, float alpha,
+                               uint16_t *out, int m, int k, int n, float alpha, bool relu,
                                uint32_t block_dim, hipStream_t stream) {
   constexpr int WM = AFIR_MM_WAVES_M, WN = AFIR_MM_WAVES_N;
   auto kernel = matmul_bias_leakyrelu_bf16_dma<WM, WN>;
@@ -425,7 +425,7 @@ LaunchStatus launch_matmul_dma(const uint16_t *a, const uint16_t *b, const uint1
   if (blocks > AFIR_MM_GRID) blocks = AFIR_MM_GRID;
   if (block_dim) blocks = block_dim;
   hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(WM * WN * 64), kLdsBytes, stream, a, b,
-                     bias, out, m, k, n, alpha, tiles_m, tiles_n);
+                     bias, out, m, k, n, alpha, relu ? 1 : 0, tiles_m, tiles_n);
   return after_launch();
 }
 

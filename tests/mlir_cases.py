@@ -174,6 +174,34 @@ func.func @mm_bias(%a : tensor<?x?xf16>, %b : tensor<?x?xf16>, %bias : tensor<?x
 MATMUL_PLAIN_BF16 = MATMUL_PLAIN_F16.replace("xf16", "xbf16").replace("f32", "bf16").replace("@mm_plain", "@mm_plain_bf16")
 MATMUL_BIAS_BF16 = MATMUL_BIAS_F16.replace("xf16", "xbf16").replace("f32", "bf16").replace("@mm_bias", "@mm_bias_bf16")
 
+# matmul -> bias add -> relu, and matmul -> relu: the runtime's BiasAddRelu epilogue
+# (include/Runtime/Mix/MatmulTilingTypes.h:13); relu spelled maximumf(x, 0.0) as in
+# test/Target/cann-translate-mix-relu-input.mlir.
+MATMUL_BIAS_RELU_F16 = MATMUL_BIAS_LEAKY_F16.replace("%alpha = arith.constant 1.0e-3 : f32", "%alpha = arith.constant 0.0 : f32") \
+    .replace("      %t = arith.mulf %x, %alpha : f32\n", "").replace("arith.maximumf %x, %t", "arith.maximumf %x, %alpha") \
+    .replace("@mm_bias_leaky", "@mm_bias_relu")
+MATMUL_BIAS_RELU_BF16 = MATMUL_BIAS_RELU_F16.replace("xf16", "xbf16").replace("f32", "bf16").replace("@mm_bias_relu", "@mm_bias_relu_bf16")
+MATMUL_RELU_F16 = """
+#all = affine_map<(d0, d1) -> (d0, d1)>
+func.func @mm_relu(%a : tensor<?x?xf16>, %b : tensor<?x?xf16>, %init : tensor<?x?xf32>) -> tensor<?x?xf32> {
+  %c0 = arith.constant 0 : index
+  %c1 = arith.constant 1 : index
+  %m = tensor.dim %init, %c0 : tensor<?x?xf32>
+  %n = tensor.dim %init, %c1 : tensor<?x?xf32>
+  %c = linalg.matmul ins(%a, %b : tensor<?x?xf16>, tensor<?x?xf16>) outs(%init : tensor<?x?xf32>) -> tensor<?x?xf32>
+  %zero = arith.constant 0.0 : f32
+  %e1 = tensor.empty(%m, %n) : tensor<?x?xf32>
+  %e = linalg.generic {indexing_maps = [#all, #all], iterator_types = ["parallel", "parallel"]}
+      ins(%c : tensor<?x?xf32>) outs(%e1 : tensor<?x?xf32>) {
+    ^bb0(%x: f32, %o: f32):
+      %v = arith.maximumf %x, %zero : f32
+      linalg.yield %v : f32
+  } -> tensor<?x?xf32>
+  return %e : tensor<?x?xf32>
+}
+"""
+MATMUL_RELU_BF16 = MATMUL_RELU_F16.replace("xf16", "xbf16").replace("f32", "bf16").replace("@mm_relu", "@mm_relu_bf16")
+
 # An AscGraph in AFIR form (the structure of python/afir-to-ascir/asc_graph.afir:1-13:
 # load, load, broadcast, add, mul, sub, store, every op with an attribute
 # dictionary): out = (x + y) - (x + y) * y with y broadcast over the rows.

@@ -236,11 +236,12 @@ def test_two_kernel_session_feeds_one_kernel_into_the_next(tmp_path):
     assert np.allclose(np.load(tmp_path / "y.npy"), want, rtol=1e-5, atol=1e-3)
 
 
-@pytest.mark.parametrize("kind", ["none", "bias"])
+@pytest.mark.parametrize("kind", ["none", "bias", "bias_relu", "relu"])
 @pytest.mark.parametrize("ty", ["f16", "bf16"])
 def test_matmul_epilogue_kinds(pkg, kind, ty):
-    """matmul with no epilogue and with a bias add only (the reference's epilogue
-    kinds "None" and "BiasAdd") on the MFMA kernels.  Small-integer operands:
+    """matmul with no epilogue, with a bias add only (the reference's epilogue
+    kinds "None" and "BiasAdd"), with bias add and relu (its runtime's
+    "BiasAddRelu") and with relu alone, on the MFMA kernels.  Small-integer operands:
     every product and partial sum is exact in float32
     (examples/matmul-add-leakyrelu/gen_data.py:29-31), so the result does not
     depend on the order of accumulation; negative sums keep their sign without a
@@ -250,7 +251,10 @@ def test_matmul_epilogue_kinds(pkg, kind, ty):
     from oracle import region_oracle as RO
     H.load()
     mlir = {("none", "f16"): MC.MATMUL_PLAIN_F16, ("bias", "f16"): MC.MATMUL_BIAS_F16,
-            ("none", "bf16"): MC.MATMUL_PLAIN_BF16, ("bias", "bf16"): MC.MATMUL_BIAS_BF16}[(kind, ty)]
+            ("none", "bf16"): MC.MATMUL_PLAIN_BF16, ("bias", "bf16"): MC.MATMUL_BIAS_BF16,
+            ("bias_relu", "f16"): MC.MATMUL_BIAS_RELU_F16, ("bias_relu", "bf16"): MC.MATMUL_BIAS_RELU_BF16,
+            ("relu", "f16"): MC.MATMUL_RELU_F16, ("relu", "bf16"): MC.MATMUL_RELU_BF16}[(kind, ty)]
+    has_bias = kind in ("bias", "bias_relu")
     p = subprocess.run([TR, "-mlir-to-hip", "-"], input=mlir, capture_output=True, text=True)
     assert p.returncode == 0, p.stderr
     for (m, k, n) in ((512, 256, 512), (96, 64, 40)):
@@ -258,15 +262,17 @@ def test_matmul_epilogue_kinds(pkg, kind, ty):
         a = rng.integers(-3, 4, (m, k)).astype(np.float32)
         b = rng.integers(-3, 4, (k, n)).astype(np.float32)
         bias = rng.integers(-8, 9, (n,)).astype(np.float32)
-        exact = a @ b + (bias[None, :] if kind == "bias" else 0.0)      # integers: exact in float32
+        exact = a @ b + (bias[None, :] if has_bias else 0.0)      # integers: exact in float32
+        if kind.endswith("relu"):
+            exact = np.maximum(exact, 0.0) + 0.0          # +0 where the sum is negative or zero
         assert np.abs(exact).max() < 2 ** 24
         if ty == "f16":
-            ins = [a.astype(np.float16), b.astype(np.float16)] + ([bias] if kind == "bias" else [])
+            ins = [a.astype(np.float16), b.astype(np.float16)] + ([bias] if has_bias else [])
             init = np.zeros((m, n), np.float32)
             want = exact.astype(np.float32)
             dev = [torch.from_numpy(x).cuda() for x in ins + [init]]
         else:
-            ins = [O.f32_to_bf16_bits(a), O.f32_to_bf16_bits(b)] + ([O.f32_to_bf16_bits(bias)] if kind == "bias" else [])
+            ins = [O.f32_to_bf16_bits(a), O.f32_to_bf16_bits(b)] + ([O.f32_to_bf16_bits(bias)] if has_bias else [])
             init = O.f32_to_bf16_bits(np.zeros((m, n), np.float32))
             want = O.f32_to_bf16_bits(exact.astype(np.float32))
             dev = [torch.from_numpy(x.view(np.int16)).cuda().view(torch.bfloat16) for x in ins + [init]]

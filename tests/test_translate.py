@@ -72,7 +72,12 @@ def test_matmul_epilogue_kinds_none_and_bias_add(pkg):
     for mlir, tail in ((MC.MATMUL_PLAIN_F16, ["matmul arg0 arg1", "store", "end"]),
                        (MC.MATMUL_BIAS_F16, ["matmul arg0 arg1", "push arg2 d1", "add", "store", "end"]),
                        (MC.MATMUL_PLAIN_BF16, ["matmul arg0 arg1", "store", "end"]),
-                       (MC.MATMUL_BIAS_BF16, ["matmul arg0 arg1", "push arg2 d1", "add", "store", "end"])):
+                       (MC.MATMUL_BIAS_BF16, ["matmul arg0 arg1", "push arg2 d1", "add", "store", "end"]),
+                       # the runtime's BiasAddRelu (include/Runtime/Mix/MatmulTilingTypes.h:13) and relu alone
+                       (MC.MATMUL_BIAS_RELU_F16, ["matmul arg0 arg1", "push arg2 d1", "add", "relu", "store", "end"]),
+                       (MC.MATMUL_BIAS_RELU_BF16, ["matmul arg0 arg1", "push arg2 d1", "add", "relu", "store", "end"]),
+                       (MC.MATMUL_RELU_F16, ["matmul arg0 arg1", "relu", "store", "end"]),
+                       (MC.MATMUL_RELU_BF16, ["matmul arg0 arg1", "relu", "store", "end"])):
         out = program_of(mlir)
         body = [l.strip() for l in out.splitlines() if l.strip() and not l.startswith("#")]
         assert body[-len(tail):] == tail, out
