@@ -102,6 +102,9 @@ uint64_t programHash(const afir_region::Program &p);
 // Kernel symbol of a segment: idx32 = positions fit 32 bits, aligned = every
 // vector access of the launch is 16-byte aligned and rows are whole vectors.
 std::string specKernelName(int segment, bool idx32, bool aligned);
+// Reduce segments also have a workgroup-per-row kernel for rows of exactly
+// 256 * unroll * width elements whose accesses are all 128-bit.
+std::string specRowsKernelName(int segment, bool idx32);
 
 // Emits the source for every segment.  Returns "" on success, else why the
 // program has no specialised form (matmul segments: those run on the

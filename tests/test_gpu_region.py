@@ -90,6 +90,49 @@ def test_reductions_within_tolerance(H, name):
     assert np.all(np.abs(got - want.astype(np.float64)) <= tol)
 
 
+@pytest.mark.parametrize("ty,n", [("f32", 1024), ("f32", 2048), ("f32", 4096), ("f16", 2048), ("f16", 4096),
+                                  ("f16", 8192), ("f32", 3072), ("f16", 1024)])
+@pytest.mark.parametrize("rows", [1, 5, 1100])
+def test_row_sums_of_workgroup_sized_rows(H, ty, n, rows):
+    """Rows of 256 lanes x 4 groups (4096 floats, 8192 halves) take the compiled
+    workgroup-per-row kernel; with 1100 rows the grid is held to 7 workgroups, so every
+    workgroup fetches rows ahead.  The other lengths stay on the wavefront-per-row
+    kernel.  Sums of small integers are exact in
+    float32 whatever the order, so the result must equal the oracle's bit for bit; a
+    second run with uniform values is held to the tolerance of a reordered sum."""
+    dt = np.float32 if ty == "f32" else np.float16
+    text = RC.C2_BCAST_ADD_ROWSUM.replace("f32", ty)
+    rng = np.random.default_rng(rows * 7 + n)
+    x = rng.integers(-4, 5, (rows, n)).astype(dt)
+    bias = rng.integers(-4, 5, (n,)).astype(dt)
+    want = RO.evaluate(text, [x, bias])
+    block_dim = 7 if rows == 1100 else 0
+    got = run(H, text, [x, bias], (rows,), block_dim=block_dim)
+    assert got.tobytes() == want.tobytes()
+    x = rng.uniform(-1, 1, (rows, n)).astype(dt)
+    bias = rng.uniform(-1, 1, (n,)).astype(dt)
+    want = RO.evaluate(text, [x, bias]).astype(np.float64)
+    got = run(H, text, [x, bias], (rows,), block_dim=block_dim).astype(np.float64)
+    scale = np.abs(x.astype(np.float64) + bias.astype(np.float64)).sum(axis=1)
+    ulp = 2.0 ** -10 if ty == "f16" else 0.0
+    assert np.all(np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-6 * scale + ulp * np.abs(want))
+
+
+def test_row_sums_with_a_row_operand_and_rank_3(H):
+    """The workgroup-per-row kernels with an operand that changes with the row (fetched
+    ahead with the matrix) and over a rank-3 space whose row is (d0, d1)."""
+    rng = np.random.default_rng(31)
+    text = RC.REDUCE_ROWBIAS                                   # r[d0] + x[d0, d1], f16, n = 8192
+    r = rng.integers(-3, 4, (300,)).astype(np.float16)
+    x = rng.integers(-3, 4, (300, 8192)).astype(np.float16)
+    assert run(H, text, [r, x], (300,), block_dim=11).tobytes() == RO.evaluate(text, [r, x]).tobytes()
+    text3 = RC.HEADER + ("arg in f32 3\narg in f32 2\narg out f32 2\nsegment 3\n size arg0.0 arg0.1 arg0.2\n outoff 0\n"
+                         " push arg0 d0 d1 d2\n push arg1 d0 d2\n mul\n reduce sum\n store\nend\n")
+    a = rng.integers(-3, 4, (7, 50, 4096)).astype(np.float32)
+    b = rng.integers(-3, 4, (7, 4096)).astype(np.float32)
+    assert run(H, text3, [a, b], (7, 50), block_dim=13).tobytes() == RO.evaluate(text3, [a, b]).tobytes()
+
+
 @pytest.mark.parametrize("shape", [(1, 1), (3, 5), (7, 8), (5, 9), (64, 1000), (2, 4099), (0, 8), (4, 0)])
 def test_ragged_shapes_and_block_dim(H, shape):
     rng = np.random.default_rng(11)

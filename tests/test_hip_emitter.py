@@ -99,6 +99,18 @@ def test_integer_regions_use_wrapping_integer_arithmetic():
     assert "ldv_i16<W, true>(R.in[0].base" in mixed and "ldd_i32(R.in[1].base" in mixed
 
 
+def test_reductions_also_get_a_workgroup_per_row_kernel():
+    src = _emit(RC.C2_BCAST_ADD_ROWSUM).stdout
+    assert "rows of exactly 4096 elements: a workgroup per row, the next row in flight" in src
+    assert "afir_region_s0_rows_i32(" in src and "afir_region_s0_rows_i64(" in src
+    rows = src[src.index("DEV void segment0_rows"):]
+    rows = rows[:rows.index("KERNEL")]
+    # the bias does not change with the row: loaded once, before the loop, not in the fetch of the next row
+    assert rows.count("ldv_f32<W, false>(R.in[1].base") == 1 and rows.count("ldv_f32<W, true>(R.in[0].base") == 2
+    assert rows.count("__builtin_amdgcn_s_barrier();") == 1
+    assert "_rows_" not in _emit(RC.C1_ADD_MUL).stdout            # parallel segments have none
+
+
 def test_identical_reads_are_loaded_once():
     src = _emit(RC.C1_ADD_MUL).stdout           # (a + b) * b reads b twice
     assert src.count("ldv_f32<W, true>(R.in[1].base") == 1 and "R.in[2]" not in src
