@@ -675,6 +675,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
       sa.out_vec = a.out_vec;
       sa.lanes_log2 = g.lanes_log2;
       sa.grid = (int)g.blocks;
+      sa.column_blocks = (int)g.column_blocks;
       bool all_aligned, row_groups = false;
       if (tile.tiled) {
         // one workgroup pass per tile of tile_p x tile_q
@@ -686,6 +687,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
         int64_t blocks = tiles < (int64_t)afir::kNumCU * 256 ? tiles : (int64_t)afir::kNumCU * 256;
         if (block_dim) blocks = block_dim;
         sa.grid = (int)blocks;
+        sa.column_blocks = 1;
         all_aligned = seg.size[last] % emit.tileQ == 0 && seg.size[tile.dim] % emit.tileP == 0 &&
                       a.out_vec;
       } else {
@@ -728,6 +730,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
         int64_t blocks = nrows < (int64_t)afir::kNumCU * 16 ? nrows : (int64_t)afir::kNumCU * 16;
         if (block_dim) blocks = block_dim;
         sa.grid = (int)blocks;
+        sa.column_blocks = 1;
       } else {
         row_groups = false;
       }

@@ -387,10 +387,12 @@ __global__ __launch_bounds__(kThreads) void fused_region_parallel(const RegionAr
   const int rows_per_pass = kThreads >> lanes_log2;
   const I local_row = (I)(threadIdx.x >> lanes_log2);
   const I first_chunk = (I)(threadIdx.x & (lanes - 1));
+  // blockIdx.y: which stretches of a long row this workgroup takes (few, long rows
+  // are spread over workgroups along the row as well)
   for (I row0 = (I)blockIdx.x * rows_per_pass; row0 < rows; row0 += (I)gridDim.x * rows_per_pass) {
     const I row = row0 + local_row;
     if (row >= rows) continue;
-    for (I chunk = first_chunk; chunk < chunks; chunk += lanes) {
+    for (I chunk = first_chunk + (I)blockIdx.y * lanes; chunk < chunks; chunk += (I)gridDim.y * lanes) {
       const I j0 = chunk * V;
       const I left = n - j0;
       const int nvalid = left >= V ? V : (int)left;
@@ -601,8 +603,18 @@ LaunchStatus plan_fused_region(const RegionArgs &args, int vec, uint32_t block_d
   const int rows_per_pass = kThreads >> lanes_log2;
   int64_t blocks = (rows + rows_per_pass - 1) / rows_per_pass;
   if (blocks > (int64_t)kNumCU * 16) blocks = (int64_t)kNumCU * 16;
-  if (block_dim) blocks = block_dim;
-  g->blocks = blocks;
+  // few rows that are longer than one pass of the workgroup: more workgroups along the row
+  const int64_t passes = (chunks + ((int64_t)1 << lanes_log2) - 1) >> lanes_log2;
+  int64_t column_blocks = (int64_t)kNumCU * 16 / blocks;
+  if (column_blocks > passes) column_blocks = passes;
+  if (column_blocks > 65535) column_blocks = 65535;
+  if (column_blocks < 1) column_blocks = 1;
+  if (block_dim) {
+    blocks = block_dim;
+    column_blocks = 1;
+  }
+  g->blocks = blocks * column_blocks;
+  g->column_blocks = column_blocks;
   g->lanes_log2 = lanes_log2;
   return ok_status();
 }
@@ -660,7 +672,8 @@ LaunchStatus launch_fused_region(const RegionArgs &args_in, uint32_t block_dim, 
   auto kernel = wide ? (idx32 ? fused_region_parallel<int, true, 16> : fused_region_parallel<int64_t, true, 16>)
                 : args.chain ? (idx32 ? fused_region_parallel<int, true, 8> : fused_region_parallel<int64_t, true, 8>)
                              : (idx32 ? fused_region_parallel<int, false, 8> : fused_region_parallel<int64_t, false, 8>);
-  hipLaunchKernelGGL(kernel, dim3((unsigned)g.blocks), dim3(kThreads), 0, stream, args, g.lanes_log2);
+  hipLaunchKernelGGL(kernel, dim3((unsigned)(g.blocks / g.column_blocks), (unsigned)g.column_blocks), dim3(kThreads), 0,
+                     stream, args, g.lanes_log2);
   return after_launch();
 }
 

@@ -106,7 +106,9 @@ LaunchStatus launch_fused_region(const RegionArgs &args, uint32_t block_dim, hip
 // Launch geometry of a segment for `vec` elements per lane and step: shared by
 // the interpreter kernels and by kernels compiled for one program.
 struct RegionGeometry {
-  int64_t blocks = 0;    // workgroups of 256 lanes
+  int64_t blocks = 0;    // workgroups of 256 lanes (parallel segments: row blocks x column blocks)
+  int64_t column_blocks = 1;   // parallel segments: workgroups that share a pass of rows, each taking
+                               // every column_blocks-th stretch of 2^lanes_log2 lane-loads of the row
   int lanes_log2 = 0;    // parallel segments: 2^lanes_log2 lanes share a row
   bool idx32 = false;    // every position fits 32 bits
   bool empty = false;    // nothing to compute

@@ -38,7 +38,7 @@ struct SpecArgs {
   int out_vec;
   int lanes_log2;
   int grid;
-  int pad;
+  int column_blocks;
   SpecInput in[8];
 };
 
@@ -714,12 +714,15 @@ class SegmentEmitter {
     line(1, "const I rows_per_pass = (I)(256 >> R.lanes_log2);");
     line(1, "const I local_row = (I)(tid >> R.lanes_log2);");
     line(1, "const I first_group = (I)tid & (lanes - 1);");
-    line(1, "for (I row0 = bid * rows_per_pass; row0 < rows; row0 += nblocks * rows_per_pass) {");
+    line(1, "// few, long rows: column_blocks workgroups share a pass of rows, each taking every column_blocks-th stretch");
+    line(1, "const I cblocks = (I)R.column_blocks, rblocks = cblocks == 1 ? nblocks : nblocks / cblocks;");
+    line(1, "const I cbid = cblocks == 1 ? (I)0 : bid / rblocks, rbid = bid - cbid * rblocks;");
+    line(1, "for (I row0 = rbid * rows_per_pass; row0 < rows; row0 += rblocks * rows_per_pass) {");
     line(2, "const I row = row0 + local_row;");
     line(2, "if (row >= rows) continue;");
     emitPositionOfRow(2);
     emitRowInvariants(2);
-    line(2, "for (I first = first_group; first < groups; first += lanes * U) {");
+    line(2, "for (I first = first_group + cbid * lanes * U; first < groups; first += cblocks * lanes * U) {");
     emitGroups(3, "first", "lanes");
     const Value v = emitExpression(3);
     std::string res = v.name;

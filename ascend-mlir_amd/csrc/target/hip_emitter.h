@@ -45,7 +45,8 @@ struct SpecArgs {
   int out_vec;         // 128-bit stores are aligned for every full vector
   int lanes_log2;      // parallel segments: lanes of the workgroup that share a row
   int grid;            // number of workgroups launched
-  int pad;
+  int column_blocks;   // parallel segments: of these, the workgroups that share a pass of rows and
+                       // split the row between them (grid is a multiple of it; 1 elsewhere)
   SpecInput in[kSpecMaxInputs];
 };
 

@@ -144,6 +144,24 @@ def test_ragged_shapes_and_block_dim(H, shape):
         assert got.tobytes() == want.tobytes()
 
 
+@pytest.mark.parametrize("shape", [(1 << 20,), ((1 << 20) + 13,), (3, 300000), (2, 5, 70001), (1, 9000)])
+def test_few_long_rows_are_spread_along_the_row(H, shape):
+    """Rank-1 tensors and a few very long rows: more workgroups than rows, each taking
+    stretches of the row; whole passes and ragged tails, f16 and f32."""
+    rng = np.random.default_rng(len(shape) * 100 + shape[-1] % 97)
+    rank = len(shape)
+    dims = " ".join(f"d{k}" for k in range(rank))
+    size = " ".join(f"arg0.{k}" for k in range(rank))
+    for ty, dt in (("f16", np.float16), ("f32", np.float32)):
+        text = RC.HEADER + (f"arg in {ty} {rank}\narg in {ty} 1\narg out {ty} {rank}\nsegment {rank}\n size {size}\n outoff 0\n"
+                            f" push arg0 {dims}\n push arg1 d{rank - 1}\n mul\n relu\n store\nend\n")
+        x = rng.uniform(-2, 2, shape).astype(dt)
+        c = rng.uniform(-2, 2, shape[-1:]).astype(dt)
+        want = RO.evaluate(text, [x, c])
+        got = run(H, text, [x, c], shape)
+        assert got.tobytes() == want.tobytes(), (ty, shape)
+
+
 def test_unaligned_bases_take_the_element_path(H):
     import torch
     rng = np.random.default_rng(12)
