@@ -693,7 +693,22 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
       } else {
         // the aligned variant has no tail handling: whole groups, whole passes
         const int64_t groups = seg.size[last] / W;
-        const int64_t per_pass = (seg.reduce ? (int64_t)64 : ((int64_t)1 << g.lanes_log2)) * U;
+        if (seg.reduce) {
+          // lanes of a wavefront that share a row: enough for one pass over a short row, the wavefront otherwise
+          const int64_t all_groups = (seg.size[last] + W - 1) / W;
+          int ll = 0;
+          while (ll < 6 && ((int64_t)U << ll) < all_groups) ++ll;
+          sa.lanes_log2 = ll;
+          if (!block_dim) {
+            int64_t nrows = 1;
+            for (int k = 0; k < last; ++k) nrows *= seg.size[k];
+            const int64_t rows_per_block = (int64_t)4 * (64 >> ll);
+            int64_t blocks = (nrows + rows_per_block - 1) / rows_per_block;
+            if (blocks > (int64_t)afir::kNumCU * 16) blocks = (int64_t)afir::kNumCU * 16;
+            sa.grid = (int)blocks;
+          }
+        }
+        const int64_t per_pass = ((int64_t)1 << sa.lanes_log2) * U;
         all_aligned = seg.size[last] % W == 0 && groups % per_pass == 0 && (seg.reduce || a.out_vec);
         // a row that fills a workgroup of 256 lanes with U groups each: a workgroup per row
         row_groups = seg.reduce && all_aligned && groups == (int64_t)256 * U;

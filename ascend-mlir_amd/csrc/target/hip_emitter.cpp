@@ -209,6 +209,13 @@ DEV float wave_sum(float v) {
   const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 48));
   return (r0 + r1) + (r2 + r3);
 }
+// ---- sum over aligned sets of `lanes` (a power of two below 64) lanes: butterfly, fixed order.
+// The lanes of a set are all active or all inactive.
+DEV float lanes_sum(float v, int lane, int lanes) {
+  for (int m = lanes >> 1; m >= 1; m >>= 1)
+    v += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ m) << 2, __builtin_bit_cast(int, v)));
+  return v;
+}
 )HIP";
 
 const char *typeTag(ElemType t) {
@@ -674,10 +681,15 @@ class SegmentEmitter {
       if (o.step != Operand::Broadcast && o.gatherDim != last_)
         line(1, "const bool vec" + id(o) + " = " + in(o) + ".vec != 0" + (o.gatherDim >= 0 ? " && " + in(o) + ".gvec != 0" : "") + ";");
     if (reduce_) {
+      line(1, "// 2^lanes_log2 (at most 64) lanes of a wavefront share a row: short rows get several rows per wavefront");
       line(1, "const int lane = tid & 63;");
+      line(1, "const I lanes = (I)1 << R.lanes_log2;");
+      line(1, "const I rows_per_wave = (I)(64 >> R.lanes_log2);");
       line(1, "const I wave = bid * 4 + (I)(tid >> 6);");
       line(1, "const I nwaves = nblocks * 4;");
-      line(1, "for (I row = wave; row < rows; row += nwaves) {");
+      line(1, "for (I row0 = wave * rows_per_wave; row0 < rows; row0 += nwaves * rows_per_wave) {");
+      line(2, "const I row = row0 + (I)(lane >> R.lanes_log2);");
+      line(2, "if (row >= rows) continue;");
       emitPositionOfRow(2);
       emitRowInvariants(2);
       line(2, "float acc[U][W];");
@@ -685,8 +697,8 @@ class SegmentEmitter {
       line(2, "for (int u = 0; u < U; ++u)");
       unroll();
       line(3, "for (int e = 0; e < W; ++e) acc[u][e] = 0.f;");
-      line(2, "for (I first = (I)lane; first < groups; first += 64 * U) {");
-      emitGroups(3, "first", "(I)64");
+      line(2, "for (I first = (I)lane & (lanes - 1); first < groups; first += lanes * U) {");
+      emitGroups(3, "first", "lanes");
       const Value v = emitExpression(3);
       unroll();
       line(3, "for (int u = 0; u < U; ++u)");
@@ -704,8 +716,8 @@ class SegmentEmitter {
       line(2, "for (int w = W / 2; w >= 1; w >>= 1)");
       unroll();
       line(3, "for (int e = 0; e < w; ++e) acc[0][e] = acc[0][2 * e] + acc[0][2 * e + 1];");
-      line(2, "const float s = wave_sum(acc[0][0]);");
-      line(2, "if (lane == 0) st_" + otag + "(R.out, (long long)row, s);");
+      line(2, "const float s = R.lanes_log2 == 6 ? wave_sum(acc[0][0]) : lanes_sum(acc[0][0], lane, (int)lanes);");
+      line(2, "if ((lane & ((int)lanes - 1)) == 0) st_" + otag + "(R.out, (long long)row, s);");
       line(1, "}");
       os_ << "}\n";
       return;

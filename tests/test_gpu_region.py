@@ -118,6 +118,20 @@ def test_row_sums_of_workgroup_sized_rows(H, ty, n, rows):
     assert np.all(np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-6 * scale + ulp * np.abs(want))
 
 
+@pytest.mark.parametrize("n", [1, 3, 8, 16, 40, 64, 100, 256, 520])
+def test_row_sums_of_short_rows(H, n):
+    """Rows shorter than a pass of the wavefront: 1, 2, 4 ... 32 lanes share a row and a
+    wavefront takes several rows; row counts that leave the last wavefront partly empty."""
+    rng = np.random.default_rng(n)
+    for ty, dt in (("f32", np.float32), ("f16", np.float16)):
+        text = RC.C2_BCAST_ADD_ROWSUM.replace("f32", ty)
+        for rows in (1, 7, 1000):
+            x = rng.integers(-4, 5, (rows, n)).astype(dt)
+            bias = rng.integers(-4, 5, (n,)).astype(dt)
+            want = RO.evaluate(text, [x, bias])
+            assert run(H, text, [x, bias], (rows,)).tobytes() == want.tobytes(), (ty, rows, n)
+
+
 def test_row_sums_with_a_row_operand_and_rank_3(H):
     """The workgroup-per-row kernels with an operand that changes with the row (fetched
     ahead with the matrix) and over a rank-3 space whose row is (d0, d1)."""
