@@ -605,8 +605,10 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
   struct PendingSegment {
     int segment;
     afir_target::SpecArgs args;
-    bool idx32, aligned;
+    bool idx32;
+    int mode;    // afir_target::SpecMode
     bool rows;   // the workgroup-per-row kernel of a reduce segment
+    bool slim;   // the kernel whose lanes take one group each (short rows)
   };
   std::vector<PendingSegment> pending;   // compiled kernels to launch, non-empty segments only
   for (const afir_region::ResolvedSegment &seg : res.segments) {
@@ -662,11 +664,18 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
       const int segment = (int)(&seg - res.segments.data());
       const afir_target::SpecShape shape = afir_target::specShape(r->program, segment, emit);
       const afir_target::SpecTile tile = afir_target::specTile(r->program, segment);
-      const int W = shape.width, U = shape.unroll;
+      const int W = shape.width;
+      // Rows of fewer than 8 x unroll groups leave most of a lane's groups empty and make a wavefront's
+      // loads touch short pieces of many rows: those run on the kernel whose lanes take one group each
+      // (it exists with 32-bit positions, for launches whose 128-bit accesses are all aligned).
+      const int64_t row_groups_all = (seg.size[seg.rank - 1] + W - 1) / W;
+      bool skip = false;
+      uint32_t failed = AFIR_HIP_OK;
+      auto prepare = [&](const int U, const bool slim, PendingSegment *made) -> bool {
       afir::RegionGeometry g;
       uint32_t rc = finish(afir::plan_fused_region(a, W * U, block_dim, &g));
-      if (rc != AFIR_HIP_OK) return rc;
-      if (g.empty) continue;
+      if (rc != AFIR_HIP_OK) { failed = rc; return false; }
+      if (g.empty) { skip = true; return false; }
       afir_target::SpecArgs sa;
       std::memset(&sa, 0, sizeof sa);
       for (int k = 0; k < 3; ++k) sa.size[k] = a.size[k];
@@ -676,7 +685,8 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
       sa.lanes_log2 = g.lanes_log2;
       sa.grid = (int)g.blocks;
       sa.column_blocks = (int)g.column_blocks;
-      bool all_aligned, row_groups = false;
+      // vectors: every 128-bit access is aligned and rows are whole vectors; whole: no pass has a tail
+      bool vectors, whole, row_groups = false;
       if (tile.tiled) {
         // one workgroup pass per tile of tile_p x tile_q
         const int64_t tq = (seg.size[last] + emit.tileQ - 1) / emit.tileQ;
@@ -688,8 +698,8 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
         if (block_dim) blocks = block_dim;
         sa.grid = (int)blocks;
         sa.column_blocks = 1;
-        all_aligned = seg.size[last] % emit.tileQ == 0 && seg.size[tile.dim] % emit.tileP == 0 &&
-                      a.out_vec;
+        vectors = a.out_vec != 0;
+        whole = seg.size[last] % emit.tileQ == 0 && seg.size[tile.dim] % emit.tileP == 0;
       } else {
         // the aligned variant has no tail handling: whole groups, whole passes
         const int64_t groups = seg.size[last] / W;
@@ -709,9 +719,10 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
           }
         }
         const int64_t per_pass = ((int64_t)1 << sa.lanes_log2) * U;
-        all_aligned = seg.size[last] % W == 0 && groups % per_pass == 0 && (seg.reduce || a.out_vec);
+        vectors = seg.size[last] % W == 0 && (seg.reduce || a.out_vec);
+        whole = groups % per_pass == 0;
         // a row that fills a workgroup of 256 lanes with U groups each: a workgroup per row
-        row_groups = seg.reduce && all_aligned && groups == (int64_t)256 * U;
+        row_groups = !slim && seg.reduce && groups == (int64_t)256 * U;
       }
       for (int i = 0; i < a.ninputs; ++i) {
         const afir::RegionInput &d = a.in[i];
@@ -731,14 +742,16 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
           for (int k = 0; k < seg.rank; ++k)
             if (k != tile.dim && seg.size[k] > 1 && (d.stride[k] * es) % 16 != 0) tvec = false;
           t.vec = tvec ? 1 : 0;
-          if (!tvec) all_aligned = false;
+          if (!tvec) vectors = false;
           continue;
         }
         // operands that are contiguous along the innermost dim are read with
         // 128-bit loads by the aligned variant
-        if (d.stride[last] == 1 && d.gdim != last && (!d.vec || (d.gdim >= 0 && !d.gvec))) all_aligned = false;
+        if (d.stride[last] == 1 && d.gdim != last && (!d.vec || (d.gdim >= 0 && !d.gvec))) vectors = false;
       }
-      if (row_groups && all_aligned) {
+      const int mode = vectors && whole ? afir_target::kSpecAligned
+                       : vectors && !tile.tiled ? afir_target::kSpecVector : afir_target::kSpecGeneral;
+      if (row_groups && mode == afir_target::kSpecAligned) {
         // up to 16 workgroups per CU walk the rows (4 to 16 measured within 1 %, 2 slower)
         int64_t nrows = 1;
         for (int k = 0; k < last; ++k) nrows *= seg.size[k];
@@ -749,7 +762,16 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
       } else {
         row_groups = false;
       }
-      pending.push_back({segment, sa, g.idx32, all_aligned, row_groups});
+      if (slim && (!g.idx32 || mode == afir_target::kSpecGeneral)) return false;
+      *made = PendingSegment{segment, sa, g.idx32, mode, row_groups, slim};
+      return true;
+      };
+      PendingSegment made;
+      bool ok = false;
+      if (!tile.tiled && shape.unroll > 1 && row_groups_all < (int64_t)8 * shape.unroll) ok = prepare(1, true, &made);
+      if (!ok && !skip && failed == AFIR_HIP_OK) ok = prepare(shape.unroll, false, &made);
+      if (failed != AFIR_HIP_OK) return failed;
+      if (ok) pending.push_back(made);
       continue;
     }
     uint32_t rc = finish(afir::launch_fused_region(a, block_dim, static_cast<hipStream_t>(stream)));
@@ -771,7 +793,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
     bool together = pending.size() > 1 && nseg <= afir_target::kSpecMaxSegments;
     int64_t total = 0;
     for (const PendingSegment &p : pending) {
-      together = together && p.idx32 == pending[0].idx32 && p.aligned == pending[0].aligned && !p.rows;
+      together = together && p.idx32 == pending[0].idx32 && p.mode == pending[0].mode && !p.rows && !p.slim;
       total += p.args.grid;
     }
     if (together && total <= 0x7fffffff) {
@@ -788,14 +810,15 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
         }
       }
       for (int k = nseg; k <= afir_target::kSpecMaxSegments; ++k) all.first[k] = next;
-      const uint32_t rc = launch(afir_target::specAllKernelName(pending[0].idx32, pending[0].aligned), &all,
+      const uint32_t rc = launch(afir_target::specAllKernelName(pending[0].idx32, pending[0].mode), &all,
                                  offsetof(afir_target::SpecAll, seg) + (size_t)nseg * sizeof(afir_target::SpecArgs),
                                  (unsigned)next);
       if (rc != AFIR_HIP_OK) return rc;
     } else {
       for (PendingSegment &p : pending) {
         const uint32_t rc = launch(p.rows ? afir_target::specRowsKernelName(p.segment, p.idx32)
-                                          : afir_target::specKernelName(p.segment, p.idx32, p.aligned),
+                                   : p.slim ? afir_target::specSlimKernelName(p.segment, p.mode)
+                                            : afir_target::specKernelName(p.segment, p.idx32, p.mode),
                                    &p.args, sizeof p.args, (unsigned)p.args.grid);
         if (rc != AFIR_HIP_OK) return rc;
       }

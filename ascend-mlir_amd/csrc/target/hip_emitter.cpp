@@ -304,6 +304,16 @@ class SegmentEmitter {
     } else {
       emitBody();
       if (reduce_) emitBodyRowGroup();
+      if (U_ > 1) {
+        // the same with one group per lane, for short rows
+        const int wide = U_;
+        U_ = 1;
+        slim_ = true;
+        emitBody();
+        slim_ = false;
+        U_ = wide;
+        hasSlim_ = true;
+      }
     }
     emitWrappers();
     return "";
@@ -477,8 +487,11 @@ class SegmentEmitter {
     if (o.step == Operand::Contiguous) {
       unroll();
       line(d, "for (int u = 0; u < U; ++u) {");
-      line(d + 1, "if (A || (full[u] && vec" + u + ")) {");
+      line(d + 1, "if (A || (full[u] && (V || vec" + u + "))) {");
       line(d + 2, "ldv_" + tag + "<W, " + nt + ">(" + r + ".base, q" + u + " + j0[u], v" + u + "[u]);");
+      line(d + 1, "} else if (V) {");
+      unroll();
+      line(d + 2, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = " + zero() + ";");
       line(d + 1, "} else {");
       unroll();
       line(d + 2, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = e < nvalid[u] ? " + ld(o.type) + "(" + r + ".base, q" + u +
@@ -492,7 +505,7 @@ class SegmentEmitter {
       line(d + 1, "const long long step = " + r + ".stride[" + std::to_string(last_) + "];");
       unroll();
       line(d + 1, "for (int u = 0; u < U; ++u) {");
-      line(d + 2, "if (step == 1 && (A || (full[u] && vec" + u + "))) {");
+      line(d + 2, "if (step == 1 && (A || (full[u] && (V || vec" + u + ")))) {");
       line(d + 3, "ldv_" + tag + "<W, " + nt + ">(" + r + ".base, q" + u + " + j0[u], v" + u + "[u]);");
       line(d + 2, "} else {");
       unroll();
@@ -657,7 +670,7 @@ class SegmentEmitter {
     line(d, "for (int u = 0; u < U; ++u) {");
     line(d + 1, "j0[u] = " + (base.empty() ? std::string() : base + " + ") + "(" + first + " + (I)u * " + lanes + ") * W;");
     line(d + 1, "const I left = n - j0[u];");
-    line(d + 1, "nvalid[u] = (A || left >= W) ? W : (left > 0 ? (int)left : 0);");
+    line(d + 1, "nvalid[u] = (A || left >= W) ? W : (V ? 0 : (left > 0 ? (int)left : 0));");
     line(d + 1, "full[u] = A || nvalid[u] == W;");
     line(d, "}");
   }
@@ -665,12 +678,15 @@ class SegmentEmitter {
   void emitBody() {
     const std::string otag = typeTag(p_.output().type);
     os_ << "\n// ---- segment " << index_ << ": iteration rank " << rank_
-        << (reduce_ ? ", row sum over the innermost dim" : ", parallel") << "; a lane takes " << U_ << " groups of " << W_
-        << " elements per pass ----\n";
-    os_ << "// I: position type.  A: every 128-bit access is aligned and every pass is whole (no tail).\n";
-    os_ << "template <typename I, bool A>\nDEV void segment" << index_
+        << (reduce_ ? ", row sum over the innermost dim" : ", parallel") << "; a lane takes " << U_
+        << (U_ == 1 ? " group of " : " groups of ") << W_ << " elements per pass"
+        << (slim_ ? " (for rows of few groups)" : "") << " ----\n";
+    os_ << "// I: position type.  M: 2 = every 128-bit access is aligned and every pass is whole (no tail);\n";
+    os_ << "// 1 = aligned and the innermost extent a multiple of W, passes may be partly empty; 0 = anything.\n";
+    os_ << "template <typename I, int M>\nDEV void segment" << index_ << (slim_ ? "_slim" : "")
         << "(const SpecArgs &R, const I bid, const I nblocks) {\n";
     line(1, "constexpr int W = " + std::to_string(W_) + ", U = " + std::to_string(U_) + ";");
+    line(1, "constexpr bool A = M == 2, V = M >= 1;");
     line(1, "const int tid = (int)__builtin_amdgcn_workitem_id_x();");
     line(1, "const I n = (I)R.size[" + std::to_string(last_) + "];");
     line(1, "const I groups = (n + (W - 1)) / W;");
@@ -749,9 +765,9 @@ class SegmentEmitter {
     unroll();
     line(3, "for (int u = 0; u < U; ++u) {");
     line(4, "const long long o = (long long)row * (long long)n + (long long)j0[u];");
-    line(4, "if (A || (full[u] && R.out_vec)) {");
+    line(4, "if (A || (full[u] && (V || R.out_vec))) {");
     line(5, "stv_" + otag + "<W>(R.out, o, " + res + "[u]);");
-    line(4, "} else {");
+    line(4, "} else if (!V) {");
     unroll();
     line(5, "for (int e = 0; e < W; ++e)");
     line(6, "if (e < nvalid[u]) st_" + otag + "(R.out, o + e, " + res + "[u][e]);");
@@ -777,7 +793,7 @@ class SegmentEmitter {
     os_ << "template <typename I>\nDEV void segment" << index_
         << "_rows(const SpecArgs &R, const I bid, const I nblocks) {\n";
     line(1, "constexpr int W = " + std::to_string(W_) + ", U = " + std::to_string(U_) + ";");
-    line(1, "constexpr bool A = true;");
+    line(1, "constexpr bool A = true, V = true;");
     line(1, "__attribute__((shared)) static float part[2][4];");
     line(1, "const int tid = (int)__builtin_amdgcn_workitem_id_x();");
     line(1, "const int lane = tid & 63, wave = tid >> 6;");
@@ -850,9 +866,10 @@ class SegmentEmitter {
         << " (dim " << p << ") x " << kTileQ << " (dim " << last_ << ") through LDS; a lane takes " << U_
         << " groups of " << W_ << " elements per row ----\n";
     os_ << "// I: position type.  A: every 128-bit access is aligned and every tile is whole.\n";
-    os_ << "template <typename I, bool A>\nDEV void segment" << index_
+    os_ << "template <typename I, int M>\nDEV void segment" << index_
         << "(const SpecArgs &R, const I bid, const I nblocks) {\n";
     line(1, "constexpr int W = " + std::to_string(W_) + ", U = " + std::to_string(U_) + ";");
+    line(1, "constexpr bool A = M == 2, V = false;   // tiles are whole and aligned, or anything goes");
     line(1, "constexpr int TP = " + std::to_string(kTileP) + ", TQ = " + std::to_string(kTileQ) + ", PITCH = TP + 1;");
     line(1, "static_assert(8 * U * W == TQ, \"eight lanes cover a tile row\");");
     line(1, "__attribute__((shared)) static " + ct() + " tile[" + std::to_string(numTiles_) + "][TQ * PITCH];");
@@ -940,11 +957,17 @@ class SegmentEmitter {
 
   void emitWrappers() {
     for (int i32 = 1; i32 >= 0; --i32)
-      for (int a = 1; a >= 0; --a)
-        os_ << "KERNEL void " << specKernelName(index_, i32 != 0, a != 0) << "(const SpecArgs R) { segment" << index_
-            << "<" << (i32 ? "int" : "long long") << ", " << (a ? "true" : "false")
+      for (int mode = kSpecAligned; mode >= kSpecGeneral; --mode) {
+        if (mode == kSpecVector && tiled()) continue;   // tiles are whole and aligned, or general
+        os_ << "KERNEL void " << specKernelName(index_, i32 != 0, mode) << "(const SpecArgs R) { segment" << index_
+            << "<" << (i32 ? "int" : "long long") << ", " << mode
             << ">(R, (" << (i32 ? "int" : "long long") << ")__builtin_amdgcn_workgroup_id_x(), ("
             << (i32 ? "int" : "long long") << ")R.grid); }\n";
+      }
+    if (hasSlim_)
+      for (int mode = kSpecAligned; mode >= kSpecVector; --mode)
+        os_ << "KERNEL void " << specSlimKernelName(index_, mode) << "(const SpecArgs R) { segment" << index_
+            << "_slim<int, " << mode << ">(R, (int)__builtin_amdgcn_workgroup_id_x(), (int)R.grid); }\n";
     if (reduce_)
       for (int i32 = 1; i32 >= 0; --i32)
         os_ << "KERNEL void " << specRowsKernelName(index_, i32 != 0) << "(const SpecArgs R) { segment" << index_
@@ -963,6 +986,8 @@ class SegmentEmitter {
   bool reduce_ = false;
   bool integer_ = false;   // 32-bit integers instead of float32 values
   bool narrow_ = false;    // ... of which the low 16 bits are the value (i16 output)
+  bool slim_ = false;      // emitting the one-group-per-lane form of the segment
+  bool hasSlim_ = false;   // ... which exists for this segment
   bool hoisted_ = false;   // row invariants and operand values are assigned, not declared
   bool keepRowConstants_ = false;   // ... and operands that are the same for every row are left alone
 
@@ -1045,16 +1070,24 @@ uint64_t programHash(const Program &p) {
   return h;
 }
 
-std::string specAllKernelName(bool idx32, bool aligned) {
-  return std::string("afir_region_all") + (idx32 ? "_i32" : "_i64") + (aligned ? "_a" : "_g");
+namespace {
+const char *modeSuffix(int mode) { return mode == kSpecAligned ? "_a" : mode == kSpecVector ? "_v" : "_g"; }
+}  // namespace
+
+std::string specAllKernelName(bool idx32, int mode) {
+  return std::string("afir_region_all") + (idx32 ? "_i32" : "_i64") + modeSuffix(mode);
 }
 
 std::string specRowsKernelName(int segment, bool idx32) {
   return "afir_region_s" + std::to_string(segment) + "_rows" + (idx32 ? "_i32" : "_i64");
 }
 
-std::string specKernelName(int segment, bool idx32, bool aligned) {
-  return "afir_region_s" + std::to_string(segment) + (idx32 ? "_i32" : "_i64") + (aligned ? "_a" : "_g");
+std::string specSlimKernelName(int segment, int mode) {
+  return "afir_region_s" + std::to_string(segment) + "_slim_i32" + modeSuffix(mode);
+}
+
+std::string specKernelName(int segment, bool idx32, int mode) {
+  return "afir_region_s" + std::to_string(segment) + (idx32 ? "_i32" : "_i64") + modeSuffix(mode);
 }
 
 std::string emitHipSource(const Program &p, const std::string &title, std::string *source,
@@ -1092,14 +1125,14 @@ std::string emitHipSource(const Program &p, const std::string &title, std::strin
     os << "static_assert(__builtin_offsetof(SpecAll, seg) == " << offsetof(SpecAll, seg)
        << ", \"launch argument layout differs from the kernel library's\");\n";
     for (int i32 = 1; i32 >= 0; --i32)
-      for (int a = 1; a >= 0; --a) {
+      for (int mode = kSpecAligned; mode >= kSpecGeneral; --mode) {
         const char *I = i32 ? "int" : "long long";
-        os << "KERNEL void " << specAllKernelName(i32 != 0, a != 0) << "(const SpecAll M) {\n";
+        os << "KERNEL void " << specAllKernelName(i32 != 0, mode) << "(const SpecAll S) {\n";
         os << "  const int b = (int)__builtin_amdgcn_workgroup_id_x();\n";
         for (int k = 0; k < nseg; ++k)
-          os << "  " << (k ? "else " : "") << (k + 1 < nseg ? "if (b < M.first[" + std::to_string(k + 1) + "]) " : "")
-             << "segment" << k << "<" << I << ", " << (a ? "true" : "false") << ">(M.seg[" << k << "], (" << I
-             << ")(b - M.first[" << k << "]), (" << I << ")(M.first[" << k + 1 << "] - M.first[" << k << "]));\n";
+          os << "  " << (k ? "else " : "") << (k + 1 < nseg ? "if (b < S.first[" + std::to_string(k + 1) + "]) " : "")
+             << "segment" << k << "<" << I << ", " << mode << ">(S.seg[" << k << "], (" << I
+             << ")(b - S.first[" << k << "]), (" << I << ")(S.first[" << k + 1 << "] - S.first[" << k << "]));\n";
         os << "}\n";
       }
   }

@@ -59,7 +59,7 @@ struct SpecAll {
   int pad;
   SpecArgs seg[kSpecMaxSegments];    // the emitted declaration holds the program's segment count
 };
-std::string specAllKernelName(bool idx32, bool aligned);
+std::string specAllKernelName(bool idx32, int mode);
 bool specAllSegments(const afir_region::Program &p);   // whether that kernel is emitted
 
 // A parallel segment that reads an operand transposed (contiguous along an
@@ -100,9 +100,17 @@ SpecShape specShape(const afir_region::Program &p, int segment, const EmitOption
 // `afir_region_program_hash`, checked when the code object is attached.
 uint64_t programHash(const afir_region::Program &p);
 
-// Kernel symbol of a segment: idx32 = positions fit 32 bits, aligned = every
-// vector access of the launch is 16-byte aligned and rows are whole vectors.
-std::string specKernelName(int segment, bool idx32, bool aligned);
+// What a launch promises, which picks the kernel variant:
+//   kSpecAligned  every 128-bit access is aligned and every pass of the lanes over a row is whole
+//   kSpecVector   every 128-bit access is aligned and the innermost extent is a multiple of the
+//                 lane width; the last pass may be partly empty (not emitted for tiled segments)
+//   kSpecGeneral  anything: tails and unaligned tensors take element accesses
+enum SpecMode { kSpecGeneral = 0, kSpecVector = 1, kSpecAligned = 2 };
+// Kernel symbol of a segment: idx32 = positions fit 32 bits.
+std::string specKernelName(int segment, bool idx32, int mode);
+// Untiled segments also have kernels whose lanes take one group each, for rows of
+// fewer than 8 x unroll groups (32-bit positions, modes kSpecAligned and kSpecVector).
+std::string specSlimKernelName(int segment, int mode);
 // Reduce segments also have a workgroup-per-row kernel for rows of exactly
 // 256 * unroll * width elements whose accesses are all 128-bit.
 std::string specRowsKernelName(int segment, bool idx32);

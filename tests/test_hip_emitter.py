@@ -104,16 +104,28 @@ def test_reductions_also_get_a_workgroup_per_row_kernel():
     assert "rows of exactly 4096 elements: a workgroup per row, the next row in flight" in src
     assert "afir_region_s0_rows_i32(" in src and "afir_region_s0_rows_i64(" in src
     rows = src[src.index("DEV void segment0_rows"):]
-    rows = rows[:rows.index("KERNEL")]
+    rows = rows[:rows.index("\n}\n")]
     # the bias does not change with the row: loaded once, before the loop, not in the fetch of the next row
     assert rows.count("ldv_f32<W, false>(R.in[1].base") == 1 and rows.count("ldv_f32<W, true>(R.in[0].base") == 2
     assert rows.count("__builtin_amdgcn_s_barrier();") == 1
     assert "_rows_" not in _emit(RC.C1_ADD_MUL).stdout            # parallel segments have none
 
 
+def test_short_rows_get_one_group_per_lane_kernels():
+    src = _emit(RC.RELU_COL_ADD).stdout
+    assert "a lane takes 1 group of 8 elements per pass (for rows of few groups)" in src
+    assert "afir_region_s0_slim_i32_a(" in src and "afir_region_s0_slim_i32_v(" in src
+    assert "afir_region_s0_slim_i32_g(" not in src and "slim_i64" not in src
+    assert "_slim" not in _emit(RC.C3_RELU_BCAST_TRANSPOSE).stdout       # tiled segments have none
+    # and the three modes of the ordinary kernels
+    for mode in "avg":
+        assert f"afir_region_s0_i32_{mode}(" in src and f"afir_region_s0_i64_{mode}(" in src
+
+
 def test_identical_reads_are_loaded_once():
     src = _emit(RC.C1_ADD_MUL).stdout           # (a + b) * b reads b twice
-    assert src.count("ldv_f32<W, true>(R.in[1].base") == 1 and "R.in[2]" not in src
+    # once in the ordinary form of the segment, once in its one-group-per-lane form
+    assert src.count("ldv_f32<W, true>(R.in[1].base") == 2 and "R.in[2]" not in src
 
 
 def test_matmul_programs_have_no_source_form():
