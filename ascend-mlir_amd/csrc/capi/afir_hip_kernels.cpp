@@ -607,7 +607,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
     afir_target::SpecArgs args;
     bool idx32;
     int mode;    // afir_target::SpecMode
-    bool rows;   // the workgroup-per-row kernel of a reduce segment
+    int rows;    // 1: the workgroup-per-row kernel of a reduce segment, 2: its form for few, long rows
     bool slim;   // the kernel whose lanes take one group each (short rows)
   };
   std::vector<PendingSegment> pending;   // compiled kernels to launch, non-empty segments only
@@ -686,7 +686,8 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
       sa.grid = (int)g.blocks;
       sa.column_blocks = (int)g.column_blocks;
       // vectors: every 128-bit access is aligned and rows are whole vectors; whole: no pass has a tail
-      bool vectors, whole, row_groups = false;
+      bool vectors, whole;
+      int row_groups = 0;
       if (tile.tiled) {
         // one workgroup pass per tile of tile_p x tile_q
         const int64_t tq = (seg.size[last] + emit.tileQ - 1) / emit.tileQ;
@@ -722,7 +723,13 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
         vectors = seg.size[last] % W == 0 && (seg.reduce || a.out_vec);
         whole = groups % per_pass == 0;
         // a row that fills a workgroup of 256 lanes with U groups each: a workgroup per row
-        row_groups = !slim && seg.reduce && groups == (int64_t)256 * U;
+        if (!slim && seg.reduce && groups == (int64_t)256 * U) row_groups = 1;
+        // few rows of several such stretches: a workgroup per row as well, pass by pass
+        int64_t nrows_all = 1;
+        for (int k = 0; k < last; ++k) nrows_all *= seg.size[k];
+        if (!slim && seg.reduce && groups >= (int64_t)512 * U && groups % ((int64_t)256 * U) == 0 &&
+            nrows_all < (int64_t)afir::kNumCU * 16)
+          row_groups = 2;
       }
       for (int i = 0; i < a.ninputs; ++i) {
         const afir::RegionInput &d = a.in[i];
@@ -760,7 +767,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
         sa.grid = (int)blocks;
         sa.column_blocks = 1;
       } else {
-        row_groups = false;
+        row_groups = 0;
       }
       if (slim && (!g.idx32 || mode == afir_target::kSpecGeneral)) return false;
       *made = PendingSegment{segment, sa, g.idx32, mode, row_groups, slim};
@@ -816,7 +823,8 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
       if (rc != AFIR_HIP_OK) return rc;
     } else {
       for (PendingSegment &p : pending) {
-        const uint32_t rc = launch(p.rows ? afir_target::specRowsKernelName(p.segment, p.idx32)
+        const uint32_t rc = launch(p.rows == 2 ? afir_target::specLongRowsKernelName(p.segment, p.idx32)
+                                   : p.rows ? afir_target::specRowsKernelName(p.segment, p.idx32)
                                    : p.slim ? afir_target::specSlimKernelName(p.segment, p.mode)
                                             : afir_target::specKernelName(p.segment, p.idx32, p.mode),
                                    &p.args, sizeof p.args, (unsigned)p.args.grid);

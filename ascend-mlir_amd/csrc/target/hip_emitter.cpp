@@ -303,7 +303,10 @@ class SegmentEmitter {
       emitBodyTiled();
     } else {
       emitBody();
-      if (reduce_) emitBodyRowGroup();
+      if (reduce_) {
+        emitBodyRowGroup();
+        emitBodyLongRows();
+      }
       if (U_ > 1) {
         // the same with one group per lane, for short rows
         const int wide = U_;
@@ -851,6 +854,95 @@ class SegmentEmitter {
     hoisted_ = false;
   }
 
+  // Row sums of a few long rows (a whole number of passes of 256 * U groups): a
+  // workgroup per row again, walking the row pass by pass with the next pass
+  // (of this row or of the workgroup's next row) in flight; the lane's partial
+  // sums run over the passes and meet as above when the row ends.  A wavefront
+  // per row would leave most of the chip idle when there are few rows.
+  void emitBodyLongRows() {
+    const std::string otag = typeTag(p_.output().type);
+    os_ << "\n// ---- segment " << index_ << ", few rows of a multiple of " << 256 * U_ * W_
+        << " elements: a workgroup per row, the next pass in flight ----\n";
+    os_ << "template <typename I>\nDEV void segment" << index_
+        << "_long(const SpecArgs &R, const I bid, const I nblocks) {\n";
+    line(1, "constexpr int W = " + std::to_string(W_) + ", U = " + std::to_string(U_) + ";");
+    line(1, "constexpr bool A = true, V = true;");
+    line(1, "__attribute__((shared)) static float part[2][4];");
+    line(1, "const int tid = (int)__builtin_amdgcn_workitem_id_x();");
+    line(1, "const int lane = tid & 63, wave = tid >> 6;");
+    line(1, "const I n = (I)R.size[" + std::to_string(last_) + "];");
+    line(1, "const I passes = n / (I)(256 * U * W);");
+    if (rank_ == 2) line(1, "const I rows = (I)R.size[0];");
+    else line(1, "const I rows = (I)(R.size[0] * R.size[1]);");
+    for (const Operand &o : operands_)
+      if (o.step != Operand::Broadcast && o.gatherDim != last_)
+        line(1, "const bool vec" + id(o) + " = " + in(o) + ".vec != 0" + (o.gatherDim >= 0 ? " && " + in(o) + ".gvec != 0" : "") + ";");
+    line(1, "I j0[U];");
+    line(1, "int nvalid[U];");
+    line(1, "bool full[U];");
+    unroll();
+    line(1, "for (int u = 0; u < U; ++u) {");
+    line(2, "j0[u] = ((I)tid + (I)u * (I)256) * W;");
+    line(2, "nvalid[u] = W;");
+    line(2, "full[u] = true;");
+    line(1, "}");
+    hoisted_ = true;
+    emitOperandDeclarations(1);
+    line(1, "I row = bid, pass = 0;");
+    line(1, "if (row < rows) {");
+    emitPositionOfRow(2);
+    emitRowInvariants(2);
+    const std::vector<Value> read = emitReads(2);
+    line(1, "}");
+    line(1, "int parity = 0;");
+    line(1, "float acc[W];");
+    unroll();
+    line(1, "for (int e = 0; e < W; ++e) acc[e] = 0.f;");
+    line(1, "while (row < rows) {");
+    const Value v = emitCompute(2, read);
+    unroll();
+    line(2, "for (int e = 0; e < W; ++e) {");
+    line(3, "float t[U];");
+    unroll();
+    line(3, "for (int u = 0; u < U; ++u) t[u] = " + v.at() + ";");
+    unroll();
+    line(3, "for (int w = U / 2; w >= 1; w >>= 1)");
+    unroll();
+    line(4, "for (int u = 0; u < w; ++u) t[u] = t[2 * u] + t[2 * u + 1];");
+    line(3, "acc[e] += t[0];");
+    line(2, "}");
+    line(2, "const bool row_ends = pass + 1 == passes;");
+    line(2, "const I next_row = row_ends ? row + nblocks : row;");
+    line(2, "const I next_pass = row_ends ? (I)0 : pass + 1;");
+    line(2, "if (next_row < rows) {");
+    unroll();
+    line(3, "for (int u = 0; u < U; ++u) j0[u] = ((I)tid + (I)u * (I)256 + next_pass * (I)(256 * U)) * W;");
+    emitPositionOfRow(3, "next_row");
+    emitRowInvariants(3);
+    emitReads(3);
+    line(2, "}");
+    line(2, "if (row_ends) {");
+    unroll();
+    line(3, "for (int w = W / 2; w >= 1; w >>= 1)");
+    unroll();
+    line(4, "for (int e = 0; e < w; ++e) acc[e] = acc[2 * e] + acc[2 * e + 1];");
+    line(3, "const float s = wave_sum(acc[0]);");
+    line(3, "if (lane == 0) part[parity][wave] = s;");
+    line(3, "__builtin_amdgcn_fence(__ATOMIC_RELEASE, \"workgroup\");");
+    line(3, "__builtin_amdgcn_s_barrier();");
+    line(3, "__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, \"workgroup\");");
+    line(3, "if (tid == 0) st_" + otag + "(R.out, (long long)row, (part[parity][0] + part[parity][1]) + (part[parity][2] + part[parity][3]));");
+    line(3, "parity ^= 1;");
+    unroll();
+    line(3, "for (int e = 0; e < W; ++e) acc[e] = 0.f;");
+    line(2, "}");
+    line(2, "row = next_row;");
+    line(2, "pass = next_pass;");
+    line(1, "}");
+    os_ << "}\n";
+    hoisted_ = false;
+  }
+
   // Parallel segment with transposed reads: a workgroup takes a tile of kTileP
   // (the dim those operands are contiguous along) x kTileQ (the innermost
   // iteration dim).  Phase 1 loads each transposed operand's tile with 128-bit
@@ -974,6 +1066,12 @@ class SegmentEmitter {
             << "_rows<" << (i32 ? "int" : "long long")
             << ">(R, (" << (i32 ? "int" : "long long") << ")__builtin_amdgcn_workgroup_id_x(), ("
             << (i32 ? "int" : "long long") << ")R.grid); }\n";
+    if (reduce_)
+      for (int i32 = 1; i32 >= 0; --i32)
+        os_ << "KERNEL void " << specLongRowsKernelName(index_, i32 != 0) << "(const SpecArgs R) { segment" << index_
+            << "_long<" << (i32 ? "int" : "long long")
+            << ">(R, (" << (i32 ? "int" : "long long") << ")__builtin_amdgcn_workgroup_id_x(), ("
+            << (i32 ? "int" : "long long") << ")R.grid); }\n";
   }
 
   const Program &p_;
@@ -1080,6 +1178,10 @@ std::string specAllKernelName(bool idx32, int mode) {
 
 std::string specRowsKernelName(int segment, bool idx32) {
   return "afir_region_s" + std::to_string(segment) + "_rows" + (idx32 ? "_i32" : "_i64");
+}
+
+std::string specLongRowsKernelName(int segment, bool idx32) {
+  return "afir_region_s" + std::to_string(segment) + "_long" + (idx32 ? "_i32" : "_i64");
 }
 
 std::string specSlimKernelName(int segment, int mode) {

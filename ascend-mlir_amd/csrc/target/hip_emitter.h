@@ -114,6 +114,9 @@ std::string specSlimKernelName(int segment, int mode);
 // Reduce segments also have a workgroup-per-row kernel for rows of exactly
 // 256 * unroll * width elements whose accesses are all 128-bit.
 std::string specRowsKernelName(int segment, bool idx32);
+// ... and one for rows of a whole number (two or more) of such stretches, launched when the
+// rows are too few to fill the chip with a wavefront each.
+std::string specLongRowsKernelName(int segment, bool idx32);
 
 // Emits the source for every segment.  Returns "" on success, else why the
 // program has no specialised form (matmul segments: those run on the

@@ -132,6 +132,28 @@ def test_row_sums_of_short_rows(H, n):
             assert run(H, text, [x, bias], (rows,)).tobytes() == want.tobytes(), (ty, rows, n)
 
 
+@pytest.mark.parametrize("ty,n", [("f32", 8192), ("f32", 3 * 4096), ("f16", 16384), ("f16", 5 * 8192)])
+def test_row_sums_of_few_long_rows(H, ty, n):
+    """A few rows of several workgroup passes each take the compiled long-row kernel: a
+    workgroup per row, pass by pass; with two workgroups for seven rows each workgroup also
+    moves on to further rows."""
+    dt = np.float32 if ty == "f32" else np.float16
+    rng = np.random.default_rng(n)
+    text = RC.C2_BCAST_ADD_ROWSUM.replace("f32", ty)
+    for rows, block_dim in ((1, 0), (7, 0), (7, 2)):
+        x = rng.integers(-2, 3, (rows, n)).astype(dt)
+        bias = rng.integers(-2, 3, (n,)).astype(dt)
+        want = RO.evaluate(text, [x, bias])
+        assert np.isfinite(want.astype(np.float32)).all()
+        assert run(H, text, [x, bias], (rows,), block_dim=block_dim).tobytes() == want.tobytes(), (rows, block_dim)
+    r = rng.integers(-1, 2, (6,)).astype(dt)                    # an operand that changes with the row
+    x = rng.integers(-3, 4, (6, n)).astype(dt)
+    text = RC.REDUCE_ROWBIAS.replace("f16", ty)
+    want = RO.evaluate(text, [r, x])
+    assert np.isfinite(want.astype(np.float32)).all()
+    assert run(H, text, [r, x], (6,), block_dim=4).tobytes() == want.tobytes()
+
+
 def test_row_sums_with_a_row_operand_and_rank_3(H):
     """The workgroup-per-row kernels with an operand that changes with the row (fetched
     ahead with the matrix) and over a rank-3 space whose row is (d0, d1)."""
