@@ -118,6 +118,13 @@ std::string compiled_function(CompiledRegion *c, const afir_region::Program &pro
       (void)hipModuleUnload(m);
       return "code object was not built from this program";
     }
+    int abi = -1;
+    if (hipModuleGetGlobal(&sym, &bytes, m, "afir_region_emit_abi") != hipSuccess || bytes != sizeof abi ||
+        hipMemcpyDtoH(&abi, sym, sizeof abi) != hipSuccess || abi != afir_target::kSpecAbiVersion) {
+      (void)hipModuleUnload(m);
+      return "code object was emitted by another version of this library (its kernels and their arguments differ); "
+             "compile the artifact again";
+    }
     // the tile / unroll choices the kernels were emitted with (older objects: the defaults)
     int opts[3] = {0, 0, 0};
     if (hipModuleGetGlobal(&sym, &bytes, m, "afir_region_emit_options") == hipSuccess && bytes == sizeof opts &&
@@ -672,106 +679,106 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
       bool skip = false;
       uint32_t failed = AFIR_HIP_OK;
       auto prepare = [&](const int U, const bool slim, PendingSegment *made) -> bool {
-      afir::RegionGeometry g;
-      uint32_t rc = finish(afir::plan_fused_region(a, W * U, block_dim, &g));
-      if (rc != AFIR_HIP_OK) { failed = rc; return false; }
-      if (g.empty) { skip = true; return false; }
-      afir_target::SpecArgs sa;
-      std::memset(&sa, 0, sizeof sa);
-      for (int k = 0; k < 3; ++k) sa.size[k] = a.size[k];
-      sa.out = a.out;
-      sa.error_flag = a.error_flag;
-      sa.out_vec = a.out_vec;
-      sa.lanes_log2 = g.lanes_log2;
-      sa.grid = (int)g.blocks;
-      sa.column_blocks = (int)g.column_blocks;
-      // vectors: every 128-bit access is aligned and rows are whole vectors; whole: no pass has a tail
-      bool vectors, whole;
-      int row_groups = 0;
-      if (tile.tiled) {
-        // one workgroup pass per tile of tile_p x tile_q
-        const int64_t tq = (seg.size[last] + emit.tileQ - 1) / emit.tileQ;
-        const int64_t tp = (seg.size[tile.dim] + emit.tileP - 1) / emit.tileP;
-        int64_t tiles = tq * tp;
-        for (int k = 0; k < last; ++k)
-          if (k != tile.dim) tiles *= seg.size[k];
-        int64_t blocks = tiles < (int64_t)afir::kNumCU * 256 ? tiles : (int64_t)afir::kNumCU * 256;
-        if (block_dim) blocks = block_dim;
-        sa.grid = (int)blocks;
-        sa.column_blocks = 1;
-        vectors = a.out_vec != 0;
-        whole = seg.size[last] % emit.tileQ == 0 && seg.size[tile.dim] % emit.tileP == 0;
-      } else {
-        // the aligned variant has no tail handling: whole groups, whole passes
-        const int64_t groups = seg.size[last] / W;
-        if (seg.reduce) {
-          // lanes of a wavefront that share a row: enough for one pass over a short row, the wavefront otherwise
-          const int64_t all_groups = (seg.size[last] + W - 1) / W;
-          int ll = 0;
-          while (ll < 6 && ((int64_t)U << ll) < all_groups) ++ll;
-          sa.lanes_log2 = ll;
-          if (!block_dim) {
-            int64_t nrows = 1;
-            for (int k = 0; k < last; ++k) nrows *= seg.size[k];
-            const int64_t rows_per_block = (int64_t)4 * (64 >> ll);
-            int64_t blocks = (nrows + rows_per_block - 1) / rows_per_block;
-            if (blocks > (int64_t)afir::kNumCU * 16) blocks = (int64_t)afir::kNumCU * 16;
-            sa.grid = (int)blocks;
+        afir::RegionGeometry g;
+        uint32_t rc = finish(afir::plan_fused_region(a, W * U, block_dim, &g));
+        if (rc != AFIR_HIP_OK) { failed = rc; return false; }
+        if (g.empty) { skip = true; return false; }
+        afir_target::SpecArgs sa;
+        std::memset(&sa, 0, sizeof sa);
+        for (int k = 0; k < 3; ++k) sa.size[k] = a.size[k];
+        sa.out = a.out;
+        sa.error_flag = a.error_flag;
+        sa.out_vec = a.out_vec;
+        sa.lanes_log2 = g.lanes_log2;
+        sa.grid = (int)g.blocks;
+        sa.column_blocks = (int)g.column_blocks;
+        // vectors: every 128-bit access is aligned and rows are whole vectors; whole: no pass has a tail
+        bool vectors, whole;
+        int row_groups = 0;
+        if (tile.tiled) {
+          // one workgroup pass per tile of tile_p x tile_q
+          const int64_t tq = (seg.size[last] + emit.tileQ - 1) / emit.tileQ;
+          const int64_t tp = (seg.size[tile.dim] + emit.tileP - 1) / emit.tileP;
+          int64_t tiles = tq * tp;
+          for (int k = 0; k < last; ++k)
+            if (k != tile.dim) tiles *= seg.size[k];
+          int64_t blocks = tiles < (int64_t)afir::kNumCU * 256 ? tiles : (int64_t)afir::kNumCU * 256;
+          if (block_dim) blocks = block_dim;
+          sa.grid = (int)blocks;
+          sa.column_blocks = 1;
+          vectors = a.out_vec != 0;
+          whole = seg.size[last] % emit.tileQ == 0 && seg.size[tile.dim] % emit.tileP == 0;
+        } else {
+          // the aligned variant has no tail handling: whole groups, whole passes
+          const int64_t groups = seg.size[last] / W;
+          if (seg.reduce) {
+            // lanes of a wavefront that share a row: enough for one pass over a short row, the wavefront otherwise
+            const int64_t all_groups = (seg.size[last] + W - 1) / W;
+            int ll = 0;
+            while (ll < 6 && ((int64_t)U << ll) < all_groups) ++ll;
+            sa.lanes_log2 = ll;
+            if (!block_dim) {
+              int64_t nrows = 1;
+              for (int k = 0; k < last; ++k) nrows *= seg.size[k];
+              const int64_t rows_per_block = (int64_t)4 * (64 >> ll);
+              int64_t blocks = (nrows + rows_per_block - 1) / rows_per_block;
+              if (blocks > (int64_t)afir::kNumCU * 16) blocks = (int64_t)afir::kNumCU * 16;
+              sa.grid = (int)blocks;
+            }
           }
+          const int64_t per_pass = ((int64_t)1 << sa.lanes_log2) * U;
+          vectors = seg.size[last] % W == 0 && (seg.reduce || a.out_vec);
+          whole = groups % per_pass == 0;
+          // a row that fills a workgroup of 256 lanes with U groups each: a workgroup per row
+          if (!slim && seg.reduce && groups == (int64_t)256 * U) row_groups = 1;
+          // few rows of several such stretches: a workgroup per row as well, pass by pass
+          int64_t nrows_all = 1;
+          for (int k = 0; k < last; ++k) nrows_all *= seg.size[k];
+          if (!slim && seg.reduce && groups >= (int64_t)512 * U && groups % ((int64_t)256 * U) == 0 &&
+              nrows_all < (int64_t)afir::kNumCU * 16)
+            row_groups = 2;
         }
-        const int64_t per_pass = ((int64_t)1 << sa.lanes_log2) * U;
-        vectors = seg.size[last] % W == 0 && (seg.reduce || a.out_vec);
-        whole = groups % per_pass == 0;
-        // a row that fills a workgroup of 256 lanes with U groups each: a workgroup per row
-        if (!slim && seg.reduce && groups == (int64_t)256 * U) row_groups = 1;
-        // few rows of several such stretches: a workgroup per row as well, pass by pass
-        int64_t nrows_all = 1;
-        for (int k = 0; k < last; ++k) nrows_all *= seg.size[k];
-        if (!slim && seg.reduce && groups >= (int64_t)512 * U && groups % ((int64_t)256 * U) == 0 &&
-            nrows_all < (int64_t)afir::kNumCU * 16)
-          row_groups = 2;
-      }
-      for (int i = 0; i < a.ninputs; ++i) {
-        const afir::RegionInput &d = a.in[i];
-        afir_target::SpecInput &t = sa.in[i];
-        t.base = d.base;
-        t.index = d.index;
-        for (int k = 0; k < 3; ++k) t.stride[k] = d.stride[k];
-        t.offset = d.offset;
-        t.gstride = d.gstride;
-        t.gextent = d.gextent;
-        t.vec = d.vec;
-        t.gvec = d.gvec;
-        if (tile.tiled && ((tile.inputs >> i) & 1u)) {
-          // staged through LDS: 128-bit loads run along the tile dim
-          const int64_t es = (int64_t)afir_region::elemTypeBytes(seg.inputs[i].type);
-          bool tvec = aligned(d.base, d.offset * es);
-          for (int k = 0; k < seg.rank; ++k)
-            if (k != tile.dim && seg.size[k] > 1 && (d.stride[k] * es) % 16 != 0) tvec = false;
-          t.vec = tvec ? 1 : 0;
-          if (!tvec) vectors = false;
-          continue;
+        for (int i = 0; i < a.ninputs; ++i) {
+          const afir::RegionInput &d = a.in[i];
+          afir_target::SpecInput &t = sa.in[i];
+          t.base = d.base;
+          t.index = d.index;
+          for (int k = 0; k < 3; ++k) t.stride[k] = d.stride[k];
+          t.offset = d.offset;
+          t.gstride = d.gstride;
+          t.gextent = d.gextent;
+          t.vec = d.vec;
+          t.gvec = d.gvec;
+          if (tile.tiled && ((tile.inputs >> i) & 1u)) {
+            // staged through LDS: 128-bit loads run along the tile dim
+            const int64_t es = (int64_t)afir_region::elemTypeBytes(seg.inputs[i].type);
+            bool tvec = aligned(d.base, d.offset * es);
+            for (int k = 0; k < seg.rank; ++k)
+              if (k != tile.dim && seg.size[k] > 1 && (d.stride[k] * es) % 16 != 0) tvec = false;
+            t.vec = tvec ? 1 : 0;
+            if (!tvec) vectors = false;
+            continue;
+          }
+          // operands that are contiguous along the innermost dim are read with
+          // 128-bit loads by the aligned variant
+          if (d.stride[last] == 1 && d.gdim != last && (!d.vec || (d.gdim >= 0 && !d.gvec))) vectors = false;
         }
-        // operands that are contiguous along the innermost dim are read with
-        // 128-bit loads by the aligned variant
-        if (d.stride[last] == 1 && d.gdim != last && (!d.vec || (d.gdim >= 0 && !d.gvec))) vectors = false;
-      }
-      const int mode = vectors && whole ? afir_target::kSpecAligned
-                       : vectors && !tile.tiled ? afir_target::kSpecVector : afir_target::kSpecGeneral;
-      if (row_groups && mode == afir_target::kSpecAligned) {
-        // up to 16 workgroups per CU walk the rows (4 to 16 measured within 1 %, 2 slower)
-        int64_t nrows = 1;
-        for (int k = 0; k < last; ++k) nrows *= seg.size[k];
-        int64_t blocks = nrows < (int64_t)afir::kNumCU * 16 ? nrows : (int64_t)afir::kNumCU * 16;
-        if (block_dim) blocks = block_dim;
-        sa.grid = (int)blocks;
-        sa.column_blocks = 1;
-      } else {
-        row_groups = 0;
-      }
-      if (slim && (!g.idx32 || mode == afir_target::kSpecGeneral)) return false;
-      *made = PendingSegment{segment, sa, g.idx32, mode, row_groups, slim};
-      return true;
+        const int mode = vectors && whole ? afir_target::kSpecAligned
+                         : vectors && !tile.tiled ? afir_target::kSpecVector : afir_target::kSpecGeneral;
+        if (row_groups && mode == afir_target::kSpecAligned) {
+          // up to 16 workgroups per CU walk the rows (4 to 16 measured within 1 %, 2 slower)
+          int64_t nrows = 1;
+          for (int k = 0; k < last; ++k) nrows *= seg.size[k];
+          int64_t blocks = nrows < (int64_t)afir::kNumCU * 16 ? nrows : (int64_t)afir::kNumCU * 16;
+          if (block_dim) blocks = block_dim;
+          sa.grid = (int)blocks;
+          sa.column_blocks = 1;
+        } else {
+          row_groups = 0;
+        }
+        if (slim && (!g.idx32 || mode == afir_target::kSpecGeneral)) return false;
+        *made = PendingSegment{segment, sa, g.idx32, mode, row_groups, slim};
+        return true;
       };
       PendingSegment made;
       bool ok = false;

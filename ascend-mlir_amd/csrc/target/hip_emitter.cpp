@@ -1212,6 +1212,7 @@ std::string emitHipSource(const Program &p, const std::string &title, std::strin
   char hash[32];
   std::snprintf(hash, sizeof hash, "0x%016llxull", (unsigned long long)programHash(p));
   os << "extern \"C\" __attribute__((device)) __attribute__((used)) const unsigned long long afir_region_program_hash = " << hash << ";\n";
+  os << "extern \"C\" __attribute__((device)) __attribute__((used)) const int afir_region_emit_abi = " << kSpecAbiVersion << ";\n";
   os << "extern \"C\" __attribute__((device)) __attribute__((used)) const int afir_region_emit_options[3] = {"
      << options.tileP << ", " << options.tileQ << ", " << options.unroll << "};   // tile_p, tile_q, unroll\n";
   for (int s = 0; s < (int)p.segments.size(); ++s) {

@@ -100,6 +100,11 @@ SpecShape specShape(const afir_region::Program &p, int segment, const EmitOption
 // `afir_region_program_hash`, checked when the code object is attached.
 uint64_t programHash(const afir_region::Program &p);
 
+// Version of the set of kernels and of the launch arguments that emitHipSource produces; the
+// code object exports it as `afir_region_emit_abi`, and a code object of another version is
+// refused when it is loaded (its kernels would be launched with the wrong names or arguments).
+constexpr int kSpecAbiVersion = 3;
+
 // What a launch promises, which picks the kernel variant:
 //   kSpecAligned  every 128-bit access is aligned and every pass of the lanes over a row is whole
 //   kSpecVector   every 128-bit access is aligned and the innermost extent is a multiple of the

@@ -410,6 +410,27 @@ def test_code_object_of_another_program_is_rejected(H, evaluator, tmp_path):
     r.close()
 
 
+def test_code_object_of_another_emitter_version_is_rejected(H, evaluator, monkeypatch, tmp_path):
+    """The code object also carries the version of the kernel set and launch arguments it
+    was emitted for; one from another version (here: the source edited) is refused when it
+    is loaded, before any of its kernels is launched."""
+    import re
+    import torch
+    if evaluator != "compiled":
+        pytest.skip("one run is enough")
+    monkeypatch.setenv("AFIR_HIP_REGION_GENERIC", "1")
+    r = H.Region(RC.C1_ADD_MUL)
+    src = r.emit_source()
+    assert re.search(r"afir_region_emit_abi = \d+;", src)
+    for edited in (re.sub(r"afir_region_emit_abi = \d+;", "afir_region_emit_abi = 1;", src),
+                   re.sub(r"afir_region_emit_abi = ", "afir_region_other = ", src)):      # another version, none
+        r.attach_code_object(H.compile_region_source(edited, str(tmp_path)))
+        a = torch.ones(4, 8, device="cuda")
+        with pytest.raises(H.AfirHipError, match="another version of this library"):
+            r(a, a, out_shape=(4, 8))
+    r.close()
+
+
 def test_preferred_code_object_outranks_a_hand_tuned_family(H, evaluator, monkeypatch, tmp_path):
     """A program that is exactly one of the hand-tuned families keeps that kernel
     when a code object is attached, unless the code object is preferred."""
