@@ -198,6 +198,47 @@ def test_few_long_rows_are_spread_along_the_row(H, shape):
         assert got.tobytes() == want.tobytes(), (ty, shape)
 
 
+def test_positions_beyond_32_bits(H):
+    """Tensors of more than 2^31 elements take the kernels with 64-bit positions: an
+    elementwise region, a row sum and a transposed read over [32776, 65536] halves (4.3 GB
+    each).  Too large for the numpy oracle to be quick, so the inputs are made on the GPU
+    and the expected values come from torch's own elementwise, sum and transpose kernels."""
+    import torch
+    rows, n = 32776, 65536
+    assert rows * n > 2 ** 31
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.empty((rows, n), dtype=torch.float16, device="cuda")
+    for r0 in range(0, rows, 4096):          # filled in pieces: no float32 copy of the whole tensor
+        part = x[r0:r0 + 4096]
+        part.copy_(torch.randint(-3, 4, part.shape, generator=gen, device="cuda", dtype=torch.int8))
+    c = torch.randint(-3, 4, (n,), generator=gen, device="cuda", dtype=torch.int8).to(torch.float16)
+    head = RC.HEADER + "arg in f16 2\narg in f16 1\n"
+    # relu(x * c): small integers, every product exact
+    text = head + "arg out f16 2\nsegment 2\n size arg0.0 arg0.1\n outoff 0\n push arg0 d0 d1\n push arg1 d1\n mul\n relu\n store\nend\n"
+    r = region(H, text)
+    out = r(x, c, out_shape=(rows, n))
+    r.close()
+    for r0 in range(0, rows, 4096):
+        assert torch.equal(out[r0:r0 + 4096], torch.relu(x[r0:r0 + 4096] * c)), r0
+    # the last rows lie beyond element 2^31
+    assert (rows - 1) * n > 2 ** 31 and bool((out[-1] == torch.relu(x[-1] * c)).all())
+    del out
+    # row sums of x * c: integers below 2^24, exact in float32 in any order
+    text = head + "arg out f32 1\nsegment 2\n size arg0.0 arg0.1\n outoff 0\n push arg0 d0 d1\n push arg1 d1\n mul\n reduce sum\n store\nend\n"
+    r = region(H, text)
+    sums = r(x, c, out_shape=(rows,))
+    r.close()
+    want = torch.cat([(x[r0:r0 + 2048].float() * c.float()).sum(dim=1) for r0 in range(0, rows, 2048)])
+    assert torch.equal(sums, want)
+    # out[j, i] = x[i, j] + c[j]: the transposed read through LDS tiles
+    text = head + "arg out f16 2\nsegment 2\n size arg0.1 arg0.0\n outoff 0\n push arg0 d1 d0\n push arg1 d0\n add\n store\nend\n"
+    r = region(H, text)
+    out = r(x, c, out_shape=(n, rows))
+    r.close()
+    for j0 in range(0, n, 8192):
+        assert torch.equal(out[j0:j0 + 8192], (x[:, j0:j0 + 8192] + c[j0:j0 + 8192]).t()), j0
+
+
 def test_unaligned_bases_take_the_element_path(H):
     import torch
     rng = np.random.default_rng(12)
