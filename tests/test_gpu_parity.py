@@ -300,6 +300,51 @@ def test_c5_empty_and_blockdim(H):
 
 # ------------------------------------------------------- dispatch by name ----
 
+def test_tensors_of_more_than_2_to_31_elements(H):
+    """The hand-tuned kernels on tensors whose element positions do not fit 32 bits.  The
+    inputs are small integers made on the GPU (too large for the numpy oracle to be quick);
+    the expected values come from torch's own elementwise, sum, transpose and indexing
+    kernels, slice by slice, and every result is exact."""
+    gen = torch.Generator(device="cuda").manual_seed(9)
+
+    def ints(shape, dtype, lo=-3, hi=4):
+        t = torch.empty(shape, dtype=dtype, device="cuda")
+        flat = t.view(-1)
+        step = 1 << 28
+        for i0 in range(0, flat.numel(), step):
+            part = flat[i0:i0 + step]
+            part.copy_(torch.randint(lo, hi, part.shape, generator=gen, device="cuda", dtype=torch.int8))
+        return t
+
+    rows, n = 32776, 65536                     # 2^31 + 2^19 elements
+    # C1: (a + b) * b, f32
+    a, b = ints((rows, n), torch.float32), ints((rows, n), torch.float32)
+    out = H.fused_add_mul(a, b)
+    for r0 in range(0, rows, 4096):
+        assert torch.equal(out[r0:r0 + 4096], (a[r0:r0 + 4096] + b[r0:r0 + 4096]) * b[r0:r0 + 4096]), r0
+    del b, out
+    # C2: row sums of x + bias, f32 (integers: exact in any order)
+    bias = ints((n,), torch.float32)
+    y = H.broadcast_add_reducesum(a, bias)
+    want = torch.cat([(a[r0:r0 + 2048] + bias).sum(dim=1) for r0 in range(0, rows, 2048)])
+    assert torch.equal(y, want)
+    del a, y, want
+    # C3: out[b, j, i] = relu(x[b, i, j]) + c[j], f16
+    x = ints((33, 8192, 8192), torch.float16)
+    c = ints((8192,), torch.float16)
+    out = H.relu_broadcast_add_transpose(x, c)
+    for k in range(33):
+        assert torch.equal(out[k], (torch.relu(x[k]) + c).t()), k
+    del x, out
+    # C4: rows of a table of 2^31 + 2^21 elements, the last rows among them
+    table = ints((2099200, 1024), torch.float16)
+    idx = torch.randint(0, 2099200, (4096,), generator=gen, device="cuda", dtype=torch.int32)
+    idx[:4] = torch.tensor([2099199, 2097152, 0, 2099198], dtype=torch.int32)
+    scale, shift = ints((1024,), torch.float16, 1, 4), ints((1024,), torch.float16)
+    got = H.gather_scale_shift(table, idx, scale, shift)
+    assert torch.equal(got, table[idx.long()] * scale + shift)
+
+
 def test_launch_by_name_and_errors(H):
     import ctypes
     L = H.load()
