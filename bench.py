@@ -39,7 +39,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # (two runs), scaled by the same counters' reading for a plain 256 MiB copy
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Source: profiles/*.txt, section (2).
 MEASURED_TRAFFIC = {"c1": 201364377, "c2": 134645398, "c3": 134331904, "c4": 134146560,
-                    "c5": 2466480128, "g1": 201360588, "g2": 134597632, "i1": 201612185,
+                    "c5": 2466480128, "g1": 201360588, "g2": 134597632, "g3": 134646386, "g4": 134155366,
+                    "i1": 201612185,
                     "i2": 135318732}
 
 
@@ -57,6 +58,37 @@ push arg1 d0 d1
 add
 push arg1 d0 d1
 mul
+store
+end
+"""
+REGION_BCAST_ADD_ROWSUM = """afir-hip-region 1
+arg in f32 2
+arg in f32 1
+arg out f32 1
+segment 2
+size arg0.0 arg0.1
+outoff 0
+push arg0 d0 d1
+push arg1 d1
+add
+reduce sum
+store
+end
+"""
+REGION_GATHER_SCALE_SHIFT = """afir-hip-region 1
+arg in f16 2
+arg in i32 1
+arg in f16 1
+arg in f16 1
+arg out f16 2
+segment 2
+size arg1.0 arg0.1
+outoff 0
+push arg0 g0:arg1 d1
+push arg2 d1
+mul
+push arg3 d1
+add
 store
 end
 """
@@ -334,13 +366,14 @@ def make_workload(key, torch, H, O, C):
                 w.work() * 20 / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
             return ev
         w.power_evidence = power_evidence
-    elif key in ("g1", "g2", "i1", "i2"):
+    elif key in ("g1", "g2", "g3", "g4", "i1", "i2"):
         # Region programs (any fused chain) next to the hand-tuned kernels:
         # g1 / i1 = the c1 chain kept off its fast path, g2 / i2 = the
         # reference's split / relu / broadcast-add / broadcast-mul / concat
         # graph (examples/split-relu-brc-add-mul) at [8192, 4096] f16.
-        # g: kernels emitted and compiled for the program; i: the interpreter
-        # kernel of the library.
+        # g3 / g4 = the c2 row sum and the c4 gather as programs, kept off
+        # their fast paths.  g: kernels emitted and compiled for the program;
+        # i: the interpreter kernel of the library.
         from oracle import region_oracle as RO
         compiled = key[0] == "g"
         how = "compiled region kernel" if compiled else "region interpreter kernel"
@@ -352,6 +385,20 @@ def make_workload(key, torch, H, O, C):
             w.title = f"{key} {how}: (a+b)*b f32 [4096,4096] as a region program"
             w.dtype = "f32"
             work = O.algorithmic_bytes("c1", m=4096, n=4096)
+        elif key[1] == "3":
+            text = REGION_BCAST_ADD_ROWSUM
+            x, bias = O.gen_c2()
+            inputs, out_shape, out_dt = [x, bias], (8192,), torch.float32
+            w.title = f"{key} {how}: rowsum(x+bias) f32 [8192,4096] as a region program"
+            w.dtype = "f32"
+            work = O.algorithmic_bytes("c2", m=8192, n=4096)
+        elif key[1] == "4":
+            text = REGION_GATHER_SCALE_SHIFT
+            inputs = list(O.gen_c4())
+            out_shape, out_dt = (32768, 1024), torch.float16
+            w.title = f"{key} {how}: table[idx]*scale+shift f16 [131072,1024], idx [32768] as a region program"
+            w.dtype = "f16"
+            work = O.algorithmic_bytes("c4", nidx=32768, dim=1024)
         else:
             text = REGION_SPLIT_RELU_BRC_ADD_MUL
             rng = np.random.default_rng(42)
@@ -370,11 +417,19 @@ def make_workload(key, torch, H, O, C):
             region.compile()     # from lib/region_cache when build() left it there
             assert region.kernel == "fused_region_compiled"
         w.work = lambda: work
-        w.nsets = 3 if key[1] == "1" else 4
+        w.nsets = 3 if key[1] in "14" else 4
         dev0 = [_dev(torch, x) for x in inputs]
         sets = []
+        idx_rng = np.random.default_rng(7)
         for i in range(w.nsets):
-            ins = dev0 if i == 0 else [dev0[0].clone()] + ([dev0[1].clone()] if key[1] == "1" else dev0[1:])
+            if i == 0:
+                ins = dev0
+            elif key[1] == "4":
+                # the table (256 MiB) is shared; every set gathers other rows
+                other = idx_rng.integers(0, 131072, 32768, dtype=np.int64).astype(np.int32)
+                ins = [dev0[0], _dev(torch, other)] + dev0[2:]
+            else:
+                ins = [dev0[0].clone()] + ([dev0[1].clone()] if key[1] == "1" else dev0[1:])
             sets.append((ins, torch.empty(out_shape, dtype=out_dt, device="cuda")))
         w.sets = sets
         dims = [d for x in inputs for d in x.shape] + list(out_shape)
@@ -385,9 +440,15 @@ def make_workload(key, torch, H, O, C):
         def parity():
             want = RO.evaluate(text, inputs)
             got = sets[0][1].cpu().numpy()
+            if key[1] == "3":      # a sum in another order: the bar of c2
+                err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+                scale = np.abs(inputs[0].astype(np.float64) + inputs[1]).sum(axis=1)
+                ok = err <= 1e-5 * np.abs(want.astype(np.float64)) + 1e-7 * scale
+                return {"bar": "<=1e-5 rel (+1e-7*sum|terms| floor) vs the region oracle", "passed": bool(ok.all()),
+                        "mismatches": int((~ok).sum()), "max_abs": float(err.max())}
+            bits = np.uint16 if key[1] in "24" else np.uint32
             return {"bar": "bit-exact vs the region oracle", "passed": got.tobytes() == want.tobytes(),
-                    "mismatches": int((got.view(np.uint16 if key[1] == "2" else np.uint32) !=
-                                       want.view(np.uint16 if key[1] == "2" else np.uint32)).sum())}
+                    "mismatches": int((got.view(bits) != want.view(bits)).sum())}
         w.parity = parity
 
         def cpu(budget_s):
@@ -441,7 +502,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "g1", "g2", "i1", "i2"])
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "g1", "g2", "g3", "g4", "i1", "i2"])
     ap.add_argument("--all", dest="all", action="store_true", default=True)
     ap.add_argument("--no-all", dest="all", action="store_false")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -476,7 +537,7 @@ def main():
             return args.warmup
         return 5 if key == "c5" else 30
 
-    order = [args.workload] + ([k for k in ["c1", "c2", "c3", "c4", "c5", "g1", "g2", "i1", "i2"]
+    order = [args.workload] + ([k for k in ["c1", "c2", "c3", "c4", "c5", "g1", "g2", "g3", "g4", "i1", "i2"]
                                 if k != args.workload] if args.all else [])
     results = []
     for key in order:
