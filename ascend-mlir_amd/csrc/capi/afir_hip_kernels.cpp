@@ -614,7 +614,8 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
     afir_target::SpecArgs args;
     bool idx32;
     int mode;    // afir_target::SpecMode
-    int rows;    // 1: the workgroup-per-row kernel of a reduce segment, 2: its form for few, long rows
+    int rows;    // 1: the workgroup-per-row kernel of a reduce segment, 2: its form for few, long rows,
+                 // 3: split (args.column_blocks workgroups per row) and join, for a handful of rows
     bool slim;   // the kernel whose lanes take one group each (short rows)
   };
   std::vector<PendingSegment> pending;   // compiled kernels to launch, non-empty segments only
@@ -737,6 +738,16 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
           if (!slim && seg.reduce && groups >= (int64_t)512 * U && groups % ((int64_t)256 * U) == 0 &&
               nrows_all < (int64_t)afir::kNumCU * 16)
             row_groups = 2;
+          // a handful of rows: the passes of a row are dealt out to about eight workgroups per CU in all
+          const int64_t passes = groups / ((int64_t)256 * U);
+          if (row_groups == 2 && nrows_all <= 64 && passes >= 8 && !block_dim) {
+            int64_t per_row = (int64_t)afir::kNumCU * 8 / nrows_all;
+            if (per_row > passes / 2) per_row = passes / 2;
+            if (per_row >= 2 && per_row * nrows_all <= afir_target::kSpecPartials) {
+              row_groups = 3;
+              sa.column_blocks = (int)per_row;
+            }
+          }
         }
         for (int i = 0; i < a.ninputs; ++i) {
           const afir::RegionInput &d = a.in[i];
@@ -765,7 +776,11 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
         }
         const int mode = vectors && whole ? afir_target::kSpecAligned
                          : vectors && !tile.tiled ? afir_target::kSpecVector : afir_target::kSpecGeneral;
-        if (row_groups && mode == afir_target::kSpecAligned) {
+        if (row_groups == 3 && mode == afir_target::kSpecAligned) {
+          int64_t nrows = 1;
+          for (int k = 0; k < last; ++k) nrows *= seg.size[k];
+          sa.grid = (int)(nrows * sa.column_blocks);
+        } else if (row_groups && mode == afir_target::kSpecAligned) {
           // up to 16 workgroups per CU walk the rows (4 to 16 measured within 1 %, 2 slower)
           int64_t nrows = 1;
           for (int k = 0; k < last; ++k) nrows *= seg.size[k];
@@ -774,6 +789,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
           sa.grid = (int)blocks;
           sa.column_blocks = 1;
         } else {
+          if (row_groups == 3) sa.column_blocks = 1;
           row_groups = 0;
         }
         if (slim && (!g.idx32 || mode == afir_target::kSpecGeneral)) return false;
@@ -830,6 +846,16 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
       if (rc != AFIR_HIP_OK) return rc;
     } else {
       for (PendingSegment &p : pending) {
+        if (p.rows == 3) {
+          uint32_t rc = launch(afir_target::specSplitRowsKernelName(p.segment, p.idx32, false), &p.args, sizeof p.args,
+                               (unsigned)p.args.grid);
+          if (rc != AFIR_HIP_OK) return rc;
+          const int64_t nrows = p.args.grid / p.args.column_blocks;
+          rc = launch(afir_target::specSplitRowsKernelName(p.segment, p.idx32, true), &p.args, sizeof p.args,
+                      (unsigned)((nrows + 3) / 4));
+          if (rc != AFIR_HIP_OK) return rc;
+          continue;
+        }
         const uint32_t rc = launch(p.rows == 2 ? afir_target::specLongRowsKernelName(p.segment, p.idx32)
                                    : p.rows ? afir_target::specRowsKernelName(p.segment, p.idx32)
                                    : p.slim ? afir_target::specSlimKernelName(p.segment, p.mode)

@@ -306,6 +306,7 @@ class SegmentEmitter {
       if (reduce_) {
         emitBodyRowGroup();
         emitBodyLongRows();
+        emitBodySplitRows();
       }
       if (U_ > 1) {
         // the same with one group per lane, for short rows
@@ -943,6 +944,103 @@ class SegmentEmitter {
     hoisted_ = false;
   }
 
+  // Row sums of a handful of very long rows, in two launches: `column_blocks`
+  // workgroups per row each sum a stretch of whole passes (the next pass in
+  // flight) and leave one float in afir_region_partials; then a wavefront per
+  // row adds the row's partial sums in a fixed order.  Deterministic, and the
+  // whole chip works on a single row if that is all there is.  The partial
+  // sums live in the code object: launches of one code object that overlap on
+  // different streams would share them.
+  void emitBodySplitRows() {
+    const std::string otag = typeTag(p_.output().type);
+    os_ << "\n// ---- segment " << index_ << ", a handful of rows of a multiple of " << 256 * U_ * W_
+        << " elements: several workgroups per row, then a join ----\n";
+    os_ << "template <typename I>\nDEV void segment" << index_
+        << "_split(const SpecArgs &R, const I bid, const I nblocks) {\n";
+    line(1, "constexpr int W = " + std::to_string(W_) + ", U = " + std::to_string(U_) + ";");
+    line(1, "constexpr bool A = true, V = true;");
+    line(1, "__attribute__((shared)) static float part[4];");
+    line(1, "const int tid = (int)__builtin_amdgcn_workitem_id_x();");
+    line(1, "const int lane = tid & 63, wave = tid >> 6;");
+    line(1, "const I n = (I)R.size[" + std::to_string(last_) + "];");
+    line(1, "const I passes = n / (I)(256 * U * W);");
+    line(1, "const I cblocks = (I)R.column_blocks;");
+    line(1, "const I row = bid / cblocks, cb = bid - row * cblocks;");
+    line(1, "const I per_block = (passes + cblocks - 1) / cblocks;");
+    line(1, "const I first_pass = cb * per_block;");
+    line(1, "const I end_pass = first_pass + per_block < passes ? first_pass + per_block : passes;");
+    line(1, "(void)nblocks;");
+    for (const Operand &o : operands_)
+      if (o.step != Operand::Broadcast && o.gatherDim != last_)
+        line(1, "const bool vec" + id(o) + " = " + in(o) + ".vec != 0" + (o.gatherDim >= 0 ? " && " + in(o) + ".gvec != 0" : "") + ";");
+    line(1, "I j0[U];");
+    line(1, "int nvalid[U];");
+    line(1, "bool full[U];");
+    unroll();
+    line(1, "for (int u = 0; u < U; ++u) {");
+    line(2, "j0[u] = ((I)tid + (I)u * (I)256 + first_pass * (I)(256 * U)) * W;");
+    line(2, "nvalid[u] = W;");
+    line(2, "full[u] = true;");
+    line(1, "}");
+    hoisted_ = true;
+    emitOperandDeclarations(1);
+    emitPositionOfRow(1);
+    emitRowInvariants(1);
+    line(1, "float acc[W];");
+    unroll();
+    line(1, "for (int e = 0; e < W; ++e) acc[e] = 0.f;");
+    line(1, "if (first_pass < end_pass) {");
+    const std::vector<Value> read = emitReads(2);
+    line(1, "}");
+    line(1, "for (I pass = first_pass; pass < end_pass; ++pass) {");
+    const Value v = emitCompute(2, read);
+    unroll();
+    line(2, "for (int e = 0; e < W; ++e) {");
+    line(3, "float t[U];");
+    unroll();
+    line(3, "for (int u = 0; u < U; ++u) t[u] = " + v.at() + ";");
+    unroll();
+    line(3, "for (int w = U / 2; w >= 1; w >>= 1)");
+    unroll();
+    line(4, "for (int u = 0; u < w; ++u) t[u] = t[2 * u] + t[2 * u + 1];");
+    line(3, "acc[e] += t[0];");
+    line(2, "}");
+    line(2, "if (pass + 1 < end_pass) {");
+    unroll();
+    line(3, "for (int u = 0; u < U; ++u) j0[u] += (I)(256 * U * W);");
+    keepRowConstants_ = false;
+    emitReads(3);
+    line(2, "}");
+    line(1, "}");
+    unroll();
+    line(1, "for (int w = W / 2; w >= 1; w >>= 1)");
+    unroll();
+    line(2, "for (int e = 0; e < w; ++e) acc[e] = acc[2 * e] + acc[2 * e + 1];");
+    line(1, "const float s = wave_sum(acc[0]);");
+    line(1, "if (lane == 0) part[wave] = s;");
+    line(1, "__builtin_amdgcn_fence(__ATOMIC_RELEASE, \"workgroup\");");
+    line(1, "__builtin_amdgcn_s_barrier();");
+    line(1, "__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, \"workgroup\");");
+    line(1, "if (tid == 0) afir_region_partials[(long long)row * (long long)cblocks + (long long)cb] = (part[0] + part[1]) + (part[2] + part[3]);");
+    os_ << "}\n";
+    hoisted_ = false;
+    os_ << "template <typename I>\nDEV void segment" << index_
+        << "_join(const SpecArgs &R, const I bid, const I nblocks) {\n";
+    line(1, "const int tid = (int)__builtin_amdgcn_workitem_id_x();");
+    line(1, "const int lane = tid & 63;");
+    if (rank_ == 2) line(1, "const I rows = (I)R.size[0];");
+    else line(1, "const I rows = (I)(R.size[0] * R.size[1]);");
+    line(1, "const I cblocks = (I)R.column_blocks;");
+    line(1, "(void)nblocks;");
+    line(1, "const I row = bid * 4 + (I)(tid >> 6);");
+    line(1, "if (row >= rows) return;");
+    line(1, "float s = 0.f;");
+    line(1, "for (I c = (I)lane; c < cblocks; c += 64) s += afir_region_partials[(long long)row * (long long)cblocks + (long long)c];");
+    line(1, "s = wave_sum(s);");
+    line(1, "if (lane == 0) st_" + otag + "(R.out, (long long)row, s);");
+    os_ << "}\n";
+  }
+
   // Parallel segment with transposed reads: a workgroup takes a tile of kTileP
   // (the dim those operands are contiguous along) x kTileQ (the innermost
   // iteration dim).  Phase 1 loads each transposed operand's tile with 128-bit
@@ -1068,6 +1166,13 @@ class SegmentEmitter {
             << (i32 ? "int" : "long long") << ")R.grid); }\n";
     if (reduce_)
       for (int i32 = 1; i32 >= 0; --i32)
+        for (int join = 0; join < 2; ++join)
+          os_ << "KERNEL void " << specSplitRowsKernelName(index_, i32 != 0, join != 0) << "(const SpecArgs R) { segment"
+              << index_ << (join ? "_join<" : "_split<") << (i32 ? "int" : "long long")
+              << ">(R, (" << (i32 ? "int" : "long long") << ")__builtin_amdgcn_workgroup_id_x(), ("
+              << (i32 ? "int" : "long long") << ")R.grid); }\n";
+    if (reduce_)
+      for (int i32 = 1; i32 >= 0; --i32)
         os_ << "KERNEL void " << specLongRowsKernelName(index_, i32 != 0) << "(const SpecArgs R) { segment" << index_
             << "_long<" << (i32 ? "int" : "long long")
             << ">(R, (" << (i32 ? "int" : "long long") << ")__builtin_amdgcn_workgroup_id_x(), ("
@@ -1180,6 +1285,10 @@ std::string specRowsKernelName(int segment, bool idx32) {
   return "afir_region_s" + std::to_string(segment) + "_rows" + (idx32 ? "_i32" : "_i64");
 }
 
+std::string specSplitRowsKernelName(int segment, bool idx32, bool join) {
+  return "afir_region_s" + std::to_string(segment) + (join ? "_join" : "_split") + (idx32 ? "_i32" : "_i64");
+}
+
 std::string specLongRowsKernelName(int segment, bool idx32) {
   return "afir_region_s" + std::to_string(segment) + "_long" + (idx32 ? "_i32" : "_i64");
 }
@@ -1215,6 +1324,12 @@ std::string emitHipSource(const Program &p, const std::string &title, std::strin
   os << "extern \"C\" __attribute__((device)) __attribute__((used)) const int afir_region_emit_abi = " << kSpecAbiVersion << ";\n";
   os << "extern \"C\" __attribute__((device)) __attribute__((used)) const int afir_region_emit_options[3] = {"
      << options.tileP << ", " << options.tileQ << ", " << options.unroll << "};   // tile_p, tile_q, unroll\n";
+  bool reduces = false;
+  for (const Segment &g : p.segments)
+    for (const Op &op : g.ops) reduces = reduces || op.code == OpCode::ReduceSum;
+  if (reduces)
+    os << "// partial row sums of the split / join kernels (shared by the launches of this code object)\n"
+       << "__attribute__((device)) float afir_region_partials[" << kSpecPartials << "];\n";
   for (int s = 0; s < (int)p.segments.size(); ++s) {
     SegmentEmitter e(p, s, os, options);
     if (std::string why = e.run(); !why.empty()) return why;

@@ -103,7 +103,7 @@ uint64_t programHash(const afir_region::Program &p);
 // Version of the set of kernels and of the launch arguments that emitHipSource produces; the
 // code object exports it as `afir_region_emit_abi`, and a code object of another version is
 // refused when it is loaded (its kernels would be launched with the wrong names or arguments).
-constexpr int kSpecAbiVersion = 3;
+constexpr int kSpecAbiVersion = 4;
 
 // What a launch promises, which picks the kernel variant:
 //   kSpecAligned  every 128-bit access is aligned and every pass of the lanes over a row is whole
@@ -122,6 +122,11 @@ std::string specRowsKernelName(int segment, bool idx32);
 // ... and one for rows of a whole number (two or more) of such stretches, launched when the
 // rows are too few to fill the chip with a wavefront each.
 std::string specLongRowsKernelName(int segment, bool idx32);
+// ... and a pair for a handful of such rows: `split` (column_blocks workgroups per row, each
+// leaving a partial sum in the code object's afir_region_partials) and `join` (a wavefront per
+// row adds them in a fixed order).  rows x column_blocks may not exceed kSpecPartials.
+constexpr int kSpecPartials = 65536;
+std::string specSplitRowsKernelName(int segment, bool idx32, bool join);
 
 // Emits the source for every segment.  Returns "" on success, else why the
 // program has no specialised form (matmul segments: those run on the

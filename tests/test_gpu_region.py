@@ -154,6 +154,26 @@ def test_row_sums_of_few_long_rows(H, ty, n):
     assert run(H, text, [r, x], (6,), block_dim=4).tobytes() == want.tobytes()
 
 
+@pytest.mark.parametrize("ty,n", [("f32", 8 * 4096), ("f32", 37 * 4096), ("f16", 16 * 8192), ("f16", 1000 * 8192)])
+@pytest.mark.parametrize("rows", [1, 3, 64])
+def test_row_sums_of_a_handful_of_very_long_rows(H, ty, n, rows):
+    """Up to 64 rows of eight or more workgroup passes: the compiled split / join pair
+    (several workgroups per row leave partial sums, a wavefront per row adds them).  Small
+    integers: exact whatever the order, so equal to the oracle bit for bit; run twice to see
+    that nothing is left over in the partial sums."""
+    dt = np.float32 if ty == "f32" else np.float16
+    if rows * n > 40_000_000:
+        pytest.skip("kept small for the numpy oracle")
+    rng = np.random.default_rng(n + rows)
+    text = RC.REDUCE_ROWBIAS.replace("f16", ty)            # r[d0] + x[d0, d1]
+    for _ in range(2):
+        r = rng.integers(-1, 2, (rows,)).astype(dt) * dt(2.0 ** -8)       # n of them stay below the f16 range
+        x = rng.integers(-2, 3, (rows, n)).astype(dt) * dt(0.25)
+        want = RO.evaluate(text, [r, x])
+        assert np.isfinite(want.astype(np.float32)).all()
+        assert run(H, text, [r, x], (rows,)).tobytes() == want.tobytes()
+
+
 def test_row_sums_with_a_row_operand_and_rank_3(H):
     """The workgroup-per-row kernels with an operand that changes with the row (fetched
     ahead with the matrix) and over a rank-3 space whose row is (d0, d1)."""

@@ -108,7 +108,12 @@ def test_reductions_also_get_a_workgroup_per_row_kernel():
     # the bias does not change with the row: loaded once, before the loop, not in the fetch of the next row
     assert rows.count("ldv_f32<W, false>(R.in[1].base") == 1 and rows.count("ldv_f32<W, true>(R.in[0].base") == 2
     assert rows.count("__builtin_amdgcn_s_barrier();") == 1
-    assert "_rows_" not in _emit(RC.C1_ADD_MUL).stdout            # parallel segments have none
+    # ... and the kernels for few long rows and for a handful of very long ones
+    for name in ("afir_region_s0_long_i32(", "afir_region_s0_split_i32(", "afir_region_s0_join_i64("):
+        assert name in src
+    assert "float afir_region_partials[65536];" in src
+    plain = _emit(RC.C1_ADD_MUL).stdout                           # parallel segments have none of these
+    assert "_rows_" not in plain and "_split_" not in plain and "afir_region_partials" not in plain
 
 
 def test_short_rows_get_one_group_per_lane_kernels():
