@@ -108,7 +108,10 @@ std::string compiled_function(CompiledRegion *c, const afir_region::Program &pro
   if (!c->loaded) {
     hipModule_t m = nullptr;
     hipError_t e = hipModuleLoadData(&m, c->image.data());
-    if (e != hipSuccess) return std::string("code object does not load: ") + hipGetErrorString(e);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      return std::string("code object does not load: ") + hipGetErrorString(e);
+    }
     hipDeviceptr_t sym = nullptr;
     size_t bytes = 0;
     unsigned long long hash = 0;
@@ -116,12 +119,14 @@ std::string compiled_function(CompiledRegion *c, const afir_region::Program &pro
     if (e == hipSuccess && bytes == sizeof hash) e = hipMemcpyDtoH(&hash, sym, sizeof hash);
     if (e != hipSuccess || bytes != sizeof hash || hash != afir_target::programHash(program)) {
       (void)hipModuleUnload(m);
+      (void)hipGetLastError();   // a symbol that is not there is reported here, not by a later launch
       return "code object was not built from this program";
     }
     int abi = -1;
     if (hipModuleGetGlobal(&sym, &bytes, m, "afir_region_emit_abi") != hipSuccess || bytes != sizeof abi ||
         hipMemcpyDtoH(&abi, sym, sizeof abi) != hipSuccess || abi != afir_target::kSpecAbiVersion) {
       (void)hipModuleUnload(m);
+      (void)hipGetLastError();
       return "code object was emitted by another version of this library (its kernels and their arguments differ); "
              "compile the artifact again";
     }
@@ -136,6 +141,8 @@ std::string compiled_function(CompiledRegion *c, const afir_region::Program &pro
         (void)hipModuleUnload(m);
         return "code object carries unusable emit options";
       }
+    } else {
+      (void)hipGetLastError();
     }
     c->module = m;
     c->loaded = true;
@@ -145,7 +152,10 @@ std::string compiled_function(CompiledRegion *c, const afir_region::Program &pro
   if (it == c->functions.end()) {
     hipFunction_t f = nullptr;
     const hipError_t e = hipModuleGetFunction(&f, c->module, name.c_str());
-    if (e != hipSuccess) return "code object lacks kernel " + name + ": " + hipGetErrorString(e);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      return "code object lacks kernel " + name + ": " + hipGetErrorString(e);
+    }
     it = c->functions.emplace(name, f).first;
   }
   *fn = it->second;
