@@ -434,6 +434,96 @@ def test_integer_unaligned_views_and_tails(H):
             assert got.tobytes() == want.tobytes(), (ty, m, n)
 
 
+def _random_region(rng):
+    """A random program with its inputs and output shape: iteration rank 1..3; operands
+    read whole, broadcast along rows or columns, transposed or gathered; one element type
+    or a mix; elementwise or a row sum; extents drawn from the classes the kernels tell
+    apart (short rows, whole vectors with partly empty passes, whole passes, ragged)."""
+    rank = int(rng.integers(1, 4))
+    reduce = rank >= 2 and rng.random() < 0.35
+    types = [["f32"], ["f16"], ["bf16"], ["f16", "f32"]][int(rng.integers(0, 4))]
+    n = int(rng.choice([1, 5, 8, 24, 40, 64, 96, 250, 256, 1000, 1024, 2048, 4096, 4099]))
+    if rank == 1:
+        n = int(rng.choice([7, 64, 1000, 33000, 70001]))
+    outer = [int(rng.choice([1, 2, 3, 17, 64, 130]))] if rank >= 2 else []
+    if rank == 3:
+        outer.append(int(rng.choice([1, 4, 9])))
+    size = outer + [n]
+    last = rank - 1
+    dims = lambda ks: " ".join(f"d{k}" for k in ks)
+    # (map text, tensor shape) of the operand kinds available at this rank
+    kinds = [(dims(range(rank)), tuple(size)), (f"d{last}", (n,))]
+    if rank >= 2:
+        kinds.append((dims(range(rank - 1)), tuple(size[:-1])))               # the same along a row
+        kinds.append((f"d{last - 1} d{last}" if rank == 3 else f"d0 0", (size[last - 1], n) if rank == 3 else (size[0], 1)))
+    if rank == 2 and not reduce:
+        kinds.append(("d1 d0", (n, size[0])))                                  # transposed
+    if rank == 3 and not reduce:
+        kinds.append(("d0 d2 d1", (size[0], n, size[1])))
+    args, shapes, pushes = [f"arg in {types[0]} {rank}"], [tuple(size)], []
+    ops = ["push arg0 " + dims(range(rank))]
+    gather = rank == 2 and rng.random() < 0.25
+    if gather:                                   # rows of a table picked by an index tensor
+        table_rows = int(rng.integers(size[0], size[0] + 50))
+        ity = ["i32", "i64"][int(rng.integers(0, 2))]
+        args += [f"arg in {types[-1]} 2", f"arg in {ity} 1"]
+        shapes += [(table_rows, n), ("index", ity, table_rows, size[0])]
+        ops += [f"push arg1 g0:arg2 d1", "add"]
+    depth = 1
+    allowed2 = ["add", "sub", "mul", "max", "min"] + ([] if reduce else ["div"])
+    allowed1 = ["relu", "neg"] + ([] if reduce else ["leaky 0.25"])
+    for _ in range(int(rng.integers(1, 7))):
+        k = int(rng.integers(0, 4))
+        if depth < 3 and k == 0 and len(args) < 6:
+            if rng.random() < 0.2:
+                ops.append("const 2")
+            else:
+                text, shape = kinds[int(rng.integers(0, len(kinds)))]
+                ty = types[int(rng.integers(0, len(types)))]
+                ops.append(f"push arg{len(args)} {text}")
+                args.append(f"arg in {ty} {len(shape)}")
+                shapes.append(shape)
+            depth += 1
+        elif depth >= 2 and k in (1, 2):
+            ops.append(allowed2[int(rng.integers(0, len(allowed2)))])
+            depth -= 1
+        else:
+            ops.append(allowed1[int(rng.integers(0, len(allowed1)))])
+    while depth > 1:
+        ops.append(["add", "sub", "max"][int(rng.integers(0, 3))])
+        depth -= 1
+    out_ty = types[0]
+    out_shape = tuple(size[:-1]) if reduce else tuple(size)
+    text = (RC.HEADER + "\n".join(args) + f"\narg out {out_ty} {len(out_shape)}\nsegment {rank}\n size "
+            + " ".join(f"arg0.{k}" for k in range(rank)) + "\n outoff 0\n " + "\n ".join(ops)
+            + ("\n reduce sum" if reduce else "") + "\n store\nend\n")
+    inputs = []
+    for a, shape in zip(args, shapes):
+        ty = a.split()[2]
+        if shape and shape[0] == "index":
+            _, ity, hi, count = shape
+            inputs.append(rng.integers(0, hi, (count,)).astype(np.int32 if ity == "i32" else np.int64))
+            continue
+        v = rng.integers(-3, 4, shape).astype(np.float32)           # small integers: sums are exact in any order
+        inputs.append(v.astype(np.float16) if ty == "f16" else O.f32_to_bf16_bits(v) if ty == "bf16" else v)
+    return text, inputs, out_shape, out_ty
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_random_programs_over_the_shape_classes(H, seed):
+    rng = np.random.default_rng(777 + seed)
+    text, inputs, out_shape, out_ty = _random_region(rng)
+    want = RO.evaluate(text, inputs)
+    got = run(H, text, inputs, out_shape)
+    if out_ty == "bf16":
+        wf, gf = O.bf16_bits_to_f32(want), O.bf16_bits_to_f32(got)
+    else:
+        wf, gf = want.astype(np.float32), got.astype(np.float32)
+    bits = np.uint32 if out_ty == "f32" else np.uint16
+    same = (got.view(bits) == want.view(bits)) | (np.isnan(wf) & np.isnan(gf))
+    assert same.all(), (text, [getattr(x, "shape", None) for x in inputs], np.argwhere(~same)[:5])
+
+
 def test_every_operation_pair_at_every_vector_position(H):
     """binary step followed by up to two activations, all combinations, on rows
     of 19 elements (two full vectors and a tail): every position of the result
