@@ -1,0 +1,77 @@
+"""The launch entry points recorded into a HIP graph and replayed: launch-bound
+chains of small kernels are meant to be captured once and replayed.  Every replay,
+with the program's own eager work and synchronisations between replays, must give
+what the same launches give eagerly.  Needs a GPU."""
+import numpy as np
+import pytest
+
+from tests import region_cases as RC
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def H(pkg):
+    from ascend_mlir_amd import hip_kernels
+    hip_kernels.load()
+    assert torch.cuda.is_available(), "no GPU visible"
+    return hip_kernels
+
+
+def test_kernels_replay_from_a_captured_graph(H, tmp_path, monkeypatch):
+    """(a + b) * b on the hand-tuned kernel, then relu(col) + x on a compiled region, then
+    the row sums of a handful of long rows (the split / join pair) -- captured together."""
+    monkeypatch.setenv("AFIR_HIP_REGION_GENERIC", "1")
+    m, n = 96, 256
+    gen = torch.Generator(device="cuda").manual_seed(3)
+
+    def ints(shape, dtype):
+        return torch.randint(-3, 4, shape, generator=gen, device="cuda", dtype=torch.int32).to(dtype)
+
+    a, b = ints((m, n), torch.float32), ints((m, n), torch.float32)
+    ab = torch.empty_like(a)
+    col, x = ints((n, 1), torch.float16), ints((m, n), torch.float16)
+    y = torch.empty_like(x)
+    long_rows = ints((2, 16 * 8192), torch.float16)
+    row_term = ints((2,), torch.float16) * 2.0 ** -8        # 131072 of them stay inside the f16 range
+    sums = torch.empty((2,), dtype=torch.float16, device="cuda")
+    elementwise = H.Region(RC.RELU_COL_ADD).compile(str(tmp_path))
+    row_sum = H.Region(RC.REDUCE_ROWBIAS).compile(str(tmp_path))
+
+    def launches():
+        return [
+            H.prepare("afir_hip_launch_fused_add_mul", [a.data_ptr(), b.data_ptr(), ab.data_ptr(), 0], H.pack_tiling(m, n)),
+            elementwise.prepare([col.data_ptr(), x.data_ptr(), y.data_ptr()], H.pack_tiling(n, 1, m, n, m, n)),
+            row_sum.prepare([row_term.data_ptr(), long_rows.data_ptr(), sums.data_ptr()],
+                            H.pack_tiling(2, 2, 16 * 8192, 2)),
+        ]
+
+    def eager():
+        for call in launches():
+            call()
+        torch.cuda.synchronize()
+        return ab.clone(), y.clone(), sums.clone()
+
+    eager()                                   # modules loaded, kernels resolved
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for call in launches():               # prepared inside: the stream is the capturing one
+            call()
+    for replay in range(4):
+        for t in (a, b, x, long_rows):        # eager work between replays: new inputs in the same buffers
+            t.copy_(ints(tuple(t.shape), t.dtype))
+        want = eager()
+        for t in (ab, y, sums):
+            t.fill_(7)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, expected, what in zip((ab, y, sums), want, ("add-mul", "region", "row sums")):
+            assert torch.equal(got, expected), (replay, what)
+    assert torch.equal(ab, (a + b) * b) and torch.equal(y, torch.relu(col.t()) + x)
+    total = long_rows.float().sum(dim=1) + 16 * 8192 * row_term.float()
+    assert bool(torch.isfinite(total.half()).all()) and torch.equal(sums, total.half())
+    elementwise.close()
+    row_sum.close()
