@@ -10,7 +10,8 @@
 //         -Xclang -target-feature -Xclang -packed-fp32-ops -o region.hsaco region.hip
 // The code object is attached to the registered program
 // (afir_hip_region_attach_code_object) and launched in place of the generic
-// interpreter kernel; results are bit-identical to it.
+// interpreter kernel; parallel segments give the same bits as that kernel, row
+// sums (float32 sums in another, fixed order) agree within rounding.
 //
 // What is fixed at emission: the iteration rank, the operation sequence, the
 // element types, which operands are broadcast / contiguous / strided / gathered
