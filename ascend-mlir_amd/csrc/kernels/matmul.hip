@@ -56,7 +56,21 @@ __device__ __forceinline__ void map_tile(int p, int tiles_m, int tiles_n, int &t
 // and out are f32 -- the types of the reference's own matmul example
 // (examples/matmul-add-leakyrelu/step0_input.mlir:10-15); same tiling, the
 // f16 MFMA, and an epilogue that stores the float32 value unrounded.
-template <int WAVES_M, int WAVES_N, int TM, int TN, bool F16IO>
+// Eight consecutive 16-bit elements, the first `valid` of them read one by one
+// (no alignment needed), the rest zeros.
+__device__ __forceinline__ u32x4 load_elements(const uint16_t *p, int valid) {
+  uint32_t h[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) h[e] = e < valid ? (uint32_t)p[e] : 0u;
+  const u32x4 v = {h[0] | (h[1] << 16), h[2] | (h[3] << 16), h[4] | (h[5] << 16), h[6] | (h[7] << 16)};
+  return v;
+}
+
+// EDGE = 1: M is arbitrary, K and N are multiples of 8 (rows start on 16-byte
+// boundaries): chunks outside the matrices are read as zeros, stores outside
+// are dropped, the K loop runs over the last, partly empty step as well.
+// EDGE = 2: any M, K, N and any alignment: the same with element accesses.
+template <int WAVES_M, int WAVES_N, int TM, int TN, bool F16IO, int EDGE>
 __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void matmul_bias_leakyrelu_mfma(
     const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
     const void *__restrict__ bias_v, void *__restrict__ out_v, int M, int K, int N,
@@ -72,7 +86,8 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void matmul_bias_leakyrelu_m
 
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
   const int wm = wave / WAVES_N, wn = wave % WAVES_N;
-  const int KT = K / kBK;
+  const int KT = EDGE ? (K + kBK - 1) / kBK : K / kBK;
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
 
   for (int p = blockIdx.x; p < tiles_m * tiles_n; p += gridDim.x) {
     int tile_m, tile_n;
@@ -95,7 +110,14 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void matmul_bias_leakyrelu_m
 #pragma unroll
       for (int i = 0; i < A_ITERS; ++i) {
         const int id = t + NT * i, row = id >> 3, c = id & 7;
-        ra[i] = *reinterpret_cast<const u32x4 *>(A + (int64_t)(m0 + row) * K + k0 + c * 8);
+        if (EDGE == 2) {
+          const int left = m0 + row < M ? K - (k0 + c * 8) : 0;
+          ra[i] = left > 0 ? load_elements(A + (int64_t)(m0 + row) * K + k0 + c * 8, left) : zero4;
+        } else if (!EDGE || (m0 + row < M && k0 + c * 8 < K)) {
+          ra[i] = *reinterpret_cast<const u32x4 *>(A + (int64_t)(m0 + row) * K + k0 + c * 8);
+        } else {
+          ra[i] = zero4;
+        }
       }
 #pragma unroll
       for (int i = 0; i < B_ITERS; ++i) {
@@ -104,9 +126,16 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void matmul_bias_leakyrelu_m
         const int kg = (((rest & 1) * 4 + kq) << 1) + half;
         const int nc = (rest >> 1) * 8 + ncl;
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          rb[i][r] = *reinterpret_cast<const u32x4 *>(B + (int64_t)(k0 + kg * 4 + r) * N + n0 +
-                                                      nc * 8);
+        for (int r = 0; r < 4; ++r) {
+          if (EDGE == 2) {
+            const int left = k0 + kg * 4 + r < K ? N - (n0 + nc * 8) : 0;
+            rb[i][r] = left > 0 ? load_elements(B + (int64_t)(k0 + kg * 4 + r) * N + n0 + nc * 8, left) : zero4;
+          } else if (!EDGE || (k0 + kg * 4 + r < K && n0 + nc * 8 < N)) {
+            rb[i][r] = *reinterpret_cast<const u32x4 *>(B + (int64_t)(k0 + kg * 4 + r) * N + n0 + nc * 8);
+          } else {
+            rb[i][r] = zero4;
+          }
+        }
       }
     };
 
@@ -188,8 +217,17 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void matmul_bias_leakyrelu_m
       for (int q = 0; q < 4; ++q) {
         const int n = n0 + (wn * TN + j) * 32 + 8 * q + 4 * lq;
         float b0, b1, b2, b3;
-        if (!bias_v) {
+        if (!bias_v || (EDGE && n >= N)) {
           b0 = b1 = b2 = b3 = -0.f;   // no bias: x + (-0) is x for every x, signed zeros included
+        } else if (EDGE == 2) {
+          float bb[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if (n + e >= N) bb[e] = -0.f;
+            else if constexpr (F16IO) bb[e] = static_cast<const float *>(bias_v)[n + e];
+            else bb[e] = __uint_as_float((uint32_t) static_cast<const uint16_t *>(bias_v)[n + e] << 16);
+          }
+          b0 = bb[0]; b1 = bb[1]; b2 = bb[2]; b3 = bb[3];
         } else if constexpr (F16IO) {
           const f32x4 bf = *reinterpret_cast<const f32x4 *>(static_cast<const float *>(bias_v) + n);
           b0 = bf[0]; b1 = bf[1]; b2 = bf[2]; b3 = bf[3];
@@ -201,6 +239,7 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void matmul_bias_leakyrelu_m
 #pragma unroll
         for (int i = 0; i < TM; ++i) {
           const int m = m0 + (wm * TM + i) * 32 + lm;
+          if (EDGE && (m >= M || n >= N)) continue;
           float v0 = acc[i][j][4 * q + 0] + b0;
           float v1 = acc[i][j][4 * q + 1] + b1;
           float v2 = acc[i][j][4 * q + 2] + b2;
@@ -209,7 +248,15 @@ __global__ __launch_bounds__(WAVES_M *WAVES_N * 64) void matmul_bias_leakyrelu_m
           v1 = fmaxf(v1, relu ? 0.f : v1 * alpha);
           v2 = fmaxf(v2, relu ? 0.f : v2 * alpha);
           v3 = fmaxf(v3, relu ? 0.f : v3 * alpha);
-          if constexpr (F16IO) {
+          if (EDGE == 2) {
+            const float vv[4] = {v0, v1, v2, v3};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              if (n + e >= N) continue;
+              if constexpr (F16IO) static_cast<float *>(out_v)[(int64_t)m * N + n + e] = vv[e];
+              else static_cast<uint16_t *>(out_v)[(int64_t)m * N + n + e] = (uint16_t)f32_to_bf16_rne(vv[e]);
+            }
+          } else if constexpr (F16IO) {
             const f32x4 w = {v0, v1, v2, v3};
             *reinterpret_cast<f32x4 *>(static_cast<float *>(out_v) + (int64_t)m * N + n) = w;
           } else {
@@ -261,18 +308,18 @@ __global__ __launch_bounds__(256) void matmul_bias_leakyrelu_any(
   }
 }
 
-template <int WAVES_M, int WAVES_N, int TM, int TN, bool F16IO>
+template <int WAVES_M, int WAVES_N, int TM, int TN, bool F16IO, int EDGE = 0>
 LaunchStatus launch_mfma(const uint16_t *a, const uint16_t *b, const void *bias, void *out, int m,
                          int k, int n, float alpha, bool relu, uint32_t block_dim, hipStream_t stream) {
   constexpr int NT = WAVES_M * WAVES_N * 64;
   constexpr int BM = WAVES_M * TM * 32, BN = WAVES_N * TN * 32;
   constexpr size_t kLds = 2 * (size_t)(BM + BN) * kPitch;
-  auto kernel = matmul_bias_leakyrelu_mfma<WAVES_M, WAVES_N, TM, TN, F16IO>;
+  auto kernel = matmul_bias_leakyrelu_mfma<WAVES_M, WAVES_N, TM, TN, F16IO, EDGE>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize,
                                                (int)kLds);
   if (attr != hipSuccess) return LaunchStatus{2u, hipGetErrorString(attr)};
-  const int tiles_m = m / BM, tiles_n = n / BN;
+  const int tiles_m = EDGE ? (m + BM - 1) / BM : m / BM, tiles_n = EDGE ? (n + BN - 1) / BN : n / BN;
   int64_t blocks = (int64_t)tiles_m * tiles_n;
   if (block_dim) blocks = block_dim;
   hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(NT), kLds, stream, a, b, bias, out, m, k,
@@ -308,6 +355,12 @@ LaunchStatus launch_matmul_any_io(const uint16_t *a, const uint16_t *b, const vo
     return launch_mfma<2, 4, 4, 2, F16IO>(a, b, bias, out, (int)m, (int)k, (int)n, alpha, relu, block_dim, stream);
   if (al && k >= kBK && k % kBK == 0 && m % 128 == 0 && n % 128 == 0)
     return launch_mfma<2, 2, 2, 2, F16IO>(a, b, bias, out, (int)m, (int)k, (int)n, alpha, relu, block_dim, stream);
+  // any M, K and N multiples of 8 (every row starts on a 16-byte boundary): the same kernel, bounds-checked
+  if (al && k >= 8 && k % 8 == 0 && n % 8 == 0 && (int64_t)((m + 127) / 128) * ((n + 127) / 128) <= 0x7fffffff)
+    return launch_mfma<2, 2, 2, 2, F16IO, 1>(a, b, bias, out, (int)m, (int)k, (int)n, alpha, relu, block_dim, stream);
+  // anything else that is not tiny: element accesses into the same MFMA loop
+  if (k >= 1 && m * n >= 128 * 128 && (int64_t)((m + 127) / 128) * ((n + 127) / 128) <= 0x7fffffff)
+    return launch_mfma<2, 2, 2, 2, F16IO, 2>(a, b, bias, out, (int)m, (int)k, (int)n, alpha, relu, block_dim, stream);
 
   const int tiles_m = (int)((m + 15) / 16), tiles_n = (int)((n + 15) / 16);
   int64_t blocks = (int64_t)tiles_m * tiles_n;

@@ -246,7 +246,11 @@ def _check_c5(got_bits, want_bits):
 
 @pytest.mark.parametrize("m,k,n", [(256, 256, 256), (512, 128, 768), (128, 64, 128),
                                    (384, 192, 128), (48, 1024, 80), (1, 1, 1), (17, 33, 65),
-                                   (256, 100, 256)])
+                                   (256, 100, 256),
+                                   # K and N multiples of 8, nothing else aligned: the bounds-checked MFMA kernel
+                                   (1, 8, 8), (130, 72, 136), (1000, 1000, 1000), (257, 8, 520), (300, 1096, 24),
+                                   # odd extents: the same kernel with element accesses
+                                   (257, 129, 513), (300, 1001, 517), (129, 1, 127), (2048, 3, 9)])
 def test_c5_small(H, m, k, n):
     a, b, bias = O.gen_c5(m, k, n)
     out = H.matmul_add_leakyrelu(dev_bf16(a), dev_bf16(b), dev_bf16(bias), 0.01)
@@ -264,6 +268,42 @@ def test_c5_integer_known_answer_exact(H):
         bits = [O.f32_to_bf16_bits(v) for v in (A, B, bias)]
         out = H.matmul_add_leakyrelu(dev_bf16(bits[0]), dev_bf16(bits[1]), dev_bf16(bits[2]), 0.01)
         assert np.array_equal(host_bf16(out), O.golden_c5(*bits, 0.01))
+
+
+@pytest.mark.parametrize("ty", ["bf16", "f16"])
+def test_c5_ragged_shapes_integer_known_answer_exact(H, ty):
+    """Shapes that are not multiples of the tiles, on small integers (every product and
+    partial sum exact in float32): the bounds-checked MFMA kernel must reproduce
+    leakyrelu(A @ B + bias) exactly and leave the rows next to the output alone."""
+    import os
+    import subprocess
+    from oracle import region_oracle as RO
+    from tests import mlir_cases as MC
+    for (m, k, n) in ((1000, 1000, 1000), (129, 136, 264), (5, 64, 8), (301, 1001, 517), (131, 7, 129)):
+        rng = np.random.default_rng(m + k)
+        a = rng.integers(-3, 4, (m, k)).astype(np.float32)
+        b = rng.integers(-3, 4, (k, n)).astype(np.float32)
+        bias = rng.integers(-8, 9, (n,)).astype(np.float32)
+        v = a @ b + bias[None, :]
+        assert np.abs(v).max() < 2 ** 24
+        if ty == "bf16":
+            bits = [O.f32_to_bf16_bits(x) for x in (a, b, bias)]
+            guard = torch.full((m + 2, n), 7.0, dtype=torch.bfloat16, device="cuda")
+            out = H.matmul_add_leakyrelu(dev_bf16(bits[0]), dev_bf16(bits[1]), dev_bf16(bits[2]), 0.25, out=guard[1:m + 1])
+            torch.cuda.synchronize()
+            assert np.array_equal(host_bf16(out), O.golden_c5(*bits, 0.25)), (m, k, n)
+            assert bool((guard[0] == 7).all()) and bool((guard[m + 1] == 7).all())
+        else:
+            tr = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "ascend-mlir_amd", "bin",
+                              "afir-translate")
+            text = subprocess.run([tr, "-mlir-to-hip", "-"], input=MC.MATMUL_BIAS_LEAKY_F16, capture_output=True,
+                                  text=True, check=True).stdout
+            r = H.Region(text)
+            ins = [a.astype(np.float16), b.astype(np.float16), bias, np.zeros((m, n), np.float32)]
+            got = r(*[dev(x) for x in ins], out_shape=(m, n)).cpu().numpy()
+            r.close()
+            assert got.tobytes() == RO.evaluate(text, ins).tobytes(), (m, k, n)
+            assert np.array_equal(got, np.maximum(v, v * np.float32(0.001)))
 
 
 def test_c5_identity_and_alpha(H):
