@@ -112,8 +112,48 @@ def build_runtime():
     return [lib, exe, at_exe, tr_exe]
 
 
+HIPCC_REGION_FLAGS = ["--genco", "--offload-arch=gfx950", "-O3", "-nogpuinc", "-ffp-contract=off",
+                      "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+
+def build_families(kernel_lib):
+    """The kernel families as compiled region kernels: lib/families/<family>.hsaco, which
+    the family launchers fall back on for shapes their specialised kernels do not take."""
+    import ctypes
+    L = ctypes.CDLL(kernel_lib)
+    L.afir_hip_family_program.restype = ctypes.c_char_p
+    L.afir_hip_family_program.argtypes = [ctypes.c_char_p]
+    L.afir_hip_region_register.argtypes = [ctypes.c_char_p, ctypes.c_size_t, ctypes.POINTER(ctypes.c_uint64)]
+    L.afir_hip_region_emit_source.argtypes = [ctypes.c_uint64, ctypes.c_char_p, ctypes.c_size_t,
+                                              ctypes.POINTER(ctypes.c_size_t)]
+    out_dir = os.path.join(LIB, "families")
+    os.makedirs(out_dir, exist_ok=True)
+    built = []
+    for family in ("broadcast_add_reducesum", "relu_broadcast_add_transpose", "gather_scale_shift"):
+        text = L.afir_hip_family_program(family.encode())
+        handle, n = ctypes.c_uint64(0), ctypes.c_size_t(0)
+        os.environ["AFIR_HIP_REGION_GENERIC"] = "1"
+        try:
+            rc = L.afir_hip_region_register(text, len(text), ctypes.byref(handle))
+        finally:
+            del os.environ["AFIR_HIP_REGION_GENERIC"]
+        if rc or L.afir_hip_region_emit_source(handle, None, 0, ctypes.byref(n)):
+            raise RuntimeError(f"cannot emit the source of family {family}")
+        buf = ctypes.create_string_buffer(n.value + 1)
+        L.afir_hip_region_emit_source(handle, buf, n.value + 1, ctypes.byref(n))
+        L.afir_hip_region_unregister(handle)
+        src = os.path.join(OBJ, family + ".hip")
+        with open(src, "wb") as f:
+            f.write(buf.value)
+        obj = os.path.join(out_dir, family + ".hsaco")
+        _run([HIPCC, *HIPCC_REGION_FLAGS, "-o", obj, src])
+        built.append(obj)
+    return built
+
+
 def build_all():
-    return [build_kernels(), *build_runtime()]
+    kernel_lib = build_kernels()
+    return [kernel_lib, *build_runtime(), *build_families(kernel_lib)]
 
 
 if __name__ == "__main__":

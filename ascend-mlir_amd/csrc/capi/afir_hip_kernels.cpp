@@ -15,7 +15,13 @@
 #include <mutex>
 #include <vector>
 
+#include <dlfcn.h>
+
+#include <fstream>
+#include <iterator>
+
 #include "../kernels/kernels.h"
+#include "family_programs.h"
 #include "../kernels/region_launch.h"
 #include "../target/hip_emitter.h"
 #include "../target/region_program.h"
@@ -351,6 +357,12 @@ std::string resolve_region(const RegisteredRegion &r, const void *tiling, size_t
 
 }  // namespace
 
+namespace {
+// (defined with the region registry below)
+bool launch_family_region(int which, uint32_t block_dim, void *stream, std::initializer_list<void *> args,
+                          void *workspace, std::initializer_list<int64_t> dims, uint32_t *rc);
+}  // namespace
+
 extern "C" {
 
 const char *afir_hip_last_error(void) { return g_last_error.c_str(); }
@@ -371,6 +383,18 @@ uint32_t afir_hip_launch_broadcast_add_reducesum(uint32_t block_dim, void *strea
   int64_t f[2];
   if (!read_fields(tiling, 2, f))
     return fail(AFIR_HIP_E_INVALID, "broadcast_add_reducesum: null tiling");
+  {
+    // The family's kernels give a wavefront or a workgroup to a row.  Rows of fewer than 512 chunks
+    // (lanes shared between rows) and fewer than 1024 rows (a workgroup or several per row) measured
+    // faster on the compiled region kernels: 100000 x 100 floats 2.5 -> 3.2 TB/s, 64 x 2^20 0.28 -> 5.4;
+    // other shapes measured the same or slower there and stay here.
+    const int64_t m = f[0], n = f[1], n4 = n / 4;
+    const bool vec = n > 0 && n % 4 == 0 && ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(bias)) & 15u) == 0;
+    uint32_t rc;
+    if (m > 0 && x && bias && y && vec && (n4 < 512 || m < 1024) &&
+        launch_family_region(0, block_dim, stream, {x, bias, y}, nullptr, {m, n, n, m}, &rc))
+      return rc;
+  }
   return finish(afir::launch_broadcast_add_reducesum(
       static_cast<const float *>(x), static_cast<const float *>(bias), static_cast<float *>(y),
       f[0], f[1], block_dim, static_cast<hipStream_t>(stream)));
@@ -382,6 +406,20 @@ uint32_t afir_hip_launch_relu_broadcast_add_transpose(uint32_t block_dim, void *
   int64_t f[3];
   if (!read_fields(tiling, 3, f))
     return fail(AFIR_HIP_E_INVALID, "relu_broadcast_add_transpose: null tiling");
+  {
+    // the specialised kernel takes whole 64 x 64 tiles of aligned tensors; other extents that are
+    // multiples of 8 (every row on a 16-byte boundary) run on the compiled region kernels, tiles with
+    // bounds checks and 128-bit accesses (64 x 1024 x 520: 2.3 -> 4.9 TB/s); the rest keeps the
+    // family's 2-byte kernel, which measured faster than element accesses there
+    const int64_t nb = f[0], m = f[1], n = f[2];
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(c) |
+                           reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+    uint32_t rc;
+    if (nb > 0 && m >= 64 && n >= 64 && x && c && out && aligned && m % 8 == 0 && n % 8 == 0 &&
+        !(m % 64 == 0 && n % 64 == 0) &&
+        launch_family_region(1, block_dim, stream, {x, c, out}, nullptr, {nb, m, n, n, nb, n, m}, &rc))
+      return rc;
+  }
   return finish(afir::launch_relu_broadcast_add_transpose(
       static_cast<const uint16_t *>(x), static_cast<const uint16_t *>(c),
       static_cast<uint16_t *>(out), f[0], f[1], f[2], block_dim,
@@ -394,6 +432,20 @@ uint32_t afir_hip_launch_gather_scale_shift(uint32_t block_dim, void *stream, vo
   int64_t f[3];
   if (!read_fields(tiling, 3, f))
     return fail(AFIR_HIP_E_INVALID, "gather_scale_shift: null tiling");
+  {
+    // rows of fewer than 256 halves leave most lanes of the family's kernels idle; the compiled
+    // region kernels give such rows one 16-byte chunk per lane (131072 x 64 table: 2.9 -> 6.6 TB/s).
+    // Longer rows measured faster here.
+    const int64_t rows = f[0], dim = f[1], nidx = f[2];
+    const bool aligned = ((reinterpret_cast<uintptr_t>(table) | reinterpret_cast<uintptr_t>(scale) |
+                           reinterpret_cast<uintptr_t>(shift) | reinterpret_cast<uintptr_t>(out)) & 15u) == 0;
+    uint32_t rc;
+    if (rows > 0 && nidx > 0 && table && indices && scale && shift && out && aligned && dim % 8 == 0 && dim > 0 &&
+        dim < 256 &&
+        launch_family_region(2, block_dim, stream, {table, indices, scale, shift, out}, workspace,
+                             {rows, dim, nidx, dim, dim, nidx, dim}, &rc))
+      return rc;
+  }
   return finish(afir::launch_gather_scale_shift(
       static_cast<const uint16_t *>(table), static_cast<const int32_t *>(indices),
       static_cast<const uint16_t *>(scale), static_cast<const uint16_t *>(shift),
@@ -424,7 +476,18 @@ uint32_t afir_hip_probe_mfma_rate(void *stream, const void *operands, void *sink
                                              static_cast<hipStream_t>(stream)));
 }
 
+namespace {
+uint32_t register_region(const char *program_text, size_t program_len, uint64_t *handle, bool generic);
+}
+
 uint32_t afir_hip_region_register(const char *program_text, size_t program_len, uint64_t *handle) {
+  bool generic = false;
+  if (const char *env = std::getenv("AFIR_HIP_REGION_GENERIC")) generic = *env && *env != '0';
+  return register_region(program_text, program_len, handle, generic);
+}
+
+namespace {
+uint32_t register_region(const char *program_text, size_t program_len, uint64_t *handle, bool generic) {
   if (!program_text || !handle) return fail(AFIR_HIP_E_INVALID, "region_register: null argument");
   auto r = std::make_shared<RegisteredRegion>();
   std::string why = afir_region::parse(std::string(program_text, program_len), &r->program);
@@ -432,15 +495,72 @@ uint32_t afir_hip_region_register(const char *program_text, size_t program_len, 
   r->fields = afir_region::tilingFieldNames(r->program);
   why = detect_fast_path(r.get());
   if (!why.empty()) return fail(AFIR_HIP_E_INVALID, why);
-  if (const char *env = std::getenv("AFIR_HIP_REGION_GENERIC"))
-    if (*env && *env != '0' && r->fast != FastPath::MatmulBiasLeaky && r->fast != FastPath::MatmulBiasLeakyF16)
-      r->fast = FastPath::None;
+  if (generic && r->fast != FastPath::MatmulBiasLeaky && r->fast != FastPath::MatmulBiasLeakyF16)
+    r->fast = FastPath::None;
   std::lock_guard<std::mutex> lock(g_region_mutex);
   *handle = g_next_region++;
   g_regions[*handle] = std::move(r);
   g_last_error.clear();
   return AFIR_HIP_OK;
 }
+
+// ---- the families' compiled form: lib/families/<family>.hsaco beside this library ----
+struct FamilyRegion {
+  const char *name;
+  const char *program;
+  std::once_flag once;
+  uint64_t handle = 0;
+  bool usable = false;
+};
+FamilyRegion g_families[] = {
+    {"broadcast_add_reducesum", afir_family::kBroadcastAddReducesum},
+    {"relu_broadcast_add_transpose", afir_family::kReluBroadcastAddTranspose},
+    {"gather_scale_shift", afir_family::kGatherScaleShift},
+};
+
+FamilyRegion *family_region(int which) {
+  FamilyRegion &f = g_families[which];
+  std::call_once(f.once, [&f] {
+    if (const char *env = std::getenv("AFIR_HIP_FAMILY_FALLBACK"))
+      if (*env == '0') return;
+    Dl_info info;
+    if (!dladdr(reinterpret_cast<const void *>(&afir_hip_kernel_count), &info) || !info.dli_fname) return;
+    std::string dir(info.dli_fname);
+    const size_t slash = dir.rfind('/');
+    dir = slash == std::string::npos ? std::string(".") : dir.substr(0, slash);
+    std::ifstream file(dir + "/families/" + f.name + ".hsaco", std::ios::binary);
+    if (!file) return;
+    const std::vector<char> image((std::istreambuf_iterator<char>(file)), std::istreambuf_iterator<char>());
+    uint64_t h = 0;
+    if (register_region(f.program, std::strlen(f.program), &h, /*generic=*/true) != AFIR_HIP_OK) return;
+    if (afir_hip_region_attach_code_object(h, image.data(), image.size()) != AFIR_HIP_OK) {
+      (void)afir_hip_region_unregister(h);
+      return;
+    }
+    f.handle = h;
+    f.usable = true;
+  });
+  return f.usable ? &f : nullptr;
+}
+
+// Runs a family's launch on its compiled region kernels.  False: not available (no code
+// object was built, or it does not load); the caller goes on with the family's own kernels.
+bool launch_family_region(int which, uint32_t block_dim, void *stream, std::initializer_list<void *> args,
+                          void *workspace, std::initializer_list<int64_t> dims, uint32_t *rc) {
+  FamilyRegion *f = family_region(which);
+  if (!f) return false;
+  std::vector<void *> a(args);
+  std::vector<int64_t> t(dims);
+  *rc = afir_hip_launch_region(f->handle, block_dim, stream, (int)a.size(), a.data(), workspace, t.data(),
+                               t.size() * sizeof(int64_t));
+  if (*rc == AFIR_HIP_E_LAUNCH) {   // e.g. a code object of another version: do without it from now on
+    f->usable = false;
+    g_last_error.clear();
+    return false;
+  }
+  return true;
+}
+}  // namespace
 
 uint32_t afir_hip_region_unregister(uint64_t handle) {
   std::lock_guard<std::mutex> lock(g_region_mutex);
@@ -880,6 +1000,13 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
 }
 
 int afir_hip_kernel_count(void) { return kNumKernels; }
+
+const char *afir_hip_family_program(const char *family) {
+  if (!family) return nullptr;
+  for (const FamilyRegion &f : g_families)
+    if (std::strcmp(f.name, family) == 0) return f.program;
+  return nullptr;
+}
 
 const AfirHipKernelInfo *afir_hip_kernel_info(int index) {
   if (index < 0 || index >= kNumKernels) return nullptr;

@@ -136,6 +136,13 @@ typedef struct AfirHipKernelInfo {
 } AfirHipKernelInfo;
 
 int afir_hip_kernel_count(void);
+/* The family as a region program (text), or NULL when it has none (the matmul and the
+ * plain add-mul chain).  The library's build compiles these programs to
+ * lib/families/<family>.hsaco; a family launcher whose specialised kernels do not fit the
+ * shapes of a launch (rows that are no multiple of the tile, short rows, few rows) runs it
+ * on those kernels.  AFIR_HIP_FAMILY_FALLBACK=0 keeps every launch on the family's own
+ * kernels.  No counterpart in the reference: its kernels are generated per graph. */
+const char *afir_hip_family_program(const char *family);
 const AfirHipKernelInfo *afir_hip_kernel_info(int index);
 const AfirHipKernelInfo *afir_hip_find_kernel(const char *name);
 

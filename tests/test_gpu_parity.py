@@ -93,7 +93,9 @@ def _check_rowsum(x, bias, y):
 
 
 @pytest.mark.parametrize("m,n", [(1, 4), (7, 5), (33, 4096), (64, 512), (5, 1000),
-                                 (130, 1028), (3, 8192), (2, 100000)])
+                                 (130, 1028), (3, 8192), (2, 100000),
+                                 # short rows and few long rows: the family's compiled region kernels
+                                 (5000, 100), (3000, 8), (2, 8 * 4096), (70, 24 * 4096), (1500, 2044)])
 def test_c2_small(H, m, n):
     x, bias = O.gen_c2(m, n)
     y = H.broadcast_add_reducesum(dev(x), dev(bias)).cpu().numpy()
@@ -130,7 +132,9 @@ def test_c2_exact_integer_rows_and_blockdim(H):
 # ---------------------------------------------------------------- C3 --------
 
 @pytest.mark.parametrize("b,m,n", [(2, 3, 5), (1, 128, 128), (3, 256, 128), (2, 128, 384),
-                                   (3, 70, 36), (1, 1, 1), (2, 129, 128), (1, 33, 250)])
+                                   (3, 70, 36), (1, 1, 1), (2, 129, 128), (1, 33, 250),
+                                   # multiples of 8 that are not whole tiles: the family's compiled region kernels
+                                   (2, 72, 136), (3, 1024, 520), (1, 200, 64), (2, 64, 72)])
 def test_c3_small_bit_exact(H, b, m, n):
     x, c = O.gen_c3(b, m, n)
     out = H.relu_broadcast_add_transpose(dev(x), dev(c)).cpu().numpy()
@@ -178,7 +182,9 @@ def test_c3_special_values(H):
 
 @pytest.mark.parametrize("rows,dim,nidx", [(512, 64, 256), (1000, 1024, 513), (100, 136, 77),
                                            (64, 8, 5), (300, 2048, 40), (50, 100, 33),
-                                           (10, 1, 7), (128, 1536, 19)])
+                                           (10, 1, 7), (128, 1536, 19),
+                                           # rows of fewer than 256 halves: the family's compiled region kernels
+                                           (4096, 64, 30000), (777, 248, 1001), (9, 16, 100000)])
 def test_c4_small_bit_exact(H, rows, dim, nidx):
     table, idx, scale, shift = O.gen_c4(rows, dim, nidx)
     idx[:3] = [0, rows - 1, rows - 1]
