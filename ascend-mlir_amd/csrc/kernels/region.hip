@@ -433,23 +433,29 @@ __global__ __launch_bounds__(kThreads) void fused_region_parallel(const RegionAr
   }
 }
 
-// Row sum over the innermost dim: one wavefront per output element, lanes
-// stride over the row in vectors of 8, float32 partial sums per vector slot,
-// fixed-order combination and a DPP wave reduction: deterministic.
+// Row sum over the innermost dim: 2^lanes_log2 lanes of a wavefront per output
+// element (the whole wavefront for rows of 64 vectors or more, fewer lanes and
+// several rows per wavefront for shorter rows), the lanes stride over the row in
+// vectors of V, float32 partial sums per vector slot, fixed-order combination
+// and a DPP wave reduction or a butterfly over the row's lanes: deterministic.
 template <typename I, bool CHAIN, int V>
-__global__ __launch_bounds__(kThreads) void fused_region_rowsum(const RegionArgs R) {
+__global__ __launch_bounds__(kThreads) void fused_region_rowsum(const RegionArgs R, int lanes_log2) {
   const int last = R.rank - 1;
   const I n = (I)R.size[last];
   const I chunks = (n + V - 1) / V;
   const I rows = (I)((R.rank == 2) ? R.size[0] : R.size[0] * R.size[1]);
   const int lane = threadIdx.x & (kWave - 1);
+  const int lanes = 1 << lanes_log2;
+  const I rows_per_wave = (I)(kWave >> lanes_log2);
   const I wave = (I)blockIdx.x * (kThreads / kWave) + (I)(threadIdx.x >> 6);
   const I nwaves = (I)gridDim.x * (kThreads / kWave);
-  for (I row = wave; row < rows; row += nwaves) {
+  for (I row0 = wave * rows_per_wave; row0 < rows; row0 += nwaves * rows_per_wave) {
+    const I row = row0 + (I)(lane >> lanes_log2);
+    if (row >= rows) continue;   // the lanes of a row leave together
     float acc[V];
 #pragma unroll
     for (int e = 0; e < V; ++e) acc[e] = 0.f;
-    for (I c = lane; c < chunks; c += kWave) {
+    for (I c = lane & (lanes - 1); c < chunks; c += lanes) {
       const I j0 = c * V;
       const I left = n - j0;
       const int nvalid = left >= V ? V : (int)left;
@@ -464,8 +470,12 @@ __global__ __launch_bounds__(kThreads) void fused_region_rowsum(const RegionArgs
 #pragma unroll
       for (int e = 0; e < w; ++e) acc[e] = acc[2 * e] + acc[2 * e + 1];
     float s = acc[0];
-    s = wave_sum(s);
-    if (lane == 0) store_elem(R.out, R.out_type, (int64_t)row, s);
+    if (lanes_log2 == 6) {
+      s = wave_sum(s);
+    } else {
+      for (int m = lanes >> 1; m >= 1; m >>= 1) s += __shfl_xor(s, m);
+    }
+    if ((lane & (lanes - 1)) == 0) store_elem(R.out, R.out_type, (int64_t)row, s);
   }
 }
 
@@ -586,11 +596,17 @@ LaunchStatus plan_fused_region(const RegionArgs &args, int vec, uint32_t block_d
     g->empty = rows == 0;
     if (g->empty) return ok_status();
     if (!args.out) return invalid("fused_region: null output pointer");
-    int64_t blocks = (rows + (kThreads / kWave) - 1) / (kThreads / kWave);
-    // up to 64 rows (waves) per CU at a time; 16 and more measured 3 % above 8 on 16384 rows of f16
+    // lanes of a wavefront that share a row: enough to cover a short row in one pass
+    const int64_t row_chunks = (args.size[args.rank - 1] + vec - 1) / vec;
+    int ll = 0;
+    while (ll < 6 && ((int64_t)1 << ll) < row_chunks) ++ll;
+    const int64_t rows_per_block = (int64_t)(kThreads / kWave) * (kWave >> ll);
+    int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
+    // up to 64 waves per CU at a time; 16 and more measured 3 % above 8 on 16384 rows of f16
     if (blocks > (int64_t)kNumCU * 16) blocks = (int64_t)kNumCU * 16;
     if (block_dim) blocks = block_dim;
     g->blocks = blocks;
+    g->lanes_log2 = ll;
     return ok_status();
   }
   g->empty = total == 0;
@@ -666,7 +682,7 @@ LaunchStatus launch_fused_region(const RegionArgs &args_in, uint32_t block_dim, 
     auto kernel = wide ? (idx32 ? fused_region_rowsum<int, true, 16> : fused_region_rowsum<int64_t, true, 16>)
                   : args.chain ? (idx32 ? fused_region_rowsum<int, true, 8> : fused_region_rowsum<int64_t, true, 8>)
                                : (idx32 ? fused_region_rowsum<int, false, 8> : fused_region_rowsum<int64_t, false, 8>);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)g.blocks), dim3(kThreads), 0, stream, args);
+    hipLaunchKernelGGL(kernel, dim3((unsigned)g.blocks), dim3(kThreads), 0, stream, args, g.lanes_log2);
     return after_launch();
   }
   auto kernel = wide ? (idx32 ? fused_region_parallel<int, true, 16> : fused_region_parallel<int64_t, true, 16>)
