@@ -747,6 +747,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
     int rows;    // 1: the workgroup-per-row kernel of a reduce segment, 2: its form for few, long rows,
                  // 3: split (args.column_blocks workgroups per row) and join, for a handful of rows
     bool slim;   // the kernel whose lanes take one group each (short rows)
+    bool elem;   // the kernel whose groups are single elements (rows off 16-byte boundaries)
   };
   std::vector<PendingSegment> pending;   // compiled kernels to launch, non-empty segments only
   for (const afir_region::ResolvedSegment &seg : res.segments) {
@@ -802,14 +803,19 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
       const int segment = (int)(&seg - res.segments.data());
       const afir_target::SpecShape shape = afir_target::specShape(r->program, segment, emit);
       const afir_target::SpecTile tile = afir_target::specTile(r->program, segment);
-      const int W = shape.width;
+      const int wideW = shape.width;
       // Rows of fewer than 8 x unroll groups leave most of a lane's groups empty and make a wavefront's
       // loads touch short pieces of many rows: those run on the kernel whose lanes take one group each
       // (it exists with 32-bit positions, for launches whose 128-bit accesses are all aligned).
-      const int64_t row_groups_all = (seg.size[seg.rank - 1] + W - 1) / W;
+      const int64_t row_groups_all = (seg.size[seg.rank - 1] + wideW - 1) / wideW;
       bool skip = false;
       uint32_t failed = AFIR_HIP_OK;
-      auto prepare = [&](const int U, const bool slim, PendingSegment *made) -> bool {
+      bool unaligned = false;   // set by a pass: some tensor's rows are off 16-byte boundaries
+      // kind 0: the ordinary kernels; 1: one group per lane; 2: single-element groups
+      auto prepare = [&](const int kind, PendingSegment *made) -> bool {
+        const int W = kind == 2 ? 1 : wideW;
+        const int U = kind == 2 ? afir_target::kSpecElementUnroll : kind == 1 ? 1 : shape.unroll;
+        const bool slim = kind == 1;
         afir::RegionGeometry g;
         uint32_t rc = finish(afir::plan_fused_region(a, W * U, block_dim, &g));
         if (rc != AFIR_HIP_OK) { failed = rc; return false; }
@@ -859,6 +865,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
           }
           const int64_t per_pass = ((int64_t)1 << sa.lanes_log2) * U;
           vectors = seg.size[last] % W == 0 && (seg.reduce || a.out_vec);
+          if (!seg.reduce && !a.out_vec) unaligned = true;
           whole = groups % per_pass == 0;
           // a row that fills a workgroup of 256 lanes with U groups each: a workgroup per row
           if (!slim && seg.reduce && groups == (int64_t)256 * U) row_groups = 1;
@@ -902,10 +909,15 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
           }
           // operands that are contiguous along the innermost dim are read with
           // 128-bit loads by the aligned variant
-          if (d.stride[last] == 1 && d.gdim != last && (!d.vec || (d.gdim >= 0 && !d.gvec))) vectors = false;
+          if (d.stride[last] == 1 && d.gdim != last && (!d.vec || (d.gdim >= 0 && !d.gvec))) {
+            vectors = false;
+            unaligned = true;
+          }
         }
-        const int mode = vectors && whole ? afir_target::kSpecAligned
+        const int mode = kind == 2 ? afir_target::kSpecGeneral
+                         : vectors && whole ? afir_target::kSpecAligned
                          : vectors && !tile.tiled ? afir_target::kSpecVector : afir_target::kSpecGeneral;
+        if (kind == 2) row_groups = 0;
         if (row_groups == 3 && mode == afir_target::kSpecAligned) {
           int64_t nrows = 1;
           for (int k = 0; k < last; ++k) nrows *= seg.size[k];
@@ -923,13 +935,16 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
           row_groups = 0;
         }
         if (slim && (!g.idx32 || mode == afir_target::kSpecGeneral)) return false;
-        *made = PendingSegment{segment, sa, g.idx32, mode, row_groups, slim};
+        *made = PendingSegment{segment, sa, g.idx32, mode, row_groups, slim, kind == 2};
         return true;
       };
       PendingSegment made;
       bool ok = false;
-      if (!tile.tiled && shape.unroll > 1 && row_groups_all < (int64_t)8 * shape.unroll) ok = prepare(1, true, &made);
-      if (!ok && !skip && failed == AFIR_HIP_OK) ok = prepare(shape.unroll, false, &made);
+      if (!tile.tiled && shape.unroll > 1 && row_groups_all < (int64_t)8 * shape.unroll) ok = prepare(1, &made);
+      if (!ok && !skip && failed == AFIR_HIP_OK) ok = prepare(0, &made);
+      // rows off 16-byte boundaries: element accesses either way, so let consecutive lanes take
+      // consecutive elements
+      if (ok && !tile.tiled && unaligned && made.mode == afir_target::kSpecGeneral && !made.slim) ok = prepare(2, &made);
       if (failed != AFIR_HIP_OK) return failed;
       if (ok) pending.push_back(made);
       continue;
@@ -953,7 +968,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
     bool together = pending.size() > 1 && nseg <= afir_target::kSpecMaxSegments;
     int64_t total = 0;
     for (const PendingSegment &p : pending) {
-      together = together && p.idx32 == pending[0].idx32 && p.mode == pending[0].mode && !p.rows && !p.slim;
+      together = together && p.idx32 == pending[0].idx32 && p.mode == pending[0].mode && !p.rows && !p.slim && !p.elem;
       total += p.args.grid;
     }
     if (together && total <= 0x7fffffff) {
@@ -988,6 +1003,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
         }
         const uint32_t rc = launch(p.rows == 2 ? afir_target::specLongRowsKernelName(p.segment, p.idx32)
                                    : p.rows ? afir_target::specRowsKernelName(p.segment, p.idx32)
+                                   : p.elem ? afir_target::specElementKernelName(p.segment, p.idx32)
                                    : p.slim ? afir_target::specSlimKernelName(p.segment, p.mode)
                                             : afir_target::specKernelName(p.segment, p.idx32, p.mode),
                                    &p.args, sizeof p.args, (unsigned)p.args.grid);

@@ -318,6 +318,19 @@ class SegmentEmitter {
         U_ = wide;
         hasSlim_ = true;
       }
+      {
+        // the same with one element per group, for tensors whose rows do not start on 16-byte
+        // boundaries: consecutive lanes take consecutive elements, so every load and store
+        // instruction of a wavefront still covers one contiguous run
+        const int wideU = U_, wideW = W_;
+        U_ = kSpecElementUnroll;
+        W_ = 1;
+        elem_ = true;
+        emitBody();
+        elem_ = false;
+        U_ = wideU;
+        W_ = wideW;
+      }
     }
     emitWrappers();
     return "";
@@ -491,15 +504,20 @@ class SegmentEmitter {
     if (o.step == Operand::Contiguous) {
       unroll();
       line(d, "for (int u = 0; u < U; ++u) {");
-      line(d + 1, "if (A || (full[u] && (V || vec" + u + "))) {");
-      line(d + 2, "ldv_" + tag + "<W, " + nt + ">(" + r + ".base, q" + u + " + j0[u], v" + u + "[u]);");
+      if (elem_) line(d + 1, "if (false) {");
+      else line(d + 1, "if (A || (full[u] && (V || vec" + u + "))) {");
+      if (!elem_) line(d + 2, "ldv_" + tag + "<W, " + nt + ">(" + r + ".base, q" + u + " + j0[u], v" + u + "[u]);");
       line(d + 1, "} else if (V) {");
       unroll();
       line(d + 2, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = " + zero() + ";");
       line(d + 1, "} else {");
       unroll();
-      line(d + 2, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = e < nvalid[u] ? " + ld(o.type) + "(" + r + ".base, q" + u +
-                      " + j0[u] + e) : " + zero() + ";");
+      // unconditional loads (of the row's last element where the lane has none), then a select:
+      // a load under a branch would be waited for before the next one is issued
+      line(d + 2, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = " + ld(o.type) + "(" + r + ".base, q" + u +
+                      " + (e < nvalid[u] ? j0[u] + e : n - 1));");
+      unroll();
+      line(d + 2, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = e < nvalid[u] ? v" + u + "[u][e] : " + zero() + ";");
       line(d + 1, "}");
       line(d, "}");
     } else {
@@ -509,12 +527,15 @@ class SegmentEmitter {
       line(d + 1, "const long long step = " + r + ".stride[" + std::to_string(last_) + "];");
       unroll();
       line(d + 1, "for (int u = 0; u < U; ++u) {");
-      line(d + 2, "if (step == 1 && (A || (full[u] && (V || vec" + u + ")))) {");
-      line(d + 3, "ldv_" + tag + "<W, " + nt + ">(" + r + ".base, q" + u + " + j0[u], v" + u + "[u]);");
+      if (elem_) line(d + 2, "if (false) {");
+      else line(d + 2, "if (step == 1 && (A || (full[u] && (V || vec" + u + ")))) {");
+      if (!elem_) line(d + 3, "ldv_" + tag + "<W, " + nt + ">(" + r + ".base, q" + u + " + j0[u], v" + u + "[u]);");
       line(d + 2, "} else {");
       unroll();
-      line(d + 3, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = e < nvalid[u] ? " + ld(o.type) + "(" + r + ".base, q" + u +
-                      " + ((long long)j0[u] + e) * step) : " + zero() + ";");
+      line(d + 3, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = " + ld(o.type) + "(" + r + ".base, q" + u +
+                      " + (long long)(e < nvalid[u] ? j0[u] + e : n - 1) * step);");
+      unroll();
+      line(d + 3, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = e < nvalid[u] ? v" + u + "[u][e] : " + zero() + ";");
       line(d + 2, "}");
       line(d + 1, "}");
       line(d, "}");
@@ -684,10 +705,10 @@ class SegmentEmitter {
     os_ << "\n// ---- segment " << index_ << ": iteration rank " << rank_
         << (reduce_ ? ", row sum over the innermost dim" : ", parallel") << "; a lane takes " << U_
         << (U_ == 1 ? " group of " : " groups of ") << W_ << " elements per pass"
-        << (slim_ ? " (for rows of few groups)" : "") << " ----\n";
+        << (slim_ ? " (for rows of few groups)" : elem_ ? " (for unaligned rows)" : "") << " ----\n";
     os_ << "// I: position type.  M: 2 = every 128-bit access is aligned and every pass is whole (no tail);\n";
     os_ << "// 1 = aligned and the innermost extent a multiple of W, passes may be partly empty; 0 = anything.\n";
-    os_ << "template <typename I, int M>\nDEV void segment" << index_ << (slim_ ? "_slim" : "")
+    os_ << "template <typename I, int M>\nDEV void segment" << index_ << (slim_ ? "_slim" : elem_ ? "_elem" : "")
         << "(const SpecArgs &R, const I bid, const I nblocks) {\n";
     line(1, "constexpr int W = " + std::to_string(W_) + ", U = " + std::to_string(U_) + ";");
     line(1, "constexpr bool A = M == 2, V = M >= 1;");
@@ -769,8 +790,9 @@ class SegmentEmitter {
     unroll();
     line(3, "for (int u = 0; u < U; ++u) {");
     line(4, "const long long o = (long long)row * (long long)n + (long long)j0[u];");
-    line(4, "if (A || (full[u] && (V || R.out_vec))) {");
-    line(5, "stv_" + otag + "<W>(R.out, o, " + res + "[u]);");
+    if (elem_) line(4, "if (false) {");
+    else line(4, "if (A || (full[u] && (V || R.out_vec))) {");
+    if (!elem_) line(5, "stv_" + otag + "<W>(R.out, o, " + res + "[u]);");
     line(4, "} else if (!V) {");
     unroll();
     line(5, "for (int e = 0; e < W; ++e)");
@@ -1154,6 +1176,11 @@ class SegmentEmitter {
             << ">(R, (" << (i32 ? "int" : "long long") << ")__builtin_amdgcn_workgroup_id_x(), ("
             << (i32 ? "int" : "long long") << ")R.grid); }\n";
       }
+    if (!tiled())
+      for (int i32 = 1; i32 >= 0; --i32)
+        os_ << "KERNEL void " << specElementKernelName(index_, i32 != 0) << "(const SpecArgs R) { segment" << index_
+            << "_elem<" << (i32 ? "int" : "long long") << ", 0>(R, (" << (i32 ? "int" : "long long")
+            << ")__builtin_amdgcn_workgroup_id_x(), (" << (i32 ? "int" : "long long") << ")R.grid); }\n";
     if (hasSlim_)
       for (int mode = kSpecAligned; mode >= kSpecVector; --mode)
         os_ << "KERNEL void " << specSlimKernelName(index_, mode) << "(const SpecArgs R) { segment" << index_
@@ -1190,6 +1217,7 @@ class SegmentEmitter {
   bool integer_ = false;   // 32-bit integers instead of float32 values
   bool narrow_ = false;    // ... of which the low 16 bits are the value (i16 output)
   bool slim_ = false;      // emitting the one-group-per-lane form of the segment
+  bool elem_ = false;      // emitting the one-element-per-group form (no 128-bit accesses)
   bool hasSlim_ = false;   // ... which exists for this segment
   bool hoisted_ = false;   // row invariants and operand values are assigned, not declared
   bool keepRowConstants_ = false;   // ... and operands that are the same for every row are left alone
@@ -1291,6 +1319,10 @@ std::string specSplitRowsKernelName(int segment, bool idx32, bool join) {
 
 std::string specLongRowsKernelName(int segment, bool idx32) {
   return "afir_region_s" + std::to_string(segment) + "_long" + (idx32 ? "_i32" : "_i64");
+}
+
+std::string specElementKernelName(int segment, bool idx32) {
+  return "afir_region_s" + std::to_string(segment) + "_elem" + (idx32 ? "_i32" : "_i64");
 }
 
 std::string specSlimKernelName(int segment, int mode) {

@@ -104,7 +104,7 @@ uint64_t programHash(const afir_region::Program &p);
 // Version of the set of kernels and of the launch arguments that emitHipSource produces; the
 // code object exports it as `afir_region_emit_abi`, and a code object of another version is
 // refused when it is loaded (its kernels would be launched with the wrong names or arguments).
-constexpr int kSpecAbiVersion = 4;
+constexpr int kSpecAbiVersion = 5;
 
 // What a launch promises, which picks the kernel variant:
 //   kSpecAligned  every 128-bit access is aligned and every pass of the lanes over a row is whole
@@ -117,6 +117,11 @@ std::string specKernelName(int segment, bool idx32, int mode);
 // Untiled segments also have kernels whose lanes take one group each, for rows of
 // fewer than 8 x unroll groups (32-bit positions, modes kSpecAligned and kSpecVector).
 std::string specSlimKernelName(int segment, int mode);
+// ... and kernels whose groups are single elements (kSpecElementUnroll of them per lane, a
+// lane-set apart), launched when rows do not start on 16-byte boundaries: every load and
+// store instruction of a wavefront then still covers one contiguous run.
+constexpr int kSpecElementUnroll = 8;
+std::string specElementKernelName(int segment, bool idx32);
 // Reduce segments also have a workgroup-per-row kernel for rows of exactly
 // 256 * unroll * width elements whose accesses are all 128-bit.
 std::string specRowsKernelName(int segment, bool idx32);
