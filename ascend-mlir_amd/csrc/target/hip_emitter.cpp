@@ -1116,9 +1116,14 @@ class SegmentEmitter {
       line(4, "if (A || (vec" + u + " && q < n && tile_p + (I)(lp + EL) <= np)) {");
       line(5, "ldv_" + tag + "<EL, " + (o.readOnce ? "true" : "false") + ">(" + rr + ".base, pos + (long long)q * sq, vals[s]);");
       line(4, "} else {");
+      line(5, "// unconditional loads, of the last element inside where the position is outside, then a select");
+      line(5, "const I qc = q < n ? q : n - 1;");
       unroll();
       line(5, "for (int e = 0; e < EL; ++e)");
-      line(6, "vals[s][e] = (q < n && tile_p + (I)(lp + e) < np) ? " + ld(o.type) + "(" + rr + ".base, pos + (long long)q * sq + e) : " + zero() + ";");
+      line(6, "vals[s][e] = " + ld(o.type) + "(" + rr + ".base, pos + (long long)qc * sq + (tile_p + (I)(lp + e) < np ? (long long)e : (long long)(np - 1) - (long long)(tile_p + (I)lp)));");
+      unroll();
+      line(5, "for (int e = 0; e < EL; ++e)");
+      line(6, "vals[s][e] = (q < n && tile_p + (I)(lp + e) < np) ? vals[s][e] : " + zero() + ";");
       line(4, "}");
       line(3, "}");
       unroll();
