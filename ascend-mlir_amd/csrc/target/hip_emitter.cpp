@@ -475,27 +475,30 @@ class SegmentEmitter {
     }
     const std::string nan = bad();
     if (o.gatherDim == last_) {
-      // one index per element
+      // one index per element.  Branch-free: every index is requested, then every element (at
+      // index 0 where the index is out of range, at the row's last position where the lane
+      // has none), then selects -- loads under branches would be issued one at a time
       line(d, "{");
       line(d + 1, std::string("const long long step = ") +
                       (o.step == Operand::Broadcast ? "0" : r + ".stride[" + std::to_string(last_) + "]") + ";");
+      line(d + 1, "long long gi[U][W];");
       unroll();
-      line(d + 1, "for (int u = 0; u < U; ++u) {");
+      line(d + 1, "for (int u = 0; u < U; ++u)");
+      unroll();
+      line(d + 2, "for (int e = 0; e < W; ++e)");
+      line(d + 3, "gi[u][e] = ld_" + std::string(typeTag(o.gatherType)) + "(" + r + ".index, (long long)(e < nvalid[u] ? j0[u] + e : n - 1));");
+      line(d + 1, "bool any_bad = false;");
+      unroll();
+      line(d + 1, "for (int u = 0; u < U; ++u)");
       unroll();
       line(d + 2, "for (int e = 0; e < W; ++e) {");
-      line(d + 3, ct() + " x = " + zero() + ";");
-      line(d + 3, "if (e < nvalid[u]) {");
-      line(d + 4, "const long long g = ld_" + std::string(typeTag(o.gatherType)) + "(" + r + ".index, (long long)j0[u] + e);");
-      line(d + 4, "if (g < 0 || g >= " + r + ".gextent) {");
-      line(d + 5, "if (R.error_flag) *R.error_flag = 1;");
-      line(d + 5, "x = " + nan + ";");
-      line(d + 4, "} else {");
-      line(d + 5, "x = " + ld(o.type) + "(" + r + ".base, q" + u + " + ((long long)j0[u] + e) * step + g * " + r + ".gstride);");
-      line(d + 4, "}");
-      line(d + 3, "}");
-      line(d + 3, "v" + u + "[u][e] = x;");
+      line(d + 3, "const bool bad = gi[u][e] < 0 || gi[u][e] >= " + r + ".gextent;");
+      line(d + 3, "any_bad = any_bad || (bad && e < nvalid[u]);");
+      line(d + 3, "const " + ct() + " x = " + ld(o.type) + "(" + r + ".base, q" + u +
+                      " + (long long)(e < nvalid[u] ? j0[u] + e : n - 1) * step + (bad ? 0 : gi[u][e]) * " + r + ".gstride);");
+      line(d + 3, "v" + u + "[u][e] = e < nvalid[u] ? (bad ? " + nan + " : x) : " + zero() + ";");
       line(d + 2, "}");
-      line(d + 1, "}");
+      line(d + 1, "if (any_bad && R.error_flag) *R.error_flag = 1;");
       line(d, "}");
       return v;
     }
