@@ -812,20 +812,20 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
       uint32_t failed = AFIR_HIP_OK;
       bool unaligned = false;   // set by a pass: some tensor's rows are off 16-byte boundaries
       // kind 0: the ordinary kernels; 1: one group per lane; 2: single-element groups
-      auto prepare = [&](const int kind, PendingSegment *made) -> bool {
+      auto prepare = [&](const afir::RegionArgs &ra, const int kind, PendingSegment *made) -> bool {
         const int W = kind == 2 ? 1 : wideW;
         const int U = kind == 2 ? afir_target::kSpecElementUnroll : kind == 1 ? 1 : shape.unroll;
         const bool slim = kind == 1;
         afir::RegionGeometry g;
-        uint32_t rc = finish(afir::plan_fused_region(a, W * U, block_dim, &g));
+        uint32_t rc = finish(afir::plan_fused_region(ra, W * U, block_dim, &g));
         if (rc != AFIR_HIP_OK) { failed = rc; return false; }
         if (g.empty) { skip = true; return false; }
         afir_target::SpecArgs sa;
         std::memset(&sa, 0, sizeof sa);
-        for (int k = 0; k < 3; ++k) sa.size[k] = a.size[k];
-        sa.out = a.out;
-        sa.error_flag = a.error_flag;
-        sa.out_vec = a.out_vec;
+        for (int k = 0; k < 3; ++k) sa.size[k] = ra.size[k];
+        sa.out = ra.out;
+        sa.error_flag = ra.error_flag;
+        sa.out_vec = ra.out_vec;
         sa.lanes_log2 = g.lanes_log2;
         sa.grid = (int)g.blocks;
         sa.column_blocks = (int)g.column_blocks;
@@ -834,29 +834,29 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
         int row_groups = 0;
         if (tile.tiled) {
           // one workgroup pass per tile of tile_p x tile_q
-          const int64_t tq = (seg.size[last] + emit.tileQ - 1) / emit.tileQ;
-          const int64_t tp = (seg.size[tile.dim] + emit.tileP - 1) / emit.tileP;
+          const int64_t tq = (ra.size[last] + emit.tileQ - 1) / emit.tileQ;
+          const int64_t tp = (ra.size[tile.dim] + emit.tileP - 1) / emit.tileP;
           int64_t tiles = tq * tp;
           for (int k = 0; k < last; ++k)
-            if (k != tile.dim) tiles *= seg.size[k];
+            if (k != tile.dim) tiles *= ra.size[k];
           int64_t blocks = tiles < (int64_t)afir::kNumCU * 256 ? tiles : (int64_t)afir::kNumCU * 256;
           if (block_dim) blocks = block_dim;
           sa.grid = (int)blocks;
           sa.column_blocks = 1;
-          vectors = a.out_vec != 0;
-          whole = seg.size[last] % emit.tileQ == 0 && seg.size[tile.dim] % emit.tileP == 0;
+          vectors = ra.out_vec != 0;
+          whole = ra.size[last] % emit.tileQ == 0 && ra.size[tile.dim] % emit.tileP == 0;
         } else {
           // the aligned variant has no tail handling: whole groups, whole passes
-          const int64_t groups = seg.size[last] / W;
+          const int64_t groups = ra.size[last] / W;
           if (seg.reduce) {
             // lanes of a wavefront that share a row: enough for one pass over a short row, the wavefront otherwise
-            const int64_t all_groups = (seg.size[last] + W - 1) / W;
+            const int64_t all_groups = (ra.size[last] + W - 1) / W;
             int ll = 0;
             while (ll < 6 && ((int64_t)U << ll) < all_groups) ++ll;
             sa.lanes_log2 = ll;
             if (!block_dim) {
               int64_t nrows = 1;
-              for (int k = 0; k < last; ++k) nrows *= seg.size[k];
+              for (int k = 0; k < last; ++k) nrows *= ra.size[k];
               const int64_t rows_per_block = (int64_t)4 * (64 >> ll);
               int64_t blocks = (nrows + rows_per_block - 1) / rows_per_block;
               if (blocks > (int64_t)afir::kNumCU * 16) blocks = (int64_t)afir::kNumCU * 16;
@@ -864,14 +864,14 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
             }
           }
           const int64_t per_pass = ((int64_t)1 << sa.lanes_log2) * U;
-          vectors = seg.size[last] % W == 0 && (seg.reduce || a.out_vec);
-          if (!seg.reduce && !a.out_vec) unaligned = true;
+          vectors = ra.size[last] % W == 0 && (seg.reduce || ra.out_vec);
+          if (!seg.reduce && !ra.out_vec) unaligned = true;
           whole = groups % per_pass == 0;
           // a row that fills a workgroup of 256 lanes with U groups each: a workgroup per row
           if (!slim && seg.reduce && groups == (int64_t)256 * U) row_groups = 1;
           // few rows of several such stretches: a workgroup per row as well, pass by pass
           int64_t nrows_all = 1;
-          for (int k = 0; k < last; ++k) nrows_all *= seg.size[k];
+          for (int k = 0; k < last; ++k) nrows_all *= ra.size[k];
           if (!slim && seg.reduce && groups >= (int64_t)512 * U && groups % ((int64_t)256 * U) == 0 &&
               nrows_all < (int64_t)afir::kNumCU * 16)
             row_groups = 2;
@@ -886,8 +886,8 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
             }
           }
         }
-        for (int i = 0; i < a.ninputs; ++i) {
-          const afir::RegionInput &d = a.in[i];
+        for (int i = 0; i < ra.ninputs; ++i) {
+          const afir::RegionInput &d = ra.in[i];
           afir_target::SpecInput &t = sa.in[i];
           t.base = d.base;
           t.index = d.index;
@@ -902,7 +902,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
             const int64_t es = (int64_t)afir_region::elemTypeBytes(seg.inputs[i].type);
             bool tvec = aligned(d.base, d.offset * es);
             for (int k = 0; k < seg.rank; ++k)
-              if (k != tile.dim && seg.size[k] > 1 && (d.stride[k] * es) % 16 != 0) tvec = false;
+              if (k != tile.dim && ra.size[k] > 1 && (d.stride[k] * es) % 16 != 0) tvec = false;
             t.vec = tvec ? 1 : 0;
             if (!tvec) vectors = false;
             continue;
@@ -920,12 +920,12 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
         if (kind == 2) row_groups = 0;
         if (row_groups == 3 && mode == afir_target::kSpecAligned) {
           int64_t nrows = 1;
-          for (int k = 0; k < last; ++k) nrows *= seg.size[k];
+          for (int k = 0; k < last; ++k) nrows *= ra.size[k];
           sa.grid = (int)(nrows * sa.column_blocks);
         } else if (row_groups && mode == afir_target::kSpecAligned) {
           // up to 16 workgroups per CU walk the rows (4 to 16 measured within 1 %, 2 slower)
           int64_t nrows = 1;
-          for (int k = 0; k < last; ++k) nrows *= seg.size[k];
+          for (int k = 0; k < last; ++k) nrows *= ra.size[k];
           int64_t blocks = nrows < (int64_t)afir::kNumCU * 16 ? nrows : (int64_t)afir::kNumCU * 16;
           if (block_dim) blocks = block_dim;
           sa.grid = (int)blocks;
@@ -940,11 +940,38 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
       };
       PendingSegment made;
       bool ok = false;
-      if (!tile.tiled && shape.unroll > 1 && row_groups_all < (int64_t)8 * shape.unroll) ok = prepare(1, &made);
-      if (!ok && !skip && failed == AFIR_HIP_OK) ok = prepare(0, &made);
+      // A single row whose length is no multiple of the vector width (a rank-1 tensor, mostly): the
+      // whole vectors go to the aligned kernels and the last few elements to the element kernel, two
+      // launches, instead of everything to the general kernel.
+      const int64_t n_last = seg.size[seg.rank - 1];
+      // (only where the row is long enough for the second launch to be worth its few microseconds)
+      bool single_row = !tile.tiled && !seg.reduce && n_last >= (int64_t)1 << 18 && n_last % wideW != 0;
+      for (int k = 0; k + 1 < seg.rank; ++k) single_row = single_row && seg.size[k] == 1;
+      for (int i = 0; i < a.ninputs; ++i) single_row = single_row && a.in[i].gdim != seg.rank - 1;
+      if (single_row) {
+        afir::RegionArgs head = a, tail = a;
+        const int64_t whole_part = n_last - n_last % wideW;
+        head.size[seg.rank - 1] = whole_part;
+        tail.size[seg.rank - 1] = n_last - whole_part;
+        tail.out = static_cast<char *>(a.out) + whole_part * (int64_t)afir_region::elemTypeBytes(seg.outType);
+        for (int i = 0; i < a.ninputs; ++i) tail.in[i].offset += a.in[i].stride[seg.rank - 1] * whole_part;
+        PendingSegment first, second;
+        bool ok1 = whole_part / wideW < (int64_t)8 * shape.unroll && shape.unroll > 1 && prepare(head, 1, &first);
+        if (!ok1 && failed == AFIR_HIP_OK) ok1 = prepare(head, 0, &first);
+        const bool ok2 = ok1 && failed == AFIR_HIP_OK && first.mode != afir_target::kSpecGeneral && prepare(tail, 2, &second);
+        if (failed != AFIR_HIP_OK) return failed;
+        if (ok1 && ok2) {
+          pending.push_back(first);
+          pending.push_back(second);
+          continue;
+        }
+        skip = false;   // not this way: as one piece below
+      }
+      if (!tile.tiled && shape.unroll > 1 && row_groups_all < (int64_t)8 * shape.unroll) ok = prepare(a, 1, &made);
+      if (!ok && !skip && failed == AFIR_HIP_OK) ok = prepare(a, 0, &made);
       // rows off 16-byte boundaries: element accesses either way, so let consecutive lanes take
       // consecutive elements
-      if (ok && !tile.tiled && unaligned && made.mode == afir_target::kSpecGeneral && !made.slim) ok = prepare(2, &made);
+      if (ok && !tile.tiled && unaligned && made.mode == afir_target::kSpecGeneral && !made.slim) ok = prepare(a, 2, &made);
       if (failed != AFIR_HIP_OK) return failed;
       if (ok) pending.push_back(made);
       continue;
