@@ -748,6 +748,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
                  // 3: split (args.column_blocks workgroups per row) and join, for a handful of rows
     bool slim;   // the kernel whose lanes take one group each (short rows)
     bool elem;   // the kernel whose groups are single elements (rows off 16-byte boundaries)
+    unsigned lds = 0;   // > 0: the kernel that stages a gathered operand's source row, with this much LDS
   };
   std::vector<PendingSegment> pending;   // compiled kernels to launch, non-empty segments only
   for (const afir_region::ResolvedSegment &seg : res.segments) {
@@ -973,6 +974,26 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
       // consecutive elements
       if (ok && !tile.tiled && unaligned && made.mode == afir_target::kSpecGeneral && !made.slim) ok = prepare(a, 2, &made);
       if (failed != AFIR_HIP_OK) return failed;
+      // a gather along the innermost dim from contiguous, aligned source rows that fit the LDS: a
+      // workgroup per row stages the source row and gathers from there
+      if (ok && !made.slim && !made.elem && made.mode != afir_target::kSpecGeneral) {
+        const afir_target::SpecStage stage = afir_target::specStage(r->program, segment);
+        if (stage.input >= 0) {
+          const afir::RegionInput &d = a.in[stage.input];
+          const int64_t bytes = d.gextent * stage.elemBytes;
+          if (d.gstride == 1 && d.vec && bytes > 0 && bytes % 16 == 0 && bytes <= afir_target::kSpecStageBytes &&
+              seg.size[seg.rank - 1] >= (int64_t)128 * shape.unroll * wideW) {   // at least half a pass of the workgroup
+            int64_t blocks = seg.size[0] < (int64_t)afir::kNumCU * 16 ? seg.size[0] : (int64_t)afir::kNumCU * 16;
+            if (block_dim) blocks = block_dim;
+            made.args.grid = (int)blocks;
+            made.args.column_blocks = 1;
+            made.lds = (unsigned)bytes;
+            const int64_t per_pass = (int64_t)256 * shape.unroll;     // the whole workgroup on a row
+            if (made.mode == afir_target::kSpecAligned && (seg.size[seg.rank - 1] / wideW) % per_pass != 0)
+              made.mode = afir_target::kSpecVector;
+          }
+        }
+      }
       if (ok) pending.push_back(made);
       continue;
     }
@@ -980,12 +1001,12 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
     if (rc != AFIR_HIP_OK) return rc;
   }
   if (!pending.empty()) {
-    auto launch = [&](const std::string &name, void *args, size_t bytes, unsigned blocks) -> uint32_t {
+    auto launch = [&](const std::string &name, void *args, size_t bytes, unsigned blocks, unsigned lds = 0) -> uint32_t {
       hipFunction_t fn = nullptr;
       const std::string no = compiled_function(compiled.get(), r->program, name, &fn);
       if (!no.empty()) return fail(AFIR_HIP_E_LAUNCH, no);
       void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &bytes, HIP_LAUNCH_PARAM_END};
-      const hipError_t e = hipModuleLaunchKernel(fn, blocks, 1, 1, 256, 1, 1, 0, static_cast<hipStream_t>(stream),
+      const hipError_t e = hipModuleLaunchKernel(fn, blocks, 1, 1, 256, 1, 1, lds, static_cast<hipStream_t>(stream),
                                                  nullptr, config);
       if (e != hipSuccess) return fail(AFIR_HIP_E_LAUNCH, std::string("compiled region kernel: ") + hipGetErrorString(e));
       return AFIR_HIP_OK;
@@ -995,7 +1016,8 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
     bool together = pending.size() > 1 && nseg <= afir_target::kSpecMaxSegments;
     int64_t total = 0;
     for (const PendingSegment &p : pending) {
-      together = together && p.idx32 == pending[0].idx32 && p.mode == pending[0].mode && !p.rows && !p.slim && !p.elem;
+      together = together && p.idx32 == pending[0].idx32 && p.mode == pending[0].mode && !p.rows && !p.slim && !p.elem &&
+                 !p.lds;
       total += p.args.grid;
     }
     if (together && total <= 0x7fffffff) {
@@ -1025,6 +1047,12 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
           const int64_t nrows = p.args.grid / p.args.column_blocks;
           rc = launch(afir_target::specSplitRowsKernelName(p.segment, p.idx32, true), &p.args, sizeof p.args,
                       (unsigned)((nrows + 3) / 4));
+          if (rc != AFIR_HIP_OK) return rc;
+          continue;
+        }
+        if (p.lds) {
+          const uint32_t rc = launch(afir_target::specStagedKernelName(p.segment, p.idx32, p.mode), &p.args, sizeof p.args,
+                                     (unsigned)p.args.grid, p.lds);
           if (rc != AFIR_HIP_OK) return rc;
           continue;
         }

@@ -209,6 +209,17 @@ DEV float wave_sum(float v) {
   const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(iv, 48));
   return (r0 + r1) + (r2 + r3);
 }
+// ---- a source row staged in LDS (dynamic: the launch gives its size), read back by index
+extern __attribute__((shared)) __attribute__((aligned(16))) unsigned short afir_stage[];
+typedef __attribute__((address_space(3))) const float lds_f32;
+typedef __attribute__((address_space(3))) const int lds_i32;
+typedef __attribute__((address_space(3))) const short lds_i16;
+DEV float stage_f16(long long i) { return (float)__builtin_bit_cast(_Float16, afir_stage[i]); }
+DEV float stage_bf16(long long i) { return as_f32((unsigned)afir_stage[i] << 16); }
+DEV float stage_f32(long long i) { return ((lds_f32 *)afir_stage)[i]; }
+DEV int staged_i16(long long i) { return (int)((lds_i16 *)afir_stage)[i]; }
+DEV int staged_i32(long long i) { return ((lds_i32 *)afir_stage)[i]; }
+
 // ---- sum over aligned sets of `lanes` (a power of two below 64) lanes: butterfly, fixed order.
 // The lanes of a set are all active or all inactive.
 DEV float lanes_sum(float v, int lane, int lanes) {
@@ -318,6 +329,11 @@ class SegmentEmitter {
         U_ = wide;
         hasSlim_ = true;
       }
+      if (stageOperand_ >= 0) {
+        stage_ = true;
+        emitBody();
+        stage_ = false;
+      }
       {
         // the same with one element per group, for tensors whose rows do not start on 16-byte
         // boundaries: consecutive lanes take consecutive elements, so every load and store
@@ -397,10 +413,25 @@ class SegmentEmitter {
           o.tileSlot = tiles++;
         }
     numTiles_ = tiles;
+    // a gather along the innermost dim from rows of a matrix (the index tensor picks the column):
+    // the source row can be staged in LDS and gathered from there
+    stageOperand_ = -1;
+    if (!reduce_ && rank_ == 2 && tileDim_ < 0) {
+      int found = -1, count = 0;
+      for (size_t i = 0; i < operands_.size(); ++i)
+        if (operands_[i].gatherDim == last_) {
+          ++count;
+          found = (int)i;
+        }
+      if (count == 1 && operands_[found].usesDim[0] && operands_[found].step == Operand::Broadcast) stageOperand_ = found;
+    }
   }
 
  public:
   bool tiled() const { return tileDim_ >= 0; }
+  // SpecArgs::in slot of the operand whose source rows the staged kernels keep in LDS, else -1
+  int stagedSlot() const { return stageOperand_ < 0 ? -1 : operands_[stageOperand_].slot; }
+  ElemType stagedType() const { return stageOperand_ < 0 ? ElemType::F32 : operands_[stageOperand_].type; }
   int tileDim() const { return tileDim_; }
   unsigned tiledInputs() const {
     unsigned mask = 0;
@@ -494,8 +525,11 @@ class SegmentEmitter {
       line(d + 2, "for (int e = 0; e < W; ++e) {");
       line(d + 3, "const bool bad = gi[u][e] < 0 || gi[u][e] >= " + r + ".gextent;");
       line(d + 3, "any_bad = any_bad || (bad && e < nvalid[u]);");
-      line(d + 3, "const " + ct() + " x = " + ld(o.type) + "(" + r + ".base, q" + u +
-                      " + (long long)(e < nvalid[u] ? j0[u] + e : n - 1) * step + (bad ? 0 : gi[u][e]) * " + r + ".gstride);");
+      if (stage_ && &o == &operands_[stageOperand_])
+        line(d + 3, "const " + ct() + " x = " + std::string(integer_ ? "staged_" : "stage_") + tag + "(bad ? 0 : gi[u][e]);");
+      else
+        line(d + 3, "const " + ct() + " x = " + ld(o.type) + "(" + r + ".base, q" + u +
+                        " + (long long)(e < nvalid[u] ? j0[u] + e : n - 1) * step + (bad ? 0 : gi[u][e]) * " + r + ".gstride);");
       line(d + 3, "v" + u + "[u][e] = e < nvalid[u] ? (bad ? " + nan + " : x) : " + zero() + ";");
       line(d + 2, "}");
       line(d + 1, "if (any_bad && R.error_flag) *R.error_flag = 1;");
@@ -708,10 +742,11 @@ class SegmentEmitter {
     os_ << "\n// ---- segment " << index_ << ": iteration rank " << rank_
         << (reduce_ ? ", row sum over the innermost dim" : ", parallel") << "; a lane takes " << U_
         << (U_ == 1 ? " group of " : " groups of ") << W_ << " elements per pass"
-        << (slim_ ? " (for rows of few groups)" : elem_ ? " (for unaligned rows)" : "") << " ----\n";
+        << (slim_ ? " (for rows of few groups)" : elem_ ? " (for unaligned rows)"
+                  : stage_ ? " (a workgroup per row, the gathered operand's source row staged in LDS)" : "") << " ----\n";
     os_ << "// I: position type.  M: 2 = every 128-bit access is aligned and every pass is whole (no tail);\n";
     os_ << "// 1 = aligned and the innermost extent a multiple of W, passes may be partly empty; 0 = anything.\n";
-    os_ << "template <typename I, int M>\nDEV void segment" << index_ << (slim_ ? "_slim" : elem_ ? "_elem" : "")
+    os_ << "template <typename I, int M>\nDEV void segment" << index_ << (slim_ ? "_slim" : elem_ ? "_elem" : stage_ ? "_stage" : "")
         << "(const SpecArgs &R, const I bid, const I nblocks) {\n";
     line(1, "constexpr int W = " + std::to_string(W_) + ", U = " + std::to_string(U_) + ";");
     line(1, "constexpr bool A = M == 2, V = M >= 1;");
@@ -766,6 +801,11 @@ class SegmentEmitter {
       os_ << "}\n";
       return;
     }
+    if (stage_) {
+      line(1, "// the workgroup walks one row at a time");
+      line(1, "const I lanes = 256, rows_per_pass = 1, local_row = 0, first_group = (I)tid;");
+      line(1, "const I cblocks = 1, rblocks = nblocks, cbid = 0, rbid = bid;");
+    } else {
     line(1, "const I lanes = (I)1 << R.lanes_log2;");
     line(1, "const I rows_per_pass = (I)(256 >> R.lanes_log2);");
     line(1, "const I local_row = (I)(tid >> R.lanes_log2);");
@@ -773,11 +813,26 @@ class SegmentEmitter {
     line(1, "// few, long rows: column_blocks workgroups share a pass of rows, each taking every column_blocks-th stretch");
     line(1, "const I cblocks = (I)R.column_blocks, rblocks = cblocks == 1 ? nblocks : nblocks / cblocks;");
     line(1, "const I cbid = cblocks == 1 ? (I)0 : bid / rblocks, rbid = bid - cbid * rblocks;");
+    }
     line(1, "for (I row0 = rbid * rows_per_pass; row0 < rows; row0 += rblocks * rows_per_pass) {");
     line(2, "const I row = row0 + local_row;");
     line(2, "if (row >= rows) continue;");
     emitPositionOfRow(2);
     emitRowInvariants(2);
+    if (stage_) {
+      const Operand &so = operands_[stageOperand_];
+      const int epv = 16 / (int)elemTypeBytes(so.type);
+      const char *ctype = elemTypeBytes(so.type) == 2 ? "unsigned short" : "unsigned";
+      line(2, "{  // the source row of operand " + id(so) + ": " + in(so) + ".gextent elements, 128-bit loads into LDS");
+      line(3, "const I chunks = (I)(" + in(so) + ".gextent / " + std::to_string(epv) + ");");
+      line(3, "const u32x4 *src = (const u32x4 *)((const " + std::string(ctype) + " *)" + in(so) + ".base + q" + id(so) + ");");
+      line(3, "for (I c = (I)tid; c < chunks; c += 256)");
+      line(4, "((__attribute__((address_space(3))) u32x4 *)afir_stage)[c] = ld128<false>(src + c);");
+      line(2, "}");
+      line(2, "__builtin_amdgcn_fence(__ATOMIC_RELEASE, \"workgroup\");");
+      line(2, "__builtin_amdgcn_s_barrier();");
+      line(2, "__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, \"workgroup\");");
+    }
     line(2, "for (I first = first_group + cbid * lanes * U; first < groups; first += cblocks * lanes * U) {");
     emitGroups(3, "first", "lanes");
     const Value v = emitExpression(3);
@@ -803,6 +858,7 @@ class SegmentEmitter {
     line(4, "}");
     line(3, "}");
     line(2, "}");
+    if (stage_) line(2, "__builtin_amdgcn_s_barrier();   // the staged row is replaced by the next one");
     line(1, "}");
     os_ << "}\n";
   }
@@ -1189,6 +1245,12 @@ class SegmentEmitter {
         os_ << "KERNEL void " << specElementKernelName(index_, i32 != 0) << "(const SpecArgs R) { segment" << index_
             << "_elem<" << (i32 ? "int" : "long long") << ", 0>(R, (" << (i32 ? "int" : "long long")
             << ")__builtin_amdgcn_workgroup_id_x(), (" << (i32 ? "int" : "long long") << ")R.grid); }\n";
+    if (stageOperand_ >= 0)
+      for (int i32 = 1; i32 >= 0; --i32)
+        for (int mode = kSpecAligned; mode >= kSpecVector; --mode)
+          os_ << "KERNEL void " << specStagedKernelName(index_, i32 != 0, mode) << "(const SpecArgs R) { segment" << index_
+              << "_stage<" << (i32 ? "int" : "long long") << ", " << mode << ">(R, (" << (i32 ? "int" : "long long")
+              << ")__builtin_amdgcn_workgroup_id_x(), (" << (i32 ? "int" : "long long") << ")R.grid); }\n";
     if (hasSlim_)
       for (int mode = kSpecAligned; mode >= kSpecVector; --mode)
         os_ << "KERNEL void " << specSlimKernelName(index_, mode) << "(const SpecArgs R) { segment" << index_
@@ -1226,6 +1288,8 @@ class SegmentEmitter {
   bool narrow_ = false;    // ... of which the low 16 bits are the value (i16 output)
   bool slim_ = false;      // emitting the one-group-per-lane form of the segment
   bool elem_ = false;      // emitting the one-element-per-group form (no 128-bit accesses)
+  bool stage_ = false;     // emitting the form that stages the gathered operand's source row in LDS
+  int stageOperand_ = -1;  // index into operands_ of that operand, else -1
   bool hasSlim_ = false;   // ... which exists for this segment
   bool hoisted_ = false;   // row invariants and operand values are assigned, not declared
   bool keepRowConstants_ = false;   // ... and operands that are the same for every row are left alone
@@ -1327,6 +1391,20 @@ std::string specSplitRowsKernelName(int segment, bool idx32, bool join) {
 
 std::string specLongRowsKernelName(int segment, bool idx32) {
   return "afir_region_s" + std::to_string(segment) + "_long" + (idx32 ? "_i32" : "_i64");
+}
+
+std::string specStagedKernelName(int segment, bool idx32, int mode) {
+  return "afir_region_s" + std::to_string(segment) + "_stage" + (idx32 ? "_i32" : "_i64") + modeSuffix(mode);
+}
+
+SpecStage specStage(const Program &p, int segment) {
+  std::ostringstream sink;
+  SegmentEmitter e(p, segment, sink);
+  e.analyze();
+  SpecStage s;
+  s.input = e.stagedSlot();
+  s.elemBytes = (int)elemTypeBytes(e.stagedType());
+  return s;
 }
 
 std::string specElementKernelName(int segment, bool idx32) {

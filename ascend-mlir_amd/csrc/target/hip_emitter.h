@@ -104,7 +104,7 @@ uint64_t programHash(const afir_region::Program &p);
 // Version of the set of kernels and of the launch arguments that emitHipSource produces; the
 // code object exports it as `afir_region_emit_abi`, and a code object of another version is
 // refused when it is loaded (its kernels would be launched with the wrong names or arguments).
-constexpr int kSpecAbiVersion = 5;
+constexpr int kSpecAbiVersion = 6;
 
 // What a launch promises, which picks the kernel variant:
 //   kSpecAligned  every 128-bit access is aligned and every pass of the lanes over a row is whole
@@ -117,6 +117,18 @@ std::string specKernelName(int segment, bool idx32, int mode);
 // Untiled segments also have kernels whose lanes take one group each, for rows of
 // fewer than 8 x unroll groups (32-bit positions, modes kSpecAligned and kSpecVector).
 std::string specSlimKernelName(int segment, int mode);
+// A parallel rank-2 segment with one operand gathered along the innermost dim from the rows
+// of a matrix (`x[d0, index[d1]]`, the reference example's column gather) also has kernels
+// that stage the operand's source row in LDS, a workgroup per row, and gather from there:
+// launched with gextent * elemBytes bytes of dynamic LDS when the source rows are contiguous,
+// 16-byte aligned, a whole number of 128-bit chunks and at most kSpecStageBytes long.
+struct SpecStage {
+  int input = -1;      // SpecArgs::in slot of that operand, -1: the segment has no such kernels
+  int elemBytes = 2;
+};
+SpecStage specStage(const afir_region::Program &p, int segment);
+constexpr int kSpecStageBytes = 64 * 1024;
+std::string specStagedKernelName(int segment, bool idx32, int mode);
 // ... and kernels whose groups are single elements (kSpecElementUnroll of them per lane, a
 // lane-set apart), launched when rows do not start on 16-byte boundaries: every load and
 // store instruction of a wavefront then still covers one contiguous run.

@@ -259,6 +259,42 @@ def test_positions_beyond_32_bits(H):
         assert torch.equal(out[j0:j0 + 8192], (x[:, j0:j0 + 8192] + c[j0:j0 + 8192]).t()), j0
 
 
+@pytest.mark.parametrize("ty,ity", [("f16", "i64"), ("f32", "i32"), ("bf16", "i32")])
+def test_column_gather_from_rows_staged_in_lds(H, ty, ity):
+    """out[i, j] = relu(data[i, idx[j]]) + bias[j] with rows long enough for the compiled kernel
+    that stages each source row in LDS (a workgroup per row); indices out of range give NaN
+    and set the flag; a source row of odd length keeps the ordinary kernel.  Bit-exact."""
+    import torch
+    rng = np.random.default_rng(21)
+    text = RC.RELU_COLGATHER_ADD.replace("f16", ty).replace("i64", ity)
+    idt = np.int64 if ity == "i64" else np.int32
+
+    def vals(shape):
+        v = rng.integers(-4, 5, shape).astype(np.float32)
+        return v.astype(np.float16) if ty == "f16" else O.f32_to_bf16_bits(v) if ty == "bf16" else v
+
+    for (m, k, n) in ((5, 4096, 8192), (3, 1000, 4100), (2, 4097, 4096)):
+        data, bias = vals((m, k)), vals((n,))
+        idx = rng.integers(0, k, (n,)).astype(idt)
+        idx[:3] = (0, k - 1, k // 2)
+        want = RO.evaluate(text, [data, idx, bias])
+        got = run(H, text, [data, idx, bias], (m, n))
+        assert got.tobytes() == want.tobytes(), (m, k, n)
+    data, bias = vals((4, 2048)), vals((4096,))
+    idx = rng.integers(0, 2048, (4096,)).astype(idt)
+    idx[7], idx[4000] = 2048, -1
+    ws = torch.zeros(2, dtype=torch.int32, device="cuda")
+    got = run(H, text, [data, idx, bias], (4, 4096), workspace=ws)
+    assert int(ws[0].item()) != 0
+    gf = O.bf16_bits_to_f32(got) if ty == "bf16" else got.astype(np.float32)
+    assert np.isnan(gf[:, 7]).all() and np.isnan(gf[:, 4000]).all()
+    good = np.ones(4096, bool)
+    good[[7, 4000]] = False
+    idx[[7, 4000]] = 0
+    want = RO.evaluate(text, [data, idx, bias])
+    assert got[:, good].tobytes() == want[:, good].tobytes()
+
+
 def test_unaligned_bases_take_the_element_path(H):
     import torch
     rng = np.random.default_rng(12)

@@ -127,6 +127,15 @@ def test_short_rows_get_one_group_per_lane_kernels():
         assert f"afir_region_s0_i32_{mode}(" in src and f"afir_region_s0_i64_{mode}(" in src
 
 
+def test_column_gathers_get_an_lds_staged_kernel():
+    src = _emit(RC.RELU_COLGATHER_ADD).stdout
+    assert "a workgroup per row, the gathered operand's source row staged in LDS" in src
+    for name in ("afir_region_s0_stage_i32_a(", "afir_region_s0_stage_i32_v(", "afir_region_s0_stage_i64_a("):
+        assert name in src
+    assert "stage_f16(bad ? 0 : gi[u][e])" in src and "afir_region_s0_stage_i32_g(" not in src
+    assert "_stage_" not in _emit(RC.C4_GATHER_SCALE_SHIFT).stdout      # rows gathered whole: nothing to stage
+
+
 def test_identical_reads_are_loaded_once():
     src = _emit(RC.C1_ADD_MUL).stdout           # (a + b) * b reads b twice
     # once in the ordinary form of the segment, once in its one-group-per-lane form
