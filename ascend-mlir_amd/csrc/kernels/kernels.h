@@ -50,6 +50,9 @@ bool matmul_dma_supported(int64_t m, int64_t k, int64_t n);
 LaunchStatus launch_matmul_dma(const uint16_t *a, const uint16_t *b, const uint16_t *bias,
                                uint16_t *out, int m, int k, int n, float alpha, bool relu,
                                uint32_t block_dim, hipStream_t stream);
+LaunchStatus launch_matmul_dma_f16(const uint16_t *a, const uint16_t *b, const float *bias,
+                                   float *out, int m, int k, int n, float alpha, bool relu,
+                                   uint32_t block_dim, hipStream_t stream);
 
 // Matrix-core issue rate from registers only (probe.hip).  operands: 64 KiB of
 // bf16 on the device, sink: 2 * 256 * 512 floats.

@@ -44,6 +44,8 @@
 // around every barrier; measured on MI355X it is 11 % slower on constant
 // operands and equal, within 1 %, on N(0, 1/sqrt(K)) operands, where the board
 // power limit sets the pace.)
+#include <type_traits>
+
 #include "kernels.h"
 
 namespace afir {
@@ -145,10 +147,16 @@ struct Drain { static constexpr bool value = false; };
 // WM x WN waves (m x n), wave tile (256/WM) x (256/WN): 2 x 4 waves of
 // 128 x 64, or 2 x 2 waves of 128 x 128 (one wave per SIMD, two thirds of the
 // LDS operand bytes per MFMA).
-template <int WM, int WN>
-__global__ __launch_bounds__(WM * WN * 64) void matmul_bias_leakyrelu_bf16_dma(
+//
+// F16IO = false: A, B, bias, out are bf16.  F16IO = true: A, B are f16, bias and
+// out are float32 (the types of the reference's own matmul example,
+// examples/matmul-add-leakyrelu/step0_input.mlir:10-15): the same rings and
+// reads (both element types are 16 bits wide), the f16 MFMA, and an epilogue
+// that stores the float32 value unrounded.
+template <int WM, int WN, bool F16IO>
+__global__ __launch_bounds__(WM * WN * 64) void matmul_bias_leakyrelu_dma(
     const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
-    const uint16_t *__restrict__ bias, uint16_t *__restrict__ out, int M, int K, int N,
+    const void *__restrict__ bias_v, void *__restrict__ out_v, int M, int K, int N,
     float alpha, int relu, int tiles_m, int tiles_n) {
   extern __shared__ __align__(1024) unsigned char smem[];
   lds_byte *const lds = (lds_byte *)smem;
@@ -245,10 +253,15 @@ __global__ __launch_bounds__(WM * WN * 64) void matmul_bias_leakyrelu_bf16_dma(
       for (int j = 0; j < TNW; ++j) {
         const u32x4 bw = {o.b[j][0].x, o.b[j][0].y, o.b[j][1].x, o.b[j][1].y};
 #pragma unroll
-        for (int i = 0; i < TMW; ++i)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              __builtin_bit_cast(bf16x8, bw), __builtin_bit_cast(bf16x8, o.a[i]), acc[i][j], 0, 0,
-              0);
+        for (int i = 0; i < TMW; ++i) {
+          if constexpr (F16IO)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                __builtin_bit_cast(f16x8, bw), __builtin_bit_cast(f16x8, o.a[i]), acc[i][j], 0, 0, 0);
+          else
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                __builtin_bit_cast(bf16x8, bw), __builtin_bit_cast(bf16x8, o.a[i]), acc[i][j], 0, 0,
+                0);
+        }
       }
     };
     // operand reads for a stage held in A slot sa / B slot sbk; the stage is the
@@ -327,42 +340,57 @@ __global__ __launch_bounds__(WM * WN * 64) void matmul_bias_leakyrelu_bf16_dma(
     }
 
     // Epilogue.  A lane holds m = lane%32, n = 8q + 4*(lane/32) + e of each
-    // 32x32 block, i.e. 8 bytes of an output row per store: written straight
-    // to memory that is 16 bytes per row per instruction, and the partial
-    // lines cost three times the write traffic.  So each wave stages 32 rows
-    // of its tile (64 n = one 128-byte line per row) in LDS and stores them as
-    // full lines, eight rows per instruction.  The rings are free once every
-    // wave has left the K loop; a wave's 4 KiB staging area is private, and
+    // 32x32 block, i.e. 8 bytes (bf16) or 16 bytes (float32) of an output row
+    // per store: written straight to memory that is a fraction of a line per row
+    // per instruction, and the partial lines of the bf16 form cost three times
+    // the write traffic.  So each wave stages 32 rows of its tile (64 n = one
+    // or two 128-byte lines per row) in LDS and stores them as full lines,
+    // eight or four rows per instruction.  The rings are free once every wave
+    // has left the K loop; a wave's 4 or 8 KiB staging area is private, and
     // the LDS unit keeps a wave's accesses in order, so no further barrier is
     // needed until the next tile refills the rings.  The 16-byte chunk column
-    // is XOR-ed with (row/2)%8: conflict-free for the 8-byte writes (32 rows
-    // x 2 halves) and for the 16-byte row reads.
+    // is XOR-ed with a function of the row: conflict-free for the 8- or
+    // 16-byte writes (32 rows x 2 halves) and for the 16-byte row reads.
     __builtin_amdgcn_s_barrier();
     {
-      constexpr int CH = TNW * 4;              // 16-byte chunks per staged row
-      constexpr int kRowBytes = CH * 16;       // 128 or 256
+      constexpr int kOutBytes = F16IO ? 4 : 2;
+      constexpr int CH = TNW * 32 * kOutBytes / 16;   // 16-byte chunks per staged row
+      constexpr int kRowBytes = CH * 16;       // 128 .. 512
       constexpr int kRowsPerPass = 64 / CH;    // rows one store instruction covers
       unsigned char *const stage = smem + wave * (32 * kRowBytes);
       const int lm = lane & 31, lq = lane >> 5;
       const int rr = lane / CH, cc = lane % CH;
       // two 128-byte rows share a swizzle value (they span the same banks as
       // one 256-byte row)
-      auto swz = [](int r) { return CH == 8 ? ((r >> 1) & 7) : (r & 15); };
-      u32x2 braw[TNW][4];
+      auto swz = [](int r) { return CH == 8 ? ((r >> 1) & 7) : (r & (CH - 1)); };
+      typedef typename std::conditional<F16IO, f32x4, u32x2>::type BiasRaw;
+      BiasRaw braw[TNW][4];
 #pragma unroll
       for (int j = 0; j < TNW; ++j)
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-          braw[j][q] = bias ? *reinterpret_cast<const u32x2 *>(bias + n0 + (wn * TNW + j) * 32 + 8 * q + 4 * lq)
-                            : u32x2{0x80008000u, 0x80008000u};   // no bias: -0, the identity of the add
+        for (int q = 0; q < 4; ++q) {
+          const int n = n0 + (wn * TNW + j) * 32 + 8 * q + 4 * lq;
+          // no bias: -0, the identity of the add
+          if constexpr (F16IO)
+            braw[j][q] = bias_v ? *reinterpret_cast<const f32x4 *>(static_cast<const float *>(bias_v) + n)
+                                : f32x4{-0.f, -0.f, -0.f, -0.f};
+          else
+            braw[j][q] = bias_v ? *reinterpret_cast<const u32x2 *>(static_cast<const uint16_t *>(bias_v) + n)
+                                : u32x2{0x80008000u, 0x80008000u};
+        }
 #pragma unroll
       for (int i = 0; i < TMW; ++i) {
 #pragma unroll
         for (int j = 0; j < TNW; ++j) {
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            const float b0 = bf16_lo(braw[j][q].x), b1 = bf16_hi(braw[j][q].x);
-            const float b2 = bf16_lo(braw[j][q].y), b3 = bf16_hi(braw[j][q].y);
+            float b0, b1, b2, b3;
+            if constexpr (F16IO) {
+              b0 = braw[j][q][0]; b1 = braw[j][q][1]; b2 = braw[j][q][2]; b3 = braw[j][q][3];
+            } else {
+              b0 = bf16_lo(braw[j][q].x); b1 = bf16_hi(braw[j][q].x);
+              b2 = bf16_lo(braw[j][q].y); b3 = bf16_hi(braw[j][q].y);
+            }
             float v0 = acc[i][j][4 * q + 0] + b0;
             float v1 = acc[i][j][4 * q + 1] + b1;
             float v2 = acc[i][j][4 * q + 2] + b2;
@@ -371,11 +399,17 @@ __global__ __launch_bounds__(WM * WN * 64) void matmul_bias_leakyrelu_bf16_dma(
             v1 = fmaxf(v1, relu ? 0.f : v1 * alpha);
             v2 = fmaxf(v2, relu ? 0.f : v2 * alpha);
             v3 = fmaxf(v3, relu ? 0.f : v3 * alpha);
-            u32x2 w;
-            w.x = pack_bf16(v0, v1);
-            w.y = pack_bf16(v2, v3);
-            const int chunk = (j * 4 + q) ^ swz(lm);
-            *reinterpret_cast<u32x2 *>(stage + lm * kRowBytes + chunk * 16 + lq * 8) = w;
+            if constexpr (F16IO) {
+              const f32x4 w = {v0, v1, v2, v3};
+              const int chunk = (j * 8 + q * 2 + lq) ^ swz(lm);
+              *reinterpret_cast<f32x4 *>(stage + lm * kRowBytes + chunk * 16) = w;
+            } else {
+              u32x2 w;
+              w.x = pack_bf16(v0, v1);
+              w.y = pack_bf16(v2, v3);
+              const int chunk = (j * 4 + q) ^ swz(lm);
+              *reinterpret_cast<u32x2 *>(stage + lm * kRowBytes + chunk * 16 + lq * 8) = w;
+            }
           }
         }
 #pragma unroll
@@ -384,7 +418,9 @@ __global__ __launch_bounds__(WM * WN * 64) void matmul_bias_leakyrelu_bf16_dma(
           const u32x4 line =
               *reinterpret_cast<const u32x4 *>(stage + r * kRowBytes + ((cc ^ swz(r)) * 16));
           const int m = m0 + (wm * TMW + i) * 32 + r;
-          *reinterpret_cast<u32x4 *>(out + (int64_t)m * N + n0 + wn * (TNW * 32) + cc * 8) = line;
+          unsigned char *const row = static_cast<unsigned char *>(out_v) +
+                                     ((int64_t)m * N + n0 + wn * (TNW * 32)) * kOutBytes;
+          *reinterpret_cast<u32x4 *>(row + cc * 16) = line;
         }
       }
     }
@@ -409,11 +445,14 @@ bool matmul_dma_supported(int64_t m, int64_t k, int64_t n) {
 #define AFIR_MM_GRID kNumCU
 #endif
 
-LaunchStatus launch_matmul_dma(const uint16_t *a, const uint16_t *b, const uint16_t *bias,
-                               uint16_t *out, int m, int k, int n, float alpha, bool relu,
-                               uint32_t block_dim, hipStream_t stream) {
+namespace {
+
+template <bool F16IO>
+LaunchStatus launch_dma(const uint16_t *a, const uint16_t *b, const void *bias, void *out, int m,
+                        int k, int n, float alpha, bool relu, uint32_t block_dim,
+                        hipStream_t stream) {
   constexpr int WM = AFIR_MM_WAVES_M, WN = AFIR_MM_WAVES_N;
-  auto kernel = matmul_bias_leakyrelu_bf16_dma<WM, WN>;
+  auto kernel = matmul_bias_leakyrelu_dma<WM, WN, F16IO>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize,
                                                kLdsBytes);
@@ -427,6 +466,20 @@ LaunchStatus launch_matmul_dma(const uint16_t *a, const uint16_t *b, const uint1
   hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(WM * WN * 64), kLdsBytes, stream, a, b,
                      bias, out, m, k, n, alpha, relu ? 1 : 0, tiles_m, tiles_n);
   return after_launch();
+}
+
+}  // namespace
+
+LaunchStatus launch_matmul_dma(const uint16_t *a, const uint16_t *b, const uint16_t *bias,
+                               uint16_t *out, int m, int k, int n, float alpha, bool relu,
+                               uint32_t block_dim, hipStream_t stream) {
+  return launch_dma<false>(a, b, bias, out, m, k, n, alpha, relu, block_dim, stream);
+}
+
+LaunchStatus launch_matmul_dma_f16(const uint16_t *a, const uint16_t *b, const float *bias,
+                                   float *out, int m, int k, int n, float alpha, bool relu,
+                                   uint32_t block_dim, hipStream_t stream) {
+  return launch_dma<true>(a, b, bias, out, m, k, n, alpha, relu, block_dim, stream);
 }
 
 }  // namespace afir

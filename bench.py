@@ -39,7 +39,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # (two runs), scaled by the same counters' reading for a plain 256 MiB copy
 # (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Source: profiles/*.txt, section (2).
 MEASURED_TRAFFIC = {"c1": 201364377, "c2": 134645398, "c3": 134331904, "c4": 134146560,
-                    "c5": 2466480128, "g1": 201360588, "g2": 134597632, "g3": 134646386, "g4": 134155366,
+                    "c5": 2369118208, "g1": 201360588, "g2": 134597632, "g3": 134646386, "g4": 134155366,
                     "i1": 201612185,
                     "i2": 135318732}
 

@@ -312,6 +312,37 @@ def test_c5_ragged_shapes_integer_known_answer_exact(H, ty):
             assert np.array_equal(got, np.maximum(v, v * np.float32(0.001)))
 
 
+def test_c5_f16_direct_to_lds_kernel_integer_known_answer_exact(H):
+    """f16 inputs, float32 bias and output (the reference example's types) at shapes of whole
+    256 x 256 tiles, enough of them for the direct-to-LDS kernel: on small integers every
+    product and partial sum is exact in float32, so the result must be leakyrelu(A @ B + bias)
+    to the bit, which also pins the permutation of the float32 epilogue's staging."""
+    import os
+    import subprocess
+    from tests import mlir_cases as MC
+    tr = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "ascend-mlir_amd", "bin",
+                      "afir-translate")
+    text = subprocess.run([tr, "-mlir-to-hip", "-"], input=MC.MATMUL_BIAS_LEAKY_F16, capture_output=True,
+                          text=True, check=True).stdout
+    r = H.Region(text)
+    for (m, k, n) in ((4096, 512, 2048), (2048, 320, 4096), (2304, 256, 3840)):
+        rng = np.random.default_rng(m + k)
+        a = rng.integers(-3, 4, (m, k)).astype(np.float32)
+        b = rng.integers(-3, 4, (k, n)).astype(np.float32)
+        bias = rng.integers(-8, 9, (n,)).astype(np.float32)
+        v = a @ b + bias[None, :]
+        assert np.abs(v).max() < 2 ** 24
+        guard = torch.full((m + 2, n), 7.0, dtype=torch.float32, device="cuda")
+        ins = [dev(a.astype(np.float16)), dev(b.astype(np.float16)), dev(bias), torch.zeros((m, n), device="cuda")]
+        got = guard[1:m + 1]
+        dims = [d for t in ins for d in t.shape] + [m, n]
+        assert r.launch_raw([t.data_ptr() for t in ins] + [got.data_ptr()], H.pack_tiling(*dims)) == 0
+        torch.cuda.synchronize()
+        assert np.array_equal(got.cpu().numpy(), np.maximum(v, v * np.float32(0.001))), (m, k, n)
+        assert bool((guard[0] == 7).all()) and bool((guard[m + 1] == 7).all())
+    r.close()
+
+
 def test_c5_identity_and_alpha(H):
     n = 256
     eye = O.f32_to_bf16_bits(np.eye(n, dtype=np.float32))
