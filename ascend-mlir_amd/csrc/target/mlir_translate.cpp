@@ -1155,6 +1155,8 @@ class Translator {
     for (const std::string &o : operands) {
       TensorP t = tensorOf(o);
       if (!t->expr || t->reduced || !t->parts.empty()) r_.fail("afir." + name + ": operand is not an elementwise value");
+      if (inTypes[in.size()].shape.size() != t->shape.size())
+        r_.fail("afir." + name + ": the type given for " + o + " has another rank than the value");
       in.push_back(t);
     }
     auto tv = std::make_shared<Tensor>();

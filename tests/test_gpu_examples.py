@@ -245,7 +245,8 @@ def test_matmul_epilogue_kinds(pkg, kind, ty):
     every product and partial sum is exact in float32
     (examples/matmul-add-leakyrelu/gen_data.py:29-31), so the result does not
     depend on the order of accumulation; negative sums keep their sign without a
-    leaky relu.  bf16 at 512x512x256 takes the direct-to-LDS kernel."""
+    leaky relu.  2048x256x4096 (128 tiles of 256x256) takes the direct-to-LDS kernel,
+    512x256x512 the register-staged one with 128x128 tiles, 96x64x40 its bounds-checked form."""
     import torch
     from ascend_mlir_amd import hip_kernels as H
     from oracle import region_oracle as RO
@@ -257,7 +258,7 @@ def test_matmul_epilogue_kinds(pkg, kind, ty):
     has_bias = kind in ("bias", "bias_relu")
     p = subprocess.run([TR, "-mlir-to-hip", "-"], input=mlir, capture_output=True, text=True)
     assert p.returncode == 0, p.stderr
-    for (m, k, n) in ((512, 256, 512), (96, 64, 40)):
+    for (m, k, n) in ((512, 256, 512), (96, 64, 40), (2048, 256, 4096)):
         rng = np.random.default_rng(7)
         a = rng.integers(-3, 4, (m, k)).astype(np.float32)
         b = rng.integers(-3, 4, (k, n)).astype(np.float32)

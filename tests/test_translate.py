@@ -145,6 +145,9 @@ def test_tiling_space_out(tmp_path):
     (MC.TWO_CHAINS_CONCAT.replace("dim(0)", "dim(1)"), "along dim 0 only"),
     (MC.C1_AFIR.replace("return %1", "return %9"), "undefined value %9"),
     (MC.RELU_COLUMN_ADD.replace("(d0, d1) -> (d1, 0)", "(d0, d1) -> (d1 + 1, 0)"), "only dimensions and constants"),
+    ("func.func @f(%a: tensor<4x8xf32>, %b: tensor<4x8xf32>) -> tensor<4x8xf32> {\n"
+     " %0 = afir.add %a, %b : (tensor<8xf32>, tensor<4x8xf32>) -> tensor<4x8xf32>\n return %0 : tensor<4x8xf32>\n}",
+     "line 2: afir.add: the type given for %a has another rank than the value"),
 ])
 def test_unsupported_input_is_rejected_with_a_diagnostic(text, why):
     rc, out, err = translate(text)
