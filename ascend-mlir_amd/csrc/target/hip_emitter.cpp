@@ -518,6 +518,8 @@ class SegmentEmitter {
       unroll();
       line(d + 2, "for (int e = 0; e < W; ++e)");
       line(d + 3, "gi[u][e] = ld_" + std::string(typeTag(o.gatherType)) + "(" + r + ".index, (long long)(e < nvalid[u] ? j0[u] + e : n - 1));");
+      if (requestHere_ && stage_ && &o == &operands_[stageOperand_])
+        line(d + 1, "request(row0 + rblocks < rows ? row0 + rblocks : row0);   // the next row's source, see above");
       line(d + 1, "bool any_bad = false;");
       unroll();
       line(d + 1, "for (int u = 0; u < U; ++u)");
@@ -541,12 +543,18 @@ class SegmentEmitter {
     if (o.step == Operand::Contiguous) {
       unroll();
       line(d, "for (int u = 0; u < U; ++u) {");
-      if (elem_) line(d + 1, "if (false) {");
-      else line(d + 1, "if (A || (full[u] && (V || vec" + u + "))) {");
-      if (!elem_) line(d + 2, "ldv_" + tag + "<W, " + nt + ">(" + r + ".base, q" + u + " + j0[u], v" + u + "[u]);");
-      line(d + 1, "} else if (V) {");
-      unroll();
-      line(d + 2, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = " + zero() + ";");
+      if (elem_) {
+        line(d + 1, "if (false) {");
+      } else {
+        // aligned kernels: no branch around the load (an empty group reads the row's first
+        // vector and drops it), so that nothing is waited for before its use
+        line(d + 1, "if (A || V) {");
+        line(d + 2, "ldv_" + tag + "<W, " + nt + ">(" + r + ".base, q" + u + " + (A || full[u] ? j0[u] : (I)0), v" + u + "[u]);");
+        unroll();
+        line(d + 2, "for (int e = 0; e < W; ++e) v" + u + "[u][e] = A || full[u] ? v" + u + "[u][e] : " + zero() + ";");
+        line(d + 1, "} else if (full[u] && vec" + u + ") {");
+        line(d + 2, "ldv_" + tag + "<W, " + nt + ">(" + r + ".base, q" + u + " + j0[u], v" + u + "[u]);");
+      }
       line(d + 1, "} else {");
       unroll();
       // unconditional loads (of the row's last element where the lane has none), then a select:
@@ -599,11 +607,13 @@ class SegmentEmitter {
     for (const Op &op : seg_.ops)
       if (op.code == OpCode::Push) {
         const int k = pushSlot_[push++];
+        if (stage_ && k == stageOperand_) continue;   // last, below
         if (!have[k]) {
           if (!(keepRowConstants_ && rowConstant(operands_[k]))) read[k] = emitRead(operands_[k], d);
           have[k] = true;
         }
       }
+    if (stage_) read[stageOperand_] = emitRead(operands_[stageOperand_], d);
     return read;
   }
 
@@ -805,6 +815,28 @@ class SegmentEmitter {
       line(1, "// the workgroup walks one row at a time");
       line(1, "const I lanes = 256, rows_per_pass = 1, local_row = 0, first_group = (I)tid;");
       line(1, "const I cblocks = 1, rblocks = nblocks, cbid = 0, rbid = bid;");
+      {
+        // A source row of at most PF * 256 chunks is requested one row ahead, into registers.
+        // The request follows the index loads of the row's first pass and precedes their first
+        // use, in straight-line code: loads return in order, so the wait for the indices leaves
+        // the younger request in flight while the row is gathered.  (Rows that are longer, and
+        // the last row, still issue the PF loads: a branch around them would make the compiler
+        // wait for everything at the join.)
+        const Operand &so = operands_[stageOperand_];
+        const int epv = 16 / (int)elemTypeBytes(so.type);
+        const char *ctype = elemTypeBytes(so.type) == 2 ? "unsigned short" : "unsigned";
+        line(1, "constexpr int PF = 4;");
+        line(1, "const I chunks = (I)(" + in(so) + ".gextent / " + std::to_string(epv) + ");");
+        line(1, "const bool ahead = chunks <= (I)(PF * 256);");
+        line(1, "u32x4 nx[PF];");
+        line(1, "auto request = [&](const I r) {   // chunks past the row's end: chunk 0 again, never stored");
+        line(2, "const u32x4 *src = (const u32x4 *)((const " + std::string(ctype) + " *)" + in(so) + ".base + (long long)((I)" +
+                    in(so) + ".offset + r * (I)" + in(so) + ".stride[0]));");
+        unroll();
+        line(2, "for (int k = 0; k < PF; ++k) nx[k] = ld128<false>(src + ((I)tid + (I)(k * 256) < chunks ? (I)tid + (I)(k * 256) : (I)0));");
+        line(1, "};");
+        line(1, "request(rbid < rows ? rbid : (I)0);");
+      }
     } else {
     line(1, "const I lanes = (I)1 << R.lanes_log2;");
     line(1, "const I rows_per_pass = (I)(256 >> R.lanes_log2);");
@@ -821,42 +853,62 @@ class SegmentEmitter {
     emitRowInvariants(2);
     if (stage_) {
       const Operand &so = operands_[stageOperand_];
-      const int epv = 16 / (int)elemTypeBytes(so.type);
       const char *ctype = elemTypeBytes(so.type) == 2 ? "unsigned short" : "unsigned";
       line(2, "{  // the source row of operand " + id(so) + ": " + in(so) + ".gextent elements, 128-bit loads into LDS");
-      line(3, "const I chunks = (I)(" + in(so) + ".gextent / " + std::to_string(epv) + ");");
-      line(3, "const u32x4 *src = (const u32x4 *)((const " + std::string(ctype) + " *)" + in(so) + ".base + q" + id(so) + ");");
-      line(3, "for (I c = (I)tid; c < chunks; c += 256)");
-      line(4, "((__attribute__((address_space(3))) u32x4 *)afir_stage)[c] = ld128<false>(src + c);");
+      line(3, "if (ahead) {");
+      unroll();
+      line(4, "for (int k = 0; k < PF; ++k)");
+      line(5, "if ((I)tid + (I)(k * 256) < chunks) ((__attribute__((address_space(3))) u32x4 *)afir_stage)[tid + k * 256] = nx[k];");
+      line(3, "} else {");
+      line(4, "const u32x4 *src = (const u32x4 *)((const " + std::string(ctype) + " *)" + in(so) + ".base + q" + id(so) + ");");
+      line(4, "for (I c = (I)tid; c < chunks; c += 256)");
+      line(5, "((__attribute__((address_space(3))) u32x4 *)afir_stage)[c] = ld128<false>(src + c);");
+      line(3, "}");
       line(2, "}");
       line(2, "__builtin_amdgcn_fence(__ATOMIC_RELEASE, \"workgroup\");");
       line(2, "__builtin_amdgcn_s_barrier();");
       line(2, "__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, \"workgroup\");");
     }
-    line(2, "for (I first = first_group + cbid * lanes * U; first < groups; first += cblocks * lanes * U) {");
-    emitGroups(3, "first", "lanes");
-    const Value v = emitExpression(3);
-    std::string res = v.name;
-    if (v.scalar) {
-      line(3, ct() + " splat[U][W];");
+    // one pass of the lanes over the row, for the groups that start at `first`
+    auto emitPass = [&]() {
+      emitGroups(3, "first", "lanes");
+      const Value v = emitExpression(3);
+      std::string res = v.name;
+      if (v.scalar) {
+        line(3, ct() + " splat[U][W];");
+        unroll();
+        line(3, "for (int u = 0; u < U; ++u)");
+        unroll();
+        line(4, "for (int e = 0; e < W; ++e) splat[u][e] = " + v.name + ";");
+        res = "splat";
+      }
       unroll();
-      line(3, "for (int u = 0; u < U; ++u)");
+      line(3, "for (int u = 0; u < U; ++u) {");
+      line(4, "const long long o = (long long)row * (long long)n + (long long)j0[u];");
+      if (elem_) line(4, "if (false) {");
+      else line(4, "if (A || (full[u] && (V || R.out_vec))) {");
+      if (!elem_) line(5, "stv_" + otag + "<W>(R.out, o, " + res + "[u]);");
+      line(4, "} else if (!V) {");
       unroll();
-      line(4, "for (int e = 0; e < W; ++e) splat[u][e] = " + v.name + ";");
-      res = "splat";
+      line(5, "for (int e = 0; e < W; ++e)");
+      line(6, "if (e < nvalid[u]) st_" + otag + "(R.out, o + e, " + res + "[u][e]);");
+      line(4, "}");
+      line(3, "}");
+    };
+    if (stage_) {
+      // the row's first pass, taken by every lane (a lane past the row's end has empty groups:
+      // these kernels run where the innermost extent is a multiple of W), requests the next row
+      line(2, "{");
+      line(3, "const I first = first_group;");
+      requestHere_ = true;
+      emitPass();
+      requestHere_ = false;
+      line(2, "}");
+      line(2, "for (I first = first_group + lanes * U; first < groups; first += lanes * U) {");
+    } else {
+      line(2, "for (I first = first_group + cbid * lanes * U; first < groups; first += cblocks * lanes * U) {");
     }
-    unroll();
-    line(3, "for (int u = 0; u < U; ++u) {");
-    line(4, "const long long o = (long long)row * (long long)n + (long long)j0[u];");
-    if (elem_) line(4, "if (false) {");
-    else line(4, "if (A || (full[u] && (V || R.out_vec))) {");
-    if (!elem_) line(5, "stv_" + otag + "<W>(R.out, o, " + res + "[u]);");
-    line(4, "} else if (!V) {");
-    unroll();
-    line(5, "for (int e = 0; e < W; ++e)");
-    line(6, "if (e < nvalid[u]) st_" + otag + "(R.out, o + e, " + res + "[u][e]);");
-    line(4, "}");
-    line(3, "}");
+    emitPass();
     line(2, "}");
     if (stage_) line(2, "__builtin_amdgcn_s_barrier();   // the staged row is replaced by the next one");
     line(1, "}");
@@ -1289,6 +1341,7 @@ class SegmentEmitter {
   bool slim_ = false;      // emitting the one-group-per-lane form of the segment
   bool elem_ = false;      // emitting the one-element-per-group form (no 128-bit accesses)
   bool stage_ = false;     // emitting the form that stages the gathered operand's source row in LDS
+  bool requestHere_ = false;   // ... and the pass that requests the next row's source
   int stageOperand_ = -1;  // index into operands_ of that operand, else -1
   bool hasSlim_ = false;   // ... which exists for this segment
   bool hoisted_ = false;   // row invariants and operand values are assigned, not declared
