@@ -295,6 +295,36 @@ def test_column_gather_from_rows_staged_in_lds(H, ty, ity):
     assert got[:, good].tobytes() == want[:, good].tobytes()
 
 
+@pytest.mark.parametrize("ty,ity", [("f16", "i64"), ("f32", "i32")])
+def test_column_gather_workgroups_that_walk_several_rows(H, ty, ity):
+    """The staged column gather requests a workgroup's next source row while it gathers the
+    current one.  Grids smaller than the number of rows (forced through block_dim, uneven
+    shares included, and more rows than the largest grid), a source row that fills the
+    look-ahead registers exactly, one chunk more than that (no look-ahead), and a row that
+    is not a multiple of 256 chunks.  Bit-exact."""
+    rng = np.random.default_rng(33)
+    text = RC.RELU_COLGATHER_ADD.replace("f16", ty).replace("i64", ity)
+    idt = np.int64 if ity == "i64" else np.int32
+    per_chunk = 8 if ty == "f16" else 4
+
+    def vals(shape):
+        v = rng.integers(-4, 5, shape).astype(np.float32)
+        return v.astype(np.float16) if ty == "f16" else v
+
+    cases = [(10, 1024 * per_chunk, 4096, 3),            # 1024 chunks: all four look-ahead registers of every lane
+             (10, 1025 * per_chunk, 4096, 3),            # one chunk more: rows are loaded when their turn comes
+             (7, 300 * per_chunk, 8192, 2),              # 300 chunks: some lanes hold two, some one
+             (11, 520, 4104, 4),                         # passes that are partly empty
+             (4500, 64 * per_chunk, 4096, 0)]            # more rows than workgroups in the default grid
+    for (m, k, n, block_dim) in cases:
+        data, bias = vals((m, k)), vals((n,))
+        idx = rng.integers(0, k, (n,)).astype(idt)
+        idx[:3] = (0, k - 1, k // 2)
+        want = RO.evaluate(text, [data, idx, bias])
+        got = run(H, text, [data, idx, bias], (m, n), block_dim=block_dim)
+        assert got.tobytes() == want.tobytes(), (m, k, n, block_dim)
+
+
 def test_unaligned_bases_take_the_element_path(H):
     import torch
     rng = np.random.default_rng(12)
