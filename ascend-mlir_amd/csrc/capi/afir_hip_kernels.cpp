@@ -749,6 +749,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
     bool slim;   // the kernel whose lanes take one group each (short rows)
     bool elem;   // the kernel whose groups are single elements (rows off 16-byte boundaries)
     unsigned lds = 0;   // > 0: the kernel that stages a gathered operand's source row, with this much LDS
+    bool stage_wave = false;   // ... its form with a wavefront per row
   };
   std::vector<PendingSegment> pending;   // compiled kernels to launch, non-empty segments only
   for (const afir_region::ResolvedSegment &seg : res.segments) {
@@ -981,6 +982,26 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
         if (stage.input >= 0) {
           const afir::RegionInput &d = a.in[stage.input];
           const int64_t bytes = d.gextent * stage.elemBytes;
+          const int64_t n_out = seg.size[seg.rank - 1];
+          const int64_t wave_pass = (int64_t)64 * shape.unroll * wideW;     // elements a wavefront covers per pass
+          // Output rows of half a pass to eight passes of a wavefront, a thousand rows or more, source
+          // rows of at most 8 KiB: a wavefront per row, four rows per workgroup, each with its own part
+          // of the LDS and no barriers (measured against a workgroup per row, f16, TB/s written:
+          // [32768, 4096] from 1024 columns 1.15 -> 3.16, [16384, 2048] 1.56 -> 2.43, [2048, 16384]
+          // 2.22 -> 2.82, [16384, 8192] from 4096 columns equal; slower with 16 KiB source rows, which
+          // leave two workgroups per CU, and with fewer rows than the chip has wavefront slots)
+          if (d.gstride == 1 && d.vec && bytes > 0 && bytes % 16 == 0 && bytes * 4 <= afir_target::kSpecStageBytes / 2 &&
+              n_out * 2 >= wave_pass && n_out <= 8 * wave_pass && seg.size[0] >= 1024) {
+            int64_t blocks = (seg.size[0] + 3) / 4;
+            if (blocks > (int64_t)afir::kNumCU * 16) blocks = (int64_t)afir::kNumCU * 16;
+            if (block_dim) blocks = block_dim;
+            made.args.grid = (int)blocks;
+            made.args.column_blocks = 1;
+            made.lds = (unsigned)(bytes * 4);
+            made.stage_wave = true;
+            if (made.mode == afir_target::kSpecAligned && (n_out / wideW) % ((int64_t)64 * shape.unroll) != 0)
+              made.mode = afir_target::kSpecVector;
+          } else
           if (d.gstride == 1 && d.vec && bytes > 0 && bytes % 16 == 0 && bytes <= afir_target::kSpecStageBytes &&
               seg.size[seg.rank - 1] >= (int64_t)128 * shape.unroll * wideW) {   // at least half a pass of the workgroup
             int64_t blocks = seg.size[0] < (int64_t)afir::kNumCU * 16 ? seg.size[0] : (int64_t)afir::kNumCU * 16;
@@ -1051,7 +1072,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
           continue;
         }
         if (p.lds) {
-          const uint32_t rc = launch(afir_target::specStagedKernelName(p.segment, p.idx32, p.mode), &p.args, sizeof p.args,
+          const uint32_t rc = launch(afir_target::specStagedKernelName(p.segment, p.idx32, p.mode, p.stage_wave), &p.args, sizeof p.args,
                                      (unsigned)p.args.grid, p.lds);
           if (rc != AFIR_HIP_OK) return rc;
           continue;

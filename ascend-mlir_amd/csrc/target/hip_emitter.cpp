@@ -332,6 +332,9 @@ class SegmentEmitter {
       if (stageOperand_ >= 0) {
         stage_ = true;
         emitBody();
+        stageWave_ = true;    // the same with a wavefront per row, for short rows
+        emitBody();
+        stageWave_ = false;
         stage_ = false;
       }
       {
@@ -519,7 +522,7 @@ class SegmentEmitter {
       line(d + 2, "for (int e = 0; e < W; ++e)");
       line(d + 3, "gi[u][e] = ld_" + std::string(typeTag(o.gatherType)) + "(" + r + ".index, (long long)(e < nvalid[u] ? j0[u] + e : n - 1));");
       if (requestHere_ && stage_ && &o == &operands_[stageOperand_])
-        line(d + 1, "request(row0 + rblocks < rows ? row0 + rblocks : row0);   // the next row's source, see above");
+        line(d + 1, "request(row + rblocks * rows_per_pass < rows ? row + rblocks * rows_per_pass : row);   // the next row's source, see above");
       line(d + 1, "bool any_bad = false;");
       unroll();
       line(d + 1, "for (int u = 0; u < U; ++u)");
@@ -528,7 +531,7 @@ class SegmentEmitter {
       line(d + 3, "const bool bad = gi[u][e] < 0 || gi[u][e] >= " + r + ".gextent;");
       line(d + 3, "any_bad = any_bad || (bad && e < nvalid[u]);");
       if (stage_ && &o == &operands_[stageOperand_])
-        line(d + 3, "const " + ct() + " x = " + std::string(integer_ ? "staged_" : "stage_") + tag + "(bad ? 0 : gi[u][e]);");
+        line(d + 3, "const " + ct() + " x = " + std::string(integer_ ? "staged_" : "stage_") + tag + "(sbase + (bad ? 0 : gi[u][e]));");
       else
         line(d + 3, "const " + ct() + " x = " + ld(o.type) + "(" + r + ".base, q" + u +
                         " + (long long)(e < nvalid[u] ? j0[u] + e : n - 1) * step + (bad ? 0 : gi[u][e]) * " + r + ".gstride);");
@@ -753,10 +756,11 @@ class SegmentEmitter {
         << (reduce_ ? ", row sum over the innermost dim" : ", parallel") << "; a lane takes " << U_
         << (U_ == 1 ? " group of " : " groups of ") << W_ << " elements per pass"
         << (slim_ ? " (for rows of few groups)" : elem_ ? " (for unaligned rows)"
+                  : stageWave_ ? " (a wavefront per row, the gathered operand's source row staged in LDS)"
                   : stage_ ? " (a workgroup per row, the gathered operand's source row staged in LDS)" : "") << " ----\n";
     os_ << "// I: position type.  M: 2 = every 128-bit access is aligned and every pass is whole (no tail);\n";
     os_ << "// 1 = aligned and the innermost extent a multiple of W, passes may be partly empty; 0 = anything.\n";
-    os_ << "template <typename I, int M>\nDEV void segment" << index_ << (slim_ ? "_slim" : elem_ ? "_elem" : stage_ ? "_stage" : "")
+    os_ << "template <typename I, int M>\nDEV void segment" << index_ << (slim_ ? "_slim" : elem_ ? "_elem" : stageWave_ ? "_stagew" : stage_ ? "_stage" : "")
         << "(const SpecArgs &R, const I bid, const I nblocks) {\n";
     line(1, "constexpr int W = " + std::to_string(W_) + ", U = " + std::to_string(U_) + ";");
     line(1, "constexpr bool A = M == 2, V = M >= 1;");
@@ -812,8 +816,18 @@ class SegmentEmitter {
       return;
     }
     if (stage_) {
-      line(1, "// the workgroup walks one row at a time");
-      line(1, "const I lanes = 256, rows_per_pass = 1, local_row = 0, first_group = (I)tid;");
+      if (stageWave_) {
+        line(1, "// every wavefront walks rows of its own: its accesses to its part of the LDS are ordered, no barriers");
+        line(1, "const int sl = tid & 63;   // lane of the row's lane set");
+        line(1, "const I lanes = 64, rows_per_pass = 4, local_row = (I)(tid >> 6), first_group = (I)sl;");
+        line(1, "const long long sbase = (long long)(tid >> 6) * " + in(operands_[stageOperand_]) + ".gextent;");
+      } else {
+        line(1, "// the workgroup walks one row at a time");
+        line(1, "const int sl = tid;");
+        line(1, "const I lanes = 256, rows_per_pass = 1, local_row = 0, first_group = (I)tid;");
+        line(1, "const long long sbase = 0;");
+      }
+      line(1, "constexpr int SL = " + std::string(stageWave_ ? "64" : "256") + ";   // lanes that share a row");
       line(1, "const I cblocks = 1, rblocks = nblocks, cbid = 0, rbid = bid;");
       {
         // A source row of at most PF * 256 chunks is requested one row ahead, into registers.
@@ -827,15 +841,17 @@ class SegmentEmitter {
         const char *ctype = elemTypeBytes(so.type) == 2 ? "unsigned short" : "unsigned";
         line(1, "constexpr int PF = 4;");
         line(1, "const I chunks = (I)(" + in(so) + ".gextent / " + std::to_string(epv) + ");");
-        line(1, "const bool ahead = chunks <= (I)(PF * 256);");
+        line(1, "const bool ahead = chunks <= (I)(PF * SL);");
+        line(1, "__attribute__((address_space(3))) u32x4 *const srow = (__attribute__((address_space(3))) u32x4 *)afir_stage + (sbase / " +
+                    std::to_string(epv) + ");");
         line(1, "u32x4 nx[PF];");
         line(1, "auto request = [&](const I r) {   // chunks past the row's end: chunk 0 again, never stored");
         line(2, "const u32x4 *src = (const u32x4 *)((const " + std::string(ctype) + " *)" + in(so) + ".base + (long long)((I)" +
                     in(so) + ".offset + r * (I)" + in(so) + ".stride[0]));");
         unroll();
-        line(2, "for (int k = 0; k < PF; ++k) nx[k] = ld128<false>(src + ((I)tid + (I)(k * 256) < chunks ? (I)tid + (I)(k * 256) : (I)0));");
+        line(2, "for (int k = 0; k < PF; ++k) nx[k] = ld128<false>(src + ((I)sl + (I)(k * SL) < chunks ? (I)sl + (I)(k * SL) : (I)0));");
         line(1, "};");
-        line(1, "request(rbid < rows ? rbid : (I)0);");
+        line(1, "request(rbid * rows_per_pass + local_row < rows ? rbid * rows_per_pass + local_row : (I)0);");
       }
     } else {
     line(1, "const I lanes = (I)1 << R.lanes_log2;");
@@ -858,15 +874,15 @@ class SegmentEmitter {
       line(3, "if (ahead) {");
       unroll();
       line(4, "for (int k = 0; k < PF; ++k)");
-      line(5, "if ((I)tid + (I)(k * 256) < chunks) ((__attribute__((address_space(3))) u32x4 *)afir_stage)[tid + k * 256] = nx[k];");
+      line(5, "if ((I)sl + (I)(k * SL) < chunks) srow[sl + k * SL] = nx[k];");
       line(3, "} else {");
       line(4, "const u32x4 *src = (const u32x4 *)((const " + std::string(ctype) + " *)" + in(so) + ".base + q" + id(so) + ");");
-      line(4, "for (I c = (I)tid; c < chunks; c += 256)");
-      line(5, "((__attribute__((address_space(3))) u32x4 *)afir_stage)[c] = ld128<false>(src + c);");
+      line(4, "for (I c = (I)sl; c < chunks; c += SL)");
+      line(5, "srow[c] = ld128<false>(src + c);");
       line(3, "}");
       line(2, "}");
       line(2, "__builtin_amdgcn_fence(__ATOMIC_RELEASE, \"workgroup\");");
-      line(2, "__builtin_amdgcn_s_barrier();");
+      if (!stageWave_) line(2, "__builtin_amdgcn_s_barrier();");
       line(2, "__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, \"workgroup\");");
     }
     // one pass of the lanes over the row, for the groups that start at `first`
@@ -910,7 +926,7 @@ class SegmentEmitter {
     }
     emitPass();
     line(2, "}");
-    if (stage_) line(2, "__builtin_amdgcn_s_barrier();   // the staged row is replaced by the next one");
+    if (stage_ && !stageWave_) line(2, "__builtin_amdgcn_s_barrier();   // the staged row is replaced by the next one");
     line(1, "}");
     os_ << "}\n";
   }
@@ -1298,11 +1314,13 @@ class SegmentEmitter {
             << "_elem<" << (i32 ? "int" : "long long") << ", 0>(R, (" << (i32 ? "int" : "long long")
             << ")__builtin_amdgcn_workgroup_id_x(), (" << (i32 ? "int" : "long long") << ")R.grid); }\n";
     if (stageOperand_ >= 0)
-      for (int i32 = 1; i32 >= 0; --i32)
-        for (int mode = kSpecAligned; mode >= kSpecVector; --mode)
-          os_ << "KERNEL void " << specStagedKernelName(index_, i32 != 0, mode) << "(const SpecArgs R) { segment" << index_
-              << "_stage<" << (i32 ? "int" : "long long") << ", " << mode << ">(R, (" << (i32 ? "int" : "long long")
-              << ")__builtin_amdgcn_workgroup_id_x(), (" << (i32 ? "int" : "long long") << ")R.grid); }\n";
+      for (int wave = 0; wave < 2; ++wave)
+        for (int i32 = 1; i32 >= 0; --i32)
+          for (int mode = kSpecAligned; mode >= kSpecVector; --mode)
+            os_ << "KERNEL void " << specStagedKernelName(index_, i32 != 0, mode, wave != 0) << "(const SpecArgs R) { segment"
+                << index_ << (wave ? "_stagew<" : "_stage<") << (i32 ? "int" : "long long") << ", " << mode << ">(R, ("
+                << (i32 ? "int" : "long long") << ")__builtin_amdgcn_workgroup_id_x(), (" << (i32 ? "int" : "long long")
+                << ")R.grid); }\n";
     if (hasSlim_)
       for (int mode = kSpecAligned; mode >= kSpecVector; --mode)
         os_ << "KERNEL void " << specSlimKernelName(index_, mode) << "(const SpecArgs R) { segment" << index_
@@ -1342,6 +1360,7 @@ class SegmentEmitter {
   bool elem_ = false;      // emitting the one-element-per-group form (no 128-bit accesses)
   bool stage_ = false;     // emitting the form that stages the gathered operand's source row in LDS
   bool requestHere_ = false;   // ... and the pass that requests the next row's source
+  bool stageWave_ = false;     // ... with a wavefront per row (four rows per workgroup, no barriers)
   int stageOperand_ = -1;  // index into operands_ of that operand, else -1
   bool hasSlim_ = false;   // ... which exists for this segment
   bool hoisted_ = false;   // row invariants and operand values are assigned, not declared
@@ -1446,8 +1465,9 @@ std::string specLongRowsKernelName(int segment, bool idx32) {
   return "afir_region_s" + std::to_string(segment) + "_long" + (idx32 ? "_i32" : "_i64");
 }
 
-std::string specStagedKernelName(int segment, bool idx32, int mode) {
-  return "afir_region_s" + std::to_string(segment) + "_stage" + (idx32 ? "_i32" : "_i64") + modeSuffix(mode);
+std::string specStagedKernelName(int segment, bool idx32, int mode, bool wave) {
+  return "afir_region_s" + std::to_string(segment) + (wave ? "_stagew" : "_stage") + (idx32 ? "_i32" : "_i64") +
+         modeSuffix(mode);
 }
 
 SpecStage specStage(const Program &p, int segment) {

@@ -104,7 +104,7 @@ uint64_t programHash(const afir_region::Program &p);
 // Version of the set of kernels and of the launch arguments that emitHipSource produces; the
 // code object exports it as `afir_region_emit_abi`, and a code object of another version is
 // refused when it is loaded (its kernels would be launched with the wrong names or arguments).
-constexpr int kSpecAbiVersion = 6;
+constexpr int kSpecAbiVersion = 7;
 
 // What a launch promises, which picks the kernel variant:
 //   kSpecAligned  every 128-bit access is aligned and every pass of the lanes over a row is whole
@@ -128,7 +128,10 @@ struct SpecStage {
 };
 SpecStage specStage(const afir_region::Program &p, int segment);
 constexpr int kSpecStageBytes = 64 * 1024;
-std::string specStagedKernelName(int segment, bool idx32, int mode);
+// wave: the variant that gives a wavefront to a row (four rows per workgroup, each with its own
+// gextent * elemBytes bytes of the LDS, no barriers), for output rows of at most two passes of
+// a wavefront.
+std::string specStagedKernelName(int segment, bool idx32, int mode, bool wave);
 // ... and kernels whose groups are single elements (kSpecElementUnroll of them per lane, a
 // lane-set apart), launched when rows do not start on 16-byte boundaries: every load and
 // store instruction of a wavefront then still covers one contiguous run.

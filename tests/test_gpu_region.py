@@ -297,8 +297,8 @@ def test_column_gather_from_rows_staged_in_lds(H, ty, ity):
 
 @pytest.mark.parametrize("ty,ity", [("f16", "i64"), ("f32", "i32")])
 def test_column_gather_workgroups_that_walk_several_rows(H, ty, ity):
-    """The staged column gather requests a workgroup's next source row while it gathers the
-    current one.  Grids smaller than the number of rows (forced through block_dim, uneven
+    """The staged column gather requests a workgroup's (or, for short output rows, a
+    wavefront's) next source row while it gathers the current one.  Grids smaller than the number of rows (forced through block_dim, uneven
     shares included, and more rows than the largest grid), a source row that fills the
     look-ahead registers exactly, one chunk more than that (no look-ahead), and a row that
     is not a multiple of 256 chunks.  Bit-exact."""
@@ -315,7 +315,11 @@ def test_column_gather_workgroups_that_walk_several_rows(H, ty, ity):
              (10, 1025 * per_chunk, 4096, 3),            # one chunk more: rows are loaded when their turn comes
              (7, 300 * per_chunk, 8192, 2),              # 300 chunks: some lanes hold two, some one
              (11, 520, 4104, 4),                         # passes that are partly empty
-             (4500, 64 * per_chunk, 4096, 0)]            # more rows than workgroups in the default grid
+             (4500, 64 * per_chunk, 4096, 0),            # more rows than workgroups in the default grid
+             # output rows of at most two passes of a wavefront: the form with a wavefront per row
+             # (launched for a thousand rows or more)
+             (1033, 64 * per_chunk, 2048, 37), (4500, 32 * per_chunk, 1032, 0), (1030, 256 * per_chunk, 1024, 100),
+             (1100, 257 * per_chunk, 2048, 64)]          # ... with a source row beyond its look-ahead registers
     for (m, k, n, block_dim) in cases:
         data, bias = vals((m, k)), vals((n,))
         idx = rng.integers(0, k, (n,)).astype(idt)

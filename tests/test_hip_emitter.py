@@ -132,9 +132,11 @@ def test_short_rows_get_one_group_per_lane_kernels():
 def test_column_gathers_get_an_lds_staged_kernel():
     src = _emit(RC.RELU_COLGATHER_ADD).stdout
     assert "a workgroup per row, the gathered operand's source row staged in LDS" in src
-    for name in ("afir_region_s0_stage_i32_a(", "afir_region_s0_stage_i32_v(", "afir_region_s0_stage_i64_a("):
+    assert "a wavefront per row, the gathered operand's source row staged in LDS" in src
+    for name in ("afir_region_s0_stage_i32_a(", "afir_region_s0_stage_i32_v(", "afir_region_s0_stage_i64_a(",
+                 "afir_region_s0_stagew_i32_a(", "afir_region_s0_stagew_i64_v("):
         assert name in src
-    assert "stage_f16(bad ? 0 : gi[u][e])" in src and "afir_region_s0_stage_i32_g(" not in src
+    assert "stage_f16(sbase + (bad ? 0 : gi[u][e]))" in src and "afir_region_s0_stage_i32_g(" not in src
     assert "_stage_" not in _emit(RC.C4_GATHER_SCALE_SHIFT).stdout      # rows gathered whole: nothing to stage
 
 
