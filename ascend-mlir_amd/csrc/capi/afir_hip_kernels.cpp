@@ -280,6 +280,65 @@ std::string detect_fast_path(RegisteredRegion *r) {
   }
   return "";
 }
+
+// The hand-tuned kernels take densely packed operands whose shapes are the
+// iteration extents.  A program can match a family and still read only part of a
+// tensor (a zero-offset extract_slice narrower than its operand keeps the plain
+// 'push'), so the shapes of a launch decide: every routed operand must be walked
+// with the strides of a dense tensor of exactly the extents the kernel assumes,
+// from element 0.  Extents of 1 leave their stride free.
+bool fast_path_fits(const RegisteredRegion &r, const afir_region::Resolved &res) {
+  if (res.segments.size() != 1) return false;
+  const afir_region::ResolvedSegment &seg = res.segments[0];
+  const int64_t *sz = seg.size;
+  auto dense = [&](const afir_region::ResolvedInput &in, std::initializer_list<int64_t> strides) {
+    if (in.offset != 0 || in.gatherIterDim >= 0) return false;
+    int k = 0;
+    for (int64_t want : strides) {
+      if (sz[k] > 1 && in.iterStride[k] != want) return false;
+      ++k;
+    }
+    return true;
+  };
+  // the output is dense by construction: resolve() checks that the one segment covers it
+  switch (r.fast) {
+    case FastPath::None:
+      return false;
+    case FastPath::AddMul:
+      for (const afir_region::ResolvedInput &in : seg.inputs)
+        if (!dense(in, {sz[1], 1})) return false;
+      return true;
+    case FastPath::BcastAddRowsum:
+      for (const afir_region::ResolvedInput &in : seg.inputs)
+        if (!(in.arg == r.fastArgs[0] ? dense(in, {sz[1], 1}) : dense(in, {0, 1}))) return false;
+      return true;
+    case FastPath::ReluBcastTranspose:
+      // iteration space (b, j, i); x is [b, i, j]
+      for (const afir_region::ResolvedInput &in : seg.inputs)
+        if (!(in.arg == r.fastArgs[0] ? dense(in, {sz[1] * sz[2], 1, sz[1]}) : dense(in, {0, 1, 0}))) return false;
+      return true;
+    case FastPath::GatherScaleShift:
+      for (const afir_region::ResolvedInput &in : seg.inputs) {
+        if (in.arg == r.fastArgs[0]) {
+          // rows of exactly the iteration width, gathered along dim 0 from the whole table
+          if (in.offset != 0 || in.gatherIterDim != 0 || (sz[1] > 1 && in.iterStride[1] != 1) ||
+              in.gatherStride != sz[1] || in.gatherExtent != res.shapes[in.arg][0])
+            return false;
+        } else if (!dense(in, {0, 1})) {
+          return false;
+        }
+      }
+      return true;
+    case FastPath::MatmulBiasLeaky:
+    case FastPath::MatmulBiasLeakyF16:
+      // resolve() has matched A [M,K], B [K,N] against the segment; the bias is read from element 0
+      for (const afir_region::ResolvedInput &in : seg.inputs)
+        if (!dense(in, {0, 1})) return false;
+      return true;
+  }
+  return false;
+}
+
 std::mutex g_region_mutex;
 std::map<uint64_t, std::shared_ptr<RegisteredRegion>> g_regions;
 uint64_t g_next_region = 1;
@@ -656,6 +715,36 @@ uint32_t afir_hip_region_argument_bytes(uint64_t handle, const void *tiling, siz
   return AFIR_HIP_OK;
 }
 
+const char *afir_hip_region_route(uint64_t handle, const void *tiling, size_t tiling_len) {
+  auto r = find_region(handle);
+  if (!r) {
+    (void)fail(AFIR_HIP_E_UNKNOWN, "no region program with that handle");
+    return "";
+  }
+  afir_region::Resolved res;
+  const std::string why = resolve_region(*r, tiling, tiling_len, &res);
+  if (!why.empty()) {
+    (void)fail(AFIR_HIP_E_INVALID, why);
+    return "";
+  }
+  g_last_error.clear();
+  const bool is_matmul = r->fast == FastPath::MatmulBiasLeaky || r->fast == FastPath::MatmulBiasLeakyF16;
+  bool has_code, prefer;
+  {
+    std::lock_guard<std::mutex> lock(g_region_mutex);
+    has_code = r->compiled != nullptr;
+    prefer = r->preferCompiled && has_code && !is_matmul;
+  }
+  if (r->fast != FastPath::None && !prefer && fast_path_fits(*r, res)) return "family";
+  if (is_matmul) {
+    (void)fail(AFIR_HIP_E_INVALID, "region: the matmul kernels read the bias from its first element, densely");
+    return "";
+  }
+  if (const char *env = std::getenv("AFIR_HIP_REGION_INTERPRET"))
+    if (*env && *env != '0') has_code = false;
+  return has_code ? "compiled" : "interpreter";
+}
+
 uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *stream, int num_args,
                                 void *const *args, void *workspace, const void *tiling,
                                 size_t tiling_len) {
@@ -679,7 +768,11 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
     prefer_compiled = r->preferCompiled && r->compiled != nullptr && r->fast != FastPath::MatmulBiasLeaky &&
                       r->fast != FastPath::MatmulBiasLeakyF16;
   }
-  if (r->fast != FastPath::None && !prefer_compiled) {
+  const bool is_matmul = r->fast == FastPath::MatmulBiasLeaky || r->fast == FastPath::MatmulBiasLeakyF16;
+  const bool fits = r->fast != FastPath::None && fast_path_fits(*r, res);
+  if (is_matmul && !fits)
+    return fail(AFIR_HIP_E_INVALID, "region: the matmul kernels read the bias from its first element, densely");
+  if (fits && !prefer_compiled) {
     const afir_region::ResolvedSegment &seg = res.segments[0];
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int *fa = r->fastArgs;

@@ -106,6 +106,7 @@ class HipExecutionRunner final : public ExecutionRunner {
   Status runDynamicLibraryArtifact(const DynamicLibraryExecutionLaunch &launch,
                                    RunArgs &args) override {
     lastKernelUs_ = -1.0;
+    lastRegionRoute_.clear();
     if (!initialized_) return Status::error("execution runner has not been initialized");
     if (args.inputs.size() + args.outputs.size() + 2 > 16)
       return Status::error("too many tensor arguments for a launcher call (16 pointer slots)");
@@ -165,6 +166,9 @@ class HipExecutionRunner final : public ExecutionRunner {
         }
       }
       if (Status st = validateRegion(lib, region, args, why); !st.ok()) return st;
+      using RouteFn = const char *(*)(uint64_t, const void *, size_t);
+      if (auto route = reinterpret_cast<RouteFn>(dlsym(lib, "afir_hip_region_route")))
+        lastRegionRoute_ = route(region, args.tiling.data(), args.tiling.size());
     }
 
     // ---- device buffers ----
@@ -262,6 +266,7 @@ class HipExecutionRunner final : public ExecutionRunner {
   }
 
   double lastKernelMicroseconds() const override { return lastKernelUs_; }
+  std::string lastRegionRoute() const override { return lastRegionRoute_; }
 
  private:
   Status validate(void *lib, const std::string &symbol, const RunArgs &args) {
@@ -340,6 +345,7 @@ class HipExecutionRunner final : public ExecutionRunner {
   hipStream_t stream_ = nullptr;
   hipEvent_t ev0_ = nullptr, ev1_ = nullptr;
   double lastKernelUs_ = -1.0;
+  std::string lastRegionRoute_;
 };
 
 }  // namespace

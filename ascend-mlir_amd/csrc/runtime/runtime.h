@@ -308,6 +308,10 @@ class ExecutionRunner {
                                            RunArgs &args) = 0;
   // Kernel time of the last run in microseconds (HIP events), < 0 if unknown.
   virtual double lastKernelMicroseconds() const { return -1.0; }
+  // Kernels the last run of a fused-region program went to: "family" (a hand-tuned
+  // kernel), "compiled" (the artifact's code object) or "interpreter" (the library's
+  // generic kernel, several times slower); "" for launcher-symbol artifacts.
+  virtual std::string lastRegionRoute() const { return ""; }
 };
 
 // The MI355X runner: alloc -> H2D -> launch -> sync -> D2H -> free

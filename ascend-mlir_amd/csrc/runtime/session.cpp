@@ -206,6 +206,9 @@ SessionSummary runSingleTask(const RunTaskSpec &task, RunnerFactory factory, int
     return fail(summary, "kernel_launch", st.message);
   const double us = runner->lastKernelMicroseconds();
   if (us >= 0) summary.runtimeCounters["kernel_ns"] = (int64_t)(us * 1e3);
+  // how a fused-region task was run; "interpreter" is the slow route (no code object in the artifact)
+  if (const std::string route = runner->lastRegionRoute(); !route.empty())
+    summary.runtimeAttributes["region_route"] = route;
   summary.runtimeCounters["block_dim"] = inv.blockDim;
   summary.runtimeCounters["tiling_bytes"] = (int64_t)args.tiling.size();
 

@@ -46,6 +46,7 @@ EXPORTED_SYMBOLS = [
     "afir_hip_region_info",
     "afir_hip_region_tiling_field",
     "afir_hip_region_kernel",
+    "afir_hip_region_route",
     "afir_hip_region_emit_source",
     "afir_hip_region_attach_code_object",
     "afir_hip_region_prefer_code_object",
@@ -411,6 +412,18 @@ class Region:
             self.close()
         except Exception:
             pass
+
+    def route(self, tiling: bytes) -> str:
+        """"family", "compiled" or "interpreter": the kernels a launch with these
+        shapes runs on (host only)."""
+        L = load()
+        L.afir_hip_region_route.restype = ctypes.c_char_p
+        L.afir_hip_region_route.argtypes = [ctypes.c_uint64, ctypes.c_void_p, ctypes.c_size_t]
+        buf = ctypes.create_string_buffer(tiling, len(tiling))
+        got = L.afir_hip_region_route(ctypes.c_uint64(self.handle), buf, len(tiling)).decode()
+        if not got:
+            raise AfirHipError(L.afir_hip_last_error().decode())
+        return got
 
     def argument_bytes(self, tiling: bytes):
         n = self.num_inputs + self.num_outputs

@@ -325,8 +325,10 @@ def make_workload(key, torch, H, O, C):
             got = sets[0][3][torch.from_numpy(rows).cuda()].view(torch.int16).cpu().numpy() \
                 .view(np.uint16)
             r = O.compare_outputs([(got, "bf16")], [(want, "bf16")], 1e-5, 1e-2)
-            return {"bar": "<=1e-2 rel (atol 1e-5), 128 sampled rows x 8192 cols",
-                    "passed": bool(r["passed"]), "mismatches": int(r["mismatches"]),
+            nonfinite = O.nonfinite_mismatches(got, want, "bf16")   # the comparator cannot see NaN
+            return {"bar": "<=1e-2 rel (atol 1e-5), 128 sampled rows x 8192 cols; no NaN / inf the golden lacks",
+                    "passed": bool(r["passed"]) and nonfinite == 0,
+                    "mismatches": int(r["mismatches"]) + nonfinite, "nonfinite_mismatches": nonfinite,
                     "max_abs": float(r["max_abs_diff"]),
                     "bit_identical_frac": float((got == want).mean())}
         w.parity = parity

@@ -187,6 +187,21 @@ uint32_t afir_hip_region_info(uint64_t handle, int *num_inputs, int *num_outputs
  * AFIR_HIP_REGION_GENERIC=1 before registering keeps every non-matmul program
  * on the generic kernel. */
 const char *afir_hip_region_kernel(uint64_t handle);
+/* Which of the three routes a launch with these shapes takes (tiling as for
+ * afir_hip_launch_region; host only, launches nothing):
+ *   "family"       the hand-tuned kernel afir_hip_region_kernel names.  Those
+ *                  kernels take densely packed operands of exactly the
+ *                  iteration extents, so a program of a family's form whose
+ *                  launch reads part of a larger tensor (a zero-offset slice
+ *                  narrower than its operand) does not take it;
+ *   "compiled"     the kernels of the attached code object;
+ *   "interpreter"  the library's interpreter kernel: correct for every
+ *                  program, at a fraction of the compiled kernels' rate.
+ * "" with afir_hip_last_error() set when the shapes do not resolve.  The
+ * reference announces how a task was run in its session.runtime.attribute.*
+ * lines (tools/runtime-session/runtime_session_main.cpp:161-183); this is the
+ * source of the region_route attribute there. */
+const char *afir_hip_region_route(uint64_t handle, const void *tiling, size_t tiling_len);
 /* Kernels compiled for one program, the counterpart of the reference's
  * generated kernel source and device binary
  * (lib/Target/CannKernel/CannTranslation.cpp:2487-2694 prints the source,

@@ -199,15 +199,18 @@ def _evaluate_integer(prog, inputs, val, out_type, out_rank):
     return res.astype(np.int16 if out_type == "i16" else np.int32)
 
 
-def evaluate(text: str, inputs):
+def evaluate(text: str, inputs, out_shape=None):
     """Runs the program on numpy inputs (bf16 tensors as uint16 bits).  Returns
-    the output array in its storage type (bf16 as uint16 bits)."""
+    the output array in its storage type (bf16 as uint16 bits).  out_shape is
+    needed only by programs whose extents refer to the output's dimensions."""
     prog = parse(text)
     args = prog["args"]
     n_in = len(args) - 1
     if len(inputs) != n_in:
         raise RegionError(f"expected {n_in} inputs, got {len(inputs)}")
     shapes = [tuple(x.shape) for x in inputs]
+    if out_shape is not None:
+        shapes.append(tuple(out_shape))
     out_type, out_rank = args[-1][1], args[-1][2]
 
     def val(ref):

@@ -177,6 +177,7 @@ def test_matmul_bf16_program_runs_on_the_mfma_kernel(pkg):
     got = out.view(torch.int16).cpu().numpy().view(np.uint16)
     res = O.compare_outputs([(got, "bf16")], [(O.golden_c5(a, b, bias, 0.01), "bf16")], 1e-5, 1e-2)
     assert res["passed"], res
+    assert O.nonfinite_mismatches(got, O.golden_c5(a, b, bias, 0.01), "bf16") == 0
     r.close()
 
 

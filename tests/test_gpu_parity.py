@@ -247,6 +247,8 @@ C5_ATOL, C5_RTOL = 1e-5, 1e-2
 def _check_c5(got_bits, want_bits):
     r = O.compare_outputs([(got_bits, "bf16")], [(want_bits, "bf16")], C5_ATOL, C5_RTOL)
     assert r["passed"], r
+    # the comparator's `diff > tol` is false for NaN: count those separately
+    assert O.nonfinite_mismatches(got_bits, want_bits, "bf16") == 0
     assert (got_bits == want_bits).mean() > 0.97
 
 

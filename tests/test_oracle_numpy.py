@@ -242,6 +242,22 @@ def test_comparator_reference_cases():
                           [(np.array([1, 2], np.int32), "i32")], 0.0, 0.0)
 
 
+def test_comparator_is_nan_blind_and_nonfinite_mismatches_is_not():
+    """The reference's `diff > atol + rtol*|e|` is false for NaN, so its comparator passes
+    a NaN where the golden is finite; the parity checks count those separately."""
+    want = np.array([1.0, -2.0, np.inf, -np.inf, np.nan, 0.0], np.float32)
+    got = np.array([np.nan, -2.0, np.inf, np.inf, np.nan, np.inf], np.float32)
+    r = O.compare_outputs([(got, "f32")], [(want, "f32")], 1e-5, 1e-2)
+    assert r["mismatches"] == 1          # only the finite-vs-inf element at the end
+    assert O.nonfinite_mismatches(got, want, "f32") == 3   # NaN vs 1, +inf vs -inf, inf vs 0
+    assert O.nonfinite_mismatches(want, want, "f32") == 0
+    # bf16 bits: 0x7fc0 NaN, 0x7f80 +inf, 0x3f80 1.0
+    gb = np.array([0x7fc0, 0x7f80, 0x3f80], np.uint16)
+    wb = np.array([0x3f80, 0x7f80, 0x3f80], np.uint16)
+    assert O.compare_outputs([(gb, "bf16")], [(wb, "bf16")], 1e-5, 1e-2)["passed"]
+    assert O.nonfinite_mismatches(gb, wb, "bf16") == 1
+
+
 def test_comparator_decode_bits():
     assert O.comparator_decode(np.array([0x3C00], np.uint16), "f16")[0] == 1.0
     assert O.comparator_decode(np.array([0x4000], np.uint16), "f16")[0] == 2.0
