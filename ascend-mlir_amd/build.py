@@ -3,7 +3,10 @@
     python ascend-mlir_amd/build.py [--force]
 
 Outputs (under ascend-mlir_amd/lib/):
-    libafir_hip_kernels.so   fused kernels + launcher C ABI
+    libafir_hip_kernels.so    fused kernels + launcher C ABI
+    libAFIRRuntimeCAPI.so     afirt_* C API + host runtime (and bin/: the CLIs)
+    families/*.hsaco          the kernel families as compiled region kernels
+    libafir_bench_probes.so   measurement aids of bench.py (not part of the product)
 """
 from __future__ import annotations
 
@@ -36,7 +39,6 @@ KERNEL_SOURCES = [
     ("kernels/gather.hip", STRICT),
     ("kernels/matmul.hip", []),
     ("kernels/matmul_dma.hip", []),
-    ("kernels/probe.hip", []),
     ("kernels/region.hip", STRICT),
     ("target/region_program.cpp", []),
     ("target/hip_emitter.cpp", []),
@@ -151,9 +153,32 @@ def build_families(kernel_lib):
     return built
 
 
+def build_probes():
+    """libafir_bench_probes.so: ceiling probes for bench.py (csrc/bench/probes.h), and the
+    direct-to-LDS matmul kernel compiled twice more with parts of its K loop left out, each
+    under a namespace name of its own."""
+    os.makedirs(LIB, exist_ok=True)
+    os.makedirs(OBJ, exist_ok=True)
+    jobs = [("bench/probes.hip", "bench_probes.o", [])]
+    for level in (1, 2):
+        jobs.append(("kernels/matmul_dma.hip", f"bench_matmul_ablate{level}.o",
+                     [f"-DAFIR_MM_ABLATE={level}", f"-Dafir=afir_abl{level}"]))
+
+    def one(job):
+        src, name, extra = job
+        obj = os.path.join(OBJ, name)
+        _run([HIPCC, *COMMON, *extra, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj])
+        return obj
+    with cf.ThreadPoolExecutor(max_workers=3) as ex:
+        objs = list(ex.map(one, jobs))
+    out = os.path.join(LIB, "libafir_bench_probes.so")
+    _run([HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", out, *objs])
+    return out
+
+
 def build_all():
     kernel_lib = build_kernels()
-    return [kernel_lib, *build_runtime(), *build_families(kernel_lib)]
+    return [kernel_lib, *build_runtime(), *build_families(kernel_lib), build_probes()]
 
 
 if __name__ == "__main__":

@@ -529,12 +529,6 @@ uint32_t afir_hip_launch_matmul_add_leakyrelu(uint32_t block_dim, void *stream, 
       /*relu=*/false, block_dim, static_cast<hipStream_t>(stream)));
 }
 
-uint32_t afir_hip_probe_mfma_rate(void *stream, const void *operands, void *sink, uint32_t iters,
-                                  uint64_t *flops) {
-  return finish(afir::launch_mfma_rate_probe(operands, static_cast<float *>(sink), iters, flops,
-                                             static_cast<hipStream_t>(stream)));
-}
-
 namespace {
 uint32_t register_region(const char *program_text, size_t program_len, uint64_t *handle, bool generic);
 }

@@ -85,7 +85,11 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 template <typename T>
 __device__ __forceinline__ T load_nt(const T *p) {
+#ifdef AFIR_PLAIN_LOADS
+  return *p;
+#else
   return __builtin_nontemporal_load(p);
+#endif
 }
 template <typename T>
 __device__ __forceinline__ void store_nt(T *p, T v) {

@@ -54,13 +54,6 @@ LaunchStatus launch_matmul_dma_f16(const uint16_t *a, const uint16_t *b, const f
                                    float *out, int m, int k, int n, float alpha, bool relu,
                                    uint32_t block_dim, hipStream_t stream);
 
-// Matrix-core issue rate from registers only (probe.hip).  operands: 64 KiB of
-// bf16 on the device, sink: 2 * 256 * 512 floats.
-constexpr size_t kMfmaProbeOperandBytes = 65536;
-constexpr size_t kMfmaProbeSinkBytes = 2 * 256 * 512 * 4;
-LaunchStatus launch_mfma_rate_probe(const void *operands, float *sink, uint32_t iters,
-                                    uint64_t *flops, hipStream_t stream);
-
 inline LaunchStatus ok_status() { return LaunchStatus{0u, ""}; }
 inline LaunchStatus invalid(const char *msg) { return LaunchStatus{1u, msg}; }
 inline LaunchStatus after_launch() {

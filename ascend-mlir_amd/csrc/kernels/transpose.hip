@@ -18,21 +18,30 @@ constexpr int kThreads = 256;
 // max(v, +0) with IEEE-754 maximum semantics: NaN propagates, -0 gives +0.
 __device__ __forceinline__ float relu_keep_nan(float v) { return (v > 0.f) ? v : ((v != v) ? v : 0.f); }
 
-// One 64x64 tile per workgroup, one workgroup pass per tile, float32 in LDS:
-// 16.6 KiB of LDS and few registers, so eight workgroups fit a CU and the
-// chip holds 2048 tiles at once.  Phase 1: a lane loads two 16-byte chunks of
-// x rows (a wave covers eight 128-byte runs per load), applies relu and + c
-// (its eight columns are fixed, so c is read once) and writes the float32
-// results to tile[i][j], rows padded to 65 words.  Phase 2: a lane reads eight
-// consecutive i of one j (a column of the padded tile: at most two lanes per bank), rounds
+// 64x64 tiles through a float32 LDS tile, two tiles in flight per workgroup.
+// Phase 1: a lane loads two 16-byte chunks of x rows (a wave covers eight
+// 128-byte runs per load), applies relu and + c (its eight columns are fixed
+// within a tile, so c is read once per tile) and writes the float32 results to
+// tile[i][j], rows padded to 65 words.  Phase 2: a lane reads eight consecutive
+// i of one j (a column of the padded tile: at most two lanes per bank), rounds
 // them to f16 and writes one 16-byte chunk of an output row; eight lanes cover
-// a 128-byte run along M.  Tiles are numbered along M first, so neighbouring
-// workgroups write neighbouring runs of the same output rows.
+// a 128-byte run along M.  The next tile's loads are issued before the current
+// tile's stores, into the other of two LDS tiles, so a workgroup needs one
+// barrier per tile and always has loads or stores outstanding.  Tiles are
+// numbered along M first, so neighbouring workgroups write neighbouring runs
+// of the same output rows.
+//
+// The loads are ordinary loads, the stores non-temporal.  This kernel moves
+// as many bytes out as in, and for such streams the non-temporal hint on the
+// LOADS costs bandwidth on MI355X: a plain 64 MiB copy measured 6.0 TB/s with
+// the hint on both sides and 6.7 with ordinary loads, this kernel 5.5 and 6.5
+// (kernels that read two or more bytes per byte written measured the other
+// way round and keep the hint on their loads).
 constexpr int kSmallTile = 64, kSmallPitch = kSmallTile + 1;
 __global__ __launch_bounds__(kThreads) void relu_bcast_add_transpose_f16_tile64(
     const uint16_t *__restrict__ x, const uint16_t *__restrict__ c, uint16_t *__restrict__ out,
     int nb, int m, int n) {
-  __shared__ float tile[kSmallTile * kSmallPitch];
+  __shared__ float tiles[2][kSmallTile * kSmallPitch];
   const int t = threadIdx.x;
   // 32-bit tile numbers (the launcher checks that they fit): a 64-bit
   // division costs hundreds of instructions before the first load
@@ -40,17 +49,26 @@ __global__ __launch_bounds__(kThreads) void relu_bcast_add_transpose_f16_tile64(
   const unsigned ntiles = (unsigned)nb * tiles_m * tiles_n;
   const int lj = (t & 7) * 8, li = t >> 3;        // phase 1: first column, row within a pass of 32
   const int oi = (t & 7) * 8, oj = t >> 3;        // phase 2: first i of the chunk, j within a pass of 32
-  for (unsigned tile_id = blockIdx.x; tile_id < ntiles; tile_id += gridDim.x) {
+  auto locate = [&](unsigned tile_id, int &m0, int &n0, int &b) {
     const unsigned rest = tile_id / tiles_m;
-    const int tm = (int)(tile_id - rest * tiles_m);
-    const int b = (int)(rest / tiles_n);
-    const int tn = (int)(rest - (unsigned)b * tiles_n);
-    const int m0 = tm * kSmallTile, n0 = tn * kSmallTile;
-    const u32x4 craw = *reinterpret_cast<const u32x4 *>(c + n0 + lj);
+    m0 = (int)(tile_id - rest * tiles_m) * kSmallTile;
+    b = (int)(rest / tiles_n);
+    n0 = (int)(rest - (unsigned)b * tiles_n) * kSmallTile;
+  };
+  unsigned tile_id = blockIdx.x;
+  if (tile_id >= ntiles) return;
+  int m0, n0, b;
+  locate(tile_id, m0, n0, b);
+  u32x4 craw = *reinterpret_cast<const u32x4 *>(c + n0 + lj);
+  u32x4 v[2];
+  {
     const uint16_t *xin = x + ((int64_t)b * m + m0 + li) * n + n0 + lj;
-    u32x4 v[2];
 #pragma unroll
-    for (int k = 0; k < 2; ++k) v[k] = load_nt(reinterpret_cast<const u32x4 *>(xin + (int64_t)(32 * k) * n));
+    for (int k = 0; k < 2; ++k) v[k] = *reinterpret_cast<const u32x4 *>(xin + (int64_t)(32 * k) * n);
+  }
+  int parity = 0;
+  for (;;) {
+    float *const tile = tiles[parity];
 #pragma unroll
     for (int k = 0; k < 2; ++k)
 #pragma unroll
@@ -59,6 +77,18 @@ __global__ __launch_bounds__(kThreads) void relu_bcast_add_transpose_f16_tile64(
         dst[0] = relu_keep_nan(f16_lo(v[k][d])) + f16_lo(craw[d]);
         dst[1] = relu_keep_nan(f16_hi(v[k][d])) + f16_hi(craw[d]);
       }
+    // request the next tile before this one is written out
+    const unsigned next_id = tile_id + gridDim.x;
+    const bool more = next_id < ntiles;
+    int next_m0 = 0, next_n0 = 0, next_b = 0;
+    if (more) {
+      locate(next_id, next_m0, next_n0, next_b);
+      craw = *reinterpret_cast<const u32x4 *>(c + next_n0 + lj);
+      const uint16_t *xin = x + ((int64_t)next_b * m + next_m0 + li) * n + next_n0 + lj;
+#pragma unroll
+      for (int k = 0; k < 2; ++k) v[k] = *reinterpret_cast<const u32x4 *>(xin + (int64_t)(32 * k) * n);
+    }
+    // one barrier per tile: the other LDS tile was last read two barriers ago
     __syncthreads();
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
@@ -69,7 +99,12 @@ __global__ __launch_bounds__(kThreads) void relu_bcast_add_transpose_f16_tile64(
         w[d] = pack_f16(tile[(oi + 2 * d) * kSmallPitch + j], tile[(oi + 2 * d + 1) * kSmallPitch + j]);
       store_nt(reinterpret_cast<u32x4 *>(out + ((int64_t)b * n + n0 + j) * m + m0 + oi), w);
     }
-    __syncthreads();
+    if (!more) break;
+    tile_id = next_id;
+    m0 = next_m0;
+    n0 = next_n0;
+    b = next_b;
+    parity ^= 1;
   }
 }
 
@@ -119,7 +154,10 @@ LaunchStatus launch_relu_broadcast_add_transpose(const uint16_t *x, const uint16
 
   if ((m % kSmallTile == 0) && (n % kSmallTile == 0) && aligned16(x) && aligned16(c) && aligned16(out) &&
       nb * (m / kSmallTile) * (n / kSmallTile) < ((int64_t)1 << 31)) {
-    int64_t blocks = nb * (m / kSmallTile) * (n / kSmallTile);   // one tile per workgroup
+    // two tiles per workgroup (4096 workgroups of two tiles measured 20.3 us on [64, 1024, 512], 2048
+    // of four 21.4, 8192 of one 20.7): the hardware deals workgroups out as slots free up, which
+    // balances better than longer walks
+    int64_t blocks = (nb * (m / kSmallTile) * (n / kSmallTile) + 1) / 2;
     if (blocks > (int64_t)kNumCU * 256) blocks = (int64_t)kNumCU * 256;
     if (block_dim) blocks = block_dim;
     hipLaunchKernelGGL(relu_bcast_add_transpose_f16_tile64, dim3((unsigned)blocks), dim3(kThreads), 0, stream,

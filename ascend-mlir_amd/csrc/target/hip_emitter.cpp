@@ -416,6 +416,18 @@ class SegmentEmitter {
           o.tileSlot = tiles++;
         }
     numTiles_ = tiles;
+    // Non-temporal loads pay when reads dominate the traffic.  A segment that writes about as many
+    // bytes as it streams in (one full-size input per output) measured faster on MI355X with
+    // ordinary loads next to its non-temporal stores: a plain copy 6.0 -> 6.7 TB/s, the tiled
+    // transpose 5.5 -> 6.5.  Two full-size inputs per output measured 7 % slower that way
+    // (6.25 -> 5.8) and a row sum, which writes next to nothing, 3 % slower; those keep the hint.
+    if (!reduce_) {
+      size_t streamed = 0;
+      for (const Operand &o : operands_)
+        if (o.readOnce) streamed += elemTypeBytes(o.type);
+      if (streamed * 4 <= elemTypeBytes(p_.output().type) * 5)
+        for (Operand &o : operands_) o.readOnce = false;
+    }
     // a gather along the innermost dim from rows of a matrix (the index tensor picks the column):
     // the source row can be staged in LDS and gathered from there
     stageOperand_ = -1;

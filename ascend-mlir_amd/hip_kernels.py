@@ -40,7 +40,6 @@ EXPORTED_SYMBOLS = [
     "afir_hip_find_kernel",
     "afir_hip_launch",
     "afir_hip_argument_bytes",
-    "afir_hip_probe_mfma_rate",
     "afir_hip_region_register",
     "afir_hip_region_unregister",
     "afir_hip_region_info",
@@ -85,8 +84,6 @@ def load():
     L.afir_hip_launch.restype = u32
     L.afir_hip_launch.argtypes = [ctypes.c_char_p, u32, vp, ctypes.c_int,
                                   ctypes.POINTER(vp), vp, vp, ctypes.c_size_t]
-    L.afir_hip_probe_mfma_rate.restype = u32
-    L.afir_hip_probe_mfma_rate.argtypes = [vp, vp, vp, u32, ctypes.POINTER(ctypes.c_uint64)]
     _lib = L
     return L
 
@@ -249,35 +246,6 @@ def prepare(symbol: str, ptrs, tiling: bytes, block_dim: int = 0, stream=None):
         if rc:
             _check(rc)
     return call
-
-
-MFMA_PROBE_OPERAND_BYTES = 65536
-MFMA_PROBE_SINK_BYTES = 1 << 20
-
-
-def probe_mfma_rate(operands, iters=20000, repeats=3):
-    """TFLOP/s at which the matrix cores retire bf16 MFMAs fed from registers,
-    for the given operand values (a device tensor of >= 65536 bytes).  Returns
-    the best of `repeats` timed launches."""
-    import torch
-    L = load()
-    if not operands.is_cuda or operands.numel() * operands.element_size() < MFMA_PROBE_OPERAND_BYTES:
-        raise AfirHipError("probe_mfma_rate: need a device tensor of at least 65536 bytes")
-    sink = torch.empty(MFMA_PROBE_SINK_BYTES // 4, dtype=torch.float32, device=operands.device)
-    flops = ctypes.c_uint64(0)
-    _check(L.afir_hip_probe_mfma_rate(_stream(None), _ptr(operands), _ptr(sink), 200,
-                                      ctypes.byref(flops)))
-    torch.cuda.synchronize()
-    best = 0.0
-    for _ in range(repeats):
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        _check(L.afir_hip_probe_mfma_rate(_stream(None), _ptr(operands), _ptr(sink), iters,
-                                          ctypes.byref(flops)))
-        e1.record()
-        torch.cuda.synchronize()
-        best = max(best, flops.value / (e0.elapsed_time(e1) * 1e-3) / 1e12)
-    return best
 
 
 # ---- fused-region programs ---------------------------------------------------

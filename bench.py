@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused-kernel hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1|c3|c4|c5]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2|c1|c3|c4|c5|...]
                     [--all/--no-all] [--no-cpu-baseline]
 
 A step is one launch of the workload's fused kernel over one batch of seeded
@@ -17,7 +17,12 @@ steps so that the working set (several hundred MB) cannot be served from the
   cpu_baseline     the C restatement of the reference golden ("port"), timed
                    on this host's cores on a bounded sample
   workloads        with --all (default): the same figures for all five
-                   configurations, each parity-checked against the oracle
+                   configurations, each parity-checked against the oracle, the
+                   region-program workloads (g*, i*) and three measured
+                   ceilings (ceil_*: probe kernels of libafir_bench_probes.so)
+  targets          per configuration: roofline.frac (the event-timed figure),
+                   the target it is read against and whether it is met;
+                   min_frac_hbm = the lowest of c1..c4
 """
 from __future__ import annotations
 
@@ -37,12 +42,26 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 
 # HBM bytes per step measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (two runs), scaled by the same counters' reading for a plain 256 MiB copy
-# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Source: profiles/*.txt, section (2).
-MEASURED_TRAFFIC = {"c1": 201364377, "c2": 134645398, "c3": 134331904, "c4": 134146560,
-                    "c5": 2369118208, "g1": 201360588, "g2": 134597632, "g3": 134646386, "g4": 134155366,
-                    "i1": 201612185,
-                    "i2": 135318732}
+# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0).  Not measured in this run: each figure
+# is copied from section (2) of the profiles/ file named beside it, which gives
+# the command that produced it.
+MEASURED_TRAFFIC = {
+    "c1": (201364377, "profiles/add_mul_f32_vec__c1_4096x4096.txt"),
+    "c2": (134645398, "profiles/bcast_add_rowsum_f32_wgrow__c2_8192x4096.txt"),
+    "c3": (134331904, "profiles/relu_bcast_add_transpose_f16_tile64__c3_64x1024x512.txt"),
+    "c4": (134146560, "profiles/gather_scale_shift_f16_grouped__c4_131072x1024_idx32768.txt"),
+    "c5": (2369118208, "profiles/matmul_bias_leakyrelu_dma__c5_8192x8192x8192.txt"),
+    "g1": (201360588, "profiles/afir_region_s0_i32_a__g1_compiled_add_mul_f32_4096x4096.txt"),
+    "g2": (134597632, "profiles/afir_region_all_i32_a__g2_compiled_split_relu_brc_f16_8192x4096.txt"),
+    "g3": (134646386, "profiles/afir_region_s0_rows_i32__g3_compiled_bcast_add_rowsum_f32_8192x4096.txt"),
+    "g4": (134155366, "profiles/afir_region_s0_i32_a__g4_compiled_gather_scale_shift_f16_131072x1024_idx32768.txt"),
+    "i1": (201612185, "profiles/fused_region_parallel__i1_interpreter_add_mul_f32_4096x4096.txt"),
+    "i2": (135318732, "profiles/fused_region_parallel__i2_interpreter_split_relu_brc_f16_8192x4096.txt"),
+}
 
+# north_star targets, read on roofline.frac (algorithmic work / event-timed launch duration / published peak)
+TARGETS = {"c1": 0.70, "c2": 0.70, "c3": 0.70, "c4": 0.70, "c5": 0.60}
+ALL_WORKLOADS = ["c1", "c2", "c3", "c4", "c5", "g1", "g2", "g3", "g4", "i1", "i2", "ceil_copy", "ceil_read", "ceil_tilecopy64"]
 
 # Region programs of the two generic-kernel workloads (grammar:
 # ascend-mlir_amd/csrc/target/region_program.h)
@@ -275,10 +294,10 @@ def make_workload(key, torch, H, O, C):
         rng = np.random.default_rng(7)
         sets = []
         for i in range(w.nsets):
-            # the table (256 MiB) is shared; each set gathers a different
-            # seeded index vector, so consecutive launches touch different rows
+            # a table (256 MiB) and a seeded index vector of its own per set: no
+            # row a launch gathers was touched by the launch before it
             ii = idx if i == 0 else rng.integers(0, 131072, 32768, dtype=np.int64).astype(np.int32)
-            sets.append((dt_, _dev(torch, ii), dsc, dsh,
+            sets.append((dt_ if i == 0 else dt_.clone(), _dev(torch, ii), dsc, dsh,
                          torch.empty((32768, 1024), dtype=torch.float16, device="cuda")))
         w.sets = sets
         w.launches = [H.prepare(w.symbol, [s[0].data_ptr(), s[1].data_ptr(), s[2].data_ptr(),
@@ -343,29 +362,58 @@ def make_workload(key, torch, H, O, C):
         w.cpu = cpu
 
         def power_evidence():
-            """Why the fraction of the published MFMA peak is what it is: the
-            board power limit sets the clock, and the power an MFMA draws
-            depends on its operand values.  Three figures: the register-only
-            MFMA rate on this workload's operands and on constant ones, and
-            this same matmul kernel on constant matrices."""
-            ev = {"mfma_only_workload_operands_tflops":
-                  round(H.probe_mfma_rate(sets[0][0]), 1)}
+            """Why the fraction of the published MFMA peak is what it is, in figures
+            measured in this run on this workload's operands: the register-only MFMA
+            rate (the board power limit sets the clock, and the power an MFMA draws
+            depends on its operand values), the same kernel with its feed and its
+            LDS reads left out, the vendor GEMM on the same operands, and all of it
+            again on constant matrices."""
+            from ascend_mlir_amd import bench_probes as P
+            flops = w.work()
+
+            def rate(launch, n=10, warm=2):
+                for i in range(warm):
+                    launch(i)
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for i in range(n):
+                    launch(i)
+                e1.record()
+                torch.cuda.synchronize()
+                return flops * n / (e0.elapsed_time(e1) * 1e-3) / 1e12
+
+            def ablated(what):
+                calls = [P.prepare("afir_bench_matmul_ablated", s[0].data_ptr(), s[1].data_ptr(), s[2].data_ptr(),
+                                   s[3].data_ptr(), 8192, 8192, 8192, what) for s in sets]
+                return lambda i: calls[i % len(calls)]()
+
+            ours = lambda i: w.launches[i % len(w.launches)]()
+            vendor = lambda i: torch.matmul(sets[i % len(sets)][0], sets[i % len(sets)][1])
+            # alternating rounds: each kernel sees the same thermal history
+            rounds = {"this_kernel": [], "vendor_gemm": [], "no_feed": [], "no_feed_no_lds_reads": []}
+            for _ in range(3):
+                rounds["vendor_gemm"].append(rate(vendor))
+                rounds["this_kernel"].append(rate(ours))
+                rounds["no_feed"].append(rate(ablated(1)))
+                rounds["no_feed_no_lds_reads"].append(rate(ablated(2)))
+            med = lambda v: round(sorted(v)[len(v) // 2], 1)
+            ev = {"mfma_only_workload_operands_tflops": round(P.mfma_rate(sets[0][0]), 1),
+                  "vendor_gemm_tflops": med(rounds["vendor_gemm"]),
+                  "vendor_gemm": "torch.matmul (hipBLASLt), no bias / activation, same operands, rounds of 10 "
+                                 "launches alternating with this kernel; median of 3",
+                  "this_kernel_alternating_tflops": med(rounds["this_kernel"]),
+                  "decomposition_tflops": {
+                      "mfma_waits_barriers": med(rounds["no_feed_no_lds_reads"]),
+                      "plus_lds_operand_reads": med(rounds["no_feed"]),
+                      "plus_global_to_lds_feed_and_epilogue": med(rounds["this_kernel"])}}
             ones = torch.ones((8192, 8192), dtype=torch.bfloat16, device="cuda")
-            ev["mfma_only_constant_operands_tflops"] = round(H.probe_mfma_rate(ones), 1)
+            ev["mfma_only_constant_operands_tflops"] = round(P.mfma_rate(ones), 1)
             launch = H.prepare(w.symbol, [ones.data_ptr(), ones.data_ptr(), sets[0][2].data_ptr(),
                                           sets[1][3].data_ptr(), 0],
                                H.pack_tiling(8192, 8192, 8192, H.f32_bits(0.01)))
-            for _ in range(3):
-                launch()
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record()
-            for _ in range(20):
-                launch()
-            e1.record()
-            torch.cuda.synchronize()
-            ev["kernel_constant_operands_tflops"] = round(
-                w.work() * 20 / (e0.elapsed_time(e1) * 1e-3) / 1e12, 1)
+            ev["kernel_constant_operands_tflops"] = round(rate(lambda i: launch(), n=20, warm=3), 1)
+            ev["vendor_gemm_constant_operands_tflops"] = round(rate(lambda i: torch.matmul(ones, ones), n=20, warm=3), 1)
             return ev
         w.power_evidence = power_evidence
     elif key in ("g1", "g2", "g3", "g4", "i1", "i2"):
@@ -427,9 +475,9 @@ def make_workload(key, torch, H, O, C):
             if i == 0:
                 ins = dev0
             elif key[1] == "4":
-                # the table (256 MiB) is shared; every set gathers other rows
+                # a table (256 MiB) of its own per set, and other rows
                 other = idx_rng.integers(0, 131072, 32768, dtype=np.int64).astype(np.int32)
-                ins = [dev0[0], _dev(torch, other)] + dev0[2:]
+                ins = [dev0[0].clone(), _dev(torch, other)] + dev0[2:]
             else:
                 ins = [dev0[0].clone()] + ([dev0[1].clone()] if key[1] == "1" else dev0[1:])
             sets.append((ins, torch.empty(out_shape, dtype=out_dt, device="cuda")))
@@ -460,6 +508,47 @@ def make_workload(key, torch, H, O, C):
             return w.work() / dt / 1e9, "full workload, numpy region oracle (1 thread), one run"
         w.cpu = cpu
         w.cpu_cores = 1
+    elif key in ("ceil_copy", "ceil_read", "ceil_tilecopy64"):
+        # Measured ceilings (probe kernels of libafir_bench_probes.so, csrc/bench/probes.h): what
+        # this chip sustains on a plain copy, on a read-only stream and on the address pattern of
+        # c3's tiled transpose with the transposition left out.  No oracle: nothing is computed.
+        from ascend_mlir_amd import bench_probes as P
+        nbytes = 64 << 20
+        w.dtype = "u8"
+        w.nsets = 4
+        w.no_cpu = True
+        srcs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device="cuda") for _ in range(w.nsets)]
+        if key == "ceil_copy":
+            w.title = "ceil_copy: 64 MiB -> 64 MiB, 128-bit non-temporal loads and stores (probe, no arithmetic)"
+            dsts = [torch.empty_like(x) for x in srcs]
+            w.work = lambda: 2 * nbytes
+            w.launches = [P.prepare("afir_bench_copy", a.data_ptr(), b.data_ptr(), nbytes) for a, b in zip(srcs, dsts)]
+            w.sets = list(zip(srcs, dsts))
+            w.parity = lambda: {"bar": "dst == src", "passed": bool(torch.equal(srcs[0], dsts[0])),
+                                "mismatches": int((srcs[0] != dsts[0]).sum().item())}
+        elif key == "ceil_read":
+            w.title = "ceil_read: 64 MiB read-only stream, 128-bit non-temporal loads (probe)"
+            sink = torch.zeros(8192, dtype=torch.float32, device="cuda")
+            w.work = lambda: nbytes
+            w.launches = [P.prepare("afir_bench_read", a.data_ptr(), sink.data_ptr(), nbytes) for a in srcs]
+            w.sets = [(a, sink) for a in srcs]
+            w.parity = lambda: {"bar": "none: nothing is written", "passed": True, "mismatches": 0}
+        else:
+            w.title = ("ceil_tilecopy64: c3's address pattern ([64,1024,512] -> [64,512,1024] f16 in 64x64 tiles, "
+                       "128-byte runs both ways) without the transposition (probe, registers only)")
+            dsts = [torch.empty_like(x) for x in srcs]
+            w.work = lambda: 2 * nbytes
+            w.launches = [P.prepare("afir_bench_tilecopy64", a.data_ptr(), b.data_ptr(), 64, 1024, 512)
+                          for a, b in zip(srcs, dsts)]
+            w.sets = list(zip(srcs, dsts))
+
+            def parity():
+                # every byte of src lands somewhere in dst: compare the byte histograms
+                a = torch.bincount(srcs[0].int(), minlength=256)
+                b = torch.bincount(dsts[0].int(), minlength=256)
+                return {"bar": "dst is a permutation of src (byte histogram)", "passed": bool(torch.equal(a, b)),
+                        "mismatches": int((a != b).sum().item())}
+            w.parity = parity
     else:
         raise SystemExit(f"unknown workload {key}")
     return w
@@ -492,8 +581,9 @@ def summarize(w, wall, ev_ms, steps):
     else:
         value, unit = work * steps / wall / 1e12, "TFLOP/s"
         achieved, peak = work / avg_launch_s / 1e12, MFMA_BF16_PEAK_TFLOPS
+    traffic, source = MEASURED_TRAFFIC.get(w.key, (None, None))
     roof = {"bound": w.bound, "achieved": round(achieved, 2), "peak": peak, "unit": unit,
-            "frac": round(achieved / peak, 4), "traffic": MEASURED_TRAFFIC.get(w.key),
+            "frac": round(achieved / peak, 4), "traffic": traffic, "traffic_source": source,
             "avg_launch_us": round(avg_launch_s * 1e6, 3),
             "work_per_launch": work}
     return value, unit, roof
@@ -504,7 +594,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5", "g1", "g2", "g3", "g4", "i1", "i2"])
+    ap.add_argument("--workload", default="c2", choices=ALL_WORKLOADS)
     ap.add_argument("--all", dest="all", action="store_true", default=True)
     ap.add_argument("--no-all", dest="all", action="store_false")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -539,8 +629,7 @@ def main():
             return args.warmup
         return 5 if key == "c5" else 30
 
-    order = [args.workload] + ([k for k in ["c1", "c2", "c3", "c4", "c5", "g1", "g2", "g3", "g4", "i1", "i2"]
-                                if k != args.workload] if args.all else [])
+    order = [args.workload] + ([k for k in ALL_WORKLOADS if k != args.workload] if args.all else [])
     results = []
     for key in order:
         w = make_workload(key, torch, H, O, C)
@@ -550,12 +639,16 @@ def main():
         par = w.parity()
         extra = (w.power_evidence() if hasattr(w, "power_evidence") and not args.no_power_evidence
                  else None)
-        entry = {"workload": w.title, "value": round(value, 2), "unit": unit, "steps": steps,
+        entry = {"key": key, "workload": w.title, "value": round(value, 2), "unit": unit, "steps": steps,
                  "warmup": warmup, "ms_per_step": round(wall * 1e3 / steps, 5), "dtype": w.dtype,
                  "buffer_sets": w.nsets, "roofline": roof, "parity": par}
         if extra is not None:
             entry["power_limit_evidence"] = extra
-        if not args.no_cpu_baseline:
+            # the same kernel against what the matrix cores sustain on these operands from registers
+            # alone, and against the vendor GEMM (a comparator here, never part of the product path)
+            roof["frac_of_mfma_only"] = round(roof["achieved"] / extra["mfma_only_workload_operands_tflops"], 4)
+            roof["vs_vendor_gemm"] = round(extra["this_kernel_alternating_tflops"] / extra["vendor_gemm_tflops"], 4)
+        if not args.no_cpu_baseline and not getattr(w, "no_cpu", False):
             budget = args.cpu_seconds if key == args.workload else min(3.0, args.cpu_seconds)
             v, sample = w.cpu(budget)
             entry["cpu_baseline"] = {"value": round(v, 4), "unit": unit,
@@ -586,11 +679,25 @@ def main():
                      ("bound", "achieved", "peak", "unit", "frac", "traffic")},
         "parity": main_e["parity"],
     }
+    line["roofline"]["traffic_source"] = main_e["roofline"]["traffic_source"]
     if "cpu_baseline" in main_e:
         line["cpu_baseline"] = {k: main_e["cpu_baseline"][k] for k in
                                 ("value", "unit", "cores", "kind", "sample")}
     line["device"] = torch.cuda.get_device_name(0)
     if args.all:
+        by_key = {e["key"]: e for e in results}
+        # the targets are read on roofline.frac: algorithmic work / average launch duration from HIP
+        # events / published peak (value, the wall-clock figure, also holds the host's launch gaps)
+        line["targets"] = {k: {"frac": by_key[k]["roofline"]["frac"], "target": t,
+                               "met": by_key[k]["roofline"]["frac"] >= t,
+                               "parity": by_key[k]["parity"]["passed"]}
+                           for k, t in TARGETS.items() if k in by_key}
+        line["min_frac_hbm"] = min(v["frac"] for k, v in line["targets"].items() if k != "c5")
+        line["targets_read_on"] = "roofline.frac (HIP events on the launch stream), not value (wall clock)"
+        ceil = {k: by_key[k]["roofline"]["achieved"] for k in ("ceil_copy", "ceil_read", "ceil_tilecopy64")
+                if k in by_key}
+        if ceil:
+            line["measured_ceilings_gbs"] = ceil
         line["workloads"] = results
     print(json.dumps(line))
 

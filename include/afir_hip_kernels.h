@@ -233,19 +233,6 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
                                 void *const *args, void *workspace, const void *tiling,
                                 size_t tiling_len);
 
-/* ---- measurement aid ----------------------------------------------------------
- * No counterpart in the reference.  Launches a kernel that does nothing but
- * issue v_mfma_f32_32x32x16_bf16 from registers on every CU (8 waves per
- * workgroup, two workgroups per CU): `operands` = 65536 bytes of bf16 on the
- * device (the values matter: the sustained clock under the board power limit
- * depends on how much the operands toggle), `sink` = 1 MiB of device memory
- * that receives one float per lane.  *flops receives the floating-point
- * operations the launch performs; the caller times it (events on `stream`). */
-#define AFIR_HIP_MFMA_PROBE_OPERAND_BYTES 65536u
-#define AFIR_HIP_MFMA_PROBE_SINK_BYTES 1048576u
-uint32_t afir_hip_probe_mfma_rate(void *stream, const void *operands, void *sink, uint32_t iters,
-                                  uint64_t *flops);
-
 #ifdef __cplusplus
 }
 #endif
