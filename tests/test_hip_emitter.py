@@ -96,7 +96,8 @@ def test_integer_regions_use_wrapping_integer_arithmetic():
     assert "stv_i16<W>(R.out" in narrow and "ldv_i16<W, " in narrow
     mixed = _emit(RC.INT_MIXED_TO_I16).stdout
     assert "a lane takes 2 groups of 8 elements per pass" in mixed          # 16 bytes of the i16 tensors
-    assert "ldv_i16<W, true>(R.in[0].base" in mixed and "ldd_i32(R.in[1].base" in mixed
+    # one streamed byte per byte written: ordinary loads (no non-temporal hint)
+    assert "ldv_i16<W, false>(R.in[0].base" in mixed and "ldd_i32(R.in[1].base" in mixed
 
 
 def test_reductions_also_get_a_workgroup_per_row_kernel():
