@@ -76,7 +76,7 @@ __global__ __launch_bounds__(kCopyThreads) void probe_copy(const u32x4 *__restri
   for (size_t base = (size_t)blockIdx.x * chunk; base < n16; base += stride) {
     u32x4 v[kCopyUnroll];
 #pragma unroll
-    for (int u = 0; u < kCopyUnroll; ++u) v[u] = afir::load_nt(src + base + u * kCopyThreads + threadIdx.x);
+    for (int u = 0; u < kCopyUnroll; ++u) v[u] = src[base + u * kCopyThreads + threadIdx.x];
 #pragma unroll
     for (int u = 0; u < kCopyUnroll; ++u) afir::store_nt(dst + base + u * kCopyThreads + threadIdx.x, v[u]);
   }
@@ -116,7 +116,7 @@ __global__ __launch_bounds__(kCopyThreads) void probe_tilecopy64(const uint16_t 
     u32x4 v[2];
 #pragma unroll
     for (int k = 0; k < 2; ++k)
-      v[k] = afir::load_nt(reinterpret_cast<const u32x4 *>(x + ((int64_t)b * m + m0 + row + 32 * k) * n + n0 + chunk));
+      v[k] = *reinterpret_cast<const u32x4 *>(x + ((int64_t)b * m + m0 + row + 32 * k) * n + n0 + chunk);
 #pragma unroll
     for (int k = 0; k < 2; ++k)
       afir::store_nt(reinterpret_cast<u32x4 *>(out + ((int64_t)b * n + n0 + row + 32 * k) * m + m0 + chunk), v[k]);

@@ -17,33 +17,54 @@
 // fills 1 KiB of contiguous LDS; which 16-byte chunk of global memory a lane
 // fetches is free, and that is where the bank swizzle goes:
 //   A: chunk c of row r lands at chunk position c ^ ((r>>1)&7);
-//   B: chunk c of row k lands at chunk position c ^ ((k&3)<<2).
-// The A operand of an MFMA is one 128-bit LDS read per lane (8 consecutive k
-// of one m).  The B operand needs 8 consecutive k of one n from a tile whose
-// rows run along n: ds_read_b64_tr_b16 does that transpose in the LDS unit
-// (within 16 lanes, lanes 4r..4r+3 address row r, lane i receives column i of
-// the four rows).  With the swizzles above both reads are bank-conflict free.
+//   B: chunk c of row k lands at chunk position c ^ ((k&3)<<2) ^ (((k>>3)&1)<<1).
+//
+// The matrix instruction is v_mfma_f32_16x16x32_bf16: K = 32 per instruction,
+// a lane holds 8 consecutive k of one row (A) or one column (B), 4 accumulator
+// registers per 16 x 16 tile.  It was chosen over v_mfma_f32_32x32x16_bf16 by
+// measurement: the chip runs this kernel against its board power limit, and
+// on operands drawn from N(0, 1/sqrt(K)) a register-only loop of the 16x16x32
+// form sustains 2040 TFLOP/s where the 32x32x16 form sustains 1765 (on
+// constant operands both reach 2470): per flop the accumulators are read and
+// written half as often.
+// The A operand of an MFMA is one 128-bit LDS read per lane.  The B operand
+// needs 8 consecutive k of one n from a tile whose rows run along n:
+// ds_read_b64_tr_b16 does that transpose in the LDS unit (within 16 lanes,
+// lanes 4r..4r+3 address row r, lane i receives column i of the four rows),
+// two of them four rows apart per operand.  With the swizzles above both
+// reads are bank-conflict free.
 //
 // The compiler cannot be trusted to wait for exactly the right stage (it
 // drains every outstanding direct-to-LDS load before any LDS read that might
-// alias one), so the operand reads are issued from inline asm and the waits
-// are explicit: s_waitcnt vmcnt(n) + s_barrier once per K step of 32, which
-// leaves the two youngest B stages and the youngest A slice in flight.
-// Operand reads are software-pipelined one k16 substep ahead of the MFMAs.
+// alias one), so the operand reads and the direct-to-LDS loads are issued from
+// inline asm and the waits are explicit: s_waitcnt vmcnt(n) + s_barrier once
+// per K step of 32, which leaves the two youngest B stages and the youngest A
+// slice in flight.
+//
+// The K loop is ONE instruction stream per wave in which every operand read
+// and every direct-to-LDS load sits behind an MFMA (pinned with scheduling
+// barriers).  All eight waves pass the workgroup barrier together, so a block
+// of reads or loads issued after it would leave the matrix units of all four
+// SIMDs idle at the same time; behind an MFMA, which occupies the unit for 16
+// cycles, an instruction issues for free.  The reads go behind the first MFMAs
+// of a phase so that the remaining ones cover their latency.  The direct-to-LDS
+// loads take a scalar base (tile, region, K position) plus a 32-bit per-lane
+// offset, so the loop spends no vector registers or instructions on addresses.
+// Measured on MI355X, 8192^3, TFLOP/s on constant / N(0, 1/sqrt(K)) operands:
+// 32x32x16 MFMAs with reads and loads in blocks 1630 / 1235; 16x16x32 in blocks
+// 1565 / 1320; 16x16x32 interleaved as described 1700 / 1350-1365 (the vendor
+// GEMM without the epilogue, same runs: 1775 / 1360-1385).
 //
 // Every tile starts its walk over K at a different offset and wraps around
 // (K-stagger): the row pitch of A and B is a large power of two, so without it
 // all workgroups of the chip ask the same few L2 / memory channels for the
 // same K offset at the same time.
 //
-// 8 waves as 2(m) x 4(n), wave tile 128 x 64 = 4 x 2 MFMA tiles of 32x32,
-// v_mfma_f32_32x32x16_bf16 with the operands swapped (B as the row operand) so
-// that a lane holds four consecutive n of one m for the fused epilogue.
-// (AFIR_MM_WAVES_N=2 builds 4 waves of 128 x 128 instead: a third fewer LDS
-// operand bytes per MFMA, but one wave per SIMD leaves the matrix unit idle
-// around every barrier; measured on MI355X it is 11 % slower on constant
-// operands and equal, within 1 %, on N(0, 1/sqrt(K)) operands, where the board
-// power limit sets the pace.)
+// 8 waves as 2(m) x 4(n), two per SIMD (one wave per SIMD cannot issue 16-cycle
+// MFMAs back to back: 1815 of 2470 TFLOP/s in a register-only loop); wave tile
+// 128 x 64 = 8 x 4 MFMA tiles of 16 x 16, with the operands swapped (B as the
+// row operand) so that a lane holds four consecutive n of one m for the fused
+// epilogue.
 #include <type_traits>
 
 #include "kernels.h"
@@ -73,9 +94,13 @@ constexpr int kSlotB = kBK * kBN * 2;     // 16 KiB
 constexpr int kRingB = kASlots * kSlotA;  // byte offset of the B ring
 constexpr int kLdsBytes = kASlots * kSlotA + kBSlots * kSlotB;  // 160 KiB
 
-typedef __attribute__((address_space(3))) unsigned char lds_byte;
-typedef __attribute__((address_space(3))) void lds_void;
-typedef __attribute__((address_space(1))) const void gbl_void;
+constexpr int kWavesM = 2, kWavesN = 4, kWaves = kWavesM * kWavesN;
+constexpr int kTM = kBM / kWavesM / 16;   // 8: 16-row MFMA tiles per wave along m
+constexpr int kTN = kBN / kWavesN / 16;   // 4: 16-column MFMA tiles per wave along n
+constexpr int kAReg = 32 / kWaves;        // 1 KiB direct-to-LDS regions per wave per A slice
+constexpr int kBReg = 16 / kWaves;        // ... per B stage
+constexpr int kSteadyVm = 2 * kBReg + kAReg;  // loads younger than what the next stage needs
+
 
 __device__ __forceinline__ void map_tile_dma(int p, int tiles_m, int tiles_n, int &tm, int &tn) {
   const int ntiles = tiles_m * tiles_n;
@@ -95,17 +120,6 @@ __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
 }
 
-// Operands of one k16 substep: TMW A fragments (m tiles, 4 KiB apart) and TNW
-// B fragments (n tiles, each two transposing 64-bit reads 4 rows apart).
-// issue_reads only issues; the registers must not be touched until
-// settle_reads, which waits for the LDS unit and hands the same registers back
-// as fresh values.
-template <int TMW, int TNW>
-struct Operands {
-  u32x4 a[TMW];
-  u32x2 b[TNW][2];
-};
-
 template <int OFF>
 __device__ __forceinline__ void read_a(uint32_t addr, u32x4 &dst) {
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(dst) : "v"(addr), "n"(OFF) : "memory");
@@ -115,34 +129,43 @@ __device__ __forceinline__ void read_b(uint32_t addr, u32x2 &dst) {
   asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=&v"(dst) : "v"(addr), "n"(OFF) : "memory");
 }
 
-template <int KS, int TMW, int TNW>  // KS: k16 substep within the B stage (0 or 1)
-__device__ __forceinline__ void issue_reads(uint32_t a_addr, const uint32_t (&b_addr)[TNW],
-                                            Operands<TMW, TNW> &o) {
-  constexpr int kOff = KS * 16 * 512;  // 16 rows of B
-  read_a<0>(a_addr, o.a[0]);
-  read_a<4096>(a_addr, o.a[1]);
-  if constexpr (TMW == 4) {
-    read_a<8192>(a_addr, o.a[2]);
-    read_a<12288>(a_addr, o.a[3]);
-  }
+// Four A fragments: m tiles 2 KiB apart (16 rows of 128 bytes), starting at tile FIRST.
+// The reads only issue; the registers must not be touched until settle().
+template <int FIRST>
+__device__ __forceinline__ void issue_a_reads(uint32_t addr, u32x4 (&a)[4]) {
+  read_a<(FIRST + 0) * 2048>(addr, a[0]);
+  read_a<(FIRST + 1) * 2048>(addr, a[1]);
+  read_a<(FIRST + 2) * 2048>(addr, a[2]);
+  read_a<(FIRST + 3) * 2048>(addr, a[3]);
+}
+// The B fragments of a stage: per n tile two transposing reads, 4 rows apart.
+__device__ __forceinline__ void issue_b_reads(const uint32_t (&addr)[kTN], u32x2 (&b)[kTN][2]) {
 #pragma unroll
-  for (int j = 0; j < TNW; ++j) {
-    read_b<kOff>(b_addr[j], o.b[j][0]);
-    read_b<kOff + 4 * 512>(b_addr[j], o.b[j][1]);
+  for (int j = 0; j < kTN; ++j) {
+    read_b<0>(addr[j], b[j][0]);
+    read_b<4 * 512>(addr[j], b[j][1]);
+  }
+}
+// Waits for the LDS unit and hands the registers back as fresh values: volatile asm
+// statements keep their order, so no use can move above the wait.
+__device__ __forceinline__ void settle_wait() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void settle(u32x4 (&a)[4]) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) asm volatile("" : "+v"(a[i]));
+}
+__device__ __forceinline__ void settle(u32x2 (&b)[kTN][2]) {
+#pragma unroll
+  for (int j = 0; j < kTN; ++j) {
+    asm volatile("" : "+v"(b[j][0]));
+    asm volatile("" : "+v"(b[j][1]));
   }
 }
 
-template <int TMW, int TNW>
-__device__ __forceinline__ void settle_reads(Operands<TMW, TNW> &o) {
-  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-  // volatile asm statements keep their order: every register counts as
-  // rewritten after the wait, so no use can move above it
-#pragma unroll
-  for (int i = 0; i < TMW; ++i) asm volatile("" : "+v"(o.a[i]));
-#pragma unroll
-  for (int j = 0; j < TNW; ++j) {
-    asm volatile("" : "+v"(o.b[j][0]));
-    asm volatile("" : "+v"(o.b[j][1]));
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+  if constexpr (I < N) {
+    f(std::integral_constant<int, I>{});
+    static_for<I + 1, N>(f);
   }
 }
 
@@ -151,49 +174,59 @@ struct Par1 { static constexpr int value = 1; };
 struct Steady { static constexpr bool value = true; };
 struct Drain { static constexpr bool value = false; };
 
-// WM x WN waves (m x n), wave tile (256/WM) x (256/WN): 2 x 4 waves of
-// 128 x 64, or 2 x 2 waves of 128 x 128 (one wave per SIMD, two thirds of the
-// LDS operand bytes per MFMA).
-//
 // F16IO = false: A, B, bias, out are bf16.  F16IO = true: A, B are f16, bias and
 // out are float32 (the types of the reference's own matmul example,
 // examples/matmul-add-leakyrelu/step0_input.mlir:10-15): the same rings and
 // reads (both element types are 16 bits wide), the f16 MFMA, and an epilogue
 // that stores the float32 value unrounded.
-template <int WM, int WN, bool F16IO>
-__global__ __launch_bounds__(WM * WN * 64) void matmul_bias_leakyrelu_dma(
+template <bool F16IO>
+__global__ __launch_bounds__(kWaves * 64) void matmul_bias_leakyrelu_dma(
     const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
     const void *__restrict__ bias_v, void *__restrict__ out_v, int M, int K, int N,
     float alpha, int relu, int tiles_m, int tiles_n) {
   extern __shared__ __align__(1024) unsigned char smem[];
-  lds_byte *const lds = (lds_byte *)smem;
-  const uint32_t lds_base = (uint32_t)(uintptr_t)lds;
+  // (address space 3 pointers are 32 bits wide: the value is the LDS byte address)
+  const uint32_t lds_base =
+      (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
 
   const int t = threadIdx.x, lane = t & 63;
-  constexpr int TMW = 8 / WM;            // 32-row MFMA tiles per wave along m
-  constexpr int TNW = 8 / WN;            // 32-column MFMA tiles per wave along n
-  constexpr int NWAVES = WM * WN;
-  constexpr int A_REG = 32 / NWAVES;     // 1 KiB direct-to-LDS regions per wave per A slice
-  constexpr int B_REG = 16 / NWAVES;     // ... per B stage
-  constexpr int kSteadyVm = 2 * B_REG + A_REG;  // loads younger than what the next stage needs
   const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-  const int wm = wave / WN, wn = wave % WN;
+  const int wm = wave / kWavesN, wn = wave % kWavesN;
   const int KT = K / kBK;   // B stages; even, the launcher requires K % 64 == 0
   const int KT2 = KT >> 1;  // A slices
 
   // ---- per-lane operand read addresses, relative to a ring slot ----
-  const int lrow = lane & 31, lk = lane >> 5;
-  // substep ks (0..3) of the slice reads chunk 2*ks + lk:  a_rd ^ (ks * 32)
-  const uint32_t a_rd =
-      (uint32_t)((wm * TMW * 32 + lrow) * 128 + (lk ^ ((lrow >> 1) & 7)) * 16);
-  const int g = lane >> 4, li = lane & 15;
-  uint32_t b_rd[TNW];
+  // A fragment of m tile i: lane reads row i*16 + lane%16, the 16-byte chunk lane/16 of the
+  // stage's 64 bytes (the second stage of a slice: chunk + 4, i.e. address ^ 64)
+  const int li = lane & 15, g = lane >> 4;
+  const uint32_t a_rd = (uint32_t)((wm * (kTM * 16) + li) * 128 + (g ^ ((li >> 1) & 7)) * 16);
+  // B fragment of n tile j: the 16-lane group g takes rows 8g .. 8g+3 (second read: +4),
+  // lanes 4r .. 4r+3 of it the 32 bytes of row r that hold the tile's 16 columns
+  // (n tile j: the tile's two chunks are 2j further on, and since those bits of the unswizzled
+  // chunk index are zero for tile 0, the swizzled address of tile j is that of tile 0 ^ 32j)
+  uint32_t b_rd0;
+  {
+    const int row = g * 8 + (li >> 2);
+    const int c16 = (wn * kTN) * 2 + ((li & 3) >> 1);
+    const int phys = c16 ^ ((row & 3) << 2) ^ (((row >> 3) & 1) << 1);
+    b_rd0 = (uint32_t)(kRingB + row * 512 + phys * 16 + (li & 1) * 8);
+  }
+
+  // ---- per-lane parts of the direct-to-LDS source addresses (bytes) ----
+  // An address is a wave-uniform base (tile, region, K position: scalar registers, advanced
+  // with scalar arithmetic) plus a 32-bit per-lane offset that depends only on the lane and on
+  // the parity of the region (row within the region, swizzled chunk), so the loads take the
+  // scalar-base form and the K loop spends no vector registers or instructions on them.
+  uint32_t a_lane[2], b_lane[2];
 #pragma unroll
-  for (int j = 0; j < TNW; ++j) {
-    const int ntile = wn * TNW + j;
-    const int c16 = ntile * 4 + (g & 1) * 2 + ((li & 3) >> 1);
-    const int phys = c16 ^ ((li >> 2) << 2);
-    b_rd[j] = (uint32_t)(kRingB + ((g >> 1) * 8 + (li >> 2)) * 512 + phys * 16 + (li & 1) * 8);
+  for (int par = 0; par < 2; ++par) {
+    // regions of a wave start at a multiple of kAReg * 8 rows (a multiple of 16): only the
+    // parity of the region enters the swizzle
+    const int arow = par * 8 + (lane >> 3);
+    a_lane[par] = (uint32_t)(((int64_t)(lane >> 3) * K + ((lane & 7) ^ ((arow >> 1) & 7)) * 8) * 2);
+    const int bk = (wave * kBReg + par) * 2 + (lane >> 5);
+    b_lane[par] = (uint32_t)(((int64_t)(lane >> 5) * N +
+                              ((lane & 31) ^ ((bk & 3) << 2) ^ (((bk >> 3) & 1) << 1)) * 8) * 2);
   }
 
   for (int p = blockIdx.x; p < tiles_m * tiles_n; p += gridDim.x) {
@@ -207,84 +240,69 @@ __global__ __launch_bounds__(WM * WN * 64) void matmul_bias_leakyrelu_dma(
         (int)(((unsigned)(tile_m * AFIR_MM_KSTAGGER_M + tile_n * AFIR_MM_KSTAGGER_N) * 2u) %
               (unsigned)KT);
 
-    // ---- per-lane global sources of the direct-to-LDS loads ----
-    // A slice: 32 regions of 1 KiB (8 rows x 128 B), A_REG per wave.
-    // B stage: 16 regions of 1 KiB (2 rows x 512 B), B_REG per wave.
-    const uint16_t *ga[A_REG], *gb[B_REG];
-#pragma unroll
-    for (int q = 0; q < A_REG; ++q) {
-      const int arow = (wave * A_REG + q) * 8 + (lane >> 3);
-      const int ac = (lane & 7) ^ ((arow >> 1) & 7);
-      ga[q] = A + (int64_t)(m0 + arow) * K + ac * 8 + (int64_t)kfirst * kBK;
-    }
-#pragma unroll
-    for (int q = 0; q < B_REG; ++q) {
-      const int bk = (wave * B_REG + q) * 2 + (lane >> 5);
-      const int bc = (lane & 31) ^ ((bk & 3) << 2);
-      gb[q] = B + (int64_t)(bk + kfirst * kBK) * N + n0 + bc * 8;
-    }
+    // ---- wave-uniform sources of the direct-to-LDS loads ----
+    // A slice: 32 regions of 1 KiB (8 rows x 128 B), kAReg per wave.
+    // B stage: 16 regions of 1 KiB (2 rows x 512 B), kBReg per wave.
+    const char *ua = reinterpret_cast<const char *>(A) +
+                     ((int64_t)(m0 + wave * (kAReg * 8)) * K + (int64_t)kfirst * kBK) * 2;
+    const char *ub = reinterpret_cast<const char *>(B) +
+                     ((int64_t)(wave * (kBReg * 2) + kfirst * kBK) * N + n0) * 2;
+    const int64_t a_region = (int64_t)K * 16;   // 8 rows of A
+    const int64_t b_region = (int64_t)N * 4;    // 2 rows of B
     int ka_next = kfirst >> 1;  // slice (64 k) the next A issue fetches
     int kb_next = kfirst;       // stage (32 k) the next B issue fetches
 
-    auto issue_a = [&](int slot) {
-      lds_byte *dst = lds + slot * kSlotA + wave * (A_REG * 1024);
-#pragma unroll
-      for (int q = 0; q < A_REG; ++q)
-        __builtin_amdgcn_global_load_lds((gbl_void *)ga[q], (lds_void *)(dst + q * 1024), 16, 0, 0);
+    // one region: lane l's 16 bytes go to lds_offset + 16 l
+    auto dma = [&](const char *base, uint32_t lane_offset, uint32_t lds_offset) {
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                   :
+                   : "s"(lds_offset), "v"(lane_offset), "s"(base)
+                   : "memory");
+    };
+    auto issue_a_region = [&](int slot, auto q_tag) {
+      constexpr int q = decltype(q_tag)::value;
+      dma(ua + q * a_region, a_lane[q & 1],
+          lds_base + (uint32_t)(slot * kSlotA + wave * (kAReg * 1024) + q * 1024));
+    };
+    auto advance_a = [&]() {
       ka_next = (ka_next + 1 == KT2) ? 0 : ka_next + 1;
-      const int64_t step = (ka_next == 0) ? -(int64_t)(KT2 - 1) * 64 : (int64_t)64;
-#pragma unroll
-      for (int q = 0; q < A_REG; ++q) ga[q] += step;
+      ua += (ka_next == 0) ? -(int64_t)(KT2 - 1) * 128 : (int64_t)128;
+    };
+    auto issue_b_region = [&](int slot, auto q_tag) {
+      constexpr int q = decltype(q_tag)::value;
+      dma(ub + q * b_region, b_lane[q & 1],
+          lds_base + (uint32_t)(kRingB + slot * kSlotB + wave * (kBReg * 1024) + q * 1024));
+    };
+    auto advance_b = [&]() {
+      kb_next = (kb_next + 1 == KT) ? 0 : kb_next + 1;
+      ub += ((kb_next == 0) ? -(int64_t)(KT - 1) : (int64_t)1) * kBK * N * 2;
+    };
+    auto issue_a = [&](int slot) {
+      static_for<0, kAReg>([&](auto q) { issue_a_region(slot, q); });
+      advance_a();
     };
     auto issue_b = [&](int slot) {
-      lds_byte *dst = lds + kRingB + slot * kSlotB + wave * (B_REG * 1024);
-#pragma unroll
-      for (int q = 0; q < B_REG; ++q)
-        __builtin_amdgcn_global_load_lds((gbl_void *)gb[q], (lds_void *)(dst + q * 1024), 16, 0, 0);
-      kb_next = (kb_next + 1 == KT) ? 0 : kb_next + 1;
-      const int64_t step = (kb_next == 0) ? -(int64_t)(KT - 1) * kBK * N : (int64_t)kBK * N;
-#pragma unroll
-      for (int q = 0; q < B_REG; ++q) gb[q] += step;
+      static_for<0, kBReg>([&](auto q) { issue_b_region(slot, q); });
+      advance_b();
     };
 
-    f32x16 acc[TMW][TNW];
+    f32x4 acc[kTM][kTN];
 #pragma unroll
-    for (int i = 0; i < TMW; ++i)
+    for (int i = 0; i < kTM; ++i)
 #pragma unroll
-      for (int j = 0; j < TNW; ++j)
+      for (int j = 0; j < kTN; ++j)
 #pragma unroll
-        for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+        for (int e = 0; e < 4; ++e) acc[i][j][e] = 0.f;
 
-    auto multiply = [&](const Operands<TMW, TNW> &o) {
-#pragma unroll
-      for (int j = 0; j < TNW; ++j) {
-        const u32x4 bw = {o.b[j][0].x, o.b[j][0].y, o.b[j][1].x, o.b[j][1].y};
-#pragma unroll
-        for (int i = 0; i < TMW; ++i) {
-          if constexpr (F16IO)
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                __builtin_bit_cast(f16x8, bw), __builtin_bit_cast(f16x8, o.a[i]), acc[i][j], 0, 0, 0);
-          else
-            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                __builtin_bit_cast(bf16x8, bw), __builtin_bit_cast(bf16x8, o.a[i]), acc[i][j], 0, 0,
-                0);
-        }
-      }
+    // LDS addresses of a stage held in A slot sa / B slot sbk; the stage is the first
+    // (par 0) or second (par 1) half of its A slice
+    auto a_address = [&](int sa, int par) {
+      return lds_base + (uint32_t)(sa * kSlotA) + (a_rd ^ (uint32_t)(par * 64));
     };
-    // operand reads for a stage held in A slot sa / B slot sbk; the stage is the
-    // first (par 0) or second (par 1) half of its A slice; h = k16 substep
-    auto reads = [&](int sa, int sbk, int par, int h, Operands<TMW, TNW> &o, bool prologue = false) {
-      if (AFIR_MM_ABLATE >= 2 && !prologue) return;
-      const uint32_t aa =
-          lds_base + (uint32_t)(sa * kSlotA) + (a_rd ^ (uint32_t)((par * 2 + h) * 32));
-      const uint32_t bb = lds_base + (uint32_t)(sbk * kSlotB);
-      uint32_t ba[TNW];
+    auto b_addresses = [&](int sbk, uint32_t (&ba)[kTN]) {
+      const uint32_t bb = lds_base + (uint32_t)(sbk * kSlotB) + b_rd0;   // ring slots are 1 KiB aligned
 #pragma unroll
-      for (int j = 0; j < TNW; ++j) ba[j] = bb + b_rd[j];
-      if (h == 0)
-        issue_reads<0>(aa, ba, o);
-      else
-        issue_reads<1>(aa, ba, o);
+      for (int j = 0; j < kTN; ++j) ba[j] = bb ^ (uint32_t)(j * 32);
     };
 
     // prologue (the launcher guarantees KT >= 8): fill both rings, oldest first
@@ -295,131 +313,231 @@ __global__ __launch_bounds__(WM * WN * 64) void matmul_bias_leakyrelu_dma(
     issue_b(2);
     issue_b(3);
     issue_a(2);
-    wait_vmcnt<3 * B_REG + 2 * A_REG>();  // everything younger than A(0), B(0)
+    wait_vmcnt<3 * kBReg + 2 * kAReg>();  // everything younger than A(0), B(0)
     __builtin_amdgcn_s_barrier();
-    Operands<TMW, TNW> even, odd;
-    reads(0, 0, 0, 0, even, true);
-    settle_reads(even);
-    if (AFIR_MM_ABLATE >= 2) odd = even;
+    // Operand registers: the A fragments of a stage in two halves (m tiles 0-3, 4-7), the B
+    // fragments of a stage twice (the stage being multiplied and the next one).
+    u32x4 a_lo[4], a_hi[4];
+    u32x2 b_cur[kTN][2], b_nxt[kTN][2];
+    {
+      uint32_t ba[kTN];
+      b_addresses(0, ba);
+      issue_a_reads<0>(a_address(0, 0), a_lo);
+      issue_b_reads(ba, b_cur);
+      settle_wait();
+      settle(a_lo);
+      settle(b_cur);
+    }
+    if (AFIR_MM_ABLATE >= 2) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a_hi[i] = a_lo[i];
+#pragma unroll
+      for (int j = 0; j < kTN; ++j) {
+        b_nxt[j][0] = b_cur[j][0];
+        b_nxt[j][1] = b_cur[j][1];
+      }
+    }
 
-    // One step of the pipeline for stage s of parity PAR:
-    //   reads(s, substep 1) in flight | MFMAs(s, substep 0)
+    // One step of the pipeline for stage s (parity PAR within its A slice), the B
+    // fragments of s in `bs`, those of s+1 going to `bn`:
+    //   reads of A(s) m tiles 4-7 in flight | MFMAs of m tiles 0-3
     //   wait until stage s+1 has landed, barrier: everyone is done reading s
-    //   reads(s+1, substep 0) in flight, refill the freed slots | MFMAs(s, substep 1)
+    //   reads of A(s+1) m tiles 0-3 and B(s+1) in flight, refill the freed slots
+    //                                        | MFMAs of m tiles 4-7
     // Refill after stage s: B(s+4) into s's B slot; after an odd s also the A
     // slice (s+5)/2 into the slot of the slice just finished.  In the steady
     // state both exist and the vmcnt is exact: younger than what stage s+1 needs
     // are exactly 2 B stages and 1 A slice.  Otherwise drain.
     int sa = 0, sb = 0;  // ring slots of the stage being multiplied
-    auto step = [&](auto par_tag, auto mode_tag, bool has_next, bool refill_b, bool refill_a) {
+    auto pin = [] { __builtin_amdgcn_sched_barrier(0); };
+    // MFMA number X of a phase: n tile X / 4, m tile FIRST + X % 4
+    auto mfma = [&](auto first_tag, auto x_tag, const u32x4 (&a)[4], const u32x2 (&b)[kTN][2]) {
+      constexpr int FIRST = decltype(first_tag)::value, X = decltype(x_tag)::value, j = X / 4, i = X % 4;
+      const u32x4 bw = {b[j][0].x, b[j][0].y, b[j][1].x, b[j][1].y};
+      if constexpr (F16IO)
+        acc[FIRST + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+            __builtin_bit_cast(f16x8, bw), __builtin_bit_cast(f16x8, a[i]), acc[FIRST + i][j], 0, 0, 0);
+      else
+        acc[FIRST + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            __builtin_bit_cast(bf16x8, bw), __builtin_bit_cast(bf16x8, a[i]), acc[FIRST + i][j], 0, 0, 0);
+    };
+    // Refills wait for the step after the one that frees their slots, so that they can go out
+    // behind the MFMAs of phase 1, which carries few operand reads: pend_b / pend_a say what the
+    // previous step left to issue, pend_sa / pend_sb into which slots.
+    bool pend_a = false, pend_b = false;
+    int pend_sa = 0, pend_sb = 0;
+    // pend_tag: what is known at compile time about the refills the previous step left: 0 none
+    // (the first step of a tile), 1 those of the steady state (a B stage; an A slice after an
+    // odd stage), 2 whatever pend_a / pend_b say
+    auto step = [&](auto par_tag, auto mode_tag, auto pend_tag, u32x2 (&bs)[kTN][2], u32x2 (&bn)[kTN][2],
+                    bool has_next, bool refill_b, bool refill_a) {
       constexpr int PAR = decltype(par_tag)::value;
       constexpr bool STEADY = decltype(mode_tag)::value;
+      constexpr int PEND = decltype(pend_tag)::value;
+      constexpr int NM = 4 * kTN;   // MFMAs per phase
       const int sb_next = (sb + 1 == kBSlots) ? 0 : sb + 1;
       const int sa_next = PAR ? ((sa + 1 == kASlots) ? 0 : sa + 1) : sa;
-      reads(sa, sb, PAR, 1, odd);
-      __builtin_amdgcn_sched_barrier(0);
-      multiply(even);
-      __builtin_amdgcn_sched_barrier(0);
-      settle_reads(odd);
-      if (STEADY || has_next) {
-        if (STEADY)
-          wait_vmcnt<kSteadyVm>();
-        else
-          wait_vmcnt<0>();
-        __builtin_amdgcn_s_barrier();
-        reads(sa_next, sb_next, PAR ^ 1, 0, even);
-        if (AFIR_MM_ABLATE == 0) {
-          if (PAR && (STEADY || refill_a)) issue_a(sa);
-          if (STEADY || refill_b) issue_b(sb);
-        }
+      // ---- phase 1: m tiles 0-3.  One item behind each MFMA: the reads of m tiles 4-7 first
+      // (they have the rest of the phase to come back), then the refills the previous step
+      // left (its A slice, if any, before its B stage).
+      {
+        const uint32_t aa = a_address(sa, PAR);
+        const bool do_a = AFIR_MM_ABLATE == 0 && (PEND == 1 ? !PAR : PEND == 2 && pend_a);
+        const bool do_b = AFIR_MM_ABLATE == 0 && (PEND == 1 || (PEND == 2 && pend_b));
+        pin();
+        static_for<0, NM>([&](auto x) {
+          constexpr int X = decltype(x)::value;
+          mfma(std::integral_constant<int, 0>{}, x, a_lo, bs);
+          pin();
+          if constexpr (X < 4) {
+            if (AFIR_MM_ABLATE < 2) read_a<(4 + X) * 2048>(aa, a_hi[X]);
+            pin();
+          } else if constexpr (!PAR && X < 4 + kAReg) {   // the step before an even stage was odd: A slice
+            if (do_a) issue_a_region(pend_sa, std::integral_constant<int, X - 4>{});
+            pin();
+          } else if constexpr (X >= 4 + kAReg && X < 4 + kAReg + kBReg) {
+            if (do_b) issue_b_region(pend_sb, std::integral_constant<int, X - 4 - kAReg>{});
+            pin();
+          }
+        });
+        if (do_a) advance_a();
+        if (do_b) advance_b();
       }
-      multiply(odd);
-      __builtin_amdgcn_sched_barrier(0);
-      if (STEADY || has_next) settle_reads(even);
+      pin();
+      settle_wait();
+      settle(a_hi);
+      pin();
+      // ---- phase 2: m tiles 4-7.  Behind the first MFMA: wait until stage s+1 has landed,
+      // barrier (everyone is done reading s); then one operand read of stage s+1 behind each
+      // of the next twelve MFMAs, in the order the next phase uses them.
+      if (STEADY || has_next) {
+        uint32_t ba[kTN];
+        b_addresses(sb_next, ba);
+        const uint32_t aa = a_address(sa_next, PAR ^ 1);
+        static_for<0, NM>([&](auto x) {
+          constexpr int X = decltype(x)::value;
+          mfma(std::integral_constant<int, 4>{}, x, a_hi, bs);
+          pin();
+          if constexpr (X == 0) {
+            if (STEADY)
+              wait_vmcnt<kSteadyVm>();
+            else
+              wait_vmcnt<0>();
+            __builtin_amdgcn_s_barrier();
+            pin();
+          }
+          if constexpr (X < 12) {
+            constexpr int R = X;   // B tile 0, A tiles 0-3, B tiles 1-3
+            if (AFIR_MM_ABLATE < 2) {
+              if constexpr (R < 2) read_b<R * 4 * 512>(ba[0], bn[0][R]);
+              else if constexpr (R < 6) read_a<(R - 2) * 2048>(aa, a_lo[R - 2]);
+              else read_b<((R - 6) % 2) * 4 * 512>(ba[1 + (R - 6) / 2], bn[1 + (R - 6) / 2][(R - 6) % 2]);
+            }
+            pin();
+          }
+        });
+        pend_b = STEADY || refill_b;
+        pend_a = PAR && (STEADY || refill_a);
+        pend_sa = sa;
+        pend_sb = sb;
+        pin();
+        settle_wait();
+        settle(a_lo);
+        settle(bn);
+      } else {
+        static_for<0, NM>([&](auto x) { mfma(std::integral_constant<int, 4>{}, x, a_hi, bs); });
+        pend_a = pend_b = false;
+      }
+      pin();
       sa = sa_next;
       sb = sb_next;
     };
 
-    int s = 0;
+    using Pend0 = std::integral_constant<int, 0>;
+    using Pend1 = std::integral_constant<int, 1>;
+    using Pend2 = std::integral_constant<int, 2>;
+    // KT >= 8 (the launcher checks): the first two stages are steady ones
+    step(Par0{}, Steady{}, Pend0{}, b_cur, b_nxt, true, true, true);
+    step(Par1{}, Steady{}, Pend1{}, b_nxt, b_cur, true, true, true);
+    int s = 2;
     for (; s + 6 < KT; s += 2) {  // both refills exist: B(s+4), B(s+5), A((s+6)/2)
-      step(Par0{}, Steady{}, true, true, true);
-      step(Par1{}, Steady{}, true, true, true);
+      step(Par0{}, Steady{}, Pend1{}, b_cur, b_nxt, true, true, true);
+      step(Par1{}, Steady{}, Pend1{}, b_nxt, b_cur, true, true, true);
     }
     for (; s < KT; s += 2) {
-      step(Par0{}, Drain{}, true, s + 4 < KT, false);
-      step(Par1{}, Drain{}, s + 2 < KT, s + 5 < KT, s + 6 < KT);
+      step(Par0{}, Drain{}, Pend2{}, b_cur, b_nxt, true, s + 4 < KT, false);
+      step(Par1{}, Drain{}, Pend2{}, b_nxt, b_cur, s + 2 < KT, s + 5 < KT, s + 6 < KT);
     }
 
-    // Epilogue.  A lane holds m = lane%32, n = 8q + 4*(lane/32) + e of each
-    // 32x32 block, i.e. 8 bytes (bf16) or 16 bytes (float32) of an output row
-    // per store: written straight to memory that is a fraction of a line per row
-    // per instruction, and the partial lines of the bf16 form cost three times
-    // the write traffic.  So each wave stages 32 rows of its tile (64 n = one
-    // or two 128-byte lines per row) in LDS and stores them as full lines,
-    // eight or four rows per instruction.  The rings are free once every wave
-    // has left the K loop; a wave's 4 or 8 KiB staging area is private, and
-    // the LDS unit keeps a wave's accesses in order, so no further barrier is
-    // needed until the next tile refills the rings.  The 16-byte chunk column
-    // is XOR-ed with a function of the row: conflict-free for the 8- or
-    // 16-byte writes (32 rows x 2 halves) and for the 16-byte row reads.
+    // Epilogue.  Of each 16 x 16 block a lane holds m = lane%16 and the four
+    // consecutive n = 4*(lane/16) + e, i.e. 8 bytes (bf16) or 16 bytes (float32)
+    // of an output row: written straight to memory that is a fraction of a line
+    // per row per instruction, and the partial lines of the bf16 form cost three
+    // times the write traffic.  So each wave stages 32 rows of its tile (two m
+    // tiles; 64 n = one or two 128-byte lines per row) in LDS and stores them as
+    // full lines, eight or four rows per instruction.  The rings are free once
+    // every wave has left the K loop; a wave's 4 or 8 KiB staging area is
+    // private, and the LDS unit keeps a wave's accesses in order, so no further
+    // barrier is needed until the next tile refills the rings.  The 16-byte
+    // chunk column is XOR-ed with a function of the row: conflict-free for the
+    // 8- or 16-byte writes and for the 16-byte row reads.
     __builtin_amdgcn_s_barrier();
     {
       constexpr int kOutBytes = F16IO ? 4 : 2;
-      constexpr int CH = TNW * 32 * kOutBytes / 16;   // 16-byte chunks per staged row
-      constexpr int kRowBytes = CH * 16;       // 128 .. 512
+      constexpr int CH = kTN * 16 * kOutBytes / 16;   // 16-byte chunks per staged row: 8 or 16
+      constexpr int kRowBytes = CH * 16;       // 128 or 256
       constexpr int kRowsPerPass = 64 / CH;    // rows one store instruction covers
       unsigned char *const stage = smem + wave * (32 * kRowBytes);
-      const int lm = lane & 31, lq = lane >> 5;
       const int rr = lane / CH, cc = lane % CH;
       // two 128-byte rows share a swizzle value (they span the same banks as
       // one 256-byte row)
       auto swz = [](int r) { return CH == 8 ? ((r >> 1) & 7) : (r & (CH - 1)); };
       typedef typename std::conditional<F16IO, f32x4, u32x2>::type BiasRaw;
-      BiasRaw braw[TNW][4];
+      BiasRaw braw[kTN];
 #pragma unroll
-      for (int j = 0; j < TNW; ++j)
+      for (int j = 0; j < kTN; ++j) {
+        const int n = n0 + (wn * kTN + j) * 16 + 4 * g;
+        // no bias: -0, the identity of the add
+        if constexpr (F16IO)
+          braw[j] = bias_v ? *reinterpret_cast<const f32x4 *>(static_cast<const float *>(bias_v) + n)
+                           : f32x4{-0.f, -0.f, -0.f, -0.f};
+        else
+          braw[j] = bias_v ? *reinterpret_cast<const u32x2 *>(static_cast<const uint16_t *>(bias_v) + n)
+                           : u32x2{0x80008000u, 0x80008000u};
+      }
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int n = n0 + (wn * TNW + j) * 32 + 8 * q + 4 * lq;
-          // no bias: -0, the identity of the add
-          if constexpr (F16IO)
-            braw[j][q] = bias_v ? *reinterpret_cast<const f32x4 *>(static_cast<const float *>(bias_v) + n)
-                                : f32x4{-0.f, -0.f, -0.f, -0.f};
-          else
-            braw[j][q] = bias_v ? *reinterpret_cast<const u32x2 *>(static_cast<const uint16_t *>(bias_v) + n)
-                                : u32x2{0x80008000u, 0x80008000u};
-        }
+      for (int ip = 0; ip < kTM / 2; ++ip) {
 #pragma unroll
-      for (int i = 0; i < TMW; ++i) {
+        for (int half = 0; half < 2; ++half) {
+          const int lm = half * 16 + li;   // row within the 32 staged rows
 #pragma unroll
-        for (int j = 0; j < TNW; ++j) {
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
+          for (int j = 0; j < kTN; ++j) {
             float b0, b1, b2, b3;
             if constexpr (F16IO) {
-              b0 = braw[j][q][0]; b1 = braw[j][q][1]; b2 = braw[j][q][2]; b3 = braw[j][q][3];
+              b0 = braw[j][0]; b1 = braw[j][1]; b2 = braw[j][2]; b3 = braw[j][3];
             } else {
-              b0 = bf16_lo(braw[j][q].x); b1 = bf16_hi(braw[j][q].x);
-              b2 = bf16_lo(braw[j][q].y); b3 = bf16_hi(braw[j][q].y);
+              b0 = bf16_lo(braw[j].x); b1 = bf16_hi(braw[j].x);
+              b2 = bf16_lo(braw[j].y); b3 = bf16_hi(braw[j].y);
             }
-            float v0 = acc[i][j][4 * q + 0] + b0;
-            float v1 = acc[i][j][4 * q + 1] + b1;
-            float v2 = acc[i][j][4 * q + 2] + b2;
-            float v3 = acc[i][j][4 * q + 3] + b3;
+            const f32x4 &c = acc[ip * 2 + half][j];
+            float v0 = c[0] + b0;
+            float v1 = c[1] + b1;
+            float v2 = c[2] + b2;
+            float v3 = c[3] + b3;
             v0 = fmaxf(v0, relu ? 0.f : v0 * alpha);
             v1 = fmaxf(v1, relu ? 0.f : v1 * alpha);
             v2 = fmaxf(v2, relu ? 0.f : v2 * alpha);
             v3 = fmaxf(v3, relu ? 0.f : v3 * alpha);
             if constexpr (F16IO) {
               const f32x4 w = {v0, v1, v2, v3};
-              const int chunk = (j * 8 + q * 2 + lq) ^ swz(lm);
+              const int chunk = (j * 4 + g) ^ swz(lm);
               *reinterpret_cast<f32x4 *>(stage + lm * kRowBytes + chunk * 16) = w;
             } else {
               u32x2 w;
               w.x = pack_bf16(v0, v1);
               w.y = pack_bf16(v2, v3);
-              const int chunk = (j * 4 + q) ^ swz(lm);
-              *reinterpret_cast<u32x2 *>(stage + lm * kRowBytes + chunk * 16 + lq * 8) = w;
+              const int chunk = (j * 2 + (g >> 1)) ^ swz(lm);
+              *reinterpret_cast<u32x2 *>(stage + lm * kRowBytes + chunk * 16 + (g & 1) * 8) = w;
             }
           }
         }
@@ -428,9 +546,9 @@ __global__ __launch_bounds__(WM * WN * 64) void matmul_bias_leakyrelu_dma(
           const int r = rr + kRowsPerPass * tq;
           const u32x4 line =
               *reinterpret_cast<const u32x4 *>(stage + r * kRowBytes + ((cc ^ swz(r)) * 16));
-          const int m = m0 + (wm * TMW + i) * 32 + r;
+          const int m = m0 + (wm * kTM + ip * 2) * 16 + r;
           unsigned char *const row = static_cast<unsigned char *>(out_v) +
-                                     ((int64_t)m * N + n0 + wn * (TNW * 32)) * kOutBytes;
+                                     ((int64_t)m * N + n0 + wn * (kTN * 16)) * kOutBytes;
           *reinterpret_cast<u32x4 *>(row + cc * 16) = line;
         }
       }
@@ -446,12 +564,6 @@ bool matmul_dma_supported(int64_t m, int64_t k, int64_t n) {
   return m % kBM == 0 && n % kBN == 0 && k % 64 == 0 && k >= 8 * kBK;
 }
 
-#ifndef AFIR_MM_WAVES_M
-#define AFIR_MM_WAVES_M 2
-#endif
-#ifndef AFIR_MM_WAVES_N
-#define AFIR_MM_WAVES_N 4
-#endif
 #ifndef AFIR_MM_GRID
 #define AFIR_MM_GRID kNumCU
 #endif
@@ -462,8 +574,7 @@ template <bool F16IO>
 LaunchStatus launch_dma(const uint16_t *a, const uint16_t *b, const void *bias, void *out, int m,
                         int k, int n, float alpha, bool relu, uint32_t block_dim,
                         hipStream_t stream) {
-  constexpr int WM = AFIR_MM_WAVES_M, WN = AFIR_MM_WAVES_N;
-  auto kernel = matmul_bias_leakyrelu_dma<WM, WN, F16IO>;
+  auto kernel = matmul_bias_leakyrelu_dma<F16IO>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize,
                                                kLdsBytes);
@@ -474,7 +585,7 @@ LaunchStatus launch_dma(const uint16_t *a, const uint16_t *b, const void *bias, 
   int64_t blocks = (int64_t)tiles_m * tiles_n;
   if (blocks > AFIR_MM_GRID) blocks = AFIR_MM_GRID;
   if (block_dim) blocks = block_dim;
-  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(WM * WN * 64), kLdsBytes, stream, a, b,
+  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kWaves * 64), kLdsBytes, stream, a, b,
                      bias, out, m, k, n, alpha, relu ? 1 : 0, tiles_m, tiles_n);
   return after_launch();
 }
