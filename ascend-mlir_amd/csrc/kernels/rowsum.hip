@@ -11,6 +11,9 @@
 // lane total is reduced across the wave with DPP (quad butterflies, row
 // mirrors) and the four 16-lane row totals are combined in a fixed order, so
 // the result is deterministic.  The broadcast operand is never materialised.
+#include <mutex>
+
+#include "afir_hip_kernels.h"
 #include "kernels.h"
 
 namespace afir {
@@ -224,3 +227,131 @@ LaunchStatus launch_broadcast_add_reducesum(const float *x, const float *bias, f
 }
 
 }  // namespace afir
+
+// ---- the entry point that allocates nothing ---------------------------------
+//
+// Few, long rows cannot fill the chip with a wavefront or a workgroup per row,
+// so the row is cut into chunks of kSplitChunk floats, one workgroup sums one
+// chunk (bias included) and leaves a float in a scratch buffer, and a second
+// kernel adds a row's partial sums in a fixed order.  The scratch buffer is a
+// file-scope device array, so this path needs no allocation and no workspace
+// from the caller; every GPU holds its own copy at its own address, looked up
+// once per device with hipGetSymbolAddress.  In host code `afir_rowsum_scratch`
+// is only the handle for that lookup, never an address to pass to a kernel.
+namespace afir {
+namespace {
+
+constexpr int kSplitThreads = 256;
+constexpr int kSplitUnroll = 8;                                  // 128-bit loads in flight per lane
+constexpr int64_t kSplitChunk = (int64_t)kSplitThreads * 4 * kSplitUnroll;   // 8192 floats = 32 KiB
+constexpr int64_t kScratchFloats = 65536;                        // 256 KiB per GPU (the array below)
+
+}  // namespace
+}  // namespace afir
+
+static __device__ __align__(256) float afir_rowsum_scratch[65536];
+static_assert(sizeof(afir_rowsum_scratch) == 65536 * sizeof(float), "the scratch array holds 65536 partial sums");
+
+namespace afir {
+namespace {
+
+// partial[row * parts + p] = sum over chunk p of row `row` of (x + bias); the last chunk may be short
+__global__ __launch_bounds__(kSplitThreads) void bcast_add_rowsum_f32_split(
+    const float *__restrict__ x, const float *__restrict__ bias, float *__restrict__ partial,
+    int64_t n, int parts) {
+  __shared__ float part[kSplitThreads / kWave];
+  const int t = threadIdx.x;
+  const int64_t row = blockIdx.x / (unsigned)parts;
+  const int p = (int)(blockIdx.x - row * (unsigned)parts);
+  const int64_t first = (int64_t)p * kSplitChunk;
+  const int64_t n4 = (n - first < kSplitChunk ? n - first : kSplitChunk) >> 2;   // 128-bit chunks here
+  const f32x4 *x4 = reinterpret_cast<const f32x4 *>(x + row * n + first);
+  const f32x4 *b4 = reinterpret_cast<const f32x4 *>(bias + first);
+  const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+  f32x4 vx[kSplitUnroll], vb[kSplitUnroll];
+#pragma unroll
+  for (int u = 0; u < kSplitUnroll; ++u) {
+    const int64_t c = t + (int64_t)u * kSplitThreads;
+    vx[u] = c < n4 ? load_nt(x4 + c) : zero;
+    vb[u] = c < n4 ? b4[c] : zero;
+  }
+  f32x4 acc = zero;
+#pragma unroll
+  for (int u = 0; u < kSplitUnroll; ++u) acc += vx[u] + vb[u];
+  float s = wave_sum((acc.x + acc.y) + (acc.z + acc.w));
+  if ((t & (kWave - 1)) == 0) part[t >> 6] = s;
+  __syncthreads();
+  if (t == 0) partial[blockIdx.x] = (part[0] + part[1]) + (part[2] + part[3]);
+}
+
+// y[row] = the row's partial sums, lane l adding those at l, l + 64, ..., then the wave reduction
+__global__ __launch_bounds__(kSplitThreads) void bcast_add_rowsum_f32_join(
+    const float *__restrict__ partial, float *__restrict__ y, int64_t m, int parts) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t row = (int64_t)blockIdx.x * (kSplitThreads / kWave) + (threadIdx.x >> 6);
+  if (row >= m) return;
+  float s = 0.f;
+  for (int p = lane; p < parts; p += kWave) s += partial[row * parts + p];
+  s = wave_sum(s);
+  if (lane == 0) y[row] = s;
+}
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+float *g_scratch[kMaxDevices];   // per device: where that GPU keeps afir_rowsum_scratch
+
+// The current device's copy of the scratch array (looked up on the first call per device).
+LaunchStatus scratch_of_current_device(float **out) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return LaunchStatus{2u, hipGetErrorString(e)};
+  if (device < 0 || device >= kMaxDevices) return invalid("broadcast_add_reducesum_noalloc: device ordinal out of range");
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch[device]) {
+    float *p = nullptr;
+    e = hipGetSymbolAddress(reinterpret_cast<void **>(&p), HIP_SYMBOL(afir_rowsum_scratch));
+    if (e != hipSuccess || !p) {
+      (void)hipGetLastError();
+      return LaunchStatus{2u, e != hipSuccess ? hipGetErrorString(e) : "no address for the scratch array"};
+    }
+    g_scratch[device] = p;
+  }
+  *out = g_scratch[device];
+  return ok_status();
+}
+
+}  // namespace
+}  // namespace afir
+
+extern "C" uint32_t afir_hip_launch_broadcast_add_reducesum_noalloc(uint32_t block_dim, void *stream, void *x,
+                                                                    void *bias, void *y, void * /*workspace*/,
+                                                                    void *tiling) {
+  using namespace afir;
+  // (errors: the code only; this entry point keeps no message and touches no heap)
+  if (!tiling) return AFIR_HIP_E_INVALID;
+  int64_t f[2];
+  __builtin_memcpy(f, tiling, sizeof f);
+  const int64_t m = f[0], n = f[1];
+  if (m < 0 || n < 0) return AFIR_HIP_E_INVALID;
+  if (m == 0) return AFIR_HIP_OK;
+  if (!y || (n > 0 && (!x || !bias))) return AFIR_HIP_E_INVALID;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const bool vec = n > 0 && n % 4 == 0 && aligned16(x) && aligned16(bias);
+  // few rows of at least two chunks: split and join through the scratch array
+  if (vec && m < 1024 && n >= 2 * kSplitChunk && !block_dim) {
+    const int64_t parts = (n + kSplitChunk - 1) / kSplitChunk;
+    if (m * parts > kScratchFloats) return AFIR_HIP_E_NOALLOC_LIMIT;
+    float *scratch = nullptr;
+    const LaunchStatus got = scratch_of_current_device(&scratch);
+    if (got.code) return got.code == 1 ? AFIR_HIP_E_INVALID : AFIR_HIP_E_LAUNCH;
+    hipLaunchKernelGGL(bcast_add_rowsum_f32_split, dim3((unsigned)(m * parts)), dim3(kSplitThreads), 0, st,
+                       static_cast<const float *>(x), static_cast<const float *>(bias), scratch, n, (int)parts);
+    hipLaunchKernelGGL(bcast_add_rowsum_f32_join, dim3((unsigned)((m + 3) / 4)), dim3(kSplitThreads), 0, st,
+                       scratch, static_cast<float *>(y), m, (int)parts);
+    return hipGetLastError() == hipSuccess ? AFIR_HIP_OK : AFIR_HIP_E_LAUNCH;
+  }
+  // every other shape runs on kernels that need no scratch memory
+  const LaunchStatus done = launch_broadcast_add_reducesum(static_cast<const float *>(x), static_cast<const float *>(bias),
+                                                          static_cast<float *>(y), m, n, block_dim, st);
+  return done.code == 0 ? AFIR_HIP_OK : done.code == 1 ? AFIR_HIP_E_INVALID : AFIR_HIP_E_LAUNCH;
+}

@@ -32,6 +32,7 @@ EXPORTED_SYMBOLS = [
     "afir_hip_last_error",
     "afir_hip_launch_fused_add_mul",
     "afir_hip_launch_broadcast_add_reducesum",
+    "afir_hip_launch_broadcast_add_reducesum_noalloc",
     "afir_hip_launch_relu_broadcast_add_transpose",
     "afir_hip_launch_gather_scale_shift",
     "afir_hip_launch_matmul_add_leakyrelu",
@@ -70,6 +71,7 @@ def load():
     L.afir_hip_last_error.restype = ctypes.c_char_p
     for name, nptr in [("afir_hip_launch_fused_add_mul", 5),
                        ("afir_hip_launch_broadcast_add_reducesum", 5),
+                       ("afir_hip_launch_broadcast_add_reducesum_noalloc", 5),
                        ("afir_hip_launch_relu_broadcast_add_transpose", 5),
                        ("afir_hip_launch_gather_scale_shift", 7),
                        ("afir_hip_launch_matmul_add_leakyrelu", 6)]:

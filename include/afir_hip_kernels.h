@@ -81,6 +81,27 @@ uint32_t afir_hip_launch_broadcast_add_reducesum(uint32_t block_dim, void *strea
                                                  void *x, void *bias, void *y,
                                                  void *workspace, void *tiling);
 
+/* The same computation for callers that must not allocate (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  No
+ * counterpart in the reference.  The launcher above may load a code object on
+ * first use and its split-and-join form for few, long rows keeps partial sums
+ * in that code object; this one calls no hipMalloc, hipFree or other
+ * allocating routine.  Rows are split when M < 1024 and N >= 16384 (chunks of
+ * 8192 floats, one partial sum each, added in a fixed order by a second
+ * kernel); the partial sums live in a 256 KiB array that the library holds on
+ * every GPU it runs on until the process ends, so M * ceil(N / 8192) must not
+ * exceed 65536: beyond that the call returns AFIR_HIP_E_NOALLOC_LIMIT and
+ * launches nothing.  Other shapes run the scratch-free kernels of the launcher
+ * above.  `workspace` is ignored.  Every call on a GPU shares that GPU's array
+ * (nothing in it has to start at zero: each partial sum is written before it
+ * is read), so calls that overlap on one GPU -- other streams, other threads
+ * -- race; serialise them.  Returns the code only: afir_hip_last_error() is
+ * not updated. */
+#define AFIR_HIP_E_NOALLOC_LIMIT 4u
+uint32_t afir_hip_launch_broadcast_add_reducesum_noalloc(uint32_t block_dim, void *stream,
+                                                         void *x, void *bias, void *y,
+                                                         void *workspace, void *tiling);
+
 /* ---- relu + broadcast add + transpose ------------------------------------
  * out[b,j,i] = f16(relu(x[b,i,j]) + c[j]); x f16 [B,M,N], c f16 [N],
  * out f16 [B,N,M].  Replaces the parallel generic with a PureTranspose input
