@@ -888,6 +888,13 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
       }
       d.depth = op.depth;
     }
+    a.ntail = 0;
+    for (const afir_region::ResolvedSegment::TailStep &t : seg.tail) {
+      afir::RegionOp &d = a.tail[a.ntail++];   // at most kMaxTailOps = kRegionMaxTail (validate)
+      d.code = region_op_code(t.code, false);
+      d.constant = t.constant;
+      d.depth = t.reversed ? 1 : 0;
+    }
     if (compiled) {
       const int segment = (int)(&seg - res.segments.data());
       const afir_target::SpecShape shape = afir_target::specShape(r->program, segment, emit);
@@ -915,6 +922,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
         sa.out = ra.out;
         sa.error_flag = ra.error_flag;
         sa.out_vec = ra.out_vec;
+        afir_target::specTailConstants(r->program, segment, res.shapes, sa.tail_const);
         sa.lanes_log2 = g.lanes_log2;
         sa.grid = (int)g.blocks;
         sa.column_blocks = (int)g.column_blocks;

@@ -433,6 +433,19 @@ __global__ __launch_bounds__(kThreads) void fused_region_parallel(const RegionAr
   }
 }
 
+// What a reduce segment does to a row's sum before storing it (mean = sum / N, ...).
+__device__ __forceinline__ float apply_tail(const RegionArgs &R, float s) {
+  for (int k = 0; k < R.ntail; ++k) {
+    const RegionOp &op = R.tail[k];
+    float a[1] = {op.depth ? op.constant : s};
+    const float b[1] = {op.depth ? s : op.constant};
+    if (region_is_binary(op.code)) binary<1>(op.code, a, b);
+    else unary<1>(op.code, op.constant, a);
+    s = a[0];
+  }
+  return s;
+}
+
 // Row sum over the innermost dim: 2^lanes_log2 lanes of a wavefront per output
 // element (the whole wavefront for rows of 64 vectors or more, fewer lanes and
 // several rows per wavefront for shorter rows), the lanes stride over the row in
@@ -475,7 +488,7 @@ __global__ __launch_bounds__(kThreads) void fused_region_rowsum(const RegionArgs
     } else {
       for (int m = lanes >> 1; m >= 1; m >>= 1) s += __shfl_xor(s, m);
     }
-    if ((lane & (lanes - 1)) == 0) store_elem(R.out, R.out_type, (int64_t)row, s);
+    if ((lane & (lanes - 1)) == 0) store_elem(R.out, R.out_type, (int64_t)row, apply_tail(R, s));
   }
 }
 

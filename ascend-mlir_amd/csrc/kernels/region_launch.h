@@ -11,6 +11,7 @@ namespace afir {
 
 constexpr int kRegionMaxInputs = 8;
 constexpr int kRegionMaxOps = 32;
+constexpr int kRegionMaxTail = 8;
 
 enum RegionType : int { kRegionF16 = 0, kRegionBF16 = 1, kRegionF32 = 2, kRegionI32 = 3, kRegionI64 = 4, kRegionI16 = 5 };
 // Values travel through float registers; an integer region keeps 32-bit two's
@@ -92,6 +93,11 @@ struct RegionArgs {
   int reduce;
   RegionInput in[kRegionMaxInputs];
   RegionOp ops[kRegionMaxOps];
+  // reduce segments: what happens to a row's sum s before it is stored, step by step:
+  // s = s (code) constant, or constant (code) s with depth = 1, or a unary operation
+  int ntail;
+  int pad_tail;
+  RegionOp tail[kRegionMaxTail];
   // filled in by the launcher
   int chain;              // 1: the fields below describe the whole expression
   int chain_first;        // x0: index into `in`, or -1 for chain_constant

@@ -40,6 +40,7 @@ struct SpecArgs {
   int grid;
   int column_blocks;
   SpecInput in[8];
+  float tail_const[4];
 };
 
 DEV float as_f32(unsigned u) { return __builtin_bit_cast(float, u); }
@@ -669,6 +670,7 @@ class SegmentEmitter {
       }
     };
     for (const Op &op : seg_.ops) {
+      if (op.code == OpCode::ReduceSum) break;   // what follows works on the row's sum: tailExpression
       switch (op.code) {
         case OpCode::Push:
           stack.push_back(read[pushSlot_[push++]]);
@@ -735,6 +737,49 @@ class SegmentEmitter {
       }
     }
     return stack.back();
+  }
+
+  // The operations after 'reduce sum' as a C expression in the row's sum `s`: constants are
+  // literals, extent constants R.tail_const[k] in program order.  `s` itself when there are none.
+  std::string tailExpression(const std::string &s) const {
+    std::vector<std::string> stack;
+    bool after = false;
+    int extent = 0;
+    for (const Op &op : seg_.ops) {
+      if (op.code == OpCode::ReduceSum) {
+        after = true;
+        stack.assign(1, s);
+        continue;
+      }
+      if (!after || op.code == OpCode::Store) continue;
+      switch (op.code) {
+        case OpCode::Const:
+          stack.push_back(op.extent ? "R.tail_const[" + std::to_string(extent++) + "]" : floatLiteral(op.constant));
+          break;
+        case OpCode::Dup:
+          stack.push_back(stack[stack.size() - 1 - op.depth]);
+          break;
+        case OpCode::Relu: stack.back() = "fmax_ieee(" + stack.back() + ", 0.f)"; break;
+        case OpCode::Leaky:
+          stack.back() = "fmax_ieee(" + stack.back() + ", (" + stack.back() + ") * " + floatLiteral(op.constant) + ")";
+          break;
+        case OpCode::Neg: stack.back() = "(-" + stack.back() + ")"; break;
+        default: {
+          const std::string b = stack.back();
+          stack.pop_back();
+          const std::string a = stack.back();
+          switch (op.code) {
+            case OpCode::Add: stack.back() = "(" + a + " + " + b + ")"; break;
+            case OpCode::Sub: stack.back() = "(" + a + " - " + b + ")"; break;
+            case OpCode::Mul: stack.back() = "(" + a + " * " + b + ")"; break;
+            case OpCode::Div: stack.back() = "(" + a + " / " + b + ")"; break;
+            case OpCode::Max: stack.back() = "fmax_ieee(" + a + ", " + b + ")"; break;
+            default: stack.back() = "fmin_ieee(" + a + ", " + b + ")"; break;
+          }
+        }
+      }
+    }
+    return after ? stack.back() : s;
   }
 
   void emitPositionOfRow(int d, const std::string &row = "row") {
@@ -822,7 +867,7 @@ class SegmentEmitter {
       unroll();
       line(3, "for (int e = 0; e < w; ++e) acc[0][e] = acc[0][2 * e] + acc[0][2 * e + 1];");
       line(2, "const float s = R.lanes_log2 == 6 ? wave_sum(acc[0][0]) : lanes_sum(acc[0][0], lane, (int)lanes);");
-      line(2, "if ((lane & ((int)lanes - 1)) == 0) st_" + otag + "(R.out, (long long)row, s);");
+      line(2, "if ((lane & ((int)lanes - 1)) == 0) st_" + otag + "(R.out, (long long)row, " + tailExpression("s") + ");");
       line(1, "}");
       os_ << "}\n";
       return;
@@ -1009,7 +1054,10 @@ class SegmentEmitter {
     line(2, "__builtin_amdgcn_fence(__ATOMIC_RELEASE, \"workgroup\");");
     line(2, "__builtin_amdgcn_s_barrier();");
     line(2, "__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, \"workgroup\");");
-    line(2, "if (tid == 0) st_" + otag + "(R.out, (long long)row, (part[parity][0] + part[parity][1]) + (part[parity][2] + part[parity][3]));");
+    line(2, "if (tid == 0) {");
+    line(3, "const float s = (part[parity][0] + part[parity][1]) + (part[parity][2] + part[parity][3]);");
+    line(3, "st_" + otag + "(R.out, (long long)row, " + tailExpression("s") + ");");
+    line(2, "}");
     line(2, "parity ^= 1;");
     line(1, "}");
     os_ << "}\n";
@@ -1093,7 +1141,10 @@ class SegmentEmitter {
     line(3, "__builtin_amdgcn_fence(__ATOMIC_RELEASE, \"workgroup\");");
     line(3, "__builtin_amdgcn_s_barrier();");
     line(3, "__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, \"workgroup\");");
-    line(3, "if (tid == 0) st_" + otag + "(R.out, (long long)row, (part[parity][0] + part[parity][1]) + (part[parity][2] + part[parity][3]));");
+    line(3, "if (tid == 0) {");
+    line(4, "const float s = (part[parity][0] + part[parity][1]) + (part[parity][2] + part[parity][3]);");
+    line(4, "st_" + otag + "(R.out, (long long)row, " + tailExpression("s") + ");");
+    line(3, "}");
     line(3, "parity ^= 1;");
     unroll();
     line(3, "for (int e = 0; e < W; ++e) acc[e] = 0.f;");
@@ -1198,7 +1249,7 @@ class SegmentEmitter {
     line(1, "float s = 0.f;");
     line(1, "for (I c = (I)lane; c < cblocks; c += 64) s += afir_region_partials[(long long)row * (long long)cblocks + (long long)c];");
     line(1, "s = wave_sum(s);");
-    line(1, "if (lane == 0) st_" + otag + "(R.out, (long long)row, s);");
+    line(1, "if (lane == 0) st_" + otag + "(R.out, (long long)row, " + tailExpression("s") + ");");
     os_ << "}\n";
   }
 
@@ -1446,6 +1497,18 @@ bool specAllSegments(const Program &p) {
     if (specTile(p, s).tiled) return false;   // LDS tiles of several segments would add up
   }
   return true;
+}
+
+void specTailConstants(const Program &p, int segment, const std::vector<std::vector<int64_t>> &shapes,
+                       float (&out)[kSpecMaxTailConsts]) {
+  for (float &v : out) v = 0.f;
+  int n = 0;
+  bool after = false;
+  for (const Op &op : p.segments[segment].ops) {
+    if (op.code == OpCode::ReduceSum) after = true;
+    if (after && op.code == OpCode::Const && op.extent && n < kSpecMaxTailConsts)
+      out[n++] = afir_region::roundThroughType((float)shapes[op.constRef.arg][op.constRef.dim], op.constType);
+  }
 }
 
 uint64_t programHash(const Program &p) {

@@ -40,7 +40,10 @@ struct Index {
 struct Expr;
 using ExprP = std::shared_ptr<const Expr>;
 struct Expr {
-  enum Kind { Input, Constant, Unary, Binary, Matmul } kind = Constant;
+  // Reduced: the row sum a tail expression works on; ExtentConst: an extent as a number
+  enum Kind { Input, Constant, Unary, Binary, Matmul, Reduced, ExtentConst } kind = Constant;
+  Ref extent;               // ExtentConst
+  ElemType extentType = ElemType::F32;   // ... rounded through this type (arith.sitofp ... to f16)
   int arg = -1, arg2 = -1;
   std::vector<Index> idx;   // Input: one per dim of the argument
   std::vector<Ref> slice;   // Input: start offsets (empty = none)
@@ -56,6 +59,7 @@ struct Tensor {
   bool filled = false;
   float fill = 0.f;
   bool reduced = false;            // expr is the summand over iterSizes
+  ExprP tail;                      // reduced: what happens to the row's sum (an expression in Expr::Reduced), or null
   std::vector<Ref> iterSizes;
   std::vector<std::shared_ptr<Tensor>> parts;  // tensor.concat along dim 0
   int directArg = -1;
@@ -63,7 +67,8 @@ struct Tensor {
 using TensorP = std::shared_ptr<Tensor>;
 
 struct Value {
-  enum Kind { None, TensorV, Float, Int, Extent, IndexV, Scalar, Accumulator } kind = None;
+  // ExtentFloat: an extent converted to a float type (arith.sitofp of a cast tensor.dim)
+  enum Kind { None, TensorV, Float, Int, Extent, ExtentFloat, IndexV, Scalar, Accumulator } kind = None;
   TensorP tensor;
   double number = 0.0;   // Float / Int
   ElemType elem = ElemType::F32;
@@ -164,7 +169,7 @@ ExprP makeBinary(OpCode op, ExprP a, ExprP b) {
 // space, its expression in the new space.
 ExprP substitute(const ExprP &e, const std::vector<Index> &with) {
   switch (e->kind) {
-    case Expr::Constant: return e;
+    case Expr::Constant: case Expr::Reduced: case Expr::ExtentConst: return e;
     case Expr::Matmul: {
       for (size_t i = 0; i < with.size(); ++i)
         if (with[i].kind != Index::Dim || with[i].dim != (int)i)
@@ -641,6 +646,37 @@ class Translator {
       v.kind = Value::Extent;
       v.extent = tv->shape[(size_t)cv.number];
       define(one(), v);
+    } else if (op == "arith.index_cast" || op == "arith.sitofp" || op == "arith.uitofp") {
+      // an extent as a number, outside any generic: index -> iN -> float (mean = sum / N,
+      // examples/broadcast-add-reduce/step0_input_mean.mlir:73-74)
+      Value &src = lookup(r_.ssa());
+      r_.expect(':');
+      parseType();
+      if (!r_.eatWord("to")) r_.fail("expected 'to' in " + op);
+      TypeInfo to = parseType();
+      Value v;
+      if (op == "arith.index_cast") {
+        if (src.kind != Value::Extent && src.kind != Value::Int) r_.fail("arith.index_cast of a value that is not an extent");
+        v = src;
+      } else if (src.kind == Value::Int) {
+        v.kind = Value::Float;
+        float f = (float)src.number;
+        if (to.elemName == "f16") f = roundThroughF16(f);
+        else if (to.elemName == "bf16") f = roundThroughBf16(f);
+        else if (to.elemName != "f32") r_.fail("unsupported float type " + to.elemName);
+        v.number = f;
+        v.scalar = makeConst(f);
+      } else {
+        if (src.kind != Value::Extent) r_.fail(op + " of a value that is not an extent");
+        if (src.extent.arg < 0) r_.fail(op + ": internal error, constant extent");
+        v.kind = Value::ExtentFloat;
+        v.extent = src.extent;
+        if (to.elemName == "f16") v.elem = ElemType::F16;
+        else if (to.elemName == "bf16") v.elem = ElemType::BF16;
+        else if (to.elemName == "f32") v.elem = ElemType::F32;
+        else r_.fail("unsupported float type " + to.elemName);
+      }
+      define(one(), v);
     } else if (op == "tensor.empty") {
       r_.expect('(');
       std::vector<Ref> dyn;
@@ -855,8 +891,16 @@ class Translator {
     if (maps.size() != ins.names.size() + 1) r_.fail("linalg.generic: one indexing map per operand is required");
     const int rank = (int)iterators.size();
     if (rank < 1 || rank > afir_region::kMaxRank) r_.fail("linalg.generic: iteration rank must be 1..3");
-    for (const AffineMap &m : maps)
+    for (AffineMap &m : maps) {
+      // A map declared over more dims than there are iterators is taken as one over the
+      // iterators when it uses no other dim: the reference's mean example reads its row sums
+      // through the two-dim map (d0, d1) -> (d0) in a one-iterator generic
+      // (examples/broadcast-add-reduce/step0_input_mean.mlir:76-80).
+      bool inside = m.numDims > rank;
+      for (const Index &ix : m.results) inside = inside && (ix.kind != Index::Dim || ix.dim < rank);
+      if (inside) m.numDims = rank;
       if (m.numDims != rank) r_.fail("linalg.generic: affine map does not match the iterator count");
+    }
     bool reduction = false;
     for (int i = 0; i < rank; ++i) {
       if (iterators[i] == "reduction") {
@@ -889,6 +933,7 @@ class Translator {
 
     body_.clear();
     inBody_ = true;
+    TensorP reducedOperand;   // set when an operand is the result of a reduction
     for (size_t i = 0; i < ins.names.size(); ++i) {
       Value v;
       const TensorP &t = inT[i];
@@ -904,6 +949,19 @@ class Translator {
         v.index.indexArg = t->directArg;
         v.blockArgOperand = (int)i;
       } else {
+        if (t->expr && t->reduced && t->parts.empty() && !reduction) {
+          // the row sums of a reduction, consumed elementwise (mean = sum / N): the generic
+          // must walk exactly the sums' index space and read nothing else
+          if (reducedOperand || !maps[i].isIdentity() || rank != (int)t->shape.size())
+            r_.fail("a reduced value can only be consumed through an identity map, once");
+          reducedOperand = t;
+          v.kind = Value::Scalar;
+          auto e = std::make_shared<Expr>();
+          e->kind = Expr::Reduced;
+          v.scalar = e;
+          body_[blockArgs[i]] = v;
+          continue;
+        }
         if (!t->expr || t->reduced || !t->parts.empty())
           r_.fail("operand " + ins.names[i] + " is not an elementwise value (uninitialised, reduced or concatenated)");
         v.kind = Value::Scalar;
@@ -947,7 +1005,16 @@ class Translator {
     auto tv = std::make_shared<Tensor>();
     tv->elem = outT->elem;
     tv->shape = outT->shape;
-    if (!reduction) {
+    if (!reduction && reducedOperand) {
+      if (yieldedAccumulates) r_.fail("a parallel generic must not read its output");
+      if (!outMap.isIdentity()) r_.fail("linalg.generic: only an identity output map is supported for parallel generics");
+      if (containsInput(yielded)) r_.fail("a generic that consumes a reduced value may combine it with constants and extents only");
+      tv->reduced = true;
+      tv->expr = reducedOperand->expr;
+      tv->iterSizes = reducedOperand->iterSizes;
+      // a tail on a tail: the earlier one takes the place of the sum
+      tv->tail = reducedOperand->tail ? replaceReduced(yielded, reducedOperand->tail) : yielded;
+    } else if (!reduction) {
       if (yieldedAccumulates) r_.fail("a parallel generic must not read its output");
       if (!outMap.isIdentity()) r_.fail("linalg.generic: only an identity output map is supported for parallel generics");
       tv->expr = yielded;
@@ -1056,9 +1123,40 @@ class Translator {
     body_[result] = out;
   }
 
+  static bool containsInput(const ExprP &e) {
+    if (e->kind == Expr::Input || e->kind == Expr::Matmul) return true;
+    if (e->kind == Expr::Unary) return containsInput(e->a);
+    if (e->kind == Expr::Binary) return containsInput(e->a) || containsInput(e->b);
+    return false;
+  }
+  static bool containsReduced(const ExprP &e) {
+    if (e->kind == Expr::Reduced) return true;
+    if (e->kind == Expr::Unary) return containsReduced(e->a);
+    if (e->kind == Expr::Binary) return containsReduced(e->a) || containsReduced(e->b);
+    return false;
+  }
+  static ExprP replaceReduced(const ExprP &e, const ExprP &with) {
+    if (e->kind == Expr::Reduced) return with;
+    if (e->kind == Expr::Unary) return makeUnary(e->op, replaceReduced(e->a, with), e->value);
+    if (e->kind == Expr::Binary) {
+      auto r = std::make_shared<Expr>(*e);
+      r->a = replaceReduced(e->a, with);
+      r->b = replaceReduced(e->b, with);
+      return r;
+    }
+    return e;
+  }
+
   ExprP scalarOf(const Value &v) {
     if (v.kind == Value::Scalar) return v.scalar;
     if (v.kind == Value::Float) return makeConst((float)v.number);
+    if (v.kind == Value::ExtentFloat) {
+      auto e = std::make_shared<Expr>();
+      e->kind = Expr::ExtentConst;
+      e->extent = v.extent;
+      e->extentType = v.elem;
+      return e;
+    }
     r_.fail("expected a floating-point scalar");
   }
 
@@ -1271,6 +1369,15 @@ class Translator {
         o.constant = e->value;
         ops->push_back(o);
         return;
+      case Expr::Reduced:
+        return;   // the row's sum: already on the stack when the tail starts
+      case Expr::ExtentConst:
+        o.code = OpCode::Const;
+        o.extent = true;
+        o.constRef = e->extent;
+        o.constType = e->extentType;
+        ops->push_back(o);
+        return;
       case Expr::Matmul:
         if (!ops->empty()) r_.fail("a matmul must be the first value of its fused region");
         o.code = OpCode::Matmul;
@@ -1309,6 +1416,23 @@ class Translator {
           if (containsMatmul(e->b)) bFirst = true;
           else if (!containsMatmul(e->a) && stackNeed(e->b) > stackNeed(e->a)) bFirst = true;
         }
+        // in a tail the sum is on the stack before anything else: it has to be the first
+        // operand evaluated, which a commuting operation can arrange and 'c - sum' cannot
+        if (containsReduced(e->b) && !containsReduced(e->a)) {
+          if (e->op == OpCode::Sub) {   // c - s is (-s) + c, exactly
+            emitExpr(e->b, ops);
+            o.code = OpCode::Neg;
+            ops->push_back(o);
+            emitExpr(e->a, ops);
+            o.code = OpCode::Add;
+            ops->push_back(o);
+            return;
+          }
+          if (e->op == OpCode::Div) r_.fail("a constant divided by a reduced value is not supported");
+          bFirst = true;
+        } else if (containsReduced(e->a)) {
+          bFirst = false;
+        }
         emitExpr(bFirst ? e->b : e->a, ops);
         emitExpr(bFirst ? e->a : e->b, ops);
         o.code = e->op;
@@ -1336,7 +1460,9 @@ class Translator {
     if (t->reduced) {
       o.code = OpCode::ReduceSum;
       g.ops.push_back(o);
+      if (t->tail) emitExpr(t->tail, &g.ops);
     }
+    o = afir_region::Op();
     o.code = OpCode::Store;
     g.ops.push_back(o);
     p->segments.push_back(std::move(g));

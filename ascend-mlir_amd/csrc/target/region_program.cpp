@@ -4,6 +4,7 @@
 
 #include <algorithm>
 #include <cerrno>
+#include <cmath>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -139,7 +140,13 @@ std::string serialize(const Program &p) {
         case OpCode::Matmul:
           s += "matmul arg" + std::to_string(o.arg) + " arg" + std::to_string(o.arg2) + "\n";
           break;
-        case OpCode::Const: s += "const " + floatText(o.constant) + "\n"; break;
+        case OpCode::Const:
+          if (o.extent)
+            s += "const " + refText(o.constRef) +
+                 (o.constType == ElemType::F32 ? std::string() : std::string(" ") + elemTypeName(o.constType)) + "\n";
+          else
+            s += "const " + floatText(o.constant) + "\n";
+          break;
         case OpCode::Leaky: s += "leaky " + floatText(o.constant) + "\n"; break;
         case OpCode::Dup: s += "dup " + std::to_string(o.depth) + "\n"; break;
         case OpCode::ReduceSum: s += "reduce sum\n"; break;
@@ -251,6 +258,15 @@ std::string parse(const std::string &text, Program *out) {
       if (tok.size() != 3 || !parseArgName(tok[1], &o.arg) || !parseArgName(tok[2], &o.arg2))
         return err(lineno, "expected 'matmul arg<A> arg<B>'");
       seg->ops.push_back(o);
+    } else if (k == "const" && tok.size() >= 2 && tok[1].compare(0, 3, "arg") == 0) {
+      Op o;
+      o.code = OpCode::Const;
+      o.extent = true;
+      if (tok.size() > 3 || !parseRef(tok[1], &o.constRef) || o.constRef.arg < 0)
+        return err(lineno, "expected 'const arg<A>.<D> [f16|bf16|f32]'");
+      if (tok.size() == 3 && (!parseElemType(tok[2], &o.constType) || !isFloat(o.constType)))
+        return err(lineno, "an extent constant is rounded through f16, bf16 or f32");
+      seg->ops.push_back(o);
     } else if (k == "const" || k == "leaky") {
       Op o;
       o.code = k == "const" ? OpCode::Const : OpCode::Leaky;
@@ -317,11 +333,46 @@ std::string validate(const Program &p) {
       if (!refOk(r)) return "region program: bad output offset reference";
     if (g.ops.empty() || g.ops.back().code != OpCode::Store) return "region program: a segment must end with 'store'";
     if ((int)g.ops.size() > kMaxOps) return "region program: too many operations in a segment";
-    int depth = 0, pushes = 0;
+    int depth = 0, pushes = 0, tailOps = 0, tailExtents = 0;
     bool reduced = false;
+    // after 'reduce sum': which stack entries derive from the sum (exactly one does at any time)
+    std::vector<bool> fromSum;
     for (size_t i = 0; i < g.ops.size(); ++i) {
       const Op &o = g.ops[i];
-      if (reduced && o.code != OpCode::Store) return "region program: only 'store' may follow 'reduce sum'";
+      if (reduced) {
+        // the tail: the row's sum combined with constants and extents
+        if (o.code == OpCode::Push || o.code == OpCode::Matmul || o.code == OpCode::ReduceSum)
+          return "region program: after 'reduce sum' only operations on constants and extents may follow";
+        // (operations among constants are folded when the shapes are known and do not count)
+        switch (o.code) {
+          case OpCode::Const:
+            fromSum.push_back(false);
+            if (o.extent && ++tailExtents > kMaxTailExtents)
+              return "region program: more than " + std::to_string(kMaxTailExtents) + " extent constants after 'reduce sum'";
+            break;
+          case OpCode::Dup:
+            if (o.depth >= 0 && o.depth < (int)fromSum.size()) {
+              if (fromSum[fromSum.size() - 1 - o.depth])
+                return "region program: the operations after 'reduce sum' must form a chain on the sum (no 'dup' of it)";
+              fromSum.push_back(false);
+            }
+            break;
+          case OpCode::Add: case OpCode::Sub: case OpCode::Mul: case OpCode::Div: case OpCode::Max: case OpCode::Min:
+            if (fromSum.size() >= 2) {
+              const bool b = fromSum.back();
+              fromSum.pop_back();
+              fromSum.back() = fromSum.back() || b;
+              if (fromSum.back()) ++tailOps;
+            }
+            break;
+          case OpCode::Relu: case OpCode::Leaky: case OpCode::Neg:
+            if (!fromSum.empty() && fromSum.back()) ++tailOps;
+            break;
+          default: break;
+        }
+        if (tailOps > kMaxTailOps)
+          return "region program: more than " + std::to_string(kMaxTailOps) + " operations on the sum after 'reduce sum'";
+      }
       switch (o.code) {
         case OpCode::Push: {
           if (o.arg < 0 || o.arg >= p.numInputs()) return "region program: push of a non-input argument";
@@ -365,6 +416,12 @@ std::string validate(const Program &p) {
           break;
         }
         case OpCode::Const:
+          if (o.extent) {
+            if (integer) return "region program: an extent constant is not available in an integer region";
+            if (!refOk(o.constRef) || o.constRef.arg < 0) return "region program: bad extent constant";
+            ++depth;
+            break;
+          }
           if (integer && (o.constant != (float)(int32_t)o.constant || o.constant >= 2147483648.f || o.constant < -2147483648.f))
             return "region program: a constant of an integer region must be a 32-bit integer";
           ++depth;
@@ -388,6 +445,7 @@ std::string validate(const Program &p) {
           if (depth != 1) return "region program: 'reduce sum' needs exactly one value";
           if (g.rank < 2) return "region program: a reduction needs an iteration rank of at least 2";
           reduced = true;
+          fromSum.assign(1, true);
           break;
         case OpCode::Store:
           if (i + 1 != g.ops.size()) return "region program: 'store' must be last";
@@ -401,6 +459,38 @@ std::string validate(const Program &p) {
     if (p.output().rank != outRank) return "region program: output rank does not match the segment";
   }
   return "";
+}
+
+float roundThroughType(float f, ElemType t) {
+  if (t != ElemType::F16 && t != ElemType::BF16) return f;
+  uint32_t x;
+  std::memcpy(&x, &f, 4);
+  if (t == ElemType::BF16) {
+    if ((x & 0x7fffffffu) > 0x7f800000u) return f;   // nan
+    x += 0x7fffu + ((x >> 16) & 1u);
+    x &= 0xffff0000u;
+    std::memcpy(&f, &x, 4);
+    return f;
+  }
+  const uint32_t sign = x & 0x80000000u;
+  x &= 0x7fffffffu;
+  if (x >= 0x7f800000u) return f;                       // inf / nan
+  if (x >= 0x477ff000u) {                               // rounds to >= 65520: inf
+    const uint32_t inf = sign | 0x7f800000u;
+    std::memcpy(&f, &inf, 4);
+    return f;
+  }
+  if (x < 0x38800000u) {                                // f16 subnormal range: quantum 2^-24
+    float a;
+    std::memcpy(&a, &x, 4);
+    const float q = std::nearbyintf(a * 16777216.0f) / 16777216.0f;
+    return sign ? -q : q;
+  }
+  x += 0xfffu + ((x >> 13) & 1u);
+  x &= ~0x1fffu;
+  x |= sign;
+  std::memcpy(&f, &x, 4);
+  return f;
 }
 
 std::vector<std::string> tilingFieldNames(const Program &p) {
@@ -453,11 +543,58 @@ std::string resolve(const Program &p, const std::vector<int64_t> &dims, Resolved
     s.outOffsetElems = off0 * outRowElems;
     s.outElems = s.size[0] * outRowElems;
 
+    bool inTail = false;
+    struct TailEntry { bool sum; float value; };
+    std::vector<TailEntry> tailStack;
     for (const Op &o : g.ops) {
       ResolvedOp ro;
       ro.code = o.code;
-      ro.constant = o.constant;
+      ro.constant = o.extent ? roundThroughType((float)value(o.constRef), o.constType) : o.constant;
       ro.depth = o.depth;
+      if (inTail && o.code != OpCode::Store) {
+        // symbolic evaluation: entries are the running sum or float32 constants
+        auto fold = [](OpCode c, float a, float b) {
+          switch (c) {
+            case OpCode::Add: return a + b;
+            case OpCode::Sub: return a - b;
+            case OpCode::Mul: return a * b;
+            case OpCode::Div: return a / b;
+            case OpCode::Max: return (a != a || b != b) ? a + b : (a == b ? (std::signbit(a) ? b : a) : (a > b ? a : b));
+            default: return (a != a || b != b) ? a + b : (a == b ? (std::signbit(a) ? a : b) : (a < b ? a : b));
+          }
+        };
+        switch (o.code) {
+          case OpCode::Const: tailStack.push_back({false, ro.constant}); break;
+          case OpCode::Dup: tailStack.push_back(tailStack[tailStack.size() - 1 - o.depth]); break;
+          case OpCode::Relu: case OpCode::Leaky: case OpCode::Neg: {
+            TailEntry &e = tailStack.back();
+            if (e.sum) {
+              s.tail.push_back({o.code, o.constant, false});
+            } else {
+              const float v = e.value;
+              e.value = o.code == OpCode::Neg ? -v : fold(OpCode::Max, v, o.code == OpCode::Relu ? 0.f : v * o.constant);
+            }
+            break;
+          }
+          default: {   // binary
+            const TailEntry b = tailStack.back();
+            tailStack.pop_back();
+            TailEntry &a = tailStack.back();
+            if (!a.sum && !b.sum) a.value = fold(o.code, a.value, b.value);
+            else if (a.sum) s.tail.push_back({o.code, b.value, false});
+            else {   // constant op sum
+              s.tail.push_back({o.code, a.value, o.code == OpCode::Sub || o.code == OpCode::Div});
+              a.sum = true;
+            }
+            break;
+          }
+        }
+        continue;
+      }
+      if (o.code == OpCode::ReduceSum) {
+        inTail = true;
+        tailStack.assign(1, TailEntry{true, 0.f});
+      }
       if (o.code == OpCode::Matmul) {
         const std::vector<int64_t> &sa = r.shapes[o.arg], &sb = r.shapes[o.arg2];
         if (sa[0] != s.size[0] || sb[1] != s.size[1] || sa[1] != sb[0])

@@ -39,10 +39,16 @@
 //     matmul argA argB          push sum_k A[d0,k] * B[k,d1] (float32 accumulation);
 //                               only as the first operation of a rank-2 segment
 //     const <float>             push a constant
+//     const <ref> [<type>]      push an extent as a number (mean = sum / N): the value of
+//                               argA.D converted to float, rounded to f16 | bf16 when a
+//                               type is given (arith.sitofp of a tensor.dim to that type)
 //     add | sub | mul | div | max | min      pop b, pop a, push a op b
 //     relu | leaky <alpha> | neg             on the top of the stack
 //     dup <n>                   push a copy of the n-th entry from the top
 //     reduce sum                sum the value over the last iteration dim
+//     ...                       after 'reduce sum': operations on the row's sum with constants
+//                               and extents only (const, the binary and unary operations,
+//                               dup; no push), e.g. 'const arg1.1 f16' 'div' for a mean
 //     store                     round to the output type and write
 //   end
 #pragma once
@@ -97,6 +103,9 @@ struct Op {
   std::vector<MapResult> map;       // Push: one per dim of the input
   std::vector<Ref> slice;           // Push: start offset per dim (empty = none)
   float constant = 0.f;             // Const, Leaky
+  bool extent = false;              // Const: the value is an extent (constRef), not `constant`
+  Ref constRef;                     // Const with extent set
+  ElemType constType = ElemType::F32;  // ... rounded through this float type
   int depth = 0;                    // Dup
 };
 
@@ -159,8 +168,22 @@ struct ResolvedSegment {
   int64_t outElems = 0;         // elements this segment writes
   ElemType outType = ElemType::F32;
   std::vector<ResolvedInput> inputs;
-  std::vector<ResolvedOp> ops;
+  std::vector<ResolvedOp> ops;    // up to and including 'reduce sum' (all of them without one), and 'store'
+  // What follows 'reduce sum', as a chain on the row's sum s (operations among constants are
+  // folded, in float32): s = s op c, or c op s when reversed (sub, div), or a unary operation.
+  struct TailStep {
+    OpCode code = OpCode::Add;
+    float constant = 0.f;   // the other operand; alpha of Leaky
+    bool reversed = false;
+  };
+  std::vector<TailStep> tail;
 };
+
+constexpr int kMaxTailOps = 8;    // operations on the sum between 'reduce sum' and 'store'
+constexpr int kMaxTailExtents = 4;   // of which extent constants
+
+// float -> f16 / bf16 -> float, round to nearest even (f32: the value itself).
+float roundThroughType(float f, ElemType t);
 
 struct Resolved {
   std::vector<std::vector<int64_t>> shapes;  // per argument

@@ -20,6 +20,13 @@ What a program means follows the reference's lowering of fused regions
                  (lib/Conversion/MarkStructuredOps/MarkStructuredOpsPass.cpp:54-147)
   concat         segments writing disjoint row ranges of the output
                  (examples/add-broadcast-concat/step0_input.mlir)
+  mean           sum, then operations on the row's sum with constants and extents
+                 (examples/broadcast-add-reduce/step0_input_mean.mlir:56-84: sum / N with N
+                 an arith.sitofp of the extent); float32 arithmetic on the float32 sum, one
+                 rounding to the output type -- the reference holds no golden for this
+                 graph (its gen_data.py writes the sum only), so where the intermediate f16
+                 tensor of the reference's IR would round the sum first, the two differ by at
+                 most one unit in the last place of the output: PARITY UNPINNED to that extent
   goldens        "compute in f32, cast to the storage type"
                  (examples/*/gen_data.py, gen_inputs.py)
 
@@ -105,6 +112,10 @@ def parse(text: str) -> dict:
             seg["ops"].append(("push", arg, m, sl))
         elif k == "matmul":
             seg["ops"].append(("matmul", int(tok[1][3:]), int(tok[2][3:])))
+        elif k == "const" and tok[1].startswith("arg"):
+            # an extent as a number, rounded through the named float type (f32 when none):
+            # arith.sitofp of a cast tensor.dim, examples/broadcast-add-reduce/step0_input_mean.mlir:73-74
+            seg["ops"].append(("constref", _ref(tok[1]), tok[2] if len(tok) > 2 else "f32"))
         elif k in ("const", "leaky"):
             seg["ops"].append((k, np.float32(float(tok[1]))))
         elif k == "dup":
@@ -254,7 +265,15 @@ def evaluate(text: str, inputs, out_shape=None):
                 b = _widen(inputs[op[2]], args[op[2]][1])
                 stack.append((a @ b).astype(np.float32))
             elif k == "const":
-                stack.append(np.full(size, op[1], dtype=np.float32))
+                stack.append(np.full(size[:-1] if reduced else size, op[1], dtype=np.float32))
+            elif k == "constref":
+                v = np.float32(val(op[1]))
+                if op[2] == "f16":
+                    with np.errstate(over="ignore"):
+                        v = np.float32(np.float16(v))
+                elif op[2] == "bf16":
+                    v = O.bf16_bits_to_f32(O.f32_to_bf16_bits(np.array([v], np.float32)))[0]
+                stack.append(np.full(size[:-1] if reduced else size, v, dtype=np.float32))
             elif k == "dup":
                 stack.append(stack[-1 - op[1]])
             elif k in ("add", "sub", "mul", "div", "max", "min"):

@@ -40,6 +40,21 @@ module {
 }
 """
 
+# the same graph followed by a division by N: the reference's mean example
+# (examples/broadcast-add-reduce/step0_input_mean.mlir:56-84), N as arith.sitofp of the extent
+ROW_BIAS_MEAN = ROW_BIAS_REDUCE.replace("@rowbias_reduce", "@rowbias_mean").replace(
+    "    return %red : tensor<?xf16>\n", """    %ni = arith.index_cast %n : index to i32
+    %nf = arith.sitofp %ni : i32 to f16
+    %e3 = tensor.empty(%m) : tensor<?xf16>
+    %mean = linalg.generic {indexing_maps = [#row1, #row1], iterator_types = ["parallel"]}
+        ins(%red : tensor<?xf16>) outs(%e3 : tensor<?xf16>) {
+      ^bb0(%x: f16, %o: f16):
+        %q = arith.divf %x, %nf : f16
+        linalg.yield %q : f16
+    } -> tensor<?xf16>
+    return %mean : tensor<?xf16>
+""").replace("#all = affine_map", "#row1 = affine_map<(d0) -> (d0)>\n#all = affine_map")
+
 RELU_COLUMN_ADD = """
 // out[n, m] = relu(col[m, 0]) + d[n, m]
 func.func @relu_column_add(%col: tensor<?x1xf16>, %d: tensor<?x?xf16>) -> tensor<?x?xf16> {

@@ -29,6 +29,12 @@ segment 2
 end
 """
 
+# c[m] = f16(sum_n (a[m] + b[m,n]) / N)    examples/broadcast-add-reduce/step0_input_mean.mlir
+MEAN_ROWBIAS = REDUCE_ROWBIAS.replace("  reduce sum\n", "  reduce sum\n  const arg1.1 f16\n  div\n")
+# the sum put through a longer chain: relu(4 - s * 0.5) * (N / 2), extents and constants mixed
+REDUCE_TAIL_CHAIN = REDUCE_ROWBIAS.replace(
+    "  reduce sum\n", "  reduce sum\n  const 0.5\n  mul\n  neg\n  const 4\n  add\n  relu\n  const arg1.1\n  const 0.5\n  mul\n  mul\n")
+
 # out[n,m] = f16(relu(data0[m,0]) + data1[n,m])   examples/relu-broadcast-transpose
 RELU_COL_ADD = HEADER + """
 arg in f16 2
@@ -233,6 +239,28 @@ def case_reduce_rowbias(m=640, n=512, seed=42):
     return REDUCE_ROWBIAS, [a, b], O.reduce_rowbias_f16(a, b)
 
 
+def mean_rowbias_f16(a, b):
+    """The mean graph's golden: the float32 row sum divided by N in float32, one rounding to
+    f16 (N goes through f16 like the IR's sitofp; exact up to 2048)."""
+    n = np.float32(np.float16(b.shape[1]))
+    s = (a.astype(np.float32)[:, None] + b.astype(np.float32)).sum(axis=1, dtype=np.float32)
+    return (s / n).astype(np.float16)
+
+
+def case_mean_rowbias(m=640, n=512, seed=42):
+    rng = np.random.default_rng(seed)
+    a, b = _u(rng, (m,)), _u(rng, (m, n))
+    return MEAN_ROWBIAS, [a, b], mean_rowbias_f16(a, b)
+
+
+def case_reduce_tail_chain(m=77, n=300, seed=9):
+    rng = np.random.default_rng(seed)
+    a, b = _u(rng, (m,)), _u(rng, (m, n), -0.1, 0.1)
+    s = (a.astype(np.float32)[:, None] + b.astype(np.float32)).sum(axis=1, dtype=np.float32)
+    t = np.maximum(np.float32(4) + -(s * np.float32(0.5)), np.float32(0))
+    return REDUCE_TAIL_CHAIN, [a, b], (t * (np.float32(n) * np.float32(0.5))).astype(np.float16)
+
+
 def case_relu_col_add(m=640, n=500, seed=42):
     rng = np.random.default_rng(seed)
     d0, d1 = _u(rng, (m, 1)), _u(rng, (n, m))
@@ -299,7 +327,8 @@ EXACT_CASES = {
     "split_relu_brc_add_mul": case_split_relu_brc_add_mul,
     "c1": case_c1, "c3": case_c3, "c4": case_c4, "add_mul_3": case_add_mul_3,
 }
-REDUCE_CASES = {"reduce_rowbias": case_reduce_rowbias, "c2": case_c2}
+REDUCE_CASES = {"reduce_rowbias": case_reduce_rowbias, "c2": case_c2, "mean_rowbias": case_mean_rowbias,
+                "reduce_tail_chain": case_reduce_tail_chain}
 
 
 # Hand-written static kernels of the reference's multi-kernel examples

@@ -118,6 +118,44 @@ def test_row_sums_of_workgroup_sized_rows(H, ty, n, rows):
     assert np.all(np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-6 * scale + ulp * np.abs(want))
 
 
+@pytest.mark.parametrize("rows,n", [(640, 512), (40, 75), (7, 40), (33, 8192), (5, 65536), (16, 1 << 20), (1000, 16)])
+def test_mean_is_the_row_sum_divided_by_the_extent_on_every_reduce_kernel(H, rows, n):
+    """reduce sum followed by a division by the extent (the reference's mean example), at shapes
+    that take each of the row-sum kernels: lanes sharing short rows, a wavefront per row, a
+    workgroup per row, a workgroup walking a long row, split and join.  On small integers the
+    sum is exact whatever the order, so the result must equal the oracle's bit for bit; on
+    uniform values it is held to one unit in the last place of the f16 result.  (The reference's
+    graph converts N to f16, which holds it exactly up to 2048 and overflows to infinity from
+    65520 on; the longer rows take N as a float32 extent.)"""
+    text = RC.MEAN_ROWBIAS if n <= 2048 else RC.MEAN_ROWBIAS.replace("const arg1.1 f16", "const arg1.1")
+    rng = np.random.default_rng(rows + n)
+    a = rng.integers(-4, 5, (rows,)).astype(np.float16)
+    b = rng.integers(-4, 5, (rows, n)).astype(np.float16)
+    want = RO.evaluate(text, [a, b])
+    got = run(H, text, [a, b], (rows,))
+    assert got.tobytes() == want.tobytes()
+    a = rng.uniform(-1, 1, (rows,)).astype(np.float16)
+    b = rng.uniform(-1, 1, (rows, n)).astype(np.float16)
+    want = RO.evaluate(text, [a, b])
+    got = run(H, text, [a, b], (rows,))
+    exact = (a.astype(np.float64)[:, None] + b.astype(np.float64)).mean(axis=1)
+    ulp = np.maximum(np.abs(exact), 2.0 ** -14) * 2.0 ** -10
+    assert np.all(np.abs(got.astype(np.float64) - exact) <= ulp + 1e-5 * np.abs(b.astype(np.float64)).mean(axis=1))
+    assert np.all(np.abs(got.astype(np.float64) - want.astype(np.float64)) <= 2 * ulp)
+
+
+def test_mean_graph_from_mlir_runs_on_every_route(H):
+    """MLIR text -> program (extent through index_cast + sitofp) -> kernels."""
+    import os
+    import subprocess
+    from tests import mlir_cases as MC
+    tr = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "ascend-mlir_amd", "bin", "afir-translate")
+    text = subprocess.run([tr, "-mlir-to-hip", "-"], input=MC.ROW_BIAS_MEAN, capture_output=True, text=True, check=True).stdout
+    _, inputs, want = RC.case_mean_rowbias(96, 2048)
+    got = run(H, text, inputs, want.shape)
+    assert np.abs(got.view(np.int16).astype(int) - want.view(np.int16).astype(int)).max() <= 1
+
+
 @pytest.mark.parametrize("n", [1, 3, 8, 16, 40, 64, 100, 256, 520])
 def test_row_sums_of_short_rows(H, n):
     """Rows shorter than a pass of the wavefront: 1, 2, 4 ... 32 lanes share a row and a

@@ -241,3 +241,15 @@ def test_emit_options_change_the_tile_and_the_unroll(tmp_path):
     q = subprocess.run([RS, "--kernel", str(src), "--output", str(tmp_path / "b"), "--name", "k",
                         "--emit-options", "tile_p=48"], capture_output=True, text=True)
     assert q.returncode == 4 and "tile_p must be a multiple of 32" in q.stderr
+
+
+def test_operations_after_reduce_sum_are_applied_to_the_row_sum_where_it_is_stored():
+    src = _emit(RC.MEAN_ROWBIAS).stdout
+    assert "float tail_const[4];" in src
+    assert src.count("(s / R.tail_const[0])") >= 4          # every kernel that stores a row sum
+    assert "v0[u][e] / " not in src                          # not per element
+    chain = _emit(RC.REDUCE_TAIL_CHAIN).stdout
+    half, four = "as_f32(0x3f000000u) /* 0.5 */", "as_f32(0x40800000u) /* 4 */"
+    assert f"(fmax_ieee(((-(s * {half})) + {four}), 0.f) * (R.tail_const[0] * {half}))" in chain
+    plain = _emit(RC.REDUCE_ROWBIAS).stdout
+    assert "R.tail_const" not in plain.split("struct SpecArgs", 1)[1].split("};", 1)[1]

@@ -180,3 +180,39 @@ def test_library_resolves_shapes_and_rejects_inconsistent_ones(H):
 def test_library_rejects_malformed_programs(H, bad, why):
     with pytest.raises(H.AfirHipError, match=why):
         H.Region(bad)
+
+
+def test_mean_tail_is_pinned_by_exact_cases():
+    """What follows 'reduce sum' works on the float32 sum.  Small integers make the sum exact
+    and a power-of-two N makes the division exact, so the mean is fixed by the mathematics:
+    it must equal the float64 mean rounded once to f16."""
+    rng = np.random.default_rng(3)
+    for m, n in ((5, 512), (64, 1024), (3, 8)):
+        a = rng.integers(-8, 9, (m,)).astype(np.float16)
+        b = rng.integers(-8, 9, (m, n)).astype(np.float16)
+        got = RO.evaluate(RC.MEAN_ROWBIAS, [a, b])
+        want = ((a.astype(np.float64)[:, None] + b.astype(np.float64)).sum(axis=1) / n).astype(np.float16)
+        assert got.dtype == np.float16 and got.tobytes() == want.tobytes()
+    # N that f16 cannot hold exactly: the IR converts the extent to f16 first (sitofp ... to f16),
+    # 2049 becomes 2048
+    a = np.zeros((2,), np.float16)
+    b = np.ones((2, 2049), np.float16)
+    assert RO.evaluate(RC.MEAN_ROWBIAS, [a, b]).tolist() == [np.float16(2049 / 2048)] * 2
+    assert RO.evaluate(RC.MEAN_ROWBIAS.replace("const arg1.1 f16", "const arg1.1"), [a, b]).tolist() == [1.0, 1.0]
+
+
+def test_mean_against_the_reference_written_sum_vector():
+    """The reference's golden script writes the row SUMS of its example (as f16); the mean of
+    the same inputs can differ from that vector divided by N only by the second rounding."""
+    from tests import golden_cases as GC
+    z = GC.load()
+    a, b, sums = (np.ascontiguousarray(z["broadcast-add-reduce/" + k]) for k in ("input_a", "input_b", "output_c"))
+    got = RO.evaluate(RC.MEAN_ROWBIAS, [a, b])
+    assert got.tobytes() == RC.mean_rowbias_f16(a, b).tobytes()
+    twice = (sums.astype(np.float32) / np.float32(b.shape[1])).astype(np.float16)
+    assert np.abs(got.view(np.int16).astype(int) - twice.view(np.int16).astype(int)).max() <= 1
+
+
+def test_reduce_tail_chain_matches_its_closed_form():
+    text, inputs, want = RC.case_reduce_tail_chain()
+    assert RO.evaluate(text, inputs).tobytes() == want.tobytes()

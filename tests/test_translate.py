@@ -183,6 +183,36 @@ def test_reference_example_inputs_translate_and_evaluate(example, case):
     assert RO.evaluate(p.stdout, inputs).tobytes() == want.tobytes()
 
 
+def test_mean_is_a_sum_with_a_tail_on_the_row_sums():
+    """Reduce followed by an elementwise generic on the sums (mean = sum / N): the extent
+    reaches the body through arith.index_cast + arith.sitofp, outside any generic."""
+    out = program_of(MC.ROW_BIAS_MEAN)
+    body = [l.strip() for l in out.splitlines() if l.strip() and not l.startswith("#")]
+    assert body[body.index("outoff 0") + 1:] == [
+        "push arg0 d0", "push arg1 d0 d1", "add", "reduce sum", "const arg1.1 f16", "div", "store", "end"]
+    _, inputs, want = RC.case_mean_rowbias(33, 96)
+    assert RO.evaluate(out, inputs).tobytes() == want.tobytes()
+    # c - sum, sum * c, max(sum, c): the sum as either operand where the operation allows it
+    for expr, tail in (("arith.subf %nf, %x", ["neg", "const arg1.1 f16", "add"]),
+                       ("arith.mulf %nf, %x", ["const arg1.1 f16", "mul"]),
+                       ("arith.maximumf %x, %nf", ["const arg1.1 f16", "max"])):
+        out = program_of(MC.ROW_BIAS_MEAN.replace("arith.divf %x, %nf", expr))
+        body = [l.strip() for l in out.splitlines() if l.strip() and not l.startswith("#")]
+        assert body[body.index("reduce sum") + 1:-2] == tail, expr
+    bad = subprocess.run([TR, "-mlir-to-hip", "-"], input=MC.ROW_BIAS_MEAN.replace("arith.divf %x, %nf", "arith.divf %nf, %x"),
+                         capture_output=True, text=True)
+    assert bad.returncode != 0 and "divided by a reduced value" in bad.stderr
+
+
+@pytest.mark.skipif(not os.path.isdir(REF_EXAMPLES), reason="reference tree not present")
+def test_reference_mean_example_translates_unchanged():
+    p = subprocess.run([TR, "-mlir-to-hip", os.path.join(REF_EXAMPLES, "broadcast-add-reduce", "step0_input_mean.mlir")],
+                       capture_output=True, text=True)
+    assert p.returncode == 0, p.stderr
+    _, inputs, want = RC.case_mean_rowbias()
+    assert RO.evaluate(p.stdout, inputs).tobytes() == want.tobytes()
+
+
 def test_asc_graph_form_with_load_store_and_attribute_dictionaries():
     out = program_of(MC.ASC_GRAPH_FORM)
     body = [l.strip() for l in out.splitlines() if l.strip() and not l.startswith("#")]
