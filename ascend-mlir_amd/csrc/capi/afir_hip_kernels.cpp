@@ -10,6 +10,7 @@
 #include <cstring>
 #include <string>
 
+#include <atomic>
 #include <map>
 #include <memory>
 #include <mutex>
@@ -82,6 +83,9 @@ enum class FastPath { None, AddMul, BcastAddRowsum, ReluBcastTranspose, GatherSc
 
 // A code object compiled for one program (afir_target::emitHipSource), loaded
 // on first launch.
+// Set when the process runs its static destructors: the HIP runtime may be gone by then.
+bool g_process_exiting = false;
+
 struct CompiledRegion {
   std::vector<char> image;
   std::mutex mutex;
@@ -89,9 +93,19 @@ struct CompiledRegion {
   afir_target::EmitOptions options;   // read from the loaded module
   hipModule_t module = nullptr;
   std::map<std::string, hipFunction_t> functions;
+  // The split / join row sum keeps its partial sums in one array of the code object.  Launches
+  // of that form are chained through this event, so that one on another stream waits for the
+  // join of the one before it instead of overwriting its partial sums.
+  std::mutex split_mutex;
+  hipEvent_t split_done = nullptr;
+  hipStream_t split_stream = nullptr;
+  bool split_recorded = false;
   ~CompiledRegion() {
-    if (!loaded) return;
+    // at process exit the module and the event are left to the operating system: unloading
+    // from a static destructor can run after the HIP runtime has shut down
+    if (!loaded || g_process_exiting) return;
     (void)hipDeviceSynchronize();   // no launch of this module may still be running
+    if (split_done) (void)hipEventDestroy(split_done);
     (void)hipModuleUnload(module);
   }
 };
@@ -342,6 +356,10 @@ bool fast_path_fits(const RegisteredRegion &r, const afir_region::Resolved &res)
 std::mutex g_region_mutex;
 std::map<uint64_t, std::shared_ptr<RegisteredRegion>> g_regions;
 uint64_t g_next_region = 1;
+// constructed after g_regions, so destroyed before it
+struct ExitMarker {
+  ~ExitMarker() { g_process_exiting = true; }
+} g_exit_marker;
 
 std::shared_ptr<RegisteredRegion> find_region(uint64_t handle) {
   std::lock_guard<std::mutex> lock(g_region_mutex);
@@ -563,7 +581,7 @@ struct FamilyRegion {
   const char *program;
   std::once_flag once;
   uint64_t handle = 0;
-  bool usable = false;
+  std::atomic<bool> usable{false};
 };
 FamilyRegion g_families[] = {
     {"broadcast_add_reducesum", afir_family::kBroadcastAddReducesum},
@@ -936,7 +954,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
           int64_t tiles = tq * tp;
           for (int k = 0; k < last; ++k)
             if (k != tile.dim) tiles *= ra.size[k];
-          int64_t blocks = tiles < (int64_t)afir::kNumCU * 256 ? tiles : (int64_t)afir::kNumCU * 256;
+          int64_t blocks = tiles < (int64_t)afir::device_cus() * 256 ? tiles : (int64_t)afir::device_cus() * 256;
           if (block_dim) blocks = block_dim;
           sa.grid = (int)blocks;
           sa.column_blocks = 1;
@@ -956,7 +974,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
               for (int k = 0; k < last; ++k) nrows *= ra.size[k];
               const int64_t rows_per_block = (int64_t)4 * (64 >> ll);
               int64_t blocks = (nrows + rows_per_block - 1) / rows_per_block;
-              if (blocks > (int64_t)afir::kNumCU * 16) blocks = (int64_t)afir::kNumCU * 16;
+              if (blocks > (int64_t)afir::device_cus() * 16) blocks = (int64_t)afir::device_cus() * 16;
               sa.grid = (int)blocks;
             }
           }
@@ -970,12 +988,12 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
           int64_t nrows_all = 1;
           for (int k = 0; k < last; ++k) nrows_all *= ra.size[k];
           if (!slim && seg.reduce && groups >= (int64_t)512 * U && groups % ((int64_t)256 * U) == 0 &&
-              nrows_all < (int64_t)afir::kNumCU * 16)
+              nrows_all < (int64_t)afir::device_cus() * 16)
             row_groups = 2;
           // a handful of rows: the passes of a row are dealt out to about eight workgroups per CU in all
           const int64_t passes = groups / ((int64_t)256 * U);
           if (row_groups == 2 && nrows_all <= 64 && passes >= 8 && !block_dim) {
-            int64_t per_row = (int64_t)afir::kNumCU * 8 / nrows_all;
+            int64_t per_row = (int64_t)afir::device_cus() * 8 / nrows_all;
             if (per_row > passes / 2) per_row = passes / 2;
             if (per_row >= 2 && per_row * nrows_all <= afir_target::kSpecPartials) {
               row_groups = 3;
@@ -1023,7 +1041,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
           // up to 16 workgroups per CU walk the rows (4 to 16 measured within 1 %, 2 slower)
           int64_t nrows = 1;
           for (int k = 0; k < last; ++k) nrows *= ra.size[k];
-          int64_t blocks = nrows < (int64_t)afir::kNumCU * 16 ? nrows : (int64_t)afir::kNumCU * 16;
+          int64_t blocks = nrows < (int64_t)afir::device_cus() * 16 ? nrows : (int64_t)afir::device_cus() * 16;
           if (block_dim) blocks = block_dim;
           sa.grid = (int)blocks;
           sa.column_blocks = 1;
@@ -1088,7 +1106,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
           if (d.gstride == 1 && d.vec && bytes > 0 && bytes % 16 == 0 && bytes * 4 <= afir_target::kSpecStageBytes / 2 &&
               n_out * 2 >= wave_pass && n_out <= 8 * wave_pass && seg.size[0] >= 1024) {
             int64_t blocks = (seg.size[0] + 3) / 4;
-            if (blocks > (int64_t)afir::kNumCU * 16) blocks = (int64_t)afir::kNumCU * 16;
+            if (blocks > (int64_t)afir::device_cus() * 16) blocks = (int64_t)afir::device_cus() * 16;
             if (block_dim) blocks = block_dim;
             made.args.grid = (int)blocks;
             made.args.column_blocks = 1;
@@ -1099,7 +1117,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
           } else
           if (d.gstride == 1 && d.vec && bytes > 0 && bytes % 16 == 0 && bytes <= afir_target::kSpecStageBytes &&
               seg.size[seg.rank - 1] >= (int64_t)128 * shape.unroll * wideW) {   // at least half a pass of the workgroup
-            int64_t blocks = seg.size[0] < (int64_t)afir::kNumCU * 16 ? seg.size[0] : (int64_t)afir::kNumCU * 16;
+            int64_t blocks = seg.size[0] < (int64_t)afir::device_cus() * 16 ? seg.size[0] : (int64_t)afir::device_cus() * 16;
             if (block_dim) blocks = block_dim;
             made.args.grid = (int)blocks;
             made.args.column_blocks = 1;
@@ -1157,6 +1175,19 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
     } else {
       for (PendingSegment &p : pending) {
         if (p.rows == 3) {
+          // split and join share the code object's partial sums with every other launch of this
+          // form: order them (a launch on another stream waits for the previous join)
+          CompiledRegion *c = compiled.get();
+          std::lock_guard<std::mutex> chain(c->split_mutex);
+          hipStream_t st = static_cast<hipStream_t>(stream);
+          if (!c->split_done && hipEventCreateWithFlags(&c->split_done, hipEventDisableTiming) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(AFIR_HIP_E_LAUNCH, "compiled region kernel: cannot create the event that orders split row sums");
+          }
+          if (c->split_recorded && c->split_stream != st && hipStreamWaitEvent(st, c->split_done, 0) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(AFIR_HIP_E_LAUNCH, "compiled region kernel: cannot order split row sums across streams");
+          }
           uint32_t rc = launch(afir_target::specSplitRowsKernelName(p.segment, p.idx32, false), &p.args, sizeof p.args,
                                (unsigned)p.args.grid);
           if (rc != AFIR_HIP_OK) return rc;
@@ -1164,6 +1195,12 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
           rc = launch(afir_target::specSplitRowsKernelName(p.segment, p.idx32, true), &p.args, sizeof p.args,
                       (unsigned)((nrows + 3) / 4));
           if (rc != AFIR_HIP_OK) return rc;
+          if (hipEventRecord(c->split_done, st) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(AFIR_HIP_E_LAUNCH, "compiled region kernel: cannot record the event that orders split row sums");
+          }
+          c->split_recorded = true;
+          c->split_stream = st;
           continue;
         }
         if (p.lds) {

@@ -9,8 +9,24 @@
 namespace afir {
 
 constexpr int kWave = 64;        // CDNA wavefront width
-constexpr int kNumCU = 256;      // MI355X compute units (8 XCDs x 32)
-constexpr int kNumXCD = 8;
+constexpr int kNumCU = 256;      // MI355X compute units (8 XCDs x 32): what the tile shapes were tuned on
+constexpr int kNumXCD = 8;       // workgroup i runs on XCD i % 8; the matmul's tile order relies on it for
+                                 // cache locality only (it is a permutation of the tiles whatever the part)
+
+// Compute units of the device the process works on, asked once.  Grid sizes follow it, so a
+// part with another CU count (a partitioned MI355X, say) gets grids of its own size; every
+// kernel is grid-strided, so any value is correct.  kNumCU if the device cannot be asked.
+inline int device_cus() {
+  static const int count = [] {
+    int device = 0, value = 0;
+    if (hipGetDevice(&device) == hipSuccess &&
+        hipDeviceGetAttribute(&value, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && value > 0)
+      return value;
+    (void)hipGetLastError();
+    return kNumCU;
+  }();
+  return count;
+}
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));

@@ -84,7 +84,7 @@ LaunchStatus launch_fused_add_mul(const float *a, const float *b, float *out, in
   if (n4 * 4 < n) {
     size_t rest = n - n4 * 4;
     size_t blocks = (rest + kThreads - 1) / kThreads;
-    if (blocks > (size_t)kNumCU * 16) blocks = (size_t)kNumCU * 16;
+    if (blocks > (size_t)device_cus() * 16) blocks = (size_t)device_cus() * 16;
     if (block_dim && blocks > block_dim) blocks = block_dim;
     hipLaunchKernelGGL(add_mul_f32_scalar, dim3((unsigned)blocks), dim3(kThreads), 0, stream,
                        a, b, out, n4 * 4, n);

@@ -200,7 +200,7 @@ LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx
   if (vec && ((int64_t)kGroups << lanes_log2) == chunks64) {
     const int rows_per_pass = kThreads >> lanes_log2;
     int64_t blocks = (nidx + rows_per_pass - 1) / rows_per_pass;
-    if (blocks > (int64_t)kNumCU * 64) blocks = (int64_t)kNumCU * 64;
+    if (blocks > (int64_t)device_cus() * 64) blocks = (int64_t)device_cus() * 64;
     if (block_dim) blocks = block_dim;
     hipLaunchKernelGGL(gather_scale_shift_f16_grouped, dim3((unsigned)blocks), dim3(kThreads), 0,
                        stream, table, idx, scale, shift, out, error_flag, (uint32_t)rows, lanes_log2,

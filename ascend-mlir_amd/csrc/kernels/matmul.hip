@@ -348,7 +348,7 @@ LaunchStatus launch_matmul_any_io(const uint16_t *a, const uint16_t *b, const vo
                   ((reinterpret_cast<uintptr_t>(bias) & (F16IO ? 15u : 7u)) == 0);
   // 256 x 256 tiles for fewer than half of the CUs: 128 x 128 tiles keep four times as many busy
   // (2048^3: 240 -> 390 TFLOP/s; at 3072^3, 144 tiles, the large ones are still faster)
-  const bool few_big_tiles = (m / 256) * (n / 256) < (int64_t)kNumCU / 2 && m % 128 == 0 && n % 128 == 0;
+  const bool few_big_tiles = (m / 256) * (n / 256) < (int64_t)device_cus() / 2 && m % 128 == 0 && n % 128 == 0;
   if (al && !few_big_tiles && matmul_dma_supported(m, k, n)) {
     if constexpr (F16IO)
       return launch_matmul_dma_f16(a, b, static_cast<const float *>(bias), static_cast<float *>(out),

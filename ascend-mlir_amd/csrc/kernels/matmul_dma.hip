@@ -565,7 +565,7 @@ bool matmul_dma_supported(int64_t m, int64_t k, int64_t n) {
 }
 
 #ifndef AFIR_MM_GRID
-#define AFIR_MM_GRID kNumCU
+#define AFIR_MM_GRID device_cus()
 #endif
 
 namespace {

@@ -616,7 +616,7 @@ LaunchStatus plan_fused_region(const RegionArgs &args, int vec, uint32_t block_d
     const int64_t rows_per_block = (int64_t)(kThreads / kWave) * (kWave >> ll);
     int64_t blocks = (rows + rows_per_block - 1) / rows_per_block;
     // up to 64 waves per CU at a time; 16 and more measured 3 % above 8 on 16384 rows of f16
-    if (blocks > (int64_t)kNumCU * 16) blocks = (int64_t)kNumCU * 16;
+    if (blocks > (int64_t)device_cus() * 16) blocks = (int64_t)device_cus() * 16;
     if (block_dim) blocks = block_dim;
     g->blocks = blocks;
     g->lanes_log2 = ll;
@@ -631,10 +631,10 @@ LaunchStatus plan_fused_region(const RegionArgs &args, int vec, uint32_t block_d
   while (lanes_log2 < 8 && ((int64_t)1 << lanes_log2) < chunks) ++lanes_log2;
   const int rows_per_pass = kThreads >> lanes_log2;
   int64_t blocks = (rows + rows_per_pass - 1) / rows_per_pass;
-  if (blocks > (int64_t)kNumCU * 16) blocks = (int64_t)kNumCU * 16;
+  if (blocks > (int64_t)device_cus() * 16) blocks = (int64_t)device_cus() * 16;
   // few rows that are longer than one pass of the workgroup: more workgroups along the row
   const int64_t passes = (chunks + ((int64_t)1 << lanes_log2) - 1) >> lanes_log2;
-  int64_t column_blocks = (int64_t)kNumCU * 16 / blocks;
+  int64_t column_blocks = (int64_t)device_cus() * 16 / blocks;
   if (column_blocks > passes) column_blocks = passes;
   if (column_blocks > 65535) column_blocks = 65535;
   if (column_blocks < 1) column_blocks = 1;

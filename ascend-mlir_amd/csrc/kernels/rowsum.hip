@@ -188,7 +188,7 @@ LaunchStatus launch_broadcast_add_reducesum(const float *x, const float *bias, f
   if (vec && (n / 4) % kRowThreads == 0 && n / 4 <= 8 * kRowThreads && aligned16(x) &&
       ((n / 4 / kRowThreads) & (n / 4 / kRowThreads - 1)) == 0) {
     // a workgroup per row
-    int64_t wblocks = (int64_t)kNumCU * AFIR_ROWSUM_WG_PER_CU;
+    int64_t wblocks = (int64_t)device_cus() * AFIR_ROWSUM_WG_PER_CU;
     if (wblocks > m) wblocks = m;
     if (block_dim) wblocks = block_dim;
     const dim3 grid((unsigned)wblocks), block(kRowThreads);
@@ -201,7 +201,7 @@ LaunchStatus launch_broadcast_add_reducesum(const float *x, const float *bias, f
   } else if (vec && n / 4 <= 16 * kWave) {
     // persistent waves: each keeps its bias chunks resident and walks several rows
     const int64_t n4 = n / 4;
-    int64_t pblocks = (int64_t)kNumCU * kWavesPerCU / kWavesPerBlock;
+    int64_t pblocks = (int64_t)device_cus() * kWavesPerCU / kWavesPerBlock;
     if (pblocks * kWavesPerBlock > m) pblocks = (m + kWavesPerBlock - 1) / kWavesPerBlock;
     if (block_dim) pblocks = block_dim;
     const dim3 grid((unsigned)pblocks), block(kThreads);

@@ -158,7 +158,7 @@ LaunchStatus launch_relu_broadcast_add_transpose(const uint16_t *x, const uint16
     // of four 21.4, 8192 of one 20.7): the hardware deals workgroups out as slots free up, which
     // balances better than longer walks
     int64_t blocks = (nb * (m / kSmallTile) * (n / kSmallTile) + 1) / 2;
-    if (blocks > (int64_t)kNumCU * 256) blocks = (int64_t)kNumCU * 256;
+    if (blocks > (int64_t)device_cus() * 256) blocks = (int64_t)device_cus() * 256;
     if (block_dim) blocks = block_dim;
     hipLaunchKernelGGL(relu_bcast_add_transpose_f16_tile64, dim3((unsigned)blocks), dim3(kThreads), 0, stream,
                        x, c, out, (int)nb, (int)m, (int)n);

@@ -709,3 +709,34 @@ def test_preferred_code_object_outranks_a_hand_tuned_family(H, evaluator, monkey
     r.prefer_code_object(False)
     assert r.kernel == "relu_broadcast_add_transpose"
     r.close()
+
+
+def test_split_row_sums_launched_from_two_streams_do_not_mix_their_partial_sums(H, evaluator):
+    """A handful of very long rows is summed by a split kernel and a join kernel that share
+    the code object's partial sums.  Launches of that form from different streams are chained
+    by the library (the second waits for the first one's join): alternating two streams and
+    two inputs, every result must be its own input's."""
+    import torch
+    if evaluator != "compiled":
+        pytest.skip("the split / join form belongs to the compiled kernels")
+    text = RC.C2_BCAST_ADD_ROWSUM
+    rows, n = 16, 1 << 20
+    rng = np.random.default_rng(5)
+    xs = [torch.from_numpy(rng.integers(-4, 5, (rows, n)).astype(np.float32)).cuda() for _ in range(2)]
+    bias = torch.from_numpy(rng.integers(-4, 5, (n,)).astype(np.float32)).cuda()
+    want = [(x.double().sum(1) + bias.double().sum()).cpu().numpy().astype(np.float32) for x in xs]
+    r = region(H, text)
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    outs = [[torch.empty((rows,), dtype=torch.float32, device="cuda") for _ in range(6)] for _ in range(2)]
+    tiling = H.pack_tiling(rows, n, n, rows)
+    torch.cuda.synchronize()
+    for k in range(6):
+        for i in range(2):
+            rc = r.launch_raw([xs[i].data_ptr(), bias.data_ptr(), outs[i][k].data_ptr()], tiling,
+                              stream=streams[i].cuda_stream)
+            assert rc == 0
+    torch.cuda.synchronize()
+    for i in range(2):
+        for k in range(6):
+            assert np.array_equal(outs[i][k].cpu().numpy(), want[i]), (i, k)
+    r.close()
