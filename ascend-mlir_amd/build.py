@@ -1,6 +1,10 @@
 """Builds the gfx950 libraries in-tree with hipcc (cross-compiles without a GPU).
 
-    python ascend-mlir_amd/build.py [--force]
+    python ascend-mlir_amd/build.py
+    python ascend-mlir_amd/build.py --variant OUT.so -DAFIR_MM_KSTAGGER_M=1 [-D...]
+        a copy of the kernel library with compile-time choices of the hand-tuned kernels
+        changed (what a tile search times against the shipped choice; bin/autotuner calls
+        this for parameters named build_<MACRO>)
 
 Outputs (under ascend-mlir_amd/lib/):
     libafir_hip_kernels.so    fused kernels + launcher C ABI
@@ -176,11 +180,46 @@ def build_probes():
     return out
 
 
+def build_variant(out, defines):
+    """The kernel library with extra -D flags.  Sources that mention none of the macros keep
+    their ordinary objects (compiled here if the build directory does not hold them)."""
+    import re
+    names = [re.match(r"-D([A-Za-z_0-9]+)", d).group(1) for d in defines]
+    tag = "_".join(d[2:].replace("=", "-") for d in defines) or "base"
+    vdir = os.path.join(os.path.dirname(os.path.abspath(out)), "obj_" + tag)
+    os.makedirs(vdir, exist_ok=True)
+    os.makedirs(OBJ, exist_ok=True)
+
+    def one(item):
+        src, extra = item
+        text = open(os.path.join(CSRC, src)).read()
+        touched = any(n in text for n in names)
+        obj = os.path.join(vdir if touched else OBJ, src.replace("/", "_") + ".o")
+        if touched or not os.path.exists(obj):
+            _run([HIPCC, *COMMON, *extra, *(defines if touched else []), "-x", "hip", "-c",
+                  os.path.join(CSRC, src), "-o", obj])
+        return obj
+    with cf.ThreadPoolExecutor(max_workers=min(8, len(KERNEL_SOURCES))) as ex:
+        objs = list(ex.map(one, KERNEL_SOURCES))
+    _run([HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", out, *objs])
+    # the families' compiled form is looked up beside the library
+    fam = os.path.join(LIB, "families")
+    link = os.path.join(os.path.dirname(os.path.abspath(out)), "families")
+    if os.path.isdir(fam) and not os.path.exists(link):
+        os.symlink(fam, link)
+    return out
+
+
 def build_all():
     kernel_lib = build_kernels()
     return [kernel_lib, *build_runtime(), *build_families(kernel_lib), build_probes()]
 
 
 if __name__ == "__main__":
-    for path in build_all():
-        print("built", os.path.relpath(path, ROOT))
+    if len(sys.argv) > 1 and sys.argv[1] == "--variant":
+        if len(sys.argv) < 3 or any(not a.startswith("-D") for a in sys.argv[3:]):
+            raise SystemExit("usage: build.py --variant OUT.so [-DNAME=VALUE ...]")
+        print("built", build_variant(sys.argv[2], sys.argv[3:]))
+    else:
+        for path in build_all():
+            print("built", os.path.relpath(path, ROOT))

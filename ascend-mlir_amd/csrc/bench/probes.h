@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-/* Issues v_mfma_f32_32x32x16_bf16 from registers on every CU (8 waves per
+/* Issues v_mfma_f32_16x16x32_bf16 (the matmul kernel's instruction) from registers on every CU (8 waves per
  * workgroup, two workgroups per CU) and nothing else.  `operands` = 65536 bytes
  * of bf16 (the VALUES matter: the sustained clock under the board power limit
  * depends on how much the operands toggle), `sink` = 1 MiB that receives one

@@ -14,7 +14,13 @@ namespace afir {
 namespace {
 
 constexpr int kThreads = 256;
-constexpr int kUnroll = 4;
+#ifndef AFIR_ELTWISE_UNROLL
+#define AFIR_ELTWISE_UNROLL 2   // 128-bit loads per input in flight per lane (2, 4, 8 measured within 3 %)
+#endif
+#ifndef AFIR_ELTWISE_WG_PER_CU
+#define AFIR_ELTWISE_WG_PER_CU 16
+#endif
+constexpr int kUnroll = AFIR_ELTWISE_UNROLL;
 
 __global__ __launch_bounds__(kThreads) void add_mul_f32_vec(const f32x4 *__restrict__ a,
                                                             const f32x4 *__restrict__ b,
@@ -84,7 +90,7 @@ LaunchStatus launch_fused_add_mul(const float *a, const float *b, float *out, in
   if (n4 * 4 < n) {
     size_t rest = n - n4 * 4;
     size_t blocks = (rest + kThreads - 1) / kThreads;
-    if (blocks > (size_t)device_cus() * 16) blocks = (size_t)device_cus() * 16;
+    if (blocks > (size_t)device_cus() * AFIR_ELTWISE_WG_PER_CU) blocks = (size_t)device_cus() * AFIR_ELTWISE_WG_PER_CU;
     if (block_dim && blocks > block_dim) blocks = block_dim;
     hipLaunchKernelGGL(add_mul_f32_scalar, dim3((unsigned)blocks), dim3(kThreads), 0, stream,
                        a, b, out, n4 * 4, n);

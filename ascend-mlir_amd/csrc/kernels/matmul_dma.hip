@@ -73,11 +73,17 @@ namespace afir {
 
 namespace {
 
+// Compile-time choices a tile search can vary (bin/autotuner, parameters build_<MACRO>;
+// ascend-mlir_amd/examples/autotune-matmul): the K offsets tiles start from, and how many
+// tile rows an XCD's 32 workgroups cover at once (their patch is GROUP_M x 32 / GROUP_M tiles).
+#ifndef AFIR_MM_GROUP_M
+#define AFIR_MM_GROUP_M 4
+#endif
 #ifndef AFIR_MM_KSTAGGER_M
-#define AFIR_MM_KSTAGGER_M 2
+#define AFIR_MM_KSTAGGER_M 1
 #endif
 #ifndef AFIR_MM_KSTAGGER_N
-#define AFIR_MM_KSTAGGER_N 1
+#define AFIR_MM_KSTAGGER_N 0
 #endif
 // Measurement builds only (the benchmark's probe library compiles this file again with
 // -DAFIR_MM_ABLATE=1 or 2 under another namespace name): 1 leaves the global -> LDS feed
@@ -106,7 +112,7 @@ __device__ __forceinline__ void map_tile_dma(int p, int tiles_m, int tiles_n, in
   const int ntiles = tiles_m * tiles_n;
   int q = p;
   if ((ntiles % kNumXCD) == 0) q = (p % kNumXCD) * (ntiles / kNumXCD) + p / kNumXCD;
-  constexpr int kGroupM = 4;
+  constexpr int kGroupM = AFIR_MM_GROUP_M;
   const int per_group = kGroupM * tiles_n;
   const int group = q / per_group, within = q % per_group;
   const int first_m = group * kGroupM;

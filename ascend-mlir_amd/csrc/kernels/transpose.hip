@@ -18,7 +18,7 @@ constexpr int kThreads = 256;
 // max(v, +0) with IEEE-754 maximum semantics: NaN propagates, -0 gives +0.
 __device__ __forceinline__ float relu_keep_nan(float v) { return (v > 0.f) ? v : ((v != v) ? v : 0.f); }
 
-// 64x64 tiles through a float32 LDS tile, two tiles in flight per workgroup.
+// 64x64 tiles through a float32 LDS tile; a workgroup that walks several tiles has two in flight.
 // Phase 1: a lane loads two 16-byte chunks of x rows (a wave covers eight
 // 128-byte runs per load), applies relu and + c (its eight columns are fixed
 // within a tile, so c is read once per tile) and writes the float32 results to
@@ -37,6 +37,9 @@ __device__ __forceinline__ float relu_keep_nan(float v) { return (v > 0.f) ? v :
 // the hint on both sides and 6.7 with ordinary loads, this kernel 5.5 and 6.5
 // (kernels that read two or more bytes per byte written measured the other
 // way round and keep the hint on their loads).
+#ifndef AFIR_TRANSPOSE_TILES_PER_WG
+#define AFIR_TRANSPOSE_TILES_PER_WG 1
+#endif
 constexpr int kSmallTile = 64, kSmallPitch = kSmallTile + 1;
 __global__ __launch_bounds__(kThreads) void relu_bcast_add_transpose_f16_tile64(
     const uint16_t *__restrict__ x, const uint16_t *__restrict__ c, uint16_t *__restrict__ out,
@@ -154,10 +157,12 @@ LaunchStatus launch_relu_broadcast_add_transpose(const uint16_t *x, const uint16
 
   if ((m % kSmallTile == 0) && (n % kSmallTile == 0) && aligned16(x) && aligned16(c) && aligned16(out) &&
       nb * (m / kSmallTile) * (n / kSmallTile) < ((int64_t)1 << 31)) {
-    // two tiles per workgroup (4096 workgroups of two tiles measured 20.3 us on [64, 1024, 512], 2048
-    // of four 21.4, 8192 of one 20.7): the hardware deals workgroups out as slots free up, which
-    // balances better than longer walks
-    int64_t blocks = (nb * (m / kSmallTile) * (n / kSmallTile) + 1) / 2;
+    // one tile per workgroup: the hardware deals workgroups out as slots free up, which balances
+    // better than walks of several tiles (8192 workgroups of one tile 19.7 us on [64, 1024, 512],
+    // 4096 of two 20.4, 2731 of three 20.9; a grid given by the caller makes a workgroup walk,
+    // with the next tile's loads in flight).  The two LDS tiles then also hold a CU to four
+    // workgroups, which measured faster than the eight that one tile allows (20.7 us).
+    int64_t blocks = (nb * (m / kSmallTile) * (n / kSmallTile) + AFIR_TRANSPOSE_TILES_PER_WG - 1) / AFIR_TRANSPOSE_TILES_PER_WG;
     if (blocks > (int64_t)device_cus() * 256) blocks = (int64_t)device_cus() * 256;
     if (block_dim) blocks = block_dim;
     hipLaunchKernelGGL(relu_bcast_add_transpose_f16_tile64, dim3((unsigned)blocks), dim3(kThreads), 0, stream,

@@ -216,20 +216,36 @@ class HipExecutionRunner final : public ExecutionRunner {
     slots[idx++] = workspace;
     slots[idx++] = args.tiling.empty() ? nullptr : args.tiling.data();
 
+    // further copies of the tensors for timed launches to rotate over
+    const int nsets = args.buffer_sets > 1 && args.timing_repeats > 0 ? args.buffer_sets : 1;
+    const size_t ntensors = args.inputs.size() + args.outputs.size();
+    std::vector<std::vector<void *>> sets(nsets, std::vector<void *>(slots, slots + 16));
+    for (int k = 1; k < nsets; ++k)
+      for (size_t i = 0; i < ntensors; ++i) {
+        const size_t bytes = i < args.inputs.size() ? args.inputs[i].nbytes() : args.outputs[i - args.inputs.size()].nbytes();
+        void *dev = nullptr;
+        hipError_t e = devAlloc(bytes, &dev);
+        if (e == hipSuccess && i < args.inputs.size() && bytes)
+          e = hipMemcpyAsync(dev, slots[i], bytes, hipMemcpyDeviceToDevice, stream_);
+        if (e != hipSuccess) { cleanup(); return Status::error(hipErr("copy of the tensors for rotation", e)); }
+        sets[k][i] = dev;
+      }
+
     // ---- launch ----
     const uint32_t bd = (uint32_t)(args.block_dim < 0 ? 0 : args.block_dim);
     double bestUs = -1.0;
     for (int rep = 0; rep <= (args.timing_repeats > 0 ? args.timing_repeats : 0); ++rep) {
+    void **use = sets[rep % nsets].data();
     (void)hipEventRecord(ev0_, stream_);
     uint32_t rc;
     if (regionLaunch) {
       const int nargs = (int)(args.inputs.size() + args.outputs.size());
-      rc = regionLaunch(region, bd, stream_, nargs, slots, workspace, args.tiling.data(),
+      rc = regionLaunch(region, bd, stream_, nargs, use, workspace, args.tiling.data(),
                         args.tiling.size());
     } else {
-      rc = launchFn(bd, stream_, slots[0], slots[1], slots[2], slots[3], slots[4], slots[5],
-                    slots[6], slots[7], slots[8], slots[9], slots[10], slots[11], slots[12],
-                    slots[13], slots[14], slots[15]);
+      rc = launchFn(bd, stream_, use[0], use[1], use[2], use[3], use[4], use[5],
+                    use[6], use[7], use[8], use[9], use[10], use[11], use[12],
+                    use[13], use[14], use[15]);
     }
     if (rc != 0) {
       std::string why = lastError ? lastError() : "";

@@ -98,6 +98,10 @@ struct RunArgs {
   // kernels are pure functions of their inputs): the reported kernel time is the
   // fastest of 1 + timing_repeats launches.  For searches that score by time.
   int timing_repeats = 0;
+  // > 1: the timed launches rotate over this many copies of the tensors on the device, so that
+  // no launch finds its inputs in the last-level cache (256 MB on MI355X) because the launch
+  // before it left them there.  The outputs handed back are those of the first copy.
+  int buffer_sets = 1;
 };
 
 // ------------------------------------------------------------------- npy ----

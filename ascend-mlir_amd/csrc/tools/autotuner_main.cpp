@@ -10,7 +10,7 @@
 //   autotuner --space tiling_space.json (--kernel K.mlir | --artifact-root DIR)
 //             --inputs a.npy,b.npy --expected e.npy --shape M=32,N=32
 //             [--output best_config.json] [--kernel-kind vec|cube|mix] [--soc S]
-//             [--atol A] [--rtol R] [--repeats N] [--device N]
+//             [--atol A] [--rtol R] [--repeats N] [--buffer-sets N] [--device N]
 //
 // tiling_space.json: {"kernel", "kernel_file", "soc", "block_dim_expr",
 //   "block_dim_values": [..] (this backend: explicit grid sizes to try, 0 =
@@ -23,7 +23,15 @@
 // compiled into its own artifact under the build directory and is not part of
 // the TilingData bytes.
 //
+// A parameter named build_<MACRO> is a compile-time choice of the hand-tuned
+// kernels (tile shapes, rings, grids: the AFIR_* macros of csrc/kernels): every
+// combination is built into a kernel library of its own under the build
+// directory (python3 build.py --variant ... -DMACRO=value, beside this tool's
+// bin/ directory; needs hipcc) and the candidate is launched from that library.
+// Like emit_* it is not part of the TilingData bytes.
+//
 // Exit codes: 0 ok, 1 no candidate passed, 2 run error, 4 bad invocation.
+#include <cctype>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -34,11 +42,24 @@
 #include <string>
 #include <vector>
 
+#include <unistd.h>
+
 #include "../runtime/runtime.h"
 
 namespace {
 
 using namespace afirt;
+
+// Directory of this executable (bin/), for the build script beside it.
+std::string toolDirectory() {
+  char buf[4096];
+  const ssize_t n = readlink("/proc/self/exe", buf, sizeof buf - 1);
+  if (n <= 0) return ".";
+  buf[n] = 0;
+  std::string path(buf);
+  const size_t slash = path.rfind('/');
+  return slash == std::string::npos ? "." : path.substr(0, slash);
+}
 
 struct Param {
   std::string name, type = "int64", shapeKey;
@@ -264,6 +285,9 @@ int main(int argc, char **argv) {
   const double atol = opt.count("atol") ? std::atof(opt["atol"].c_str()) : 1.0;
   const double rtol = opt.count("rtol") ? std::atof(opt["rtol"].c_str()) : 1e-2;
   const int repeats = opt.count("repeats") ? std::max(1, std::atoi(opt["repeats"].c_str())) : 5;
+  // --buffer-sets N: the timed launches of a candidate rotate over N copies of its tensors on the
+  // device, so that repeated launches are not served from the last-level cache
+  const int bufferSets = opt.count("buffer-sets") ? std::max(1, std::atoi(opt["buffer-sets"].c_str())) : 1;
 
   DynamicLibraryExecutionLaunch launch;
   launch.sharedLibraryPath = artifact.sharedLibraryPath;
@@ -300,10 +324,14 @@ int main(int argc, char **argv) {
     // tiling bytes in the order of the space
     std::vector<TilingField> fields;
     std::vector<std::pair<std::string, int64_t>> values;
-    std::map<std::string, int64_t> emitOptions;
+    std::map<std::string, int64_t> emitOptions, buildMacros;
     for (const Param &p : space) {
       if (p.name.rfind("emit_", 0) == 0) {
         emitOptions[p.name.substr(5)] = vars[p.name];
+        continue;
+      }
+      if (p.name.rfind("build_", 0) == 0) {
+        buildMacros[p.name.substr(6)] = vars[p.name];
         continue;
       }
       fields.push_back({p.name, p.type});
@@ -329,6 +357,36 @@ int main(int argc, char **argv) {
         continue;
       }
       candidateArtifact = *a;
+    }
+    // hand-tuned kernels built with these choices: one kernel library per combination
+    if (!buildMacros.empty() && !testing) {
+      const std::string variantDir = !baseRequest.outputDir.empty() ? baseRequest.outputDir
+                                     : opt.count("build-dir")        ? opt["build-dir"]
+                                                                     : opt["space"] + ".artifact";
+      std::string lib = variantDir + "/variant";
+      std::string flags;
+      for (const auto &kv : buildMacros) {
+        for (char ch : kv.first)
+          if (!(std::isalnum((unsigned char)ch) || ch == '_')) return usage("build_* parameter names must be macro names");
+        lib += "_" + kv.first + std::to_string(kv.second);
+        flags += " -D" + kv.first + "=" + std::to_string(kv.second);
+      }
+      lib += ".so";
+      if (!std::ifstream(lib).good()) {
+        const std::string cmd = "mkdir -p '" + variantDir + "' && python3 '" + toolDirectory() +
+                                "/../build.py' --variant '" + lib + "'" + flags + " > '" + lib + ".log' 2>&1";
+        if (std::system(cmd.c_str()) != 0) {
+          for (int64_t bd : dims) {
+            ++index;
+            std::printf("[%zu/%zu]", index, total);
+            for (const auto &kv : combo) std::printf(" %s=%lld", kv.first.c_str(), (long long)kv.second);
+            std::printf(" block_dim=%lld ... FAIL  the kernel library does not build with these choices (%s.log)\n",
+                        (long long)bd, lib.c_str());
+          }
+          continue;
+        }
+      }
+      candidateArtifact.sharedLibraryPath = lib;
     }
     launch.sharedLibraryPath = candidateArtifact.sharedLibraryPath;
     launch.symbolName = candidateArtifact.sharedLibrarySymbol;
@@ -361,6 +419,7 @@ int main(int argc, char **argv) {
       // one run: the kernel is launched 1 + (repeats - 1) times on the same device buffers
       double bestNs = -1;
       args.timing_repeats = repeats - 1;
+      args.buffer_sets = bufferSets;
       Status st = runner->runDynamicLibraryArtifact(launch, args);
       const double us = runner->lastKernelMicroseconds();
       if (st.ok() && us >= 0) bestNs = us * 1e3;

@@ -513,7 +513,9 @@ def make_workload(key, torch, H, O, C):
         # this chip sustains on a plain copy, on a read-only stream and on the address pattern of
         # c3's tiled transpose with the transposition left out.  No oracle: nothing is computed.
         from ascend_mlir_amd import bench_probes as P
-        nbytes = 64 << 20
+        # 128 MiB for the read-only stream: as long a launch as the copies' (a 10 us launch would
+        # measure the host's launch rate)
+        nbytes = (128 << 20) if key == "ceil_read" else (64 << 20)
         w.dtype = "u8"
         w.nsets = 4
         w.no_cpu = True
@@ -527,7 +529,7 @@ def make_workload(key, torch, H, O, C):
             w.parity = lambda: {"bar": "dst == src", "passed": bool(torch.equal(srcs[0], dsts[0])),
                                 "mismatches": int((srcs[0] != dsts[0]).sum().item())}
         elif key == "ceil_read":
-            w.title = "ceil_read: 64 MiB read-only stream, 128-bit non-temporal loads (probe)"
+            w.title = "ceil_read: 128 MiB read-only stream, 128-bit non-temporal loads (probe)"
             sink = torch.zeros(8192, dtype=torch.float32, device="cuda")
             w.work = lambda: nbytes
             w.launches = [P.prepare("afir_bench_read", a.data_ptr(), sink.data_ptr(), nbytes) for a in srcs]

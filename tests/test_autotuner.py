@@ -130,3 +130,40 @@ def test_emit_parameters_compile_one_artifact_per_candidate(tmp_path):
             "--shape", "B=2", "--output", str(tmp_path / "best.json"), "--build-dir", str(tmp_path / "art2"),
             "--testing-driver=hip-success")
     assert p.returncode == 0 and p.stdout.count(" FAIL ") == 2 and "tile_q must be 64, 128 or 256" in p.stdout
+
+
+def test_build_parameters_stay_out_of_the_tiling_bytes(tmp_path):
+    """build_<MACRO> parameters choose a variant of the hand-tuned kernel library; like emit_*
+    they are enumerated with the rest of the space and never reach the TilingData bytes.  The
+    testing driver builds nothing."""
+    space = {"block_dim_values": [0],
+             "tiling_params": [{"name": "build_AFIR_ROWSUM_WG_PER_CU", "values": [1, 2, 4]}, *DIMS]}
+    p = _at(*_setup(tmp_path, space), "--shape", "M=8,N=32", "--buffer-sets", "3")
+    assert p.returncode == 0, p.stderr + p.stdout
+    lines = [l for l in p.stdout.splitlines() if l.startswith("[")]
+    assert len(lines) == 3 and all(" OK " in l for l in lines)
+    assert [l.split()[1] for l in lines] == [f"build_AFIR_ROWSUM_WG_PER_CU={v}" for v in (1, 2, 4)]
+    best = json.loads((tmp_path / "best.json").read_text())
+    assert best["config"]["build_AFIR_ROWSUM_WG_PER_CU"] in (1, 2, 4)
+    assert {k: v for k, v in best["config"].items() if not k.startswith("build_")} == \
+        {"dim_arg0_0": 8, "dim_arg1_0": 8, "dim_arg1_1": 32, "dim_arg2_0": 8}
+
+
+def test_kernel_library_variant_builds_only_what_the_macro_touches(tmp_path):
+    """build.py --variant: the library a build_* candidate loads.  Only the sources that
+    mention the macro are recompiled; the result exports the launchers of the ordinary library
+    and finds the families' code objects beside it."""
+    import ctypes
+    import sys
+    out = tmp_path / "variant_AFIR_ELTWISE_UNROLL4.so"
+    p = subprocess.run([sys.executable, os.path.join(ROOT, "ascend-mlir_amd", "build.py"), "--variant", str(out),
+                        "-DAFIR_ELTWISE_UNROLL=4"], capture_output=True, text=True)
+    assert p.returncode == 0, p.stderr + p.stdout
+    assert sorted(os.listdir(tmp_path / "obj_AFIR_ELTWISE_UNROLL-4")) == ["kernels_eltwise.hip.o"]
+    assert os.path.isdir(tmp_path / "families")
+    lib = ctypes.CDLL(str(out))
+    for sym in ("afir_hip_launch_fused_add_mul", "afir_hip_launch_region", "afir_hip_launch_matmul_add_leakyrelu"):
+        assert hasattr(lib, sym), sym
+    bad = subprocess.run([sys.executable, os.path.join(ROOT, "ascend-mlir_amd", "build.py"), "--variant", str(out),
+                          "AFIR_ELTWISE_UNROLL=4"], capture_output=True, text=True)
+    assert bad.returncode != 0 and "usage" in bad.stderr
