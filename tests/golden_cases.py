@@ -46,3 +46,21 @@ def cases():
     yield "microcase-relu_only", None, RELU_ONLY, [g(e + "input")], g(e + "expected"), True
     e = "real-npu-microcases/broadcast_add/"
     yield "microcase-broadcast_add", None, BROADCAST_ADD, [g(e + "input"), g(e + "bias")], g(e + "expected"), True
+
+
+def mean_case():
+    """The reference's mean graph (examples/broadcast-add-reduce/step0_input_mean.mlir) on the vectors its
+    gen_data.py wrote for the sum.  The reference holds no mean output; its sum does fix the mean to one
+    f16 ulp: mean = sum / N, and output_c is that sum rounded to f16 once already."""
+    z = load()
+    e = "broadcast-add-reduce/"
+    a, b, c = (np.ascontiguousarray(z[e + k]) for k in ("input_a", "input_b", "output_c"))
+    want = (c.astype(np.float32) / np.float32(b.shape[1])).astype(np.float16)
+    return MC.ROW_BIAS_MEAN, [a, b], want
+
+
+def within_one_f16_ulp(got, want):
+    g = got.astype(np.float64)
+    w = want.astype(np.float64)
+    ulp = np.maximum(np.abs(np.spacing(want).astype(np.float64)), 2.0 ** -24)
+    return bool(np.all(np.abs(g - w) <= ulp))

@@ -50,3 +50,13 @@ def test_translated_graph_evaluates_to_the_reference_output(case):
     got = RO.evaluate(program, inputs)
     assert got.dtype == want.dtype and got.shape == want.shape
     assert got.tobytes() == want.tobytes()      # numpy pairwise f32 sum in both: the reduce is exact too
+
+
+def test_mean_graph_agrees_with_the_reference_sum_vector():
+    mlir, inputs, want = GC.mean_case()
+    p = subprocess.run([TR, "-mlir-to-hip", "-"], input=mlir, capture_output=True, text=True)
+    assert p.returncode == 0, p.stderr
+    got = RO.evaluate(p.stdout, inputs)
+    assert got.dtype == want.dtype and got.shape == want.shape
+    assert GC.within_one_f16_ulp(got, want)
+    assert np.mean(got.view(np.uint16) == want.view(np.uint16)) > 0.5     # the second rounding moves the rest by one ulp

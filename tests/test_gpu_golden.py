@@ -41,3 +41,23 @@ def test_kernel_reproduces_the_reference_output(pkg, monkeypatch, tmp_path_facto
     else:   # f32 row sum in another order, one rounding to f16
         assert np.all(np.abs(got.astype(np.float64) - want.astype(np.float64))
                       <= 2.0 ** -10 * np.abs(want.astype(np.float64)) + 1e-3)
+
+
+@pytest.mark.parametrize("generic", ["routed", "generic", "compiled"])
+def test_mean_kernel_agrees_with_the_reference_sum_vector(pkg, monkeypatch, tmp_path_factory, generic):
+    import torch
+    from ascend_mlir_amd import hip_kernels as H
+    H.load()
+    mlir, inputs, want = GC.mean_case()
+    p = subprocess.run([TR, "-mlir-to-hip", "-"], input=mlir, capture_output=True, text=True)
+    assert p.returncode == 0, p.stderr
+    monkeypatch.setenv("AFIR_HIP_REGION_GENERIC", "0" if generic == "routed" else "1")
+    r = H.Region(p.stdout)
+    if generic == "compiled":
+        r.compile(cache_dir=str(tmp_path_factory.mktemp("region_cache")))
+        assert r.kernel == "fused_region_compiled"
+    got = r(*[torch.from_numpy(x).cuda() for x in inputs], out_shape=want.shape).cpu().numpy()
+    r.close()
+    # sum in another order, then the division: one ulp for each
+    g, w = got.astype(np.float64), want.astype(np.float64)
+    assert np.all(np.abs(g - w) <= 2.0 ** -9 * np.abs(w) + 1e-5)
