@@ -682,6 +682,10 @@ def main():
         "parity": main_e["parity"],
     }
     line["roofline"]["traffic_source"] = main_e["roofline"]["traffic_source"]
+    if "power_limit_evidence" in main_e and not args.all:
+        for k in ("frac_of_mfma_only", "vs_vendor_gemm"):
+            line["roofline"][k] = main_e["roofline"][k]
+        line["power_limit_evidence"] = main_e["power_limit_evidence"]
     if "cpu_baseline" in main_e:
         line["cpu_baseline"] = {k: main_e["cpu_baseline"][k] for k in
                                 ("value", "unit", "cores", "kind", "sample")}
