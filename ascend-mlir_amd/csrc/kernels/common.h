@@ -72,6 +72,14 @@ __device__ __forceinline__ uint32_t f32_to_bf16_rne(float f) {
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   return (f32_to_bf16_rne(lo) & 0xffffu) | (f32_to_bf16_rne(hi) << 16);
 }
+// The same two roundings in one instruction (v_cvt_pk_bf16_f32): bit-identical to pack_bf16 on
+// every pair of non-NaN floats; a NaN stays a NaN (quiet bit set, top payload bits kept).
+__device__ __forceinline__ uint32_t pack_bf16_hw(float lo, float hi) {
+  typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+  typedef float f32x2_t __attribute__((ext_vector_type(2)));
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
 
 // ---- wavefront reduction on DPP -------------------------------------------
 

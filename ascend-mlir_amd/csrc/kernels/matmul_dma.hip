@@ -235,62 +235,98 @@ __global__ __launch_bounds__(kWaves * 64) void matmul_bias_leakyrelu_dma(
                               ((lane & 31) ^ ((bk & 3) << 2) ^ (((bk >> 3) & 1) << 1)) * 8) * 2);
   }
 
-  for (int p = blockIdx.x; p < tiles_m * tiles_n; p += gridDim.x) {
+  // ---- state of the tile whose rings are being filled (set by begin_tile) ----
+  // wave-uniform sources of the direct-to-LDS loads:
+  // A slice: 32 regions of 1 KiB (8 rows x 128 B), kAReg per wave.
+  // B stage: 16 regions of 1 KiB (2 rows x 512 B), kBReg per wave.
+  int m0 = 0, n0 = 0;
+  const char *ua = nullptr, *ub = nullptr;
+  const int64_t a_region = (int64_t)K * 16;   // 8 rows of A
+  const int64_t b_region = (int64_t)N * 4;    // 2 rows of B
+  int ka_next = 0;  // slice (64 k) the next A issue fetches
+  int kb_next = 0;  // stage (32 k) the next B issue fetches
+  auto begin_tile = [&](int p) {
     int tile_m, tile_n;
     map_tile_dma(p, tiles_m, tiles_n, tile_m, tile_n);
-    const int m0 = tile_m * kBM, n0 = tile_n * kBN;
-
+    m0 = tile_m * kBM;
+    n0 = tile_n * kBN;
     // K-stagger: this tile walks stages kfirst, kfirst+1, ..., wrapping at KT.
     // kfirst is even so that A slices (two stages) stay aligned.
     const int kfirst =
         (int)(((unsigned)(tile_m * AFIR_MM_KSTAGGER_M + tile_n * AFIR_MM_KSTAGGER_N) * 2u) %
               (unsigned)KT);
+    ua = reinterpret_cast<const char *>(A) +
+         ((int64_t)(m0 + wave * (kAReg * 8)) * K + (int64_t)kfirst * kBK) * 2;
+    ub = reinterpret_cast<const char *>(B) +
+         ((int64_t)(wave * (kBReg * 2) + kfirst * kBK) * N + n0) * 2;
+    ka_next = kfirst >> 1;
+    kb_next = kfirst;
+  };
+  // one region: lane l's 16 bytes go to lds_offset + 16 l
+  auto dma = [&](const char *base, uint32_t lane_offset, uint32_t lds_offset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_offset), "v"(lane_offset), "s"(base)
+                 : "memory");
+  };
+  auto issue_a_region = [&](int slot, auto q_tag) {
+    constexpr int q = decltype(q_tag)::value;
+    dma(ua + q * a_region, a_lane[q & 1],
+        lds_base + (uint32_t)(slot * kSlotA + wave * (kAReg * 1024) + q * 1024));
+  };
+  auto advance_a = [&]() {
+    ka_next = (ka_next + 1 == KT2) ? 0 : ka_next + 1;
+    ua += (ka_next == 0) ? -(int64_t)(KT2 - 1) * 128 : (int64_t)128;
+  };
+  auto issue_b_region = [&](int slot, auto q_tag) {
+    constexpr int q = decltype(q_tag)::value;
+    dma(ub + q * b_region, b_lane[q & 1],
+        lds_base + (uint32_t)(kRingB + slot * kSlotB + wave * (kBReg * 1024) + q * 1024));
+  };
+  auto advance_b = [&]() {
+    kb_next = (kb_next + 1 == KT) ? 0 : kb_next + 1;
+    ub += ((kb_next == 0) ? -(int64_t)(KT - 1) : (int64_t)1) * kBK * N * 2;
+  };
+  auto issue_a = [&](int slot) {
+    static_for<0, kAReg>([&](auto q) { issue_a_region(slot, q); });
+    advance_a();
+  };
+  auto issue_b = [&](int slot) {
+    static_for<0, kBReg>([&](auto q) { issue_b_region(slot, q); });
+    advance_b();
+  };
+  // The fill of both rings at the start of a tile, oldest first: A(0) B(0) B(1) A(1) B(2) B(3)
+  // A(2) (the launcher guarantees KT >= 8).  All of it but A(2) is issued *during the epilogue
+  // of the previous tile*, one region behind each block of epilogue arithmetic: the rings are
+  // free once every wave has left the K loop, the epilogue stages its rows in A slot 2, and so
+  // the first stages of the next tile are in LDS (and the issue cost of 160 KiB of loads is paid
+  // behind vector arithmetic) by the time the epilogue's last store is out.  The float32 output
+  // form needs twice the staging room and keeps the whole fill after its epilogue.
+  constexpr bool kEarlyFill = !F16IO;
+  constexpr int kEarlyRegions = 2 * kAReg + 4 * kBReg;
+  auto early_fill_item = [&](auto x_tag) {
+    constexpr int X = decltype(x_tag)::value;
+    constexpr int a0 = 0, b0 = kAReg, b1 = b0 + kBReg, a1 = b1 + kBReg, b2 = a1 + kAReg, b3 = b2 + kBReg;
+    if constexpr (X < b0) issue_a_region(0, std::integral_constant<int, X - a0>{});
+    else if constexpr (X < b1) issue_b_region(0, std::integral_constant<int, X - b0>{});
+    else if constexpr (X < a1) issue_b_region(1, std::integral_constant<int, X - b1>{});
+    else if constexpr (X < b2) issue_a_region(1, std::integral_constant<int, X - a1>{});
+    else if constexpr (X < b3) issue_b_region(2, std::integral_constant<int, X - b2>{});
+    else issue_b_region(3, std::integral_constant<int, X - b3>{});
+    if constexpr (X == b0 - 1 || X == b2 - 1) advance_a();
+    if constexpr (X == b1 - 1 || X == a1 - 1 || X == b3 - 1 || X == kEarlyRegions - 1) advance_b();
+  };
 
-    // ---- wave-uniform sources of the direct-to-LDS loads ----
-    // A slice: 32 regions of 1 KiB (8 rows x 128 B), kAReg per wave.
-    // B stage: 16 regions of 1 KiB (2 rows x 512 B), kBReg per wave.
-    const char *ua = reinterpret_cast<const char *>(A) +
-                     ((int64_t)(m0 + wave * (kAReg * 8)) * K + (int64_t)kfirst * kBK) * 2;
-    const char *ub = reinterpret_cast<const char *>(B) +
-                     ((int64_t)(wave * (kBReg * 2) + kfirst * kBK) * N + n0) * 2;
-    const int64_t a_region = (int64_t)K * 16;   // 8 rows of A
-    const int64_t b_region = (int64_t)N * 4;    // 2 rows of B
-    int ka_next = kfirst >> 1;  // slice (64 k) the next A issue fetches
-    int kb_next = kfirst;       // stage (32 k) the next B issue fetches
-
-    // one region: lane l's 16 bytes go to lds_offset + 16 l
-    auto dma = [&](const char *base, uint32_t lane_offset, uint32_t lds_offset) {
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                   :
-                   : "s"(lds_offset), "v"(lane_offset), "s"(base)
-                   : "memory");
-    };
-    auto issue_a_region = [&](int slot, auto q_tag) {
-      constexpr int q = decltype(q_tag)::value;
-      dma(ua + q * a_region, a_lane[q & 1],
-          lds_base + (uint32_t)(slot * kSlotA + wave * (kAReg * 1024) + q * 1024));
-    };
-    auto advance_a = [&]() {
-      ka_next = (ka_next + 1 == KT2) ? 0 : ka_next + 1;
-      ua += (ka_next == 0) ? -(int64_t)(KT2 - 1) * 128 : (int64_t)128;
-    };
-    auto issue_b_region = [&](int slot, auto q_tag) {
-      constexpr int q = decltype(q_tag)::value;
-      dma(ub + q * b_region, b_lane[q & 1],
-          lds_base + (uint32_t)(kRingB + slot * kSlotB + wave * (kBReg * 1024) + q * 1024));
-    };
-    auto advance_b = [&]() {
-      kb_next = (kb_next + 1 == KT) ? 0 : kb_next + 1;
-      ub += ((kb_next == 0) ? -(int64_t)(KT - 1) : (int64_t)1) * kBK * N * 2;
-    };
-    auto issue_a = [&](int slot) {
-      static_for<0, kAReg>([&](auto q) { issue_a_region(slot, q); });
-      advance_a();
-    };
-    auto issue_b = [&](int slot) {
-      static_for<0, kBReg>([&](auto q) { issue_b_region(slot, q); });
-      advance_b();
-    };
+  const int total_tiles = tiles_m * tiles_n;
+  if ((int)blockIdx.x < total_tiles) {
+    begin_tile(blockIdx.x);
+    static_for<0, kEarlyRegions>([&](auto x) { early_fill_item(x); });
+    issue_a(2);
+  }
+  for (int p = blockIdx.x; p < total_tiles; p += gridDim.x) {
+    // the tile being computed (m0 / n0 move on to the next tile during the epilogue)
+    const int out_m0 = m0, out_n0 = n0;
+    const bool has_next_tile = p + (int)gridDim.x < total_tiles;
 
     f32x4 acc[kTM][kTN];
 #pragma unroll
@@ -311,15 +347,11 @@ __global__ __launch_bounds__(kWaves * 64) void matmul_bias_leakyrelu_dma(
       for (int j = 0; j < kTN; ++j) ba[j] = bb ^ (uint32_t)(j * 32);
     };
 
-    // prologue (the launcher guarantees KT >= 8): fill both rings, oldest first
-    issue_a(0);
-    issue_b(0);
-    issue_b(1);
-    issue_a(1);
-    issue_b(2);
-    issue_b(3);
-    issue_a(2);
-    wait_vmcnt<3 * kBReg + 2 * kAReg>();  // everything younger than A(0), B(0)
+    // the rings were filled before the loop or during the previous epilogue.  At most the loads
+    // younger than A(0), B(0) may be outstanding; stores of the previous epilogue that are still
+    // on their way only make this wait stricter (loads complete in order among themselves, so
+    // A(0) or B(0) outstanding means all the younger loads are too: more than the bound).
+    wait_vmcnt<3 * kBReg + 2 * kAReg>();
     __builtin_amdgcn_s_barrier();
     // Operand registers: the A fragments of a stage in two halves (m tiles 0-3, 4-7), the B
     // fragments of a stage twice (the stage being multiplied and the next one).
@@ -355,6 +387,9 @@ __global__ __launch_bounds__(kWaves * 64) void matmul_bias_leakyrelu_dma(
     // state both exist and the vmcnt is exact: younger than what stage s+1 needs
     // are exactly 2 B stages and 1 A slice.  Otherwise drain.
     int sa = 0, sb = 0;  // ring slots of the stage being multiplied
+    // (opaque: with known slots the compiler precomputes the operand addresses of the first two
+    // steps once per kernel, spills them, and the reload waits for the whole ring fill)
+    asm volatile("" : "+s"(sa), "+s"(sb));
     auto pin = [] { __builtin_amdgcn_sched_barrier(0); };
     // MFMA number X of a phase: n tile X / 4, m tile FIRST + X % 4
     auto mfma = [&](auto first_tag, auto x_tag, const u32x4 (&a)[4], const u32x2 (&b)[kTN][2]) {
@@ -484,17 +519,28 @@ __global__ __launch_bounds__(kWaves * 64) void matmul_bias_leakyrelu_dma(
     // full lines, eight or four rows per instruction.  The rings are free once
     // every wave has left the K loop; a wave's 4 or 8 KiB staging area is
     // private, and the LDS unit keeps a wave's accesses in order, so no further
-    // barrier is needed until the next tile refills the rings.  The 16-byte
+    // barrier is needed until the staging room is refilled.  The 16-byte
     // chunk column is XOR-ed with a function of the row: conflict-free for the
     // 8- or 16-byte writes and for the 16-byte row reads.
     __builtin_amdgcn_s_barrier();
+    if (has_next_tile) begin_tile(p + (int)gridDim.x);
     {
       constexpr int kOutBytes = F16IO ? 4 : 2;
       constexpr int CH = kTN * 16 * kOutBytes / 16;   // 16-byte chunks per staged row: 8 or 16
       constexpr int kRowBytes = CH * 16;       // 128 or 256
       constexpr int kRowsPerPass = 64 / CH;    // rows one store instruction covers
-      unsigned char *const stage = smem + wave * (32 * kRowBytes);
-      const int rr = lane / CH, cc = lane % CH;
+      // The lane number again, opaque to the compiler: everything per lane that the epilogue
+      // needs (staging addresses, bias columns, output rows) is then computed here, once per
+      // tile, instead of once per kernel.  Hoisted out of the tile loop those values do not fit
+      // the register file beside the K loop, and a reload from scratch memory makes the compiler
+      // wait for *every* outstanding memory operation - each store of the epilogue and the fill of
+      // the next tile - before it goes on.
+      int lane_e;
+      asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(lane_e));
+      const int li = lane_e & 15, g = lane_e >> 4;
+      // bf16: A slot 2, which the early fill of the next tile leaves alone
+      unsigned char *const stage = smem + (kEarlyFill ? 2 * kSlotA : 0) + wave * (32 * kRowBytes);
+      const int rr = lane_e / CH, cc = lane_e % CH;
       // two 128-byte rows share a swizzle value (they span the same banks as
       // one 256-byte row)
       auto swz = [](int r) { return CH == 8 ? ((r >> 1) & 7) : (r & (CH - 1)); };
@@ -502,7 +548,7 @@ __global__ __launch_bounds__(kWaves * 64) void matmul_bias_leakyrelu_dma(
       BiasRaw braw[kTN];
 #pragma unroll
       for (int j = 0; j < kTN; ++j) {
-        const int n = n0 + (wn * kTN + j) * 16 + 4 * g;
+        const int n = out_n0 + (wn * kTN + j) * 16 + 4 * g;
         // no bias: -0, the identity of the add
         if constexpr (F16IO)
           braw[j] = bias_v ? *reinterpret_cast<const f32x4 *>(static_cast<const float *>(bias_v) + n)
@@ -511,56 +557,71 @@ __global__ __launch_bounds__(kWaves * 64) void matmul_bias_leakyrelu_dma(
           braw[j] = bias_v ? *reinterpret_cast<const u32x2 *>(static_cast<const uint16_t *>(bias_v) + n)
                            : u32x2{0x80008000u, 0x80008000u};
       }
-#pragma unroll
-      for (int ip = 0; ip < kTM / 2; ++ip) {
-#pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          const int lm = half * 16 + li;   // row within the 32 staged rows
-#pragma unroll
-          for (int j = 0; j < kTN; ++j) {
-            float b0, b1, b2, b3;
-            if constexpr (F16IO) {
-              b0 = braw[j][0]; b1 = braw[j][1]; b2 = braw[j][2]; b3 = braw[j][3];
-            } else {
-              b0 = bf16_lo(braw[j].x); b1 = bf16_hi(braw[j].x);
-              b2 = bf16_lo(braw[j].y); b3 = bf16_hi(braw[j].y);
+      // the activation is a launch argument: one copy of the passes per kind, chosen by a
+      // wave-uniform branch, so that no value pays a select
+      auto passes = [&](auto relu_tag) {
+        constexpr bool RELU = decltype(relu_tag)::value;
+        static_for<0, kTM / 2>([&](auto ip_tag) {
+          constexpr int ip = decltype(ip_tag)::value;
+          static_for<0, 2 * kTN>([&](auto hj_tag) {
+            constexpr int half = decltype(hj_tag)::value / kTN, j = decltype(hj_tag)::value % kTN;
+            const int lm = half * 16 + li;   // row within the 32 staged rows
+            {
+              float b0, b1, b2, b3;
+              if constexpr (F16IO) {
+                b0 = braw[j][0]; b1 = braw[j][1]; b2 = braw[j][2]; b3 = braw[j][3];
+              } else {
+                b0 = bf16_lo(braw[j].x); b1 = bf16_hi(braw[j].x);
+                b2 = bf16_lo(braw[j].y); b3 = bf16_hi(braw[j].y);
+              }
+              // one region of the next tile's fill behind each block of arithmetic
+              if constexpr (kEarlyFill && (ip * 2 + half) * kTN + j < kEarlyRegions) {
+                if (has_next_tile)
+                  early_fill_item(std::integral_constant<int, (ip * 2 + half) * kTN + j>{});
+              }
+              const f32x4 &c = acc[ip * 2 + half][j];
+              float v0 = c[0] + b0;
+              float v1 = c[1] + b1;
+              float v2 = c[2] + b2;
+              float v3 = c[3] + b3;
+              v0 = fmaxf(v0, RELU ? 0.f : v0 * alpha);
+              v1 = fmaxf(v1, RELU ? 0.f : v1 * alpha);
+              v2 = fmaxf(v2, RELU ? 0.f : v2 * alpha);
+              v3 = fmaxf(v3, RELU ? 0.f : v3 * alpha);
+              if constexpr (F16IO) {
+                const f32x4 w = {v0, v1, v2, v3};
+                const int chunk = (j * 4 + g) ^ swz(lm);
+                *reinterpret_cast<f32x4 *>(stage + lm * kRowBytes + chunk * 16) = w;
+              } else {
+                u32x2 w;
+                w.x = pack_bf16_hw(v0, v1);
+                w.y = pack_bf16_hw(v2, v3);
+                const int chunk = (j * 2 + (g >> 1)) ^ swz(lm);
+                *reinterpret_cast<u32x2 *>(stage + lm * kRowBytes + chunk * 16 + (g & 1) * 8) = w;
+              }
             }
-            const f32x4 &c = acc[ip * 2 + half][j];
-            float v0 = c[0] + b0;
-            float v1 = c[1] + b1;
-            float v2 = c[2] + b2;
-            float v3 = c[3] + b3;
-            v0 = fmaxf(v0, relu ? 0.f : v0 * alpha);
-            v1 = fmaxf(v1, relu ? 0.f : v1 * alpha);
-            v2 = fmaxf(v2, relu ? 0.f : v2 * alpha);
-            v3 = fmaxf(v3, relu ? 0.f : v3 * alpha);
-            if constexpr (F16IO) {
-              const f32x4 w = {v0, v1, v2, v3};
-              const int chunk = (j * 4 + g) ^ swz(lm);
-              *reinterpret_cast<f32x4 *>(stage + lm * kRowBytes + chunk * 16) = w;
-            } else {
-              u32x2 w;
-              w.x = pack_bf16(v0, v1);
-              w.y = pack_bf16(v2, v3);
-              const int chunk = (j * 2 + (g >> 1)) ^ swz(lm);
-              *reinterpret_cast<u32x2 *>(stage + lm * kRowBytes + chunk * 16 + (g & 1) * 8) = w;
-            }
+          });
+#pragma unroll
+          for (int tq = 0; tq < 32 / kRowsPerPass; ++tq) {
+            const int r = rr + kRowsPerPass * tq;
+            const u32x4 line =
+                *reinterpret_cast<const u32x4 *>(stage + r * kRowBytes + ((cc ^ swz(r)) * 16));
+            const int m = out_m0 + (wm * kTM + ip * 2) * 16 + r;
+            unsigned char *const row = static_cast<unsigned char *>(out_v) +
+                                       ((int64_t)m * N + out_n0 + wn * (kTN * 16)) * kOutBytes;
+            *reinterpret_cast<u32x4 *>(row + cc * 16) = line;
           }
-        }
-#pragma unroll
-        for (int tq = 0; tq < 32 / kRowsPerPass; ++tq) {
-          const int r = rr + kRowsPerPass * tq;
-          const u32x4 line =
-              *reinterpret_cast<const u32x4 *>(stage + r * kRowBytes + ((cc ^ swz(r)) * 16));
-          const int m = m0 + (wm * kTM + ip * 2) * 16 + r;
-          unsigned char *const row = static_cast<unsigned char *>(out_v) +
-                                     ((int64_t)m * N + n0 + wn * (kTN * 16)) * kOutBytes;
-          *reinterpret_cast<u32x4 *>(row + cc * 16) = line;
-        }
-      }
+        });
+      };
+      if (relu) passes(std::true_type{});
+      else passes(std::false_type{});
     }
-    // every wave must be done reading the rings before the next tile refills them
+    // every wave must be done with its staging rows before the rest of the next fill lands there
     __builtin_amdgcn_s_barrier();
+    if (has_next_tile) {
+      if constexpr (!kEarlyFill) static_for<0, kEarlyRegions>([&](auto x) { early_fill_item(x); });
+      issue_a(2);
+    }
   }
 }
 
