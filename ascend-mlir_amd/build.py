@@ -159,12 +159,12 @@ def build_families(kernel_lib):
 
 def build_probes():
     """libafir_bench_probes.so: ceiling probes for bench.py (csrc/bench/probes.h), and the
-    direct-to-LDS matmul kernel compiled twice more with parts of its K loop left out, each
+    direct-to-LDS matmul kernel compiled three more times with parts of its K loop left out, each
     under a namespace name of its own."""
     os.makedirs(LIB, exist_ok=True)
     os.makedirs(OBJ, exist_ok=True)
     jobs = [("bench/probes.hip", "bench_probes.o", [])]
-    for level in (1, 2):
+    for level in (1, 2, 3):
         jobs.append(("kernels/matmul_dma.hip", f"bench_matmul_ablate{level}.o",
                      [f"-DAFIR_MM_ABLATE={level}", f"-Dafir=afir_abl{level}"]))
 

@@ -38,7 +38,10 @@ uint32_t afir_bench_mfma_rate(void *stream, const void *operands, void *sink, ui
  *             operand reads, waits and barriers remain (operands stay those of
  *             the first K steps);
  *   what = 2  no LDS operand reads either: MFMAs on the registers the first
- *             reads filled, waits and barriers remain.
+ *             reads filled, waits and barriers remain;
+ *   what = 3  the whole kernel, but every global -> LDS load reads the same
+ *             1 KiB: the loads are issued and write LDS as always, without the
+ *             L2 / fabric / HBM traffic and latency behind them.
  * Same arguments as the kernel's launcher (bf16 A [m,k], B [k,n], bias [n], out
  * [m,n]; m, n multiples of 256, k of 64); the output is meaningless. */
 uint32_t afir_bench_matmul_ablated(void *stream, const void *a, const void *b, const void *bias,

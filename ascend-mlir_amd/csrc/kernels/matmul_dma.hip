@@ -55,6 +55,14 @@
 // 1565 / 1320; 16x16x32 interleaved as described 1700 / 1350-1365 (the vendor
 // GEMM without the epilogue, same runs: 1775 / 1360-1385).
 //
+// What the loop then waits for is the memory system behind the loads: with every
+// load pointed at the same 1 KiB (issue and LDS-write cost only) the kernel runs
+// 2095 / 1600, with real addresses 1770 / 1385.  A stage has only as long to
+// arrive as the rings are deep, so the refills go out as early as the barrier
+// allows (the B stage right behind the barrier of the step that frees its slot:
+// 1875 / 1455), and between tiles nothing drains: the first stages of the next
+// tile are requested during the epilogue (per-tile overhead 13 -> 6.5 us of 250).
+//
 // Every tile starts its walk over K at a different offset and wraps around
 // (K-stagger): the row pitch of A and B is a large power of two, so without it
 // all workgroups of the chip ask the same few L2 / memory channels for the
@@ -88,9 +96,23 @@ namespace {
 // Measurement builds only (the benchmark's probe library compiles this file again with
 // -DAFIR_MM_ABLATE=1 or 2 under another namespace name): 1 leaves the global -> LDS feed
 // out of the K loop after the prologue, 2 the LDS operand reads as well, so that what
-// remains can be timed on its own.  Such a build computes nothing meaningful.
+// remains can be timed on its own; 3 keeps every load but points all of them at the same
+// 1 KiB (the cost of issuing the loads and writing LDS, without the memory system behind
+// them).  Such a build computes nothing meaningful.
 #ifndef AFIR_MM_ABLATE
 #define AFIR_MM_ABLATE 0
+#endif
+// MFMAs between two refill loads of a phase (1: back to back; 2 measured 0.5 % faster)
+// 1: the B stage that a step frees is refilled in that step's second phase, right after the
+// barrier, instead of in the next step's first phase (0).  A B stage then has 3 steps to
+// arrive instead of 2.2: 1400 -> 1455 TFLOP/s on the workload's operands, 1770 -> 1875 on
+// constants.  (The same move for the A slice, six loads in one phase beside its twelve operand
+// reads, measured 6 % slower: the reads come back late.)
+#ifndef AFIR_MM_B_EARLY
+#define AFIR_MM_B_EARLY 1
+#endif
+#ifndef AFIR_MM_DMA_STRIDE
+#define AFIR_MM_DMA_STRIDE 2
 #endif
 constexpr int kBK = 32;                   // K per B stage
 constexpr int kBM = 256, kBN = 256;
@@ -264,6 +286,10 @@ __global__ __launch_bounds__(kWaves * 64) void matmul_bias_leakyrelu_dma(
   };
   // one region: lane l's 16 bytes go to lds_offset + 16 l
   auto dma = [&](const char *base, uint32_t lane_offset, uint32_t lds_offset) {
+    if (AFIR_MM_ABLATE == 3) {   // every load reads the same 1 KiB: the issue and LDS-write cost alone
+      base = reinterpret_cast<const char *>(A);
+      lane_offset = (uint32_t)lane * 16u;
+    }
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
                  : "s"(lds_offset), "v"(lane_offset), "s"(base)
@@ -366,7 +392,7 @@ __global__ __launch_bounds__(kWaves * 64) void matmul_bias_leakyrelu_dma(
       settle(a_lo);
       settle(b_cur);
     }
-    if (AFIR_MM_ABLATE >= 2) {
+    if (AFIR_MM_ABLATE == 2) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) a_hi[i] = a_lo[i];
 #pragma unroll
@@ -382,10 +408,12 @@ __global__ __launch_bounds__(kWaves * 64) void matmul_bias_leakyrelu_dma(
     //   wait until stage s+1 has landed, barrier: everyone is done reading s
     //   reads of A(s+1) m tiles 0-3 and B(s+1) in flight, refill the freed slots
     //                                        | MFMAs of m tiles 4-7
-    // Refill after stage s: B(s+4) into s's B slot; after an odd s also the A
-    // slice (s+5)/2 into the slot of the slice just finished.  In the steady
-    // state both exist and the vmcnt is exact: younger than what stage s+1 needs
-    // are exactly 2 B stages and 1 A slice.  Otherwise drain.
+    // Refill after stage s: B(s+4) into s's B slot, right after the barrier of step s; after
+    // an odd s also the A slice (s+5)/2 into the slot of the slice just finished, behind the
+    // first MFMAs of step s+1.  In the steady state both exist and the vmcnt is exact: the
+    // loads younger than what stage s+1 needs are 2 B stages and 2 A slices at an even s
+    // (B(s+2), B(s+3), and the slices issued in steps s-2 and s), 2 B stages and 1 A slice at
+    // an odd s.  Otherwise drain.
     int sa = 0, sb = 0;  // ring slots of the stage being multiplied
     // (opaque: with known slots the compiler precomputes the operand addresses of the first two
     // steps once per kernel, spills them, and the reload waits for the whole ring fill)
@@ -402,9 +430,10 @@ __global__ __launch_bounds__(kWaves * 64) void matmul_bias_leakyrelu_dma(
         acc[FIRST + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
             __builtin_bit_cast(bf16x8, bw), __builtin_bit_cast(bf16x8, a[i]), acc[FIRST + i][j], 0, 0, 0);
     };
-    // Refills wait for the step after the one that frees their slots, so that they can go out
-    // behind the MFMAs of phase 1, which carries few operand reads: pend_b / pend_a say what the
-    // previous step left to issue, pend_sa / pend_sb into which slots.
+    // The A refill waits for the step after the one that frees its slot, so that it goes out
+    // behind the MFMAs of phase 1, which carries few operand reads: pend_a says whether the
+    // previous step left one to issue, pend_sa into which slot (pend_b / pend_sb: the same for
+    // the B stage when AFIR_MM_B_EARLY is 0).
     bool pend_a = false, pend_b = false;
     int pend_sa = 0, pend_sb = 0;
     // pend_tag: what is known at compile time about the refills the previous step left: 0 none
@@ -423,21 +452,24 @@ __global__ __launch_bounds__(kWaves * 64) void matmul_bias_leakyrelu_dma(
       // left (its A slice, if any, before its B stage).
       {
         const uint32_t aa = a_address(sa, PAR);
-        const bool do_a = AFIR_MM_ABLATE == 0 && (PEND == 1 ? !PAR : PEND == 2 && pend_a);
-        const bool do_b = AFIR_MM_ABLATE == 0 && (PEND == 1 || (PEND == 2 && pend_b));
+        const bool do_a = (AFIR_MM_ABLATE == 0 || AFIR_MM_ABLATE == 3) && (PEND == 1 ? !PAR : PEND == 2 && pend_a);
+        const bool do_b = !AFIR_MM_B_EARLY && (AFIR_MM_ABLATE == 0 || AFIR_MM_ABLATE == 3) &&
+                          (PEND == 1 || (PEND == 2 && pend_b));
         pin();
         static_for<0, NM>([&](auto x) {
           constexpr int X = decltype(x)::value;
           mfma(std::integral_constant<int, 0>{}, x, a_lo, bs);
           pin();
+          constexpr int kStride = AFIR_MM_DMA_STRIDE;   // MFMAs between two refill loads
+          constexpr int I = X >= 4 && (X - 4) % kStride == 0 ? (X - 4) / kStride : -1;
           if constexpr (X < 4) {
-            if (AFIR_MM_ABLATE < 2) read_a<(4 + X) * 2048>(aa, a_hi[X]);
+            if (AFIR_MM_ABLATE != 2) read_a<(4 + X) * 2048>(aa, a_hi[X]);
             pin();
-          } else if constexpr (!PAR && X < 4 + kAReg) {   // the step before an even stage was odd: A slice
-            if (do_a) issue_a_region(pend_sa, std::integral_constant<int, X - 4>{});
+          } else if constexpr (!PAR && I >= 0 && I < kAReg) {   // the step before an even stage was odd: A slice
+            if (do_a) issue_a_region(pend_sa, std::integral_constant<int, I>{});
             pin();
-          } else if constexpr (X >= 4 + kAReg && X < 4 + kAReg + kBReg) {
-            if (do_b) issue_b_region(pend_sb, std::integral_constant<int, X - 4 - kAReg>{});
+          } else if constexpr (I >= kAReg && I < kAReg + kBReg) {
+            if (do_b) issue_b_region(pend_sb, std::integral_constant<int, I - kAReg>{});
             pin();
           }
         });
@@ -461,7 +493,7 @@ __global__ __launch_bounds__(kWaves * 64) void matmul_bias_leakyrelu_dma(
           pin();
           if constexpr (X == 0) {
             if (STEADY)
-              wait_vmcnt<kSteadyVm>();
+              wait_vmcnt<AFIR_MM_B_EARLY ? (PAR ? 2 * kBReg + kAReg : 2 * kBReg + 2 * kAReg) : kSteadyVm>();
             else
               wait_vmcnt<0>();
             __builtin_amdgcn_s_barrier();
@@ -469,15 +501,22 @@ __global__ __launch_bounds__(kWaves * 64) void matmul_bias_leakyrelu_dma(
           }
           if constexpr (X < 12) {
             constexpr int R = X;   // B tile 0, A tiles 0-3, B tiles 1-3
-            if (AFIR_MM_ABLATE < 2) {
+            if (AFIR_MM_ABLATE != 2) {
               if constexpr (R < 2) read_b<R * 4 * 512>(ba[0], bn[0][R]);
               else if constexpr (R < 6) read_a<(R - 2) * 2048>(aa, a_lo[R - 2]);
               else read_b<((R - 6) % 2) * 4 * 512>(ba[1 + (R - 6) / 2], bn[1 + (R - 6) / 2][(R - 6) % 2]);
             }
             pin();
           }
+          if constexpr (AFIR_MM_B_EARLY && X >= 1 && X < 1 + kBReg) {
+            // everyone is past the barrier: stage s is read, its B slot takes stage s + 4
+            if ((AFIR_MM_ABLATE == 0 || AFIR_MM_ABLATE == 3) && (STEADY || refill_b))
+              issue_b_region(sb, std::integral_constant<int, X - 1>{});
+            pin();
+          }
         });
-        pend_b = STEADY || refill_b;
+        if (AFIR_MM_B_EARLY && (AFIR_MM_ABLATE == 0 || AFIR_MM_ABLATE == 3) && (STEADY || refill_b)) advance_b();
+        pend_b = !AFIR_MM_B_EARLY && (STEADY || refill_b);
         pend_a = PAR && (STEADY || refill_a);
         pend_sa = sa;
         pend_sb = sb;

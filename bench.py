@@ -391,12 +391,14 @@ def make_workload(key, torch, H, O, C):
             ours = lambda i: w.launches[i % len(w.launches)]()
             vendor = lambda i: torch.matmul(sets[i % len(sets)][0], sets[i % len(sets)][1])
             # alternating rounds: each kernel sees the same thermal history
-            rounds = {"this_kernel": [], "vendor_gemm": [], "no_feed": [], "no_feed_no_lds_reads": []}
+            rounds = {"this_kernel": [], "vendor_gemm": [], "no_feed": [], "no_feed_no_lds_reads": [],
+                      "loads_of_one_kib": []}
             for _ in range(3):
                 rounds["vendor_gemm"].append(rate(vendor))
                 rounds["this_kernel"].append(rate(ours))
                 rounds["no_feed"].append(rate(ablated(1)))
                 rounds["no_feed_no_lds_reads"].append(rate(ablated(2)))
+                rounds["loads_of_one_kib"].append(rate(ablated(3)))
             med = lambda v: round(sorted(v)[len(v) // 2], 1)
             ev = {"mfma_only_workload_operands_tflops": round(P.mfma_rate(sets[0][0]), 1),
                   "vendor_gemm_tflops": med(rounds["vendor_gemm"]),
@@ -406,7 +408,8 @@ def make_workload(key, torch, H, O, C):
                   "decomposition_tflops": {
                       "mfma_waits_barriers": med(rounds["no_feed_no_lds_reads"]),
                       "plus_lds_operand_reads": med(rounds["no_feed"]),
-                      "plus_global_to_lds_feed_and_epilogue": med(rounds["this_kernel"])}}
+                      "plus_load_issue_and_lds_writes": med(rounds["loads_of_one_kib"]),
+                      "plus_memory_system_behind_the_loads": med(rounds["this_kernel"])}}
             ones = torch.ones((8192, 8192), dtype=torch.bfloat16, device="cuda")
             ev["mfma_only_constant_operands_tflops"] = round(P.mfma_rate(ones), 1)
             launch = H.prepare(w.symbol, [ones.data_ptr(), ones.data_ptr(), sets[0][2].data_ptr(),
