@@ -28,13 +28,25 @@ constexpr int kThreads = 256;
 constexpr int kRowsInFlight = AFIR_GATHER_RIF;
 constexpr int kPassesPerBlock = AFIR_GATHER_PASSES;
 
-__device__ __forceinline__ u32x4 scale_shift(u32x4 t, const float *s, const float *h) {
+// t * s + h on eight halves, parameters kept as f16 pairs.  The product of two f16 values is
+// exact in float32 (11 x 11 significant bits), so the fused multiply-add rounds exactly where
+// the float32 multiply followed by the float32 add of the golden rounds: once, at the add.
+// Written this way each pair costs two v_fma_mix_f32 (f16 operands read in place) and one
+// v_cvt_pk_f16_f32 instead of six conversions, two multiplies, two adds and a pack; with the
+// row loads of 32768 rows in flight that arithmetic was 10 % of the kernel's time.
+__device__ __forceinline__ u32x4 scale_shift_packed(u32x4 t, u32x4 s, u32x4 h) {
+  typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
   u32x4 r;
 #pragma unroll
   for (int d = 0; d < 4; ++d) {
-    float lo = f16_lo(t[d]) * s[2 * d] + h[2 * d];
-    float hi = f16_hi(t[d]) * s[2 * d + 1] + h[2 * d + 1];
-    r[d] = pack_f16(lo, hi);
+    // (copies first: __builtin_bit_cast applied to a vector element reads element 0 with this compiler)
+    const uint32_t tw = t[d], sw = s[d], hw = h[d];
+    const half2_t tv = __builtin_bit_cast(half2_t, tw), sv = __builtin_bit_cast(half2_t, sw),
+                  hv = __builtin_bit_cast(half2_t, hw);
+    half2_t o;
+    o.x = (_Float16)__builtin_fmaf((float)tv.x, (float)sv.x, (float)hv.x);
+    o.y = (_Float16)__builtin_fmaf((float)tv.y, (float)sv.y, (float)hv.y);
+    r[d] = __builtin_bit_cast(uint32_t, o);
   }
   return r;
 }
@@ -61,14 +73,6 @@ __global__ __launch_bounds__(kThreads) void gather_scale_shift_f16_vec(
     for (int col = lane_col; col < chunks; col += lanes_per_row) {
       u32x4 sraw = *reinterpret_cast<const u32x4 *>(scale + (int64_t)col * 8);
       u32x4 hraw = *reinterpret_cast<const u32x4 *>(shift + (int64_t)col * 8);
-      float s[8], h[8];
-#pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        s[2 * d] = f16_lo(sraw[d]);
-        s[2 * d + 1] = f16_hi(sraw[d]);
-        h[2 * d] = f16_lo(hraw[d]);
-        h[2 * d + 1] = f16_hi(hraw[d]);
-      }
       for (int64_t r = r_begin + slot; r < r_end; r += (int64_t)rows_per_pass * kRowsInFlight) {
         // Branch-free fetch: rows past the end re-read the last row, indices
         // outside the table read row 0; both are discarded below.  All index
@@ -92,7 +96,7 @@ __global__ __launch_bounds__(kThreads) void gather_scale_shift_f16_vec(
         for (int u = 0; u < kRowsInFlight; ++u) {
           const int64_t rr = r + (int64_t)u * rows_per_pass;
           if (rr < r_end) {
-            u32x4 res = good[u] ? scale_shift(v[u], s, h) : nan_row;
+            u32x4 res = good[u] ? scale_shift_packed(v[u], sraw, hraw) : nan_row;
             store_nt(reinterpret_cast<u32x4 *>(out + rr * dim) + col, res);
             if (!good[u] && error_flag && col == 0) atomicOr(error_flag, 1);
           }
@@ -108,6 +112,19 @@ __global__ __launch_bounds__(kThreads) void gather_scale_shift_f16_vec(
 // lane has four loads in flight; 256 / lanes rows per workgroup pass.  The
 // lane's four scale / shift chunks stay in registers.
 constexpr int kGroups = 4;
+// Consecutive passes a workgroup takes, all their row loads in flight together (1, 2 and 4
+// measured 26.2 / 26.5 / 27.3 us on the 32768 x 1024 gather).
+// Workgroups per CU the grid is capped at (further rows are walked grid-strided).  Few, long-lived
+// workgroups (2 ... 16 per CU) with the next block's indices requested ahead measured 1-10 % slower
+// than one block of rows per workgroup on the 32768 x 1024 gather.
+#ifndef AFIR_GATHER_GROUPED_WG_PER_CU
+#define AFIR_GATHER_GROUPED_WG_PER_CU 64
+#endif
+#ifndef AFIR_GATHER_GROUPED_PASSES
+#define AFIR_GATHER_GROUPED_PASSES 1
+#endif
+constexpr int kGroupedPasses = AFIR_GATHER_GROUPED_PASSES;
+
 __global__ __launch_bounds__(kThreads) void gather_scale_shift_f16_grouped(
     const uint16_t *__restrict__ table, const int32_t *__restrict__ idx,
     const uint16_t *__restrict__ scale, const uint16_t *__restrict__ shift,
@@ -119,34 +136,57 @@ __global__ __launch_bounds__(kThreads) void gather_scale_shift_f16_grouped(
   const int col0 = threadIdx.x & (lanes - 1);
   const int64_t dim = (int64_t)lanes * kGroups * 8;
   const u32x4 nan_row = {0x7e007e00u, 0x7e007e00u, 0x7e007e00u, 0x7e007e00u};
-  float s[kGroups][8], h[kGroups][8];
+  // scale and shift: every row group of the workgroup needs the same lanes * kGroups chunks of
+  // each.  Loaded by the lanes of each row group separately that is 128 bytes per lane, twice
+  // what a lane gathers per pass; instead the workgroup fetches the two vectors once (one chunk
+  // of each per lane and round), parks them in LDS and every lane picks its chunks up from
+  // there.  The fetch goes out behind the first block's row loads, so it costs no latency.
+  extern __shared__ u32x4 params[];            // scale chunks, then shift chunks
+  const int nchunks = lanes * kGroups;          // chunks per row
+  u32x4 sraw[kGroups], hraw[kGroups];
+  bool staged = false;
+  const int64_t rows_per_block = (int64_t)rows_per_pass * kGroupedPasses;
+  for (int64_t r0 = (int64_t)blockIdx.x * rows_per_block; r0 < nidx; r0 += (int64_t)gridDim.x * rows_per_block) {
+    // all indices of the block's passes, then all their row loads, then the stores: rows past
+    // the end re-read the last row and indices outside the table read row 0, both dropped below
+    uint32_t src[kGroupedPasses];
+    bool good[kGroupedPasses];
+    u32x4 v[kGroupedPasses][kGroups];
 #pragma unroll
-  for (int u = 0; u < kGroups; ++u) {
-    const int col = col0 + u * lanes;
-    const u32x4 sraw = *reinterpret_cast<const u32x4 *>(scale + (int64_t)col * 8);
-    const u32x4 hraw = *reinterpret_cast<const u32x4 *>(shift + (int64_t)col * 8);
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-      s[u][2 * d] = f16_lo(sraw[d]);
-      s[u][2 * d + 1] = f16_hi(sraw[d]);
-      h[u][2 * d] = f16_lo(hraw[d]);
-      h[u][2 * d + 1] = f16_hi(hraw[d]);
+    for (int p = 0; p < kGroupedPasses; ++p) {
+      const int64_t r = r0 + (int64_t)p * rows_per_pass + local_row;
+      src[p] = (uint32_t)idx[r < nidx ? r : nidx - 1];
     }
-  }
-  for (int64_t r0 = (int64_t)blockIdx.x * rows_per_pass; r0 < nidx; r0 += (int64_t)gridDim.x * rows_per_pass) {
-    const int64_t r = r0 + local_row;
-    if (r >= nidx) continue;
-    const uint32_t src = (uint32_t)idx[r];
-    const bool good = src < rows;
-    const u32x4 *row = reinterpret_cast<const u32x4 *>(table + (int64_t)(good ? src : 0u) * dim);
-    u32x4 v[kGroups];
 #pragma unroll
-    for (int u = 0; u < kGroups; ++u) v[u] = row[col0 + u * lanes];
-    u32x4 *dst = reinterpret_cast<u32x4 *>(out + r * dim);
+    for (int p = 0; p < kGroupedPasses; ++p) {
+      good[p] = src[p] < rows;
+      const u32x4 *row = reinterpret_cast<const u32x4 *>(table + (int64_t)(good[p] ? src[p] : 0u) * dim);
 #pragma unroll
-    for (int u = 0; u < kGroups; ++u)
-      store_nt(dst + col0 + u * lanes, good ? scale_shift(v[u], s[u], h[u]) : nan_row);
-    if (!good && error_flag && col0 == 0) atomicOr(error_flag, 1);
+      for (int u = 0; u < kGroups; ++u) v[p][u] = row[col0 + u * lanes];
+    }
+    if (!staged) {   // (the trip count is the same for every lane of the workgroup)
+      for (int c = threadIdx.x; c < nchunks; c += kThreads) {
+        params[c] = *reinterpret_cast<const u32x4 *>(scale + (int64_t)c * 8);
+        params[nchunks + c] = *reinterpret_cast<const u32x4 *>(shift + (int64_t)c * 8);
+      }
+      __syncthreads();
+#pragma unroll
+      for (int u = 0; u < kGroups; ++u) {
+        sraw[u] = params[col0 + u * lanes];
+        hraw[u] = params[nchunks + col0 + u * lanes];
+      }
+      staged = true;
+    }
+#pragma unroll
+    for (int p = 0; p < kGroupedPasses; ++p) {
+      const int64_t r = r0 + (int64_t)p * rows_per_pass + local_row;
+      if (r >= nidx) continue;
+      u32x4 *dst = reinterpret_cast<u32x4 *>(out + r * dim);
+#pragma unroll
+      for (int u = 0; u < kGroups; ++u)
+        store_nt(dst + col0 + u * lanes, good[p] ? scale_shift_packed(v[p][u], sraw[u], hraw[u]) : nan_row);
+      if (!good[p] && error_flag && col0 == 0) atomicOr(error_flag, 1);
+    }
   }
 }
 
@@ -198,11 +238,12 @@ LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx
   int lanes_log2 = 0;
   while (lanes_log2 < 8 && ((int64_t)kGroups << lanes_log2) < chunks64) ++lanes_log2;
   if (vec && ((int64_t)kGroups << lanes_log2) == chunks64) {
-    const int rows_per_pass = kThreads >> lanes_log2;
-    int64_t blocks = (nidx + rows_per_pass - 1) / rows_per_pass;
-    if (blocks > (int64_t)device_cus() * 64) blocks = (int64_t)device_cus() * 64;
+    const int64_t rows_per_block = (int64_t)(kThreads >> lanes_log2) * kGroupedPasses;
+    int64_t blocks = (nidx + rows_per_block - 1) / rows_per_block;
+    if (blocks > (int64_t)device_cus() * AFIR_GATHER_GROUPED_WG_PER_CU) blocks = (int64_t)device_cus() * AFIR_GATHER_GROUPED_WG_PER_CU;
     if (block_dim) blocks = block_dim;
-    hipLaunchKernelGGL(gather_scale_shift_f16_grouped, dim3((unsigned)blocks), dim3(kThreads), 0,
+    const size_t lds = (size_t)2 * (kGroups << lanes_log2) * 16;   // scale and shift, 16-byte chunks
+    hipLaunchKernelGGL(gather_scale_shift_f16_grouped, dim3((unsigned)blocks), dim3(kThreads), lds,
                        stream, table, idx, scale, shift, out, error_flag, (uint32_t)rows, lanes_log2,
                        nidx);
   } else if (vec) {

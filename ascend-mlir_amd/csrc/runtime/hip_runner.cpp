@@ -234,32 +234,61 @@ class HipExecutionRunner final : public ExecutionRunner {
     // ---- launch ----
     const uint32_t bd = (uint32_t)(args.block_dim < 0 ? 0 : args.block_dim);
     double bestUs = -1.0;
-    for (int rep = 0; rep <= (args.timing_repeats > 0 ? args.timing_repeats : 0); ++rep) {
-    void **use = sets[rep % nsets].data();
-    (void)hipEventRecord(ev0_, stream_);
-    uint32_t rc;
-    if (regionLaunch) {
-      const int nargs = (int)(args.inputs.size() + args.outputs.size());
-      rc = regionLaunch(region, bd, stream_, nargs, use, workspace, args.tiling.data(),
-                        args.tiling.size());
-    } else {
-      rc = launchFn(bd, stream_, use[0], use[1], use[2], use[3], use[4], use[5],
-                    use[6], use[7], use[8], use[9], use[10], use[11], use[12],
-                    use[13], use[14], use[15]);
-    }
-    if (rc != 0) {
+    auto launchOnce = [&](void **use) -> uint32_t {
+      if (regionLaunch) {
+        const int nargs = (int)(args.inputs.size() + args.outputs.size());
+        return regionLaunch(region, bd, stream_, nargs, use, workspace, args.tiling.data(), args.tiling.size());
+      }
+      return launchFn(bd, stream_, use[0], use[1], use[2], use[3], use[4], use[5], use[6], use[7], use[8],
+                      use[9], use[10], use[11], use[12], use[13], use[14], use[15]);
+    };
+    auto launchFailed = [&](uint32_t rc) {
       std::string why = lastError ? lastError() : "";
       (void)hipStreamSynchronize(stream_);
       cleanup();
       return Status::error(format("dynamic library artifact launch failed: rc=%u", rc) +
                            (why.empty() ? "" : " (" + why + ")"));
+    };
+    const int repeats = args.timing_repeats > 0 ? args.timing_repeats : 0;
+    const bool continuous = repeats > 0 && args.ramp_ms > 0;
+    // the first launch (the only one without timing_repeats), and every launch when the timed
+    // launches are separated by synchronisations
+    for (int rep = 0; rep <= (continuous ? 0 : repeats); ++rep) {
+      void **use = sets[rep % nsets].data();
+      (void)hipEventRecord(ev0_, stream_);
+      const uint32_t rc = launchOnce(use);
+      if (rc != 0) return launchFailed(rc);
+      (void)hipEventRecord(ev1_, stream_);
+      hipError_t e = hipStreamSynchronize(stream_);
+      if (e != hipSuccess) { cleanup(); return Status::error(hipErr("hipStreamSynchronize", e)); }
+      float ms = 0.f;
+      if (hipEventElapsedTime(&ms, ev0_, ev1_) == hipSuccess && (bestUs < 0 || (double)ms * 1e3 < bestUs))
+        bestUs = (double)ms * 1e3;
     }
-    (void)hipEventRecord(ev1_, stream_);
-    hipError_t e = hipStreamSynchronize(stream_);
-    if (e != hipSuccess) { cleanup(); return Status::error(hipErr("hipStreamSynchronize", e)); }
-    float ms = 0.f;
-    if (hipEventElapsedTime(&ms, ev0_, ev1_) == hipSuccess && (bestUs < 0 || (double)ms * 1e3 < bestUs))
-      bestUs = (double)ms * 1e3;
+    if (continuous) {
+      int next = 1;
+      const auto until = std::chrono::steady_clock::now() + std::chrono::duration<double, std::milli>(args.ramp_ms);
+      while (std::chrono::steady_clock::now() < until) {
+        for (int i = 0; i < 16; ++i) {
+          const uint32_t rc = launchOnce(sets[next++ % nsets].data());
+          if (rc != 0) return launchFailed(rc);
+        }
+        (void)hipStreamSynchronize(stream_);
+      }
+      // the timed launches: one pair of events around all of them, the score is their average
+      // (an event between every two launches costs about 2 us of idle device per launch)
+      uint32_t rc = 0;
+      (void)hipEventRecord(ev0_, stream_);
+      for (int rep = 0; rep < repeats && rc == 0; ++rep) rc = launchOnce(sets[next++ % nsets].data());
+      (void)hipEventRecord(ev1_, stream_);
+      hipError_t e = hipStreamSynchronize(stream_);
+      const bool ok = true;
+      if (rc == 0 && e == hipSuccess) {
+        float ms = 0.f;
+        if (hipEventElapsedTime(&ms, ev0_, ev1_) == hipSuccess) bestUs = (double)ms * 1e3 / repeats;
+      }
+      if (rc != 0) return launchFailed(rc);
+      if (!ok || e != hipSuccess) { cleanup(); return Status::error(hipErr("timed launches", ok ? e : hipErrorOutOfMemory)); }
     }
     lastKernelUs_ = bestUs;
 

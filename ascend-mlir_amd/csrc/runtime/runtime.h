@@ -102,6 +102,12 @@ struct RunArgs {
   // no launch finds its inputs in the last-level cache (256 MB on MI355X) because the launch
   // before it left them there.  The outputs handed back are those of the first copy.
   int buffer_sets = 1;
+  // > 0 (with timing_repeats): before the timed launches the kernel is launched back to back for
+  // this many milliseconds, and the timed launches then follow each other without a host
+  // synchronisation in between; the reported time is their average.  The device needs 50-100 ms of
+  // continuous work to settle at its sustained clocks; launches separated by synchronisations
+  // never get there and read 3-10 % slow.
+  double ramp_ms = 0.0;
 };
 
 // ------------------------------------------------------------------- npy ----

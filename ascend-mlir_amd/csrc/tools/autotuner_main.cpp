@@ -10,7 +10,7 @@
 //   autotuner --space tiling_space.json (--kernel K.mlir | --artifact-root DIR)
 //             --inputs a.npy,b.npy --expected e.npy --shape M=32,N=32
 //             [--output best_config.json] [--kernel-kind vec|cube|mix] [--soc S]
-//             [--atol A] [--rtol R] [--repeats N] [--buffer-sets N] [--device N]
+//             [--atol A] [--rtol R] [--repeats N] [--buffer-sets N] [--ramp-ms MS] [--device N]
 //
 // tiling_space.json: {"kernel", "kernel_file", "soc", "block_dim_expr",
 //   "block_dim_values": [..] (this backend: explicit grid sizes to try, 0 =
@@ -288,6 +288,9 @@ int main(int argc, char **argv) {
   // --buffer-sets N: the timed launches of a candidate rotate over N copies of its tensors on the
   // device, so that repeated launches are not served from the last-level cache
   const int bufferSets = opt.count("buffer-sets") ? std::max(1, std::atoi(opt["buffer-sets"].c_str())) : 1;
+  // --ramp-ms MS: each candidate is launched back to back for MS milliseconds before its timed
+  // launches, which then run without synchronisations in between (the device's sustained clocks)
+  const double rampMs = opt.count("ramp-ms") ? std::max(0.0, std::atof(opt["ramp-ms"].c_str())) : 0.0;
 
   DynamicLibraryExecutionLaunch launch;
   launch.sharedLibraryPath = artifact.sharedLibraryPath;
@@ -420,6 +423,7 @@ int main(int argc, char **argv) {
       double bestNs = -1;
       args.timing_repeats = repeats - 1;
       args.buffer_sets = bufferSets;
+      args.ramp_ms = rampMs;
       Status st = runner->runDynamicLibraryArtifact(launch, args);
       const double us = runner->lastKernelMicroseconds();
       if (st.ok() && us >= 0) bestNs = us * 1e3;

@@ -20,6 +20,9 @@ import sys
 import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
+# copies of the tensors the timed launches rotate over: at least 1 GiB of inputs read between two
+# launches on the same copy, so that the 256 MB last-level cache serves none of the reads
+BUFFER_SETS = {"eltwise": 8, "rowsum": 8, "transpose-family": 16, "gather": 16, "matmul": 2}
 
 
 def bf16_bits(x):
@@ -81,7 +84,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("family", choices=["eltwise", "rowsum", "transpose-family", "gather", "matmul"])
     ap.add_argument("--out", default=None)
-    ap.add_argument("--repeats", default="20")
+    ap.add_argument("--repeats", default="200")
     args = ap.parse_args()
     out = args.out or f"/tmp/autotune-{args.family}"
     os.makedirs(out, exist_ok=True)
@@ -91,7 +94,8 @@ def main():
            "--kernel", os.path.join(here, "kernel.region"),
            "--inputs", ",".join(os.path.join(out, n + ".npy") for n in inputs),
            "--expected", os.path.join(out, "expected.npy"), "--atol", atol, "--rtol", rtol,
-           "--repeats", args.repeats, "--buffer-sets", "4", "--build-dir", os.path.join(out, "artifacts"),
+           "--repeats", args.repeats, "--buffer-sets", str(BUFFER_SETS[args.family]), "--ramp-ms", "100",
+           "--build-dir", os.path.join(out, "artifacts"),
            "--shape", "S=1", "--output", os.path.join(out, "best_config.json")]
     print("+", " ".join(cmd), flush=True)
     sys.exit(subprocess.run(cmd).returncode)

@@ -6,8 +6,10 @@
 
 A step is one launch of the workload's fused kernel over one batch of seeded
 synthetic input already resident in HBM.  Buffer sets are rotated between
-steps so that the working set (several hundred MB) cannot be served from the
-256 MB last-level cache.  Prints ONE JSON line.
+steps: every HBM-bound workload cycles over at least 1 GiB of inputs, so that
+none of its reads can be served from the 256 MB last-level cache (see
+MIN_CYCLIC_READ_BYTES).  Before the W warmup steps the workload is launched
+untimed for --ramp-ms (the device's sustained clocks).  Prints ONE JSON line.
 
   value            algorithmic GB/s (TFLOP/s for c5) over the K timed steps,
                    wall clock between two device synchronisations
@@ -156,6 +158,19 @@ def load_package():
     return mod
 
 
+# The last-level cache (256 MB "Infinity Cache", memory side) serves reads of anything that was
+# read within the previous 256 MB of reads; writes pass through it.  A plain copy measures
+# 6.7 TB/s while the launches cycle over <= 256 MiB of sources and 5.67 TB/s from 512 MiB on
+# (the same kernel, the same launch sizes).  Every HBM-bound workload therefore cycles over
+# enough copies of its inputs that the bytes it reads come back only after at least this many
+# other bytes have been read: what is timed is HBM, not that cache.
+MIN_CYCLIC_READ_BYTES = 1 << 30
+
+
+def sets_for(read_bytes_per_launch):
+    return max(2, -(-MIN_CYCLIC_READ_BYTES // int(read_bytes_per_launch)))
+
+
 class Workload:
     """One configuration: seeded inputs, launch closures over `nsets` buffer
     sets, algorithmic work, parity check and CPU baseline."""
@@ -188,7 +203,7 @@ def make_workload(key, torch, H, O, C):
         w.title = "c1 fused add->mul out=(a+b)*b f32 [4096,4096]"
         w.dtype, w.symbol = "f32", "afir_hip_launch_fused_add_mul"
         w.work = lambda: O.algorithmic_bytes("c1", m=4096, n=4096)
-        w.nsets = 3
+        w.nsets = sets_for(a.nbytes + b.nbytes)
         sets = []
         da, db = _dev(torch, a), _dev(torch, b)
         for i in range(w.nsets):
@@ -220,7 +235,7 @@ def make_workload(key, torch, H, O, C):
         w.title = "c2 broadcast-add-reduce y=rowsum(x+bias) f32 [8192,4096]+[4096]->[8192]"
         w.dtype, w.symbol = "f32", "afir_hip_launch_broadcast_add_reducesum"
         w.work = lambda: O.algorithmic_bytes("c2", m=8192, n=4096)
-        w.nsets = 4
+        w.nsets = sets_for(x.nbytes)
         dx, dbias = _dev(torch, x), _dev(torch, bias)
         sets = []
         for i in range(w.nsets):
@@ -256,7 +271,7 @@ def make_workload(key, torch, H, O, C):
         w.title = "c3 relu-broadcast-transpose out=transpose(relu(x)+c) f16 [64,1024,512]->[64,512,1024]"
         w.dtype, w.symbol = "f16", "afir_hip_launch_relu_broadcast_add_transpose"
         w.work = lambda: O.algorithmic_bytes("c3", b=64, m=1024, n=512)
-        w.nsets = 4
+        w.nsets = sets_for(x.nbytes)
         dx, dc = _dev(torch, x), _dev(torch, c)
         sets = []
         for i in range(w.nsets):
@@ -289,15 +304,16 @@ def make_workload(key, torch, H, O, C):
                    "int32 idx [32768]")
         w.dtype, w.symbol = "f16", "afir_hip_launch_gather_scale_shift"
         w.work = lambda: O.algorithmic_bytes("c4", nidx=32768, dim=1024)
-        w.nsets = 3
+        # a launch reads 64 MiB of gathered rows: a seeded index vector of its own per set, the sets
+        # dealt over four tables (1 GiB), so that a row comes up again only after 1 GiB of other rows
+        w.nsets = sets_for(32768 * 1024 * 2)
         dt_, dsc, dsh = _dev(torch, table), _dev(torch, scale), _dev(torch, shift)
+        tables = [dt_] + [dt_.clone() for _ in range(3)]
         rng = np.random.default_rng(7)
         sets = []
         for i in range(w.nsets):
-            # a table (256 MiB) and a seeded index vector of its own per set: no
-            # row a launch gathers was touched by the launch before it
             ii = idx if i == 0 else rng.integers(0, 131072, 32768, dtype=np.int64).astype(np.int32)
-            sets.append((dt_ if i == 0 else dt_.clone(), _dev(torch, ii), dsc, dsh,
+            sets.append((tables[i % 4], _dev(torch, ii), dsc, dsh,
                          torch.empty((32768, 1024), dtype=torch.float16, device="cuda")))
         w.sets = sets
         w.launches = [H.prepare(w.symbol, [s[0].data_ptr(), s[1].data_ptr(), s[2].data_ptr(),
@@ -470,17 +486,19 @@ def make_workload(key, torch, H, O, C):
             region.compile()     # from lib/region_cache when build() left it there
             assert region.kernel == "fused_region_compiled"
         w.work = lambda: work
-        w.nsets = 3 if key[1] in "14" else 4
+        w.nsets = sets_for(32768 * 1024 * 2 if key[1] == "4" else
+                           inputs[0].nbytes + (inputs[1].nbytes if key[1] == "1" else 0))
         dev0 = [_dev(torch, x) for x in inputs]
+        tables = [dev0[0]] + ([dev0[0].clone() for _ in range(3)] if key[1] == "4" else [])
         sets = []
         idx_rng = np.random.default_rng(7)
         for i in range(w.nsets):
             if i == 0:
                 ins = dev0
             elif key[1] == "4":
-                # a table (256 MiB) of its own per set, and other rows
+                # other rows for every set, the sets dealt over four tables (as in c4)
                 other = idx_rng.integers(0, 131072, 32768, dtype=np.int64).astype(np.int32)
-                ins = [dev0[0].clone(), _dev(torch, other)] + dev0[2:]
+                ins = [tables[i % 4], _dev(torch, other)] + dev0[2:]
             else:
                 ins = [dev0[0].clone()] + ([dev0[1].clone()] if key[1] == "1" else dev0[1:])
             sets.append((ins, torch.empty(out_shape, dtype=out_dt, device="cuda")))
@@ -520,7 +538,7 @@ def make_workload(key, torch, H, O, C):
         # measure the host's launch rate)
         nbytes = (128 << 20) if key == "ceil_read" else (64 << 20)
         w.dtype = "u8"
-        w.nsets = 4
+        w.nsets = sets_for(nbytes)
         w.no_cpu = True
         srcs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device="cuda") for _ in range(w.nsets)]
         if key == "ceil_copy":
@@ -559,8 +577,19 @@ def make_workload(key, torch, H, O, C):
     return w
 
 
-def run_workload(w, torch, steps, warmup):
+def run_workload(w, torch, steps, warmup, ramp_ms=0.0):
     n = len(w.launches)
+    # The device takes some 50-100 ms of continuous work to settle at its sustained clocks (the
+    # first launches after an idle period run 3-8 % slower): launches of the same workload,
+    # untimed, until ramp_ms have passed; then the W warmup steps, then the K timed ones.
+    if ramp_ms > 0:
+        t_end = time.perf_counter() + ramp_ms * 1e-3
+        i = 0
+        while time.perf_counter() < t_end:
+            for _ in range(16):
+                w.launches[i % n]()
+                i += 1
+            torch.cuda.synchronize()
     for i in range(warmup):
         w.launches[i % n]()
     torch.cuda.synchronize()
@@ -599,6 +628,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None)
     ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--ramp-ms", type=float, default=100.0,
+                    help="untimed launches of the workload for this long before the warmup steps, so that "
+                         "the device is at its sustained clocks when the timed region starts (0: none)")
     ap.add_argument("--workload", default="c2", choices=ALL_WORKLOADS)
     ap.add_argument("--all", dest="all", action="store_true", default=True)
     ap.add_argument("--no-all", dest="all", action="store_false")
@@ -639,7 +671,7 @@ def main():
     for key in order:
         w = make_workload(key, torch, H, O, C)
         steps, warmup = steps_for(key), warm_for(key)
-        wall, ev_ms = run_workload(w, torch, steps, warmup)
+        wall, ev_ms = run_workload(w, torch, steps, warmup, args.ramp_ms)
         value, unit, roof = summarize(w, wall, ev_ms, steps)
         par = w.parity()
         extra = (w.power_evidence() if hasattr(w, "power_evidence") and not args.no_power_evidence
@@ -679,7 +711,7 @@ def main():
         "ms_per_step": main_e["ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": main_e["dtype"], "data": "synthetic",
         "config": {"workload": main_e["workload"], "seed": 42,
-                   "buffer_sets": main_e["buffer_sets"]},
+                   "buffer_sets": main_e["buffer_sets"], "ramp_ms": args.ramp_ms},
         "roofline": {k: main_e["roofline"][k] for k in
                      ("bound", "achieved", "peak", "unit", "frac", "traffic")},
         "parity": main_e["parity"],
