@@ -120,18 +120,27 @@ constexpr int kGroups = 4;
 #ifndef AFIR_GATHER_GROUPED_WG_PER_CU
 #define AFIR_GATHER_GROUPED_WG_PER_CU 64
 #endif
+#ifndef AFIR_GATHER_NT_LOADS
+#define AFIR_GATHER_NT_LOADS 0
+#endif
 #ifndef AFIR_GATHER_GROUPED_PASSES
-#define AFIR_GATHER_GROUPED_PASSES 1
+#define AFIR_GATHER_GROUPED_PASSES 2
 #endif
 constexpr int kGroupedPasses = AFIR_GATHER_GROUPED_PASSES;
+// lanes of a workgroup of the grouped kernel: with more row groups per workgroup the scale / shift
+// vectors are fetched for more rows at once
+#ifndef AFIR_GATHER_GROUPED_THREADS
+#define AFIR_GATHER_GROUPED_THREADS 1024
+#endif
+constexpr int kGroupedThreads = AFIR_GATHER_GROUPED_THREADS;
 
-__global__ __launch_bounds__(kThreads) void gather_scale_shift_f16_grouped(
+__global__ __launch_bounds__(kGroupedThreads) void gather_scale_shift_f16_grouped(
     const uint16_t *__restrict__ table, const int32_t *__restrict__ idx,
     const uint16_t *__restrict__ scale, const uint16_t *__restrict__ shift,
     uint16_t *__restrict__ out, int32_t *__restrict__ error_flag, uint32_t rows, int lanes_log2,
     int64_t nidx) {
   const int lanes = 1 << lanes_log2;
-  const int rows_per_pass = kThreads >> lanes_log2;
+  const int rows_per_pass = kGroupedThreads >> lanes_log2;
   const int local_row = threadIdx.x >> lanes_log2;
   const int col0 = threadIdx.x & (lanes - 1);
   const int64_t dim = (int64_t)lanes * kGroups * 8;
@@ -162,10 +171,11 @@ __global__ __launch_bounds__(kThreads) void gather_scale_shift_f16_grouped(
       good[p] = src[p] < rows;
       const u32x4 *row = reinterpret_cast<const u32x4 *>(table + (int64_t)(good[p] ? src[p] : 0u) * dim);
 #pragma unroll
-      for (int u = 0; u < kGroups; ++u) v[p][u] = row[col0 + u * lanes];
+      for (int u = 0; u < kGroups; ++u)
+        v[p][u] = AFIR_GATHER_NT_LOADS ? __builtin_nontemporal_load(row + col0 + u * lanes) : row[col0 + u * lanes];
     }
     if (!staged) {   // (the trip count is the same for every lane of the workgroup)
-      for (int c = threadIdx.x; c < nchunks; c += kThreads) {
+      for (int c = threadIdx.x; c < nchunks; c += kGroupedThreads) {
         params[c] = *reinterpret_cast<const u32x4 *>(scale + (int64_t)c * 8);
         params[nchunks + c] = *reinterpret_cast<const u32x4 *>(shift + (int64_t)c * 8);
       }
@@ -238,12 +248,12 @@ LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx
   int lanes_log2 = 0;
   while (lanes_log2 < 8 && ((int64_t)kGroups << lanes_log2) < chunks64) ++lanes_log2;
   if (vec && ((int64_t)kGroups << lanes_log2) == chunks64) {
-    const int64_t rows_per_block = (int64_t)(kThreads >> lanes_log2) * kGroupedPasses;
+    const int64_t rows_per_block = (int64_t)(kGroupedThreads >> lanes_log2) * kGroupedPasses;
     int64_t blocks = (nidx + rows_per_block - 1) / rows_per_block;
     if (blocks > (int64_t)device_cus() * AFIR_GATHER_GROUPED_WG_PER_CU) blocks = (int64_t)device_cus() * AFIR_GATHER_GROUPED_WG_PER_CU;
     if (block_dim) blocks = block_dim;
     const size_t lds = (size_t)2 * (kGroups << lanes_log2) * 16;   // scale and shift, 16-byte chunks
-    hipLaunchKernelGGL(gather_scale_shift_f16_grouped, dim3((unsigned)blocks), dim3(kThreads), lds,
+    hipLaunchKernelGGL(gather_scale_shift_f16_grouped, dim3((unsigned)blocks), dim3(kGroupedThreads), lds,
                        stream, table, idx, scale, shift, out, error_flag, (uint32_t)rows, lanes_log2,
                        nidx);
   } else if (vec) {
