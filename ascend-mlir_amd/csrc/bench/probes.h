@@ -47,10 +47,10 @@ uint32_t afir_bench_mfma_rate(void *stream, const void *operands, void *sink, ui
 uint32_t afir_bench_matmul_ablated(void *stream, const void *a, const void *b, const void *bias,
                                    void *out, int m, int k, int n, int what);
 
-/* Grid-strided copy, 128-bit ordinary loads and non-temporal stores (the
- * fastest of the four combinations for a stream that writes as much as it
- * reads: 6.7 TB/s against 6.0 with the hint on both sides), four in flight per
- * lane; bytes must be a multiple of 16384. */
+/* Grid-strided copy, 128-bit non-temporal loads and stores, four in flight per
+ * lane: the fastest of the load / store policy pairs for a stream that comes
+ * from HBM and writes as much as it reads (5.90 TB/s; ordinary loads 5.76,
+ * ordinary stores 5.5-5.7).  bytes must be a multiple of 16384. */
 uint32_t afir_bench_copy(void *stream, const void *src, void *dst, size_t bytes);
 
 /* Read-only stream: every lane sums what it loads (128-bit non-temporal loads)

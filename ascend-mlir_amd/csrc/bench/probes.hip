@@ -82,7 +82,7 @@ __global__ __launch_bounds__(kCopyThreads) void probe_copy(const u32x4 *__restri
   for (size_t base = (size_t)blockIdx.x * chunk; base < n16; base += stride) {
     u32x4 v[kCopyUnroll];
 #pragma unroll
-    for (int u = 0; u < kCopyUnroll; ++u) v[u] = src[base + u * kCopyThreads + threadIdx.x];
+    for (int u = 0; u < kCopyUnroll; ++u) v[u] = afir::load_nt(src + base + u * kCopyThreads + threadIdx.x);
 #pragma unroll
     for (int u = 0; u < kCopyUnroll; ++u) afir::store_nt(dst + base + u * kCopyThreads + threadIdx.x, v[u]);
   }

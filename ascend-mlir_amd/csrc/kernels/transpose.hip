@@ -31,12 +31,14 @@ __device__ __forceinline__ float relu_keep_nan(float v) { return (v > 0.f) ? v :
 // numbered along M first, so neighbouring workgroups write neighbouring runs
 // of the same output rows.
 //
-// The loads are ordinary loads, the stores non-temporal.  This kernel moves
-// as many bytes out as in, and for such streams the non-temporal hint on the
-// LOADS costs bandwidth on MI355X: a plain 64 MiB copy measured 6.0 TB/s with
-// the hint on both sides and 6.7 with ordinary loads, this kernel 5.5 and 6.5
-// (kernels that read two or more bytes per byte written measured the other
-// way round and keep the hint on their loads).
+// The loads are ordinary loads, the stores non-temporal (AFIR_TRANSPOSE_NT_LOADS, searched):
+// with inputs that come from HBM the hint on the loads makes no difference here (23.7 against
+// 23.9 us), and when a caller's inputs were read recently enough to sit in the 256 MB
+// last-level cache, ordinary loads find them there (5.5 against 6.5 TB/s when the launches
+// cycle over 256 MiB of inputs).
+#ifndef AFIR_TRANSPOSE_NT_LOADS
+#define AFIR_TRANSPOSE_NT_LOADS 0
+#endif
 #ifndef AFIR_TRANSPOSE_TILES_PER_WG
 #define AFIR_TRANSPOSE_TILES_PER_WG 1
 #endif
@@ -67,7 +69,8 @@ __global__ __launch_bounds__(kThreads) void relu_bcast_add_transpose_f16_tile64(
   {
     const uint16_t *xin = x + ((int64_t)b * m + m0 + li) * n + n0 + lj;
 #pragma unroll
-    for (int k = 0; k < 2; ++k) v[k] = *reinterpret_cast<const u32x4 *>(xin + (int64_t)(32 * k) * n);
+    for (int k = 0; k < 2; ++k) v[k] = AFIR_TRANSPOSE_NT_LOADS ? load_nt(reinterpret_cast<const u32x4 *>(xin + (int64_t)(32 * k) * n))
+                                      : *reinterpret_cast<const u32x4 *>(xin + (int64_t)(32 * k) * n);
   }
   int parity = 0;
   for (;;) {
@@ -89,7 +92,8 @@ __global__ __launch_bounds__(kThreads) void relu_bcast_add_transpose_f16_tile64(
       craw = *reinterpret_cast<const u32x4 *>(c + next_n0 + lj);
       const uint16_t *xin = x + ((int64_t)next_b * m + next_m0 + li) * n + next_n0 + lj;
 #pragma unroll
-      for (int k = 0; k < 2; ++k) v[k] = *reinterpret_cast<const u32x4 *>(xin + (int64_t)(32 * k) * n);
+      for (int k = 0; k < 2; ++k) v[k] = AFIR_TRANSPOSE_NT_LOADS ? load_nt(reinterpret_cast<const u32x4 *>(xin + (int64_t)(32 * k) * n))
+                                      : *reinterpret_cast<const u32x4 *>(xin + (int64_t)(32 * k) * n);
     }
     // one barrier per tile: the other LDS tile was last read two barriers ago
     __syncthreads();

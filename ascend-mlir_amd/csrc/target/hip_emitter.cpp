@@ -417,11 +417,12 @@ class SegmentEmitter {
           o.tileSlot = tiles++;
         }
     numTiles_ = tiles;
-    // Non-temporal loads pay when reads dominate the traffic.  A segment that writes about as many
-    // bytes as it streams in (one full-size input per output) measured faster on MI355X with
-    // ordinary loads next to its non-temporal stores: a plain copy 6.0 -> 6.7 TB/s, the tiled
-    // transpose 5.5 -> 6.5.  Two full-size inputs per output measured 7 % slower that way
-    // (6.25 -> 5.8) and a row sum, which writes next to nothing, 3 % slower; those keep the hint.
+    // Non-temporal loads pay when reads dominate the traffic (two full-size inputs per output:
+    // 6.25 against 5.8 TB/s; a row sum 3 %).  A segment that writes about as many bytes as it
+    // streams in (one full-size input per output) keeps ordinary loads next to its non-temporal
+    // stores: from HBM the two measure within 2 % of each other, and inputs that a previous launch
+    // left in the 256 MB last-level cache are found there only by ordinary loads (a copy cycling
+    // over 256 MiB: 6.7 against 6.0 TB/s, the tiled transpose 6.5 against 5.5).
     if (!reduce_) {
       size_t streamed = 0;
       for (const Operand &o : operands_)

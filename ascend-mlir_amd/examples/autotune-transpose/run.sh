@@ -25,4 +25,4 @@ np.save(out + "/expected.npy", np.ascontiguousarray(e.transpose(0, 2, 1)))
 PY
 "$HERE/../../bin/autotuner" --space "$HERE/tiling_space.json" --kernel "$HERE/kernel.region" \
   --inputs "$OUT/x.npy,$OUT/c.npy" --expected "$OUT/expected.npy" --shape B=64 --atol 0 --rtol 0 \
-  --repeats 20 --build-dir "$OUT/artifacts" --output "$OUT/best_config.json"
+  --repeats 200 --buffer-sets 16 --ramp-ms 100 --build-dir "$OUT/artifacts" --output "$OUT/best_config.json"

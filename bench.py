@@ -542,7 +542,7 @@ def make_workload(key, torch, H, O, C):
         w.no_cpu = True
         srcs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device="cuda") for _ in range(w.nsets)]
         if key == "ceil_copy":
-            w.title = "ceil_copy: 64 MiB -> 64 MiB, 128-bit loads, non-temporal stores (probe, no arithmetic)"
+            w.title = "ceil_copy: 64 MiB -> 64 MiB, 128-bit non-temporal loads and stores (probe, no arithmetic)"
             dsts = [torch.empty_like(x) for x in srcs]
             w.work = lambda: 2 * nbytes
             w.launches = [P.prepare("afir_bench_copy", a.data_ptr(), b.data_ptr(), nbytes) for a, b in zip(srcs, dsts)]
