@@ -43,6 +43,7 @@ KERNEL_SOURCES = [
     ("kernels/gather.hip", STRICT),
     ("kernels/matmul.hip", []),
     ("kernels/matmul_dma.hip", []),
+    ("kernels/matmul_layouts.hip", []),
     ("kernels/region.hip", STRICT),
     ("target/region_program.cpp", []),
     ("target/hip_emitter.cpp", []),

@@ -217,7 +217,9 @@ std::string detect_fast_path(RegisteredRegion *r) {
     size_t at = 1;
     int bias = -1;
     float alpha = 1.f;   // max(v, v * 1) is v
-    if (at + 1 < ops.size() && is_push(ops[at], 2, {1}) && ops[at + 1].code == OpCode::Add) {
+    // (the bias runs along the last iteration dim: d1, or d2 of a batched product)
+    if (at + 1 < ops.size() && (g.rank == 3 ? is_push(ops[at], 3, {2}) : is_push(ops[at], 2, {1})) &&
+        ops[at + 1].code == OpCode::Add) {
       bias = ops[at].arg;
       at += 2;
     }
@@ -345,9 +347,10 @@ bool fast_path_fits(const RegisteredRegion &r, const afir_region::Resolved &res)
       return true;
     case FastPath::MatmulBiasLeaky:
     case FastPath::MatmulBiasLeakyF16:
-      // resolve() has matched A [M,K], B [K,N] against the segment; the bias is read from element 0
+      // resolve() has matched A and B (transposed, batched or not) against the segment; the bias is
+      // read from element 0 along the last iteration dim
       for (const afir_region::ResolvedInput &in : seg.inputs)
-        if (!dense(in, {0, 1})) return false;
+        if (!(seg.rank == 3 ? dense(in, {0, 0, 1}) : dense(in, {0, 1}))) return false;
       return true;
   }
   return false;
@@ -811,15 +814,16 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
             static_cast<uint16_t *>(out), static_cast<int32_t *>(workspace), res.shapes[fa[0]][0],
             seg.size[1], seg.size[0], block_dim, st));
       case FastPath::MatmulBiasLeaky:
-        return finish(afir::launch_matmul_add_leakyrelu(
+      case FastPath::MatmulBiasLeakyF16: {
+        // plain [M,K] x [K,N] products go to the direct-to-LDS / register-staged kernels, transposed
+        // and batched operands to the layout kernels (launch_matmul_layouts picks)
+        const afir_region::ResolvedOp &mm = seg.ops[0];
+        const int b0 = seg.rank == 3 ? 1 : 0;
+        return finish(afir::launch_matmul_layouts(
             static_cast<const uint16_t *>(args[fa[0]]), static_cast<const uint16_t *>(args[fa[1]]),
-            fa[2] >= 0 ? static_cast<const uint16_t *>(args[fa[2]]) : nullptr, static_cast<uint16_t *>(out),
-            seg.size[0], res.shapes[fa[0]][1], seg.size[1], r->alpha, r->relu, block_dim, st));
-      case FastPath::MatmulBiasLeakyF16:
-        return finish(afir::launch_matmul_add_leakyrelu_f16(
-            static_cast<const uint16_t *>(args[fa[0]]), static_cast<const uint16_t *>(args[fa[1]]),
-            fa[2] >= 0 ? static_cast<const float *>(args[fa[2]]) : nullptr, static_cast<float *>(out),
-            seg.size[0], res.shapes[fa[0]][1], seg.size[1], r->alpha, r->relu, block_dim, st));
+            fa[2] >= 0 ? args[fa[2]] : nullptr, out, r->fast == FastPath::MatmulBiasLeakyF16, mm.batch, seg.size[b0],
+            mm.k, seg.size[b0 + 1], mm.transA, mm.transB, r->alpha, r->relu, block_dim, st));
+      }
       case FastPath::None: break;
     }
   }

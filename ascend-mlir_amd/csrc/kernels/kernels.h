@@ -45,6 +45,15 @@ LaunchStatus launch_matmul_add_leakyrelu_f16(const uint16_t *a, const uint16_t *
                                              float alpha, bool relu, uint32_t block_dim,
                                              hipStream_t stream);
 
+// Matmul with transposed and / or batched operands (matmul_layouts.hip): A as [M, K] or, with
+// trans_a, [K, M]; B as [K, N] or, with trans_b, [N, K]; `batch` independent products of
+// densely packed matrices; bias [N] (null: none) shared by the batches.  f16io selects f16 A, B
+// with float32 bias and out; otherwise everything is bf16.  Plain, unbatched calls go to the
+// kernels above.
+LaunchStatus launch_matmul_layouts(const uint16_t *a, const uint16_t *b, const void *bias, void *out, bool f16io,
+                                   int64_t batch, int64_t m, int64_t k, int64_t n, bool trans_a, bool trans_b,
+                                   float alpha, bool relu, uint32_t block_dim, hipStream_t stream);
+
 // Fast path of the matmul for tile-aligned shapes (matmul_dma.hip).
 bool matmul_dma_supported(int64_t m, int64_t k, int64_t n);
 LaunchStatus launch_matmul_dma(const uint16_t *a, const uint16_t *b, const uint16_t *bias,

@@ -323,10 +323,6 @@ __global__ __launch_bounds__(kWaves * 64) void matmul_bias_leakyrelu_dma(
     static_for<0, kAReg>([&](auto q) { issue_a_region(slot, q); });
     advance_a();
   };
-  auto issue_b = [&](int slot) {
-    static_for<0, kBReg>([&](auto q) { issue_b_region(slot, q); });
-    advance_b();
-  };
   // The fill of both rings at the start of a tile, oldest first: A(0) B(0) B(1) A(1) B(2) B(3)
   // A(2) (the launcher guarantees KT >= 8).  All of it but A(2) is issued *during the epilogue
   // of the previous tile*, one region behind each block of epilogue arithmetic: the rings are

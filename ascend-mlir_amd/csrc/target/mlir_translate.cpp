@@ -45,6 +45,7 @@ struct Expr {
   Ref extent;               // ExtentConst
   ElemType extentType = ElemType::F32;   // ... rounded through this type (arith.sitofp ... to f16)
   int arg = -1, arg2 = -1;
+  bool transA = false, transB = false;   // Matmul: operand stored transposed
   std::vector<Index> idx;   // Input: one per dim of the argument
   std::vector<Ref> slice;   // Input: start offsets (empty = none)
   float value = 0.f;        // Constant; alpha of Leaky
@@ -700,7 +701,17 @@ class Translator {
     } else if (op == "linalg.generic") {
       parseGeneric(results);
     } else if (op == "linalg.matmul") {
-      parseMatmul(one());
+      parseMatmul(one(), op, false, false, false);
+    } else if (op == "linalg.matmul_transpose_a") {
+      parseMatmul(one(), op, true, false, false);
+    } else if (op == "linalg.matmul_transpose_b") {
+      parseMatmul(one(), op, false, true, false);
+    } else if (op == "linalg.batch_matmul") {
+      parseMatmul(one(), op, false, false, true);
+    } else if (op == "linalg.batch_matmul_transpose_a") {
+      parseMatmul(one(), op, true, false, true);
+    } else if (op == "linalg.batch_matmul_transpose_b") {
+      parseMatmul(one(), op, false, true, true);
     } else if (op == "tensor.extract_slice") {
       parseExtractSlice(one());
     } else if (op == "tensor.concat") {
@@ -768,27 +779,36 @@ class Translator {
     defineTensor(result, tv);
   }
 
-  void parseMatmul(const std::string &result) {
+  // linalg.matmul and its relatives: the matmul-like ops the reference's recogniser takes
+  // (lib/Conversion/MarkStructuredOps/AnnotateMixMatmulSemanticsPass.cpp:244-256).
+  //   matmul_transpose_a: A is [K, M]; matmul_transpose_b: B is [N, K];
+  //   batch_matmul*: a leading batch dim on A, B and the result.
+  void parseMatmul(const std::string &result, const std::string &op, bool ta, bool tb, bool batched) {
     if (r_.peek() == '{') { r_.eat('{'); skipDict(); }
     Operands ins = parseOperandGroup("ins"), outs = parseOperandGroup("outs");
-    if (ins.names.size() != 2 || outs.names.size() != 1) r_.fail("linalg.matmul needs two inputs and one init");
+    if (ins.names.size() != 2 || outs.names.size() != 1) r_.fail(op + " needs two inputs and one init");
     TypeInfo rt = outs.types[0];
     if (r_.eatArrow()) rt = parseType();
     TensorP a = tensorOf(ins.names[0]), b = tensorOf(ins.names[1]), init = tensorOf(outs.names[0]);
-    if (a->directArg < 0 || b->directArg < 0 || a->shape.size() != 2 || b->shape.size() != 2)
-      r_.fail("linalg.matmul operands must be rank-2 function arguments");
+    const size_t rank = batched ? 3 : 2, b0 = batched ? 1 : 0;
+    if (a->directArg < 0 || b->directArg < 0 || a->shape.size() != rank || b->shape.size() != rank)
+      r_.fail(op + " operands must be rank-" + std::to_string(rank) + " function arguments");
     // The init is taken as zero: the reference's mix kernel overwrites C
     // (Matmul IterateAll, lib/Target/CannKernel/CannTranslation.cpp:1584-1628)
     // and its example passes an all-zero tensor.
     if (init->expr && !(init->directArg >= 0) && !(init->filled && init->fill == 0.f))
-      r_.fail("linalg.matmul init must be a function argument, an empty tensor or a zero fill");
+      r_.fail(op + " init must be a function argument, an empty tensor or a zero fill");
     auto e = std::make_shared<Expr>();
     e->kind = Expr::Matmul;
     e->arg = a->directArg;
     e->arg2 = b->directArg;
+    e->transA = ta;
+    e->transB = tb;
     auto tv = std::make_shared<Tensor>();
     tv->elem = rt.elemKnown ? rt.elem : init->elem;
-    tv->shape = {a->shape[0], b->shape[1]};
+    if (batched) tv->shape.push_back(a->shape[0]);
+    tv->shape.push_back(a->shape[b0 + (ta ? 1 : 0)]);
+    tv->shape.push_back(b->shape[b0 + (tb ? 0 : 1)]);
     tv->expr = e;
     defineTensor(result, tv);
   }
@@ -1383,6 +1403,8 @@ class Translator {
         o.code = OpCode::Matmul;
         o.arg = e->arg;
         o.arg2 = e->arg2;
+        o.transA = e->transA;
+        o.transB = e->transB;
         ops->push_back(o);
         return;
       case Expr::Input: {

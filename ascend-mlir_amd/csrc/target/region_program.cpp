@@ -138,7 +138,8 @@ std::string serialize(const Program &p) {
           break;
         }
         case OpCode::Matmul:
-          s += "matmul arg" + std::to_string(o.arg) + " arg" + std::to_string(o.arg2) + "\n";
+          s += "matmul arg" + std::to_string(o.arg) + " arg" + std::to_string(o.arg2) +
+               (o.transA ? " ta" : "") + (o.transB ? " tb" : "") + "\n";
           break;
         case OpCode::Const:
           if (o.extent)
@@ -255,8 +256,13 @@ std::string parse(const std::string &text, Program *out) {
     } else if (k == "matmul") {
       Op o;
       o.code = OpCode::Matmul;
-      if (tok.size() != 3 || !parseArgName(tok[1], &o.arg) || !parseArgName(tok[2], &o.arg2))
-        return err(lineno, "expected 'matmul arg<A> arg<B>'");
+      if (tok.size() < 3 || tok.size() > 5 || !parseArgName(tok[1], &o.arg) || !parseArgName(tok[2], &o.arg2))
+        return err(lineno, "expected 'matmul arg<A> arg<B> [ta] [tb]'");
+      for (size_t i = 3; i < tok.size(); ++i) {
+        if (tok[i] == "ta" && !o.transA && !o.transB) o.transA = true;
+        else if (tok[i] == "tb" && !o.transB) o.transB = true;
+        else return err(lineno, "expected 'matmul arg<A> arg<B> [ta] [tb]'");
+      }
       seg->ops.push_back(o);
     } else if (k == "const" && tok.size() >= 2 && tok[1].compare(0, 3, "arg") == 0) {
       Op o;
@@ -407,10 +413,12 @@ std::string validate(const Program &p) {
         }
         case OpCode::Matmul: {
           if (integer) return "region program: 'matmul' is not available in an integer region";
-          if (i != 0 || g.rank != 2) return "region program: 'matmul' must open a rank-2 segment";
+          if (i != 0 || (g.rank != 2 && g.rank != 3))
+            return "region program: 'matmul' must open a rank-2 segment (rank-3: batched)";
           for (int a : {o.arg, o.arg2}) {
             if (a < 0 || a >= p.numInputs()) return "region program: matmul of a non-input argument";
-            if (p.args[a].rank != 2 || !isFloat(p.args[a].type)) return "region program: matmul operands must be rank-2 float tensors";
+            if (p.args[a].rank != g.rank || !isFloat(p.args[a].type))
+              return "region program: matmul operands must be float tensors of the segment's rank";
           }
           ++depth;
           break;
@@ -597,11 +605,18 @@ std::string resolve(const Program &p, const std::vector<int64_t> &dims, Resolved
       }
       if (o.code == OpCode::Matmul) {
         const std::vector<int64_t> &sa = r.shapes[o.arg], &sb = r.shapes[o.arg2];
-        if (sa[0] != s.size[0] || sb[1] != s.size[1] || sa[1] != sb[0])
+        const size_t b0 = sa.size() - 2;   // 1 with a leading batch dim
+        const int64_t am = sa[b0 + (o.transA ? 1 : 0)], ak = sa[b0 + (o.transA ? 0 : 1)];
+        const int64_t bk = sb[b0 + (o.transB ? 1 : 0)], bn = sb[b0 + (o.transB ? 0 : 1)];
+        if (am != s.size[b0] || bn != s.size[b0 + 1] || ak != bk ||
+            (b0 && (sa[0] != s.size[0] || sb[0] != s.size[0])))
           return "region: matmul operand shapes do not agree with the segment";
         ro.arg = o.arg;
         ro.arg2 = o.arg2;
-        ro.k = sa[1];
+        ro.k = ak;
+        ro.batch = b0 ? s.size[0] : 1;
+        ro.transA = o.transA;
+        ro.transB = o.transB;
       }
       if (o.code == OpCode::Push) {
         const std::vector<int64_t> &shape = r.shapes[o.arg];

@@ -36,8 +36,13 @@
 //                               integer constant, or g<k>:argI (dim r is indexed
 //                               by the rank-1 index tensor I at iteration dim k)
 //                               slice: per-dim start offsets of an extract_slice
-//     matmul argA argB          push sum_k A[d0,k] * B[k,d1] (float32 accumulation);
-//                               only as the first operation of a rank-2 segment
+//     matmul argA argB [ta] [tb]
+//                               push sum_k A[d0,k] * B[k,d1] (float32 accumulation); only as
+//                               the first operation of a rank-2 segment.  ta: A is stored
+//                               transposed, [K,M]; tb: B is stored as [N,K]
+//                               (linalg.matmul_transpose_a / _b).  Opening a rank-3 segment
+//                               it is the batched product out[b] = A[b] x B[b] of rank-3
+//                               operands (linalg.batch_matmul*), d0 being the batch
 //     const <float>             push a constant
 //     const <ref> [<type>]      push an extent as a number (mean = sum / N): the value of
 //                               argA.D converted to float, rounded to f16 | bf16 when a
@@ -100,6 +105,7 @@ struct Op {
   OpCode code = OpCode::Add;
   int arg = -1;                     // Push; Matmul: the [M,K] operand
   int arg2 = -1;                    // Matmul: the [K,N] operand
+  bool transA = false, transB = false;   // Matmul: the operand is stored transposed
   std::vector<MapResult> map;       // Push: one per dim of the input
   std::vector<Ref> slice;           // Push: start offset per dim (empty = none)
   float constant = 0.f;             // Const, Leaky
@@ -156,6 +162,8 @@ struct ResolvedOp {
   int input = -1;      // Push: index into ResolvedSegment::inputs
   int arg = -1, arg2 = -1;  // Matmul: argument indices
   int64_t k = 0;            // Matmul: contraction extent
+  int64_t batch = 1;        // Matmul: independent products (rank-3 segment)
+  bool transA = false, transB = false;
   float constant = 0.f;
   int depth = 0;
 };

@@ -111,7 +111,8 @@ def parse(text: str) -> dict:
                     m.append(("const", int(t)))
             seg["ops"].append(("push", arg, m, sl))
         elif k == "matmul":
-            seg["ops"].append(("matmul", int(tok[1][3:]), int(tok[2][3:])))
+            # 'ta' / 'tb': the operand is stored transposed (linalg.matmul_transpose_a / _b)
+            seg["ops"].append(("matmul", int(tok[1][3:]), int(tok[2][3:]), "ta" in tok[3:], "tb" in tok[3:]))
         elif k == "const" and tok[1].startswith("arg"):
             # an extent as a number, rounded through the named float type (f32 when none):
             # arith.sitofp of a cast tensor.dim, examples/broadcast-add-reduce/step0_input_mean.mlir:73-74
@@ -261,8 +262,14 @@ def evaluate(text: str, inputs, out_shape=None):
             elif k == "matmul":
                 # float32 product as the reference golden computes it
                 # (examples/matmul-add-leakyrelu/gen_data.py:33: A.f32 @ B.f32)
+                # transposed storage is undone first; rank-3 operands are batches of matrices
+                # (numpy's @ multiplies the last two dims: linalg.batch_matmul)
                 a = _widen(inputs[op[1]], args[op[1]][1])
                 b = _widen(inputs[op[2]], args[op[2]][1])
+                if op[3]:
+                    a = np.swapaxes(a, -1, -2)
+                if op[4]:
+                    b = np.swapaxes(b, -1, -2)
                 stack.append((a @ b).astype(np.float32))
             elif k == "const":
                 stack.append(np.full(size[:-1] if reduced else size, op[1], dtype=np.float32))

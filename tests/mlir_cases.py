@@ -444,3 +444,24 @@ func.func @int_chain(%a : tensor<?x?xi32>, %b : tensor<?x?xi32>) -> tensor<?x?xi
   return %4 : tensor<?x?xi32>
 }
 """
+
+# The other matmul-like ops the reference's recogniser takes
+# (lib/Conversion/MarkStructuredOps/AnnotateMixMatmulSemanticsPass.cpp:244-256):
+# transposed operands and batches.
+MATMUL_TRANSPOSE_A_F16 = MATMUL_PLAIN_F16.replace("linalg.matmul ", "linalg.matmul_transpose_a ") \
+    .replace("@mm_plain", "@mm_ta")
+MATMUL_TRANSPOSE_B_F16 = MATMUL_PLAIN_F16.replace("linalg.matmul ", "linalg.matmul_transpose_b ") \
+    .replace("@mm_plain", "@mm_tb")
+MATMUL_TRANSPOSE_B_BIAS_LEAKY_BF16 = MATMUL_BIAS_LEAKY_BF16.replace("linalg.matmul ", "linalg.matmul_transpose_b ") \
+    .replace("@mm_bias_leaky_bf16", "@mm_tb_bias_leaky_bf16")
+BATCH_MATMUL_BF16 = """
+func.func @bmm(%a : tensor<?x?x?xbf16>, %b : tensor<?x?x?xbf16>, %init : tensor<?x?x?xbf16>) -> tensor<?x?x?xbf16> {
+  %c = linalg.batch_matmul ins(%a, %b : tensor<?x?x?xbf16>, tensor<?x?x?xbf16>)
+                           outs(%init : tensor<?x?x?xbf16>) -> tensor<?x?x?xbf16>
+  return %c : tensor<?x?x?xbf16>
+}
+"""
+BATCH_MATMUL_TRANSPOSE_B_F16 = BATCH_MATMUL_BF16.replace("xbf16", "xf16").replace("linalg.batch_matmul ", "linalg.batch_matmul_transpose_b ") \
+    .replace("outs(%init : tensor<?x?x?xf16>) -> tensor<?x?x?xf16>", "outs(%init : tensor<?x?x?xf32>) -> tensor<?x?x?xf32>") \
+    .replace("%init : tensor<?x?x?xf16>) -> tensor<?x?x?xf16> {", "%init : tensor<?x?x?xf32>) -> tensor<?x?x?xf32> {") \
+    .replace("return %c : tensor<?x?x?xf16>", "return %c : tensor<?x?x?xf32>").replace("@bmm", "@bmm_tb")

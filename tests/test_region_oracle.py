@@ -216,3 +216,25 @@ def test_mean_against_the_reference_written_sum_vector():
 def test_reduce_tail_chain_matches_its_closed_form():
     text, inputs, want = RC.case_reduce_tail_chain()
     assert RO.evaluate(text, inputs).tobytes() == want.tobytes()
+
+
+def test_matmul_layout_flags_against_numpy():
+    """'ta' / 'tb' and the batched rank-3 form against numpy on the operands put back in the
+    plain layout (float32 product of the widened operands, as the reference's golden computes it,
+    examples/matmul-add-leakyrelu/gen_data.py:33)."""
+    rng = np.random.default_rng(5)
+    m, k, n, nb = 5, 7, 3, 4
+    a = rng.standard_normal((m, k)).astype(np.float16)
+    b = rng.standard_normal((k, n)).astype(np.float16)
+    want = a.astype(np.float32) @ b.astype(np.float32)
+    head = RC.HEADER + "arg in f16 2\narg in f16 2\narg out f32 2\nsegment 2\n size arg2.0 arg2.1\n outoff 0\n"
+    for flags, aa, bb in (("", a, b), (" ta", a.T.copy(), b), (" tb", a, b.T.copy()), (" ta tb", a.T.copy(), b.T.copy())):
+        got = RO.evaluate(head + f" matmul arg0 arg1{flags}\n store\nend\n", [aa, bb], out_shape=(m, n))
+        assert got.dtype == np.float32 and np.array_equal(got, want), flags
+    a3 = rng.standard_normal((nb, m, k)).astype(np.float16)
+    b3 = rng.standard_normal((nb, n, k)).astype(np.float16)
+    want3 = np.stack([a3[i].astype(np.float32) @ b3[i].astype(np.float32).T for i in range(nb)])
+    prog = (RC.HEADER + "arg in f16 3\narg in f16 3\narg out f32 3\nsegment 3\n size arg2.0 arg2.1 arg2.2\n outoff 0\n"
+            " matmul arg0 arg1 tb\n store\nend\n")
+    got = RO.evaluate(prog, [a3, b3], out_shape=(nb, m, n))
+    assert np.array_equal(got, want3)

@@ -332,3 +332,32 @@ def test_reference_matmul_example_translates():
                        capture_output=True, text=True)
     assert p.returncode == 0, p.stderr
     assert "matmul arg0 arg1\npush arg2 d1\nadd\nleaky 0.00100000005\nstore" in p.stdout
+
+
+def test_transposed_and_batched_matmul_ops(pkg):
+    """linalg.matmul_transpose_a / _b and linalg.batch_matmul*: the other matmul-like ops of the
+    reference's recogniser (AnnotateMixMatmulSemanticsPass.cpp:244-256) become 'matmul' with
+    'ta' / 'tb', or open a rank-3 segment."""
+    from ascend_mlir_amd import hip_kernels as H
+    def body(mlir):
+        return [l.strip() for l in program_of(mlir).splitlines() if l.strip() and not l.startswith("#")]
+    b = body(MC.MATMUL_TRANSPOSE_A_F16)
+    assert b[-3:] == ["matmul arg0 arg1 ta", "store", "end"] and "segment 2" in b
+    b = body(MC.MATMUL_TRANSPOSE_B_F16)
+    assert b[-3:] == ["matmul arg0 arg1 tb", "store", "end"]
+    b = body(MC.MATMUL_TRANSPOSE_B_BIAS_LEAKY_BF16)
+    assert b[-6:] == ["matmul arg0 arg1 tb", "push arg2 d1", "add", "leaky 0.0100097656", "store", "end"]   # 1e-2 as a bf16 constant
+    b = body(MC.BATCH_MATMUL_BF16)
+    assert b[-3:] == ["matmul arg0 arg1", "store", "end"] and "segment 3" in b
+    assert [l for l in b if l.startswith("arg")] == ["arg in bf16 3", "arg in bf16 3", "arg in bf16 3", "arg out bf16 3"]
+    b = body(MC.BATCH_MATMUL_TRANSPOSE_B_F16)
+    assert b[-3:] == ["matmul arg0 arg1 tb", "store", "end"] and "segment 3" in b
+    for mlir in (MC.MATMUL_TRANSPOSE_A_F16, MC.MATMUL_TRANSPOSE_B_BIAS_LEAKY_BF16, MC.BATCH_MATMUL_BF16,
+                 MC.BATCH_MATMUL_TRANSPOSE_B_F16):
+        r = H.Region(program_of(mlir))      # registers: the matmul kernels take it
+        assert r.kernel.startswith("matmul_add_leakyrelu")
+        r.close()
+    # flags are part of the grammar: anything else after the operands is refused
+    bad = program_of(MC.MATMUL_TRANSPOSE_B_F16).replace("matmul arg0 arg1 tb", "matmul arg0 arg1 tb ta")
+    with pytest.raises(H.AfirHipError, match=r"\[ta\] \[tb\]"):
+        H.Region(bad)
