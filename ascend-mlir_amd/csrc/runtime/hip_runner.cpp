@@ -281,14 +281,11 @@ class HipExecutionRunner final : public ExecutionRunner {
       (void)hipEventRecord(ev0_, stream_);
       for (int rep = 0; rep < repeats && rc == 0; ++rep) rc = launchOnce(sets[next++ % nsets].data());
       (void)hipEventRecord(ev1_, stream_);
-      hipError_t e = hipStreamSynchronize(stream_);
-      const bool ok = true;
-      if (rc == 0 && e == hipSuccess) {
-        float ms = 0.f;
-        if (hipEventElapsedTime(&ms, ev0_, ev1_) == hipSuccess) bestUs = (double)ms * 1e3 / repeats;
-      }
+      const hipError_t e = hipStreamSynchronize(stream_);
       if (rc != 0) return launchFailed(rc);
-      if (!ok || e != hipSuccess) { cleanup(); return Status::error(hipErr("timed launches", ok ? e : hipErrorOutOfMemory)); }
+      if (e != hipSuccess) { cleanup(); return Status::error(hipErr("hipStreamSynchronize (timed launches)", e)); }
+      float ms = 0.f;
+      if (hipEventElapsedTime(&ms, ev0_, ev1_) == hipSuccess) bestUs = (double)ms * 1e3 / repeats;
     }
     lastKernelUs_ = bestUs;
 

@@ -209,7 +209,8 @@ ExprP substitute(const ExprP &e, const std::vector<Index> &with) {
 // value at (d + offsets) of every read
 ExprP offsetReads(const ExprP &e, const std::vector<Ref> &offsets) {
   switch (e->kind) {
-    case Expr::Constant: return e;
+    case Expr::Constant: case Expr::ExtentConst: return e;
+    case Expr::Reduced: throw Failure("extract_slice of a reduced value is not supported");
     case Expr::Matmul: throw Failure("extract_slice of a matmul result is not supported");
     case Expr::Unary: return makeUnary(e->op, offsetReads(e->a, offsets), e->value);
     case Expr::Binary: {
