@@ -86,3 +86,29 @@ def test_autotune_tile_shapes_of_a_transposing_region(tmp_path):
     assert len(lines) == 4 and all(" OK " in l and "max_abs_diff=0" in l for l in lines), p.stdout
     best = json.loads((tmp_path / "best.json").read_text())
     assert (best["config"]["emit_tile_p"], best["config"]["emit_tile_q"]) in [(32, 64), (32, 128), (64, 64), (64, 128)]
+
+
+def test_rotating_buffer_sets_and_ramp(tmp_path):
+    """--buffer-sets N: the timed launches rotate over N device copies of the tensors; --ramp-ms:
+    a candidate is launched back to back before it is timed and scored by the average of its
+    timed launches.  The output handed back (and validated) is that of the first copy; the score
+    stays a positive kernel time."""
+    rng = np.random.default_rng(6)
+    a = rng.standard_normal(2048).astype(np.float16)
+    b = rng.standard_normal((2048, 1024)).astype(np.float16)
+    np.save(tmp_path / "a.npy", a)
+    np.save(tmp_path / "b.npy", b)
+    want = (a[:, None].astype(np.float32) + b.astype(np.float32)).sum(axis=1).astype(np.float16)
+    p = _run(tmp_path, want, "--atol", "0.25", "--rtol", "0.01", "--buffer-sets", "3", "--ramp-ms", "5",
+             "--repeats", "24")
+    assert p.returncode == 0, p.stdout + p.stderr
+    lines = [l for l in p.stdout.splitlines() if l.startswith("[")]
+    assert len(lines) == 4 and all(" OK " in l for l in lines), p.stdout
+    scores = [float(l.split("score=")[1].split()[0]) for l in lines]
+    assert all(0 < s < 5_000_000 for s in scores)
+    best = json.loads((tmp_path / "best.json").read_text())
+    assert best["best"]["score"] == round(min(scores)) and best["best"]["max_abs_diff"] <= 0.25
+    # a wrong expectation still fails every candidate: the rotation does not hide the first copy's output
+    p = _run(tmp_path, want + np.float16(3.0), "--atol", "0.25", "--rtol", "0.01", "--buffer-sets", "3",
+             "--ramp-ms", "5", "--repeats", "8")
+    assert p.returncode == 1 and p.stdout.count(" FAIL ") == 4
