@@ -5,6 +5,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 namespace afir {
 
@@ -26,6 +27,35 @@ inline int device_cus() {
     return kNumCU;
   }();
   return count;
+}
+
+// Read / write phase separation (the one-shot kernels of gather.hip and transpose.hip): a launch
+// whose lanes are all resident at once requests everything it reads, holds its stores back
+// until the chip's reads have been served, and then writes.  The hold is a time: ticks of the
+// real-time counter the device reads with wall_clock64() (100 MHz on MI355X), counted from the
+// start of each workgroup, base_ns + read_bytes / (gb_per_s GB/s).  AFIR_HIP_PHASED=0 in the
+// environment switches the phased kernels off (the launchers then take their other kernels).
+inline bool phased_enabled() {
+  const char *env = getenv("AFIR_HIP_PHASED");
+  return !(env && env[0] == '0');
+}
+inline int wall_clock_khz() {
+  static const int khz = [] {
+    int device = 0, value = 0;
+    if (hipGetDevice(&device) == hipSuccess &&
+        hipDeviceGetAttribute(&value, hipDeviceAttributeWallClockRate, device) == hipSuccess && value > 0)
+      return value;
+    (void)hipGetLastError();
+    return 100000;
+  }();
+  return khz;
+}
+constexpr int kPhaseHoldMaxTicks = 1 << 14;      // ~164 us at 100 MHz: no launch waits longer than this
+constexpr int kPhaseSpinLimit = 1 << 15;         // polls of the counter, whatever it reads
+inline int phase_hold_ticks(int64_t read_bytes, int base_ns, int gb_per_s) {
+  const double ns = (double)base_ns + (double)read_bytes / (double)gb_per_s;
+  const double ticks = ns * 1e-6 * (double)wall_clock_khz();
+  return ticks > (double)kPhaseHoldMaxTicks ? kPhaseHoldMaxTicks : (int)ticks;
 }
 
 typedef float f32x4 __attribute__((ext_vector_type(4)));

@@ -43,9 +43,15 @@ __device__ __forceinline__ u32x4 scale_shift_packed(u32x4 t, u32x4 s, u32x4 h) {
     const uint32_t tw = t[d], sw = s[d], hw = h[d];
     const half2_t tv = __builtin_bit_cast(half2_t, tw), sv = __builtin_bit_cast(half2_t, sw),
                   hv = __builtin_bit_cast(half2_t, hw);
+    // (the empty asm keeps the float32 results as values of their own: left alone, the compiler
+    // folds the conversion into the multiply-add in some contexts (v_fma_mixlo_f16), which rounds
+    // once, to f16, where the golden rounds to float32 first)
+    float lo = __builtin_fmaf((float)tv.x, (float)sv.x, (float)hv.x);
+    float hi = __builtin_fmaf((float)tv.y, (float)sv.y, (float)hv.y);
+    asm("" : "+v"(lo), "+v"(hi));
     half2_t o;
-    o.x = (_Float16)__builtin_fmaf((float)tv.x, (float)sv.x, (float)hv.x);
-    o.y = (_Float16)__builtin_fmaf((float)tv.y, (float)sv.y, (float)hv.y);
+    o.x = (_Float16)lo;
+    o.y = (_Float16)hi;
     r[d] = __builtin_bit_cast(uint32_t, o);
   }
   return r;
@@ -200,6 +206,99 @@ __global__ __launch_bounds__(kGroupedThreads) void gather_scale_shift_f16_groupe
   }
 }
 
+// The same row layout for gathers that fit the chip in one go (every lane of every workgroup
+// resident at once: 2048 lanes per CU at 64 registers, eight 16-byte chunks per lane), with the
+// reads and the writes of the whole chip separated in time.  HBM serves a pure read stream and a
+// pure write stream faster than their mixture (64 MiB copied: 22.7 us mixed; 10.7 + 11.2 us as a
+// read kernel followed by a write kernel), so every lane requests all its chunks at once and
+// holds its stores back until `hold_ticks` of the real-time counter have passed since its
+// workgroup started: by then the reads of all workgroups, which start within a microsecond or
+// two of each other, have been served.  The wait is bounded and only shapes the timing: the
+// stores are the same whenever they leave.  Measured on the 32768 x 1024 gather: 23.9 -> 21.6 us;
+// on 24576 rows 20.5 -> 16.4, 8192 rows 8.6 -> 6.4.  The hold that measured best is the time the
+// gathered bytes take at AFIR_GATHER_PHASE_GBS plus AFIR_GATHER_PHASE_BASE_NS, for 8192 to 32768
+// rows alike (half a microsecond either side costs 2 %).  It is tuned for indices spread over
+// the table: when most of the gathered rows come out of the caches (2048 distinct rows in 32768
+// indices) the reads end early, the hold is too long and the launch takes 21 us instead of 15.
+#ifndef AFIR_GATHER_PHASED
+#define AFIR_GATHER_PHASED 1
+#endif
+#ifndef AFIR_GATHER_PHASED_THREADS
+#define AFIR_GATHER_PHASED_THREADS 256
+#endif
+#ifndef AFIR_GATHER_PHASE_GBS
+#define AFIR_GATHER_PHASE_GBS 6900
+#endif
+#ifndef AFIR_GATHER_PHASE_BASE_NS
+#define AFIR_GATHER_PHASE_BASE_NS 300
+#endif
+constexpr int kPhasedThreads = AFIR_GATHER_PHASED_THREADS;
+constexpr int kPhasedPasses = 2;
+constexpr int kPhasedLanesPerCU = 2048;
+
+__global__ __launch_bounds__(kPhasedThreads, 8) void gather_scale_shift_f16_phased(
+    const uint16_t *__restrict__ table, const int32_t *__restrict__ idx,
+    const uint16_t *__restrict__ scale, const uint16_t *__restrict__ shift,
+    uint16_t *__restrict__ out, int32_t *__restrict__ error_flag, uint32_t rows, int lanes_log2,
+    int hold_ticks) {
+  const long long t_start = wall_clock64();
+  const int lanes = 1 << lanes_log2;
+  const int rows_per_pass = kPhasedThreads >> lanes_log2;
+  const int local_row = threadIdx.x >> lanes_log2;
+  const int col0 = threadIdx.x & (lanes - 1);
+  const int dim = lanes * kGroups * 8;
+  const int nchunks = lanes * kGroups;          // chunks per row
+  extern __shared__ u32x4 params[];            // scale chunks, then shift chunks
+  const int64_t r0 = (int64_t)blockIdx.x * (rows_per_pass * kPhasedPasses);
+
+  uint32_t src[kPhasedPasses];
+  bool good[kPhasedPasses];
+  u32x4 v[kPhasedPasses][kGroups];
+#pragma unroll
+  for (int p = 0; p < kPhasedPasses; ++p) {
+    src[p] = (uint32_t)idx[r0 + p * rows_per_pass + local_row];
+  }
+#pragma unroll
+  for (int p = 0; p < kPhasedPasses; ++p) {
+    good[p] = src[p] < rows;
+    const u32x4 *row = reinterpret_cast<const u32x4 *>(table + (int64_t)(good[p] ? src[p] : 0u) * dim) + col0;
+#pragma unroll
+    for (int u = 0; u < kGroups; ++u) v[p][u] = row[u * lanes];
+  }
+  for (int c = threadIdx.x; c < nchunks; c += kPhasedThreads) {
+    params[c] = *reinterpret_cast<const u32x4 *>(scale + (int64_t)c * 8);
+    params[nchunks + c] = *reinterpret_cast<const u32x4 *>(shift + (int64_t)c * 8);
+  }
+  // (the asm makes the loads' results exist here, so the wait for them sits before the hold)
+#pragma unroll
+  for (int p = 0; p < kPhasedPasses; ++p)
+#pragma unroll
+    for (int u = 0; u < kGroups; ++u) asm volatile("" : "+v"(v[p][u]));
+  __syncthreads();
+  for (int spin = 0; spin < kPhaseSpinLimit && wall_clock64() - t_start < hold_ticks; ++spin)
+    __builtin_amdgcn_s_sleep(1);
+
+  // stores: a base per (pass, chunk group) that is the same for the whole workgroup (scalar
+  // registers) plus one 32-bit offset per lane.  The lane's scale / shift chunks come from LDS at
+  // their use: held in registers across the loads they would push the kernel past 64 registers.
+  const u32x4 nan_row = {0x7e007e00u, 0x7e007e00u, 0x7e007e00u, 0x7e007e00u};
+  char *block_out = reinterpret_cast<char *>(out) + r0 * dim * 2;
+  const uint32_t lane_off = (uint32_t)(local_row * dim + col0 * 8) * 2u;
+#pragma unroll
+  for (int u = 0; u < kGroups; ++u) {
+    const u32x4 sraw = params[col0 + u * lanes], hraw = params[nchunks + col0 + u * lanes];
+#pragma unroll
+    for (int p = 0; p < kPhasedPasses; ++p) {
+      char *base = block_out + ((int64_t)p * rows_per_pass * dim + (int64_t)u * lanes * 8) * 2;
+      const u32x4 res = good[p] ? scale_shift_packed(v[p][u], sraw, hraw) : nan_row;
+      // (s_nop: the store reads its four data registers over the following cycles)
+      asm volatile("global_store_dwordx4 %0, %1, %2 nt\n\ts_nop 1" ::"v"(lane_off), "v"(res), "s"(base) : "memory");
+    }
+  }
+  const bool bad = !(good[0] && good[1]);
+  if (bad && error_flag && col0 == 0) atomicOr(error_flag, 1);
+}
+
 // Any dim / alignment: one wave per row, 2-byte accesses.
 __global__ __launch_bounds__(kThreads) void gather_scale_shift_f16_any(
     const uint16_t *__restrict__ table, const int32_t *__restrict__ idx,
@@ -247,6 +346,23 @@ LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx
   const int64_t chunks64 = dim / 8;
   int lanes_log2 = 0;
   while (lanes_log2 < 8 && ((int64_t)kGroups << lanes_log2) < chunks64) ++lanes_log2;
+  // whole blocks of a gather that fits the chip at once: the phased kernel; rows left over: below
+  const int64_t phased_rows_per_block = (int64_t)(kPhasedThreads >> (lanes_log2 < 8 ? lanes_log2 : 8)) * kPhasedPasses;
+  const int64_t phased_blocks = nidx / phased_rows_per_block;
+  if (AFIR_GATHER_PHASED && vec && ((int64_t)kGroups << lanes_log2) == chunks64 && !block_dim &&
+      (1 << lanes_log2) <= kPhasedThreads && phased_blocks > 0 &&
+      phased_blocks * kPhasedThreads <= (int64_t)device_cus() * kPhasedLanesPerCU && phased_enabled()) {
+    const size_t lds = (size_t)2 * (kGroups << lanes_log2) * 16;   // scale and shift, 16-byte chunks
+    const int hold_ticks = phase_hold_ticks(phased_blocks * phased_rows_per_block * dim * 2,
+                                            AFIR_GATHER_PHASE_BASE_NS, AFIR_GATHER_PHASE_GBS);
+    hipLaunchKernelGGL(gather_scale_shift_f16_phased, dim3((unsigned)phased_blocks), dim3(kPhasedThreads), lds,
+                       stream, table, idx, scale, shift, out, error_flag, (uint32_t)rows, lanes_log2, hold_ticks);
+    const int64_t done = phased_blocks * phased_rows_per_block;
+    if (done == nidx) return after_launch();
+    idx += done;
+    out += done * dim;
+    nidx -= done;
+  }
   if (vec && ((int64_t)kGroups << lanes_log2) == chunks64) {
     const int64_t rows_per_block = (int64_t)(kGroupedThreads >> lanes_log2) * kGroupedPasses;
     int64_t blocks = (nidx + rows_per_block - 1) / rows_per_block;

@@ -239,6 +239,39 @@ def test_c4_blockdim(H):
         assert out.tobytes() == want.tobytes()
 
 
+# Gathers whose rows are 32 * 2^k halves and that fit the chip at once take the kernel that
+# separates the chip's reads from its writes in time (whole blocks of rows; rows left over take
+# the other kernel in a second launch).  AFIR_HIP_PHASED=0 keeps a launch off it.
+@pytest.mark.parametrize("dim,nidx", [(1024, 16), (1024, 17), (1024, 513), (1024, 4099), (256, 64), (256, 1000),
+                                      (2048, 8), (2048, 77), (8192, 2), (8192, 31), (32, 512), (32, 70001),
+                                      (1024, 40000)])
+def test_c4_phased_route_bit_exact(H, dim, nidx, monkeypatch):
+    rows = 3000
+    table, idx, scale, shift = O.gen_c4(rows, dim, nidx)
+    idx[:2] = [rows - 1, 0]
+    idx[-1] = rows - 1
+    want = O.golden_c4(table, idx, scale, shift)
+    out = H.gather_scale_shift(dev(table), dev(idx), dev(scale), dev(shift)).cpu().numpy()
+    assert out.tobytes() == want.tobytes()
+    monkeypatch.setenv("AFIR_HIP_PHASED", "0")
+    out = H.gather_scale_shift(dev(table), dev(idx), dev(scale), dev(shift)).cpu().numpy()
+    assert out.tobytes() == want.tobytes()
+
+
+def test_c4_phased_route_flags_bad_indices(H):
+    table, idx, scale, shift = O.gen_c4(500, 1024, 100)
+    idx[[3, 40, 99]] = [500, -7, 1 << 30]       # rows 3 and 40 in whole blocks, 99 among the rows left over
+    ws = torch.zeros(2, dtype=torch.int32, device="cuda")
+    out = H.gather_scale_shift(dev(table), dev(idx), dev(scale), dev(shift), workspace=ws).cpu().numpy()
+    assert int(ws[0].item()) != 0
+    good = np.ones(100, bool)
+    good[[3, 40, 99]] = False
+    assert np.isnan(out[~good]).all()
+    idx2 = idx.copy()
+    idx2[~good] = 0
+    assert out[good].tobytes() == O.golden_c4(table, idx2, scale, shift)[good].tobytes()
+
+
 # ---------------------------------------------------------------- C5 --------
 
 C5_ATOL, C5_RTOL = 1e-5, 1e-2
