@@ -115,6 +115,103 @@ __global__ __launch_bounds__(kThreads) void relu_bcast_add_transpose_f16_tile64(
   }
 }
 
+// The same tiles for shapes that fit the chip in one go (every lane of every workgroup resident
+// at once: eight workgroups per CU, 64 registers, one LDS tile each), with the reads and the
+// writes of the whole chip separated in time: HBM serves a pure read stream and a pure write
+// stream faster than their mixture.  A workgroup takes four tiles that follow each other along N
+// (it reads 512-byte runs; consecutive workgroups continue along N, so the requests of a moment
+// fall into the same memory pages), requests all of them at once, transposes each as it arrives
+// -- the LDS work sits in the shadow of the chip's reads -- and keeps the finished chunks in
+// registers until `hold_ticks` of the real-time counter have passed since it started: by then
+// the reads of all workgroups, which start within a microsecond or two of each other, have been
+// served, and the stores leave back to back.  The wait is bounded and only shapes the timing:
+// the stores are the same whenever they leave.  c is added after the transposition (a lane
+// then needs one value per output row instead of eight per tile).
+// Measured (us per launch, other kernel -> this one): [64, 1024, 512] 23.6 -> 21.3,
+// [32, 1024, 512] 13.4 -> 11.0, [16, 2048, 1024] 23.9 -> 20.8, [4, 4096, 2048] 25.2 -> 21.9; the
+// best hold is the time the bytes read take at AFIR_TRANSPOSE_PHASE_GBS plus
+// AFIR_TRANSPOSE_PHASE_BASE_NS (5 % either side costs 2 %).  Below 24 MiB the other kernel is as
+// fast or faster (one tile per workgroup spreads a small shape over more CUs) and stays in use;
+// four tiles along M or 2 x 2 per workgroup measured 0.71 and 0.74 of peak at their best holds
+// against 0.79.
+#ifndef AFIR_TRANSPOSE_PHASED
+#define AFIR_TRANSPOSE_PHASED 1
+#endif
+#ifndef AFIR_TRANSPOSE_PHASE_GBS
+#define AFIR_TRANSPOSE_PHASE_GBS 6900
+#endif
+#ifndef AFIR_TRANSPOSE_PHASE_BASE_NS
+#define AFIR_TRANSPOSE_PHASE_BASE_NS 300
+#endif
+constexpr int kPhasedTiles = 4;           // tiles per workgroup, along N
+constexpr int kPhasedLanesPerCU = 2048;
+constexpr int kPhasedMinGroupsPerCU = 3;  // smaller launches take the other kernel
+__global__ __launch_bounds__(kThreads, 8) void relu_bcast_add_transpose_f16_phased(
+    const uint16_t *__restrict__ x, const uint16_t *__restrict__ c, uint16_t *__restrict__ out,
+    int nb, int m, int n, int hold_ticks) {
+  const long long t_start = wall_clock64();
+  __shared__ float tile[kSmallTile * kSmallPitch];
+  __shared__ float cs[kSmallTile * kPhasedTiles];
+  const int t = threadIdx.x;
+  const unsigned tiles_m = (unsigned)(m / kSmallTile), groups_n = (unsigned)(n / (kSmallTile * kPhasedTiles));
+  const int lj = (t & 7) * 8, li = t >> 3;        // loads: first column, row within a pass of 32
+  const int oi = (t & 7) * 8, oj = t >> 3;        // stores: first i of the chunk, j within a pass of 32
+  const unsigned rest = blockIdx.x / groups_n;
+  const int n0 = (int)(blockIdx.x - rest * groups_n) * (kSmallTile * kPhasedTiles);
+  const int b = (int)(rest / tiles_m);
+  const int m0 = (int)(rest - (unsigned)b * tiles_m) * kSmallTile;
+  u32x4 v[kPhasedTiles][2];
+  {
+    const uint16_t *xin = x + ((int64_t)b * m + m0 + li) * n + n0 + lj;
+#pragma unroll
+    for (int q = 0; q < kPhasedTiles; ++q)
+#pragma unroll
+      for (int k = 0; k < 2; ++k)
+        v[q][k] = *reinterpret_cast<const u32x4 *>(xin + (int64_t)(32 * k) * n + kSmallTile * q);
+  }
+  cs[t] = (float)__builtin_bit_cast(_Float16, c[n0 + t]);
+#pragma unroll
+  for (int q = 0; q < kPhasedTiles; ++q) {
+#pragma unroll
+    for (int k = 0; k < 2; ++k)
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        float *dst = tile + (li + 32 * k) * kSmallPitch + lj + 2 * d;
+        dst[0] = relu_keep_nan(f16_lo(v[q][k][d]));
+        dst[1] = relu_keep_nan(f16_hi(v[q][k][d]));
+      }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int j = oj + 32 * k;
+      const float cj = cs[kSmallTile * q + j];
+#pragma unroll
+      for (int d = 0; d < 4; ++d)
+        v[q][k][d] = pack_f16(tile[(oi + 2 * d) * kSmallPitch + j] + cj, tile[(oi + 2 * d + 1) * kSmallPitch + j] + cj);
+    }
+    __syncthreads();
+  }
+  // (the asm makes the finished chunks exist here, so nothing of the above is left for after the hold)
+#pragma unroll
+  for (int q = 0; q < kPhasedTiles; ++q)
+#pragma unroll
+    for (int k = 0; k < 2; ++k) asm volatile("" : "+v"(v[q][k]));
+  for (int spin = 0; spin < kPhaseSpinLimit && wall_clock64() - t_start < hold_ticks; ++spin)
+    __builtin_amdgcn_s_sleep(1);
+  // stores: a base per (tile, pass) that is the same for the whole workgroup (scalar registers)
+  // plus one 32-bit offset per lane
+  char *block_out = reinterpret_cast<char *>(out + ((int64_t)b * n + n0) * m + m0);
+  const uint32_t lane_off = (uint32_t)(oj * m + oi) * 2u;
+#pragma unroll
+  for (int q = 0; q < kPhasedTiles; ++q)
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      char *base = block_out + (int64_t)(kSmallTile * q + 32 * k) * m * 2;
+      // (s_nop: the store reads its four data registers over the following cycles)
+      asm volatile("global_store_dwordx4 %0, %1, %2 nt\n\ts_nop 1" ::"v"(lane_off), "v"(v[q][k]), "s"(base) : "memory");
+    }
+}
+
 // Any shape / alignment: 32x32 tiles through a padded LDS array, 2-byte accesses.
 __global__ __launch_bounds__(kThreads) void relu_bcast_add_transpose_f16_any(
     const uint16_t *__restrict__ x, const uint16_t *__restrict__ c, uint16_t *__restrict__ out,
@@ -159,8 +256,16 @@ LaunchStatus launch_relu_broadcast_add_transpose(const uint16_t *x, const uint16
     return invalid("relu_broadcast_add_transpose: extent exceeds 2^31-1");
   if (nb > INT64_MAX / m / n / 4) return invalid("relu_broadcast_add_transpose: extent overflow");
 
-  if ((m % kSmallTile == 0) && (n % kSmallTile == 0) && aligned16(x) && aligned16(c) && aligned16(out) &&
-      nb * (m / kSmallTile) * (n / kSmallTile) < ((int64_t)1 << 31)) {
+  const bool tiled = (m % kSmallTile == 0) && (n % kSmallTile == 0) && aligned16(x) && aligned16(c) && aligned16(out) &&
+                     nb * (m / kSmallTile) * (n / kSmallTile) < ((int64_t)1 << 31);
+  const int64_t groups = tiled && n % (kSmallTile * kPhasedTiles) == 0 ? nb * (m / kSmallTile) * (n / (kSmallTile * kPhasedTiles)) : 0;
+  if (AFIR_TRANSPOSE_PHASED && !block_dim && groups >= (int64_t)device_cus() * kPhasedMinGroupsPerCU &&
+      groups * kThreads <= (int64_t)device_cus() * kPhasedLanesPerCU && (int64_t)32 * m * 2 < ((int64_t)1 << 31) &&
+      phased_enabled()) {
+    const int hold_ticks = phase_hold_ticks(nb * m * n * 2, AFIR_TRANSPOSE_PHASE_BASE_NS, AFIR_TRANSPOSE_PHASE_GBS);
+    hipLaunchKernelGGL(relu_bcast_add_transpose_f16_phased, dim3((unsigned)groups), dim3(kThreads), 0, stream,
+                       x, c, out, (int)nb, (int)m, (int)n, hold_ticks);
+  } else if (tiled) {
     // one tile per workgroup: the hardware deals workgroups out as slots free up, which balances
     // better than walks of several tiles (8192 workgroups of one tile 19.7 us on [64, 1024, 512],
     // 4096 of two 20.4, 2731 of three 20.9; a grid given by the caller makes a workgroup walk,

@@ -178,6 +178,24 @@ def test_c3_special_values(H):
     assert out[ok].tobytes() == want[ok].tobytes()
 
 
+# Shapes of whole 64 x 256 tile groups between 24 and 64 MiB take the kernel that separates the
+# chip's reads from its writes in time; AFIR_HIP_PHASED=0 keeps a launch on the other kernel.
+@pytest.mark.parametrize("b,m,n", [(12, 1024, 1024), (3, 4096, 1024), (40, 512, 768), (64, 512, 1024)])
+def test_c3_phased_route_bit_exact(H, b, m, n, monkeypatch):
+    x, c = O.gen_c3(b, m, n)
+    x[0, 0, :8] = [np.nan, -np.inf, np.inf, -0.0, 6e-8, -6e-8, 65504, -65504]
+    x[-1, -1, -4:] = [np.nan, -0.0, 65504, -1.0]
+    c[3] = -0.0
+    with np.errstate(all="ignore"):
+        want = O.golden_c3(x, c)
+    ok = ~np.isnan(want)
+    for phased in ("1", "0"):
+        monkeypatch.setenv("AFIR_HIP_PHASED", phased)
+        out = H.relu_broadcast_add_transpose(dev(x), dev(c)).cpu().numpy()
+        assert np.array_equal(np.isnan(out), np.isnan(want))
+        assert out[ok].tobytes() == want[ok].tobytes()
+
+
 # ---------------------------------------------------------------- C4 --------
 
 @pytest.mark.parametrize("rows,dim,nidx", [(512, 64, 256), (1000, 1024, 513), (100, 136, 77),
