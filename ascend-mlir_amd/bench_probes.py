@@ -26,6 +26,8 @@ def load():
                        ("afir_bench_matmul_ablated", [vp, vp, vp, vp, vp, ctypes.c_int, ctypes.c_int,
                                                       ctypes.c_int, ctypes.c_int]),
                        ("afir_bench_copy", [vp, vp, vp, ctypes.c_size_t]),
+                       ("afir_bench_copy_phased", [vp, vp, vp, ctypes.c_size_t]),
+                       ("afir_bench_fill", [vp, vp, ctypes.c_size_t, u32]),
                        ("afir_bench_read", [vp, vp, vp, ctypes.c_size_t]),
                        ("afir_bench_tilecopy64", [vp, vp, vp, ctypes.c_int, ctypes.c_int, ctypes.c_int])]:
         fn = getattr(L, name)

@@ -53,6 +53,18 @@ uint32_t afir_bench_matmul_ablated(void *stream, const void *a, const void *b, c
  * ordinary stores 5.5-5.7).  bytes must be a multiple of 16384. */
 uint32_t afir_bench_copy(void *stream, const void *src, void *dst, size_t bytes);
 
+/* Write-only stream: every lane stores a value of its own (128-bit non-temporal
+ * stores, grid-strided).  bytes must be a multiple of 16384. */
+uint32_t afir_bench_fill(void *stream, void *dst, size_t bytes, uint32_t seed);
+
+/* The copy with the chip's reads and writes separated in time, the way the
+ * one-shot gather and transpose kernels do it: every lane of the launch is
+ * resident at once (2048 lanes per CU, eight 16-byte chunks each, so at most
+ * 64 MiB on 256 CUs), requests all its chunks, and holds its stores back until
+ * the real-time counter says the chip's reads have been served (300 ns + bytes
+ * at 6.7 TB/s after the workgroup's start).  bytes must be a multiple of 32768. */
+uint32_t afir_bench_copy_phased(void *stream, const void *src, void *dst, size_t bytes);
+
 /* Read-only stream: every lane sums what it loads (128-bit non-temporal loads)
  * and one float per workgroup goes to `sink` (>= 8192 floats). */
 uint32_t afir_bench_read(void *stream, const void *src, void *sink, size_t bytes);

@@ -129,6 +129,34 @@ __global__ __launch_bounds__(kCopyThreads) void probe_tilecopy64(const uint16_t 
   }
 }
 
+// write-only stream: every lane stores a value of its own
+__global__ __launch_bounds__(kCopyThreads) void probe_fill(u32x4 *__restrict__ dst, size_t n16, uint32_t seed) {
+  const size_t chunk = (size_t)kCopyThreads * kCopyUnroll, stride = (size_t)gridDim.x * chunk;
+  const u32x4 v = {seed, threadIdx.x, blockIdx.x, seed * 3u};
+  for (size_t base = (size_t)blockIdx.x * chunk; base < n16; base += stride) {
+#pragma unroll
+    for (int u = 0; u < kCopyUnroll; ++u) afir::store_nt(dst + base + u * kCopyThreads + threadIdx.x, v);
+  }
+}
+
+// the copy with every lane resident at once (eight 16-byte chunks per lane) and the stores held
+// back until `hold_ticks` of the real-time counter after the workgroup's start
+constexpr int kPhasedChunks = 8;
+__global__ __launch_bounds__(kCopyThreads, 8) void probe_copy_phased(const u32x4 *__restrict__ src,
+                                                                     u32x4 *__restrict__ dst, int hold_ticks) {
+  const long long t_start = wall_clock64();
+  const size_t base = (size_t)blockIdx.x * (kCopyThreads * kPhasedChunks) + threadIdx.x;
+  u32x4 v[kPhasedChunks];
+#pragma unroll
+  for (int u = 0; u < kPhasedChunks; ++u) v[u] = afir::load_nt(src + base + u * kCopyThreads);
+#pragma unroll
+  for (int u = 0; u < kPhasedChunks; ++u) asm volatile("" : "+v"(v[u]));
+  for (int spin = 0; spin < afir::kPhaseSpinLimit && wall_clock64() - t_start < hold_ticks; ++spin)
+    __builtin_amdgcn_s_sleep(1);
+#pragma unroll
+  for (int u = 0; u < kPhasedChunks; ++u) afir::store_nt(dst + base + u * kCopyThreads, v[u]);
+}
+
 uint32_t done() { return hipGetLastError() == hipSuccess ? 0u : 2u; }
 
 }  // namespace
@@ -164,6 +192,25 @@ uint32_t afir_bench_copy(void *stream, const void *src, void *dst, size_t bytes)
   if (!src || !dst || bytes == 0 || bytes % 16384 != 0 || !afir::aligned16(src) || !afir::aligned16(dst)) return 1u;
   hipLaunchKernelGGL(probe_copy, dim3(4u * kNumCU), dim3(kCopyThreads), 0, static_cast<hipStream_t>(stream),
                      static_cast<const u32x4 *>(src), static_cast<u32x4 *>(dst), bytes / 16);
+  return done();
+}
+
+uint32_t afir_bench_fill(void *stream, void *dst, size_t bytes, uint32_t seed) {
+  if (!dst || bytes == 0 || bytes % 16384 != 0 || !afir::aligned16(dst)) return 1u;
+  hipLaunchKernelGGL(probe_fill, dim3(8u * kNumCU), dim3(kCopyThreads), 0, static_cast<hipStream_t>(stream),
+                     static_cast<u32x4 *>(dst), bytes / 16, seed);
+  return done();
+}
+
+uint32_t afir_bench_copy_phased(void *stream, const void *src, void *dst, size_t bytes) {
+  const size_t per_block = (size_t)kCopyThreads * kPhasedChunks * 16;
+  if (!src || !dst || bytes == 0 || bytes % per_block != 0 || !afir::aligned16(src) || !afir::aligned16(dst)) return 1u;
+  // (every lane resident at once: 2048 lanes per CU)
+  if (bytes / per_block * kCopyThreads > (size_t)afir::device_cus() * 2048) return 1u;
+  const int hold_ticks = afir::phase_hold_ticks((int64_t)bytes, 300, 6700);
+  hipLaunchKernelGGL(probe_copy_phased, dim3((unsigned)(bytes / per_block)), dim3(kCopyThreads), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const u32x4 *>(src), static_cast<u32x4 *>(dst),
+                     hold_ticks);
   return done();
 }
 

@@ -6,12 +6,13 @@
 // golden style examples/gather-elementwise-fusion/gen_data.py:62-67: f32
 // arithmetic, one round-to-nearest-even to f16).
 //
-// HBM-bound: each gathered row is read once and written once.  A lane owns one
-// 16-byte column chunk for the whole launch, so its eight scale and shift
-// values live in registers as f32.  A wave covers 1 KiB of a row per load;
-// kRowsInFlight rows are fetched before the first is used, and the row index
-// of each is wave-uniform.  The product of two f16 values is exact in f32, so
-// the fused multiply-add rounds exactly like the unfused golden.
+// HBM-bound: each gathered row is read once and written once.  Four kernels, picked by the
+// launcher: rows of 32 * 2^k halves that fit the chip at once take the kernel that separates
+// the chip's reads from its writes in time (gather_scale_shift_f16_phased), larger launches of
+// such rows the grouped kernel, other 16-byte aligned rows the kernel in which a lane owns one
+// column chunk for the whole launch (gather_scale_shift_f16_vec), anything else the element
+// kernel.  The product of two f16 values is exact in f32, so the fused multiply-add they share
+// rounds exactly like the unfused golden.
 #include "kernels.h"
 
 namespace afir {
@@ -224,10 +225,10 @@ __global__ __launch_bounds__(kGroupedThreads) void gather_scale_shift_f16_groupe
 #define AFIR_GATHER_PHASED 1
 #endif
 #ifndef AFIR_GATHER_PHASED_THREADS
-#define AFIR_GATHER_PHASED_THREADS 256
+#define AFIR_GATHER_PHASED_THREADS 512
 #endif
 #ifndef AFIR_GATHER_PHASE_GBS
-#define AFIR_GATHER_PHASE_GBS 6900
+#define AFIR_GATHER_PHASE_GBS 6700
 #endif
 #ifndef AFIR_GATHER_PHASE_BASE_NS
 #define AFIR_GATHER_PHASE_BASE_NS 300

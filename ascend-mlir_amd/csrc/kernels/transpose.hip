@@ -138,7 +138,7 @@ __global__ __launch_bounds__(kThreads) void relu_bcast_add_transpose_f16_tile64(
 #define AFIR_TRANSPOSE_PHASED 1
 #endif
 #ifndef AFIR_TRANSPOSE_PHASE_GBS
-#define AFIR_TRANSPOSE_PHASE_GBS 6900
+#define AFIR_TRANSPOSE_PHASE_GBS 6700
 #endif
 #ifndef AFIR_TRANSPOSE_PHASE_BASE_NS
 #define AFIR_TRANSPOSE_PHASE_BASE_NS 300

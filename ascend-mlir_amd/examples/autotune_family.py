@@ -8,7 +8,7 @@ builds the kernel library once per combination of the build_<MACRO> parameters
 in the family's tiling_space.json, launches and validates every candidate and
 scores it by kernel time.
 
-    autotune_family.py eltwise|rowsum|transpose-family|gather|matmul [--out DIR] [--repeats N]
+    autotune_family.py eltwise|rowsum|transpose-family|gather|matmul [--out DIR] [--repeats N] [--space FILE]
 
 Needs a GPU and hipcc.  Prints the autotuner's candidate table; best_config.json
 is left in DIR."""
@@ -85,12 +85,15 @@ def main():
     ap.add_argument("family", choices=["eltwise", "rowsum", "transpose-family", "gather", "matmul"])
     ap.add_argument("--out", default=None)
     ap.add_argument("--repeats", default="200")
+    ap.add_argument("--space", default="tiling_space.json",
+                    help="file in the family's directory (tiling_space_unphased.json: the gather / transpose "
+                         "kernels that do not separate reads from writes)")
     args = ap.parse_args()
     out = args.out or f"/tmp/autotune-{args.family}"
     os.makedirs(out, exist_ok=True)
     inputs, atol, rtol = generate(args.family, out)
     here = os.path.join(HERE, "autotune-" + args.family)
-    cmd = [os.path.join(HERE, "..", "bin", "autotuner"), "--space", os.path.join(here, "tiling_space.json"),
+    cmd = [os.path.join(HERE, "..", "bin", "autotuner"), "--space", os.path.join(here, args.space),
            "--kernel", os.path.join(here, "kernel.region"),
            "--inputs", ",".join(os.path.join(out, n + ".npy") for n in inputs),
            "--expected", os.path.join(out, "expected.npy"), "--atol", atol, "--rtol", rtol,

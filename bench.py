@@ -50,8 +50,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 MEASURED_TRAFFIC = {
     "c1": (201357516, "profiles/add_mul_f32_vec__c1_4096x4096.txt"),
     "c2": (134633062, "profiles/bcast_add_rowsum_f32_wgrow__c2_8192x4096.txt"),
-    "c3": (134292992, "profiles/relu_bcast_add_transpose_f16_tile64__c3_64x1024x512.txt"),
-    "c4": (133786214, "profiles/gather_scale_shift_f16_grouped__c4_131072x1024_idx32768.txt"),
+    "c3": (134392320, "profiles/relu_bcast_add_transpose_f16_phased__c3_64x1024x512.txt"),
+    "c4": (133753344, "profiles/gather_scale_shift_f16_phased__c4_131072x1024_idx32768.txt"),
     "c5": (1804635136, "profiles/matmul_bias_leakyrelu_dma__c5_8192x8192x8192.txt"),
     "g1": (201367040, "profiles/afir_region_s0_i32_a__g1_compiled_add_mul_f32_4096x4096.txt"),
     "g2": (134618931, "profiles/afir_region_all_i32_a__g2_compiled_split_relu_brc_f16_8192x4096.txt"),
@@ -63,7 +63,8 @@ MEASURED_TRAFFIC = {
 
 # north_star targets, read on roofline.frac (algorithmic work / event-timed launch duration / published peak)
 TARGETS = {"c1": 0.70, "c2": 0.70, "c3": 0.70, "c4": 0.70, "c5": 0.60}
-ALL_WORKLOADS = ["c1", "c2", "c3", "c4", "c5", "g1", "g2", "g3", "g4", "i1", "i2", "ceil_copy", "ceil_read", "ceil_tilecopy64"]
+CEILINGS = ["ceil_copy", "ceil_copy_phased", "ceil_read", "ceil_write", "ceil_tilecopy64"]
+ALL_WORKLOADS = ["c1", "c2", "c3", "c4", "c5", "g1", "g2", "g3", "g4", "i1", "i2"] + CEILINGS
 
 # Region programs of the two generic-kernel workloads (grammar:
 # ascend-mlir_amd/csrc/target/region_program.h)
@@ -529,14 +530,16 @@ def make_workload(key, torch, H, O, C):
             return w.work() / dt / 1e9, "full workload, numpy region oracle (1 thread), one run"
         w.cpu = cpu
         w.cpu_cores = 1
-    elif key in ("ceil_copy", "ceil_read", "ceil_tilecopy64"):
+    elif key in CEILINGS:
         # Measured ceilings (probe kernels of libafir_bench_probes.so, csrc/bench/probes.h): what
-        # this chip sustains on a plain copy, on a read-only stream and on the address pattern of
-        # c3's tiled transpose with the transposition left out.  No oracle: nothing is computed.
+        # this chip sustains on a plain copy, on a copy whose reads and writes are separated in time
+        # (what the one-shot kernels of c3 and c4 do), on a read-only and a write-only stream, and on
+        # the address pattern of c3's other kernel with the transposition left out.  No oracle:
+        # nothing is computed.
         from ascend_mlir_amd import bench_probes as P
         # 128 MiB for the read-only stream: as long a launch as the copies' (a 10 us launch would
         # measure the host's launch rate)
-        nbytes = (128 << 20) if key == "ceil_read" else (64 << 20)
+        nbytes = (128 << 20) if key in ("ceil_read", "ceil_write") else (64 << 20)
         w.dtype = "u8"
         w.nsets = sets_for(nbytes)
         w.no_cpu = True
@@ -549,6 +552,27 @@ def make_workload(key, torch, H, O, C):
             w.sets = list(zip(srcs, dsts))
             w.parity = lambda: {"bar": "dst == src", "passed": bool(torch.equal(srcs[0], dsts[0])),
                                 "mismatches": int((srcs[0] != dsts[0]).sum().item())}
+        elif key == "ceil_copy_phased":
+            w.title = ("ceil_copy_phased: 64 MiB -> 64 MiB with every lane resident at once and the stores held "
+                       "back until the chip's reads have been served (probe, no arithmetic)")
+            dsts = [torch.empty_like(x) for x in srcs]
+            w.work = lambda: 2 * nbytes
+            w.launches = [P.prepare("afir_bench_copy_phased", a.data_ptr(), b.data_ptr(), nbytes)
+                          for a, b in zip(srcs, dsts)]
+            w.sets = list(zip(srcs, dsts))
+            w.parity = lambda: {"bar": "dst == src", "passed": bool(torch.equal(srcs[0], dsts[0])),
+                                "mismatches": int((srcs[0] != dsts[0]).sum().item())}
+        elif key == "ceil_write":
+            w.title = "ceil_write: 128 MiB write-only stream, 128-bit non-temporal stores (probe)"
+            w.work = lambda: nbytes
+            w.launches = [P.prepare("afir_bench_fill", a.data_ptr(), nbytes, 7 + i) for i, a in enumerate(srcs)]
+            w.sets = [(a,) for a in srcs]
+
+            def parity():
+                words = srcs[0].view(torch.int32).view(-1, 4)
+                ok = bool((words[:, 0] == 7).all().item()) and bool((words[:, 3] == 21).all().item())
+                return {"bar": "every chunk holds the launch's seed", "passed": ok, "mismatches": 0 if ok else 1}
+            w.parity = parity
         elif key == "ceil_read":
             w.title = "ceil_read: 128 MiB read-only stream, 128-bit non-temporal loads (probe)"
             sink = torch.zeros(8192, dtype=torch.float32, device="cuda")
@@ -735,7 +759,7 @@ def main():
                            for k, t in TARGETS.items() if k in by_key}
         line["min_frac_hbm"] = min(v["frac"] for k, v in line["targets"].items() if k != "c5")
         line["targets_read_on"] = "roofline.frac (HIP events on the launch stream), not value (wall clock)"
-        ceil = {k: by_key[k]["roofline"]["achieved"] for k in ("ceil_copy", "ceil_read", "ceil_tilecopy64")
+        ceil = {k: by_key[k]["roofline"]["achieved"] for k in CEILINGS
                 if k in by_key}
         if ceil:
             line["measured_ceilings_gbs"] = ceil
