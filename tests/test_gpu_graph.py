@@ -75,3 +75,55 @@ def test_kernels_replay_from_a_captured_graph(H, tmp_path, monkeypatch):
     assert bool(torch.isfinite(total.half()).all()) and torch.equal(sums, total.half())
     elementwise.close()
     row_sum.close()
+
+
+def test_phased_kernels_replay_from_a_captured_graph(H):
+    """The gather and the transpose on the kernels that hold their stores back by the device's
+    real-time counter (the gather with rows left over: a second launch of the other kernel),
+    captured together: the hold lives inside the kernels, so replays behave like eager launches."""
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    rows, dim, nidx = 5000, 1024, 4099
+    table = torch.randn((rows, dim), generator=gen, device="cuda").half()
+    scale = torch.randn((dim,), generator=gen, device="cuda").half()
+    shift = torch.randn((dim,), generator=gen, device="cuda").half()
+    idx = torch.randint(0, rows, (nidx,), generator=gen, device="cuda", dtype=torch.int32)
+    gathered = torch.empty((nidx, dim), dtype=torch.float16, device="cuda")
+    b, m, n = 12, 1024, 1024
+    x = torch.randn((b, m, n), generator=gen, device="cuda").half()
+    c = torch.randn((n,), generator=gen, device="cuda").half()
+    xt = torch.empty((b, n, m), dtype=torch.float16, device="cuda")
+
+    def launches():
+        return [
+            H.prepare("afir_hip_launch_gather_scale_shift",
+                      [table.data_ptr(), idx.data_ptr(), scale.data_ptr(), shift.data_ptr(), gathered.data_ptr(), 0],
+                      H.pack_tiling(rows, dim, nidx)),
+            H.prepare("afir_hip_launch_relu_broadcast_add_transpose", [x.data_ptr(), c.data_ptr(), xt.data_ptr(), 0],
+                      H.pack_tiling(b, m, n)),
+        ]
+
+    def eager():
+        for call in launches():
+            call()
+        torch.cuda.synchronize()
+        return gathered.clone(), xt.clone()
+
+    eager()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for call in launches():
+            call()
+    for replay in range(3):
+        idx.copy_(torch.randint(0, rows, (nidx,), generator=gen, device="cuda", dtype=torch.int32))
+        x.copy_(torch.randn((b, m, n), generator=gen, device="cuda").half())
+        want = eager()
+        gathered.fill_(7)
+        xt.fill_(7)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, expected, what in zip((gathered, xt), want, ("gather", "transpose")):
+            assert torch.equal(got, expected), (replay, what)
+    # f32 multiply and add (the product of two halves is exact in f32), one rounding to f16
+    assert torch.equal(gathered, (table[idx.long()].float() * scale.float() + shift.float()).half())
+    assert torch.equal(xt, (torch.relu(x.float()) + c.float()).half().transpose(1, 2))
