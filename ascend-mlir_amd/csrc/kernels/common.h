@@ -58,6 +58,25 @@ inline int phase_hold_ticks(int64_t read_bytes, int base_ns, int gb_per_s) {
   return ticks > (double)kPhaseHoldMaxTicks ? kPhaseHoldMaxTicks : (int)ticks;
 }
 
+// The hold of one workgroup of a phased launch, called once its own loads have arrived.  The
+// chip serves the loads of a one-wave launch in the order of its workgroups (measured: the time
+// from a workgroup's start to its last load grows linearly with blockIdx.x, 1.8 us for the first
+// eighth of a 64 MiB copy, 8.7 us for the last), so a workgroup can tell from its own wait and its
+// place in the launch when the last workgroup's loads will be back: latency + (wait - latency)
+// * workgroups / (place + 1).  That estimate is too noisy to replace the formula (8 % for the
+// late workgroups, more for the early ones, where 5 % cost 2 %), but it shows when the reads run
+// much faster than the formula assumes (rows that repeat and come out of the caches, an input
+// that still sits in the last-level cache): below the fraction `below` of the formula's hold the
+// estimate is used.  (With indices spread over the table, fractions from 0.5 to 0.8 measured the
+// same as never using it; the kernels ship 0.7.)
+constexpr int kPhaseLatencyTicks = 80;    // under every measured wait for a first load (0.9 us)
+__device__ __forceinline__ int phase_hold_here(int hold_ticks, long long t_start, float below) {
+  const int waited = (int)(wall_clock64() - t_start);
+  const float over = waited > kPhaseLatencyTicks ? (float)(waited - kPhaseLatencyTicks) : 0.f;
+  const float estimate = (float)kPhaseLatencyTicks + over * (float)gridDim.x / (float)(blockIdx.x + 1u);
+  return estimate < below * (float)hold_ticks ? (int)estimate : hold_ticks;
+}
+
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));

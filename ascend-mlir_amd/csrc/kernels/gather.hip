@@ -224,11 +224,16 @@ __global__ __launch_bounds__(kGroupedThreads) void gather_scale_shift_f16_groupe
 #ifndef AFIR_GATHER_PHASED
 #define AFIR_GATHER_PHASED 1
 #endif
+// a workgroup whose own loads came back so early that its place in the launch predicts the end of
+// the chip's reads before this percentage of the hold cuts the hold short (phase_hold_here; 0: never)
+#ifndef AFIR_PHASE_ESTIMATE
+#define AFIR_PHASE_ESTIMATE 70
+#endif
 #ifndef AFIR_GATHER_PHASED_THREADS
-#define AFIR_GATHER_PHASED_THREADS 512
+#define AFIR_GATHER_PHASED_THREADS 256
 #endif
 #ifndef AFIR_GATHER_PHASE_GBS
-#define AFIR_GATHER_PHASE_GBS 6700
+#define AFIR_GATHER_PHASE_GBS 6500
 #endif
 #ifndef AFIR_GATHER_PHASE_BASE_NS
 #define AFIR_GATHER_PHASE_BASE_NS 300
@@ -276,6 +281,9 @@ __global__ __launch_bounds__(kPhasedThreads, 8) void gather_scale_shift_f16_phas
 #pragma unroll
     for (int u = 0; u < kGroups; ++u) asm volatile("" : "+v"(v[p][u]));
   __syncthreads();
+#if AFIR_PHASE_ESTIMATE
+  hold_ticks = phase_hold_here(hold_ticks, t_start, AFIR_PHASE_ESTIMATE * 0.01f);
+#endif
   for (int spin = 0; spin < kPhaseSpinLimit && wall_clock64() - t_start < hold_ticks; ++spin)
     __builtin_amdgcn_s_sleep(1);
 

@@ -137,8 +137,13 @@ __global__ __launch_bounds__(kThreads) void relu_bcast_add_transpose_f16_tile64(
 #ifndef AFIR_TRANSPOSE_PHASED
 #define AFIR_TRANSPOSE_PHASED 1
 #endif
+// a workgroup whose own loads came back so early that its place in the launch predicts the end of
+// the chip's reads before this percentage of the hold cuts the hold short (phase_hold_here; 0: never)
+#ifndef AFIR_PHASE_ESTIMATE
+#define AFIR_PHASE_ESTIMATE 70
+#endif
 #ifndef AFIR_TRANSPOSE_PHASE_GBS
-#define AFIR_TRANSPOSE_PHASE_GBS 6700
+#define AFIR_TRANSPOSE_PHASE_GBS 6900
 #endif
 #ifndef AFIR_TRANSPOSE_PHASE_BASE_NS
 #define AFIR_TRANSPOSE_PHASE_BASE_NS 300
@@ -196,6 +201,9 @@ __global__ __launch_bounds__(kThreads, 8) void relu_bcast_add_transpose_f16_phas
   for (int q = 0; q < kPhasedTiles; ++q)
 #pragma unroll
     for (int k = 0; k < 2; ++k) asm volatile("" : "+v"(v[q][k]));
+#if AFIR_PHASE_ESTIMATE
+  hold_ticks = phase_hold_here(hold_ticks, t_start, AFIR_PHASE_ESTIMATE * 0.01f);
+#endif
   for (int spin = 0; spin < kPhaseSpinLimit && wall_clock64() - t_start < hold_ticks; ++spin)
     __builtin_amdgcn_s_sleep(1);
   // stores: a base per (tile, pass) that is the same for the whole workgroup (scalar registers)
