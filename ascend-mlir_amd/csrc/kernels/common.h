@@ -63,12 +63,14 @@ inline int phase_hold_ticks(int64_t read_bytes, int base_ns, int gb_per_s) {
 // from a workgroup's start to its last load grows linearly with blockIdx.x, 1.8 us for the first
 // eighth of a 64 MiB copy, 8.7 us for the last), so a workgroup can tell from its own wait and its
 // place in the launch when the last workgroup's loads will be back: latency + (wait - latency)
-// * workgroups / (place + 1).  That estimate is too noisy to replace the formula (8 % for the
-// late workgroups, more for the early ones, where 5 % cost 2 %), but it shows when the reads run
-// much faster than the formula assumes (rows that repeat and come out of the caches, an input
-// that still sits in the last-level cache): below the fraction `below` of the formula's hold the
-// estimate is used.  (With indices spread over the table, fractions from 0.5 to 0.8 measured the
-// same as never using it; the kernels ship 0.7.)
+// * workgroups / (place + 1).  Alone that estimate is a poor hold (it overshoots for the early
+// workgroups, whose small waits it multiplies most: 0.64-0.66 of peak against 0.75-0.78), but it
+// is a good lower cut of the formula's: it falls under it when the reads run faster than the
+// formula assumes (rows that repeat and come out of the caches, an input that still sits in the
+// last-level cache), and then the workgroup waits only that long.  `below` is the fraction of the
+// formula's hold under which the estimate is taken: with indices spread over the table every
+// fraction from 0 (never) to 1 measures the same; with repeating rows 1 is the fastest (32768
+// indices over 2048 rows: 23.2 us never, 17.0 at 1; the kernel without a hold 16.0).
 constexpr int kPhaseLatencyTicks = 80;    // under every measured wait for a first load (0.9 us)
 __device__ __forceinline__ int phase_hold_here(int hold_ticks, long long t_start, float below) {
   const int waited = (int)(wall_clock64() - t_start);

@@ -218,16 +218,19 @@ __global__ __launch_bounds__(kGroupedThreads) void gather_scale_shift_f16_groupe
 // stores are the same whenever they leave.  Measured on the 32768 x 1024 gather: 23.9 -> 21.6 us;
 // on 24576 rows 20.5 -> 16.4, 8192 rows 8.6 -> 6.4.  The hold that measured best is the time the
 // gathered bytes take at AFIR_GATHER_PHASE_GBS plus AFIR_GATHER_PHASE_BASE_NS, for 8192 to 32768
-// rows alike (half a microsecond either side costs 2 %).  It is tuned for indices spread over
-// the table: when most of the gathered rows come out of the caches (2048 distinct rows in 32768
-// indices) the reads end early, the hold is too long and the launch takes 21 us instead of 15.
+// rows alike (a third of a microsecond either side costs 1 %).  The formula assumes rows that come
+// from HBM; when they repeat and come out of the caches the reads end early, and a workgroup
+// that sees its own loads back ahead of its place in the launch cuts its hold short
+// (phase_hold_here in common.h): 32768 indices over 2048 distinct rows 17.0 us (23.2 without
+// the cut, 16.0 on the kernel without a hold).
 #ifndef AFIR_GATHER_PHASED
 #define AFIR_GATHER_PHASED 1
 #endif
 // a workgroup whose own loads came back so early that its place in the launch predicts the end of
-// the chip's reads before this percentage of the hold cuts the hold short (phase_hold_here; 0: never)
+// the chip's reads before this percentage of the formula's hold waits only until then
+// (phase_hold_here; 100: the shorter of the two, 0: always the formula)
 #ifndef AFIR_PHASE_ESTIMATE
-#define AFIR_PHASE_ESTIMATE 70
+#define AFIR_PHASE_ESTIMATE 100
 #endif
 #ifndef AFIR_GATHER_PHASED_THREADS
 #define AFIR_GATHER_PHASED_THREADS 256

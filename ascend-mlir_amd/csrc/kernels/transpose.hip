@@ -138,9 +138,10 @@ __global__ __launch_bounds__(kThreads) void relu_bcast_add_transpose_f16_tile64(
 #define AFIR_TRANSPOSE_PHASED 1
 #endif
 // a workgroup whose own loads came back so early that its place in the launch predicts the end of
-// the chip's reads before this percentage of the hold cuts the hold short (phase_hold_here; 0: never)
+// the chip's reads before this percentage of the formula's hold waits only until then
+// (phase_hold_here; 100: the shorter of the two, 0: always the formula)
 #ifndef AFIR_PHASE_ESTIMATE
-#define AFIR_PHASE_ESTIMATE 70
+#define AFIR_PHASE_ESTIMATE 100
 #endif
 #ifndef AFIR_TRANSPOSE_PHASE_GBS
 #define AFIR_TRANSPOSE_PHASE_GBS 6900
