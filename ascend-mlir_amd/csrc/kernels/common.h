@@ -50,6 +50,12 @@ inline int wall_clock_khz() {
   }();
   return khz;
 }
+// A shape beyond the chip's resident lanes goes out as two phased launches of about equal size
+// (the end of the first and the start of the second separate its writes from the other's reads):
+// 3-7 % ahead of the unphased kernels at 96-128 MiB.  From three launches on the gaps between
+// them cost what the separation gains (a 195 MiB gather: 3 % behind), so those shapes stay on
+// the unphased kernels.
+constexpr int kPhaseMaxLaunches = 2;
 constexpr int kPhaseHoldMaxTicks = 1 << 14;      // ~164 us at 100 MHz: no launch waits longer than this
 constexpr int kPhaseSpinLimit = 1 << 15;         // polls of the counter, whatever it reads
 inline int phase_hold_ticks(int64_t read_bytes, int base_ns, int gb_per_s) {

@@ -7,9 +7,9 @@
 // arithmetic, one round-to-nearest-even to f16).
 //
 // HBM-bound: each gathered row is read once and written once.  Four kernels, picked by the
-// launcher: rows of 32 * 2^k halves that fit the chip at once take the kernel that separates
-// the chip's reads from its writes in time (gather_scale_shift_f16_phased), larger launches of
-// such rows the grouped kernel, other 16-byte aligned rows the kernel in which a lane owns one
+// launcher: rows of 32 * 2^k halves, up to twice what fits the chip at once, take the kernel that
+// separates the chip's reads from its writes in time (gather_scale_shift_f16_phased), larger
+// launches of such rows the grouped kernel, other 16-byte aligned rows the kernel in which a lane owns one
 // column chunk for the whole launch (gather_scale_shift_f16_vec), anything else the element
 // kernel.  The product of two f16 values is exact in f32, so the fused multiply-add they share
 // rounds exactly like the unfused golden.
@@ -358,17 +358,27 @@ LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx
   const int64_t chunks64 = dim / 8;
   int lanes_log2 = 0;
   while (lanes_log2 < 8 && ((int64_t)kGroups << lanes_log2) < chunks64) ++lanes_log2;
-  // whole blocks of a gather that fits the chip at once: the phased kernel; rows left over: below
+  // Whole blocks of rows go to the phased kernel, which wants every lane of a launch resident at
+  // once: a gather of up to twice that goes out as two launches (kPhaseMaxLaunches).  Rows left
+  // over, and larger gathers: below.
   const int64_t phased_rows_per_block = (int64_t)(kPhasedThreads >> (lanes_log2 < 8 ? lanes_log2 : 8)) * kPhasedPasses;
   const int64_t phased_blocks = nidx / phased_rows_per_block;
   if (AFIR_GATHER_PHASED && vec && ((int64_t)kGroups << lanes_log2) == chunks64 && !block_dim &&
       (1 << lanes_log2) <= kPhasedThreads && phased_blocks > 0 &&
-      phased_blocks * kPhasedThreads <= (int64_t)device_cus() * kPhasedLanesPerCU && phased_enabled()) {
+      phased_blocks <= kPhaseMaxLaunches * ((int64_t)device_cus() * kPhasedLanesPerCU / kPhasedThreads) && phased_enabled()) {
     const size_t lds = (size_t)2 * (kGroups << lanes_log2) * 16;   // scale and shift, 16-byte chunks
-    const int hold_ticks = phase_hold_ticks(phased_blocks * phased_rows_per_block * dim * 2,
-                                            AFIR_GATHER_PHASE_BASE_NS, AFIR_GATHER_PHASE_GBS);
-    hipLaunchKernelGGL(gather_scale_shift_f16_phased, dim3((unsigned)phased_blocks), dim3(kPhasedThreads), lds,
-                       stream, table, idx, scale, shift, out, error_flag, (uint32_t)rows, lanes_log2, hold_ticks);
+    const int64_t capacity = (int64_t)device_cus() * kPhasedLanesPerCU / kPhasedThreads;   // blocks per launch
+    const int64_t launches = (phased_blocks + capacity - 1) / capacity;
+    const int64_t take = (phased_blocks + launches - 1) / launches;
+    for (int64_t b0 = 0; b0 < phased_blocks; b0 += take) {
+      const int64_t nblocks = phased_blocks - b0 < take ? phased_blocks - b0 : take;
+      const int64_t row0 = b0 * phased_rows_per_block;
+      const int hold_ticks = phase_hold_ticks(nblocks * phased_rows_per_block * dim * 2, AFIR_GATHER_PHASE_BASE_NS,
+                                              AFIR_GATHER_PHASE_GBS);
+      hipLaunchKernelGGL(gather_scale_shift_f16_phased, dim3((unsigned)nblocks), dim3(kPhasedThreads), lds, stream,
+                         table, idx + row0, scale, shift, out + row0 * dim, error_flag, (uint32_t)rows, lanes_log2,
+                         hold_ticks);
+    }
     const int64_t done = phased_blocks * phased_rows_per_block;
     if (done == nidx) return after_launch();
     idx += done;

@@ -267,13 +267,22 @@ LaunchStatus launch_relu_broadcast_add_transpose(const uint16_t *x, const uint16
 
   const bool tiled = (m % kSmallTile == 0) && (n % kSmallTile == 0) && aligned16(x) && aligned16(c) && aligned16(out) &&
                      nb * (m / kSmallTile) * (n / kSmallTile) < ((int64_t)1 << 31);
-  const int64_t groups = tiled && n % (kSmallTile * kPhasedTiles) == 0 ? nb * (m / kSmallTile) * (n / (kSmallTile * kPhasedTiles)) : 0;
-  if (AFIR_TRANSPOSE_PHASED && !block_dim && groups >= (int64_t)device_cus() * kPhasedMinGroupsPerCU &&
-      groups * kThreads <= (int64_t)device_cus() * kPhasedLanesPerCU && (int64_t)32 * m * 2 < ((int64_t)1 << 31) &&
-      phased_enabled()) {
-    const int hold_ticks = phase_hold_ticks(nb * m * n * 2, AFIR_TRANSPOSE_PHASE_BASE_NS, AFIR_TRANSPOSE_PHASE_GBS);
-    hipLaunchKernelGGL(relu_bcast_add_transpose_f16_phased, dim3((unsigned)groups), dim3(kThreads), 0, stream,
-                       x, c, out, (int)nb, (int)m, (int)n, hold_ticks);
+  // The phased kernel wants every lane of a launch resident at once: a shape of up to twice that
+  // goes out as two launches of whole batches (kPhaseMaxLaunches).
+  const int64_t groups_per_batch = tiled && n % (kSmallTile * kPhasedTiles) == 0 ? (m / kSmallTile) * (n / (kSmallTile * kPhasedTiles)) : 0;
+  const int64_t capacity = (int64_t)device_cus() * kPhasedLanesPerCU / kThreads;   // groups per launch
+  if (AFIR_TRANSPOSE_PHASED && !block_dim && groups_per_batch > 0 && groups_per_batch <= capacity &&
+      nb * groups_per_batch >= (int64_t)device_cus() * kPhasedMinGroupsPerCU && (int64_t)32 * m * 2 < ((int64_t)1 << 31) &&
+      (nb + capacity / groups_per_batch - 1) / (capacity / groups_per_batch) <= kPhaseMaxLaunches && phased_enabled()) {
+    const int64_t batches_per_launch = capacity / groups_per_batch;
+    const int64_t launches = (nb + batches_per_launch - 1) / batches_per_launch;
+    const int64_t take = (nb + launches - 1) / launches;
+    for (int64_t b0 = 0; b0 < nb; b0 += take) {
+      const int64_t nbl = nb - b0 < take ? nb - b0 : take;
+      const int hold_ticks = phase_hold_ticks(nbl * m * n * 2, AFIR_TRANSPOSE_PHASE_BASE_NS, AFIR_TRANSPOSE_PHASE_GBS);
+      hipLaunchKernelGGL(relu_bcast_add_transpose_f16_phased, dim3((unsigned)(nbl * groups_per_batch)), dim3(kThreads), 0,
+                         stream, x + b0 * m * n, c, out + b0 * m * n, (int)nbl, (int)m, (int)n, hold_ticks);
+    }
   } else if (tiled) {
     // one tile per workgroup: the hardware deals workgroups out as slots free up, which balances
     // better than walks of several tiles (8192 workgroups of one tile 19.7 us on [64, 1024, 512],

@@ -178,9 +178,11 @@ def test_c3_special_values(H):
     assert out[ok].tobytes() == want[ok].tobytes()
 
 
-# Shapes of whole 64 x 256 tile groups between 24 and 64 MiB take the kernel that separates the
-# chip's reads from its writes in time; AFIR_HIP_PHASED=0 keeps a launch on the other kernel.
-@pytest.mark.parametrize("b,m,n", [(12, 1024, 1024), (3, 4096, 1024), (40, 512, 768), (64, 512, 1024)])
+# Shapes of whole 64 x 256 tile groups from 24 MiB up take the kernel that separates the chip's
+# reads from its writes in time (up to 128 MiB, in launches of at most 64 MiB); AFIR_HIP_PHASED=0
+# keeps a launch on the other kernel.
+@pytest.mark.parametrize("b,m,n", [(12, 1024, 1024), (3, 4096, 1024), (40, 512, 768), (64, 512, 1024),
+                                   (81, 1024, 512), (130, 1024, 512)])     # the last two: 41 + 40 batches; past two launches' worth
 def test_c3_phased_route_bit_exact(H, b, m, n, monkeypatch):
     x, c = O.gen_c3(b, m, n)
     x[0, 0, :8] = [np.nan, -np.inf, np.inf, -0.0, 6e-8, -6e-8, 65504, -65504]
@@ -257,12 +259,12 @@ def test_c4_blockdim(H):
         assert out.tobytes() == want.tobytes()
 
 
-# Gathers whose rows are 32 * 2^k halves and that fit the chip at once take the kernel that
-# separates the chip's reads from its writes in time (whole blocks of rows; rows left over take
-# the other kernel in a second launch).  AFIR_HIP_PHASED=0 keeps a launch off it.
+# Gathers whose rows are 32 * 2^k halves take the kernel that separates the chip's reads from its
+# writes in time (whole blocks of rows, up to 128 MiB in launches of at most 64 MiB; rows left
+# over take the other kernel in a launch of their own).  AFIR_HIP_PHASED=0 keeps a launch off it.
 @pytest.mark.parametrize("dim,nidx", [(1024, 16), (1024, 17), (1024, 513), (1024, 4099), (256, 64), (256, 1000),
                                       (2048, 8), (2048, 77), (8192, 2), (8192, 31), (32, 512), (32, 70001),
-                                      (1024, 40000)])
+                                      (1024, 40000), (1024, 70003)])     # the last two: two launches; past two launches' worth
 def test_c4_phased_route_bit_exact(H, dim, nidx, monkeypatch):
     rows = 3000
     table, idx, scale, shift = O.gen_c4(rows, dim, nidx)
