@@ -86,8 +86,8 @@ def main():
     ap.add_argument("--out", default=None)
     ap.add_argument("--repeats", default="200")
     ap.add_argument("--space", default="tiling_space.json",
-                    help="file in the family's directory (tiling_space_unphased.json: the gather / transpose "
-                         "kernels that do not separate reads from writes)")
+                    help="file in the family's directory (tiling_space_unphased.json: the eltwise / gather / "
+                         "transpose kernels that do not separate reads from writes)")
     args = ap.parse_args()
     out = args.out or f"/tmp/autotune-{args.family}"
     os.makedirs(out, exist_ok=True)

@@ -53,6 +53,25 @@ def test_c1_full_size_bit_exact(H):
     assert out.tobytes() == O.golden_c1(a, b).tobytes()
 
 
+# From 16 MiB of output up to 128 MiB the whole 32 KiB blocks of the chain take the kernel that
+# separates the chip's reads from its writes in time (two launches above 64 MiB); what is left
+# over takes the other kernels.  AFIR_HIP_PHASED=0 keeps a launch off it.
+@pytest.mark.parametrize("shape", [(2048, 2049), (3001, 2999), (6000, 4096), (9000, 4096)])
+def test_c1_phased_route_bit_exact(H, shape, monkeypatch):
+    a, b = O.gen_c1(shape)
+    a.ravel()[:8] = [0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, 3e38, 1.0]
+    b.ravel()[:8] = [0.0, 0.0, 1.0, np.inf, 1.0, 1e-45, 3e38, -1.0]
+    a.ravel()[-3:] = [np.nan, -0.0, 3e38]
+    with np.errstate(all="ignore"):
+        want = O.golden_c1(a, b)
+    ok = ~np.isnan(want)
+    for phased in ("1", "0"):
+        monkeypatch.setenv("AFIR_HIP_PHASED", phased)
+        out = H.fused_add_mul(dev(a), dev(b)).cpu().numpy()
+        assert np.array_equal(np.isnan(out), np.isnan(want))
+        assert out[ok].tobytes() == want[ok].tobytes()
+
+
 def test_c1_empty_unaligned_and_blockdim(H):
     e = torch.empty((0, 16), dtype=torch.float32, device="cuda")
     assert H.fused_add_mul(e, e).shape == (0, 16)
