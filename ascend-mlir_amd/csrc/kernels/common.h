@@ -35,7 +35,10 @@ inline int device_cus() {
 // real-time counter the device reads with wall_clock64() (100 MHz on MI355X), counted from the
 // start of each workgroup, base_ns + read_bytes / (gb_per_s GB/s).  AFIR_HIP_PHASED=0 in the
 // environment switches the phased kernels off (the launchers then take their other kernels).
+// (The rates are those of the whole chip: a partition of it, with its share of the CUs, keeps
+// to the other kernels.)
 inline bool phased_enabled() {
+  if (device_cus() != kNumCU) return false;
   const char *env = getenv("AFIR_HIP_PHASED");
   return !(env && env[0] == '0');
 }
