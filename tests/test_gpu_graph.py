@@ -127,3 +127,39 @@ def test_phased_kernels_replay_from_a_captured_graph(H):
     # f32 multiply and add (the product of two halves is exact in f32), one rounding to f16
     assert torch.equal(gathered, (table[idx.long()].float() * scale.float() + shift.float()).half())
     assert torch.equal(xt, (torch.relu(x.float()) + c.float()).half().transpose(1, 2))
+
+
+def test_phased_kernels_that_overlap_on_two_streams(H):
+    """The gather, the transpose and the add-mul chain on the kernels that hold their stores back,
+    launched on two streams at once, several times over: the kernels then share the chip, which
+    the hold does not expect -- it may cost time, never results."""
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    rows, dim, nidx = 4000, 1024, 16384
+    table = torch.randn((rows, dim), generator=gen, device="cuda").half()
+    scale = torch.randn((dim,), generator=gen, device="cuda").half()
+    shift = torch.randn((dim,), generator=gen, device="cuda").half()
+    idx = torch.randint(0, rows, (nidx,), generator=gen, device="cuda", dtype=torch.int32)
+    b, m, n = 24, 1024, 512
+    x = torch.randn((b, m, n), generator=gen, device="cuda").half()
+    c = torch.randn((n,), generator=gen, device="cuda").half()
+    p = torch.randn((2048, 4096), generator=gen, device="cuda")
+    q = torch.randn((2048, 4096), generator=gen, device="cuda")
+    want_g = (table[idx.long()].float() * scale.float() + shift.float()).half()
+    want_t = (torch.relu(x.float()) + c.float()).half().transpose(1, 2).contiguous()
+    want_e = (p + q) * q
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    for rep in range(5):
+        got_g = torch.full((nidx, dim), 7, dtype=torch.float16, device="cuda")
+        got_t = torch.full((b, n, m), 7, dtype=torch.float16, device="cuda")
+        got_e = torch.full((2048, 4096), 7, dtype=torch.float32, device="cuda")
+        torch.cuda.synchronize()
+        H.gather_scale_shift(table, idx, scale, shift, out=got_g, stream=s1.cuda_stream)
+        H.relu_broadcast_add_transpose(x, c, out=got_t, stream=s2.cuda_stream)
+        H.fused_add_mul(p, q, out=got_e, stream=s1.cuda_stream)
+        H.relu_broadcast_add_transpose(x, c, out=got_t, stream=s2.cuda_stream)
+        H.gather_scale_shift(table, idx, scale, shift, out=got_g, stream=s2.cuda_stream)
+        torch.cuda.synchronize()
+        assert torch.equal(got_g, want_g), rep
+        assert torch.equal(got_t, want_t), rep
+        assert torch.equal(got_e, want_e), rep
