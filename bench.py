@@ -48,7 +48,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # is copied from section (2) of the profiles/ file named beside it, which gives
 # the command that produced it.
 MEASURED_TRAFFIC = {
-    "c1": (201422950, "profiles/add_mul_f32_phased__c1_4096x4096.txt"),
+    "c1": (201424896, "profiles/add_mul_f32_phased__c1_4096x4096.txt"),
     "c2": (134633062, "profiles/bcast_add_rowsum_f32_wgrow__c2_8192x4096.txt"),
     "c3": (134401536, "profiles/relu_bcast_add_transpose_f16_phased__c3_64x1024x512.txt"),
     "c4": (133902950, "profiles/gather_scale_shift_f16_phased__c4_131072x1024_idx32768.txt"),
