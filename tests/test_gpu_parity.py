@@ -56,7 +56,9 @@ def test_c1_full_size_bit_exact(H):
 # From 16 MiB of output up to 128 MiB the whole 32 KiB blocks of the chain take the kernel that
 # separates the chip's reads from its writes in time (two launches above 64 MiB); what is left
 # over takes the other kernels.  AFIR_HIP_PHASED=0 keeps a launch off it.
-@pytest.mark.parametrize("shape", [(2048, 2049), (3001, 2999), (6000, 4096), (9000, 4096)])
+@pytest.mark.parametrize("shape", [(2048, 2049), (3001, 2999), (6000, 4096), (9000, 4096),
+                                   # at the limits: 512 blocks (the fewest), one row less, 4096 blocks, half a block more
+                                   (1024, 4096), (1023, 4096), (8192, 4096), (8193, 4096)])
 def test_c1_phased_route_bit_exact(H, shape, monkeypatch):
     a, b = O.gen_c1(shape)
     a.ravel()[:8] = [0.0, -0.0, np.inf, -np.inf, np.nan, 1e-45, 3e38, 1.0]
@@ -201,7 +203,9 @@ def test_c3_special_values(H):
 # reads from its writes in time (up to 128 MiB, in launches of at most 64 MiB); AFIR_HIP_PHASED=0
 # keeps a launch on the other kernel.
 @pytest.mark.parametrize("b,m,n", [(12, 1024, 1024), (3, 4096, 1024), (40, 512, 768), (64, 512, 1024),
-                                   (81, 1024, 512), (130, 1024, 512)])     # the last two: 41 + 40 batches; past two launches' worth
+                                   (81, 1024, 512), (130, 1024, 512),      # 41 + 40 batches; past two launches' worth
+                                   # at the limits: 767 tile groups (one too few), 4096 (two full launches), 4128
+                                   (13, 3776, 256), (128, 1024, 512), (129, 1024, 512)])
 def test_c3_phased_route_bit_exact(H, b, m, n, monkeypatch):
     x, c = O.gen_c3(b, m, n)
     x[0, 0, :8] = [np.nan, -np.inf, np.inf, -0.0, 6e-8, -6e-8, 65504, -65504]
@@ -283,7 +287,8 @@ def test_c4_blockdim(H):
 # over take the other kernel in a launch of their own).  AFIR_HIP_PHASED=0 keeps a launch off it.
 @pytest.mark.parametrize("dim,nidx", [(1024, 16), (1024, 17), (1024, 513), (1024, 4099), (256, 64), (256, 1000),
                                       (2048, 8), (2048, 77), (8192, 2), (8192, 31), (32, 512), (32, 70001),
-                                      (1024, 40000), (1024, 70003)])     # the last two: two launches; past two launches' worth
+                                      (1024, 40000), (1024, 70003),      # two launches; past two launches' worth
+                                      (1024, 65536), (1024, 65552)])     # at the limit: two full launches, one block more
 def test_c4_phased_route_bit_exact(H, dim, nidx, monkeypatch):
     rows = 3000
     table, idx, scale, shift = O.gen_c4(rows, dim, nidx)
