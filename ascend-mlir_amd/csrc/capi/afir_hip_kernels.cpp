@@ -447,6 +447,13 @@ extern "C" {
 
 const char *afir_hip_last_error(void) { return g_last_error.c_str(); }
 
+const char *afir_hip_last_launch(uint32_t *workgroups, uint32_t *threads) {
+  const afir::LaunchNote &note = afir::last_launch_note();
+  if (workgroups) *workgroups = note.workgroups;
+  if (threads) *threads = note.threads;
+  return note.kernel;
+}
+
 uint32_t afir_hip_launch_fused_add_mul(uint32_t block_dim, void *stream, void *a, void *b,
                                        void *out, void * /*workspace*/, void *tiling) {
   int64_t f[2];
@@ -944,7 +951,7 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
         sa.out = ra.out;
         sa.error_flag = ra.error_flag;
         sa.out_vec = ra.out_vec;
-        afir_target::specTailConstants(r->program, segment, res.shapes, sa.tail_const);
+        afir_target::specExtentConstants(r->program, segment, res.shapes, sa.extent_const);
         sa.lanes_log2 = g.lanes_log2;
         sa.grid = (int)g.blocks;
         sa.column_blocks = (int)g.column_blocks;
@@ -1144,6 +1151,9 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
       const std::string no = compiled_function(compiled.get(), r->program, name, &fn);
       if (!no.empty()) return fail(AFIR_HIP_E_LAUNCH, no);
       void *config[] = {HIP_LAUNCH_PARAM_BUFFER_POINTER, args, HIP_LAUNCH_PARAM_BUFFER_SIZE, &bytes, HIP_LAUNCH_PARAM_END};
+      thread_local std::string launched;   // the note keeps a pointer to the name
+      launched = name;
+      afir::last_launch_note() = afir::LaunchNote{launched.c_str(), blocks, 256u};
       const hipError_t e = hipModuleLaunchKernel(fn, blocks, 1, 1, 256, 1, 1, lds, static_cast<hipStream_t>(stream),
                                                  nullptr, config);
       if (e != hipSuccess) return fail(AFIR_HIP_E_LAUNCH, std::string("compiled region kernel: ") + hipGetErrorString(e));

@@ -204,4 +204,18 @@ int afirt_executor_run_file(AfirtExecutor executor, const char *binary_path,
   return 0;
 }
 
+int afirt_executor_last_launch(AfirtExecutor executor, int64_t *kernel_ns, uint32_t *workgroups,
+                               uint32_t *threads, char *kernel_name, size_t name_len) {
+  auto *h = reinterpret_cast<ExecutorHandle *>(executor);
+  if (!h || !h->initialized || !h->runner) return 1;
+  const double us = h->runner->lastKernelMicroseconds();
+  const auto grid = h->runner->lastLaunchedGrid();
+  if (us < 0 || !grid.workgroups) return 1;
+  if (kernel_ns) *kernel_ns = (int64_t)(us * 1e3);
+  if (workgroups) *workgroups = grid.workgroups;
+  if (threads) *threads = grid.threads;
+  writeErr(kernel_name, name_len, grid.kernel);
+  return 0;
+}
+
 }  // extern "C"

@@ -88,6 +88,24 @@ __device__ __forceinline__ int phase_hold_here(int hold_ticks, long long t_start
   return estimate < below * (float)hold_ticks ? (int)estimate : hold_ticks;
 }
 
+// What the calling thread launched last: kernel, workgroups, lanes per workgroup.  A runner reads
+// it back after a launcher call to report the grid the launcher chose (afir_hip_last_launch).
+struct LaunchNote {
+  const char *kernel;
+  unsigned workgroups, threads;
+};
+inline LaunchNote &last_launch_note() {
+  static thread_local LaunchNote note{"", 0u, 0u};
+  return note;
+}
+#define AFIR_LAUNCH(name, kernel, grid, block, lds, stream, ...)                                     \
+  do {                                                                                              \
+    const dim3 afir_grid_ = (grid), afir_block_ = (block);                                          \
+    ::afir::last_launch_note() = ::afir::LaunchNote{name, afir_grid_.x * afir_grid_.y * afir_grid_.z, \
+                                                    afir_block_.x * afir_block_.y * afir_block_.z};  \
+    hipLaunchKernelGGL(kernel, afir_grid_, afir_block_, lds, stream, __VA_ARGS__);                  \
+  } while (0)
+
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));

@@ -164,7 +164,7 @@ LaunchStatus launch_fused_add_mul(const float *a, const float *b, float *out, in
       const size_t nblocks = phased_blocks - b0 < take ? phased_blocks - b0 : take;
       const int hold_ticks = phase_hold_ticks((int64_t)(nblocks * kPhasedChunksPerBlock * 32), AFIR_ELTWISE_PHASE_BASE_NS,
                                               AFIR_ELTWISE_PHASE_GBS);
-      hipLaunchKernelGGL(add_mul_f32_phased, dim3((unsigned)nblocks), dim3(kThreads), 0, stream,
+      AFIR_LAUNCH("add_mul_f32_phased", add_mul_f32_phased, dim3((unsigned)nblocks), dim3(kThreads), 0, stream,
                          reinterpret_cast<const f32x4 *>(a) + b0 * kPhasedChunksPerBlock,
                          reinterpret_cast<const f32x4 *>(b) + b0 * kPhasedChunksPerBlock,
                          reinterpret_cast<f32x4 *>(out) + b0 * kPhasedChunksPerBlock, hold_ticks);
@@ -176,7 +176,7 @@ LaunchStatus launch_fused_add_mul(const float *a, const float *b, float *out, in
     size_t blocks = (rest4 + (size_t)kThreads * kUnroll - 1) / ((size_t)kThreads * kUnroll);
     if (block_dim) blocks = block_dim;
     if (blocks > 0x7fffffffu) blocks = 0x7fffffffu;
-    hipLaunchKernelGGL(add_mul_f32_vec, dim3((unsigned)blocks), dim3(kThreads), 0, stream,
+    AFIR_LAUNCH("add_mul_f32_vec", add_mul_f32_vec, dim3((unsigned)blocks), dim3(kThreads), 0, stream,
                        reinterpret_cast<const f32x4 *>(a) + done4, reinterpret_cast<const f32x4 *>(b) + done4,
                        reinterpret_cast<f32x4 *>(out) + done4, rest4);
   }
@@ -185,7 +185,7 @@ LaunchStatus launch_fused_add_mul(const float *a, const float *b, float *out, in
     size_t blocks = (rest + kThreads - 1) / kThreads;
     if (blocks > (size_t)device_cus() * AFIR_ELTWISE_WG_PER_CU) blocks = (size_t)device_cus() * AFIR_ELTWISE_WG_PER_CU;
     if (block_dim && blocks > block_dim) blocks = block_dim;
-    hipLaunchKernelGGL(add_mul_f32_scalar, dim3((unsigned)blocks), dim3(kThreads), 0, stream,
+    AFIR_LAUNCH("add_mul_f32_scalar", add_mul_f32_scalar, dim3((unsigned)blocks), dim3(kThreads), 0, stream,
                        a, b, out, n4 * 4, n);
   }
   return after_launch();

@@ -375,7 +375,7 @@ LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx
       const int64_t row0 = b0 * phased_rows_per_block;
       const int hold_ticks = phase_hold_ticks(nblocks * phased_rows_per_block * dim * 2, AFIR_GATHER_PHASE_BASE_NS,
                                               AFIR_GATHER_PHASE_GBS);
-      hipLaunchKernelGGL(gather_scale_shift_f16_phased, dim3((unsigned)nblocks), dim3(kPhasedThreads), lds, stream,
+      AFIR_LAUNCH("gather_scale_shift_f16_phased", gather_scale_shift_f16_phased, dim3((unsigned)nblocks), dim3(kPhasedThreads), lds, stream,
                          table, idx + row0, scale, shift, out + row0 * dim, error_flag, (uint32_t)rows, lanes_log2,
                          hold_ticks);
     }
@@ -391,7 +391,7 @@ LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx
     if (blocks > (int64_t)device_cus() * AFIR_GATHER_GROUPED_WG_PER_CU) blocks = (int64_t)device_cus() * AFIR_GATHER_GROUPED_WG_PER_CU;
     if (block_dim) blocks = block_dim;
     const size_t lds = (size_t)2 * (kGroups << lanes_log2) * 16;   // scale and shift, 16-byte chunks
-    hipLaunchKernelGGL(gather_scale_shift_f16_grouped, dim3((unsigned)blocks), dim3(kGroupedThreads), lds,
+    AFIR_LAUNCH("gather_scale_shift_f16_grouped", gather_scale_shift_f16_grouped, dim3((unsigned)blocks), dim3(kGroupedThreads), lds,
                        stream, table, idx, scale, shift, out, error_flag, (uint32_t)rows, lanes_log2,
                        nidx);
   } else if (vec) {
@@ -406,14 +406,14 @@ LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx
     int64_t blocks = (nidx + rows_per_block - 1) / rows_per_block;
     if (block_dim) blocks = block_dim;
     if (blocks > 0x7fffffff) blocks = 0x7fffffff;
-    hipLaunchKernelGGL(gather_scale_shift_f16_vec, dim3((unsigned)blocks), dim3(kThreads), 0,
+    AFIR_LAUNCH("gather_scale_shift_f16_vec", gather_scale_shift_f16_vec, dim3((unsigned)blocks), dim3(kThreads), 0,
                        stream, table, idx, scale, shift, out, error_flag, (uint32_t)rows, chunks,
                        nidx, lanes_per_row, rows_per_block);
   } else {
     int64_t blocks = (nidx + 3) / 4;
     if (block_dim) blocks = block_dim;
     if (blocks > 0x7fffffff) blocks = 0x7fffffff;
-    hipLaunchKernelGGL(gather_scale_shift_f16_any, dim3((unsigned)blocks), dim3(kThreads), 0,
+    AFIR_LAUNCH("gather_scale_shift_f16_any", gather_scale_shift_f16_any, dim3((unsigned)blocks), dim3(kThreads), 0,
                        stream, table, idx, scale, shift, out, error_flag, (uint32_t)rows, dim,
                        nidx);
   }

@@ -322,7 +322,7 @@ LaunchStatus launch_mfma(const uint16_t *a, const uint16_t *b, const void *bias,
   const int tiles_m = EDGE ? (m + BM - 1) / BM : m / BM, tiles_n = EDGE ? (n + BN - 1) / BN : n / BN;
   int64_t blocks = (int64_t)tiles_m * tiles_n;
   if (block_dim) blocks = block_dim;
-  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(NT), kLds, stream, a, b, bias, out, m, k,
+  AFIR_LAUNCH("matmul_bias_leakyrelu_mfma", kernel, dim3((unsigned)blocks), dim3(NT), kLds, stream, a, b, bias, out, m, k,
                      n, alpha, relu ? 1 : 0, tiles_m, tiles_n);
   return after_launch();
 }
@@ -372,7 +372,7 @@ LaunchStatus launch_matmul_any_io(const uint16_t *a, const uint16_t *b, const vo
   int64_t blocks = (int64_t)tiles_m * tiles_n;
   if (block_dim) blocks = block_dim;
   if (blocks > 0x7fffffff) blocks = 0x7fffffff;
-  hipLaunchKernelGGL(matmul_bias_leakyrelu_any<F16IO>, dim3((unsigned)blocks), dim3(256), 0, stream,
+  AFIR_LAUNCH("matmul_bias_leakyrelu_any<F16IO>", matmul_bias_leakyrelu_any<F16IO>, dim3((unsigned)blocks), dim3(256), 0, stream,
                      a, b, bias, out, (int)m, (int)k, (int)n, alpha, relu ? 1 : 0, tiles_m, tiles_n);
   return after_launch();
 }

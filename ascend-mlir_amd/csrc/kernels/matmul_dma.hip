@@ -697,7 +697,7 @@ LaunchStatus launch_dma(const uint16_t *a, const uint16_t *b, const void *bias, 
   int64_t blocks = (int64_t)tiles_m * tiles_n;
   if (blocks > AFIR_MM_GRID) blocks = AFIR_MM_GRID;
   if (block_dim) blocks = block_dim;
-  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(kWaves * 64), kLdsBytes, stream, a, b,
+  AFIR_LAUNCH("matmul_bias_leakyrelu_dma", kernel, dim3((unsigned)blocks), dim3(kWaves * 64), kLdsBytes, stream, a, b,
                      bias, out, m, k, n, alpha, relu ? 1 : 0, tiles_m, tiles_n);
   return after_launch();
 }

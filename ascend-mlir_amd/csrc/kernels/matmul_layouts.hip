@@ -276,7 +276,7 @@ LaunchStatus launch_layout_mfma(const uint16_t *a, const uint16_t *b, const void
   const int tiles_m = (m + kLT - 1) / kLT, tiles_n = (n + kLT - 1) / kLT;
   int64_t blocks = (int64_t)tiles_m * tiles_n;
   if (block_dim) blocks = block_dim;
-  hipLaunchKernelGGL(kernel, dim3((unsigned)blocks, (unsigned)batch), dim3(kLThreads), kLds, stream, a, b, bias, out,
+  AFIR_LAUNCH("matmul_layout_mfma", kernel, dim3((unsigned)blocks, (unsigned)batch), dim3(kLThreads), kLds, stream, a, b, bias, out,
                      m, k, n, (int64_t)m * k, (int64_t)k * n, (int64_t)m * n, alpha, relu ? 1 : 0, tiles_m, tiles_n);
   return after_launch();
 }
@@ -311,7 +311,7 @@ LaunchStatus launch_layouts_io(const uint16_t *a, const uint16_t *b, const void 
   int64_t blocks = (int64_t)tiles_m * tiles_n;
   if (block_dim) blocks = block_dim;
   if (blocks > 0x7fffffff) blocks = 0x7fffffff;
-  hipLaunchKernelGGL(matmul_layout_any<F16IO>, dim3((unsigned)blocks, (unsigned)batch), dim3(256), 0, stream, a, b,
+  AFIR_LAUNCH("matmul_layout_any<F16IO>", matmul_layout_any<F16IO>, dim3((unsigned)blocks, (unsigned)batch), dim3(256), 0, stream, a, b,
                      bias, out, (int)m, (int)k, (int)n, ta ? 1 : 0, tb ? 1 : 0, m * k, k * n, m * n, alpha,
                      relu ? 1 : 0, tiles_m, tiles_n);
   return after_launch();

@@ -695,13 +695,13 @@ LaunchStatus launch_fused_region(const RegionArgs &args_in, uint32_t block_dim, 
     auto kernel = wide ? (idx32 ? fused_region_rowsum<int, true, 16> : fused_region_rowsum<int64_t, true, 16>)
                   : args.chain ? (idx32 ? fused_region_rowsum<int, true, 8> : fused_region_rowsum<int64_t, true, 8>)
                                : (idx32 ? fused_region_rowsum<int, false, 8> : fused_region_rowsum<int64_t, false, 8>);
-    hipLaunchKernelGGL(kernel, dim3((unsigned)g.blocks), dim3(kThreads), 0, stream, args, g.lanes_log2);
+    AFIR_LAUNCH("fused_region_rowsum", kernel, dim3((unsigned)g.blocks), dim3(kThreads), 0, stream, args, g.lanes_log2);
     return after_launch();
   }
   auto kernel = wide ? (idx32 ? fused_region_parallel<int, true, 16> : fused_region_parallel<int64_t, true, 16>)
                 : args.chain ? (idx32 ? fused_region_parallel<int, true, 8> : fused_region_parallel<int64_t, true, 8>)
                              : (idx32 ? fused_region_parallel<int, false, 8> : fused_region_parallel<int64_t, false, 8>);
-  hipLaunchKernelGGL(kernel, dim3((unsigned)(g.blocks / g.column_blocks), (unsigned)g.column_blocks), dim3(kThreads), 0,
+  AFIR_LAUNCH("fused_region_parallel", kernel, dim3((unsigned)(g.blocks / g.column_blocks), (unsigned)g.column_blocks), dim3(kThreads), 0,
                      stream, args, g.lanes_log2);
   return after_launch();
 }

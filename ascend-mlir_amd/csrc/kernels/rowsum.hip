@@ -193,10 +193,10 @@ LaunchStatus launch_broadcast_add_reducesum(const float *x, const float *bias, f
     if (block_dim) wblocks = block_dim;
     const dim3 grid((unsigned)wblocks), block(kRowThreads);
     switch ((int)(n / 4 / kRowThreads)) {
-      case 1: hipLaunchKernelGGL(bcast_add_rowsum_f32_wgrow<1>, grid, block, 0, stream, x, bias, y, m, n); break;
-      case 2: hipLaunchKernelGGL(bcast_add_rowsum_f32_wgrow<2>, grid, block, 0, stream, x, bias, y, m, n); break;
-      case 4: hipLaunchKernelGGL(bcast_add_rowsum_f32_wgrow<4>, grid, block, 0, stream, x, bias, y, m, n); break;
-      default: hipLaunchKernelGGL(bcast_add_rowsum_f32_wgrow<8>, grid, block, 0, stream, x, bias, y, m, n); break;
+      case 1: AFIR_LAUNCH("bcast_add_rowsum_f32_wgrow<1>", bcast_add_rowsum_f32_wgrow<1>, grid, block, 0, stream, x, bias, y, m, n); break;
+      case 2: AFIR_LAUNCH("bcast_add_rowsum_f32_wgrow<2>", bcast_add_rowsum_f32_wgrow<2>, grid, block, 0, stream, x, bias, y, m, n); break;
+      case 4: AFIR_LAUNCH("bcast_add_rowsum_f32_wgrow<4>", bcast_add_rowsum_f32_wgrow<4>, grid, block, 0, stream, x, bias, y, m, n); break;
+      default: AFIR_LAUNCH("bcast_add_rowsum_f32_wgrow<8>", bcast_add_rowsum_f32_wgrow<8>, grid, block, 0, stream, x, bias, y, m, n); break;
     }
   } else if (vec && n / 4 <= 16 * kWave) {
     // persistent waves: each keeps its bias chunks resident and walks several rows
@@ -206,7 +206,7 @@ LaunchStatus launch_broadcast_add_reducesum(const float *x, const float *bias, f
     if (block_dim) pblocks = block_dim;
     const dim3 grid((unsigned)pblocks), block(kThreads);
     auto launch = [&](auto kernel) {
-      hipLaunchKernelGGL(kernel, grid, block, 0, stream, x, bias, y, m, n);
+      AFIR_LAUNCH("bcast_add_rowsum_f32_resident", kernel, grid, block, 0, stream, x, bias, y, m, n);
     };
     if (n4 == 16 * kWave) launch(bcast_add_rowsum_f32_resident<16, true>);
     else if (n4 == 8 * kWave) launch(bcast_add_rowsum_f32_resident<8, true>);
@@ -217,10 +217,10 @@ LaunchStatus launch_broadcast_add_reducesum(const float *x, const float *bias, f
     else if (n4 <= 8 * kWave) launch(bcast_add_rowsum_f32_resident<8, false>);
     else launch(bcast_add_rowsum_f32_resident<16, false>);
   } else if (vec) {
-    hipLaunchKernelGGL(bcast_add_rowsum_f32_vec, dim3((unsigned)blocks), dim3(kThreads), 0,
+    AFIR_LAUNCH("bcast_add_rowsum_f32_vec", bcast_add_rowsum_f32_vec, dim3((unsigned)blocks), dim3(kThreads), 0,
                        stream, x, bias, y, m, n);
   } else {
-    hipLaunchKernelGGL(bcast_add_rowsum_f32_scalar, dim3((unsigned)blocks), dim3(kThreads), 0,
+    AFIR_LAUNCH("bcast_add_rowsum_f32_scalar", bcast_add_rowsum_f32_scalar, dim3((unsigned)blocks), dim3(kThreads), 0,
                        stream, x, bias, y, m, n);
   }
   return after_launch();
@@ -344,9 +344,9 @@ extern "C" uint32_t afir_hip_launch_broadcast_add_reducesum_noalloc(uint32_t blo
     float *scratch = nullptr;
     const LaunchStatus got = scratch_of_current_device(&scratch);
     if (got.code) return got.code == 1 ? AFIR_HIP_E_INVALID : AFIR_HIP_E_LAUNCH;
-    hipLaunchKernelGGL(bcast_add_rowsum_f32_split, dim3((unsigned)(m * parts)), dim3(kSplitThreads), 0, st,
+    AFIR_LAUNCH("bcast_add_rowsum_f32_split", bcast_add_rowsum_f32_split, dim3((unsigned)(m * parts)), dim3(kSplitThreads), 0, st,
                        static_cast<const float *>(x), static_cast<const float *>(bias), scratch, n, (int)parts);
-    hipLaunchKernelGGL(bcast_add_rowsum_f32_join, dim3((unsigned)((m + 3) / 4)), dim3(kSplitThreads), 0, st,
+    AFIR_LAUNCH("bcast_add_rowsum_f32_join", bcast_add_rowsum_f32_join, dim3((unsigned)((m + 3) / 4)), dim3(kSplitThreads), 0, st,
                        scratch, static_cast<float *>(y), m, (int)parts);
     return hipGetLastError() == hipSuccess ? AFIR_HIP_OK : AFIR_HIP_E_LAUNCH;
   }

@@ -280,7 +280,7 @@ LaunchStatus launch_relu_broadcast_add_transpose(const uint16_t *x, const uint16
     for (int64_t b0 = 0; b0 < nb; b0 += take) {
       const int64_t nbl = nb - b0 < take ? nb - b0 : take;
       const int hold_ticks = phase_hold_ticks(nbl * m * n * 2, AFIR_TRANSPOSE_PHASE_BASE_NS, AFIR_TRANSPOSE_PHASE_GBS);
-      hipLaunchKernelGGL(relu_bcast_add_transpose_f16_phased, dim3((unsigned)(nbl * groups_per_batch)), dim3(kThreads), 0,
+      AFIR_LAUNCH("relu_bcast_add_transpose_f16_phased", relu_bcast_add_transpose_f16_phased, dim3((unsigned)(nbl * groups_per_batch)), dim3(kThreads), 0,
                          stream, x + b0 * m * n, c, out + b0 * m * n, (int)nbl, (int)m, (int)n, hold_ticks);
     }
   } else if (tiled) {
@@ -292,13 +292,13 @@ LaunchStatus launch_relu_broadcast_add_transpose(const uint16_t *x, const uint16
     int64_t blocks = (nb * (m / kSmallTile) * (n / kSmallTile) + AFIR_TRANSPOSE_TILES_PER_WG - 1) / AFIR_TRANSPOSE_TILES_PER_WG;
     if (blocks > (int64_t)device_cus() * 256) blocks = (int64_t)device_cus() * 256;
     if (block_dim) blocks = block_dim;
-    hipLaunchKernelGGL(relu_bcast_add_transpose_f16_tile64, dim3((unsigned)blocks), dim3(kThreads), 0, stream,
+    AFIR_LAUNCH("relu_bcast_add_transpose_f16_tile64", relu_bcast_add_transpose_f16_tile64, dim3((unsigned)blocks), dim3(kThreads), 0, stream,
                        x, c, out, (int)nb, (int)m, (int)n);
   } else {
     int64_t blocks = nb * ((m + 31) / 32) * ((n + 31) / 32);
     if (block_dim) blocks = block_dim;
     if (blocks > 0x7fffffff) blocks = 0x7fffffff;
-    hipLaunchKernelGGL(relu_bcast_add_transpose_f16_any, dim3((unsigned)blocks), dim3(kThreads),
+    AFIR_LAUNCH("relu_bcast_add_transpose_f16_any", relu_bcast_add_transpose_f16_any, dim3((unsigned)blocks), dim3(kThreads),
                        0, stream, x, c, out, (int)nb, (int)m, (int)n);
   }
   return after_launch();

@@ -532,6 +532,10 @@ Expected<RunTaskSpec> parseTask(const Json &root, const std::optional<std::strin
     spec.invocation.tiling = tb;
   }
   if (auto v = root.getInteger("block_dim")) spec.invocation.blockDim = (int)*v;
+  if (auto v = root.getInteger("hip_grid")) {
+    if (*v < 0 || *v > (1 << 30)) return Status::error("hip_grid must be between 0 and 2^30");
+    spec.invocation.hipGrid = (int)*v;
+  }
   if (auto v = root.getInteger("workspace_size")) {
     if (*v < 0) return Status::error("workspace_size must be non-negative");
     spec.invocation.workspaceSize = (size_t)*v;

@@ -19,6 +19,7 @@
 #include <hip/hip_runtime.h>
 
 #include <chrono>
+#include <cstdlib>
 #include <cstring>
 
 #include "runtime.h"
@@ -107,6 +108,7 @@ class HipExecutionRunner final : public ExecutionRunner {
                                    RunArgs &args) override {
     lastKernelUs_ = -1.0;
     lastRegionRoute_.clear();
+    lastGrid_ = {};
     if (!initialized_) return Status::error("execution runner has not been initialized");
     if (args.inputs.size() + args.outputs.size() + 2 > 16)
       return Status::error("too many tensor arguments for a launcher call (16 pointer slots)");
@@ -232,7 +234,17 @@ class HipExecutionRunner final : public ExecutionRunner {
       }
 
     // ---- launch ----
-    const uint32_t bd = (uint32_t)(args.block_dim < 0 ? 0 : args.block_dim);
+    // The launcher's first argument is a number of workgroups (0 = its own choice).  The
+    // caller's block_dim is an Ascend AI-core count and becomes that only on request.
+    uint32_t bd = 0;
+    lastGrid_.source = "launcher";
+    if (args.hip_grid > 0) {
+      bd = (uint32_t)args.hip_grid;
+      lastGrid_.source = "hip_grid";
+    } else if (const char *env = getenv("AFIR_HIP_HONOUR_BLOCK_DIM"); env && env[0] == '1' && args.block_dim > 0) {
+      bd = (uint32_t)args.block_dim;
+      lastGrid_.source = "block_dim";
+    }
     double bestUs = -1.0;
     auto launchOnce = [&](void **use) -> uint32_t {
       if (regionLaunch) {
@@ -288,6 +300,9 @@ class HipExecutionRunner final : public ExecutionRunner {
       if (hipEventElapsedTime(&ms, ev0_, ev1_) == hipSuccess) bestUs = (double)ms * 1e3 / repeats;
     }
     lastKernelUs_ = bestUs;
+    using LastLaunchFn = const char *(*)(uint32_t *, uint32_t *);
+    if (auto last = reinterpret_cast<LastLaunchFn>(dlsym(lib, "afir_hip_last_launch")))
+      if (const char *name = last(&lastGrid_.workgroups, &lastGrid_.threads)) lastGrid_.kernel = name;
 
     // ---- data errors reported through the workspace ----
     int32_t flag = 0;
@@ -309,6 +324,7 @@ class HipExecutionRunner final : public ExecutionRunner {
 
   double lastKernelMicroseconds() const override { return lastKernelUs_; }
   std::string lastRegionRoute() const override { return lastRegionRoute_; }
+  LaunchedGrid lastLaunchedGrid() const override { return lastGrid_; }
 
  private:
   Status validate(void *lib, const std::string &symbol, const RunArgs &args) {
@@ -388,6 +404,7 @@ class HipExecutionRunner final : public ExecutionRunner {
   hipEvent_t ev0_ = nullptr, ev1_ = nullptr;
   double lastKernelUs_ = -1.0;
   std::string lastRegionRoute_;
+  LaunchedGrid lastGrid_;
 };
 
 }  // namespace

@@ -92,7 +92,15 @@ struct RunArgs {
   std::vector<NDArray> inputs;
   std::vector<NDArray> outputs;   // pre-allocated, filled by the run
   std::vector<uint8_t> tiling;    // packed TilingData bytes (little-endian)
+  // The caller's block_dim, in the reference's unit: a number of Ascend AI cores (its callers pass
+  // 1, 8 or 40: python/runtime/executor.py:183, test/tools/runtime/test_capi_runtime.cpp:171-174,
+  // examples/broadcast-add-reduce/run.sh:259).  It says nothing about a 256-CU GPU, so the HIP
+  // runner records it and leaves the grid to the launcher, unless the process opts in with
+  // AFIR_HIP_HONOUR_BLOCK_DIM=1 (then a positive block_dim is the number of workgroups).
   int block_dim = 1;
+  // Workgroups to launch, for callers that mean a HIP grid (the run manifest's "hip_grid", the
+  // tile search's block_dim_values); 0 = the launcher sizes the grid for the device.
+  int hip_grid = 0;
   size_t workspace_size = 8192;
   // Extra timed launches of the same kernel on the same device buffers (the
   // kernels are pure functions of their inputs): the reported kernel time is the
@@ -267,6 +275,7 @@ struct ExecutionInvocation {
   std::vector<TensorBinding> inputs, outputs, expectedOutputs;
   std::optional<TilingBinding> tiling;
   int blockDim = 1;
+  int hipGrid = 0;        // "hip_grid": workgroups to launch, 0 = the launcher's choice
   size_t workspaceSize = 8192;
   bool enableProfiling = false;
   double atol = 1.0;
@@ -322,6 +331,13 @@ class ExecutionRunner {
   // kernel), "compiled" (the artifact's code object) or "interpreter" (the library's
   // generic kernel, several times slower); "" for launcher-symbol artifacts.
   virtual std::string lastRegionRoute() const { return ""; }
+  // The last kernel the last run launched and its grid; "" / 0 if unknown.  gridSource says who
+  // chose the grid: "launcher", "hip_grid" or "block_dim" (AFIR_HIP_HONOUR_BLOCK_DIM=1).
+  struct LaunchedGrid {
+    std::string kernel, source;
+    uint32_t workgroups = 0, threads = 0;
+  };
+  virtual LaunchedGrid lastLaunchedGrid() const { return {}; }
 };
 
 // The MI355X runner: alloc -> H2D -> launch -> sync -> D2H -> free

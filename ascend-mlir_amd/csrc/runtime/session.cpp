@@ -129,6 +129,7 @@ SessionSummary runSingleTask(const RunTaskSpec &task, RunnerFactory factory, int
   // ---- bindings ----
   RunArgs args;
   args.block_dim = inv.blockDim;
+  args.hip_grid = inv.hipGrid;
   args.workspace_size = inv.workspaceSize;
   auto tiling = packTilingBytes(inv.tiling);
   if (!tiling) return fail(summary, "bindings", tiling.error());
@@ -210,6 +211,12 @@ SessionSummary runSingleTask(const RunTaskSpec &task, RunnerFactory factory, int
   if (const std::string route = runner->lastRegionRoute(); !route.empty())
     summary.runtimeAttributes["region_route"] = route;
   summary.runtimeCounters["block_dim"] = inv.blockDim;
+  // the grid that ran (block_dim is the reference's AI-core count and does not size it)
+  if (const auto grid = runner->lastLaunchedGrid(); grid.workgroups) {
+    summary.runtimeAttributes["grid"] = std::to_string(grid.workgroups) + "x" + std::to_string(grid.threads);
+    summary.runtimeAttributes["grid_source"] = grid.source;
+    summary.runtimeAttributes["kernel"] = grid.kernel;
+  }
   summary.runtimeCounters["tiling_bytes"] = (int64_t)args.tiling.size();
 
   // ---- validate ----

@@ -40,7 +40,7 @@ struct SpecArgs {
   int grid;
   int column_blocks;
   SpecInput in[8];
-  float tail_const[4];
+  float extent_const[8];
 };
 
 DEV float as_f32(unsigned u) { return __builtin_bit_cast(float, u); }
@@ -652,7 +652,7 @@ class SegmentEmitter {
 
   Value emitCompute(int d, const std::vector<Value> &read) {
     std::vector<Value> stack;
-    int push = 0, temp = 0;
+    int push = 0, temp = 0, extent = 0;
     auto fresh = [&](bool scalar) {
       Value v;
       v.name = "t" + std::to_string(temp++);
@@ -678,7 +678,9 @@ class SegmentEmitter {
           break;
         case OpCode::Const: {
           Value v = fresh(true);
-          define(v, integer_ ? intLiteral(op.constant) : floatLiteral(op.constant));
+          // an extent is known at the launch, not here: it arrives with the arguments
+          if (op.extent) define(v, "R.extent_const[" + std::to_string(extent++) + "]");
+          else define(v, integer_ ? intLiteral(op.constant) : floatLiteral(op.constant));
           stack.push_back(v);
           break;
         }
@@ -741,7 +743,8 @@ class SegmentEmitter {
   }
 
   // The operations after 'reduce sum' as a C expression in the row's sum `s`: constants are
-  // literals, extent constants R.tail_const[k] in program order.  `s` itself when there are none.
+  // literals, extent constants R.extent_const[k], k counting the segment's extent constants in
+  // program order (those before 'reduce sum' come first).  `s` itself when there are none.
   std::string tailExpression(const std::string &s) const {
     std::vector<std::string> stack;
     bool after = false;
@@ -752,10 +755,11 @@ class SegmentEmitter {
         stack.assign(1, s);
         continue;
       }
+      if (!after && op.code == OpCode::Const && op.extent) ++extent;
       if (!after || op.code == OpCode::Store) continue;
       switch (op.code) {
         case OpCode::Const:
-          stack.push_back(op.extent ? "R.tail_const[" + std::to_string(extent++) + "]" : floatLiteral(op.constant));
+          stack.push_back(op.extent ? "R.extent_const[" + std::to_string(extent++) + "]" : floatLiteral(op.constant));
           break;
         case OpCode::Dup:
           stack.push_back(stack[stack.size() - 1 - op.depth]);
@@ -1500,16 +1504,13 @@ bool specAllSegments(const Program &p) {
   return true;
 }
 
-void specTailConstants(const Program &p, int segment, const std::vector<std::vector<int64_t>> &shapes,
-                       float (&out)[kSpecMaxTailConsts]) {
+void specExtentConstants(const Program &p, int segment, const std::vector<std::vector<int64_t>> &shapes,
+                         float (&out)[kSpecMaxExtentConsts]) {
   for (float &v : out) v = 0.f;
   int n = 0;
-  bool after = false;
-  for (const Op &op : p.segments[segment].ops) {
-    if (op.code == OpCode::ReduceSum) after = true;
-    if (after && op.code == OpCode::Const && op.extent && n < kSpecMaxTailConsts)
+  for (const Op &op : p.segments[segment].ops)
+    if (op.code == OpCode::Const && op.extent && n < kSpecMaxExtentConsts)
       out[n++] = afir_region::roundThroughType((float)shapes[op.constRef.arg][op.constRef.dim], op.constType);
-  }
 }
 
 uint64_t programHash(const Program &p) {

@@ -40,7 +40,7 @@ struct SpecInput {
   int gvec;            // ... also after adding any multiple of gstride
 };
 constexpr int kSpecMaxInputs = 8;
-constexpr int kSpecMaxTailConsts = afir_region::kMaxTailExtents;
+constexpr int kSpecMaxExtentConsts = afir_region::kMaxSegmentExtents;
 struct SpecArgs {
   long long size[3];
   void *out;
@@ -51,13 +51,13 @@ struct SpecArgs {
   int column_blocks;   // parallel segments: of these, the workgroups that share a pass of rows and
                        // split the row between them (grid is a multiple of it; 1 elsewhere)
   SpecInput in[kSpecMaxInputs];
-  float tail_const[kSpecMaxTailConsts];   // reduce segments: the extent constants of the operations
-                                          // after 'reduce sum', in program order (resolved per launch)
+  float extent_const[kSpecMaxExtentConsts];   // the segment's extent constants ('const argA.D'), in program
+                                              // order, before and after 'reduce sum' (resolved per launch)
 };
-// The values of a segment's extent constants after 'reduce sum' for a launch's shapes (what
-// goes into SpecArgs::tail_const): shapes[a][d] = extent of dim d of argument a.
-void specTailConstants(const afir_region::Program &p, int segment,
-                       const std::vector<std::vector<int64_t>> &shapes, float (&out)[kSpecMaxTailConsts]);
+// The values of a segment's extent constants for a launch's shapes (what goes into
+// SpecArgs::extent_const): shapes[a][d] = extent of dim d of argument a.
+void specExtentConstants(const afir_region::Program &p, int segment,
+                         const std::vector<std::vector<int64_t>> &shapes, float (&out)[kSpecMaxExtentConsts]);
 
 // Programs of 2..kSpecMaxSegments segments also get one kernel that runs all
 // of them in a single launch (segments write disjoint row ranges of the
@@ -112,7 +112,7 @@ uint64_t programHash(const afir_region::Program &p);
 // Version of the set of kernels and of the launch arguments that emitHipSource produces; the
 // code object exports it as `afir_region_emit_abi`, and a code object of another version is
 // refused when it is loaded (its kernels would be launched with the wrong names or arguments).
-constexpr int kSpecAbiVersion = 8;
+constexpr int kSpecAbiVersion = 9;
 
 // What a launch promises, which picks the kernel variant:
 //   kSpecAligned  every 128-bit access is aligned and every pass of the lanes over a row is whole

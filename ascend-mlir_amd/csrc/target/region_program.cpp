@@ -339,7 +339,7 @@ std::string validate(const Program &p) {
       if (!refOk(r)) return "region program: bad output offset reference";
     if (g.ops.empty() || g.ops.back().code != OpCode::Store) return "region program: a segment must end with 'store'";
     if ((int)g.ops.size() > kMaxOps) return "region program: too many operations in a segment";
-    int depth = 0, pushes = 0, tailOps = 0, tailExtents = 0;
+    int depth = 0, pushes = 0, tailOps = 0, tailExtents = 0, extents = 0;
     bool reduced = false;
     // after 'reduce sum': which stack entries derive from the sum (exactly one does at any time)
     std::vector<bool> fromSum;
@@ -427,6 +427,8 @@ std::string validate(const Program &p) {
           if (o.extent) {
             if (integer) return "region program: an extent constant is not available in an integer region";
             if (!refOk(o.constRef) || o.constRef.arg < 0) return "region program: bad extent constant";
+            if (++extents > kMaxSegmentExtents)
+              return "region program: more than " + std::to_string(kMaxSegmentExtents) + " extent constants in a segment";
             ++depth;
             break;
           }

@@ -189,6 +189,7 @@ struct ResolvedSegment {
 
 constexpr int kMaxTailOps = 8;    // operations on the sum between 'reduce sum' and 'store'
 constexpr int kMaxTailExtents = 4;   // of which extent constants
+constexpr int kMaxSegmentExtents = 8;   // extent constants of one segment, before and after 'reduce sum'
 
 // float -> f16 / bf16 -> float, round to nearest even (f32: the value itself).
 float roundThroughType(float f, ElemType t);

@@ -408,6 +408,7 @@ int main(int argc, char **argv) {
       RunArgs args;
       args.tiling = *packed;
       args.block_dim = (int)bd;
+      args.hip_grid = (int)bd;     // a candidate's block_dim is a HIP grid here, not an AI-core count
       args.inputs.resize(base.inputs.size());
       for (size_t i = 0; i < base.inputs.size(); ++i) {
         args.inputs[i].shape = base.inputs[i].shape;

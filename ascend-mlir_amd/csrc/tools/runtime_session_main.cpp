@@ -25,10 +25,19 @@ class SuccessfulTestingRunner final : public ExecutionRunner {
   ExecutionRunnerMode mode() const override { return ExecutionRunnerMode::Simulation; }
   Status initialize(int) override { return Status::success(); }
   Status runFile(const FileExecutionLaunch &, RunArgs &) override { return Status::success(); }
-  Status runDynamicLibraryArtifact(const DynamicLibraryExecutionLaunch &, RunArgs &) override {
+  Status runDynamicLibraryArtifact(const DynamicLibraryExecutionLaunch &, RunArgs &args) override {
+    // the grid rule of the HIP runner, without a launch: "hip_grid" is a grid, block_dim is not
+    grid_.kernel = "testing";
+    grid_.source = args.hip_grid > 0 ? "hip_grid" : "launcher";
+    grid_.workgroups = args.hip_grid > 0 ? (uint32_t)args.hip_grid : 2048u;
+    grid_.threads = 256;
     return Status::success();
   }
   double lastKernelMicroseconds() const override { return 12.5; }   // a fixed figure for the profile tests
+  LaunchedGrid lastLaunchedGrid() const override { return grid_; }
+
+ private:
+  LaunchedGrid grid_;
 };
 std::unique_ptr<ExecutionRunner> makeTestingRunner() {
   return std::make_unique<SuccessfulTestingRunner>();

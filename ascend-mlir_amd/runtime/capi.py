@@ -12,7 +12,7 @@ MAGIC_ELF_AICUBE = 0x41494343
 EXPORTED_SYMBOLS = [
     "afirt_compiler_create", "afirt_compiler_destroy", "afirt_compiler_compile",
     "afirt_executor_create", "afirt_executor_destroy", "afirt_executor_initialize",
-    "afirt_executor_run", "afirt_executor_run_file",
+    "afirt_executor_run", "afirt_executor_run_file", "afirt_executor_last_launch",
 ]
 
 
@@ -63,5 +63,8 @@ def load_capi() -> ctypes.CDLL:
     L.afirt_executor_run.argtypes = [vp, ctypes.POINTER(ctypes.c_uint8), sz] + run_tail
     L.afirt_executor_run_file.restype = ctypes.c_int
     L.afirt_executor_run_file.argtypes = [vp, cp] + run_tail
+    L.afirt_executor_last_launch.restype = ctypes.c_int
+    L.afirt_executor_last_launch.argtypes = [vp, ctypes.POINTER(ctypes.c_int64), ctypes.POINTER(ctypes.c_uint32),
+                                             ctypes.POINTER(ctypes.c_uint32), cp, sz]
     _lib = L
     return L

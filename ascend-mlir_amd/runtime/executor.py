@@ -37,8 +37,12 @@ class HipRuntime:
         self._initialized = True
 
     def run(self, binary_data: bytes, function_name: str, inputs: Sequence[np.ndarray],
-            outputs: List[np.ndarray], tiling_data: Optional[bytes] = None, block_dim: int = 0,
+            outputs: List[np.ndarray], tiling_data: Optional[bytes] = None, block_dim: int = 1,
             magic: int = MAGIC_ELF_AIVEC) -> List[np.ndarray]:
+        """block_dim keeps the reference's meaning and default (a number of Ascend AI cores,
+        python/runtime/executor.py:183): it is recorded, and the kernel's launcher sizes the HIP
+        grid for the device.  AFIR_HIP_HONOUR_BLOCK_DIM=1 in the environment makes a positive
+        block_dim the number of workgroups instead."""
         lib = load_capi()
         vp, sz = ctypes.c_void_p, ctypes.c_size_t
         bin_arr = (ctypes.c_uint8 * max(len(binary_data), 1)).from_buffer_copy(
@@ -67,6 +71,17 @@ class HipRuntime:
         return outputs
 
 
+    def last_launch(self) -> dict:
+        """Device time and grid of the last run's kernel (afirt_executor_last_launch)."""
+        ns, wg, th = ctypes.c_int64(0), ctypes.c_uint32(0), ctypes.c_uint32(0)
+        name = ctypes.create_string_buffer(128)
+        if load_capi().afirt_executor_last_launch(self._handle, ctypes.byref(ns), ctypes.byref(wg),
+                                                  ctypes.byref(th), name, len(name)) != 0:
+            raise ExecutorError("no kernel has run on this executor")
+        return {"kernel_ns": ns.value, "workgroups": wg.value, "threads": th.value,
+                "kernel": name.value.decode(errors="replace")}
+
+
 AscendRuntime = HipRuntime   # the reference's name for this role
 
 
@@ -81,7 +96,7 @@ class KernelExecutor:
         self._initialized = True
 
     def execute(self, binary_data, function_name, inputs, outputs, tiling_data=None,
-                block_dim: int = 0, magic: int = MAGIC_ELF_AIVEC):
+                block_dim: int = 1, magic: int = MAGIC_ELF_AIVEC):
         if not self._initialized:
             self.initialize()
         return self.runtime.run(binary_data, function_name, inputs, outputs, tiling_data,

@@ -62,6 +62,15 @@ extern "C" {
 /* Message for the calling thread's most recent non-zero return ("" if none). */
 const char *afir_hip_last_error(void);
 
+/* The kernel the calling thread launched last through this library: its name
+ * (a static or thread-owned string, "" before the first launch), the number of
+ * workgroups and the lanes per workgroup.  A launcher call may launch several
+ * kernels (two halves of a large shape, split + join); this is the last one.
+ * Either pointer may be NULL.  No counterpart in the reference, whose launches
+ * take the caller's block_dim as given; here block_dim 0 leaves the grid to
+ * the launcher and a runner reports what it chose. */
+const char *afir_hip_last_launch(uint32_t *workgroups, uint32_t *threads);
+
 /* ---- fused elementwise chain: out = (a + b) * b ---------------------------
  * Replaces the lowering of afir.add -> afir.mul
  * (lib/Conversion/AFIRToASCIR/Math/Elementwise.cpp:25-57; chain from

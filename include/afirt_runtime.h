@@ -69,6 +69,20 @@ int afirt_executor_run_file(AfirtExecutor executor, const char *binary_path,
                             size_t tiling_len, int block_dim, uint32_t magic, char *err_buf,
                             size_t err_len);
 
+/* No counterpart in the reference.  What the executor's last successful run
+ * launched: the kernel's device time in ns (HIP events around the launch; the
+ * reference reports its simulator's cycle count through trace.json only), the
+ * number of workgroups and lanes per workgroup of the last kernel, and its name
+ * (truncated into kernel_name).  Any out pointer may be NULL.  Returns non-zero
+ * when there has been no such run.
+ *
+ * block_dim of the two run calls above is the reference's unit, a number of
+ * Ascend AI cores (its callers pass 1, 8 and 40).  It does not size the HIP
+ * grid: the launcher does, for the device's compute units.  A process that
+ * really means workgroups sets AFIR_HIP_HONOUR_BLOCK_DIM=1. */
+int afirt_executor_last_launch(AfirtExecutor executor, int64_t *kernel_ns, uint32_t *workgroups,
+                               uint32_t *threads, char *kernel_name, size_t name_len);
+
 #ifdef __cplusplus
 }
 #endif

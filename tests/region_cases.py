@@ -35,6 +35,24 @@ MEAN_ROWBIAS = REDUCE_ROWBIAS.replace("  reduce sum\n", "  reduce sum\n  const a
 REDUCE_TAIL_CHAIN = REDUCE_ROWBIAS.replace(
     "  reduce sum\n", "  reduce sum\n  const 0.5\n  mul\n  neg\n  const 4\n  add\n  relu\n  const arg1.1\n  const 0.5\n  mul\n  mul\n")
 
+# extents outside the tail: out[m,n] = f16(b[m,n] / f16(N) * f32(M)) per element, and a row sum of
+# terms that were divided by the extent first, c[m] = f16(sum_n ((a[m] + b[m,n]) / N) * M)
+PARALLEL_DIV_EXTENT = HEADER + """
+arg in f16 2
+arg out f16 2
+segment 2
+  size arg0.0 arg0.1
+  outoff 0
+  push arg0 d0 d1
+  const arg0.1 f16
+  div
+  const arg0.0
+  mul
+  store
+end
+"""
+PRE_REDUCE_DIV_EXTENT = REDUCE_ROWBIAS.replace("  add\n  reduce sum\n", "  add\n  const arg1.1\n  div\n  reduce sum\n  const arg1.0\n  mul\n")
+
 # out[n,m] = f16(relu(data0[m,0]) + data1[n,m])   examples/relu-broadcast-transpose
 RELU_COL_ADD = HEADER + """
 arg in f16 2
@@ -253,6 +271,23 @@ def case_mean_rowbias(m=640, n=512, seed=42):
     return MEAN_ROWBIAS, [a, b], mean_rowbias_f16(a, b)
 
 
+def case_parallel_div_extent(m=70, n=333, seed=5):
+    rng = np.random.default_rng(seed)
+    b = _u(rng, (m, n), -4.0, 4.0)
+    want = b.astype(np.float32) / np.float32(np.float16(n)) * np.float32(m)
+    return PARALLEL_DIV_EXTENT, [b], want.astype(np.float16)
+
+
+def case_pre_reduce_div_extent(m=96, n=256, seed=6):
+    """Small integers over a power-of-two N: every quotient and every partial sum is exact in
+    float32, so the result does not depend on the order of the sum."""
+    rng = np.random.default_rng(seed)
+    a = rng.integers(-4, 5, (m,)).astype(np.float16)
+    b = rng.integers(-4, 5, (m, n)).astype(np.float16)
+    terms = (a.astype(np.float32)[:, None] + b.astype(np.float32)) / np.float32(n)
+    return PRE_REDUCE_DIV_EXTENT, [a, b], (terms.sum(axis=1, dtype=np.float32) * np.float32(m)).astype(np.float16)
+
+
 def case_reduce_tail_chain(m=77, n=300, seed=9):
     rng = np.random.default_rng(seed)
     a, b = _u(rng, (m,)), _u(rng, (m, n), -0.1, 0.1)
@@ -326,6 +361,7 @@ EXACT_CASES = {
     "add_broadcast_concat": case_add_broadcast_concat,
     "split_relu_brc_add_mul": case_split_relu_brc_add_mul,
     "c1": case_c1, "c3": case_c3, "c4": case_c4, "add_mul_3": case_add_mul_3,
+    "parallel_div_extent": case_parallel_div_extent, "pre_reduce_div_extent": case_pre_reduce_div_extent,
 }
 REDUCE_CASES = {"reduce_rowbias": case_reduce_rowbias, "c2": case_c2, "mean_rowbias": case_mean_rowbias,
                 "reduce_tail_chain": case_reduce_tail_chain}

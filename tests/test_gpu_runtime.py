@@ -214,3 +214,89 @@ def test_cli_validation_failure_exit_code(tmp_path):
     p = _rs("--run-manifest", str(tmp_path / "m.json"), "--run")
     assert p.returncode == 2
     assert "session.validation=fail" in p.stderr and "session.error_stage=validate" in p.stderr
+
+
+# ------------------------------------- block_dim of the reference's callers --
+
+def _full_size(family):
+    if family == "fused_add_mul":
+        a, b = O.gen_c1((4096, 4096))
+        return ([a, b], np.empty_like(a), dict(dim_arg0_0=4096, dim_arg0_1=4096), O.golden_c1(a, b))
+    table, idx, scale, shift = O.gen_c4(131072, 1024, 32768)
+    return ([table, idx, scale, shift], np.empty((32768, 1024), np.float16),
+            dict(dim_arg0_0=131072, dim_arg0_1=1024, dim_arg1_0=32768), O.golden_c4(table, idx, scale, shift))
+
+
+@pytest.mark.parametrize("family", ["fused_add_mul", "gather_scale_shift"])
+def test_reference_block_dim_values_do_not_size_the_grid(R, executor, tmp_path, family):
+    """The reference's callers pass an Ascend AI-core count as block_dim: 1 by default
+    (python/runtime/executor.py:183), 8 (test/tools/runtime/test_capi_runtime.cpp:171-174),
+    40 (examples/broadcast-add-reduce/run.sh:259).  Through afirt_executor_run those values must
+    reach the same kernel on the same grid, at the same speed, as the launcher's own choice, at
+    the benchmark's full size, bit-exact against the oracle."""
+    _, binary = _compile(R, tmp_path, family)
+    inputs, out, dims, want = _full_size(family)
+    tiling = R.TilingSchema.for_kernel(family).pack(**dims)
+    seen = {}
+    for block_dim in (0, 1, 8, 40):
+        best = None
+        for _ in range(3):                      # the fastest of three: a first launch runs at idle clocks
+            out[...] = 0
+            got = executor.execute(binary, family, inputs, [out], tiling, block_dim=block_dim)
+            assert got[0].tobytes() == want.tobytes(), block_dim
+            note = executor.runtime.last_launch()
+            best = note if best is None or note["kernel_ns"] < best["kernel_ns"] else best
+        seen[block_dim] = best
+    base = seen[0]
+    assert base["workgroups"] >= 1024 and "phased" in base["kernel"], base
+    for block_dim in (1, 8, 40):
+        s = seen[block_dim]
+        assert (s["kernel"], s["workgroups"], s["threads"]) == (base["kernel"], base["workgroups"], base["threads"])
+        assert s["kernel_ns"] <= 1.10 * base["kernel_ns"], (block_dim, s, base)
+
+
+def test_block_dim_sizes_the_grid_only_on_request(R, executor, tmp_path, monkeypatch):
+    """AFIR_HIP_HONOUR_BLOCK_DIM=1 makes a positive block_dim the number of workgroups; a run
+    manifest says the same with "hip_grid", and the session reports the grid that ran."""
+    _, binary = _compile(R, tmp_path, "fused_add_mul")
+    a, b = O.gen_c1((300, 1000))
+    tiling = R.TilingSchema.for_kernel("fused_add_mul").pack(dim_arg0_0=300, dim_arg0_1=1000)
+    out = np.empty_like(a)
+    executor.execute(binary, "fused_add_mul", [a, b], [out], tiling, block_dim=8)
+    auto = executor.runtime.last_launch()
+    assert auto["workgroups"] > 8
+    monkeypatch.setenv("AFIR_HIP_HONOUR_BLOCK_DIM", "1")
+    executor.execute(binary, "fused_add_mul", [a, b], [out], tiling, block_dim=8)
+    assert executor.runtime.last_launch()["workgroups"] == 8
+    assert out.tobytes() == O.golden_c1(a, b).tobytes()
+    executor.execute(binary, "fused_add_mul", [a, b], [out], tiling, block_dim=0)
+    assert executor.runtime.last_launch()["workgroups"] == auto["workgroups"]
+    monkeypatch.delenv("AFIR_HIP_HONOUR_BLOCK_DIM")
+
+    src = _descriptor(tmp_path, "fused_add_mul")
+    art = tmp_path / "artifact"
+    assert _rs("--kernel", str(src), "--output", str(art), "--name", "k").returncode == 0
+    np.save(tmp_path / "a.npy", a)
+    np.save(tmp_path / "b.npy", b)
+    np.save(tmp_path / "e.npy", O.golden_c1(a, b))
+    (tmp_path / "ts.json").write_text(json.dumps(
+        {"tiling_params": [{"name": "dim_arg0_0"}, {"name": "dim_arg0_1"}]}))
+    m = {"task_id": "main", "backend": "hip", "artifact_root": str(art),
+         "inputs": [{"name": "a", "path": str(tmp_path / "a.npy")},
+                    {"name": "b", "path": str(tmp_path / "b.npy")}],
+         "outputs": [{"name": "o", "path": str(tmp_path / "o.npy")}],
+         "expected_outputs": [{"name": "o", "path": str(tmp_path / "e.npy")}],
+         "tiling": {"schema": str(tmp_path / "ts.json"), "params": "dim_arg0_0=300,dim_arg0_1=1000"},
+         "block_dim": 40, "atol": 0, "rtol": 0}
+    (tmp_path / "m.json").write_text(json.dumps(m))
+    p = _rs("--run-manifest", str(tmp_path / "m.json"), "--run")
+    assert p.returncode == 0, p.stdout + p.stderr
+    assert "session.runtime.attribute.grid_source=launcher" in p.stdout
+    assert f"session.runtime.attribute.grid={auto['workgroups']}x{auto['threads']}" in p.stdout
+    assert "session.runtime.counter.block_dim=40" in p.stdout
+    m["hip_grid"] = 24
+    (tmp_path / "m.json").write_text(json.dumps(m))
+    p = _rs("--run-manifest", str(tmp_path / "m.json"), "--run")
+    assert p.returncode == 0, p.stdout + p.stderr
+    assert "session.runtime.attribute.grid_source=hip_grid" in p.stdout
+    assert "session.runtime.attribute.grid=24x" in p.stdout

@@ -245,11 +245,31 @@ def test_emit_options_change_the_tile_and_the_unroll(tmp_path):
 
 def test_operations_after_reduce_sum_are_applied_to_the_row_sum_where_it_is_stored():
     src = _emit(RC.MEAN_ROWBIAS).stdout
-    assert "float tail_const[4];" in src
-    assert src.count("(s / R.tail_const[0])") >= 4          # every kernel that stores a row sum
+    assert "float extent_const[8];" in src
+    assert src.count("(s / R.extent_const[0])") >= 4        # every kernel that stores a row sum
     assert "v0[u][e] / " not in src                          # not per element
     chain = _emit(RC.REDUCE_TAIL_CHAIN).stdout
     half, four = "as_f32(0x3f000000u) /* 0.5 */", "as_f32(0x40800000u) /* 4 */"
-    assert f"(fmax_ieee(((-(s * {half})) + {four}), 0.f) * (R.tail_const[0] * {half}))" in chain
+    assert f"(fmax_ieee(((-(s * {half})) + {four}), 0.f) * (R.extent_const[0] * {half}))" in chain
     plain = _emit(RC.REDUCE_ROWBIAS).stdout
-    assert "R.tail_const" not in plain.split("struct SpecArgs", 1)[1].split("};", 1)[1]
+    assert "R.extent_const" not in plain.split("struct SpecArgs", 1)[1].split("};", 1)[1]
+
+
+def test_extent_constants_outside_the_tail_are_launch_arguments_too():
+    """An extent is not known when the kernel is emitted: wherever it stands in the segment it
+    is read from the launch arguments, numbered in program order (a literal 0 there once made
+    `x / N` a division by zero on the compiled route only)."""
+    par = _emit(RC.PARALLEL_DIV_EXTENT)
+    assert par.returncode == 0, par.stderr
+    assert "= R.extent_const[0];" in par.stdout and "= R.extent_const[1];" in par.stdout
+    assert "as_f32(0x00000000u)" not in par.stdout.split("KERNEL void", 1)[0].split("segment0", 1)[1]
+    pre = _emit(RC.PRE_REDUCE_DIV_EXTENT).stdout
+    assert "= R.extent_const[0];" in pre                    # per element, before the sum
+    assert src_count(pre, "(s * R.extent_const[1])") >= 4   # on the sum, numbered after it
+    many = RC.PARALLEL_DIV_EXTENT.replace("  const arg0.0\n  mul\n", "  const arg0.0\n  mul\n" * 8)
+    p = _emit(many)
+    assert p.returncode != 0 and "more than 8 extent constants in a segment" in p.stderr
+
+
+def src_count(src, needle):
+    return src.count(needle)

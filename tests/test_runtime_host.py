@@ -372,6 +372,15 @@ def test_cli_profiling_writes_trace_and_retained_summary(tmp_path):
     assert summary["total_score"] == summary["total_cycle_count"] == 12500
     assert summary["runtime"]["counters"]["kernel_ns"] == 12500
     assert summary["runtime"]["attributes"]["kernel_name"] == "example"
+    # block_dim is the reference's AI-core count: recorded, never the grid; "hip_grid" is one
+    assert kv["session.runtime.counter.block_dim"] == "3"
+    assert kv["session.runtime.attribute.grid_source"] == "launcher" and kv["session.runtime.attribute.grid"] == "2048x256"
+    p = subprocess.run([RS, "--run-manifest", _manifest(tmp_path, block_dim=40, hip_grid=24), "--run",
+                        "--testing-driver=hip-success"], capture_output=True, text=True, env=dict(os.environ, TMPDIR=str(tmp)))
+    assert "session.runtime.attribute.grid=24x256" in p.stdout and "session.runtime.attribute.grid_source=hip_grid" in p.stdout
+    p = subprocess.run([RS, "--run-manifest", _manifest(tmp_path, hip_grid=-1), "--run", "--testing-driver=hip-success"],
+                       capture_output=True, text=True)
+    assert p.returncode == 4 and "hip_grid must be between" in p.stderr
     # without "profiling" nothing is written
     p = subprocess.run([RS, "--run-manifest", _manifest(tmp_path), "--run", "--testing-driver=hip-success"],
                        capture_output=True, text=True, env=dict(os.environ, TMPDIR=str(tmp)))
