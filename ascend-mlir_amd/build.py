@@ -159,33 +159,46 @@ def build_families(kernel_lib):
 
 
 def build_probes():
-    """libafir_bench_probes.so: ceiling probes for bench.py (csrc/bench/probes.h), and the
-    direct-to-LDS matmul kernel compiled three more times with parts of its K loop left out, each
-    under a namespace name of its own."""
+    """libafir_bench_probes.so: ceiling probes for bench.py (csrc/bench/probes.h), among them
+    the direct-to-LDS matmul kernel instantiated with parts of its K loop left out
+    (csrc/bench/matmul_feed_probes.h)."""
     os.makedirs(LIB, exist_ok=True)
     os.makedirs(OBJ, exist_ok=True)
-    jobs = [("bench/probes.hip", "bench_probes.o", [])]
-    for level in (1, 2, 3):
-        jobs.append(("kernels/matmul_dma.hip", f"bench_matmul_ablate{level}.o",
-                     [f"-DAFIR_MM_ABLATE={level}", f"-Dafir=afir_abl{level}"]))
-
-    def one(job):
-        src, name, extra = job
-        obj = os.path.join(OBJ, name)
-        _run([HIPCC, *COMMON, *extra, "-x", "hip", "-c", os.path.join(CSRC, src), "-o", obj])
-        return obj
-    with cf.ThreadPoolExecutor(max_workers=3) as ex:
-        objs = list(ex.map(one, jobs))
+    obj = os.path.join(OBJ, "bench_probes.o")
+    _run([HIPCC, *COMMON, "-x", "hip", "-c", os.path.join(CSRC, "bench/probes.hip"), "-o", obj])
     out = os.path.join(LIB, "libafir_bench_probes.so")
-    _run([HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", out, *objs])
+    _run([HIPCC, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", out, obj])
     return out
 
 
+def _source_closure(src):
+    """Text of a source file and of every header of this tree it includes, directly or not."""
+    import re
+    seen, todo, text = set(), [os.path.join(CSRC, src)], []
+    while todo:
+        path = os.path.normpath(todo.pop())
+        if path in seen or not os.path.exists(path):
+            continue
+        seen.add(path)
+        body = open(path).read()
+        text.append(body)
+        for inc in re.findall(r'^\s*#\s*include\s+"([^"]+)"', body, flags=re.M):
+            todo.append(os.path.join(os.path.dirname(path), inc))
+            todo.append(os.path.join(ROOT, "include", inc))
+    return "\n".join(text)
+
+
 def build_variant(out, defines):
-    """The kernel library with extra -D flags.  Sources that mention none of the macros keep
-    their ordinary objects (compiled here if the build directory does not hold them)."""
+    """The kernel library with extra -D flags.  A source is recompiled with them when it, or a
+    header it includes, uses one of the macros (as a whole identifier); the others keep their
+    ordinary objects (compiled here if the build directory does not hold them).  A macro that
+    no source uses is an error: the variant would be the shipped library under another name."""
     import re
     names = [re.match(r"-D([A-Za-z_0-9]+)", d).group(1) for d in defines]
+    closures = {src: _source_closure(src) for src, _ in KERNEL_SOURCES}
+    for n in names:
+        if not any(re.search(r"\b" + re.escape(n) + r"\b", t) for t in closures.values()):
+            raise SystemExit(f"build.py --variant: no kernel source or header uses {n}")
     tag = "_".join(d[2:].replace("=", "-") for d in defines) or "base"
     vdir = os.path.join(os.path.dirname(os.path.abspath(out)), "obj_" + tag)
     os.makedirs(vdir, exist_ok=True)
@@ -193,8 +206,7 @@ def build_variant(out, defines):
 
     def one(item):
         src, extra = item
-        text = open(os.path.join(CSRC, src)).read()
-        touched = any(n in text for n in names)
+        touched = any(re.search(r"\b" + re.escape(n) + r"\b", closures[src]) for n in names)
         obj = os.path.join(vdir if touched else OBJ, src.replace("/", "_") + ".o")
         if touched or not os.path.exists(obj):
             _run([HIPCC, *COMMON, *extra, *(defines if touched else []), "-x", "hip", "-c",

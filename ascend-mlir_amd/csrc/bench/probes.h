@@ -30,8 +30,8 @@ extern "C" {
 uint32_t afir_bench_mfma_rate(void *stream, const void *operands, void *sink, uint32_t iters,
                               uint64_t *flops);
 
-/* The direct-to-LDS matmul kernel (csrc/kernels/matmul_dma.hip, compiled a second
- * and third time for this library) with parts of its K loop removed, so that a
+/* The direct-to-LDS matmul kernel (csrc/kernels/matmul_dma_kernel.h, instantiated here
+ * with the feed policies of matmul_feed_probes.h) with parts of its K loop removed, so that a
  * matmul's distance from the register-only MFMA rate can be split into its
  * causes on the workload's own operands:
  *   what = 1  no global -> LDS feed after the prologue: the MFMAs, their LDS
@@ -41,7 +41,11 @@ uint32_t afir_bench_mfma_rate(void *stream, const void *operands, void *sink, ui
  *             reads filled, waits and barriers remain;
  *   what = 3  the whole kernel, but every global -> LDS load reads the same
  *             1 KiB: the loads are issued and write LDS as always, without the
- *             L2 / fabric / HBM traffic and latency behind them.
+ *             L2 / fabric / HBM traffic and latency behind them;
+ *   what = 4  the whole kernel with real addresses, but the walk over K wraps
+ *             after 256 k, so that an XCD's operand panels stay in its L2:
+ *             every load is an L2 hit (1 -> 3 -> 4 -> the kernel: issue cost,
+ *             cost of L2 hits, cost of L2 misses).
  * Same arguments as the kernel's launcher (bf16 A [m,k], B [k,n], bias [n], out
  * [m,n]; m, n multiples of 256, k of 64); the output is meaningless. */
 uint32_t afir_bench_matmul_ablated(void *stream, const void *a, const void *b, const void *bias,

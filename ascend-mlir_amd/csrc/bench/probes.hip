@@ -12,6 +12,7 @@
 #include "probes.h"
 
 #include "../kernels/kernels.h"
+#include "matmul_feed_probes.h"
 
 namespace afir {
 
@@ -49,24 +50,6 @@ __global__ __launch_bounds__(kProbeThreads) void mfma_rate_probe(const u32x4 *__
 }
 
 }  // namespace afir
-
-// csrc/kernels/matmul_dma.hip compiled with -DAFIR_MM_ABLATE=1 / 2 / 3 and -Dafir=afir_abl1 / 2 / 3
-namespace afir_abl1 {
-struct LaunchStatus { uint32_t code; const char *message; };
-LaunchStatus launch_matmul_dma(const uint16_t *a, const uint16_t *b, const uint16_t *bias, uint16_t *out, int m,
-                               int k, int n, float alpha, bool relu, uint32_t block_dim, hipStream_t stream);
-bool matmul_dma_supported(int64_t m, int64_t k, int64_t n);
-}  // namespace afir_abl1
-namespace afir_abl2 {
-struct LaunchStatus { uint32_t code; const char *message; };
-LaunchStatus launch_matmul_dma(const uint16_t *a, const uint16_t *b, const uint16_t *bias, uint16_t *out, int m,
-                               int k, int n, float alpha, bool relu, uint32_t block_dim, hipStream_t stream);
-}  // namespace afir_abl2
-namespace afir_abl3 {
-struct LaunchStatus { uint32_t code; const char *message; };
-LaunchStatus launch_matmul_dma(const uint16_t *a, const uint16_t *b, const uint16_t *bias, uint16_t *out, int m,
-                               int k, int n, float alpha, bool relu, uint32_t block_dim, hipStream_t stream);
-}  // namespace afir_abl3
 
 namespace {
 
@@ -178,14 +161,16 @@ uint32_t afir_bench_mfma_rate(void *stream, const void *operands, void *sink, ui
 
 uint32_t afir_bench_matmul_ablated(void *stream, const void *a, const void *b, const void *bias, void *out, int m,
                                    int k, int n, int what) {
-  if (!a || !b || !bias || !out || (what < 1 || what > 3) || !afir_abl1::matmul_dma_supported(m, k, n)) return 1u;
+  namespace dma = afir::dma;
+  if (!a || !b || !bias || !out || (what < 1 || what > 4) || !dma::supported(m, k, n)) return 1u;
   const uint16_t *pa = static_cast<const uint16_t *>(a), *pb = static_cast<const uint16_t *>(b);
-  const uint16_t *pbias = static_cast<const uint16_t *>(bias);
-  uint16_t *po = static_cast<uint16_t *>(out);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  if (what == 1) return afir_abl1::launch_matmul_dma(pa, pb, pbias, po, m, k, n, 0.01f, false, 0, st).code;
-  if (what == 2) return afir_abl2::launch_matmul_dma(pa, pb, pbias, po, m, k, n, 0.01f, false, 0, st).code;
-  return afir_abl3::launch_matmul_dma(pa, pb, pbias, po, m, k, n, 0.01f, false, 0, st).code;
+  switch (what) {
+    case 1: return dma::launch<false, dma::NoLoads>("matmul_dma_no_loads", pa, pb, bias, out, m, k, n, 0.01f, false, 0, st).code;
+    case 2: return dma::launch<false, dma::NoLoadsNoReads>("matmul_dma_no_loads_no_reads", pa, pb, bias, out, m, k, n, 0.01f, false, 0, st).code;
+    case 3: return dma::launch<false, dma::LoadsOfOneKiB>("matmul_dma_loads_of_one_kib", pa, pb, bias, out, m, k, n, 0.01f, false, 0, st).code;
+    default: return dma::launch<false, dma::L2Resident>("matmul_dma_l2_resident", pa, pb, bias, out, m, k, n, 0.01f, false, 0, st).code;
+  }
 }
 
 uint32_t afir_bench_copy(void *stream, const void *src, void *dst, size_t bytes) {

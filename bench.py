@@ -411,13 +411,14 @@ def make_workload(key, torch, H, O, C):
             vendor = lambda i: torch.matmul(sets[i % len(sets)][0], sets[i % len(sets)][1])
             # alternating rounds: each kernel sees the same thermal history
             rounds = {"this_kernel": [], "vendor_gemm": [], "no_feed": [], "no_feed_no_lds_reads": [],
-                      "loads_of_one_kib": []}
+                      "loads_of_one_kib": [], "l2_resident": []}
             for _ in range(3):
                 rounds["vendor_gemm"].append(rate(vendor))
                 rounds["this_kernel"].append(rate(ours))
                 rounds["no_feed"].append(rate(ablated(1)))
                 rounds["no_feed_no_lds_reads"].append(rate(ablated(2)))
                 rounds["loads_of_one_kib"].append(rate(ablated(3)))
+                rounds["l2_resident"].append(rate(ablated(4)))
             med = lambda v: round(sorted(v)[len(v) // 2], 1)
             ev = {"mfma_only_workload_operands_tflops": round(P.mfma_rate(sets[0][0]), 1),
                   "vendor_gemm_tflops": med(rounds["vendor_gemm"]),
@@ -428,7 +429,8 @@ def make_workload(key, torch, H, O, C):
                       "mfma_waits_barriers": med(rounds["no_feed_no_lds_reads"]),
                       "plus_lds_operand_reads": med(rounds["no_feed"]),
                       "plus_load_issue_and_lds_writes": med(rounds["loads_of_one_kib"]),
-                      "plus_memory_system_behind_the_loads": med(rounds["this_kernel"])}}
+                      "plus_l2_hits_operands_resident_in_l2": med(rounds["l2_resident"]),
+                      "plus_l2_misses_the_kernel": med(rounds["this_kernel"])}}
             ones = torch.ones((8192, 8192), dtype=torch.bfloat16, device="cuda")
             ev["mfma_only_constant_operands_tflops"] = round(P.mfma_rate(ones), 1)
             launch = H.prepare(w.symbol, [ones.data_ptr(), ones.data_ptr(), sets[0][2].data_ptr(),
