@@ -42,6 +42,30 @@ inline bool phased_enabled() {
   const char *env = getenv("AFIR_HIP_PHASED");
   return !(env && env[0] == '0');
 }
+// A tuning constant that a deployer can change without rebuilding: the value of the environment
+// variable `name` when it is set to an integer within [lo, hi], else `fallback` (the compile-time
+// choice, which is what the tile searches found on a whole MI355X).  Read at every launch, so a
+// search can step through values within one process.
+inline int env_int(const char *name, int fallback, int lo, int hi) {
+  const char *env = getenv(name);
+  if (!env || !*env) return fallback;
+  char *end = nullptr;
+  const long v = strtol(env, &end, 10);
+  return (end && *end == '\0' && v >= lo && v <= hi) ? (int)v : fallback;
+}
+// Workgroups of `kernel` that fit a compute unit at once, given its workgroup size and the
+// dynamic LDS of the launch (registers and static LDS are the kernel's own): what a launch that
+// wants all of its lanes resident together may count on.  0 if the runtime cannot say.
+template <typename Kernel>
+inline int resident_blocks_per_cu(Kernel kernel, int threads, size_t dynamic_lds) {
+  int blocks = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&blocks, reinterpret_cast<const void *>(kernel), threads,
+                                                   dynamic_lds) != hipSuccess) {
+    (void)hipGetLastError();
+    return 0;
+  }
+  return blocks;
+}
 inline int wall_clock_khz() {
   static const int khz = [] {
     int device = 0, value = 0;

@@ -155,15 +155,17 @@ LaunchStatus launch_fused_add_mul(const float *a, const float *b, float *out, in
   // whole blocks of a launch of up to twice the chip's resident lanes: the phased kernel
   // (kPhaseMaxLaunches); what is left over: below
   const size_t phased_blocks = n4 / kPhasedChunksPerBlock;
-  const size_t capacity = (size_t)device_cus() * kPhasedLanesPerCU / kThreads;   // blocks per launch
-  if (AFIR_ELTWISE_PHASED && !block_dim && phased_blocks >= (size_t)device_cus() * AFIR_ELTWISE_PHASED_MIN_WG_PER_CU &&
+  static const int fit = resident_blocks_per_cu(add_mul_f32_phased, kThreads, 0);   // workgroups per compute unit
+  const size_t capacity = fit >= kPhasedLanesPerCU / kThreads ? (size_t)device_cus() * kPhasedLanesPerCU / kThreads : 0;   // blocks per launch
+  const int base_ns = env_int("AFIR_ELTWISE_PHASE_BASE_NS", AFIR_ELTWISE_PHASE_BASE_NS, 0, 100000);
+  const int gbs = env_int("AFIR_ELTWISE_PHASE_GBS", AFIR_ELTWISE_PHASE_GBS, 100, 100000);
+  if (AFIR_ELTWISE_PHASED && !block_dim && capacity > 0 && phased_blocks >= (size_t)device_cus() * AFIR_ELTWISE_PHASED_MIN_WG_PER_CU &&
       phased_blocks <= kPhaseMaxLaunches * capacity && phased_enabled()) {
     const size_t launches = (phased_blocks + capacity - 1) / capacity;
     const size_t take = (phased_blocks + launches - 1) / launches;
     for (size_t b0 = 0; b0 < phased_blocks; b0 += take) {
       const size_t nblocks = phased_blocks - b0 < take ? phased_blocks - b0 : take;
-      const int hold_ticks = phase_hold_ticks((int64_t)(nblocks * kPhasedChunksPerBlock * 32), AFIR_ELTWISE_PHASE_BASE_NS,
-                                              AFIR_ELTWISE_PHASE_GBS);
+      const int hold_ticks = phase_hold_ticks((int64_t)(nblocks * kPhasedChunksPerBlock * 32), base_ns, gbs);
       AFIR_LAUNCH("add_mul_f32_phased", add_mul_f32_phased, dim3((unsigned)nblocks), dim3(kThreads), 0, stream,
                          reinterpret_cast<const f32x4 *>(a) + b0 * kPhasedChunksPerBlock,
                          reinterpret_cast<const f32x4 *>(b) + b0 * kPhasedChunksPerBlock,

@@ -363,18 +363,29 @@ LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx
   // over, and larger gathers: below.
   const int64_t phased_rows_per_block = (int64_t)(kPhasedThreads >> (lanes_log2 < 8 ? lanes_log2 : 8)) * kPhasedPasses;
   const int64_t phased_blocks = nidx / phased_rows_per_block;
-  if (AFIR_GATHER_PHASED && vec && ((int64_t)kGroups << lanes_log2) == chunks64 && !block_dim &&
-      (1 << lanes_log2) <= kPhasedThreads && phased_blocks > 0 &&
-      phased_blocks <= kPhaseMaxLaunches * ((int64_t)device_cus() * kPhasedLanesPerCU / kPhasedThreads) && phased_enabled()) {
-    const size_t lds = (size_t)2 * (kGroups << lanes_log2) * 16;   // scale and shift, 16-byte chunks
-    const int64_t capacity = (int64_t)device_cus() * kPhasedLanesPerCU / kPhasedThreads;   // blocks per launch
+  // blocks per launch: what is resident at once.  Rows of 8192 halves park 32 KiB of scale / shift
+  // per workgroup in LDS, and then five workgroups fit a compute unit, not eight.
+  const size_t lds = (size_t)2 * (kGroups << lanes_log2) * 16;   // scale and shift, 16-byte chunks
+  int64_t capacity = 0;
+  if (AFIR_GATHER_PHASED && vec && lanes_log2 <= 8 && (1 << lanes_log2) <= kPhasedThreads) {
+    static int fit[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};   // per row length, asked once (0: not yet)
+    if (fit[lanes_log2] == 0) {
+      const int n = resident_blocks_per_cu(gather_scale_shift_f16_phased, kPhasedThreads, lds);
+      fit[lanes_log2] = n > 0 ? n : -1;
+    }
+    const int wanted = kPhasedLanesPerCU / kPhasedThreads;
+    capacity = (int64_t)device_cus() * (fit[lanes_log2] < wanted ? (fit[lanes_log2] > 0 ? fit[lanes_log2] : 0) : wanted);
+  }
+  if (AFIR_GATHER_PHASED && vec && ((int64_t)kGroups << lanes_log2) == chunks64 && !block_dim && capacity > 0 &&
+      phased_blocks > 0 && phased_blocks <= kPhaseMaxLaunches * capacity && phased_enabled()) {
+    const int base_ns = env_int("AFIR_GATHER_PHASE_BASE_NS", AFIR_GATHER_PHASE_BASE_NS, 0, 100000);
+    const int gbs = env_int("AFIR_GATHER_PHASE_GBS", AFIR_GATHER_PHASE_GBS, 100, 100000);
     const int64_t launches = (phased_blocks + capacity - 1) / capacity;
     const int64_t take = (phased_blocks + launches - 1) / launches;
     for (int64_t b0 = 0; b0 < phased_blocks; b0 += take) {
       const int64_t nblocks = phased_blocks - b0 < take ? phased_blocks - b0 : take;
       const int64_t row0 = b0 * phased_rows_per_block;
-      const int hold_ticks = phase_hold_ticks(nblocks * phased_rows_per_block * dim * 2, AFIR_GATHER_PHASE_BASE_NS,
-                                              AFIR_GATHER_PHASE_GBS);
+      const int hold_ticks = phase_hold_ticks(nblocks * phased_rows_per_block * dim * 2, base_ns, gbs);
       AFIR_LAUNCH("gather_scale_shift_f16_phased", gather_scale_shift_f16_phased, dim3((unsigned)nblocks), dim3(kPhasedThreads), lds, stream,
                          table, idx + row0, scale, shift, out + row0 * dim, error_flag, (uint32_t)rows, lanes_log2,
                          hold_ticks);
@@ -390,7 +401,6 @@ LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx
     int64_t blocks = (nidx + rows_per_block - 1) / rows_per_block;
     if (blocks > (int64_t)device_cus() * AFIR_GATHER_GROUPED_WG_PER_CU) blocks = (int64_t)device_cus() * AFIR_GATHER_GROUPED_WG_PER_CU;
     if (block_dim) blocks = block_dim;
-    const size_t lds = (size_t)2 * (kGroups << lanes_log2) * 16;   // scale and shift, 16-byte chunks
     AFIR_LAUNCH("gather_scale_shift_f16_grouped", gather_scale_shift_f16_grouped, dim3((unsigned)blocks), dim3(kGroupedThreads), lds,
                        stream, table, idx, scale, shift, out, error_flag, (uint32_t)rows, lanes_log2,
                        nidx);

@@ -270,7 +270,10 @@ LaunchStatus launch_relu_broadcast_add_transpose(const uint16_t *x, const uint16
   // The phased kernel wants every lane of a launch resident at once: a shape of up to twice that
   // goes out as two launches of whole batches (kPhaseMaxLaunches).
   const int64_t groups_per_batch = tiled && n % (kSmallTile * kPhasedTiles) == 0 ? (m / kSmallTile) * (n / (kSmallTile * kPhasedTiles)) : 0;
-  const int64_t capacity = (int64_t)device_cus() * kPhasedLanesPerCU / kThreads;   // groups per launch
+  static const int fit = resident_blocks_per_cu(relu_bcast_add_transpose_f16_phased, kThreads, 0);   // workgroups per compute unit
+  const int64_t capacity = fit >= kPhasedLanesPerCU / kThreads ? (int64_t)device_cus() * kPhasedLanesPerCU / kThreads : 0;   // groups per launch
+  const int base_ns = env_int("AFIR_TRANSPOSE_PHASE_BASE_NS", AFIR_TRANSPOSE_PHASE_BASE_NS, 0, 100000);
+  const int gbs = env_int("AFIR_TRANSPOSE_PHASE_GBS", AFIR_TRANSPOSE_PHASE_GBS, 100, 100000);
   if (AFIR_TRANSPOSE_PHASED && !block_dim && groups_per_batch > 0 && groups_per_batch <= capacity &&
       nb * groups_per_batch >= (int64_t)device_cus() * kPhasedMinGroupsPerCU && (int64_t)32 * m * 2 < ((int64_t)1 << 31) &&
       (nb + capacity / groups_per_batch - 1) / (capacity / groups_per_batch) <= kPhaseMaxLaunches && phased_enabled()) {
@@ -279,7 +282,7 @@ LaunchStatus launch_relu_broadcast_add_transpose(const uint16_t *x, const uint16
     const int64_t take = (nb + launches - 1) / launches;
     for (int64_t b0 = 0; b0 < nb; b0 += take) {
       const int64_t nbl = nb - b0 < take ? nb - b0 : take;
-      const int hold_ticks = phase_hold_ticks(nbl * m * n * 2, AFIR_TRANSPOSE_PHASE_BASE_NS, AFIR_TRANSPOSE_PHASE_GBS);
+      const int hold_ticks = phase_hold_ticks(nbl * m * n * 2, base_ns, gbs);
       AFIR_LAUNCH("relu_bcast_add_transpose_f16_phased", relu_bcast_add_transpose_f16_phased, dim3((unsigned)(nbl * groups_per_batch)), dim3(kThreads), 0,
                          stream, x + b0 * m * n, c, out + b0 * m * n, (int)nbl, (int)m, (int)n, hold_ticks);
     }

@@ -30,6 +30,12 @@
 // bin/ directory; needs hipcc) and the candidate is launched from that library.
 // Like emit_* it is not part of the TilingData bytes.
 //
+// A parameter named env_<NAME> is a launch-time choice of the hand-tuned kernels
+// that they read from the environment (the AFIR_*_PHASE_GBS / _BASE_NS holds of
+// the kernels that separate reads from writes): the candidate runs with NAME set
+// to the value, in this process and from the one shipped library.  Not part of
+// the TilingData bytes either.
+//
 // Exit codes: 0 ok, 1 no candidate passed, 2 run error, 4 bad invocation.
 #include <cctype>
 #include <cmath>
@@ -70,7 +76,8 @@ struct Param {
 
 // Testing-only runner (--testing-driver=hip-success): no device, outputs stay
 // zero, and the reported kernel time shrinks with block_dim so that a search
-// has a defined winner.
+// has a defined winner; AFIR_TESTING_EXTRA_US in the environment is added to it
+// (what an env_* parameter looks like to a kernel that reads it).
 class TestingRunner final : public ExecutionRunner {
  public:
   ExecutionRunnerMode mode() const override { return ExecutionRunnerMode::Simulation; }
@@ -78,6 +85,7 @@ class TestingRunner final : public ExecutionRunner {
   Status runFile(const FileExecutionLaunch &, RunArgs &) override { return Status::success(); }
   Status runDynamicLibraryArtifact(const DynamicLibraryExecutionLaunch &, RunArgs &args) override {
     us_ = 1000.0 / (1 + args.block_dim);
+    if (const char *extra = getenv("AFIR_TESTING_EXTRA_US")) us_ += std::atof(extra);
     return Status::success();
   }
   double lastKernelMicroseconds() const override { return us_; }
@@ -327,8 +335,12 @@ int main(int argc, char **argv) {
     // tiling bytes in the order of the space
     std::vector<TilingField> fields;
     std::vector<std::pair<std::string, int64_t>> values;
-    std::map<std::string, int64_t> emitOptions, buildMacros;
+    std::map<std::string, int64_t> emitOptions, buildMacros, envValues;
     for (const Param &p : space) {
+      if (p.name.rfind("env_", 0) == 0) {
+        envValues[p.name.substr(4)] = vars[p.name];
+        continue;
+      }
       if (p.name.rfind("emit_", 0) == 0) {
         emitOptions[p.name.substr(5)] = vars[p.name];
         continue;
@@ -398,6 +410,17 @@ int main(int argc, char **argv) {
     launch.preferCodeObject = candidateArtifact.codeObjectPreferred;
     auto packed = TilingSchema::fromFields(fields).pack(values);
     if (!packed) return usage(packed.error().c_str());
+    // launch-time choices read from the environment: set for this combination's runs
+    struct EnvGuard {
+      std::vector<std::string> names;
+      ~EnvGuard() { for (const std::string &n : names) unsetenv(n.c_str()); }
+    } envGuard;
+    for (const auto &kv : envValues) {
+      for (char ch : kv.first)
+        if (!(std::isalnum((unsigned char)ch) || ch == '_')) return usage("env_* parameter names must be variable names");
+      setenv(kv.first.c_str(), std::to_string(kv.second).c_str(), 1);
+      envGuard.names.push_back(kv.first);
+    }
 
     for (int64_t bd : dims) {
       ++index;

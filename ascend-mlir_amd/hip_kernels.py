@@ -52,6 +52,7 @@ EXPORTED_SYMBOLS = [
     "afir_hip_region_prefer_code_object",
     "afir_hip_region_argument_bytes",
     "afir_hip_launch_region",
+    "afir_hip_last_launch",
 ]
 
 _lib = None
@@ -69,6 +70,8 @@ def load():
     L = ctypes.CDLL(KERNELS_LIB)
     vp, u32 = ctypes.c_void_p, ctypes.c_uint32
     L.afir_hip_last_error.restype = ctypes.c_char_p
+    L.afir_hip_last_launch.restype = ctypes.c_char_p
+    L.afir_hip_last_launch.argtypes = [ctypes.POINTER(u32), ctypes.POINTER(u32)]
     for name, nptr in [("afir_hip_launch_fused_add_mul", 5),
                        ("afir_hip_launch_broadcast_add_reducesum", 5),
                        ("afir_hip_launch_broadcast_add_reducesum_noalloc", 5),
@@ -88,6 +91,13 @@ def load():
                                   ctypes.POINTER(vp), vp, vp, ctypes.c_size_t]
     _lib = L
     return L
+
+
+def last_launch() -> dict:
+    """The kernel this thread launched last through the library, and its grid."""
+    wg, th = ctypes.c_uint32(0), ctypes.c_uint32(0)
+    name = load().afir_hip_last_launch(ctypes.byref(wg), ctypes.byref(th))
+    return {"kernel": (name or b"").decode(), "workgroups": wg.value, "threads": th.value}
 
 
 def kernel_table():

@@ -167,3 +167,22 @@ def test_kernel_library_variant_builds_only_what_the_macro_touches(tmp_path):
     bad = subprocess.run([sys.executable, os.path.join(ROOT, "ascend-mlir_amd", "build.py"), "--variant", str(out),
                           "AFIR_ELTWISE_UNROLL=4"], capture_output=True, text=True)
     assert bad.returncode != 0 and "usage" in bad.stderr
+
+
+def test_env_parameters_are_set_for_their_candidate_only(tmp_path):
+    """env_<NAME>: a launch-time choice the kernels read from the environment (the holds of the
+    kernels that separate reads from writes).  The candidate runs with NAME set, the value is
+    not part of the tiling bytes, and best_config.json records the winner."""
+    space = {"block_dim_values": [0],
+             "tiling_params": DIMS + [{"name": "env_AFIR_TESTING_EXTRA_US", "type": "int64", "values": [30, 10, 20]}]}
+    p = _at(*_setup(tmp_path, space), "--shape", "M=8,N=32", "--repeats", "2")
+    assert p.returncode == 0, p.stderr + p.stdout
+    lines = [l for l in p.stdout.splitlines() if l.startswith("[")]
+    assert len(lines) == 3
+    # the testing driver adds the variable's value (us) to its fixed 1000 us at block_dim 0
+    assert [l.split("score=")[1].split()[0] for l in lines] == ["1030000", "1010000", "1020000"]
+    best = json.loads((tmp_path / "best.json").read_text())
+    assert best["config"]["env_AFIR_TESTING_EXTRA_US"] == 10 and best["best"]["score"] == 1010000
+    bad = dict(space, tiling_params=DIMS + [{"name": "env_BAD-NAME", "type": "int64", "values": [1]}])
+    p = _at(*_setup(tmp_path, bad), "--shape", "M=8,N=32")
+    assert p.returncode == 4 and "variable names" in p.stderr

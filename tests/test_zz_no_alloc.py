@@ -68,3 +68,37 @@ def test_noalloc_rowsum_refuses_what_does_not_fit_the_scratch_array(H):
     assert rc == 4                          # AFIR_HIP_E_NOALLOC_LIMIT
     torch.cuda.synchronize()
     assert bool((y == 7).all())
+
+
+def test_noalloc_rowsum_replays_from_a_captured_graph(H):
+    """What the entry point is for: recorded into a HIP graph (after a first eager call on the
+    device, which looks the scratch array's address up) and replayed.  Every replay, with new
+    inputs written eagerly between the replays, gives what the ordinary entry point gives on
+    the same inputs: exactly, on small integers."""
+    import torch
+    m, n = 12, 3 * 8192 + 64                # split form: 12 rows x 4 chunks, the last one short
+    gen = torch.Generator(device="cuda").manual_seed(11)
+
+    def ints(shape):
+        return torch.randint(-4, 5, shape, generator=gen, device="cuda", dtype=torch.int32).float()
+
+    x, bias = ints((m, n)), ints((n,))
+    y = torch.empty((m,), dtype=torch.float32, device="cuda")
+    y_plain = torch.empty_like(y)
+    tiling = H.pack_tiling(m, n)
+    H.prepare(NOALLOC, [x.data_ptr(), bias.data_ptr(), y.data_ptr(), 0], tiling)()    # the warm first call
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        H.prepare(NOALLOC, [x.data_ptr(), bias.data_ptr(), y.data_ptr(), 0], tiling)()   # prepared inside: the capturing stream
+    plain = H.prepare(PLAIN, [x.data_ptr(), bias.data_ptr(), y_plain.data_ptr(), 0], tiling)
+    for replay in range(4):
+        x.copy_(ints((m, n)))
+        bias.copy_(ints((n,)))
+        plain()
+        y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, y_plain), replay
+        assert torch.equal(y.double(), x.double().sum(1) + bias.double().sum()), replay
