@@ -93,6 +93,10 @@ struct CompiledRegion {
   afir_target::EmitOptions options;   // read from the loaded module
   hipModule_t module = nullptr;
   std::map<std::string, hipFunction_t> functions;
+  // the kernels that separate reads from writes: per segment whether it has one (filled at the
+  // first launch), and per (kernel, dynamic LDS) how many of its workgroups fit a compute unit
+  std::vector<afir_target::SpecPhased> phased;
+  std::map<std::pair<std::string, unsigned>, int> resident;
   // The split / join row sum keeps its partial sums in one array of the code object.  Launches
   // of that form are chained through this event, so that one on another stream waits for the
   // join of the one before it instead of overwriting its partial sums.
@@ -866,6 +870,35 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
     bool elem;   // the kernel whose groups are single elements (rows off 16-byte boundaries)
     unsigned lds = 0;   // > 0: the kernel that stages a gathered operand's source row, with this much LDS
     bool stage_wave = false;   // ... its form with a wavefront per row
+    bool phased = false;       // the kernel that separates reads from writes (lds: its row vectors)
+    int64_t phased_bytes = 0;  // ... and what this launch of it reads
+    int phased_rate = 0;       // ... at this many GB/s, by what it reads
+  };
+  // Hold of the emitted kernels that separate reads from writes: base + bytes read / rate.  The
+  // rate the chip serves a launch's reads at depends on what is read (searched on [4096, 4096] f32
+  // (a + b) * b, the split / relu / broadcast graph at [8192, 4096] f16 and 32768 gathered rows of
+  // 1024 halves; 5 % either side costs about 1 %): two streamed operands 6700 GB/s, one 6900,
+  // rows gathered through an index tensor 6100.  AFIR_REGION_PHASE_GBS overrides all three.
+  const int region_hold_base_ns = afir::env_int("AFIR_REGION_PHASE_BASE_NS", 300, 0, 100000);
+  const int region_hold_gbs = afir::env_int("AFIR_REGION_PHASE_GBS", 0, 100, 100000);
+  auto region_hold_rate = [&](bool gathered, int streamed) {
+    return region_hold_gbs ? region_hold_gbs : gathered ? 6100 : streamed > 1 ? 6700 : 6900;
+  };
+  // workgroups of a compiled kernel that fit a compute unit with `lds` bytes of dynamic LDS
+  auto resident_per_cu = [&](const std::string &name, unsigned lds) -> int {
+    hipFunction_t fn = nullptr;
+    if (!compiled_function(compiled.get(), r->program, name, &fn).empty()) return 0;
+    std::lock_guard<std::mutex> lock(compiled->mutex);
+    const auto key = std::make_pair(name, lds);
+    auto it = compiled->resident.find(key);
+    if (it != compiled->resident.end()) return it->second;
+    int n = 0;
+    if (hipModuleOccupancyMaxActiveBlocksPerMultiprocessor(&n, fn, 256, lds) != hipSuccess) {
+      (void)hipGetLastError();
+      n = 0;
+    }
+    compiled->resident[key] = n;
+    return n;
   };
   std::vector<PendingSegment> pending;   // compiled kernels to launch, non-empty segments only
   for (const afir_region::ResolvedSegment &seg : res.segments) {
@@ -1064,6 +1097,96 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
         *made = PendingSegment{segment, sa, g.idx32, mode, row_groups, slim, kind == 2};
         return true;
       };
+      // The kernel that separates the chip's reads from its writes: every lane of the launch
+      // resident at once (eight workgroups of 256 lanes per compute unit, eight 16-byte groups
+      // per lane: 64 MiB of output per launch, up to two launches), for shapes of whole
+      // workgroups whose accesses are all aligned.  Anything else: the kernels below.
+      auto prepare_phased = [&]() -> bool {
+        if (block_dim || tile.tiled || seg.reduce || !afir::phased_enabled()) return false;
+        if (const char *env = std::getenv("AFIR_HIP_REGION_PHASED"))
+          if (env[0] == '0') return false;
+        {
+          std::lock_guard<std::mutex> lock(compiled->mutex);
+          if (compiled->phased.empty())
+            for (size_t k = 0; k < r->program.segments.size(); ++k)
+              compiled->phased.push_back(afir_target::specPhased(r->program, (int)k));
+        }
+        const afir_target::SpecPhased ph = compiled->phased[segment];
+        if (!ph.eligible) return false;
+        const int last = seg.rank - 1;
+        const int W = 16 / ph.elemBytes, G = afir_target::kSpecPhasedGroups;
+        const int64_t n = a.size[last];
+        if (n <= 0 || n % W != 0 || !a.out_vec) return false;
+        for (int i = 0; i < a.ninputs; ++i) {
+          const afir::RegionInput &d = a.in[i];
+          if (d.stride[last] == 0) continue;   // one value per row
+          if (d.stride[last] != 1 || !d.vec || (d.gdim >= 0 && !d.gvec)) return false;
+        }
+        int64_t nrows = 1;
+        for (int k = 0; k < last; ++k) nrows *= a.size[k];
+        const int64_t gpr = n / W;   // groups per row
+        int ll = 0;
+        int64_t cblocks = 1, blocks = 0;
+        if (gpr % G == 0 && gpr / G <= 256 && ((gpr / G) & (gpr / G - 1)) == 0) {
+          while (((int64_t)1 << ll) < gpr / G) ++ll;
+          const int64_t rows_per_block = 256 >> ll;
+          if (nrows % rows_per_block != 0) return false;
+          blocks = nrows / rows_per_block;
+        } else if (gpr % (256 * G) == 0 && ph.vectors == 0) {
+          ll = 8;
+          cblocks = gpr / (256 * G);
+          blocks = nrows * cblocks;
+        } else {
+          return false;
+        }
+        const int64_t lds = (int64_t)ph.vectors * n * ph.elemBytes;
+        if (lds > 16 * 1024) return false;
+        afir::RegionGeometry g;
+        if (afir::plan_fused_region(a, W * 4, 0, &g).code != 0 || g.empty || !g.idx32) return false;
+        const std::string name = afir_target::specPhasedKernelName(segment);
+        if (resident_per_cu(name, (unsigned)lds) < 8) return false;
+        const int64_t capacity = (int64_t)afir::device_cus() * 8;
+        if (blocks < (int64_t)afir::device_cus() * 2 || blocks > afir::kPhaseMaxLaunches * capacity) return false;
+        const int64_t launches = (blocks + capacity - 1) / capacity;
+        const int64_t take = (blocks + launches - 1) / launches;
+        for (int64_t b0 = 0; b0 < blocks; b0 += take) {
+          const int64_t nb = blocks - b0 < take ? blocks - b0 : take;
+          afir_target::SpecArgs sa;
+          std::memset(&sa, 0, sizeof sa);
+          for (int k = 0; k < 3; ++k) sa.size[k] = a.size[k];
+          sa.out = a.out;
+          sa.error_flag = a.error_flag;
+          sa.out_vec = 1;
+          afir_target::specExtentConstants(r->program, segment, res.shapes, sa.extent_const);
+          sa.lanes_log2 = ll;
+          sa.grid = (int)nb;
+          sa.column_blocks = (int)cblocks;
+          sa.first_block = (int)b0;
+          for (int i = 0; i < a.ninputs; ++i) {
+            const afir::RegionInput &d = a.in[i];
+            afir_target::SpecInput &t = sa.in[i];
+            t.base = d.base;
+            t.index = d.index;
+            for (int k = 0; k < 3; ++k) t.stride[k] = d.stride[k];
+            t.offset = d.offset;
+            t.gstride = d.gstride;
+            t.gextent = d.gextent;
+            t.vec = d.vec;
+            t.gvec = d.gvec;
+          }
+          PendingSegment made{segment, sa, true, afir_target::kSpecAligned, 0, false, false};
+          made.lds = (unsigned)lds;
+          made.phased = true;
+          made.phased_bytes = nb * 256 * G * 16 * ph.streamed;
+          bool gathered = false;
+          for (int i = 0; i < a.ninputs; ++i) gathered = gathered || a.in[i].gdim >= 0;
+          made.phased_rate = region_hold_rate(gathered, ph.streamed);
+          made.args.hold_ticks = afir::phase_hold_ticks(made.phased_bytes, region_hold_base_ns, made.phased_rate);
+          pending.push_back(made);
+        }
+        return true;
+      };
+      if (prepare_phased()) continue;
       PendingSegment made;
       bool ok = false;
       // A single row whose length is no multiple of the vector width (a rank-1 tensor, mostly): the
@@ -1162,13 +1285,45 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
     // segments that agree on the kernel variant go out as one launch
     const int nseg = (int)res.segments.size();
     bool together = pending.size() > 1 && nseg <= afir_target::kSpecMaxSegments;
-    int64_t total = 0;
+    // ... also those that separate reads from writes, when one launch of all of them is still
+    // resident at once: the hold is then that of everything the launch reads
+    bool together_phased = together;
+    int64_t total = 0, phased_bytes = 0;
+    double phased_ns = 0;   // the segments' reads one after the other, each at its rate
+    unsigned phased_lds = 0;
     for (const PendingSegment &p : pending) {
       together = together && p.idx32 == pending[0].idx32 && p.mode == pending[0].mode && !p.rows && !p.slim && !p.elem &&
-                 !p.lds;
+                 !p.lds && !p.phased;
+      together_phased = together_phased && p.phased && p.args.first_block == 0 &&
+                        (&p == &pending[0] || p.segment != (&p)[-1].segment);
       total += p.args.grid;
+      phased_bytes += p.phased_bytes;
+      if (p.phased_rate) phased_ns += (double)p.phased_bytes / p.phased_rate;
+      phased_lds = p.lds > phased_lds ? p.lds : phased_lds;
     }
-    if (together && total <= 0x7fffffff) {
+    together_phased = together_phased && total <= (int64_t)afir::device_cus() * 8 &&
+                      resident_per_cu(afir_target::specAllPhasedKernelName(), phased_lds) >= 8;
+    if (together_phased) {
+      afir_target::SpecAll all;
+      std::memset(&all, 0, sizeof all);
+      int next = 0;
+      size_t at = 0;
+      for (int k = 0; k < nseg; ++k) {
+        all.first[k] = next;
+        if (at < pending.size() && pending[at].segment == k) {
+          all.seg[k] = pending[at].args;
+          all.seg[k].hold_ticks = afir::phase_hold_ticks(
+              phased_bytes, region_hold_base_ns, phased_ns > 0 ? (int)((double)phased_bytes / phased_ns) : 6900);
+          next += pending[at].args.grid;
+          ++at;
+        }
+      }
+      for (int k = nseg; k <= afir_target::kSpecMaxSegments; ++k) all.first[k] = next;
+      const uint32_t rc = launch(afir_target::specAllPhasedKernelName(), &all,
+                                 offsetof(afir_target::SpecAll, seg) + (size_t)nseg * sizeof(afir_target::SpecArgs),
+                                 (unsigned)next, phased_lds);
+      if (rc != AFIR_HIP_OK) return rc;
+    } else if (together && total <= 0x7fffffff) {
       afir_target::SpecAll all;
       std::memset(&all, 0, sizeof all);
       int next = 0;
@@ -1215,6 +1370,12 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
           }
           c->split_recorded = true;
           c->split_stream = st;
+          continue;
+        }
+        if (p.phased) {
+          const uint32_t rc = launch(afir_target::specPhasedKernelName(p.segment), &p.args, sizeof p.args,
+                                     (unsigned)p.args.grid, p.lds);
+          if (rc != AFIR_HIP_OK) return rc;
           continue;
         }
         if (p.lds) {

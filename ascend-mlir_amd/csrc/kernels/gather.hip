@@ -364,7 +364,8 @@ LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx
   const int64_t phased_rows_per_block = (int64_t)(kPhasedThreads >> (lanes_log2 < 8 ? lanes_log2 : 8)) * kPhasedPasses;
   const int64_t phased_blocks = nidx / phased_rows_per_block;
   // blocks per launch: what is resident at once.  Rows of 8192 halves park 32 KiB of scale / shift
-  // per workgroup in LDS, and then five workgroups fit a compute unit, not eight.
+  // per workgroup in LDS, and then five workgroups fit a compute unit, not the eight that put
+  // 64 MiB in flight: such launches measured 4-11 % behind the grouped kernel and take it.
   const size_t lds = (size_t)2 * (kGroups << lanes_log2) * 16;   // scale and shift, 16-byte chunks
   int64_t capacity = 0;
   if (AFIR_GATHER_PHASED && vec && lanes_log2 <= 8 && (1 << lanes_log2) <= kPhasedThreads) {
@@ -374,7 +375,7 @@ LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx
       fit[lanes_log2] = n > 0 ? n : -1;
     }
     const int wanted = kPhasedLanesPerCU / kPhasedThreads;
-    capacity = (int64_t)device_cus() * (fit[lanes_log2] < wanted ? (fit[lanes_log2] > 0 ? fit[lanes_log2] : 0) : wanted);
+    capacity = fit[lanes_log2] >= wanted ? (int64_t)device_cus() * wanted : 0;
   }
   if (AFIR_GATHER_PHASED && vec && ((int64_t)kGroups << lanes_log2) == chunks64 && !block_dim && capacity > 0 &&
       phased_blocks > 0 && phased_blocks <= kPhaseMaxLaunches * capacity && phased_enabled()) {

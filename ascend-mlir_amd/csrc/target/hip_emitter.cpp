@@ -20,6 +20,8 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 #define DEV static __attribute__((device)) inline __attribute__((always_inline))
 #define KERNEL extern "C" __attribute__((global)) __attribute__((amdgpu_flat_work_group_size(256, 256)))
+// eight workgroups of 256 lanes per compute unit: at most 64 vector registers
+#define PHASED_KERNEL KERNEL __attribute__((amdgpu_waves_per_eu(8, 8)))
 
 struct SpecInput {
   const void *base;
@@ -41,6 +43,8 @@ struct SpecArgs {
   int column_blocks;
   SpecInput in[8];
   float extent_const[8];
+  int hold_ticks;
+  int first_block;
 };
 
 DEV float as_f32(unsigned u) { return __builtin_bit_cast(float, u); }
@@ -192,6 +196,75 @@ template <int V> DEV void stv_i16(void *o, long long i, const int (&v)[V]) {
   }
 }
 
+// ---- one 16-byte chunk <-> W values (the phased kernels keep packed results in registers)
+DEV void cvt_f32(const u32x4 raw, float (&v)[4]) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) v[e] = as_f32(raw[e]);
+}
+DEV void cvt_f16(const u32x4 raw, float (&v)[8]) {
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const unsigned word = raw[d];
+    const f16x2 h = __builtin_bit_cast(f16x2, word);
+    v[2 * d] = (float)h.x;
+    v[2 * d + 1] = (float)h.y;
+  }
+}
+DEV void cvt_bf16(const u32x4 raw, float (&v)[8]) {
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    v[2 * d] = as_f32(raw[d] << 16);
+    v[2 * d + 1] = as_f32(raw[d] & 0xffff0000u);
+  }
+}
+DEV void cvt_i32(const u32x4 raw, int (&v)[4]) {
+#pragma unroll
+  for (int e = 0; e < 4; ++e) v[e] = (int)raw[e];
+}
+DEV void cvt_i16(const u32x4 raw, int (&v)[8]) {
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    const unsigned word = raw[d];
+    v[2 * d] = (int)(word << 16) >> 16;
+    v[2 * d + 1] = (int)word >> 16;
+  }
+}
+DEV u32x4 pk_f32(const float (&v)[4]) {
+  u32x4 w;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) w[e] = as_u32(v[e]);
+  return w;
+}
+DEV u32x4 pk_f16(const float (&v)[8]) {
+  u32x4 w;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) {
+    f16x2 h;
+    h.x = (_Float16)v[2 * d];
+    h.y = (_Float16)v[2 * d + 1];
+    w[d] = __builtin_bit_cast(unsigned, h);
+  }
+  return w;
+}
+DEV u32x4 pk_bf16(const float (&v)[8]) {
+  u32x4 w;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) w[d] = (bf16_rne(v[2 * d]) & 0xffffu) | (bf16_rne(v[2 * d + 1]) << 16);
+  return w;
+}
+DEV u32x4 pk_i32(const int (&v)[4]) {
+  u32x4 w;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) w[e] = (unsigned)v[e];
+  return w;
+}
+DEV u32x4 pk_i16(const int (&v)[8]) {
+  u32x4 w;
+#pragma unroll
+  for (int d = 0; d < 4; ++d) w[d] = ((unsigned)v[2 * d] & 0xffffu) | ((unsigned)v[2 * d + 1] << 16);
+  return w;
+}
+
 // ---- sum over the 64 lanes of a wavefront, fixed order: quad butterflies,
 // half-row and row mirrors, then the four row totals
 template <int C> DEV float dpp_add(float v) {
@@ -270,6 +343,9 @@ struct Operand {
   int contiguousDim = -1;  // the iteration dim the operand's innermost dim follows, else -1
   bool tiled = false;
   int tileSlot = 0;        // which LDS tile
+  // the operand in the kernel that separates reads from writes (specPhased)
+  enum Phase { PhaseScalar, PhaseStreamed, PhaseVector, PhaseOther } phase = PhaseOther;
+  int vectorSlot = 0;      // PhaseVector: which stretch of the LDS
 };
 
 bool sameRead(const Op &a, const Op &b) {
@@ -320,6 +396,7 @@ class SegmentEmitter {
         emitBodyLongRows();
         emitBodySplitRows();
       }
+      if (phased_.eligible) emitBodyPhased();
       if (U_ > 1) {
         // the same with one group per lane, for short rows
         const int wide = U_;
@@ -442,10 +519,49 @@ class SegmentEmitter {
         }
       if (count == 1 && operands_[found].usesDim[0] && operands_[found].step == Operand::Broadcast) stageOperand_ = found;
     }
+    classifyForPhases();
+  }
+
+  // Whether the segment has the form that separates its reads from its writes (specPhased), and
+  // what each operand is in it.
+  void classifyForPhases() {
+    phased_ = SpecPhased();
+    if (reduce_ || tileDim_ >= 0 || stageOperand_ >= 0) return;
+    const size_t es = elemTypeBytes(p_.output().type);
+    int streamed = 0, vectors = 0;
+    for (Operand &o : operands_) {
+      o.phase = Operand::PhaseOther;
+      if (o.gatherDim == last_) return;
+      if (o.step == Operand::Broadcast) {
+        o.phase = Operand::PhaseScalar;
+        continue;
+      }
+      if (o.step != Operand::Contiguous || elemTypeBytes(o.type) != es) return;
+      bool all = true, none = o.gatherDim < 0;
+      for (int k = 0; k < last_; ++k) {
+        if (!(o.usesDim[k] || o.gatherDim == k)) all = false;
+        if (o.usesDim[k]) none = false;
+      }
+      if (all) {
+        o.phase = Operand::PhaseStreamed;
+        ++streamed;
+      } else if (none) {
+        o.phase = Operand::PhaseVector;
+        o.vectorSlot = vectors++;
+      } else {
+        return;
+      }
+    }
+    if (streamed < 1 || streamed > 2 || vectors > kSpecPhasedMaxVectors) return;
+    phased_.eligible = true;
+    phased_.streamed = streamed;
+    phased_.vectors = vectors;
+    phased_.elemBytes = (int)es;
   }
 
  public:
   bool tiled() const { return tileDim_ >= 0; }
+  SpecPhased phased() const { return phased_; }
   // SpecArgs::in slot of the operand whose source rows the staged kernels keep in LDS, else -1
   int stagedSlot() const { return stageOperand_ < 0 ? -1 : operands_[stageOperand_].slot; }
   ElemType stagedType() const { return stageOperand_ < 0 ? ElemType::F32 : operands_[stageOperand_].type; }
@@ -993,6 +1109,133 @@ class SegmentEmitter {
     os_ << "}\n";
   }
 
+  // The form that separates the chip's reads from its writes in time (specPhased).  HBM serves
+  // a pure read stream and a pure write stream faster than their mixture, so a launch whose
+  // lanes are all resident at once first requests everything, computes as the loads arrive,
+  // keeps the packed results in registers, and stores once the chip's reads have been served:
+  // R.hold_ticks of the real-time counter after the workgroup started (a time, so that no
+  // workgroup has to hear from another).  The hold shapes the timing only.
+  void emitBodyPhased() {
+    const std::string otag = typeTag(p_.output().type);
+    const int wideU = U_;
+    const int G = kSpecPhasedGroups, rounds = phased_.streamed;
+    U_ = G / rounds;
+    os_ << "\n// ---- segment " << index_ << ", reads and writes separated in time: every lane of the launch resident at once,\n"
+        << "// " << G << " groups of " << W_ << " elements per lane in " << rounds << (rounds == 1 ? " round" : " rounds")
+        << ", the packed results held in registers until the chip's reads are done ----\n";
+    os_ << "template <typename I>\nDEV void segment" << index_ << "_phased(const SpecArgs &R, const I bid, const int place, const int nblocks) {\n";
+    line(1, "constexpr int W = " + std::to_string(W_) + ", G = " + std::to_string(G) + ", U = " + std::to_string(U_) + ";");
+    line(1, "constexpr bool A = true, V = true;");
+    line(1, "const long long t_start = (long long)__builtin_readsteadycounter();");
+    line(1, "const int tid = (int)__builtin_amdgcn_workitem_id_x();");
+    line(1, "const I n = (I)R.size[" + std::to_string(last_) + "];");
+    for (const Operand &o : operands_)
+      if (o.step != Operand::Broadcast)
+        line(1, "const bool vec" + id(o) + " = true;");
+    line(1, "const I lanes = (I)1 << R.lanes_log2;");
+    line(1, "const I rows_per_block = (I)(256 >> R.lanes_log2);");
+    line(1, "// rows of more than a workgroup's 2048 groups: column_blocks workgroups per row, a stretch each");
+    line(1, "const I cblocks = (I)R.column_blocks;");
+    line(1, "const I rb = cblocks == 1 ? bid : bid / cblocks, cb = bid - rb * cblocks;");
+    line(1, "const I row = rb * rows_per_block + (I)(tid >> R.lanes_log2);");
+    line(1, "const I first_group = cb * (I)(256 * G) + ((I)tid & (lanes - 1));");
+    emitPositionOfRow(1);
+    emitRowInvariants(1);
+    line(1, "u32x4 res[G];");
+    if (phased_.vectors) {
+      line(1, "// the row vectors, 16-byte chunks: [vector][chunk of the row]");
+      line(1, "__attribute__((address_space(3))) u32x4 *const rowvec = (__attribute__((address_space(3))) u32x4 *)afir_stage;");
+      line(1, "const int row_chunks = (int)(n / W);");
+    }
+    for (int r = 0; r < rounds; ++r) {
+      line(1, "{   // round " + std::to_string(r));
+      line(2, "const I first = first_group + (I)" + std::to_string(r * U_) + " * lanes;");
+      emitGroups(2, "first", "lanes");
+      // every load of the round is issued as a raw 16-byte chunk before anything is converted;
+      // the groups are then converted, computed and packed one at a time, so that the round
+      // needs the registers of its chunks and of one group's values, not of all of them
+      std::vector<Value> read(operands_.size());
+      for (size_t k = 0; k < operands_.size(); ++k) {
+        const Operand &o = operands_[k];
+        if (o.phase == Operand::PhaseScalar) {
+          read[k].name = "s" + id(o);
+          read[k].scalar = true;
+        } else if (o.phase == Operand::PhaseStreamed) {
+          const std::string u = id(o), es = std::to_string(elemTypeBytes(o.type));
+          line(2, "u32x4 raw" + u + "[U];");
+          unroll();
+          line(2, "for (int u = 0; u < U; ++u)");
+          line(3, "raw" + u + "[u] = ld128<" + (o.readOnce ? "true" : "false") + ">((const u32x4 *)((const char *)" + in(o) +
+                      ".base + (q" + u + " + (long long)j0[u]) * " + es + "));");
+        }
+      }
+      if (r == 0 && phased_.vectors) {
+        line(2, "// behind the row loads: the row vectors into LDS, once per workgroup");
+        for (const Operand &o : operands_)
+          if (o.phase == Operand::PhaseVector) {
+            const std::string es = std::to_string(elemTypeBytes(o.type));
+            line(2, "for (int c = tid; c < row_chunks; c += 256)");
+            line(3, "rowvec[" + std::to_string(o.vectorSlot) + " * row_chunks + c] = ld128<false>((const u32x4 *)((const char *)" +
+                        in(o) + ".base + " + in(o) + ".offset * " + es + ") + c);");
+          }
+        line(2, "__builtin_amdgcn_fence(__ATOMIC_RELEASE, \"workgroup\");");
+        line(2, "__builtin_amdgcn_s_barrier();");
+        line(2, "__builtin_amdgcn_fence(__ATOMIC_ACQUIRE, \"workgroup\");");
+      }
+      unroll();
+      line(2, "for (int g = 0; g < " + std::to_string(U_) + "; ++g) {");
+      line(3, "constexpr int U = 1;   // one group at a time from here on");
+      for (size_t k = 0; k < operands_.size(); ++k) {
+        const Operand &o = operands_[k];
+        if (o.phase == Operand::PhaseScalar) continue;
+        const std::string u = id(o), tag = typeTag(o.type);
+        line(3, ct() + " v" + u + "[U][W];");
+        if (o.phase == Operand::PhaseStreamed) {
+          line(3, "cvt_" + tag + "(raw" + u + "[g], v" + u + "[0]);");
+          if (o.gatherDim >= 0) {
+            unroll();
+            line(3, "for (int e = 0; e < W; ++e) v" + u + "[0][e] = bad" + u + " ? " + bad() + " : v" + u + "[0][e];");
+          }
+        } else {
+          line(3, "cvt_" + tag + "(rowvec[" + std::to_string(o.vectorSlot) + " * row_chunks + (int)(j0[g] / W)], v" + u + "[0]);");
+        }
+        read[k].name = "v" + u;
+        read[k].scalar = false;
+      }
+      const Value v = emitCompute(3, read);
+      if (v.scalar) {
+        line(3, ct() + " splat[W];");
+        unroll();
+        line(3, "for (int e = 0; e < W; ++e) splat[e] = " + v.name + ";");
+        line(3, "res[" + std::to_string(r * U_) + " + g] = pk_" + otag + "(splat);");
+      } else {
+        line(3, "res[" + std::to_string(r * U_) + " + g] = pk_" + otag + "(" + v.name + "[0]);");
+      }
+      line(2, "}");
+      line(1, "}");
+    }
+    line(1, "// the results exist here, so the wait for the loads sits before the hold");
+    unroll();
+    line(1, "for (int g = 0; g < G; ++g) asm volatile(\"\" : \"+v\"(res[g]));");
+    line(1, "{");
+    line(2, "// A workgroup whose own loads came back early can tell from its place in the launch when the");
+    line(2, "// last workgroup's will (the chip serves a one-wave launch in the order of its workgroups):");
+    line(2, "// it waits for the shorter of that estimate and the launch's hold.");
+    line(2, "int hold = R.hold_ticks;");
+    line(2, "const int waited = (int)((long long)__builtin_readsteadycounter() - t_start);");
+    line(2, "const float over = waited > 80 ? (float)(waited - 80) : 0.f;");
+    line(2, "const float estimate = 80.f + over * (float)nblocks / (float)(place + 1);");
+    line(2, "if (estimate < (float)hold) hold = (int)estimate;");
+    line(2, "for (int spin = 0; spin < (1 << 15) && (long long)__builtin_readsteadycounter() - t_start < hold; ++spin)");
+    line(3, "__builtin_amdgcn_s_sleep(1);");
+    line(1, "}");
+    line(1, "u32x4 *const out_row = (u32x4 *)R.out + ((long long)row * (long long)n) / W;");
+    unroll();
+    line(1, "for (int g = 0; g < G; ++g) __builtin_nontemporal_store(res[g], out_row + (first_group + (I)g * lanes));");
+    os_ << "}\n";
+    U_ = wideU;
+  }
+
   // Row sums of rows of exactly 256 * U groups, every access 128-bit: a
   // workgroup owns a row (lane t takes the groups t, t + 256, ...), so the grid
   // walks the operands like a linear stream, and the operands of the
@@ -1376,6 +1619,9 @@ class SegmentEmitter {
             << ">(R, (" << (i32 ? "int" : "long long") << ")__builtin_amdgcn_workgroup_id_x(), ("
             << (i32 ? "int" : "long long") << ")R.grid); }\n";
       }
+    if (phased_.eligible)
+      os_ << "PHASED_KERNEL void " << specPhasedKernelName(index_) << "(const SpecArgs R) { segment" << index_
+          << "_phased<int>(R, (int)__builtin_amdgcn_workgroup_id_x() + R.first_block, (int)__builtin_amdgcn_workgroup_id_x(), R.grid); }\n";
     if (!tiled())
       for (int i32 = 1; i32 >= 0; --i32)
         os_ << "KERNEL void " << specElementKernelName(index_, i32 != 0) << "(const SpecArgs R) { segment" << index_
@@ -1433,6 +1679,7 @@ class SegmentEmitter {
   bool hasSlim_ = false;   // ... which exists for this segment
   bool hoisted_ = false;   // row invariants and operand values are assigned, not declared
   bool keepRowConstants_ = false;   // ... and operands that are the same for every row are left alone
+  SpecPhased phased_;      // the form that separates reads from writes, if the segment has one
 
   bool rowConstant(const Operand &o) const {
     if (o.gatherDim >= 0) return false;
@@ -1547,6 +1794,18 @@ std::string specStagedKernelName(int segment, bool idx32, int mode, bool wave) {
          modeSuffix(mode);
 }
 
+SpecPhased specPhased(const Program &p, int segment) {
+  const Segment &g = p.segments[segment];
+  if (!g.ops.empty() && g.ops[0].code == OpCode::Matmul) return SpecPhased();
+  std::ostringstream sink;
+  SegmentEmitter e(p, segment, sink);
+  e.analyze();
+  return e.phased();
+}
+
+std::string specPhasedKernelName(int segment) { return "afir_region_s" + std::to_string(segment) + "_phased_i32"; }
+std::string specAllPhasedKernelName() { return "afir_region_all_phased_i32"; }
+
 SpecStage specStage(const Program &p, int segment) {
   std::ostringstream sink;
   SegmentEmitter e(p, segment, sink);
@@ -1621,6 +1880,16 @@ std::string emitHipSource(const Program &p, const std::string &title, std::strin
              << ")(b - S.first[" << k << "]), (" << I << ")(S.first[" << k + 1 << "] - S.first[" << k << "]));\n";
         os << "}\n";
       }
+    bool every = true;
+    for (int k = 0; k < nseg; ++k) every = every && specPhased(p, k).eligible;
+    if (every) {
+      os << "PHASED_KERNEL void " << specAllPhasedKernelName() << "(const SpecAll S) {\n";
+      os << "  const int b = (int)__builtin_amdgcn_workgroup_id_x();\n";
+      for (int k = 0; k < nseg; ++k)
+        os << "  " << (k ? "else " : "") << (k + 1 < nseg ? "if (b < S.first[" + std::to_string(k + 1) + "]) " : "")
+           << "segment" << k << "_phased<int>(S.seg[" << k << "], b - S.first[" << k << "], b, S.first[" << nseg << "]);\n";
+      os << "}\n";
+    }
   }
   *source = os.str();
   return "";

@@ -53,6 +53,8 @@ struct SpecArgs {
   SpecInput in[kSpecMaxInputs];
   float extent_const[kSpecMaxExtentConsts];   // the segment's extent constants ('const argA.D'), in program
                                               // order, before and after 'reduce sum' (resolved per launch)
+  int hold_ticks;      // phased kernels: ticks of the real-time counter a workgroup holds its stores back
+  int first_block;     // phased kernels: number of the launch's first workgroup (a shape sent as two launches)
 };
 // The values of a segment's extent constants for a launch's shapes (what goes into
 // SpecArgs::extent_const): shapes[a][d] = extent of dim d of argument a.
@@ -112,7 +114,7 @@ uint64_t programHash(const afir_region::Program &p);
 // Version of the set of kernels and of the launch arguments that emitHipSource produces; the
 // code object exports it as `afir_region_emit_abi`, and a code object of another version is
 // refused when it is loaded (its kernels would be launched with the wrong names or arguments).
-constexpr int kSpecAbiVersion = 9;
+constexpr int kSpecAbiVersion = 10;
 
 // What a launch promises, which picks the kernel variant:
 //   kSpecAligned  every 128-bit access is aligned and every pass of the lanes over a row is whole
@@ -156,6 +158,31 @@ std::string specLongRowsKernelName(int segment, bool idx32);
 // row adds them in a fixed order).  rows x column_blocks may not exceed kSpecPartials.
 constexpr int kSpecPartials = 65536;
 std::string specSplitRowsKernelName(int segment, bool idx32, bool join);
+
+// A parallel segment whose operands are of three kinds only -- streamed (contiguous along the
+// innermost dim and addressed by every outer dim, or rows gathered through an index tensor along
+// an outer dim: one or two of them), row vectors (contiguous along the innermost dim, the same for
+// every row: up to four) and values broadcast along the innermost dim -- with every streamed
+// operand, row vector and the output of one element size, also has a kernel that separates its
+// reads from its writes in time: every lane of the launch is resident at once, takes
+// kSpecPhasedGroups groups of 16 bytes of output, computes them as its loads arrive (in as many
+// rounds as there are streamed operands), keeps the packed results in registers and stores them
+// once SpecArgs::hold_ticks of the real-time counter have passed since the workgroup started.
+// Launched with 32-bit positions for shapes of whole workgroups whose accesses are all aligned:
+// rows of 8 * 2^k groups, k <= 8, a workgroup covering 256 >> k rows (lanes_log2 = k,
+// column_blocks = 1; the row vectors staged in `vectors x row bytes` of dynamic LDS), or rows of a
+// multiple of 2048 groups without row vectors (lanes_log2 = 8, column_blocks = stretches per row).
+struct SpecPhased {
+  bool eligible = false;
+  int streamed = 0;      // operands read once per output element: the rounds of the kernel
+  int vectors = 0;       // row vectors staged in LDS
+  int elemBytes = 4;     // element size of the output, the streamed operands and the row vectors
+};
+constexpr int kSpecPhasedGroups = 8;
+constexpr int kSpecPhasedMaxVectors = 4;
+SpecPhased specPhased(const afir_region::Program &p, int segment);
+std::string specPhasedKernelName(int segment);
+std::string specAllPhasedKernelName();   // every segment of a program in one such launch
 
 // Emits the source for every segment.  Returns "" on success, else why the
 // program has no specialised form (matmul segments: those run on the

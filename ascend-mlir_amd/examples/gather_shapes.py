@@ -7,7 +7,8 @@ output + indices + the two vectors).
 
 Every shape is checked once, bit for bit, against the same expression in torch
 (float32 arithmetic, one rounding to f16).  The timed launches rotate over eight index vectors
-into a table of 131072 rows, so that a launch finds none of its rows in the last-level cache.
+into a table of at least 1 GiB (131072 rows or more), so that a launch finds few of its rows in
+the 256 MB last-level cache.
 
     gather_shapes.py [--steps N]
 
@@ -21,9 +22,9 @@ import time
 import numpy as np
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SHAPES = [(1024, 32768), (1024, 65536), (4096, 4096), (4096, 8192), (4096, 16384), (4096, 32768),
+SHAPES = [(256, 131072), (1024, 32768), (1024, 65536), (4096, 4096), (4096, 8192), (4096, 16384), (4096, 32768),
           (8192, 2048), (8192, 4096), (8192, 5120), (8192, 8192), (8192, 32768)]
-TABLE_ROWS = 131072
+MIN_TABLE_ROWS, MIN_TABLE_BYTES = 131072, 1 << 30
 
 
 def load_package():
@@ -46,6 +47,7 @@ def main():
     g = torch.Generator(device="cuda").manual_seed(42)
     print("# dim  rows  MiB_gathered | phased: kernel grid us GB/s | unphased: kernel grid us GB/s | ratio", flush=True)
     for dim, nidx in SHAPES:
+        TABLE_ROWS = max(MIN_TABLE_ROWS, MIN_TABLE_BYTES // (dim * 2))
         table = (torch.randn(TABLE_ROWS, dim, device="cuda", generator=g) * 0.02).to(torch.float16)
         scale = (torch.rand(dim, device="cuda", generator=g) + 0.5).to(torch.float16)
         shift = (torch.rand(dim, device="cuda", generator=g) * 0.2 - 0.1).to(torch.float16)

@@ -302,28 +302,27 @@ def test_c4_phased_route_bit_exact(H, dim, nidx, monkeypatch):
     assert out.tobytes() == want.tobytes()
 
 
-def test_c4_phased_launch_is_sized_by_what_fits_a_compute_unit(H, monkeypatch):
+def test_c4_phased_launch_needs_every_lane_resident(H, monkeypatch):
     """Rows of 8192 halves park 32 KiB of scale / shift per workgroup in LDS: five workgroups fit a
-    compute unit, not the eight the register count allows, so a launch that wants every lane
-    resident at once takes at most 5 x 256 workgroups and 4096 such rows go out as two launches.
-    The hold constants are read from the environment at every launch: a hold far too short or
-    too long changes the timing only."""
+    compute unit, not the eight that put a whole launch in flight at once, so such gathers keep to
+    the grouped kernel (asked of the runtime: the occupancy of the kernel with that much LDS).
+    Rows of 4096 halves fit.  The hold constants are read from the environment at every launch: a
+    hold far too short or too long changes the timing only."""
     table, idx, scale, shift = O.gen_c4(5000, 8192, 4096)
+    out = H.gather_scale_shift(dev(table), dev(idx), dev(scale), dev(shift)).cpu().numpy()
+    assert out.tobytes() == O.golden_c4(table, idx, scale, shift).tobytes()
+    assert H.last_launch()["kernel"] == "gather_scale_shift_f16_grouped"
+    table, idx, scale, shift = O.gen_c4(5000, 4096, 8192)
     want = O.golden_c4(table, idx, scale, shift)
     args = (dev(table), dev(idx), dev(scale), dev(shift))
     out = H.gather_scale_shift(*args).cpu().numpy()
     note = H.last_launch()
     assert out.tobytes() == want.tobytes()
-    assert note["kernel"] == "gather_scale_shift_f16_phased" and note["workgroups"] == 1024 and note["threads"] == 256
+    assert note["kernel"] == "gather_scale_shift_f16_phased" and note["workgroups"] == 2048 and note["threads"] == 256
     for gbs, base in (("100000", "0"), ("1000", "5000")):
         monkeypatch.setenv("AFIR_GATHER_PHASE_GBS", gbs)
         monkeypatch.setenv("AFIR_GATHER_PHASE_BASE_NS", base)
         assert H.gather_scale_shift(*args).cpu().numpy().tobytes() == want.tobytes()
-    # 1024-half rows leave the launch at eight workgroups per compute unit
-    table, idx, scale, shift = O.gen_c4(5000, 1024, 32768)
-    out = H.gather_scale_shift(dev(table), dev(idx), dev(scale), dev(shift)).cpu().numpy()
-    assert out.tobytes() == O.golden_c4(table, idx, scale, shift).tobytes()
-    assert H.last_launch()["workgroups"] == 2048
 
 
 def test_c4_phased_route_flags_bad_indices(H):

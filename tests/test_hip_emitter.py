@@ -273,3 +273,24 @@ def test_extent_constants_outside_the_tail_are_launch_arguments_too():
 
 def src_count(src, needle):
     return src.count(needle)
+
+
+def test_segments_that_can_separate_reads_from_writes_get_the_phased_kernel():
+    """One or two streamed operands, row vectors and per-row values, one element size: the segment
+    also has afir_region_s<k>_phased_i32 (eight 16-byte groups per lane, packed results held in
+    registers through a timed hold); programs of several such segments also one kernel for all.
+    Row sums, transposed reads, gathers along the innermost dim and mixed element sizes do not."""
+    c1 = _emit(RC.C1_ADD_MUL).stdout
+    assert "PHASED_KERNEL void afir_region_s0_phased_i32(const SpecArgs R)" in c1
+    assert "in 2 rounds" in c1 and "u32x4 raw0[U];" in c1 and "u32x4 raw1[U];" in c1 and "rowvec" not in c1
+    assert "__builtin_amdgcn_s_sleep(1);" in c1 and "R.hold_ticks" in c1
+    c4 = _emit(RC.C4_GATHER_SCALE_SHIFT).stdout
+    assert "afir_region_s0_phased_i32" in c4 and "in 1 round" in c4
+    assert "rowvec[0 * row_chunks + c]" in c4 and "rowvec[1 * row_chunks + c]" in c4     # scale and shift through LDS
+    split = _emit(RC.SPLIT_RELU_BRC_ADD_MUL).stdout
+    assert "afir_region_s0_phased_i32" in split and "afir_region_s1_phased_i32" in split
+    assert "PHASED_KERNEL void afir_region_all_phased_i32(const SpecAll S)" in split
+    for text in (RC.C2_BCAST_ADD_ROWSUM, RC.C3_RELU_BCAST_TRANSPOSE, RC.RELU_COLGATHER_ADD, RC.RELU_COL_ADD):
+        assert "_phased_i32" not in _emit(text).stdout
+    mixed = RC.C1_ADD_MUL.replace("arg out f32 2", "arg out f16 2")
+    assert "_phased_i32" not in _emit(mixed).stdout
