@@ -938,7 +938,10 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
     a.nops = 0;
     for (const afir_region::ResolvedOp &op : seg.ops) {
       const bool integer = afir_region::isRegionInt(seg.outType);
-      const int code = region_op_code(op.code, integer, seg.outType == afir_region::ElemType::I16);
+      int code = region_op_code(op.code, integer, seg.outType == afir_region::ElemType::I16);
+      if (op.code == afir_region::OpCode::Cast)   // a cast to f32 changes nothing
+        code = op.castType == afir_region::ElemType::F16 ? (int)afir::kRegionCastF16
+               : op.castType == afir_region::ElemType::BF16 ? (int)afir::kRegionCastBF16 : -1;
       if (code < 0) continue;
       afir::RegionOp &d = a.ops[a.nops++];
       d.code = code;
@@ -952,8 +955,11 @@ uint32_t afir_hip_launch_region(uint64_t handle, uint32_t block_dim, void *strea
     }
     a.ntail = 0;
     for (const afir_region::ResolvedSegment::TailStep &t : seg.tail) {
+      if (t.code == afir_region::OpCode::Cast && t.castType == afir_region::ElemType::F32) continue;
       afir::RegionOp &d = a.tail[a.ntail++];   // at most kMaxTailOps = kRegionMaxTail (validate)
-      d.code = region_op_code(t.code, false);
+      d.code = t.code == afir_region::OpCode::Cast
+                   ? (t.castType == afir_region::ElemType::F16 ? (int)afir::kRegionCastF16 : (int)afir::kRegionCastBF16)
+                   : region_op_code(t.code, false);
       d.constant = t.constant;
       d.depth = t.reversed ? 1 : 0;
     }

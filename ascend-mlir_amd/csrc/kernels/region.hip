@@ -234,6 +234,14 @@ __device__ __forceinline__ void unary(int code, float c, float (&a)[V]) {
 #pragma unroll
       for (int e = 0; e < V; ++e) a[e] = -a[e];
       break;
+    case kRegionCastF16:
+#pragma unroll
+      for (int e = 0; e < V; ++e) a[e] = (float)(_Float16)a[e];
+      break;
+    case kRegionCastBF16:
+#pragma unroll
+      for (int e = 0; e < V; ++e) a[e] = __uint_as_float(f32_to_bf16_rne(a[e]) << 16);
+      break;
     case kRegionReluI:
 #pragma unroll
       for (int e = 0; e < V; ++e) a[e] = __float_as_int(a[e]) > 0 ? a[e] : 0.f;

@@ -19,6 +19,7 @@ enum RegionType : int { kRegionF16 = 0, kRegionBF16 = 1, kRegionF32 = 2, kRegion
 enum RegionOpCode : int {
   kRegionPush = 0, kRegionConst, kRegionAdd, kRegionSub, kRegionMul, kRegionDiv, kRegionMax,
   kRegionMin, kRegionRelu, kRegionLeaky, kRegionNeg, kRegionDup,
+  kRegionCastF16, kRegionCastBF16,   // round to that type (nearest even) and widen again
   kRegionAddI = 16, kRegionSubI, kRegionMulI, kRegionMaxI, kRegionMinI, kRegionReluI, kRegionNegI,
   // comparisons of an i16 region look at the low 16 bits of their operands (add, sub, mul
   // and neg agree modulo 2^16 whatever the upper bits hold, and the store truncates)
@@ -30,7 +31,7 @@ __host__ __device__ inline bool region_is_binary(int code) {
 }
 __host__ __device__ inline bool region_is_unary(int code) {
   return code == kRegionRelu || code == kRegionLeaky || code == kRegionNeg || code == kRegionReluI ||
-         code == kRegionNegI || code == kRegionReluI16;
+         code == kRegionNegI || code == kRegionReluI16 || code == kRegionCastF16 || code == kRegionCastBF16;
 }
 __host__ __device__ inline bool region_is_16bit(int type) {
   return type == kRegionF16 || type == kRegionBF16 || type == kRegionI16;

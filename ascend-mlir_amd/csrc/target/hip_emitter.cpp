@@ -65,6 +65,10 @@ DEV unsigned bf16_rne(float f) {
   const unsigned r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
   return (f != f) ? ((u >> 16) | 0x40u) : r;
 }
+// round to the narrower type (nearest even) and widen again
+DEV float rt_f16(float x) { return (float)(_Float16)x; }
+DEV float rt_bf16(float x) { return as_f32(bf16_rne(x) << 16); }
+DEV float rt_f32(float x) { return x; }
 DEV void st_f32(void *o, long long i, float x) { ((float *)o)[i] = x; }
 DEV void st_f16(void *o, long long i, float x) {
   ((unsigned short *)o)[i] = __builtin_bit_cast(unsigned short, (_Float16)x);
@@ -836,6 +840,14 @@ class SegmentEmitter {
           stack.push_back(v);
           break;
         }
+        case OpCode::Cast: {
+          const Value a = stack.back();
+          stack.pop_back();
+          Value v = fresh(a.scalar);
+          define(v, std::string("rt_") + typeTag(op.constType) + "(" + a.at() + ")");
+          stack.push_back(v);
+          break;
+        }
         case OpCode::Relu: case OpCode::Leaky: case OpCode::Neg: {
           const Value a = stack.back();
           stack.pop_back();
@@ -885,6 +897,7 @@ class SegmentEmitter {
           stack.back() = "fmax_ieee(" + stack.back() + ", (" + stack.back() + ") * " + floatLiteral(op.constant) + ")";
           break;
         case OpCode::Neg: stack.back() = "(-" + stack.back() + ")"; break;
+        case OpCode::Cast: stack.back() = std::string("rt_") + typeTag(op.constType) + "(" + stack.back() + ")"; break;
         default: {
           const std::string b = stack.back();
           stack.pop_back();

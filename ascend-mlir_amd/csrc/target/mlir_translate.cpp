@@ -43,7 +43,8 @@ struct Expr {
   // Reduced: the row sum a tail expression works on; ExtentConst: an extent as a number
   enum Kind { Input, Constant, Unary, Binary, Matmul, Reduced, ExtentConst } kind = Constant;
   Ref extent;               // ExtentConst
-  ElemType extentType = ElemType::F32;   // ... rounded through this type (arith.sitofp ... to f16)
+  ElemType extentType = ElemType::F32;   // ... rounded through this type (arith.sitofp ... to f16);
+                                         // Unary Cast: the type the value is rounded to
   int arg = -1, arg2 = -1;
   bool transA = false, transB = false;   // Matmul: operand stored transposed
   std::vector<Index> idx;   // Input: one per dim of the argument
@@ -139,6 +140,23 @@ ExprP makeUnary(OpCode op, ExprP a, float alpha = 0.f) {
   e->value = alpha;
   return e;
 }
+// x rounded to `type` and widened again (arith.truncf + arith.extf, afir.cast); float32 keeps x
+ExprP makeCast(ElemType type, ExprP a) {
+  if (type == ElemType::F32) return a;
+  if (a->kind == Expr::Unary && a->op == OpCode::Cast && a->extentType == type) return a;
+  auto e = std::make_shared<Expr>();
+  e->kind = Expr::Unary;
+  e->op = OpCode::Cast;
+  e->extentType = type;
+  e->a = std::move(a);
+  return e;
+}
+// the same unary node over another operand
+ExprP withOperand(const ExprP &unary, ExprP a) {
+  auto e = std::make_shared<Expr>(*unary);
+  e->a = std::move(a);
+  return e;
+}
 bool isConst(const ExprP &e, float v) { return e->kind == Expr::Constant && e->value == v && !std::signbit(e->value); }
 
 ExprP makeBinary(OpCode op, ExprP a, ExprP b) {
@@ -177,7 +195,7 @@ ExprP substitute(const ExprP &e, const std::vector<Index> &with) {
           throw Failure("a matmul result can only be consumed through identity maps");
       return e;
     }
-    case Expr::Unary: return makeUnary(e->op, substitute(e->a, with), e->value);
+    case Expr::Unary: return withOperand(e, substitute(e->a, with));
     case Expr::Binary: {
       auto r = std::make_shared<Expr>(*e);
       r->a = substitute(e->a, with);
@@ -212,7 +230,7 @@ ExprP offsetReads(const ExprP &e, const std::vector<Ref> &offsets) {
     case Expr::Constant: case Expr::ExtentConst: return e;
     case Expr::Reduced: throw Failure("extract_slice of a reduced value is not supported");
     case Expr::Matmul: throw Failure("extract_slice of a matmul result is not supported");
-    case Expr::Unary: return makeUnary(e->op, offsetReads(e->a, offsets), e->value);
+    case Expr::Unary: return withOperand(e, offsetReads(e->a, offsets));
     case Expr::Binary: {
       auto r = std::make_shared<Expr>(*e);
       r->a = offsetReads(e->a, offsets);
@@ -713,6 +731,16 @@ class Translator {
       parseMatmul(one(), op, true, false, true);
     } else if (op == "linalg.batch_matmul_transpose_b") {
       parseMatmul(one(), op, false, true, true);
+    } else if (op == "linalg.elementwise") {
+      parseElementwise(one());
+    } else if (op == "linalg.transpose") {
+      parseTranspose(one());
+    } else if (op == "linalg.broadcast") {
+      parseBroadcast(one());
+    } else if (op == "tensor.collapse_shape" || op == "tensor.expand_shape") {
+      parseReshape(one(), op == "tensor.expand_shape");
+    } else if (namedElementwise(op.compare(0, 7, "linalg.") == 0 ? op.substr(7) : std::string(), nullptr, nullptr)) {
+      parseNamedElementwise(one(), op.substr(7));
     } else if (op == "tensor.extract_slice") {
       parseExtractSlice(one());
     } else if (op == "tensor.concat") {
@@ -728,7 +756,31 @@ class Translator {
   void parseConstant(const std::string &result) {
     Value v;
     if (r_.eatWord("true") || r_.eatWord("false")) r_.fail("boolean constants are not supported");
-    if (r_.peekIdent() == "dense") r_.fail("dense constants are not supported");
+    if (r_.peekIdent() == "dense") {
+      // dense<c> : tensor<...>: a tensor of one value (what linalg ops take as an init)
+      r_.ident();
+      r_.expect('<');
+      if (r_.peek() == '[') r_.fail("dense constants other than splats (dense<c>) are not supported");
+      const double c = r_.number();
+      r_.expect('>');
+      r_.expect(':');
+      TypeInfo t = parseType();
+      if (!t.isTensor || !t.elemKnown || !afir_region::isFloat(t.elem)) r_.fail("a dense splat must be a float tensor");
+      auto tv = std::make_shared<Tensor>();
+      tv->elem = t.elem;
+      for (int64_t d : t.shape) {
+        if (d < 0) r_.fail("a dense constant has a static shape");
+        tv->shape.push_back(Ref::value(d));
+      }
+      float f = (float)c;
+      if (t.elem == ElemType::F16) f = roundThroughF16(f);
+      else if (t.elem == ElemType::BF16) f = roundThroughBf16(f);
+      tv->filled = true;
+      tv->fill = f;
+      tv->expr = makeConst(f);
+      defineTensor(result, tv);
+      return;
+    }
     bool isInt = false;
     const double n = r_.number(&isInt);
     r_.expect(':');
@@ -811,6 +863,227 @@ class Translator {
     tv->shape.push_back(a->shape[b0 + (ta ? 1 : 0)]);
     tv->shape.push_back(b->shape[b0 + (tb ? 0 : 1)]);
     tv->expr = e;
+    defineTensor(result, tv);
+  }
+
+  // ---- named linalg ops (what the reference's --linalg-mark / --linalg-add-broadcast consume:
+  // test/Dialect/AFIR/Transforms/linalgMark.mlir:35-44, linalgAddBroadcast.mlir:3-23) ----
+  // the arithmetic of linalg.<name> / #linalg.elementwise_kind<name>: false for a kind this
+  // backend has no lowering for (the transcendental functions)
+  static bool namedElementwise(const std::string &name, OpCode *code, int *arity) {
+    static const struct { const char *n; OpCode c; int arity; } table[] = {
+        {"add", OpCode::Add, 2}, {"sub", OpCode::Sub, 2}, {"mul", OpCode::Mul, 2}, {"div", OpCode::Div, 2},
+        {"max", OpCode::Max, 2}, {"min", OpCode::Min, 2}, {"max_signed", OpCode::Max, 2},
+        {"min_signed", OpCode::Min, 2}, {"negf", OpCode::Neg, 1}, {"abs", OpCode::Neg, -1}};
+    for (const auto &e : table)
+      if (name == e.n) {
+        if (code) *code = e.c;
+        if (arity) *arity = e.arity;
+        return true;
+      }
+    return false;
+  }
+  // result of an elementwise op over `ins` read through `maps` (one per input, then the output's)
+  void defineElementwise(const std::string &result, const std::string &kind, const Operands &ins, const Operands &outs,
+                         std::vector<AffineMap> maps) {
+    OpCode code = OpCode::Add;
+    int arity = 0;
+    if (!namedElementwise(kind, &code, &arity)) r_.fail("elementwise kind '" + kind + "' has no HIP lowering");
+    const int want = arity < 0 ? 1 : arity;
+    if ((int)ins.names.size() != want || outs.names.size() != 1)
+      r_.fail("elementwise '" + kind + "' takes " + std::to_string(want) + " input(s) and one init");
+    TensorP outT = tensorOf(outs.names[0]);
+    const int rank = (int)outT->shape.size();
+    if (maps.empty()) {   // identity maps: operands of the output's shape
+      AffineMap id;
+      id.numDims = rank;
+      for (int d = 0; d < rank; ++d) { Index ix; ix.dim = d; id.results.push_back(ix); }
+      maps.assign(ins.names.size() + 1, id);
+    }
+    if (maps.size() != ins.names.size() + 1) r_.fail("elementwise: one indexing map per operand is required");
+    if (!maps.back().isIdentity() || maps.back().numDims != rank) r_.fail("elementwise: the output map must be the identity");
+    std::vector<ExprP> v;
+    for (size_t i = 0; i < ins.names.size(); ++i) {
+      TensorP t = tensorOf(ins.names[i]);
+      if (!t->expr || t->reduced || !t->parts.empty() || !afir_region::isFloat(t->elem))
+        r_.fail("elementwise: operand " + ins.names[i] + " is not an elementwise float value");
+      if (maps[i].numDims != rank || maps[i].results.size() != t->shape.size())
+        r_.fail("elementwise: the map of operand " + std::to_string(i) + " does not match its rank");
+      v.push_back(substitute(t->expr, maps[i].results));
+    }
+    auto tv = std::make_shared<Tensor>();
+    tv->elem = outT->elem;
+    tv->shape = outT->shape;
+    if (arity == 2) tv->expr = makeBinary(code, v[0], v[1]);
+    else if (arity == 1) tv->expr = makeUnary(code, v[0]);
+    else tv->expr = makeBinary(OpCode::Max, v[0], makeUnary(OpCode::Neg, v[0]));   // |x| = max(x, -x), exactly
+    defineTensor(result, tv);
+  }
+  // linalg.elementwise kind=#linalg.elementwise_kind<add> [indexing_maps = [...]] ins(...) outs(...) [-> type]
+  void parseElementwise(const std::string &result) {
+    if (!r_.eatWord("kind")) r_.fail("expected 'kind=' in linalg.elementwise");
+    r_.expect('=');
+    r_.sigil('#', "an elementwise kind");
+    r_.expect('<');
+    const std::string kind = r_.ident();
+    r_.expect('>');
+    std::vector<AffineMap> maps;
+    if (r_.eatWord("indexing_maps")) {
+      r_.expect('=');
+      r_.expect('[');
+      do maps.push_back(parseMapRef()); while (r_.eat(','));
+      r_.expect(']');
+    }
+    if (r_.peek() == '{') { r_.eat('{'); skipDict(); }
+    Operands ins = parseOperandGroup("ins"), outs = parseOperandGroup("outs");
+    if (r_.eatArrow()) parseType();
+    defineElementwise(result, kind, ins, outs, maps);
+  }
+  // linalg.add / sub / mul / div / max / min / negf / abs ins(...) outs(...) [-> type]
+  void parseNamedElementwise(const std::string &result, const std::string &kind) {
+    if (r_.peek() == '{') { r_.eat('{'); skipDict(); }
+    Operands ins = parseOperandGroup("ins"), outs = parseOperandGroup("outs");
+    if (r_.eatArrow()) parseType();
+    defineElementwise(result, kind, ins, outs, {});
+  }
+  std::vector<int64_t> parseIntList(const char *keyword) {
+    if (!r_.eatWord(keyword)) r_.fail(std::string("expected '") + keyword + " = [...]'");
+    r_.expect('=');
+    std::vector<int64_t> v;
+    r_.expect('[');
+    if (!r_.eat(']')) {
+      do v.push_back(r_.integer()); while (r_.eat(','));
+      r_.expect(']');
+    }
+    return v;
+  }
+  TensorP elementwiseSource(const std::string &name, const char *what) {
+    TensorP t = tensorOf(name);
+    if (!t->expr || t->reduced || !t->parts.empty()) r_.fail(std::string(what) + " of a value that is not elementwise");
+    return t;
+  }
+  // linalg.transpose ins(%a : t) outs(%b : t) permutation = [p0, p1, ...]: result dim i is input dim p_i
+  void parseTranspose(const std::string &result) {
+    Operands ins = parseOperandGroup("ins"), outs = parseOperandGroup("outs");
+    if (ins.names.size() != 1 || outs.names.size() != 1) r_.fail("linalg.transpose takes one input and one init");
+    const std::vector<int64_t> perm = parseIntList("permutation");
+    if (r_.eatArrow()) parseType();
+    TensorP in = elementwiseSource(ins.names[0], "linalg.transpose"), outT = tensorOf(outs.names[0]);
+    const size_t rank = in->shape.size();
+    if (perm.size() != rank || outT->shape.size() != rank) r_.fail("linalg.transpose: the permutation does not match the rank");
+    std::vector<Index> with(rank);
+    std::vector<bool> seen(rank, false);
+    auto tv = std::make_shared<Tensor>();
+    tv->elem = outT->elem;
+    for (size_t i = 0; i < rank; ++i) {
+      if (perm[i] < 0 || perm[i] >= (int64_t)rank || seen[(size_t)perm[i]]) r_.fail("linalg.transpose: not a permutation");
+      seen[(size_t)perm[i]] = true;
+      with[(size_t)perm[i]].dim = (int)i;
+      tv->shape.push_back(in->shape[(size_t)perm[i]]);
+    }
+    tv->expr = substitute(in->expr, with);
+    defineTensor(result, tv);
+  }
+  // linalg.broadcast ins(%a : t) outs(%b : t) dimensions = [...]: the result dims that are added
+  void parseBroadcast(const std::string &result) {
+    Operands ins = parseOperandGroup("ins"), outs = parseOperandGroup("outs");
+    if (ins.names.size() != 1 || outs.names.size() != 1) r_.fail("linalg.broadcast takes one input and one init");
+    const std::vector<int64_t> added = parseIntList("dimensions");
+    if (r_.eatArrow()) parseType();
+    TensorP in = elementwiseSource(ins.names[0], "linalg.broadcast"), outT = tensorOf(outs.names[0]);
+    const size_t rank = outT->shape.size();
+    if (in->shape.size() + added.size() != rank) r_.fail("linalg.broadcast: input rank + added dims must be the result rank");
+    std::vector<bool> isAdded(rank, false);
+    for (int64_t d : added) {
+      if (d < 0 || d >= (int64_t)rank || isAdded[(size_t)d]) r_.fail("linalg.broadcast: bad 'dimensions'");
+      isAdded[(size_t)d] = true;
+    }
+    std::vector<Index> with;
+    auto tv = std::make_shared<Tensor>();
+    tv->elem = in->elem;
+    size_t own = 0;
+    for (size_t d = 0; d < rank; ++d) {
+      if (isAdded[d]) {
+        tv->shape.push_back(outT->shape[d]);
+      } else {
+        Index ix;
+        ix.dim = (int)d;
+        with.push_back(ix);
+        tv->shape.push_back(in->shape[own++]);
+      }
+    }
+    tv->expr = substitute(in->expr, with);
+    defineTensor(result, tv);
+  }
+  // tensor.collapse_shape %x [[0, 1], [2]] : tensor<8x1x32xf32> into tensor<8x32xf32>
+  // tensor.expand_shape %x [[0, 1], [2]] output_shape [8, 1, 32] : tensor<8x32xf32> into tensor<8x1x32xf32>
+  // Supported where a reassociation group holds at most one dim whose (static) extent is not 1:
+  // dims of extent 1 come and go, nothing is re-linearised.
+  void parseReshape(const std::string &result, bool expand) {
+    TensorP src = elementwiseSource(r_.ssa(), expand ? "tensor.expand_shape" : "tensor.collapse_shape");
+    std::vector<std::vector<int64_t>> groups;
+    r_.expect('[');
+    if (!r_.eat(']')) {
+      do {
+        std::vector<int64_t> g;
+        r_.expect('[');
+        if (!r_.eat(']')) {
+          do g.push_back(r_.integer()); while (r_.eat(','));
+          r_.expect(']');
+        }
+        groups.push_back(g);
+      } while (r_.eat(','));
+      r_.expect(']');
+    }
+    if (r_.eatWord("output_shape")) (void)parseSliceList();   // [4, 1, %n]: the result type says the same
+    r_.expect(':');
+    TypeInfo from = parseType();
+    if (!r_.eatWord("into")) r_.fail("expected 'into' in a reshape");
+    TypeInfo to = parseType();
+    const TypeInfo &wide = expand ? to : from, &narrow = expand ? from : to;   // wide: the side with more dims
+    if (groups.size() != narrow.shape.size() || from.shape.size() != src->shape.size())
+      r_.fail("reshape: the reassociation does not match the types");
+    // per group: the one wide dim that is not a static 1 (-1: all are 1)
+    std::vector<int> keep(groups.size(), -1);
+    size_t expect = 0;
+    for (size_t g = 0; g < groups.size(); ++g)
+      for (int64_t d : groups[g]) {
+        if (d != (int64_t)expect++ || d >= (int64_t)wide.shape.size()) r_.fail("reshape: reassociation indices must be 0, 1, 2, ... in order");
+        if (wide.shape[(size_t)d] == 1) continue;
+        if (keep[g] >= 0) r_.fail("reshapes that merge or split dims of extent other than 1 are not supported");
+        keep[g] = (int)d;
+      }
+    if (expect != wide.shape.size()) r_.fail("reshape: the reassociation does not cover every dim");
+    auto tv = std::make_shared<Tensor>();
+    tv->elem = src->elem;
+    std::vector<Index> with(src->shape.size());
+    if (!expand) {
+      // source = wide: its kept dim of group g is result dim g, the others are read at 0
+      for (size_t g = 0; g < groups.size(); ++g) {
+        for (int64_t d : groups[g]) {
+          Index ix;
+          if ((int)d == keep[g]) ix.dim = (int)g;
+          else { ix.kind = Index::Const; ix.c = 0; }
+          with[(size_t)d] = ix;
+        }
+        tv->shape.push_back(keep[g] >= 0 ? src->shape[(size_t)keep[g]] : Ref::value(1));
+      }
+    } else {
+      // source = narrow: its dim g is the kept result dim of group g (or index 0 if none)
+      tv->shape.assign(wide.shape.size(), Ref::value(1));
+      for (size_t g = 0; g < groups.size(); ++g) {
+        Index ix;
+        if (keep[g] >= 0) {
+          ix.dim = keep[g];
+          tv->shape[(size_t)keep[g]] = src->shape[g];
+        } else {
+          ix.kind = Index::Const;
+          ix.c = 0;
+        }
+        with[g] = ix;
+      }
+    }
+    tv->expr = substitute(src->expr, with);
     defineTensor(result, tv);
   }
 
@@ -979,7 +1252,8 @@ class Translator {
           v.kind = Value::Scalar;
           auto e = std::make_shared<Expr>();
           e->kind = Expr::Reduced;
-          v.scalar = e;
+          // the sums sit in a tensor of t's element type before this generic reads them
+          v.scalar = makeCast(t->elem, e);
           body_[blockArgs[i]] = v;
           continue;
         }
@@ -1120,6 +1394,18 @@ class Translator {
       parseType();
       out.kind = Value::Scalar;
       out.scalar = makeUnary(OpCode::Neg, scalarOf(v));
+    } else if (op == "arith.truncf" || op == "arith.extf") {
+      // mixed-precision chains: truncf rounds to the narrower type (nearest even); extf is
+      // exact, the value is already one of the narrower type
+      Value v = lookup(r_.ssa());
+      r_.expect(':');
+      parseType();
+      if (!r_.eatWord("to")) r_.fail("expected 'to' in " + op);
+      TypeInfo to = parseType();
+      if (!to.elemKnown || !afir_region::isFloat(to.elem)) r_.fail(op + " to a type that is not f16, bf16 or f32");
+      if (v.blockArgOperand == -2) r_.fail("the accumulated value may only be yielded");
+      out.kind = Value::Scalar;
+      out.scalar = op == "arith.truncf" ? makeCast(to.elem, scalarOf(v)) : scalarOf(v);
     } else {
       const OpCode code = binaryOp(op);
       Value a = lookup(r_.ssa());
@@ -1158,7 +1444,7 @@ class Translator {
   }
   static ExprP replaceReduced(const ExprP &e, const ExprP &with) {
     if (e->kind == Expr::Reduced) return with;
-    if (e->kind == Expr::Unary) return makeUnary(e->op, replaceReduced(e->a, with), e->value);
+    if (e->kind == Expr::Unary) return withOperand(e, replaceReduced(e->a, with));
     if (e->kind == Expr::Binary) {
       auto r = std::make_shared<Expr>(*e);
       r->a = replaceReduced(e->a, with);
@@ -1315,13 +1601,19 @@ class Translator {
       return;
     }
     {
-      static const char *const unary[] = {"load", "store", "abs", "relu", "neg", "leaky_relu", "broadcast", "sum"};
+      static const char *const unary[] = {"load", "store", "abs", "relu", "neg", "leaky_relu", "broadcast", "sum", "cast"};
       bool known = false;
       for (const char *u : unary) known = known || name == u;
       if (!known) r_.fail("afir." + name + " has no HIP lowering");
     }
     if (in.size() != 1) r_.fail("afir." + name + " takes one operand");
-    if (name == "load" || name == "store") {
+    if (name == "cast") {
+      // include/Dialect/AFIR/Ops/Basic/cast.td:22-25, between the float types: the value
+      // rounded to the result's element type (a widening cast changes nothing)
+      if (integer || !afir_region::isFloat(in[0]->elem)) r_.fail("afir.cast between integer types has no HIP lowering");
+      tv->shape = in[0]->shape;
+      tv->expr = tv->elem == in[0]->elem ? in[0]->expr : makeCast(tv->elem, in[0]->expr);   // (to f32: exact, no cast)
+    } else if (name == "load" || name == "store") {
       // data movement between global memory and the core in an AscGraph
       // (include/Dialect/AFIR/Ops/Basic/data.td:31-32): the value itself
       tv->shape = in[0]->shape;
@@ -1428,6 +1720,7 @@ class Translator {
         emitExpr(e->a, ops);
         o.code = e->op;
         o.constant = e->value;
+        o.constType = e->extentType;   // Cast
         ops->push_back(o);
         return;
       case Expr::Binary: {
@@ -1485,6 +1778,8 @@ class Translator {
       g.ops.push_back(o);
       if (t->tail) emitExpr(t->tail, &g.ops);
     }
+    // a last rounding to the output's own type is what the store does
+    if (!g.ops.empty() && g.ops.back().code == OpCode::Cast && g.ops.back().constType == t->elem) g.ops.pop_back();
     o = afir_region::Op();
     o.code = OpCode::Store;
     g.ops.push_back(o);

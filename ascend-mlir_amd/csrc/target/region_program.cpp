@@ -149,6 +149,7 @@ std::string serialize(const Program &p) {
             s += "const " + floatText(o.constant) + "\n";
           break;
         case OpCode::Leaky: s += "leaky " + floatText(o.constant) + "\n"; break;
+        case OpCode::Cast: s += std::string("cast ") + elemTypeName(o.constType) + "\n"; break;
         case OpCode::Dup: s += "dup " + std::to_string(o.depth) + "\n"; break;
         case OpCode::ReduceSum: s += "reduce sum\n"; break;
         default:
@@ -281,6 +282,12 @@ std::string parse(const std::string &text, Program *out) {
       o.constant = std::strtof(tok[1].c_str(), &end);
       if (*end) return err(lineno, "bad number '" + tok[1] + "'");
       seg->ops.push_back(o);
+    } else if (k == "cast") {
+      Op o;
+      o.code = OpCode::Cast;
+      if (tok.size() != 2 || !parseElemType(tok[1], &o.constType) || !isFloat(o.constType))
+        return err(lineno, "expected 'cast f16|bf16|f32'");
+      seg->ops.push_back(o);
     } else if (k == "dup") {
       Op o;
       o.code = OpCode::Dup;
@@ -371,7 +378,7 @@ std::string validate(const Program &p) {
               if (fromSum.back()) ++tailOps;
             }
             break;
-          case OpCode::Relu: case OpCode::Leaky: case OpCode::Neg:
+          case OpCode::Relu: case OpCode::Leaky: case OpCode::Neg: case OpCode::Cast:
             if (!fromSum.empty() && fromSum.back()) ++tailOps;
             break;
           default: break;
@@ -446,8 +453,10 @@ std::string validate(const Program &p) {
           if (depth < 2) return "region program: binary operation on fewer than two values";
           --depth;
           break;
-        case OpCode::Relu: case OpCode::Leaky: case OpCode::Neg:
+        case OpCode::Relu: case OpCode::Leaky: case OpCode::Neg: case OpCode::Cast:
           if (integer && o.code == OpCode::Leaky) return "region program: 'leaky' is not available in an integer region";
+          if (integer && o.code == OpCode::Cast) return "region program: 'cast' is not available in an integer region";
+          if (o.code == OpCode::Cast && !isFloat(o.constType)) return "region program: 'cast' to a type that is not f16, bf16 or f32";
           if (depth < 1) return "region program: unary operation on an empty stack";
           break;
         case OpCode::ReduceSum:
@@ -561,6 +570,7 @@ std::string resolve(const Program &p, const std::vector<int64_t> &dims, Resolved
       ro.code = o.code;
       ro.constant = o.extent ? roundThroughType((float)value(o.constRef), o.constType) : o.constant;
       ro.depth = o.depth;
+      ro.castType = o.constType;
       if (inTail && o.code != OpCode::Store) {
         // symbolic evaluation: entries are the running sum or float32 constants
         auto fold = [](OpCode c, float a, float b) {
@@ -576,13 +586,14 @@ std::string resolve(const Program &p, const std::vector<int64_t> &dims, Resolved
         switch (o.code) {
           case OpCode::Const: tailStack.push_back({false, ro.constant}); break;
           case OpCode::Dup: tailStack.push_back(tailStack[tailStack.size() - 1 - o.depth]); break;
-          case OpCode::Relu: case OpCode::Leaky: case OpCode::Neg: {
+          case OpCode::Relu: case OpCode::Leaky: case OpCode::Neg: case OpCode::Cast: {
             TailEntry &e = tailStack.back();
             if (e.sum) {
-              s.tail.push_back({o.code, o.constant, false});
+              s.tail.push_back({o.code, o.constant, false, o.constType});
             } else {
               const float v = e.value;
-              e.value = o.code == OpCode::Neg ? -v : fold(OpCode::Max, v, o.code == OpCode::Relu ? 0.f : v * o.constant);
+              e.value = o.code == OpCode::Cast ? roundThroughType(v, o.constType)
+                        : o.code == OpCode::Neg ? -v : fold(OpCode::Max, v, o.code == OpCode::Relu ? 0.f : v * o.constant);
             }
             break;
           }

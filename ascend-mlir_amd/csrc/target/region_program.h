@@ -49,6 +49,9 @@
 //                               type is given (arith.sitofp of a tensor.dim to that type)
 //     add | sub | mul | div | max | min      pop b, pop a, push a op b
 //     relu | leaky <alpha> | neg             on the top of the stack
+//     cast <f16|bf16|f32>       round the top of the stack to that type and widen it again
+//                               (arith.truncf / arith.extf, afir.cast; a row sum that the IR
+//                               keeps in a narrower tensor before the next operation reads it)
 //     dup <n>                   push a copy of the n-th entry from the top
 //     reduce sum                sum the value over the last iteration dim
 //     ...                       after 'reduce sum': operations on the row's sum with constants
@@ -92,7 +95,7 @@ struct Ref {
   static Ref value(int64_t c) { Ref r; r.constant = c; return r; }
 };
 
-enum class OpCode { Push, Const, Add, Sub, Mul, Div, Max, Min, Relu, Leaky, Neg, Dup, ReduceSum, Store, Matmul };
+enum class OpCode { Push, Const, Add, Sub, Mul, Div, Max, Min, Relu, Leaky, Neg, Dup, ReduceSum, Store, Matmul, Cast };
 
 struct MapResult {
   enum Kind { IterDim, Constant, Gather } kind = IterDim;
@@ -111,7 +114,7 @@ struct Op {
   float constant = 0.f;             // Const, Leaky
   bool extent = false;              // Const: the value is an extent (constRef), not `constant`
   Ref constRef;                     // Const with extent set
-  ElemType constType = ElemType::F32;  // ... rounded through this float type
+  ElemType constType = ElemType::F32;  // ... rounded through this float type; Cast: the type
   int depth = 0;                    // Dup
 };
 
@@ -166,6 +169,7 @@ struct ResolvedOp {
   bool transA = false, transB = false;
   float constant = 0.f;
   int depth = 0;
+  ElemType castType = ElemType::F32;   // Cast
 };
 
 struct ResolvedSegment {
@@ -183,6 +187,7 @@ struct ResolvedSegment {
     OpCode code = OpCode::Add;
     float constant = 0.f;   // the other operand; alpha of Leaky
     bool reversed = false;
+    ElemType castType = ElemType::F32;   // Cast
   };
   std::vector<TailStep> tail;
 };

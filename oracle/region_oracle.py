@@ -22,11 +22,16 @@ What a program means follows the reference's lowering of fused regions
                  (examples/add-broadcast-concat/step0_input.mlir)
   mean           sum, then operations on the row's sum with constants and extents
                  (examples/broadcast-add-reduce/step0_input_mean.mlir:56-84: sum / N with N
-                 an arith.sitofp of the extent); float32 arithmetic on the float32 sum, one
-                 rounding to the output type -- the reference holds no golden for this
-                 graph (its gen_data.py writes the sum only), so where the intermediate f16
-                 tensor of the reference's IR would round the sum first, the two differ by at
-                 most one unit in the last place of the output: PARITY UNPINNED to that extent
+                 an arith.sitofp of the extent).  The IR keeps the sum in an f16 tensor
+                 before the division reads it, so the program rounds it there ('reduce sum',
+                 'cast f16', then the division in float32 and one rounding to the output type,
+                 which for two f16 operands is the correctly rounded f16 quotient).  The
+                 reference holds no golden for this graph (its gen_data.py writes the sum
+                 only); the test ties the mean to that sum vector
+  cast           round to f16 / bf16 (nearest even, overflow to infinity) and widen again:
+                 arith.truncf + arith.extf, afir.cast
+                 (include/Dialect/AFIR/Ops/Basic/cast.td:22-25), pinned against numpy's
+                 float16 conversion and the bf16 bit formula of the comparator
   goldens        "compute in f32, cast to the storage type"
                  (examples/*/gen_data.py, gen_inputs.py)
 
@@ -121,6 +126,10 @@ def parse(text: str) -> dict:
             seg["ops"].append((k, np.float32(float(tok[1]))))
         elif k == "dup":
             seg["ops"].append(("dup", int(tok[1])))
+        elif k == "cast":
+            if tok[1] not in ("f16", "bf16", "f32"):
+                raise RegionError("cast to a type that is not f16, bf16 or f32")
+            seg["ops"].append(("cast", tok[1]))
         elif k == "reduce":
             seg["ops"].append(("reduce",))
         else:
@@ -297,6 +306,17 @@ def evaluate(text: str, inputs, out_shape=None):
                     stack.append(ieee_max(x, (x * op[1]).astype(np.float32)))
             elif k == "neg":
                 stack.append(-stack.pop())
+            elif k == "cast":
+                # round to the narrower type (nearest even, overflow to infinity) and widen again:
+                # arith.truncf followed by arith.extf, afir.cast
+                # (include/Dialect/AFIR/Ops/Basic/cast.td:22-25)
+                x = stack.pop()
+                if op[1] == "f16":
+                    with np.errstate(over="ignore"):
+                        x = x.astype(np.float16).astype(np.float32)
+                elif op[1] == "bf16":
+                    x = O.bf16_bits_to_f32(O.f32_to_bf16_bits(np.ascontiguousarray(x, dtype=np.float32))).reshape(x.shape)
+                stack.append(x)
             elif k == "reduce":
                 # float32 accumulation in numpy's pairwise order, as the
                 # reference goldens do it; a kernel's own summation order is

@@ -50,8 +50,8 @@ def cases():
 
 def mean_case():
     """The reference's mean graph (examples/broadcast-add-reduce/step0_input_mean.mlir) on the vectors its
-    gen_data.py wrote for the sum.  The reference holds no mean output; its sum does fix the mean to one
-    f16 ulp: mean = sum / N, and output_c is that sum rounded to f16 once already."""
+    gen_data.py wrote for the sum.  The reference holds no mean output, but output_c is the f16 tensor of
+    sums that the graph's division reads: mean = output_c / N, rounded once."""
     z = load()
     e = "broadcast-add-reduce/"
     a, b, c = (np.ascontiguousarray(z[e + k]) for k in ("input_a", "input_b", "output_c"))

@@ -465,3 +465,62 @@ BATCH_MATMUL_TRANSPOSE_B_F16 = BATCH_MATMUL_BF16.replace("xbf16", "xf16").replac
     .replace("outs(%init : tensor<?x?x?xf16>) -> tensor<?x?x?xf16>", "outs(%init : tensor<?x?x?xf32>) -> tensor<?x?x?xf32>") \
     .replace("%init : tensor<?x?x?xf16>) -> tensor<?x?x?xf16> {", "%init : tensor<?x?x?xf32>) -> tensor<?x?x?xf32> {") \
     .replace("return %c : tensor<?x?x?xf16>", "return %c : tensor<?x?x?xf32>").replace("@bmm", "@bmm_tb")
+
+# a mixed-precision chain: f32 values rounded to f16 where the IR says so (arith.truncf), widened
+# again (arith.extf, exact) and used in float32 arithmetic:
+# out = f16(f32(f16(a)) + f32(b)) * a), a f32 [m, n], b f16 [n]
+MIXED_PRECISION_CHAIN = """
+func.func @mixed(%a : tensor<?x?xf32>, %b : tensor<?xf16>) -> tensor<?x?xf16> {
+  %c0 = arith.constant 0 : index
+  %c1 = arith.constant 1 : index
+  %m = tensor.dim %a, %c0 : tensor<?x?xf32>
+  %n = tensor.dim %a, %c1 : tensor<?x?xf32>
+  %e = tensor.empty(%m, %n) : tensor<?x?xf16>
+  %o = linalg.generic {indexing_maps = [affine_map<(d0, d1) -> (d0, d1)>, affine_map<(d0, d1) -> (d1)>,
+                                        affine_map<(d0, d1) -> (d0, d1)>], iterator_types = ["parallel", "parallel"]}
+      ins(%a, %b : tensor<?x?xf32>, tensor<?xf16>) outs(%e : tensor<?x?xf16>) {
+    ^bb0(%x: f32, %y: f16, %q: f16):
+      %t = arith.truncf %x : f32 to f16
+      %tw = arith.extf %t : f16 to f32
+      %yw = arith.extf %y : f16 to f32
+      %s = arith.addf %tw, %yw : f32
+      %v = arith.mulf %s, %x : f32
+      %r = arith.truncf %v : f32 to f16
+      linalg.yield %r : f16
+  } -> tensor<?x?xf16>
+  return %o : tensor<?x?xf16>
+}
+"""
+
+# the named linalg ops and reshapes the reference's --linalg-mark / --linalg-add-broadcast passes
+# consume and produce (test/Dialect/AFIR/Transforms/linalgMark.mlir:35-44,
+# linalgAddBroadcast.mlir:17-21), and afir.cast between float types
+# (include/Dialect/AFIR/Ops/Basic/cast.td:22-25):
+# out = bf16((a + transpose(b)) * broadcast(c)) widened to f32, a [4, 8], b [8, 4], c [8]
+NAMED_OPS_GRAPH = """
+func.func @named(%a : tensor<4x8xf32>, %b : tensor<8x4xf32>, %c : tensor<8xf32>) -> tensor<4x8xf32> {
+  %z = arith.constant dense<0.0> : tensor<4x8xf32>
+  %e1 = tensor.empty() : tensor<4x8xf32>
+  %bt = linalg.transpose ins(%b : tensor<8x4xf32>) outs(%e1 : tensor<4x8xf32>) permutation = [1, 0]
+  %s = linalg.add ins(%a, %bt : tensor<4x8xf32>, tensor<4x8xf32>) outs(%z : tensor<4x8xf32>) -> tensor<4x8xf32>
+  %e2 = tensor.empty() : tensor<4x8xf32>
+  %cb = linalg.broadcast ins(%c : tensor<8xf32>) outs(%e2 : tensor<4x8xf32>) dimensions = [0]
+  %m = linalg.mul ins(%s, %cb : tensor<4x8xf32>, tensor<4x8xf32>) outs(%z : tensor<4x8xf32>) -> tensor<4x8xf32>
+  %x = tensor.expand_shape %m [[0, 1], [2]] output_shape [4, 1, 8] : tensor<4x8xf32> into tensor<4x1x8xf32>
+  %y = tensor.collapse_shape %x [[0, 1], [2]] : tensor<4x1x8xf32> into tensor<4x8xf32>
+  %r = afir.cast %y : tensor<4x8xf32> -> tensor<4x8xbf16>
+  %w = afir.cast %r : tensor<4x8xbf16> -> tensor<4x8xf32>
+  return %w : tensor<4x8xf32>
+}
+"""
+
+# linalg.elementwise with broadcast maps, dynamic shapes: out[i, j, k] = a[j, k] - c[i, 0, k]
+ELEMENTWISE_KIND_SUB = """
+func.func @ew_sub(%a : tensor<?x?xf16>, %c : tensor<?x1x?xf16>, %init : tensor<?x?x?xf16>) -> tensor<?x?x?xf16> {
+  %r = linalg.elementwise kind=#linalg.elementwise_kind<sub>
+      indexing_maps = [affine_map<(d0, d1, d2) -> (d1, d2)>, affine_map<(d0, d1, d2) -> (d0, 0, d2)>,
+                       affine_map<(d0, d1, d2) -> (d0, d1, d2)>]
+      ins(%a, %c : tensor<?x?xf16>, tensor<?x1x?xf16>) outs(%init : tensor<?x?x?xf16>) -> tensor<?x?x?xf16>
+  return %r : tensor<?x?x?xf16>
+}
+"""

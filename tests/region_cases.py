@@ -30,7 +30,8 @@ end
 """
 
 # c[m] = f16(sum_n (a[m] + b[m,n]) / N)    examples/broadcast-add-reduce/step0_input_mean.mlir
-MEAN_ROWBIAS = REDUCE_ROWBIAS.replace("  reduce sum\n", "  reduce sum\n  const arg1.1 f16\n  div\n")
+# (the IR keeps the sums in an f16 tensor before the division reads them: 'cast f16')
+MEAN_ROWBIAS = REDUCE_ROWBIAS.replace("  reduce sum\n", "  reduce sum\n  cast f16\n  const arg1.1 f16\n  div\n")
 # the sum put through a longer chain: relu(4 - s * 0.5) * (N / 2), extents and constants mixed
 REDUCE_TAIL_CHAIN = REDUCE_ROWBIAS.replace(
     "  reduce sum\n", "  reduce sum\n  const 0.5\n  mul\n  neg\n  const 4\n  add\n  relu\n  const arg1.1\n  const 0.5\n  mul\n  mul\n")
@@ -258,11 +259,13 @@ def case_reduce_rowbias(m=640, n=512, seed=42):
 
 
 def mean_rowbias_f16(a, b):
-    """The mean graph's golden: the float32 row sum divided by N in float32, one rounding to
-    f16 (N goes through f16 like the IR's sitofp; exact up to 2048)."""
+    """The mean graph's golden: the float32 row sum rounded to f16 (the IR's tensor<?xf16> of
+    sums), divided by N (through f16 like the IR's sitofp; exact up to 2048): the correctly
+    rounded f16 quotient of two f16 values, computed in float32."""
     n = np.float32(np.float16(b.shape[1]))
-    s = (a.astype(np.float32)[:, None] + b.astype(np.float32)).sum(axis=1, dtype=np.float32)
-    return (s / n).astype(np.float16)
+    with np.errstate(over="ignore"):
+        s = (a.astype(np.float32)[:, None] + b.astype(np.float32)).sum(axis=1, dtype=np.float32).astype(np.float16)
+    return (s.astype(np.float32) / n).astype(np.float16)
 
 
 def case_mean_rowbias(m=640, n=512, seed=42):
@@ -286,6 +289,74 @@ def case_pre_reduce_div_extent(m=96, n=256, seed=6):
     b = rng.integers(-4, 5, (m, n)).astype(np.float16)
     terms = (a.astype(np.float32)[:, None] + b.astype(np.float32)) / np.float32(n)
     return PRE_REDUCE_DIV_EXTENT, [a, b], (terms.sum(axis=1, dtype=np.float32) * np.float32(m)).astype(np.float16)
+
+
+# mixed precision: out = f16((f32(f16(a)) + b) * a), a f32, b f16 per column; and the same
+# rounding through bf16 in the middle of a float32 chain, out = f32(bf16(a * b) - b)
+CAST_CHAIN_F16 = HEADER + """
+arg in f32 2
+arg in f16 1
+arg out f16 2
+segment 2
+  size arg0.0 arg0.1
+  outoff 0
+  push arg0 d0 d1
+  cast f16
+  push arg1 d1
+  add
+  push arg0 d0 d1
+  mul
+  store
+end
+"""
+CAST_CHAIN_BF16 = HEADER + """
+arg in f32 2
+arg in f32 2
+arg out f32 2
+segment 2
+  size arg0.0 arg0.1
+  outoff 0
+  push arg0 d0 d1
+  push arg1 d0 d1
+  mul
+  cast bf16
+  push arg1 d0 d1
+  sub
+  store
+end
+"""
+
+
+def _special_f32(rng, shape):
+    """Uniform values with the float32 corner cases of a rounding mixed in: ties, values that
+    overflow f16, f16 subnormals, infinities, NaN, both zeros."""
+    x = rng.uniform(-4, 4, shape).astype(np.float32)
+    flat = x.reshape(-1)
+    corners = np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e6, -1e6, 6e-8, 3e-8, 2.98e-8, np.inf, -np.inf, np.nan,
+                        1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11, 2049.0, 2051.0, 1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8],
+                       np.float32)
+    flat[:corners.size] = corners
+    return x
+
+
+def case_cast_chain_f16(m=70, n=333, seed=11):
+    rng = np.random.default_rng(seed)
+    a = _special_f32(rng, (m, n))
+    b = rng.uniform(-2, 2, (n,)).astype(np.float16)
+    with np.errstate(all="ignore"):
+        want = ((a.astype(np.float16).astype(np.float32) + b.astype(np.float32)) * a).astype(np.float16)
+    return CAST_CHAIN_F16, [a, b], want
+
+
+def case_cast_chain_bf16(m=64, n=256, seed=12):
+    rng = np.random.default_rng(seed)
+    a = _special_f32(rng, (m, n))
+    b = rng.uniform(-2, 2, (m, n)).astype(np.float32)
+    with np.errstate(all="ignore"):
+        p = (a * b).astype(np.float32)
+        rounded = O.bf16_bits_to_f32(O.f32_to_bf16_bits(p))
+        want = (rounded - b).astype(np.float32)
+    return CAST_CHAIN_BF16, [a, b], want
 
 
 def case_reduce_tail_chain(m=77, n=300, seed=9):
@@ -362,6 +433,7 @@ EXACT_CASES = {
     "split_relu_brc_add_mul": case_split_relu_brc_add_mul,
     "c1": case_c1, "c3": case_c3, "c4": case_c4, "add_mul_3": case_add_mul_3,
     "parallel_div_extent": case_parallel_div_extent, "pre_reduce_div_extent": case_pre_reduce_div_extent,
+    "cast_chain_f16": case_cast_chain_f16, "cast_chain_bf16": case_cast_chain_bf16,
 }
 REDUCE_CASES = {"reduce_rowbias": case_reduce_rowbias, "c2": case_c2, "mean_rowbias": case_mean_rowbias,
                 "reduce_tail_chain": case_reduce_tail_chain}

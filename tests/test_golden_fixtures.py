@@ -58,5 +58,4 @@ def test_mean_graph_agrees_with_the_reference_sum_vector():
     assert p.returncode == 0, p.stderr
     got = RO.evaluate(p.stdout, inputs)
     assert got.dtype == want.dtype and got.shape == want.shape
-    assert GC.within_one_f16_ulp(got, want)
-    assert np.mean(got.view(np.uint16) == want.view(np.uint16)) > 0.5     # the second rounding moves the rest by one ulp
+    assert got.tobytes() == want.tobytes()    # the graph divides the f16 sums the reference wrote

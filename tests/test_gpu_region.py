@@ -156,6 +156,32 @@ def test_mean_graph_from_mlir_runs_on_every_route(H):
     assert np.abs(got.view(np.int16).astype(int) - want.view(np.int16).astype(int)).max() <= 1
 
 
+def test_mixed_precision_and_named_op_graphs_from_mlir_run_on_every_route(H):
+    """MLIR text with arith.truncf / extf, linalg named ops, unit-dim reshapes and afir.cast
+    (tests/mlir_cases.py) -> program -> the interpreter's two evaluators and the compiled
+    kernels, bit for bit against the region oracle."""
+    import os
+    import subprocess
+    from tests import mlir_cases as MC
+    tr = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "ascend-mlir_amd", "bin", "afir-translate")
+    rng = np.random.default_rng(21)
+    a = rng.uniform(-3, 3, (33, 520)).astype(np.float32)
+    a[0, :6] = [65519.9, 65520.0, 1e6, 6e-8, np.nan, -np.inf]
+    b = rng.uniform(-3, 3, (520,)).astype(np.float16)
+    text = subprocess.run([tr, "-mlir-to-hip", "-"], input=MC.MIXED_PRECISION_CHAIN, capture_output=True, text=True, check=True).stdout
+    with np.errstate(all="ignore"):
+        want = RO.evaluate(text, [a, b])
+    got = run(H, text, [a, b], a.shape)
+    assert got.tobytes() == want.tobytes()
+    text = subprocess.run([tr, "-mlir-to-hip", "-"], input=MC.NAMED_OPS_GRAPH, capture_output=True, text=True, check=True).stdout
+    x, y, c = (rng.uniform(-2, 2, sh).astype(np.float32) for sh in ((4, 8), (8, 4), (8,)))
+    assert run(H, text, [x, y, c], (4, 8)).tobytes() == RO.evaluate(text, [x, y, c]).tobytes()
+    text = subprocess.run([tr, "-mlir-to-hip", "-"], input=MC.ELEMENTWISE_KIND_SUB, capture_output=True, text=True, check=True).stdout
+    p, q = rng.uniform(-2, 2, (7, 40)).astype(np.float16), rng.uniform(-2, 2, (5, 1, 40)).astype(np.float16)
+    init = np.zeros((5, 7, 40), np.float16)
+    assert run(H, text, [p, q, init], (5, 7, 40)).tobytes() == RO.evaluate(text, [p, q, init]).tobytes()
+
+
 @pytest.mark.parametrize("n", [1, 3, 8, 16, 40, 64, 100, 256, 520])
 def test_row_sums_of_short_rows(H, n):
     """Rows shorter than a pass of the wavefront: 1, 2, 4 ... 32 lanes share a row and a

@@ -246,7 +246,7 @@ def test_emit_options_change_the_tile_and_the_unroll(tmp_path):
 def test_operations_after_reduce_sum_are_applied_to_the_row_sum_where_it_is_stored():
     src = _emit(RC.MEAN_ROWBIAS).stdout
     assert "float extent_const[8];" in src
-    assert src.count("(s / R.extent_const[0])") >= 4        # every kernel that stores a row sum
+    assert src.count("(rt_f16(s) / R.extent_const[0])") >= 4        # every kernel that stores a row sum
     assert "v0[u][e] / " not in src                          # not per element
     chain = _emit(RC.REDUCE_TAIL_CHAIN).stdout
     half, four = "as_f32(0x3f000000u) /* 0.5 */", "as_f32(0x40800000u) /* 4 */"

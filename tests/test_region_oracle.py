@@ -198,19 +198,27 @@ def test_mean_tail_is_pinned_by_exact_cases():
     a = np.zeros((2,), np.float16)
     b = np.ones((2, 2049), np.float16)
     assert RO.evaluate(RC.MEAN_ROWBIAS, [a, b]).tolist() == [np.float16(2049 / 2048)] * 2
-    assert RO.evaluate(RC.MEAN_ROWBIAS.replace("const arg1.1 f16", "const arg1.1"), [a, b]).tolist() == [1.0, 1.0]
+    # ... and the sum: the IR keeps it in an f16 tensor, where 2049 is 2048 as well ('cast f16');
+    # a program without that rounding divides the float32 sum
+    assert RO.evaluate(RC.MEAN_ROWBIAS.replace("const arg1.1 f16", "const arg1.1"), [a, b]).tolist() == [1 - 2.0 ** -11] * 2
+    plain = RC.MEAN_ROWBIAS.replace("  cast f16\n", "").replace("const arg1.1 f16", "const arg1.1")
+    assert RO.evaluate(plain, [a, b]).tolist() == [1.0, 1.0]
+    # a sum beyond the f16 range is infinite in that tensor, and so is the mean
+    b = np.full((2, 2048), 40.0, np.float16)
+    assert np.isinf(RO.evaluate(RC.MEAN_ROWBIAS, [a, b])).all()
+    assert RO.evaluate(RC.MEAN_ROWBIAS.replace("  cast f16\n", ""), [a, b]).tolist() == [40.0, 40.0]
 
 
 def test_mean_against_the_reference_written_sum_vector():
-    """The reference's golden script writes the row SUMS of its example (as f16); the mean of
-    the same inputs can differ from that vector divided by N only by the second rounding."""
+    """The reference's golden script writes the row SUMS of its example (as f16), which is the
+    tensor the mean graph's division reads: the mean is that vector divided by N, exactly."""
     from tests import golden_cases as GC
     z = GC.load()
     a, b, sums = (np.ascontiguousarray(z["broadcast-add-reduce/" + k]) for k in ("input_a", "input_b", "output_c"))
     got = RO.evaluate(RC.MEAN_ROWBIAS, [a, b])
     assert got.tobytes() == RC.mean_rowbias_f16(a, b).tobytes()
     twice = (sums.astype(np.float32) / np.float32(b.shape[1])).astype(np.float16)
-    assert np.abs(got.view(np.int16).astype(int) - twice.view(np.int16).astype(int)).max() <= 1
+    assert got.tobytes() == twice.tobytes()
 
 
 def test_reduce_tail_chain_matches_its_closed_form():
@@ -238,3 +246,33 @@ def test_matmul_layout_flags_against_numpy():
             " matmul arg0 arg1 tb\n store\nend\n")
     got = RO.evaluate(prog, [a3, b3], out_shape=(nb, m, n))
     assert np.array_equal(got, want3)
+
+
+def test_cast_is_the_rounding_of_the_storage_types():
+    """'cast f16' / 'cast bf16' against numpy's float16 conversion and the bf16 bit formula the
+    comparator decodes with (round to nearest even, overflow to infinity, NaN stays NaN), value
+    by value on the corner cases: ties, the f16 overflow threshold, subnormals, zeros of both signs."""
+    prog = RC.HEADER + "arg in f32 1\narg out f32 1\nsegment 1\n size arg0.0\n outoff 0\n push arg0 d0\n cast %s\n store\nend\n"
+    x = np.array([0.0, -0.0, 1.0, 1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11, 1.0 + 2.0 ** -10, 2049.0, 2051.0, 65504.0, 65519.99,
+                  65520.0, -65520.0, 1e9, 6e-8, 2.9802322e-8, 2.99e-8, 5.9604645e-8, -1e-10, np.inf, -np.inf, np.nan,
+                  1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8, 3.4e38, 1.0 + 2.0 ** -7 + 2.0 ** -20], np.float32)
+    got = RO.evaluate(prog % "f16", [x])
+    by_hand = np.array([0.0, -0.0, 1.0, 1.0, 1.0 + 2.0 ** -9, 1.0 + 2.0 ** -10, 2048.0, 2052.0, 65504.0, 65504.0,
+                        np.inf, -np.inf, np.inf, 2.0 ** -24, 0.0, 2.0 ** -24, 2.0 ** -24, -0.0, np.inf, -np.inf, np.nan,
+                        1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8, np.inf, 1.0 + 2.0 ** -7], np.float32)
+    assert np.array_equal(got, by_hand, equal_nan=True) and np.signbit(got[1]) and np.signbit(got[17])
+    with np.errstate(over="ignore"):
+        assert np.array_equal(got, x.astype(np.float16).astype(np.float32), equal_nan=True)
+    got = RO.evaluate(prog % "bf16", [x])
+    by_hand_bf16 = {1.0 + 2.0 ** -8: 1.0, 1.0 + 3 * 2.0 ** -8: 1.0 + 2.0 ** -6, 1.0 + 2.0 ** -7 + 2.0 ** -20: 1.0 + 2.0 ** -7,
+                    65504.0: 65536.0, 3.4e38: np.inf, 2049.0: 2048.0}
+    for value, want in by_hand_bf16.items():
+        assert got[np.flatnonzero(x == np.float32(value))[0]] == np.float32(want), value
+    u = x.view(np.uint32).astype(np.uint64)
+    formula = (((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16).astype(np.uint32).view(np.float32)
+    finite = ~np.isnan(x)
+    assert np.array_equal(got[finite], formula[finite]) and np.isnan(got[~finite]).all()
+    assert np.array_equal(RO.evaluate(prog % "f32", [x]), x, equal_nan=True)
+    rng = np.random.default_rng(0)
+    y = rng.standard_normal(100000).astype(np.float32) * np.float32(1000)
+    assert np.array_equal(RO.evaluate(prog % "f16", [y]), y.astype(np.float16).astype(np.float32))

@@ -189,7 +189,7 @@ def test_mean_is_a_sum_with_a_tail_on_the_row_sums():
     out = program_of(MC.ROW_BIAS_MEAN)
     body = [l.strip() for l in out.splitlines() if l.strip() and not l.startswith("#")]
     assert body[body.index("outoff 0") + 1:] == [
-        "push arg0 d0", "push arg1 d0 d1", "add", "reduce sum", "const arg1.1 f16", "div", "store", "end"]
+        "push arg0 d0", "push arg1 d0 d1", "add", "reduce sum", "cast f16", "const arg1.1 f16", "div", "store", "end"]
     _, inputs, want = RC.case_mean_rowbias(33, 96)
     assert RO.evaluate(out, inputs).tobytes() == want.tobytes()
     # c - sum, sum * c, max(sum, c): the sum as either operand where the operation allows it
@@ -198,7 +198,7 @@ def test_mean_is_a_sum_with_a_tail_on_the_row_sums():
                        ("arith.maximumf %x, %nf", ["const arg1.1 f16", "max"])):
         out = program_of(MC.ROW_BIAS_MEAN.replace("arith.divf %x, %nf", expr))
         body = [l.strip() for l in out.splitlines() if l.strip() and not l.startswith("#")]
-        assert body[body.index("reduce sum") + 1:-2] == tail, expr
+        assert body[body.index("reduce sum") + 1:-2] == ["cast f16"] + tail, expr    # the sums are an f16 tensor
     bad = subprocess.run([TR, "-mlir-to-hip", "-"], input=MC.ROW_BIAS_MEAN.replace("arith.divf %x, %nf", "arith.divf %nf, %x"),
                          capture_output=True, text=True)
     assert bad.returncode != 0 and "divided by a reduced value" in bad.stderr
@@ -247,14 +247,18 @@ def test_reference_afir_lit_functions_translate():
     good = ["test_add", "test_sub", "test_mul", "test_div", "test_truediv", "test_minimum", "test_maximum",
             "test_relu", "test_neg", "test_leaky_relu", "test_abs", "test_abs_f16", "test_broadcast", "test_load",
             "test_store", "test_sum_reduce", "test_reduce_3d", "test_binary_1d", "test_binary_3d", "test_unary_1d",
-            "test_unary_3d", "test_add_output_double_buffer", "test_abs_output_vector_out"]
+            "test_unary_3d", "test_add_output_double_buffer", "test_abs_output_vector_out",
+            "test_cast_f16_to_f32", "test_cast_f32_to_f16", "test_cast_output_vector_out"]
     for fn in good:
         p = subprocess.run([TR, "-mlir-to-hip", AFIR_LIT, "--function", fn], capture_output=True, text=True)
         assert p.returncode == 0, (fn, p.stderr)
         assert p.stdout.startswith(f"# kernel {fn}\nafir-hip-region 1\n") and p.stdout.rstrip().endswith("store\nend")
-    for fn, op in (("test_exp", "afir.exp"), ("test_eq", "afir.eq"), ("test_cast_f16_to_f32", "afir.cast")):
+    for fn, op in (("test_exp", "afir.exp"), ("test_eq", "afir.eq")):
         p = subprocess.run([TR, "-mlir-to-hip", AFIR_LIT, "--function", fn], capture_output=True, text=True)
         assert p.returncode == 1 and f"{op} has no HIP lowering" in p.stderr, (fn, p.stderr)
+    # a cast from an integer tensor is outside the float chains this backend lowers
+    p = subprocess.run([TR, "-mlir-to-hip", AFIR_LIT, "--function", "test_cast"], capture_output=True, text=True)
+    assert p.returncode == 1 and "integer and floating-point tensors" in p.stderr, p.stderr
     p = subprocess.run([TR, "-mlir-to-hip", AFIR_LIT, "--function", "nope"], capture_output=True, text=True)
     assert p.returncode == 1 and "no function @nope" in p.stderr
 
@@ -361,3 +365,77 @@ def test_transposed_and_batched_matmul_ops(pkg):
     bad = program_of(MC.MATMUL_TRANSPOSE_B_F16).replace("matmul arg0 arg1 tb", "matmul arg0 arg1 tb ta")
     with pytest.raises(H.AfirHipError, match=r"\[ta\] \[tb\]"):
         H.Region(bad)
+
+
+def _body(text):
+    out = program_of(text)
+    return [l.strip() for l in out.splitlines() if l.strip() and not l.startswith("#")]
+
+
+def test_mixed_precision_chain_rounds_where_the_ir_truncates():
+    """arith.truncf is a rounding to the narrower type ('cast f16'), arith.extf changes nothing;
+    the last truncf to the output's own type is the store's rounding."""
+    body = _body(MC.MIXED_PRECISION_CHAIN)
+    assert body[body.index("outoff 0") + 1:] == [
+        "push arg0 d0 d1", "cast f16", "push arg1 d1", "add", "push arg0 d0 d1", "mul", "store", "end"]
+    rng = np.random.default_rng(8)
+    a = rng.uniform(-3, 3, (5, 40)).astype(np.float32)
+    b = rng.uniform(-3, 3, (40,)).astype(np.float16)
+    want = ((a.astype(np.float16).astype(np.float32) + b.astype(np.float32)) * a).astype(np.float16)
+    assert RO.evaluate(program_of(MC.MIXED_PRECISION_CHAIN), [a, b]).tobytes() == want.tobytes()
+    # without the inner rounding the result differs: the cast is not decoration
+    plain = ((a + b.astype(np.float32)) * a).astype(np.float16)
+    assert plain.tobytes() != want.tobytes()
+
+
+def test_named_linalg_ops_reshapes_and_float_casts():
+    """linalg.transpose / add / broadcast / mul, a dense splat as init, expand_shape and
+    collapse_shape of a unit dim, afir.cast down to bf16 and up again."""
+    body = _body(MC.NAMED_OPS_GRAPH)
+    assert body[body.index("outoff 0") + 1:] == [
+        "push arg0 d0 d1", "push arg1 d1 d0", "add", "push arg2 d1", "mul", "cast bf16", "store", "end"]
+    assert "size 4 8" in body
+    rng = np.random.default_rng(9)
+    a, b, c = (rng.uniform(-2, 2, s).astype(np.float32) for s in ((4, 8), (8, 4), (8,)))
+    v = (a + b.T) * c[None, :]
+    u = v.view(np.uint32)
+    want = (((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16).astype(np.uint32).view(np.float32)     # bf16, nearest even
+    assert RO.evaluate(program_of(MC.NAMED_OPS_GRAPH), [a, b, c]).tobytes() == want.tobytes()
+
+
+def test_linalg_elementwise_with_broadcast_maps():
+    body = _body(MC.ELEMENTWISE_KIND_SUB)
+    assert body[body.index("outoff 0") + 1:] == ["push arg0 d1 d2", "push arg1 d0 0 d2", "sub", "store", "end"]
+    assert "size arg2.0 arg2.1 arg2.2" in body
+    for kind in ("tanh", "exp", "erf"):
+        bad = subprocess.run([TR, "-mlir-to-hip", "-"], input=MC.ELEMENTWISE_KIND_SUB.replace("<sub>", f"<{kind}>"),
+                             capture_output=True, text=True)
+        assert bad.returncode == 1 and f"elementwise kind '{kind}' has no HIP lowering" in bad.stderr
+    # reshapes that re-linearise, and dense constants that are not splats, are refused by name
+    bad = subprocess.run([TR, "-mlir-to-hip", "-"], capture_output=True, text=True, input=MC.NAMED_OPS_GRAPH.replace(
+        "[[0, 1], [2]] : tensor<4x1x8xf32> into tensor<4x8xf32>", "[[0, 1, 2]] : tensor<4x1x8xf32> into tensor<32xf32>"))
+    assert bad.returncode == 1 and "merge or split dims of extent other than 1" in bad.stderr
+    bad = subprocess.run([TR, "-mlir-to-hip", "-"], capture_output=True, text=True,
+                         input=MC.NAMED_OPS_GRAPH.replace("dense<0.0> : tensor<4x8xf32>", "dense<[[1.0]]> : tensor<1x1xf32>"))
+    assert bad.returncode == 1 and "other than splats" in bad.stderr
+
+
+LINALG_ADD_BROADCAST = "/root/reference/test/Dialect/AFIR/Transforms/linalgAddBroadcast.mlir"
+
+
+@pytest.mark.skipif(not os.path.isfile(LINALG_ADD_BROADCAST), reason="reference tree not present")
+def test_reference_linalg_add_broadcast_input_translates():
+    """The input of the reference's --linalg-add-broadcast test (a linalg.elementwise add with
+    broadcasting maps) translates as it stands; its tanh function is refused by kind."""
+    p = subprocess.run([TR, "-mlir-to-hip", LINALG_ADD_BROADCAST, "--function", "unary_broadcast_addf"],
+                       capture_output=True, text=True)
+    assert p.returncode == 0, p.stderr
+    body = [l.strip() for l in p.stdout.splitlines() if l.strip() and not l.startswith("#")]
+    assert body[body.index("outoff 0") + 1:] == ["push arg0 d1 d2", "push arg1 d0 0 d2", "add", "store", "end"]
+    rng = np.random.default_rng(10)
+    a, c = rng.uniform(-1, 1, (16, 32)).astype(np.float32), rng.uniform(-1, 1, (8, 1, 32)).astype(np.float32)
+    init = np.zeros((8, 16, 32), np.float32)
+    assert RO.evaluate(p.stdout, [a, c, init]).tobytes() == (a[None] + c).tobytes()
+    p = subprocess.run([TR, "-mlir-to-hip", LINALG_ADD_BROADCAST, "--function", "unary_broadcast_tanh"],
+                       capture_output=True, text=True)
+    assert p.returncode == 1 and "elementwise kind 'tanh' has no HIP lowering" in p.stderr
