@@ -52,6 +52,14 @@ DEV unsigned as_u32(float f) { return __builtin_bit_cast(unsigned, f); }
 DEV float fmax_ieee(float a, float b) { return __builtin_elementwise_maximum(a, b); }
 DEV float fmin_ieee(float a, float b) { return __builtin_elementwise_minimum(a, b); }
 
+// A float32 value as the compiler may not look into it.  Without this, the conversion of a
+// product to f16 is selected as one v_fma_mixlo_f16 with a zero addend: a single rounding of the
+// exact product where the program asks for two (to float32, then to f16), and +0 where the
+// product is -0.
+DEV float f32_value(float x) {
+  asm("" : "+v"(x));
+  return x;
+}
 // ---- element access: float32 in registers, one round-to-nearest-even on store
 DEV float ld_f32(const void *b, long long i) { return ((const float *)b)[i]; }
 DEV float ld_f16(const void *b, long long i) {
@@ -66,12 +74,12 @@ DEV unsigned bf16_rne(float f) {
   return (f != f) ? ((u >> 16) | 0x40u) : r;
 }
 // round to the narrower type (nearest even) and widen again
-DEV float rt_f16(float x) { return (float)(_Float16)x; }
+DEV float rt_f16(float x) { return (float)(_Float16)f32_value(x); }
 DEV float rt_bf16(float x) { return as_f32(bf16_rne(x) << 16); }
 DEV float rt_f32(float x) { return x; }
 DEV void st_f32(void *o, long long i, float x) { ((float *)o)[i] = x; }
 DEV void st_f16(void *o, long long i, float x) {
-  ((unsigned short *)o)[i] = __builtin_bit_cast(unsigned short, (_Float16)x);
+  ((unsigned short *)o)[i] = __builtin_bit_cast(unsigned short, (_Float16)f32_value(x));
 }
 DEV void st_bf16(void *o, long long i, float x) { ((unsigned short *)o)[i] = (unsigned short)bf16_rne(x); }
 
@@ -131,8 +139,8 @@ template <int V> DEV void stv_f16(void *o, long long i, const float (&v)[V]) {
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
       f16x2 h;
-      h.x = (_Float16)v[8 * q + 2 * d];
-      h.y = (_Float16)v[8 * q + 2 * d + 1];
+      h.x = (_Float16)f32_value(v[8 * q + 2 * d]);
+      h.y = (_Float16)f32_value(v[8 * q + 2 * d + 1]);
       w[d] = __builtin_bit_cast(unsigned, h);
     }
     __builtin_nontemporal_store(w, p + q);
@@ -244,8 +252,8 @@ DEV u32x4 pk_f16(const float (&v)[8]) {
 #pragma unroll
   for (int d = 0; d < 4; ++d) {
     f16x2 h;
-    h.x = (_Float16)v[2 * d];
-    h.y = (_Float16)v[2 * d + 1];
+    h.x = (_Float16)f32_value(v[2 * d]);
+    h.y = (_Float16)f32_value(v[2 * d + 1]);
     w[d] = __builtin_bit_cast(unsigned, h);
   }
   return w;

@@ -126,8 +126,9 @@ def test_mean_is_the_row_sum_divided_by_the_extent_on_every_reduce_kernel(H, row
     sum is exact whatever the order, so the result must equal the oracle's bit for bit; on
     uniform values it is held to one unit in the last place of the f16 result.  (The reference's
     graph converts N to f16, which holds it exactly up to 2048 and overflows to infinity from
-    65520 on; the longer rows take N as a float32 extent.)"""
-    text = RC.MEAN_ROWBIAS if n <= 2048 else RC.MEAN_ROWBIAS.replace("const arg1.1 f16", "const arg1.1")
+    65520 on, and keeps the sums in an f16 tensor, where a row of a million terms overflows as
+    well; the longer rows take N as a float32 extent and divide the float32 sum.)"""
+    text = RC.MEAN_ROWBIAS if n <= 2048 else RC.MEAN_ROWBIAS.replace("const arg1.1 f16", "const arg1.1").replace("  cast f16\n", "")
     rng = np.random.default_rng(rows + n)
     a = rng.integers(-4, 5, (rows,)).astype(np.float16)
     b = rng.integers(-4, 5, (rows, n)).astype(np.float16)
