@@ -23,6 +23,7 @@
 // anything else takes the element kernel below.  v_mfma_f32_32x32x16 with the
 // operands swapped, so that a lane holds four consecutive n of one m for the
 // epilogue.
+#include <mutex>
 #include <type_traits>
 
 #include "kernels.h"
@@ -281,6 +282,105 @@ LaunchStatus launch_layout_mfma(const uint16_t *a, const uint16_t *b, const void
   return after_launch();
 }
 
+// ---- large products with a transposed operand: transpose it, then the direct-to-LDS kernel ----
+//
+// The direct-to-LDS kernel (matmul_dma_kernel.h) wants A as rows along K and B as rows along N.
+// An operand stored the other way round is first brought into that form by an HBM-bound tiled
+// transpose into scratch memory of the stream (a read and a write of the operand: 45-55 us for
+// 8192 x 8192 16-bit elements against 770 us of multiplication), which then runs as it does for
+// the plain layout: 6-7 % behind it, against 40-60 % behind on the register-staged kernel above.
+// 64 x 64 tiles of 16-bit elements through LDS, 128-bit loads and stores on both sides.
+constexpr int kTrTile = 64, kTrPitch = 72;   // pitch in elements: rows of the LDS tile stay 16-byte aligned
+__global__ __launch_bounds__(256) void transpose_u16_tile64(const uint16_t *__restrict__ src, uint16_t *__restrict__ dst,
+                                                            int rows, int cols) {
+  __shared__ __align__(16) uint16_t tile[kTrTile * kTrPitch];   // [column of src][row of src]
+  const int tiles_c = cols / kTrTile;
+  const int tr = blockIdx.x / tiles_c, tc = blockIdx.x - tr * tiles_c;
+  const int t = threadIdx.x, chunk = t & 7, line = t >> 3;    // a lane moves two 16-byte chunks
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int r = line + 32 * h;
+    const u32x4 v = *reinterpret_cast<const u32x4 *>(src + (int64_t)(tr * kTrTile + r) * cols + tc * kTrTile + chunk * 8);
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      tile[(chunk * 8 + 2 * d) * kTrPitch + r] = (uint16_t)(v[d] & 0xffffu);
+      tile[(chunk * 8 + 2 * d + 1) * kTrPitch + r] = (uint16_t)(v[d] >> 16);
+    }
+  }
+  __syncthreads();
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int c = line + 32 * h;
+    const u32x4 v = *reinterpret_cast<const u32x4 *>(tile + c * kTrPitch + chunk * 8);
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(dst + (int64_t)(tc * kTrTile + c) * rows + tr * kTrTile + chunk * 8));
+  }
+}
+
+// dst[c][r] = src[r][c] for a rows x cols matrix of 16-bit elements (both multiples of 64)
+void launch_transpose_u16(const uint16_t *src, uint16_t *dst, int64_t rows, int64_t cols, hipStream_t stream) {
+  const int64_t tiles = (rows / kTrTile) * (cols / kTrTile);
+  AFIR_LAUNCH("transpose_u16_tile64", transpose_u16_tile64, dim3((unsigned)tiles), dim3(256), 0, stream, src, dst, (int)rows,
+              (int)cols);
+}
+
+// Scratch memory of the stream's order (hipMallocAsync): the device's default pool, told once
+// to keep what is freed instead of returning it to the system at the next synchronisation.
+void *stream_scratch(size_t bytes, hipStream_t stream) {
+  static std::once_flag keep[64];
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  std::call_once(keep[device], [device] {
+    hipMemPool_t pool = nullptr;
+    uint64_t threshold = UINT64_MAX;
+    if (hipDeviceGetDefaultMemPool(&pool, device) != hipSuccess ||
+        hipMemPoolSetAttribute(pool, hipMemPoolAttrReleaseThreshold, &threshold) != hipSuccess)
+      (void)hipGetLastError();
+  });
+  void *p = nullptr;
+  if (hipMallocAsync(&p, bytes, stream) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  return p;
+}
+
+// The route above, when the shape is one the direct-to-LDS kernel takes and the stream can
+// allocate; false: not taken, nothing was launched.
+template <bool F16IO>
+bool launch_transposed_then_dma(const uint16_t *a, const uint16_t *b, const void *bias, void *out, int64_t m, int64_t k,
+                                int64_t n, bool ta, bool tb, float alpha, bool relu, hipStream_t stream, LaunchStatus *status) {
+  // (the same choice as the plain layout makes: products of fewer 256 x 256 tiles than half the
+  // compute units keep to smaller tiles)
+  if (!matmul_dma_supported(m, k, n) || (m / 256) * (n / 256) < (int64_t)device_cus() / 2) return false;
+  if (!aligned16(a) || !aligned16(b) || !aligned16(out) || (reinterpret_cast<uintptr_t>(bias) & (F16IO ? 15u : 7u))) return false;
+  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return false;   // no allocations inside a graph capture: the register-staged kernel
+  }
+  uint16_t *at = nullptr, *bt = nullptr;
+  if (ta && !(at = static_cast<uint16_t *>(stream_scratch((size_t)m * k * 2, stream)))) return false;
+  if (tb && !(bt = static_cast<uint16_t *>(stream_scratch((size_t)k * n * 2, stream)))) {
+    if (at) (void)hipFreeAsync(at, stream);
+    return false;
+  }
+  if (ta) launch_transpose_u16(a, at, k, m, stream);   // stored [K, M] -> [M, K]
+  if (tb) launch_transpose_u16(b, bt, n, k, stream);   // stored [N, K] -> [K, N]
+  const uint16_t *pa = ta ? at : a, *pb = tb ? bt : b;
+  if constexpr (F16IO)
+    *status = launch_matmul_dma_f16(pa, pb, static_cast<const float *>(bias), static_cast<float *>(out), (int)m, (int)k,
+                                    (int)n, alpha, relu, 0, stream);
+  else
+    *status = launch_matmul_dma(pa, pb, static_cast<const uint16_t *>(bias), static_cast<uint16_t *>(out), (int)m, (int)k,
+                                (int)n, alpha, relu, 0, stream);
+  if (at) (void)hipFreeAsync(at, stream);
+  if (bt) (void)hipFreeAsync(bt, stream);
+  return true;
+}
+
 template <bool F16IO>
 LaunchStatus launch_layouts_io(const uint16_t *a, const uint16_t *b, const void *bias, void *out, int64_t batch,
                                int64_t m, int64_t k, int64_t n, bool ta, bool tb, float alpha, bool relu,
@@ -300,6 +400,10 @@ LaunchStatus launch_layouts_io(const uint16_t *a, const uint16_t *b, const void 
   const bool rows16 = a_run % 8 == 0 && b_run % 8 == 0 && n % 8 == 0 && k >= 1 &&
                       (batch == 1 || ((m * k) % 8 == 0 && (k * n) % 8 == 0 && (m * n) % 8 == 0));
   const int64_t tiles = ((m + kLT - 1) / kLT) * ((n + kLT - 1) / kLT);
+  if (batch == 1 && !block_dim && (ta || tb)) {
+    LaunchStatus status = ok_status();
+    if (launch_transposed_then_dma<F16IO>(a, b, bias, out, m, k, n, ta, tb, alpha, relu, stream, &status)) return status;
+  }
   if (al && rows16 && m * n >= 64 * 64 && tiles <= 0x7fffffff) {
     const int bi = (int)batch, mi = (int)m, ki = (int)k, ni = (int)n;
     if (ta && tb) return launch_layout_mfma<true, true, F16IO>(a, b, bias, out, bi, mi, ki, ni, alpha, relu, block_dim, stream);

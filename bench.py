@@ -64,7 +64,10 @@ MEASURED_TRAFFIC = {
 # north_star targets, read on roofline.frac (algorithmic work / event-timed launch duration / published peak)
 TARGETS = {"c1": 0.70, "c2": 0.70, "c3": 0.70, "c4": 0.70, "c5": 0.60}
 CEILINGS = ["ceil_copy", "ceil_copy_phased", "ceil_read", "ceil_write", "ceil_tilecopy64"]
-ALL_WORKLOADS = ["c1", "c2", "c3", "c4", "c5", "g1", "g2", "g3", "g4", "i1", "i2"] + CEILINGS
+# m_ta / m_tb: c5's product with A (B) stored transposed, as region programs
+# (linalg.matmul_transpose_a / _b of the reference's matmul recogniser)
+LAYOUTS = ["m_ta", "m_tb"]
+ALL_WORKLOADS = ["c1", "c2", "c3", "c4", "c5", "g1", "g2", "g3", "g4", "i1", "i2"] + LAYOUTS + CEILINGS
 
 # Region programs of the two generic-kernel workloads (grammar:
 # ascend-mlir_amd/csrc/target/region_program.h)
@@ -440,6 +443,43 @@ def make_workload(key, torch, H, O, C):
             ev["vendor_gemm_constant_operands_tflops"] = round(rate(lambda i: torch.matmul(ones, ones), n=20, warm=3), 1)
             return ev
         w.power_evidence = power_evidence
+    elif key in LAYOUTS:
+        # c5's operands, one of them stored transposed; the product is c5's, so its golden is too
+        ta = key == "m_ta"
+        a, b, bias = O.gen_c5()
+        flags = " ta" if ta else " tb"
+        w.title = (f"{key} matmul-add-leakyrelu bf16 8192x8192x8192 with {'A stored as [K, M]' if ta else 'B stored as [N, K]'} "
+                   f"(linalg.matmul_transpose_{'a' if ta else 'b'}), as a region program")
+        w.dtype, w.bound, w.no_cpu = "bf16", "mfma", True
+        w.work = lambda: O.algorithmic_flops_c5(8192, 8192, 8192)
+        w.nsets = 2
+        text = ("afir-hip-region 1\narg in bf16 2\narg in bf16 2\narg in bf16 1\narg out bf16 2\nsegment 2\n"
+                f" size arg3.0 arg3.1\n outoff 0\n matmul arg0 arg1{flags}\n push arg2 d1\n add\n leaky 0.01\n store\nend\n")
+        region = H.Region(text)
+        da, db, dbias = _dev_bf16(torch, a), _dev_bf16(torch, b), _dev_bf16(torch, bias)
+        if ta:
+            da = da.t().contiguous()
+        else:
+            db = db.t().contiguous()
+        sets = []
+        for i in range(w.nsets):
+            ia, ib = (da, db) if i == 0 else (da.clone(), db.clone())
+            sets.append((ia, ib, dbias, torch.empty((8192, 8192), dtype=torch.bfloat16, device="cuda")))
+        w.sets = sets
+        w.region = region
+        tiling = H.pack_tiling(8192, 8192, 8192, 8192, 8192, 8192, 8192)
+        w.launches = [region.prepare([s[0].data_ptr(), s[1].data_ptr(), s[2].data_ptr(), s[3].data_ptr()], tiling) for s in sets]
+
+        def parity():
+            rows = np.arange(0, 8192, 61)[:128]
+            want = O.golden_c5_rows(a, b, bias, rows, 0.01)
+            got = sets[0][3][torch.from_numpy(rows).cuda()].view(torch.int16).cpu().numpy().view(np.uint16)
+            r = O.compare_outputs([(got, "bf16")], [(want, "bf16")], 1e-5, 1e-2)
+            nonfinite = O.nonfinite_mismatches(got, want, "bf16")
+            return {"bar": "<=1e-2 rel (atol 1e-5), 128 sampled rows x 8192 cols; no NaN / inf the golden lacks",
+                    "passed": bool(r["passed"]) and nonfinite == 0, "mismatches": int(r["mismatches"]) + nonfinite,
+                    "nonfinite_mismatches": nonfinite, "kernel": H.last_launch()["kernel"]}
+        w.parity = parity
     elif key in ("g1", "g2", "g3", "g4", "i1", "i2"):
         # Region programs (any fused chain) next to the hand-tuned kernels:
         # g1 / i1 = the c1 chain kept off its fast path, g2 / i2 = the
@@ -687,12 +727,12 @@ def main():
     def steps_for(key):
         if args.steps is not None:
             return args.steps
-        return 50 if key == "c5" else 300
+        return 50 if key == "c5" or key in LAYOUTS else 300
 
     def warm_for(key):
         if args.warmup is not None:
             return args.warmup
-        return 5 if key == "c5" else 30
+        return 5 if key == "c5" or key in LAYOUTS else 30
 
     order = [args.workload] + ([k for k in ALL_WORKLOADS if k != args.workload] if args.all else [])
     results = []
@@ -763,6 +803,11 @@ def main():
         line["targets_read_on"] = "roofline.frac (HIP events on the launch stream), not value (wall clock)"
         line["other_fracs"] = {k: e["roofline"]["frac"] for k, e in by_key.items()
                                if k not in TARGETS and k not in CEILINGS}
+        if "c5" in by_key:   # the transposed layouts against the plain one
+            for k in LAYOUTS:
+                if k in by_key:
+                    line["other_fracs"][k + "_vs_c5"] = round(by_key[k]["roofline"]["achieved"] /
+                                                              by_key["c5"]["roofline"]["achieved"], 4)
         ceil = {k: by_key[k]["roofline"]["achieved"] for k in CEILINGS
                 if k in by_key}
         if ceil:

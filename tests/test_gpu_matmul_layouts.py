@@ -103,6 +103,25 @@ def test_transposed_operands_integer_known_answer_exact(H, ty, flags, m, k, n):
 
 
 @pytest.mark.parametrize("ty", ["bf16", "f16"])
+@pytest.mark.parametrize("flags", [" ta", " tb", " ta tb"])
+def test_large_transposed_products_take_the_direct_to_lds_kernel(H, ty, flags):
+    """Whole 256 x 256 tiles, at least half as many as the chip has compute units: the transposed
+    operand is transposed into scratch memory of the stream and the product runs on the kernel of
+    the plain layout.  Small integers: exact, whatever the order of summation."""
+    m, k, n = 3072, 512, 3072
+    rng = np.random.default_rng(5)
+    a, b, bias = _operands(rng, ty, 0, m, k, n, "ta" in flags, "tb" in flags, True)
+    text = _program(2, ty, flags, True)
+    want = RO.evaluate(text, [a, b, bias], out_shape=(m, n))
+    got = _run(H, text, [a, b, bias], ty, (m, n))
+    assert H.last_launch()["kernel"].startswith("matmul_bias_leakyrelu_dma"), H.last_launch()
+    assert got.tobytes() == want.tobytes()
+    # twice in a row on the same stream: the scratch memory of the first call is free again
+    got = _run(H, text, [a, b, bias], ty, (m, n))
+    assert got.tobytes() == want.tobytes()
+
+
+@pytest.mark.parametrize("ty", ["bf16", "f16"])
 @pytest.mark.parametrize("flags", ["", " ta", " tb"])
 @pytest.mark.parametrize("batch,m,k,n", [(3, 128, 64, 128), (5, 136, 72, 40), (2, 77, 33, 19), (1, 64, 64, 64),
                                          (16, 256, 128, 256)])
