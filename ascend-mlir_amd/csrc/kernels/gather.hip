@@ -241,18 +241,24 @@ __global__ __launch_bounds__(kGroupedThreads) void gather_scale_shift_f16_groupe
 #ifndef AFIR_GATHER_PHASE_BASE_NS
 #define AFIR_GATHER_PHASE_BASE_NS 300
 #endif
+// Workgroups of kPhasedThreads lanes where eight of them fit a compute unit beside their scale /
+// shift chunks in LDS; rows of 8192 halves park 32 KiB per workgroup, and then four workgroups of
+// kPhasedWideThreads lanes keep the same 2048 lanes per CU resident (8192 x 8192 rows gathered:
+// 44.8 us against 49.0 on the grouped kernel; 1024-half rows are 1.5 % slower this way).
 constexpr int kPhasedThreads = AFIR_GATHER_PHASED_THREADS;
+constexpr int kPhasedWideThreads = 512;
 constexpr int kPhasedPasses = 2;
 constexpr int kPhasedLanesPerCU = 2048;
 
-__global__ __launch_bounds__(kPhasedThreads, 8) void gather_scale_shift_f16_phased(
+template <int kWg>
+__global__ __launch_bounds__(kWg, kPhasedLanesPerCU / kWg) void gather_scale_shift_f16_phased(
     const uint16_t *__restrict__ table, const int32_t *__restrict__ idx,
     const uint16_t *__restrict__ scale, const uint16_t *__restrict__ shift,
     uint16_t *__restrict__ out, int32_t *__restrict__ error_flag, uint32_t rows, int lanes_log2,
     int hold_ticks) {
   const long long t_start = wall_clock64();
   const int lanes = 1 << lanes_log2;
-  const int rows_per_pass = kPhasedThreads >> lanes_log2;
+  const int rows_per_pass = kWg >> lanes_log2;
   const int local_row = threadIdx.x >> lanes_log2;
   const int col0 = threadIdx.x & (lanes - 1);
   const int dim = lanes * kGroups * 8;
@@ -274,7 +280,7 @@ __global__ __launch_bounds__(kPhasedThreads, 8) void gather_scale_shift_f16_phas
 #pragma unroll
     for (int u = 0; u < kGroups; ++u) v[p][u] = row[u * lanes];
   }
-  for (int c = threadIdx.x; c < nchunks; c += kPhasedThreads) {
+  for (int c = threadIdx.x; c < nchunks; c += kWg) {
     params[c] = *reinterpret_cast<const u32x4 *>(scale + (int64_t)c * 8);
     params[nchunks + c] = *reinterpret_cast<const u32x4 *>(shift + (int64_t)c * 8);
   }
@@ -361,24 +367,37 @@ LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx
   // Whole blocks of rows go to the phased kernel, which wants every lane of a launch resident at
   // once: a gather of up to twice that goes out as two launches (kPhaseMaxLaunches).  Rows left
   // over, and larger gathers: below.
-  const int64_t phased_rows_per_block = (int64_t)(kPhasedThreads >> (lanes_log2 < 8 ? lanes_log2 : 8)) * kPhasedPasses;
-  const int64_t phased_blocks = nidx / phased_rows_per_block;
-  // blocks per launch: what is resident at once.  Rows of 8192 halves park 32 KiB of scale / shift
-  // per workgroup in LDS, and then five workgroups fit a compute unit, not the eight that put
-  // 64 MiB in flight: such launches measured 4-11 % behind the grouped kernel and take it.
-  const size_t lds = (size_t)2 * (kGroups << lanes_log2) * 16;   // scale and shift, 16-byte chunks
-  int64_t capacity = 0;
-  if (AFIR_GATHER_PHASED && vec && lanes_log2 <= 8 && (1 << lanes_log2) <= kPhasedThreads) {
-    static int fit[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};   // per row length, asked once (0: not yet)
-    if (fit[lanes_log2] == 0) {
-      const int n = resident_blocks_per_cu(gather_scale_shift_f16_phased, kPhasedThreads, lds);
-      fit[lanes_log2] = n > 0 ? n : -1;
+  // blocks per launch: what is resident at once, asked of the runtime with the launch's LDS (scale
+  // and shift, 16-byte chunks).  With fewer resident lanes than 2048 per CU (five workgroups of 256
+  // lanes on rows of 8192 halves) such launches measured 4-11 % behind the grouped kernel.
+  const size_t lds = (size_t)2 * (kGroups << lanes_log2) * 16;
+  int phased_threads = 0;
+  if (AFIR_GATHER_PHASED && vec && lanes_log2 <= 8) {
+    static int threads_for[9] = {0, 0, 0, 0, 0, 0, 0, 0, 0};   // per row length, asked once (0: not yet, -1: none)
+    if (threads_for[lanes_log2] == 0) {
+      threads_for[lanes_log2] = -1;
+      if ((1 << lanes_log2) <= kPhasedThreads &&
+          resident_blocks_per_cu(gather_scale_shift_f16_phased<kPhasedThreads>, kPhasedThreads, lds) >= kPhasedLanesPerCU / kPhasedThreads)
+        threads_for[lanes_log2] = kPhasedThreads;
+      else if (kPhasedWideThreads > kPhasedThreads &&
+               resident_blocks_per_cu(gather_scale_shift_f16_phased<kPhasedWideThreads>, kPhasedWideThreads, lds) >=
+                   kPhasedLanesPerCU / kPhasedWideThreads)
+        threads_for[lanes_log2] = kPhasedWideThreads;
     }
-    const int wanted = kPhasedLanesPerCU / kPhasedThreads;
-    capacity = fit[lanes_log2] >= wanted ? (int64_t)device_cus() * wanted : 0;
+    if (threads_for[lanes_log2] > 0) phased_threads = threads_for[lanes_log2];
   }
+  const int64_t phased_rows_per_block = phased_threads ? (int64_t)(phased_threads >> lanes_log2) * kPhasedPasses : 1;
+  const int64_t phased_blocks = phased_threads ? nidx / phased_rows_per_block : 0;
+  const int64_t capacity = phased_threads ? (int64_t)device_cus() * (kPhasedLanesPerCU / phased_threads) : 0;
+  // (a launch whose last wave of workgroups leaves many compute units idle gains nothing: 640
+  // workgroups of 512 lanes on 256 CUs measured 5 % behind the grouped kernel)
+  const auto fills_the_chip = [&](int64_t blocks) {
+    const int64_t cus = device_cus(), waves = (blocks + cus - 1) / cus;
+    return blocks <= cus || blocks * 10 >= waves * cus * 9;
+  };
   if (AFIR_GATHER_PHASED && vec && ((int64_t)kGroups << lanes_log2) == chunks64 && !block_dim && capacity > 0 &&
-      phased_blocks > 0 && phased_blocks <= kPhaseMaxLaunches * capacity && phased_enabled()) {
+      phased_blocks > 0 && phased_blocks <= kPhaseMaxLaunches * capacity && phased_enabled() &&
+      fills_the_chip((phased_blocks + (phased_blocks + capacity - 1) / capacity - 1) / ((phased_blocks + capacity - 1) / capacity))) {
     const int base_ns = env_int("AFIR_GATHER_PHASE_BASE_NS", AFIR_GATHER_PHASE_BASE_NS, 0, 100000);
     const int gbs = env_int("AFIR_GATHER_PHASE_GBS", AFIR_GATHER_PHASE_GBS, 100, 100000);
     const int64_t launches = (phased_blocks + capacity - 1) / capacity;
@@ -387,9 +406,14 @@ LaunchStatus launch_gather_scale_shift(const uint16_t *table, const int32_t *idx
       const int64_t nblocks = phased_blocks - b0 < take ? phased_blocks - b0 : take;
       const int64_t row0 = b0 * phased_rows_per_block;
       const int hold_ticks = phase_hold_ticks(nblocks * phased_rows_per_block * dim * 2, base_ns, gbs);
-      AFIR_LAUNCH("gather_scale_shift_f16_phased", gather_scale_shift_f16_phased, dim3((unsigned)nblocks), dim3(kPhasedThreads), lds, stream,
-                         table, idx + row0, scale, shift, out + row0 * dim, error_flag, (uint32_t)rows, lanes_log2,
-                         hold_ticks);
+      if (phased_threads == kPhasedThreads)
+        AFIR_LAUNCH("gather_scale_shift_f16_phased", gather_scale_shift_f16_phased<kPhasedThreads>, dim3((unsigned)nblocks),
+                    dim3(kPhasedThreads), lds, stream, table, idx + row0, scale, shift, out + row0 * dim, error_flag,
+                    (uint32_t)rows, lanes_log2, hold_ticks);
+      else
+        AFIR_LAUNCH("gather_scale_shift_f16_phased", gather_scale_shift_f16_phased<kPhasedWideThreads>, dim3((unsigned)nblocks),
+                    dim3(kPhasedWideThreads), lds, stream, table, idx + row0, scale, shift, out + row0 * dim, error_flag,
+                    (uint32_t)rows, lanes_log2, hold_ticks);
     }
     const int64_t done = phased_blocks * phased_rows_per_block;
     if (done == nidx) return after_launch();

@@ -303,12 +303,19 @@ def test_c4_phased_route_bit_exact(H, dim, nidx, monkeypatch):
 
 
 def test_c4_phased_launch_needs_every_lane_resident(H, monkeypatch):
-    """Rows of 8192 halves park 32 KiB of scale / shift per workgroup in LDS: five workgroups fit a
-    compute unit, not the eight that put a whole launch in flight at once, so such gathers keep to
-    the grouped kernel (asked of the runtime: the occupancy of the kernel with that much LDS).
-    Rows of 4096 halves fit.  The hold constants are read from the environment at every launch: a
-    hold far too short or too long changes the timing only."""
+    """Rows of 8192 halves park 32 KiB of scale / shift per workgroup in LDS: five workgroups of
+    256 lanes fit a compute unit, not the eight that put a whole launch in flight at once (asked
+    of the runtime: the occupancy of the kernel with that much LDS), so such gathers run as four
+    workgroups of 512 lanes per compute unit; a row count whose workgroups would leave many
+    compute units idle at the end keeps to the grouped kernel.  Rows of 4096 halves fit as 256
+    lanes.  The hold constants are read from the environment at every launch: a hold far too
+    short or too long changes the timing only."""
     table, idx, scale, shift = O.gen_c4(5000, 8192, 4096)
+    out = H.gather_scale_shift(dev(table), dev(idx), dev(scale), dev(shift)).cpu().numpy()
+    assert out.tobytes() == O.golden_c4(table, idx, scale, shift).tobytes()
+    note = H.last_launch()
+    assert note["kernel"] == "gather_scale_shift_f16_phased" and note["workgroups"] == 1024 and note["threads"] == 512
+    table, idx, scale, shift = O.gen_c4(5000, 8192, 2560)      # 640 workgroups: 2.5 per compute unit
     out = H.gather_scale_shift(dev(table), dev(idx), dev(scale), dev(shift)).cpu().numpy()
     assert out.tobytes() == O.golden_c4(table, idx, scale, shift).tobytes()
     assert H.last_launch()["kernel"] == "gather_scale_shift_f16_grouped"
