@@ -286,33 +286,52 @@ LaunchStatus launch_layout_mfma(const uint16_t *a, const uint16_t *b, const void
 //
 // The direct-to-LDS kernel (matmul_dma_kernel.h) wants A as rows along K and B as rows along N.
 // An operand stored the other way round is first brought into that form by an HBM-bound tiled
-// transpose into scratch memory of the stream (a read and a write of the operand: 45-55 us for
-// 8192 x 8192 16-bit elements against 770 us of multiplication), which then runs as it does for
-// the plain layout: 6-7 % behind it, against 40-60 % behind on the register-staged kernel above.
-// 64 x 64 tiles of 16-bit elements through LDS, 128-bit loads and stores on both sides.
-constexpr int kTrTile = 64, kTrPitch = 72;   // pitch in elements: rows of the LDS tile stay 16-byte aligned
+// transpose into scratch memory of the stream (a read and a write of the operand: 52 us for
+// 8192 x 8192 16-bit elements against 750-770 us of multiplication), which then runs as it does
+// for the plain layout: 6-7 % behind it, against 40-60 % behind on the register-staged kernel above.
+// 64 x 64 tiles of 16-bit elements through LDS, 128-bit loads and stores on both sides.  In LDS an
+// element takes a 32-bit word and a tile row 65 words: the eight words a lane writes per chunk and
+// the eight it reads per output chunk then fall into different banks for every lane of a wave
+// (neither this nor 16-bit writes into rows of 72 halves is what bounds the kernel: both measured
+// the same; the order of the tiles below and the non-temporal loads are what moved it).
+constexpr int kTrTile = 64, kTrPitch = 65;   // pitch in 32-bit words
+constexpr int kTrBand = 32;
 __global__ __launch_bounds__(256) void transpose_u16_tile64(const uint16_t *__restrict__ src, uint16_t *__restrict__ dst,
                                                             int rows, int cols) {
-  __shared__ __align__(16) uint16_t tile[kTrTile * kTrPitch];   // [column of src][row of src]
-  const int tiles_c = cols / kTrTile;
-  const int tr = blockIdx.x / tiles_c, tc = blockIdx.x - tr * tiles_c;
+  __shared__ uint32_t tile[kTrTile * kTrPitch];   // [column of src][row of src]
+  // Tiles in bands of kTrBand tile rows, a band walked down its rows first: the workgroups that
+  // run together then cover runs of 4 KiB along the rows of dst and of 8 KiB along those of src.
+  // Walked along the rows of src alone (runs of 16 KiB read, 128 bytes written at a pitch that
+  // is a large power of two) the same kernel took 70 us for 8192 x 8192 instead of 52; bands of
+  // 8 / 16 / 24 / 48 / 64 / all rows: 57 / 56 / 53.4 / 56 / 58 / 59.
+  const int tiles_c = cols / kTrTile, tiles_r = rows / kTrTile;
+  const int per_band = kTrBand * tiles_c;
+  const int band = blockIdx.x / per_band, within = blockIdx.x - band * per_band;
+  const int height = tiles_r - band * kTrBand < kTrBand ? tiles_r - band * kTrBand : kTrBand;
+  const int tc = within / height, tr = band * kTrBand + (within - tc * height);
   const int t = threadIdx.x, chunk = t & 7, line = t >> 3;    // a lane moves two 16-byte chunks
+  u32x4 v[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+    v[h] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + (int64_t)(tr * kTrTile + line + 32 * h) * cols + tc * kTrTile + chunk * 8));
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
     const int r = line + 32 * h;
-    const u32x4 v = *reinterpret_cast<const u32x4 *>(src + (int64_t)(tr * kTrTile + r) * cols + tc * kTrTile + chunk * 8);
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
-      tile[(chunk * 8 + 2 * d) * kTrPitch + r] = (uint16_t)(v[d] & 0xffffu);
-      tile[(chunk * 8 + 2 * d + 1) * kTrPitch + r] = (uint16_t)(v[d] >> 16);
+      tile[(chunk * 8 + 2 * d) * kTrPitch + r] = v[h][d] & 0xffffu;
+      tile[(chunk * 8 + 2 * d + 1) * kTrPitch + r] = v[h][d] >> 16;
     }
   }
   __syncthreads();
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
     const int c = line + 32 * h;
-    const u32x4 v = *reinterpret_cast<const u32x4 *>(tile + c * kTrPitch + chunk * 8);
-    __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(dst + (int64_t)(tc * kTrTile + c) * rows + tr * kTrTile + chunk * 8));
+    const uint32_t *w = tile + c * kTrPitch + chunk * 8;
+    u32x4 o;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) o[d] = w[2 * d] | (w[2 * d + 1] << 16);
+    __builtin_nontemporal_store(o, reinterpret_cast<u32x4 *>(dst + (int64_t)(tc * kTrTile + c) * rows + tr * kTrTile + chunk * 8));
   }
 }
 
