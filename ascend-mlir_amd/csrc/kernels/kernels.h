@@ -62,6 +62,10 @@ LaunchStatus launch_matmul_dma(const uint16_t *a, const uint16_t *b, const uint1
 LaunchStatus launch_matmul_dma_f16(const uint16_t *a, const uint16_t *b, const float *bias,
                                    float *out, int m, int k, int n, float alpha, bool relu,
                                    uint32_t block_dim, hipStream_t stream);
+// `batch` products of one shape, A [batch, m, k], B [batch, k, n], out [batch, m, n] densely
+// packed, the bias [n] shared (null: none); shapes as matmul_dma_supported(m, k, n) says
+LaunchStatus launch_matmul_dma_batched(const uint16_t *a, const uint16_t *b, const void *bias, void *out, bool f16io,
+                                       int batch, int m, int k, int n, float alpha, bool relu, hipStream_t stream);
 
 inline LaunchStatus ok_status() { return LaunchStatus{0u, ""}; }
 inline LaunchStatus invalid(const char *msg) { return LaunchStatus{1u, msg}; }

@@ -93,4 +93,13 @@ LaunchStatus launch_matmul_dma_f16(const uint16_t *a, const uint16_t *b, const f
                                           block_dim, stream);
 }
 
+LaunchStatus launch_matmul_dma_batched(const uint16_t *a, const uint16_t *b, const void *bias, void *out, bool f16io,
+                                       int batch, int m, int k, int n, float alpha, bool relu, hipStream_t stream) {
+  if (f16io)
+    return dma::launch<true, dma::FullFeed, true>("matmul_bias_leakyrelu_dma_f16_batched", a, b, bias, out, m, k, n, alpha,
+                                                  relu, 0, stream, batch);
+  return dma::launch<false, dma::FullFeed, true>("matmul_bias_leakyrelu_dma_batched", a, b, bias, out, m, k, n, alpha, relu,
+                                                 0, stream, batch);
+}
+
 }  // namespace afir

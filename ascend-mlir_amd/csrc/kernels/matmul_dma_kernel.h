@@ -232,11 +232,14 @@ struct Drain { static constexpr bool value = false; };
 // examples/matmul-add-leakyrelu/step0_input.mlir:10-15): the same rings and
 // reads (both element types are 16 bits wide), the f16 MFMA, and an epilogue
 // that stores the float32 value unrounded.
-template <bool F16IO, typename Feed>
+// Batched = true: `M` rows are a stack of independent products of tiles_m_batch tile rows each
+// (A [batch, m, K] and out [batch, m, N] densely packed are one tall matrix each; only B changes
+// with the batch: b_batch_stride elements further on per batch).  The bias is shared.
+template <bool F16IO, typename Feed, bool Batched = false>
 __global__ __launch_bounds__(kWaves * 64) void matmul_bias_leakyrelu_dma(
     const uint16_t *__restrict__ A, const uint16_t *__restrict__ B,
     const void *__restrict__ bias_v, void *__restrict__ out_v, int M, int K, int N,
-    float alpha, int relu, int tiles_m, int tiles_n) {
+    float alpha, int relu, int tiles_m, int tiles_n, int tiles_m_batch, int64_t b_batch_stride) {
   extern __shared__ __align__(1024) unsigned char smem[];
   // (address space 3 pointers are 32 bits wide: the value is the LDS byte address)
   const uint32_t lds_base =
@@ -317,7 +320,9 @@ __global__ __launch_bounds__(kWaves * 64) void matmul_bias_leakyrelu_dma(
     const int kfirst = first_stage(tile_m, tile_n);
     ua = reinterpret_cast<const char *>(A) +
          ((int64_t)(m0 + wave * (kAReg * 8)) * K + (int64_t)kfirst * kBK) * 2;
-    ub = reinterpret_cast<const char *>(B) +
+    const uint16_t *b_of_batch = B;
+    if constexpr (Batched) b_of_batch += (int64_t)(tile_m / tiles_m_batch) * b_batch_stride;
+    ub = reinterpret_cast<const char *>(b_of_batch) +
          ((int64_t)(wave * (kBReg * 2) + kfirst * kBK) * N + n0) * 2;
     ka_next = kfirst >> 1;
     kb_next = kfirst;
@@ -337,7 +342,9 @@ __global__ __launch_bounds__(kWaves * 64) void matmul_bias_leakyrelu_dma(
     const int k = (first_stage(tile_m, tile_n) + ahead) % KW;
     const int pw = wave - kFeedWaves;
     ua = reinterpret_cast<const char *>(A) + ((int64_t)(tile_m * kBM + pw * 64) * K + (int64_t)k * kBK) * 2;
-    ub = reinterpret_cast<const char *>(B) + ((int64_t)(k * kBK + pw * 16) * N + tile_n * kBN) * 2;
+    const uint16_t *b_of_batch = B;
+    if constexpr (Batched) b_of_batch += (int64_t)(tile_m / tiles_m_batch) * b_batch_stride;
+    ub = reinterpret_cast<const char *>(b_of_batch) + ((int64_t)(k * kBK + pw * 16) * N + tile_n * kBN) * 2;
     ka_next = k >> 1;
     pf_tile = p;
     pf_left = KT - ahead;
@@ -759,22 +766,25 @@ inline bool supported(int64_t m, int64_t k, int64_t n) {
 #define AFIR_MM_GRID device_cus()
 #endif
 
-template <bool F16IO, typename Feed>
+// batch > 1 (with Batched): `m` is the extent of one product; A and out hold `batch` of them one
+// after the other, B likewise (k * n elements apart)
+template <bool F16IO, typename Feed, bool Batched = false>
 LaunchStatus launch(const char *name, const uint16_t *a, const uint16_t *b, const void *bias, void *out, int m,
-                    int k, int n, float alpha, bool relu, uint32_t block_dim, hipStream_t stream) {
-  auto kernel = matmul_bias_leakyrelu_dma<F16IO, Feed>;
+                    int k, int n, float alpha, bool relu, uint32_t block_dim, hipStream_t stream, int batch = 1) {
+  auto kernel = matmul_bias_leakyrelu_dma<F16IO, Feed, Batched>;
   static hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize,
                                                kLdsBytes);
   if (attr != hipSuccess) return LaunchStatus{2u, hipGetErrorString(attr)};
-  const int tiles_m = m / kBM, tiles_n = n / kBN;
+  if (!Batched && batch != 1) return LaunchStatus{1u, "matmul: this instance takes one product"};
+  const int tiles_m_batch = m / kBM, tiles_m = tiles_m_batch * batch, tiles_n = n / kBN;
   // One workgroup fills a CU's LDS, so the grid is persistent: one workgroup
   // per CU, each walking its share of the tiles.
   int64_t blocks = (int64_t)tiles_m * tiles_n;
   if (blocks > AFIR_MM_GRID) blocks = AFIR_MM_GRID;
   if (block_dim) blocks = block_dim;
   AFIR_LAUNCH(name, kernel, dim3((unsigned)blocks), dim3(kWaves * 64), kLdsBytes, stream, a, b,
-              bias, out, m, k, n, alpha, relu ? 1 : 0, tiles_m, tiles_n);
+              bias, out, m * batch, k, n, alpha, relu ? 1 : 0, tiles_m, tiles_n, tiles_m_batch, (int64_t)k * n);
   return after_launch();
 }
 

@@ -309,6 +309,8 @@ __global__ __launch_bounds__(256) void transpose_u16_tile64(const uint16_t *__re
   const int band = blockIdx.x / per_band, within = blockIdx.x - band * per_band;
   const int height = tiles_r - band * kTrBand < kTrBand ? tiles_r - band * kTrBand : kTrBand;
   const int tc = within / height, tr = band * kTrBand + (within - tc * height);
+  src += (int64_t)blockIdx.y * rows * cols;   // one matrix per blockIdx.y, densely packed
+  dst += (int64_t)blockIdx.y * rows * cols;
   const int t = threadIdx.x, chunk = t & 7, line = t >> 3;    // a lane moves two 16-byte chunks
   u32x4 v[2];
 #pragma unroll
@@ -335,11 +337,11 @@ __global__ __launch_bounds__(256) void transpose_u16_tile64(const uint16_t *__re
   }
 }
 
-// dst[c][r] = src[r][c] for a rows x cols matrix of 16-bit elements (both multiples of 64)
-void launch_transpose_u16(const uint16_t *src, uint16_t *dst, int64_t rows, int64_t cols, hipStream_t stream) {
+// dst[z][c][r] = src[z][r][c] for `batch` rows x cols matrices of 16-bit elements (both multiples of 64)
+void launch_transpose_u16(const uint16_t *src, uint16_t *dst, int64_t batch, int64_t rows, int64_t cols, hipStream_t stream) {
   const int64_t tiles = (rows / kTrTile) * (cols / kTrTile);
-  AFIR_LAUNCH("transpose_u16_tile64", transpose_u16_tile64, dim3((unsigned)tiles), dim3(256), 0, stream, src, dst, (int)rows,
-              (int)cols);
+  AFIR_LAUNCH("transpose_u16_tile64", transpose_u16_tile64, dim3((unsigned)tiles, (unsigned)batch), dim3(256), 0, stream, src, dst,
+              (int)rows, (int)cols);
 }
 
 // Scratch memory of the stream's order (hipMallocAsync): the device's default pool, told once
@@ -366,30 +368,44 @@ void *stream_scratch(size_t bytes, hipStream_t stream) {
   return p;
 }
 
-// The route above, when the shape is one the direct-to-LDS kernel takes and the stream can
-// allocate; false: not taken, nothing was launched.
+// The direct-to-LDS kernel for transposed and / or batched operands, when the shape is one it
+// takes and, with a transposed operand, the stream can allocate; false: not taken, nothing was
+// launched.  A batch is a stack of products to that kernel (its tiles are dealt out over the whole
+// stack), so sixteen products of 1024^3 fill the chip like one of 4096 x 1024 x 4096.
 template <bool F16IO>
-bool launch_transposed_then_dma(const uint16_t *a, const uint16_t *b, const void *bias, void *out, int64_t m, int64_t k,
-                                int64_t n, bool ta, bool tb, float alpha, bool relu, hipStream_t stream, LaunchStatus *status) {
+bool launch_on_dma(const uint16_t *a, const uint16_t *b, const void *bias, void *out, int64_t batch, int64_t m, int64_t k,
+                   int64_t n, bool ta, bool tb, float alpha, bool relu, hipStream_t stream, LaunchStatus *status) {
   // (the same choice as the plain layout makes: products of fewer 256 x 256 tiles than half the
   // compute units keep to smaller tiles)
-  if (!matmul_dma_supported(m, k, n) || (m / 256) * (n / 256) < (int64_t)device_cus() / 2) return false;
+  if (!matmul_dma_supported(m, k, n) || batch * (m / 256) * (n / 256) < (int64_t)device_cus() / 2) return false;
+  if (!env_int("AFIR_HIP_MATMUL_LAYOUTS_DIRECT", 1, 0, 1)) return false;   // 0: the register-staged kernel (to compare)
+  // Two transposes cost 2 x 2 bytes x (m k + k n) of HBM traffic against 2 m k n flops: with both
+  // operands transposed and products under 2048 x 2048 outputs they cost as much as the product
+  // itself (16 x 1024^3: 445 TFLOP/s this way, 503 on the register-staged kernel; 8 x 2048^3: 794
+  // against 685; 32 x 1024 x 4096 x 1024: 683 against 616).  One transposed operand measured
+  // level or ahead on every shape tried (64 x 512^3: 376-392 against 339-382).
+  if (ta && tb && !((m >= 2048 && n >= 2048) || k >= 4096)) return false;
+  if (batch * m > 0x7fffffff || batch * (m / 256) * (n / 256) > 0x7fffffff) return false;
   if (!aligned16(a) || !aligned16(b) || !aligned16(out) || (reinterpret_cast<uintptr_t>(bias) & (F16IO ? 15u : 7u))) return false;
-  hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
-    (void)hipGetLastError();
-    return false;   // no allocations inside a graph capture: the register-staged kernel
-  }
   uint16_t *at = nullptr, *bt = nullptr;
-  if (ta && !(at = static_cast<uint16_t *>(stream_scratch((size_t)m * k * 2, stream)))) return false;
-  if (tb && !(bt = static_cast<uint16_t *>(stream_scratch((size_t)k * n * 2, stream)))) {
-    if (at) (void)hipFreeAsync(at, stream);
-    return false;
+  if (ta || tb) {
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+      (void)hipGetLastError();
+      return false;   // no allocations inside a graph capture: the register-staged kernel
+    }
+    if (ta && !(at = static_cast<uint16_t *>(stream_scratch((size_t)batch * m * k * 2, stream)))) return false;
+    if (tb && !(bt = static_cast<uint16_t *>(stream_scratch((size_t)batch * k * n * 2, stream)))) {
+      if (at) (void)hipFreeAsync(at, stream);
+      return false;
+    }
+    if (ta) launch_transpose_u16(a, at, batch, k, m, stream);   // stored [K, M] -> [M, K]
+    if (tb) launch_transpose_u16(b, bt, batch, n, k, stream);   // stored [N, K] -> [K, N]
   }
-  if (ta) launch_transpose_u16(a, at, k, m, stream);   // stored [K, M] -> [M, K]
-  if (tb) launch_transpose_u16(b, bt, n, k, stream);   // stored [N, K] -> [K, N]
   const uint16_t *pa = ta ? at : a, *pb = tb ? bt : b;
-  if constexpr (F16IO)
+  if (batch > 1)
+    *status = launch_matmul_dma_batched(pa, pb, bias, out, F16IO, (int)batch, (int)m, (int)k, (int)n, alpha, relu, stream);
+  else if constexpr (F16IO)
     *status = launch_matmul_dma_f16(pa, pb, static_cast<const float *>(bias), static_cast<float *>(out), (int)m, (int)k,
                                     (int)n, alpha, relu, 0, stream);
   else
@@ -419,9 +435,9 @@ LaunchStatus launch_layouts_io(const uint16_t *a, const uint16_t *b, const void 
   const bool rows16 = a_run % 8 == 0 && b_run % 8 == 0 && n % 8 == 0 && k >= 1 &&
                       (batch == 1 || ((m * k) % 8 == 0 && (k * n) % 8 == 0 && (m * n) % 8 == 0));
   const int64_t tiles = ((m + kLT - 1) / kLT) * ((n + kLT - 1) / kLT);
-  if (batch == 1 && !block_dim && (ta || tb)) {
+  if (!block_dim && (batch > 1 || ta || tb)) {
     LaunchStatus status = ok_status();
-    if (launch_transposed_then_dma<F16IO>(a, b, bias, out, m, k, n, ta, tb, alpha, relu, stream, &status)) return status;
+    if (launch_on_dma<F16IO>(a, b, bias, out, batch, m, k, n, ta, tb, alpha, relu, stream, &status)) return status;
   }
   if (al && rows16 && m * n >= 64 * 64 && tiles <= 0x7fffffff) {
     const int bi = (int)batch, mi = (int)m, ki = (int)k, ni = (int)n;

@@ -66,7 +66,8 @@ TARGETS = {"c1": 0.70, "c2": 0.70, "c3": 0.70, "c4": 0.70, "c5": 0.60}
 CEILINGS = ["ceil_copy", "ceil_copy_phased", "ceil_read", "ceil_write", "ceil_tilecopy64"]
 # m_ta / m_tb: c5's product with A (B) stored transposed, as region programs
 # (linalg.matmul_transpose_a / _b of the reference's matmul recogniser)
-LAYOUTS = ["m_ta", "m_tb"]
+# m_b16: sixteen independent products of 1024^3 in one launch (linalg.batch_matmul), same epilogue
+LAYOUTS = ["m_ta", "m_tb", "m_b16"]
 ALL_WORKLOADS = ["c1", "c2", "c3", "c4", "c5", "g1", "g2", "g3", "g4", "i1", "i2"] + LAYOUTS + CEILINGS
 
 # Region programs of the two generic-kernel workloads (grammar:
@@ -443,6 +444,42 @@ def make_workload(key, torch, H, O, C):
             ev["vendor_gemm_constant_operands_tflops"] = round(rate(lambda i: torch.matmul(ones, ones), n=20, warm=3), 1)
             return ev
         w.power_evidence = power_evidence
+    elif key == "m_b16":
+        nb, dim = 16, 1024
+        w.title = ("m_b16 batch of 16 matmul-add-leakyrelu bf16 1024x1024x1024 (linalg.batch_matmul + the same epilogue), "
+                   "as a region program")
+        w.dtype, w.bound, w.no_cpu = "bf16", "mfma", True
+        w.work = lambda: nb * O.algorithmic_flops_c5(dim, dim, dim)
+        w.nsets = 8
+        text = ("afir-hip-region 1\narg in bf16 3\narg in bf16 3\narg in bf16 1\narg out bf16 3\nsegment 3\n"
+                " size arg3.0 arg3.1 arg3.2\n outoff 0\n matmul arg0 arg1\n push arg2 d2\n add\n leaky 0.01\n store\nend\n")
+        region = H.Region(text)
+        parts = [O.gen_c5(dim, dim, dim, seed=O.SEED + z) for z in range(nb)]
+        a = np.stack([p[0] for p in parts])
+        b = np.stack([p[1] for p in parts])
+        bias = parts[0][2]
+        da, db, dbias = _dev_bf16(torch, a), _dev_bf16(torch, b), _dev_bf16(torch, bias)
+        sets = []
+        for i in range(w.nsets):
+            ia, ib = (da, db) if i == 0 else (da.clone(), db.clone())
+            sets.append((ia, ib, dbias, torch.empty((nb, dim, dim), dtype=torch.bfloat16, device="cuda")))
+        w.sets = sets
+        w.region = region
+        tiling = H.pack_tiling(nb, dim, dim, nb, dim, dim, dim, nb, dim, dim)
+        w.launches = [region.prepare([s[0].data_ptr(), s[1].data_ptr(), s[2].data_ptr(), s[3].data_ptr()], tiling) for s in sets]
+
+        def parity():
+            rows = np.arange(0, dim, 17)[:32]
+            bad = nonfinite = 0
+            for z in (0, 7, 15):
+                want = O.golden_c5_rows(a[z], b[z], bias, rows, 0.01)
+                got = sets[0][3][z][torch.from_numpy(rows).cuda()].view(torch.int16).cpu().numpy().view(np.uint16)
+                bad += int(O.compare_outputs([(got, "bf16")], [(want, "bf16")], 1e-5, 1e-2)["mismatches"])
+                nonfinite += O.nonfinite_mismatches(got, want, "bf16")
+            return {"bar": "<=1e-2 rel (atol 1e-5), 32 sampled rows x 1024 cols of batches 0, 7, 15; no NaN / inf the golden lacks",
+                    "passed": bad == 0 and nonfinite == 0, "mismatches": bad + nonfinite,
+                    "nonfinite_mismatches": nonfinite, "kernel": H.last_launch()["kernel"]}
+        w.parity = parity
     elif key in LAYOUTS:
         # c5's operands, one of them stored transposed; the product is c5's, so its golden is too
         ta = key == "m_ta"
@@ -727,12 +764,12 @@ def main():
     def steps_for(key):
         if args.steps is not None:
             return args.steps
-        return 50 if key == "c5" or key in LAYOUTS else 300
+        return 50 if key in ("c5", "m_ta", "m_tb") else 300
 
     def warm_for(key):
         if args.warmup is not None:
             return args.warmup
-        return 5 if key == "c5" or key in LAYOUTS else 30
+        return 5 if key in ("c5", "m_ta", "m_tb") else 30
 
     order = [args.workload] + ([k for k in ALL_WORKLOADS if k != args.workload] if args.all else [])
     results = []
@@ -804,7 +841,7 @@ def main():
         line["other_fracs"] = {k: e["roofline"]["frac"] for k, e in by_key.items()
                                if k not in TARGETS and k not in CEILINGS}
         if "c5" in by_key:   # the transposed layouts against the plain one
-            for k in LAYOUTS:
+            for k in ("m_ta", "m_tb"):
                 if k in by_key:
                     line["other_fracs"][k + "_vs_c5"] = round(by_key[k]["roofline"]["achieved"] /
                                                               by_key["c5"]["roofline"]["achieved"], 4)

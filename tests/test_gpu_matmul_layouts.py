@@ -122,6 +122,26 @@ def test_large_transposed_products_take_the_direct_to_lds_kernel(H, ty, flags):
 
 
 @pytest.mark.parametrize("ty", ["bf16", "f16"])
+@pytest.mark.parametrize("flags,batch,m,k,n", [(f, b, m, k, n) for f in ("", " ta", " tb")
+                                               for (b, m, k, n) in ((16, 256, 512, 2048), (6, 512, 256, 3072))] +
+                         [(" ta tb", 16, 512, 4096, 1024)])
+def test_large_batched_products_take_the_direct_to_lds_kernel(H, ty, flags, batch, m, k, n):
+    """A batch of products of whole 256 x 256 tiles, at least half as many tiles in all as the chip
+    has compute units, is one stack of tiles to the direct-to-LDS kernel: one tile row per product
+    (16 x 256 rows), and two per product with the kernel's groups of four tile rows straddling
+    products (6 x 512 rows).  Transposed operands are transposed per product first (both of them
+    only where that pays: long K or large outputs).  Small integers: exact."""
+    rng = np.random.default_rng(batch * 100 + m)
+    a, b, bias = _operands(rng, ty, batch, m, k, n, "ta" in flags, "tb" in flags, True)
+    text = _program(3, ty, flags, True)
+    want = RO.evaluate(text, [a, b, bias], out_shape=(batch, m, n))
+    got = _run(H, text, [a, b, bias], ty, (batch, m, n))
+    assert H.last_launch()["kernel"].startswith("matmul_bias_leakyrelu_dma"), H.last_launch()
+    assert "batched" in H.last_launch()["kernel"]
+    assert got.tobytes() == want.tobytes()
+
+
+@pytest.mark.parametrize("ty", ["bf16", "f16"])
 @pytest.mark.parametrize("flags", ["", " ta", " tb"])
 @pytest.mark.parametrize("batch,m,k,n", [(3, 128, 64, 128), (5, 136, 72, 40), (2, 77, 33, 19), (1, 64, 64, 64),
                                          (16, 256, 128, 256)])
