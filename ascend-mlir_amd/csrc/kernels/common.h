@@ -35,12 +35,13 @@ inline int device_cus() {
 // real-time counter the device reads with wall_clock64() (100 MHz on MI355X), counted from the
 // start of each workgroup, base_ns + read_bytes / (gb_per_s GB/s).  AFIR_HIP_PHASED=0 in the
 // environment switches the phased kernels off (the launchers then take their other kernels).
-// (The rates are those of the whole chip: a partition of it, with its share of the CUs, keeps
-// to the other kernels.)
+// (The default rates are those of the whole chip: a partition of it, with its share of the CUs,
+// keeps to the other kernels unless AFIR_HIP_PHASED=1 says that the deployer has set the rates
+// for it, the AFIR_*_PHASE_GBS variables below.)
 inline bool phased_enabled() {
-  if (device_cus() != kNumCU) return false;
   const char *env = getenv("AFIR_HIP_PHASED");
-  return !(env && env[0] == '0');
+  if (env && env[0] == '0') return false;
+  return device_cus() == kNumCU || (env && env[0] == '1');
 }
 // A tuning constant that a deployer can change without rebuilding: the value of the environment
 // variable `name` when it is set to an integer within [lo, hi], else `fallback` (the compile-time
