@@ -569,11 +569,13 @@ def test_integer_unaligned_views_and_tails(H):
             assert got.tobytes() == want.tobytes(), (ty, m, n)
 
 
-def _random_region(rng):
+def _random_region(rng, extras=False):
     """A random program with its inputs and output shape: iteration rank 1..3; operands
     read whole, broadcast along rows or columns, transposed or gathered; one element type
     or a mix; elementwise or a row sum; extents drawn from the classes the kernels tell
-    apart (short rows, whole vectors with partly empty passes, whole passes, ragged)."""
+    apart (short rows, whole vectors with partly empty passes, whole passes, ragged).
+    extras: also roundings to a narrower type in the chain and, in elementwise programs,
+    extent constants (the runtime extent of an argument as a value)."""
     rank = int(rng.integers(1, 4))
     reduce = rank >= 2 and rng.random() < 0.35
     types = [["f32"], ["f16"], ["bf16"], ["f16", "f32"]][int(rng.integers(0, 4))]
@@ -607,10 +609,14 @@ def _random_region(rng):
     depth = 1
     allowed2 = ["add", "sub", "mul", "max", "min"] + ([] if reduce else ["div"])
     allowed1 = ["relu", "neg"] + ([] if reduce else ["leaky 0.25"])
+    if extras:
+        allowed1 += ["cast f16", "cast bf16"]
     for _ in range(int(rng.integers(1, 7))):
         k = int(rng.integers(0, 4))
         if depth < 3 and k == 0 and len(args) < 6:
-            if rng.random() < 0.2:
+            if extras and not reduce and rng.random() < 0.3:
+                ops.append(f"const arg0.{int(rng.integers(0, rank))} {['f32', 'f16', 'bf16'][int(rng.integers(0, 3))]}")
+            elif rng.random() < 0.2:
                 ops.append("const 2")
             else:
                 text, shape = kinds[int(rng.integers(0, len(kinds)))]
@@ -644,10 +650,11 @@ def _random_region(rng):
     return text, inputs, out_shape, out_ty
 
 
-@pytest.mark.parametrize("seed", range(60))
+@pytest.mark.parametrize("seed", range(60 + 40))
 def test_random_programs_over_the_shape_classes(H, seed):
+    """(seeds from 60 on: with roundings in the chain and extent constants)"""
     rng = np.random.default_rng(777 + seed)
-    text, inputs, out_shape, out_ty = _random_region(rng)
+    text, inputs, out_shape, out_ty = _random_region(rng, extras=seed >= 60)
     want = RO.evaluate(text, inputs)
     got = run(H, text, inputs, out_shape)
     if out_ty == "bf16":
