@@ -121,6 +121,11 @@ struct FullFeed {
 #ifndef AFIR_MM_NT_STORE
 #define AFIR_MM_NT_STORE 1
 #endif
+// the order of a phase's sixteen MFMAs: 0 walks the four m tiles under one n tile (consecutive
+// instructions share the B fragment), 1 the four n tiles under one m tile (they share the A one)
+#ifndef AFIR_MM_MFMA_A_OUTER
+#define AFIR_MM_MFMA_A_OUTER 0
+#endif
 #ifndef AFIR_MM_DMA_STRIDE
 #define AFIR_MM_DMA_STRIDE 2
 #endif
@@ -497,7 +502,8 @@ __global__ __launch_bounds__(kWaves * 64) void matmul_bias_leakyrelu_dma(
     auto pin = [] { __builtin_amdgcn_sched_barrier(0); };
     // MFMA number X of a phase: n tile X / 4, m tile FIRST + X % 4
     auto mfma = [&](auto first_tag, auto x_tag, const u32x4 (&a)[4], const u32x2 (&b)[kTN][2]) {
-      constexpr int FIRST = decltype(first_tag)::value, X = decltype(x_tag)::value, j = X / 4, i = X % 4;
+      constexpr int FIRST = decltype(first_tag)::value, X = decltype(x_tag)::value;
+      constexpr int j = AFIR_MM_MFMA_A_OUTER ? X % 4 : X / 4, i = AFIR_MM_MFMA_A_OUTER ? X / 4 : X % 4;
       const u32x4 bw = {b[j][0].x, b[j][0].y, b[j][1].x, b[j][1].y};
       if constexpr (F16IO)
         acc[FIRST + i][j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
