@@ -47,6 +47,7 @@ KERNEL_SOURCES = [
     ("kernels/region.hip", STRICT),
     ("target/region_program.cpp", []),
     ("target/hip_emitter.cpp", []),
+    ("target/hiprtc_compile.cpp", []),
     ("capi/afir_hip_kernels.cpp", []),
 ]
 
@@ -80,7 +81,8 @@ def build_kernels():
 
 RUNTIME_SOURCES = ["runtime/support.cpp", "runtime/artifact.cpp", "runtime/session.cpp",
                    "runtime/hip_runner.cpp", "capi/afirt_runtime.cpp",
-                   "target/region_program.cpp", "target/mlir_translate.cpp", "target/hip_emitter.cpp"]
+                   "target/region_program.cpp", "target/mlir_translate.cpp", "target/hip_emitter.cpp",
+                   "target/hiprtc_compile.cpp"]
 HOST = ["-std=c++17", "-O2", "-fPIC", "-Wall", "-Wno-unused-result",
         "-D__HIP_PLATFORM_AMD__", "-I", "/opt/rocm/include", "-I", os.path.join(ROOT, "include")]
 CXX = os.environ.get("CXX", "g++")

@@ -25,6 +25,7 @@
 #include "family_programs.h"
 #include "../kernels/region_launch.h"
 #include "../target/hip_emitter.h"
+#include "../target/hiprtc_compile.h"
 #include "../target/region_program.h"
 
 namespace {
@@ -719,6 +720,20 @@ uint32_t afir_hip_region_attach_code_object(uint64_t handle, const void *image, 
   r->compiled = std::move(c);
   g_last_error.clear();
   return AFIR_HIP_OK;
+}
+
+uint32_t afir_hip_region_compile(uint64_t handle, void *image_out, size_t capacity, size_t *image_len) {
+  auto r = find_region(handle);
+  if (!r) return fail(AFIR_HIP_E_UNKNOWN, "no region program with that handle");
+  std::string source;
+  std::string why = afir_target::emitHipSource(r->program, "region", &source);
+  if (!why.empty()) return fail(AFIR_HIP_E_INVALID, "no specialised kernel: " + why);
+  std::vector<char> image;
+  why = afir_target::compileWithHiprtc(source, &image);
+  if (!why.empty()) return fail(AFIR_HIP_E_INVALID, why);
+  if (image_len) *image_len = image.size();
+  if (image_out && capacity >= image.size()) std::memcpy(image_out, image.data(), image.size());
+  return afir_hip_region_attach_code_object(handle, image.data(), image.size());
 }
 
 const char *afir_hip_region_tiling_field(uint64_t handle, int index) {

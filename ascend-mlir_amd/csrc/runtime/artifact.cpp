@@ -31,6 +31,7 @@
 #include <sstream>
 
 #include "../target/hip_emitter.h"
+#include "../target/hiprtc_compile.h"
 #include "../target/mlir_translate.h"
 
 extern char **environ;
@@ -251,9 +252,23 @@ Expected<std::string> compileRegionCodeObject(const std::string &programText, co
       }
   }
   if (hipcc.empty() && access("/opt/rocm/bin/hipcc", X_OK) == 0) hipcc = "/opt/rocm/bin/hipcc";
-  if (hipcc.empty()) return Status::error("hipcc not found (set HIPCC); the source is kept at " + srcPath);
-  std::vector<std::string> argv = {hipcc, "--genco", "--offload-arch=gfx950", "-O3", "-nogpuinc", "-ffp-contract=off",
-                                   "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-o", objPath, srcPath};
+  // No hipcc on this host (or AFIR_HIP_COMPILER=hiprtc): the runtime-compilation library of the
+  // HIP runtime compiles the same source with the same options inside the process.
+  const char *which = std::getenv("AFIR_HIP_COMPILER");
+  const bool wantRtc = which && std::string(which) == "hiprtc", onlyHipcc = which && std::string(which) == "hipcc";
+  if (onlyHipcc && hipcc.empty()) return Status::error("hipcc not found (set HIPCC); the source is kept at " + srcPath);
+  if (wantRtc || (!onlyHipcc && (hipcc.empty() || access(hipcc.c_str(), X_OK) != 0))) {
+    std::vector<char> image;
+    if (std::string why = afir_target::compileWithHiprtc(source, &image); !why.empty())
+      return Status::error((wantRtc ? std::string() : "hipcc not found (set HIPCC), and ") + why +
+                           "; the source is kept at " + srcPath);
+    std::ofstream f(objPath, std::ios::trunc | std::ios::binary);
+    if (!f || !f.write(image.data(), (std::streamsize)image.size())) return Status::error("cannot write " + objPath);
+    return objName;
+  }
+  std::vector<std::string> argv = {hipcc, "--genco"};
+  for (const std::string &o : afir_target::regionCompileOptions()) argv.push_back(o);
+  argv.insert(argv.end(), {"-o", objPath, srcPath});
   std::vector<char *> cargv;
   for (std::string &a : argv) cargv.push_back(a.data());
   cargv.push_back(nullptr);

@@ -49,6 +49,7 @@ EXPORTED_SYMBOLS = [
     "afir_hip_region_route",
     "afir_hip_region_emit_source",
     "afir_hip_region_attach_code_object",
+    "afir_hip_region_compile",
     "afir_hip_region_prefer_code_object",
     "afir_hip_region_argument_bytes",
     "afir_hip_launch_region",
@@ -374,10 +375,24 @@ class Region:
         self.kernel = L.afir_hip_region_kernel(ctypes.c_uint64(self.handle)).decode()
         return self
 
-    def compile(self, cache_dir: str = None):
-        """Emit, compile with hipcc and attach; the code object is kept in
-        `cache_dir` (default: lib/region_cache beside the libraries) under the
-        hash of its source, so a program is compiled once."""
+    def compile(self, cache_dir: str = None, in_process: bool = None):
+        """Emit, compile and attach.  With hipcc (the default where it exists) the code
+        object is kept in `cache_dir` (default: lib/region_cache beside the libraries)
+        under the hash of its source, so a program is compiled once.  in_process=True, or
+        no hipcc on this host: compiled inside the process by the HIP runtime's own
+        compiler library (afir_hip_region_compile), nothing cached."""
+        import shutil
+        if in_process is None:
+            in_process = not (shutil.which("hipcc") or os.path.exists("/opt/rocm/bin/hipcc"))
+        if in_process:
+            L = load()
+            L.afir_hip_region_compile.restype = ctypes.c_uint32
+            L.afir_hip_region_compile.argtypes = [ctypes.c_uint64, ctypes.c_void_p, ctypes.c_size_t,
+                                                  ctypes.POINTER(ctypes.c_size_t)]
+            n = ctypes.c_size_t(0)
+            _check(L.afir_hip_region_compile(ctypes.c_uint64(self.handle), None, 0, ctypes.byref(n)))
+            self.kernel = L.afir_hip_region_kernel(ctypes.c_uint64(self.handle)).decode()
+            return self
         source = self.emit_source()
         self.attach_code_object(compile_region_source(source, cache_dir))
         return self

@@ -249,6 +249,17 @@ const char *afir_hip_region_route(uint64_t handle, const void *tiling, size_t ti
  * that kernel.  Matmul programs have no source form (AFIR_HIP_E_INVALID). */
 uint32_t afir_hip_region_emit_source(uint64_t handle, char *buffer, size_t capacity, size_t *length);
 uint32_t afir_hip_region_attach_code_object(uint64_t handle, const void *image, size_t image_len);
+/* Emit, compile and attach in one call, inside the process: the source of
+ * afir_hip_region_emit_source is compiled for gfx950 by the runtime-compilation
+ * library of the HIP runtime (libhiprtc, opened on first use), with the options
+ * hipcc is given for the same source, so a host that has the runtime but no
+ * hipcc still gets the program's own kernels instead of the interpreter.  Host
+ * only (no device is touched; the code object is loaded at the first launch).
+ * The code object is also copied to image_out when it fits `capacity` (a caller
+ * that keeps artifacts), and its size stored in *image_len; both may be null.
+ * The reference compiles its generated sources with an external compiler
+ * (lib/Runtime/Compilation/KernelCompiler.cpp); this is that step without one. */
+uint32_t afir_hip_region_compile(uint64_t handle, void *image_out, size_t capacity, size_t *image_len);
 /* prefer != 0: the attached code object runs even when the program is one of
  * the hand-tuned families (which otherwise keep their kernel).  Used for
  * artifacts compiled with explicit emit options and by tile searches, where

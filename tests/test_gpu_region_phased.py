@@ -144,3 +144,24 @@ def test_shapes_outside_the_phased_form_keep_to_the_other_kernels(H, cache, monk
         assert "phased" not in H.last_launch()["kernel"], shape
         assert out.tobytes() == ((a + b) * b).tobytes(), shape
     r.close()
+
+
+@pytest.mark.parametrize("name", ["c1", "c3", "c4", "relu_colgather_add", "split_relu_brc_add_mul", "cast_chain_f16",
+                                  "reduce_rowbias", "mean_rowbias"])
+def test_regions_compiled_inside_the_process_give_the_same_bits(H, cache, monkeypatch, name):
+    """afir_hip_region_compile (the HIP runtime's compiler library, no hipcc) against the code
+    object hipcc builds from the same source: the same output, bit for bit, and (for the
+    elementwise cases) the oracle's."""
+    monkeypatch.setenv("AFIR_HIP_REGION_GENERIC", "1")
+    exact = name in RC.EXACT_CASES
+    text, inputs, want = (RC.EXACT_CASES if exact else RC.REDUCE_CASES)[name]()
+    outs = []
+    for in_process in (True, False):
+        r = H.Region(text).compile(cache_dir=cache, in_process=in_process)
+        assert r.kernel == "fused_region_compiled"
+        dev = [_dev(x, r.arg_types[i]) for i, x in enumerate(inputs)]
+        outs.append(_host(r(*dev, out_shape=want.shape), r.arg_types[-1]))
+        r.close()
+    assert outs[0].tobytes() == outs[1].tobytes()
+    if exact:
+        assert outs[0].tobytes() == want.tobytes()

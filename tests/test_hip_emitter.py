@@ -187,9 +187,47 @@ def test_artifact_without_compiler_keeps_the_program(tmp_path):
     assert "program:\nafir-hip-region 1" in (art / "k.hipk").read_text()
     sub = tmp_path / "b"
     sub.mkdir()
-    manifest, art = _compile(sub, env={"HIPCC": "/nonexistent/hipcc"})
+    manifest, art = _compile(sub, env={"HIPCC": "/nonexistent/hipcc", "AFIR_HIP_COMPILER": "hipcc"})
     assert any(l.startswith("code_object_note=cannot start /nonexistent/hipcc") for l in manifest)
     assert (art / "k.hip").exists() and not (art / "k.hsaco").exists()
+
+
+def test_artifact_without_hipcc_is_compiled_inside_the_process(tmp_path):
+    """No hipcc on the host (or AFIR_HIP_COMPILER=hiprtc): the HIP runtime's own compiler library
+    builds the same source with the same options, and the artifact holds the same kernels."""
+    for i, env in enumerate(({"HIPCC": "/nonexistent/hipcc"}, {"AFIR_HIP_COMPILER": "hiprtc"})):
+        sub = tmp_path / str(i)
+        sub.mkdir()
+        manifest, art = _compile(sub, env=env)
+        assert "code_object_path=k.hsaco" in manifest, manifest
+        image = (art / "k.hsaco").read_bytes()
+        assert image[:4] == b"\x7fELF" and b"afir_region_s1_i64_g" in image and b"afir_region_program_hash" in image
+        assert subprocess.run([RS, "--artifact-root", str(art)], capture_output=True).returncode == 0
+
+
+def test_capi_compiles_a_region_inside_the_process(pkg):
+    """afir_hip_region_compile: emit + compile + attach without hipcc and without a device."""
+    from ascend_mlir_amd import hip_kernels as H
+    L = H.load()
+    r = H.Region(RC.RELU_COL_ADD)
+    assert r.kernel != "fused_region_compiled"
+    r.compile(in_process=True)
+    assert r.kernel == "fused_region_compiled"
+    u64, sz = ctypes.c_uint64, ctypes.c_size_t
+    L.afir_hip_region_compile.restype = ctypes.c_uint32
+    L.afir_hip_region_compile.argtypes = [u64, ctypes.c_void_p, sz, ctypes.POINTER(sz)]
+    n = sz(0)
+    assert L.afir_hip_region_compile(u64(r.handle), None, 0, ctypes.byref(n)) == 0 and n.value > 1000
+    buf = ctypes.create_string_buffer(n.value)
+    assert L.afir_hip_region_compile(u64(r.handle), buf, n.value, None) == 0
+    assert buf.raw[:4] == b"\x7fELF" and b"afir_region_s0_i32_a" in buf.raw
+    assert L.afir_hip_region_compile(u64(424242), None, 0, None) != 0 and b"no region program" in L.afir_hip_last_error()
+    r.close()
+    prog = subprocess.run([TR, "-mlir-to-hip", "-"], input=MC.MATMUL_BIAS_LEAKY_BF16, capture_output=True, text=True).stdout
+    m = H.Region(prog)
+    with pytest.raises(H.AfirHipError, match="no specialised kernel"):
+        m.compile(in_process=True)
+    m.close()
 
 
 def test_capi_emit_and_attach_without_gpu(pkg):
