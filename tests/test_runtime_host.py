@@ -28,7 +28,7 @@ def test_cpp_host_tests(tmp_path):
            os.path.join(PKG, "csrc", "runtime", "artifact.cpp"),
            os.path.join(PKG, "csrc", "runtime", "session.cpp"),
            os.path.join(PKG, "csrc", "target", "region_program.cpp"),
-           os.path.join(PKG, "csrc", "target", "hip_emitter.cpp"),
+           os.path.join(PKG, "csrc", "target", "hip_emitter.cpp"), os.path.join(PKG, "csrc", "target", "hiprtc_compile.cpp"),
            os.path.join(PKG, "csrc", "target", "mlir_translate.cpp")]
     subprocess.run(["g++", "-std=c++17", "-O1", "-Wall", "-I", os.path.join(PKG, "csrc", "runtime"),
                     "-I", os.path.join(ROOT, "include"), *src, "-ldl", "-o", str(exe)], check=True)
