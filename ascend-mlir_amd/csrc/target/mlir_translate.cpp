@@ -735,6 +735,8 @@ class Translator {
       parseElementwise(one());
     } else if (op == "linalg.transpose") {
       parseTranspose(one());
+    } else if (op == "linalg.reduce") {
+      parseReduce(one());
     } else if (op == "linalg.broadcast") {
       parseBroadcast(one());
     } else if (op == "tensor.collapse_shape" || op == "tensor.expand_shape") {
@@ -874,7 +876,10 @@ class Translator {
     static const struct { const char *n; OpCode c; int arity; } table[] = {
         {"add", OpCode::Add, 2}, {"sub", OpCode::Sub, 2}, {"mul", OpCode::Mul, 2}, {"div", OpCode::Div, 2},
         {"max", OpCode::Max, 2}, {"min", OpCode::Min, 2}, {"max_signed", OpCode::Max, 2},
-        {"min_signed", OpCode::Min, 2}, {"negf", OpCode::Neg, 1}, {"abs", OpCode::Neg, -1}};
+        {"min_signed", OpCode::Min, 2}, {"negf", OpCode::Neg, 1}, {"abs", OpCode::Neg, -1},
+        // arities below -1 name a form built from the chain's own operations:
+        // copy: x, square: x * x, reciprocal: 1 / x
+        {"copy", OpCode::Add, -2}, {"square", OpCode::Mul, -3}, {"reciprocal", OpCode::Div, -4}};
     for (const auto &e : table)
       if (name == e.n) {
         if (code) *code = e.c;
@@ -916,6 +921,9 @@ class Translator {
     tv->shape = outT->shape;
     if (arity == 2) tv->expr = makeBinary(code, v[0], v[1]);
     else if (arity == 1) tv->expr = makeUnary(code, v[0]);
+    else if (arity == -2) tv->expr = v[0];
+    else if (arity == -3) tv->expr = makeBinary(OpCode::Mul, v[0], v[0]);
+    else if (arity == -4) tv->expr = makeBinary(OpCode::Div, makeConst(1.f), v[0]);
     else tv->expr = makeBinary(OpCode::Max, v[0], makeUnary(OpCode::Neg, v[0]));   // |x| = max(x, -x), exactly
     defineTensor(result, tv);
   }
@@ -982,6 +990,62 @@ class Translator {
       tv->shape.push_back(in->shape[(size_t)perm[i]]);
     }
     tv->expr = substitute(in->expr, with);
+    defineTensor(result, tv);
+  }
+  // linalg.reduce ins(%a : t) outs(%init : t') dimensions = [last] (%x: f32, %acc: f32) { addf; yield }
+  // or the short form linalg.reduce { arith.addf } ins(...) outs(...) dimensions = [last]: the sum
+  // over the innermost dim into a zero-filled init, the one reduction this backend lowers (the
+  // reference lowers only sums: ComputeConversion.cpp:731-740)
+  void parseReduce(const std::string &result) {
+    bool sum = false;
+    if (r_.peek() == '{') {   // short form: the combiner's name in braces
+      r_.eat('{');
+      sum = r_.ident() == "arith.addf";
+      if (r_.peek() == '{') { r_.eat('{'); skipDict(); }
+      r_.expect('}');
+      if (!sum) r_.fail("linalg.reduce: only a sum (arith.addf) has a HIP lowering");
+    }
+    Operands ins = parseOperandGroup("ins"), outs = parseOperandGroup("outs");
+    if (ins.names.size() != 1 || outs.names.size() != 1) r_.fail("linalg.reduce takes one input and one init");
+    const std::vector<int64_t> dims = parseIntList("dimensions");
+    if (r_.peek() == '(') {   // the combiner region: (%in: f32, %acc: f32) { %s = arith.addf %in, %acc : f32  linalg.yield %s : f32 }
+      r_.eat('(');
+      std::vector<std::string> args;
+      do { args.push_back(r_.ssa()); r_.expect(':'); parseType(); } while (r_.eat(','));
+      r_.expect(')');
+      r_.expect('{');
+      if (args.size() != 2) r_.fail("linalg.reduce: the combiner takes two scalars");
+      const std::string value = r_.ssa();
+      r_.expect('=');
+      if (r_.ident() != "arith.addf") r_.fail("linalg.reduce: only a sum (arith.addf) has a HIP lowering");
+      const std::string x = r_.ssa();
+      r_.expect(',');
+      const std::string y = r_.ssa();
+      if (!((x == args[0] && y == args[1]) || (x == args[1] && y == args[0])))
+        r_.fail("linalg.reduce: the combiner must add its two arguments");
+      if (r_.eatWord("fastmath")) { r_.expect('<'); r_.skipBalanced(); r_.expect('>'); }
+      r_.expect(':');
+      parseType();
+      if (r_.ident() != "linalg.yield" || r_.ssa() != value) r_.fail("linalg.reduce: the combiner must yield its sum");
+      r_.expect(':');
+      parseType();
+      r_.expect('}');
+      sum = true;
+    }
+    if (!sum) r_.fail("linalg.reduce needs a combiner");
+    if (r_.eatArrow()) parseType();
+    TensorP in = elementwiseSource(ins.names[0], "linalg.reduce"), outT = tensorOf(outs.names[0]);
+    const size_t rank = in->shape.size();
+    if (rank < 2 || dims.size() != 1 || dims[0] != (int64_t)rank - 1 || outT->shape.size() != rank - 1)
+      r_.fail("linalg.reduce: only a reduction of the innermost dim of a tensor of rank 2 or 3 has a HIP lowering");
+    if (!afir_region::isFloat(in->elem)) r_.fail("linalg.reduce: only float tensors");
+    if (!(outT->filled && outT->fill == 0.f)) r_.fail("linalg.reduce needs a zero-filled init (linalg.fill 0)");
+    auto tv = std::make_shared<Tensor>();
+    tv->elem = outT->elem;
+    tv->shape = outT->shape;
+    tv->reduced = true;
+    tv->expr = in->expr;
+    tv->iterSizes = in->shape;
     defineTensor(result, tv);
   }
   // linalg.broadcast ins(%a : t) outs(%b : t) dimensions = [...]: the result dims that are added

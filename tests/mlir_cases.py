@@ -524,3 +524,32 @@ func.func @ew_sub(%a : tensor<?x?xf16>, %c : tensor<?x1x?xf16>, %init : tensor<?
   return %r : tensor<?x?x?xf16>
 }
 """
+
+
+# A row sum written with named ops only: linalg.square / broadcast / add / reciprocal / copy and
+# linalg.reduce with an addf combiner over the innermost dim (the op names of the reference's
+# --linalg-mark groups 1 and 2, lib/Dialect/AFIR/Transforms/LinalgMark.cpp:45-62):
+# y[i] = sum_j 1 / (x[i,j]^2 + b[j])
+NAMED_REDUCE_GRAPH = """
+func.func @sq_recip_rowsum(%x: tensor<?x?xf32>, %b: tensor<?xf32>) -> tensor<?xf32> {
+  %c0 = arith.constant 0 : index
+  %c1 = arith.constant 1 : index
+  %m = tensor.dim %x, %c0 : tensor<?x?xf32>
+  %n = tensor.dim %x, %c1 : tensor<?x?xf32>
+  %e = tensor.empty(%m, %n) : tensor<?x?xf32>
+  %sq = linalg.square ins(%x : tensor<?x?xf32>) outs(%e : tensor<?x?xf32>) -> tensor<?x?xf32>
+  %bb = linalg.broadcast ins(%b : tensor<?xf32>) outs(%e : tensor<?x?xf32>) dimensions = [0]
+  %s = linalg.add ins(%sq, %bb : tensor<?x?xf32>, tensor<?x?xf32>) outs(%e : tensor<?x?xf32>) -> tensor<?x?xf32>
+  %r = linalg.reciprocal ins(%s : tensor<?x?xf32>) outs(%e : tensor<?x?xf32>) -> tensor<?x?xf32>
+  %cp = linalg.copy ins(%r : tensor<?x?xf32>) outs(%e : tensor<?x?xf32>) -> tensor<?x?xf32>
+  %zero = arith.constant 0.0 : f32
+  %ie = tensor.empty(%m) : tensor<?xf32>
+  %init = linalg.fill ins(%zero : f32) outs(%ie : tensor<?xf32>) -> tensor<?xf32>
+  %red = linalg.reduce ins(%cp : tensor<?x?xf32>) outs(%init : tensor<?xf32>) dimensions = [1]
+    (%in: f32, %acc: f32) {
+      %0 = arith.addf %in, %acc : f32
+      linalg.yield %0 : f32
+    }
+  return %red : tensor<?xf32>
+}
+"""

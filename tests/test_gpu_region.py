@@ -181,6 +181,12 @@ def test_mixed_precision_and_named_op_graphs_from_mlir_run_on_every_route(H):
     p, q = rng.uniform(-2, 2, (7, 40)).astype(np.float16), rng.uniform(-2, 2, (5, 1, 40)).astype(np.float16)
     init = np.zeros((5, 7, 40), np.float16)
     assert run(H, text, [p, q, init], (5, 7, 40)).tobytes() == RO.evaluate(text, [p, q, init]).tobytes()
+    # linalg.reduce over named elementwise ops: a row sum, <= 1e-5 relative
+    text = subprocess.run([tr, "-mlir-to-hip", "-"], input=MC.NAMED_REDUCE_GRAPH, capture_output=True, text=True, check=True).stdout
+    x, bias = rng.uniform(1, 2, (37, 1000)).astype(np.float32), rng.uniform(0, 1, (1000,)).astype(np.float32)
+    want = (1.0 / (x.astype(np.float64) ** 2 + bias.astype(np.float64))).sum(axis=1)
+    got = run(H, text, [x, bias], (37,)).astype(np.float64)
+    assert np.all(np.abs(got - want) <= 1e-5 * np.abs(want))
 
 
 @pytest.mark.parametrize("n", [1, 3, 8, 16, 40, 64, 100, 256, 520])

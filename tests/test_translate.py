@@ -420,6 +420,29 @@ def test_linalg_elementwise_with_broadcast_maps():
     assert bad.returncode == 1 and "other than splats" in bad.stderr
 
 
+def test_named_reduce_and_unary_forms():
+    """linalg.reduce with an addf combiner (region form and the short { arith.addf } form) is the
+    row sum; linalg.square / reciprocal / copy are forms of mul / div / nothing."""
+    body = _body(MC.NAMED_REDUCE_GRAPH)
+    want_ops = ["const 1", "push arg0 d0 d1", "push arg0 d0 d1", "mul", "push arg1 d1", "add", "div", "reduce sum", "store", "end"]
+    assert body[body.index("outoff 0") + 1:] == want_ops
+    region_form = MC.NAMED_REDUCE_GRAPH
+    a, b = region_form.index("  %red = linalg.reduce"), region_form.index("  return")
+    short = (region_form[:a] + "  %red = linalg.reduce { arith.addf } ins(%cp : tensor<?x?xf32>) outs(%init : tensor<?xf32>) "
+             "dimensions = [1]\n" + region_form[b:])
+    assert _body(short) == body
+    rng = np.random.default_rng(13)
+    x, bias = rng.uniform(1, 2, (9, 300)).astype(np.float32), rng.uniform(0, 1, (300,)).astype(np.float32)
+    got = RO.evaluate(program_of(MC.NAMED_REDUCE_GRAPH), [x, bias])
+    ref = (1.0 / (x.astype(np.float64) ** 2 + bias.astype(np.float64))).sum(axis=1)
+    assert got.dtype == np.float32 and np.allclose(got, ref, rtol=1e-5, atol=0)
+    for frm, to, msg in (("arith.addf %in, %acc", "arith.mulf %in, %acc", "only a sum"),
+                         ("dimensions = [1]", "dimensions = [0]", "innermost dim"),
+                         ("arith.constant 0.0 : f32", "arith.constant 1.0 : f32", "zero-filled init")):
+        bad = subprocess.run([TR, "-mlir-to-hip", "-"], input=region_form.replace(frm, to), capture_output=True, text=True)
+        assert bad.returncode == 1 and msg in bad.stderr, (frm, bad.stderr)
+
+
 LINALG_ADD_BROADCAST = "/root/reference/test/Dialect/AFIR/Transforms/linalgAddBroadcast.mlir"
 
 
