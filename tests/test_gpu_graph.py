@@ -163,3 +163,58 @@ def test_phased_kernels_that_overlap_on_two_streams(H):
         assert torch.equal(got_g, want_g), rep
         assert torch.equal(got_t, want_t), rep
         assert torch.equal(got_e, want_e), rep
+
+
+def test_matmul_layouts_replay_from_a_captured_graph(H):
+    """A large product with a transposed operand allocates scratch memory of its stream when it is
+    launched eagerly; under a capture it may not, and keeps to the kernel that needs none.  A
+    batch of products needs no scratch on either route.  Small integers: both routes give the
+    same bits, and every replay must match the eager launches on the same inputs."""
+    m, k, n, nb = 3072, 512, 3072, 8
+    gen = torch.Generator(device="cuda").manual_seed(5)
+
+    def ints(shape):
+        return torch.randint(-3, 4, shape, generator=gen, device="cuda", dtype=torch.int32).to(torch.bfloat16)
+
+    def program(rank, flags):
+        size = " ".join(f"arg2.{d}" for d in range(rank))
+        return (RC.HEADER + f"arg in bf16 {rank}\narg in bf16 {rank}\narg out bf16 {rank}\nsegment {rank}\n size {size}\n"
+                f" outoff 0\n matmul arg0 arg1{flags}\n store\nend\n")
+    at, b = ints((k, m)), ints((k, n))                      # A stored [K, M]
+    ba, bb = ints((nb, 512, 256)), ints((nb, 256, 1024))    # 8 x 2 x 4 = 64 tiles: the register-staged kernel
+    c, bc = torch.empty((m, n), dtype=torch.bfloat16, device="cuda"), torch.empty((nb, 512, 1024), dtype=torch.bfloat16, device="cuda")
+    transposed, batched = H.Region(program(2, " ta")), H.Region(program(3, ""))
+
+    def launches():
+        return [transposed.prepare([at.data_ptr(), b.data_ptr(), c.data_ptr()], H.pack_tiling(k, m, k, n, m, n)),
+                batched.prepare([ba.data_ptr(), bb.data_ptr(), bc.data_ptr()],
+                                H.pack_tiling(nb, 512, 256, nb, 256, 1024, nb, 512, 1024))]
+
+    def eager():
+        names = []
+        for call in launches():
+            call()
+            names.append(H.last_launch()["kernel"])
+        torch.cuda.synchronize()
+        return c.clone(), bc.clone(), names
+    _, _, names = eager()
+    assert names[0].startswith("matmul_bias_leakyrelu_dma"), names     # eagerly: transposed into scratch, then the direct kernel
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for call in launches():
+            call()
+        captured = H.last_launch()["kernel"]
+    for replay in range(3):
+        for t in (at, b, ba, bb):
+            t.copy_(ints(tuple(t.shape)))
+        want_c, want_bc, _ = eager()
+        c.fill_(7)
+        bc.fill_(7)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(c, want_c) and torch.equal(bc, want_bc), replay
+    assert torch.equal(c, (at.float().t() @ b.float()).bfloat16())      # exact sums, one rounding to bf16
+    assert captured  # (whichever kernel the batch took: it allocates nothing)
+    transposed.close()
+    batched.close()
