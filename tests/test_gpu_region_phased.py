@@ -8,6 +8,7 @@ Reference semantics of the regions: lib/Conversion/LinalgToAscendC/ComputeConver
 import numpy as np
 import pytest
 
+from oracle import afir_oracle as O
 from oracle import region_oracle as RO
 from tests import region_cases as RC
 
@@ -165,3 +166,83 @@ def test_regions_compiled_inside_the_process_give_the_same_bits(H, cache, monkey
     assert outs[0].tobytes() == outs[1].tobytes()
     if exact:
         assert outs[0].tobytes() == want.tobytes()
+
+
+def _random_phased_program(rng):
+    """A random elementwise program of the form the phased kernels take: one or two operands
+    streamed with the output, row vectors, per-row values and constants, all of one element size,
+    roundings and extent constants among the operations; rank 2 or 3, 16-64 MiB of output."""
+    ty = ["f32", "f16", "bf16"][int(rng.integers(0, 3))]
+    esize = 4 if ty == "f32" else 2
+    rank = int(rng.integers(2, 4))
+    n = int(rng.choice([1024, 2048, 4096, 8192]))                 # row length: 8 * 2^k groups
+    rows = (int(rng.choice([16, 32, 48])) << 20) // (n * esize)   # 16 / 32 / 48 MiB of output
+    size = [rows, n] if rank == 2 else [4, rows // 4, n]
+    last = rank - 1
+    dims = " ".join(f"d{k}" for k in range(rank))
+    kinds = [(dims, tuple(size)), (f"d{last}", (n,)), (" ".join(f"d{k}" for k in range(last)), tuple(size[:-1]))]
+    args, shapes = [f"arg in {ty} {rank}"], [tuple(size)]
+    ops = [f"push arg0 {dims}"]
+    depth, streamed, vectors = 1, 1, 0
+    for _ in range(int(rng.integers(2, 8))):
+        k = int(rng.integers(0, 4))
+        if depth < 3 and k == 0 and len(args) < 5:
+            pick = int(rng.integers(0, 5))
+            if pick == 0:
+                ops.append("const 1.5")
+            elif pick == 1:
+                ops.append(f"const arg0.{int(rng.integers(0, rank))} f32")
+            else:
+                which = int(rng.choice([0, 1, 1, 2])) if streamed < 2 else int(rng.choice([1, 1, 2]))
+                text, shape = kinds[which]
+                streamed += which == 0
+                vectors += which == 1
+                ops.append(f"push arg{len(args)} {text}")
+                args.append(f"arg in {ty} {len(shape)}")
+                shapes.append(shape)
+            depth += 1
+        elif depth >= 2 and k in (1, 2):
+            ops.append(["add", "sub", "mul", "max", "min", "div"][int(rng.integers(0, 6))])
+            depth -= 1
+        else:
+            ops.append(["relu", "neg", "leaky 0.25", "cast f16", "cast bf16"][int(rng.integers(0, 5))])
+    while depth > 1:
+        ops.append(["add", "sub", "max"][int(rng.integers(0, 3))])
+        depth -= 1
+    text = (RC.HEADER + "\n".join(args) + f"\narg out {ty} {rank}\nsegment {rank}\n size "
+            + " ".join(f"arg0.{k}" for k in range(rank)) + "\n outoff 0\n " + "\n ".join(ops) + "\n store\nend\n")
+    inputs = []
+    for shape in shapes:
+        v = rng.uniform(-2, 2, shape).astype(np.float32)
+        inputs.append(v if ty == "f32" else v.astype(np.float16) if ty == "f16" else O.f32_to_bf16_bits(v))
+    # row vectors are staged in LDS, 16 KiB of them at most
+    return text, inputs, tuple(size), ty, vectors * n * esize <= 16384
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_programs_at_phased_shapes(H, cache, monkeypatch, seed):
+    """Random chains at shapes the phased kernels take, bit for bit against the oracle, with the
+    phased kernels on (checked by name) and off."""
+    monkeypatch.setenv("AFIR_HIP_REGION_GENERIC", "1")
+    rng = np.random.default_rng(4000 + seed)
+    text, inputs, out_shape, ty, fits = _random_phased_program(rng)
+    with np.errstate(all="ignore"):
+        want = RO.evaluate(text, inputs)
+    r = H.Region(text).compile(cache_dir=cache)
+    dev = [_dev(x, r.arg_types[i]) for i, x in enumerate(inputs)]
+    results = []
+    for phased in (None, "0"):
+        if phased is None:
+            monkeypatch.delenv("AFIR_HIP_REGION_PHASED", raising=False)
+        else:
+            monkeypatch.setenv("AFIR_HIP_REGION_PHASED", phased)
+        results.append(_host(r(*dev, out_shape=out_shape), r.arg_types[-1]))
+        if phased is None:
+            assert (H.last_launch()["kernel"] == "afir_region_s0_phased_i32") == fits, (text, H.last_launch())
+    r.close()
+    bits = np.uint32 if ty == "f32" else np.uint16
+    wf = O.bf16_bits_to_f32(want) if ty == "bf16" else want.astype(np.float32)
+    for got in results:
+        gf = O.bf16_bits_to_f32(got) if ty == "bf16" else got.astype(np.float32)
+        same = (got.view(bits) == want.view(bits)) | (np.isnan(wf) & np.isnan(gf))
+        assert same.all(), (text, np.argwhere(~same)[:5])
