@@ -357,6 +357,20 @@ LaunchStatus launch_matmul_any_io(const uint16_t *a, const uint16_t *b, const vo
       return launch_matmul_dma(a, b, static_cast<const uint16_t *>(bias), static_cast<uint16_t *>(out),
                                (int)m, (int)k, (int)n, alpha, relu, block_dim, stream);
   }
+  // A row count that is no multiple of 256 over shapes the direct-to-LDS kernel otherwise takes
+  // (rows are what varies in practice: a batch, a sequence): the whole tiles on that kernel and
+  // the last m % 256 rows in a launch of their own on the bounds-checked kernel below, instead
+  // of everything on the latter (8200 x 8192 x 8192: 680 -> 1400 TFLOP/s).  The two launches
+  // write disjoint rows.
+  const int64_t m_whole = m - m % 256;
+  if (al && !block_dim && m_whole < m && matmul_dma_supported(256, k, n) &&
+      (m_whole / 256) * (n / 256) >= (int64_t)device_cus() / 2) {
+    const LaunchStatus whole = launch_matmul_any_io<F16IO>(a, b, bias, out, m_whole, k, n, alpha, relu, 0, stream);
+    if (whole.code != 0) return whole;
+    const int64_t out_bytes = F16IO ? 4 : 2;
+    return launch_matmul_any_io<F16IO>(a + m_whole * k, b, bias, static_cast<char *>(out) + m_whole * n * out_bytes, m - m_whole,
+                                       k, n, alpha, relu, 0, stream);
+  }
   if (al && !few_big_tiles && k >= kBK && k % kBK == 0 && m % 256 == 0 && n % 256 == 0)
     return launch_mfma<2, 4, 4, 2, F16IO>(a, b, bias, out, (int)m, (int)k, (int)n, alpha, relu, block_dim, stream);
   if (al && k >= kBK && k % kBK == 0 && m % 128 == 0 && n % 128 == 0)
