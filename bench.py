@@ -15,7 +15,9 @@ untimed for --ramp-ms (the device's sustained clocks).  Prints ONE JSON line.
                    wall clock between two device synchronisations
   roofline         algorithmic bytes (flops) per launch / average launch
                    duration from HIP events recorded on the launch stream
-                   around the same K steps, against the published peak
+                   around the last K - 1 of the same K steps (launches that
+                   follow a launch: the host's way from the synchronisation to
+                   its first launch is not kernel time), against the published peak
   cpu_baseline     the C restatement of the reference golden ("port"), timed
                    on this host's cores on a bounded sample
   workloads        with --all (default): the same figures for all five
@@ -698,22 +700,29 @@ def run_workload(w, torch, steps, warmup, ramp_ms=0.0):
     for i in range(warmup):
         w.launches[i % n]()
     torch.cuda.synchronize()
+    # The wall clock brackets exactly the K timed steps between two synchronisations.  The events
+    # bracket the last K - 1 of them: the first event sits behind the first timed launch, so what
+    # they time is launches that follow a launch, not the host's way from the synchronisation to
+    # its first launch (3-15 us of idle device, which at K = 20 would read as 1-4 % of every step).
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
-    e0.record()
+    if steps < 2:
+        e0.record()
     for i in range(steps):
         w.launches[i % n]()
+        if i == 0 and steps >= 2:
+            e0.record()
     e1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
     ev_ms = e0.elapsed_time(e1)
-    return wall, ev_ms
+    return wall, ev_ms, (steps - 1 if steps >= 2 else steps)
 
 
-def summarize(w, wall, ev_ms, steps):
+def summarize(w, wall, ev_ms, steps, ev_steps):
     work = w.work()
-    avg_launch_s = ev_ms / 1e3 / steps
+    avg_launch_s = ev_ms / 1e3 / ev_steps
     if w.bound == "hbm":
         value, unit = work * steps / wall / 1e9, "GB/s"
         achieved, peak = work / avg_launch_s / 1e9, HBM_PEAK_GBS
@@ -776,8 +785,8 @@ def main():
     for key in order:
         w = make_workload(key, torch, H, O, C)
         steps, warmup = steps_for(key), warm_for(key)
-        wall, ev_ms = run_workload(w, torch, steps, warmup, args.ramp_ms)
-        value, unit, roof = summarize(w, wall, ev_ms, steps)
+        wall, ev_ms, ev_steps = run_workload(w, torch, steps, warmup, args.ramp_ms)
+        value, unit, roof = summarize(w, wall, ev_ms, steps, ev_steps)
         par = w.parity()
         extra = (w.power_evidence() if hasattr(w, "power_evidence") and not args.no_power_evidence
                  else None)
