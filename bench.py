@@ -50,16 +50,16 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 # is copied from section (2) of the profiles/ file named beside it, which gives
 # the command that produced it.
 MEASURED_TRAFFIC = {
-    "c1": (201414144, "profiles/add_mul_f32_phased__c1_4096x4096.txt"),
-    "c2": (134633062, "profiles/bcast_add_rowsum_f32_wgrow__c2_8192x4096.txt"),
-    "c3": (134403072, "profiles/relu_bcast_add_transpose_f16_phased__c3_64x1024x512.txt"),
-    "c4": (133898240, "profiles/gather_scale_shift_f16_phased__c4_131072x1024_idx32768.txt"),
-    "c5": (1804703744, "profiles/matmul_bias_leakyrelu_dma__c5_8192x8192x8192.txt"),
-    "g1": (201444044, "profiles/afir_region_s0_phased_i32__g1_compiled_add_mul_f32_4096x4096.txt"),
-    "g2": (134748160, "profiles/afir_region_all_phased_i32__g2_compiled_split_relu_brc_f16_8192x4096.txt"),
-    "g3": (134647808, "profiles/afir_region_s0_rows_i32__g3_compiled_bcast_add_rowsum_f32_8192x4096.txt"),
-    "g4": (133944832, "profiles/afir_region_s0_phased_i32__g4_compiled_gather_scale_shift_f16_131072x1024_idx32768.txt"),
-    "i1": (201612185, "profiles/fused_region_parallel__i1_interpreter_add_mul_f32_4096x4096.txt"),
+    "c1": (201417113, "profiles/add_mul_f32_phased__c1_4096x4096.txt"),
+    "c2": (134633066, "profiles/bcast_add_rowsum_f32_wgrow__c2_8192x4096.txt"),
+    "c3": (134387302, "profiles/relu_bcast_add_transpose_f16_phased__c3_64x1024x512.txt"),
+    "c4": (133898035, "profiles/gather_scale_shift_f16_phased__c4_131072x1024_idx32768.txt"),
+    "c5": (1804801024, "profiles/matmul_bias_leakyrelu_dma__c5_8192x8192x8192.txt"),
+    "g1": (201432473, "profiles/afir_region_s0_phased_i32__g1_compiled_add_mul_f32_4096x4096.txt"),
+    "g2": (134726553, "profiles/afir_region_all_phased_i32__g2_compiled_split_relu_brc_f16_8192x4096.txt"),
+    "g3": (134646784, "profiles/afir_region_s0_rows_i32__g3_compiled_bcast_add_rowsum_f32_8192x4096.txt"),
+    "g4": (133937868, "profiles/afir_region_s0_phased_i32__g4_compiled_gather_scale_shift_f16_131072x1024_idx32768.txt"),
+    "i1": (201611468, "profiles/fused_region_parallel__i1_interpreter_add_mul_f32_4096x4096.txt"),
     "i2": (135332659, "profiles/fused_region_parallel__i2_interpreter_split_relu_brc_f16_8192x4096.txt"),
 }
 
