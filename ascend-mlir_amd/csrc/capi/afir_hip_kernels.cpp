@@ -722,6 +722,21 @@ uint32_t afir_hip_region_attach_code_object(uint64_t handle, const void *image, 
   return AFIR_HIP_OK;
 }
 
+uint32_t afir_hip_region_load(uint64_t handle) {
+  auto r = find_region(handle);
+  if (!r) return fail(AFIR_HIP_E_UNKNOWN, "no region program with that handle");
+  std::shared_ptr<CompiledRegion> c;
+  {
+    std::lock_guard<std::mutex> lock(g_region_mutex);
+    c = r->compiled;
+  }
+  if (!c) return AFIR_HIP_OK;   // nothing attached: the interpreter needs no loading
+  const std::string why = compiled_function(c.get(), r->program, "", nullptr);
+  if (!why.empty()) return fail(AFIR_HIP_E_LAUNCH, why);
+  g_last_error.clear();
+  return AFIR_HIP_OK;
+}
+
 uint32_t afir_hip_region_compile(uint64_t handle, void *image_out, size_t capacity, size_t *image_len) {
   auto r = find_region(handle);
   if (!r) return fail(AFIR_HIP_E_UNKNOWN, "no region program with that handle");

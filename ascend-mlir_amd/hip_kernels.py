@@ -50,6 +50,7 @@ EXPORTED_SYMBOLS = [
     "afir_hip_region_emit_source",
     "afir_hip_region_attach_code_object",
     "afir_hip_region_compile",
+    "afir_hip_region_load",
     "afir_hip_region_prefer_code_object",
     "afir_hip_region_argument_bytes",
     "afir_hip_launch_region",

@@ -249,6 +249,13 @@ const char *afir_hip_region_route(uint64_t handle, const void *tiling, size_t ti
  * that kernel.  Matmul programs have no source form (AFIR_HIP_E_INVALID). */
 uint32_t afir_hip_region_emit_source(uint64_t handle, char *buffer, size_t capacity, size_t *length);
 uint32_t afir_hip_region_attach_code_object(uint64_t handle, const void *image, size_t image_len);
+/* Loads the attached code object on the current device now and checks it against
+ * the program (hash, kernel-set version), which the first launch would otherwise
+ * do: for callers that time their first launch or are about to capture one into
+ * a graph.  Nothing attached: nothing to do, success.  No counterpart in the
+ * reference, whose runner loads its device binary per run
+ * (lib/Runtime/Execution/NativeExecutionRunner.cpp:372-528). */
+uint32_t afir_hip_region_load(uint64_t handle);
 /* Emit, compile and attach in one call, inside the process: the source of
  * afir_hip_region_emit_source is compiled for gfx950 by the runtime-compilation
  * library of the HIP runtime (libhiprtc, opened on first use), with the options
