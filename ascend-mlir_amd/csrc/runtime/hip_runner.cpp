@@ -32,6 +32,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <map>
+#include <mutex>
 
 #include "runtime.h"
 
@@ -120,6 +121,10 @@ class HipExecutionRunner final : public ExecutionRunner {
 
   Status runDynamicLibraryArtifact(const DynamicLibraryExecutionLaunch &launch,
                                    RunArgs &args) override {
+    // one run at a time per runner: the stream, the timing events and what is kept between runs
+    // are the runner's.  (The reference's C API has no locks and is called from one thread; threads
+    // that share an executor here take turns.)
+    std::lock_guard<std::mutex> runLock(runMutex_);
     lastKernelUs_ = -1.0;
     lastRegionRoute_.clear();
     lastGrid_ = {};
@@ -402,6 +407,7 @@ class HipExecutionRunner final : public ExecutionRunner {
       (void)hipFree(p);
     }
   }
+  std::mutex runMutex_;
   std::map<std::string, void *> libs_;
   std::map<std::string, CachedRegion> regions_;
   std::multimap<size_t, void *> pool_;
