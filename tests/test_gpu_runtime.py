@@ -238,15 +238,16 @@ def test_reference_block_dim_values_do_not_size_the_grid(R, executor, tmp_path, 
     inputs, out, dims, want = _full_size(family)
     tiling = R.TilingSchema.for_kernel(family).pack(**dims)
     seen = {}
-    for block_dim in (0, 1, 8, 40):
-        best = None
-        for _ in range(3):                      # the fastest of three: a first launch runs at idle clocks
+    # the fastest of five per value, the values taking turns: a launch that follows a host copy
+    # runs at whatever clocks the device has reached, and drifts of that kind hit every value alike
+    for _ in range(5):
+        for block_dim in (0, 1, 8, 40):
             out[...] = 0
             got = executor.execute(binary, family, inputs, [out], tiling, block_dim=block_dim)
             assert got[0].tobytes() == want.tobytes(), block_dim
             note = executor.runtime.last_launch()
-            best = note if best is None or note["kernel_ns"] < best["kernel_ns"] else best
-        seen[block_dim] = best
+            best = seen.get(block_dim)
+            seen[block_dim] = note if best is None or note["kernel_ns"] < best["kernel_ns"] else best
     base = seen[0]
     assert base["workgroups"] >= 1024 and "phased" in base["kernel"], base
     for block_dim in (1, 8, 40):
