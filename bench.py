@@ -444,6 +444,13 @@ def make_workload(key, torch, H, O, C):
                                H.pack_tiling(8192, 8192, 8192, H.f32_bits(0.01)))
             ev["kernel_constant_operands_tflops"] = round(rate(lambda i: launch(), n=20, warm=3), 1)
             ev["vendor_gemm_constant_operands_tflops"] = round(rate(lambda i: torch.matmul(ones, ones), n=20, warm=3), 1)
+            # the board's own power reading against its cap while each kind of operand runs
+            # (hwmon of the amdgpu driver; absent where the driver does not expose it)
+            cap = _board_power("power1_cap")
+            if cap:
+                ev["board_power_cap_w"] = cap
+                ev["board_power_w_this_kernel_workload_operands"] = _power_while(torch, ours)
+                ev["board_power_w_this_kernel_constant_operands"] = _power_while(torch, lambda i: launch())
             return ev
         w.power_evidence = power_evidence
     elif key == "m_b16":
@@ -684,6 +691,34 @@ def make_workload(key, torch, H, O, C):
     return w
 
 
+def _board_power(name="power1_input"):
+    """Watts from the amdgpu driver's hwmon file of the first card that has one, or None."""
+    import glob
+    for path in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/" + name)):
+        try:
+            with open(path) as f:
+                return round(int(f.read().strip()) / 1e6, 1)
+        except (OSError, ValueError):
+            continue
+    return None
+
+
+def _power_while(torch, launch, seconds=1.0):
+    """Median board power over the second half of `seconds` of back-to-back launches."""
+    readings, i = [], 0
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            launch(i)
+            i += 1
+        torch.cuda.synchronize()
+        if time.perf_counter() - t0 > seconds / 2:
+            p = _board_power()
+            if p is not None:
+                readings.append(p)
+    return sorted(readings)[len(readings) // 2] if readings else None
+
+
 def run_workload(w, torch, steps, warmup, ramp_ms=0.0):
     n = len(w.launches)
     # The device takes some 50-100 ms of continuous work to settle at its sustained clocks (the
@@ -864,7 +899,9 @@ def main():
                                   "frac_of_mfma_only": r5.get("frac_of_mfma_only"),
                                   "vs_vendor_gemm": r5.get("vs_vendor_gemm"),
                                   "vendor_gemm_tflops": ev.get("vendor_gemm_tflops"),
-                                  "this_kernel_alternating_tflops": ev.get("this_kernel_alternating_tflops")}
+                                  "this_kernel_alternating_tflops": ev.get("this_kernel_alternating_tflops"),
+                                  "board_power_w": ev.get("board_power_w_this_kernel_workload_operands"),
+                                  "board_power_cap_w": ev.get("board_power_cap_w")}
         line["targets"] = {k: {"frac": by_key[k]["roofline"]["frac"], "target": t,
                                "met": by_key[k]["roofline"]["frac"] >= t,
                                "parity": by_key[k]["parity"]["passed"],
