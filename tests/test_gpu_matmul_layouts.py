@@ -139,6 +139,11 @@ def test_large_batched_products_take_the_direct_to_lds_kernel(H, ty, flags, batc
     assert H.last_launch()["kernel"].startswith("matmul_bias_leakyrelu_dma"), H.last_launch()
     assert "batched" in H.last_launch()["kernel"]
     assert got.tobytes() == want.tobytes()
+    if not flags:                               # the same batch without bias and activation
+        text = _program(3, ty, flags, False)
+        want = RO.evaluate(text, [a, b], out_shape=(batch, m, n))
+        got = _run(H, text, [a, b], ty, (batch, m, n))
+        assert "batched" in H.last_launch()["kernel"] and got.tobytes() == want.tobytes()
 
 
 @pytest.mark.parametrize("ty", ["bf16", "f16"])
