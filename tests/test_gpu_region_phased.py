@@ -246,3 +246,26 @@ def test_random_programs_at_phased_shapes(H, cache, monkeypatch, seed):
         gf = O.bf16_bits_to_f32(got) if ty == "bf16" else got.astype(np.float32)
         same = (got.view(bits) == want.view(bits)) | (np.isnan(wf) & np.isnan(gf))
         assert same.all(), (text, np.argwhere(~same)[:5])
+
+
+def test_a_code_object_can_be_loaded_ahead_of_the_first_launch(H, cache):
+    """afir_hip_region_load: nothing attached is nothing to do; an attached code object is loaded
+    and checked against the program now (what the first launch would otherwise do), so an image
+    built from another program is refused here, before anything is launched."""
+    import ctypes
+    L = H.load()
+    L.afir_hip_region_load.restype = ctypes.c_uint32
+    L.afir_hip_region_load.argtypes = [ctypes.c_uint64]
+    r = H.Region(RC.C1_ADD_MUL)
+    assert L.afir_hip_region_load(ctypes.c_uint64(r.handle)) == 0          # the interpreter needs no loading
+    r.compile(cache_dir=cache)
+    assert L.afir_hip_region_load(ctypes.c_uint64(r.handle)) == 0
+    assert L.afir_hip_region_load(ctypes.c_uint64(r.handle)) == 0          # already loaded
+    other = H.Region(RC.RELU_COL_ADD)
+    image = H.compile_region_source(r.emit_source(), cache)
+    other.attach_code_object(image)
+    assert L.afir_hip_region_load(ctypes.c_uint64(other.handle)) != 0
+    assert b"not built from this program" in L.afir_hip_last_error()
+    assert L.afir_hip_region_load(ctypes.c_uint64(987654321)) != 0
+    r.close()
+    other.close()
